@@ -1,0 +1,179 @@
+/*
+ * C ABI of libnt_hip.so: hand-written gfx950 (MI355X) kernels for the programs
+ * that ninetoothed.make produces (tiled matmul / addmm, row softmax, fused
+ * scaled-dot-product attention forward, conv2d as implicit GEMM).
+ *
+ * The type layer is the one the reference emits into its generated
+ * `ninetoothed.h` (reference: src/ninetoothed/aot.py:558-586): tensors travel
+ * BY VALUE as {data, shape, strides} with strides counted in ELEMENTS, the
+ * stream is an opaque pointer (a hipStream_t here), and every launch function
+ * returns an int: 0 on success, a hipError_t value when the runtime refuses
+ * the launch, NINETOOTHED_NO_KERNEL (1) when no kernel exists for the given
+ * configuration (reference: src/ninetoothed/build.py:167-170 `return 1;`).
+ * Zero-dimensional tensors carry scalars: `data` points to a HOST double
+ * (floating point) or a HOST int64_t (integer / boolean), `shape` and
+ * `strides` are not read (reference: src/ninetoothed/aot.py:725-733, 624-628).
+ *
+ * Launches are asynchronous on the given stream, never synchronise and never
+ * allocate; the caller owns every buffer.  All functions are re-entrant.
+ */
+#ifndef NINETOOTHED_HIP_H
+#define NINETOOTHED_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NINETOOTHED_TRUE 1
+#define NINETOOTHED_FALSE 0
+#define NINETOOTHED_NONE 0
+
+/* returned when no kernel matches the request (dtype / rank / block sizes) */
+#define NINETOOTHED_NO_KERNEL 1
+
+/* same member order as the reference's enum (src/ninetoothed/aot.py:524-537) */
+enum NineToothedDataType {
+    NINETOOTHED_INT8,
+    NINETOOTHED_INT16,
+    NINETOOTHED_INT32,
+    NINETOOTHED_INT64,
+    NINETOOTHED_UINT8,
+    NINETOOTHED_UINT16,
+    NINETOOTHED_UINT32,
+    NINETOOTHED_UINT64,
+    NINETOOTHED_FLOAT16,
+    NINETOOTHED_BFLOAT16,
+    NINETOOTHED_FLOAT32,
+    NINETOOTHED_FLOAT64
+};
+
+typedef struct {
+    void *data;
+    uint64_t *shape;
+    int64_t *strides;
+} NineToothedTensor;
+
+typedef void *NineToothedStream;
+
+typedef int NineToothedResult;
+
+/*
+ * Block-size arguments (`block_size_*`) are the values of the arrangement's
+ * meta symbols.  0 means "library's choice" (the tuned / heuristic tile); a
+ * positive value is honoured when a kernel instance with that tile exists and
+ * otherwise mapped to the nearest instance -- results do not depend on it.
+ */
+
+/* output[M,N] = lhs[M,K] @ rhs[K,N], fp32 accumulation, one rounding on store.
+ * Replaces the kernel generated for tests/test_matmul.py:14-45 (== README.md:40-62):
+ * generated launch function src/ninetoothed/generation.py:545-600.
+ * `dtype` is the element type of lhs/rhs; `output_dtype` that of output
+ * (FLOAT16, BFLOAT16 or FLOAT32).  Any strides are accepted. */
+NineToothedResult launch_nt_matmul(NineToothedStream stream,
+                                   NineToothedTensor lhs,
+                                   NineToothedTensor rhs,
+                                   NineToothedTensor output,
+                                   int dtype, int output_dtype,
+                                   int block_size_m, int block_size_n,
+                                   int block_size_k);
+
+/* output = beta * input + alpha * round_to_dtype(mat1 @ mat2), epilogue in fp32.
+ * Replaces the kernel generated for tests/test_addmm.py:13-38 (argument order
+ * input, mat1, mat2, beta, alpha, output as in its application).  beta and
+ * alpha are 0-d tensors holding a host double. */
+NineToothedResult launch_nt_addmm(NineToothedStream stream,
+                                  NineToothedTensor input,
+                                  NineToothedTensor mat1,
+                                  NineToothedTensor mat2,
+                                  NineToothedTensor beta,
+                                  NineToothedTensor alpha,
+                                  NineToothedTensor output,
+                                  int dtype,
+                                  int block_size_m, int block_size_n,
+                                  int block_size_k);
+
+/* output[r, :] = softmax(input[r, :]) over the last of two dims, in fp32
+ * arithmetic.  Replaces the kernel generated for tests/test_softmax.py:10-27
+ * (one program per row, BLOCK_SIZE >= row length). */
+NineToothedResult launch_nt_softmax(NineToothedStream stream,
+                                    NineToothedTensor input,
+                                    NineToothedTensor output,
+                                    int dtype, int block_size);
+
+/* o = softmax(scale * q k^T [+ causal mask]) v for q,k,v,o of shape
+ * [batch, heads, seq, head_dim] (k/v may have their own seq length).
+ * Replaces the kernel generated for tests/test_attention.py:14-70; that
+ * program has scale == 1, the scale tensor (0-d, host double) is this
+ * library's extension for the 1/sqrt(head_dim) configuration.
+ * is_causal is a 0-d tensor holding a host int64_t. */
+NineToothedResult launch_nt_attention(NineToothedStream stream,
+                                      NineToothedTensor q,
+                                      NineToothedTensor k,
+                                      NineToothedTensor v,
+                                      NineToothedTensor is_causal,
+                                      NineToothedTensor scale,
+                                      NineToothedTensor o,
+                                      int dtype,
+                                      int block_size_m, int block_size_n);
+
+/* output[N,K,P,Q] = conv2d(input[N,C,H,W], filter[K,C,R,S]) with stride 1,
+ * dilation 1 and zero padding (padding_h, padding_w), computed as the implicit
+ * GEMM [N*P*Q, C*R*S] x [C*R*S, K] the arrangement of
+ * tests/test_conv2d.py:13-48 describes. */
+NineToothedResult launch_nt_conv2d(NineToothedStream stream,
+                                   NineToothedTensor input,
+                                   NineToothedTensor filter,
+                                   NineToothedTensor output,
+                                   int dtype,
+                                   int padding_h, int padding_w,
+                                   int block_size_m, int block_size_n,
+                                   int block_size_k);
+
+/* ---- tile selection (stands in for the reference's Triton autotuner,
+ * src/ninetoothed/generation.py:372-516 and src/ninetoothed/auto_tuner.py:11-152) ---- */
+
+/* Number of GEMM kernel instances compiled into the library. */
+int nt_gemm_num_configs(void);
+
+/* Writes a short description ("256x256x64 w8 s2 ...") of instance `config`
+ * into `buffer` (at most `size` bytes, NUL terminated).  Returns 0, or
+ * NINETOOTHED_NO_KERNEL for an unknown index. */
+NineToothedResult nt_gemm_config_name(int config, char *buffer, int size);
+
+/* Runs instance `config` (as launch_nt_addmm when input.data != NULL, as
+ * launch_nt_matmul otherwise).  Returns NINETOOTHED_NO_KERNEL when the
+ * instance cannot handle the shapes / strides given. */
+NineToothedResult launch_nt_gemm_config(NineToothedStream stream, int config,
+                                        NineToothedTensor input,
+                                        NineToothedTensor mat1,
+                                        NineToothedTensor mat2,
+                                        NineToothedTensor beta,
+                                        NineToothedTensor alpha,
+                                        NineToothedTensor output,
+                                        int dtype, int output_dtype);
+
+/* Times every instance that accepts the problem (hipEvents on `stream`,
+ * `iters` launches each after 2 warm-ups; this call synchronises) and stores
+ * the winner in the per-device cache that launch_nt_matmul / launch_nt_addmm
+ * consult when block sizes are 0.  Returns 0 and the winner in *best_config,
+ * its average time in *best_ms. */
+NineToothedResult nt_tune_gemm(NineToothedStream stream,
+                               NineToothedTensor input,
+                               NineToothedTensor mat1,
+                               NineToothedTensor mat2,
+                               NineToothedTensor beta,
+                               NineToothedTensor alpha,
+                               NineToothedTensor output,
+                               int dtype, int output_dtype, int iters,
+                               int *best_config, float *best_ms);
+
+/* Library version string, e.g. "nt_hip 0.1 gfx950". */
+const char *nt_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* NINETOOTHED_HIP_H */

@@ -1,0 +1,414 @@
+// C ABI for the GEMM family: launch_nt_matmul, launch_nt_addmm,
+// launch_nt_conv2d and the tile-selection entry points.
+#include <mutex>
+#include <shared_mutex>
+#include <unordered_map>
+#include <vector>
+#include <cstdio>
+#include <cstring>
+
+#include "gemm_fast.h"
+#include "gemm_generic.h"
+
+namespace nt {
+namespace {
+
+struct GemmProblem {
+    int dtype, out_dtype;
+    int m, n, k;
+    const void *a, *b, *bias;
+    void *c;
+    int64_t sam, sak, sbk, sbn, scm, scn, sim, sin;
+    float alpha, beta;
+    bool addmm() const { return bias != nullptr; }
+};
+
+int g_tile_order = 0;  // see GemmParams::order; changed only by measurement builds
+
+typedef hipError_t (*LaunchFn)(const GemmProblem &, hipStream_t);
+typedef bool (*AcceptFn)(const GemmProblem &);
+
+struct GemmInstance {
+    const char *name;
+    int bm, bn, bk;
+    AcceptFn accepts;
+    LaunchFn launch;
+};
+
+template <int BM, int BN, int BK, int kStages>
+bool fast_accepts(const GemmProblem &q) {
+    if (q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) return false;
+    if (q.out_dtype != q.dtype) return false;
+    if (q.m <= 0 || q.n <= 0 || q.k <= 0) return false;
+    if (q.m % BM || q.n % BN || q.k % BK) return false;
+    if (q.sak != 1 || q.sbn != 1 || q.scn != 1) return false;
+    if (q.sam % 8 || q.sbk % 8 || q.sam < q.k || q.sbk < q.n || q.scm < q.n) return false;
+    if (((uintptr_t)q.a & 15) || ((uintptr_t)q.b & 15) || ((uintptr_t)q.c & 15) || q.scm % 8) return false;
+    // per-lane 32-bit byte offsets inside one tile panel
+    if ((int64_t)BM * q.sam * 2 >= (int64_t(1) << 31)) return false;
+    if ((int64_t)q.k * q.sbk * 2 >= (int64_t(1) << 31)) return false;
+    return true;
+}
+
+void fill_params(GemmParams &p, const GemmProblem &q, int bm, int bn) {
+    p.a = q.a;
+    p.b = q.b;
+    p.c = q.c;
+    p.bias = q.bias;
+    p.m = q.m;
+    p.n = q.n;
+    p.k = q.k;
+    p.lda = q.sam;
+    p.ldb = q.sbk;
+    p.ldc = q.scm;
+    p.bias_stride_m = q.sim;
+    p.bias_stride_n = q.sin;
+    p.alpha = q.alpha;
+    p.beta = q.beta;
+    p.tiles_m = q.m / bm;
+    p.tiles_n = q.n / bn;
+    p.order = g_tile_order;
+    p.bias_vector = q.bias != nullptr && q.sin == 1 && q.sim % 8 == 0 && ((uintptr_t)q.bias & 15) == 0;
+}
+
+template <typename T, int BM, int BN, int BK, int WM, int WN, int kStages, int kOcc, int kAblate, int kLoad, int kAux>
+hipError_t fast_launch_typed(const GemmProblem &q, hipStream_t stream) {
+    GemmParams p;
+    fill_params(p, q, BM, BN);
+    const dim3 grid(p.tiles_m * p.tiles_n), block(WM * WN * 64);
+    if (q.addmm()) {
+        auto kernel = gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, true, kAblate, kLoad, kAux>;
+        kernel<<<grid, block, 0, stream>>>(p);
+    } else {
+        auto kernel = gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, false, kAblate, kLoad, kAux>;
+        kernel<<<grid, block, 0, stream>>>(p);
+    }
+    return hipGetLastError();
+}
+
+template <int BM, int BN, int BK, int WM, int WN, int kStages, int kOcc, int kAblate = 0, int kLoad = 1, int kAux = 0>
+hipError_t fast_launch(const GemmProblem &q, hipStream_t stream) {
+    if (q.dtype == NINETOOTHED_FLOAT16) return fast_launch_typed<half_t, BM, BN, BK, WM, WN, kStages, kOcc, kAblate, kLoad, kAux>(q, stream);
+    return fast_launch_typed<bf16_t, BM, BN, BK, WM, WN, kStages, kOcc, kAblate, kLoad, kAux>(q, stream);
+}
+
+bool generic_accepts(const GemmProblem &q) {
+    if (q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) return false;
+    if (q.out_dtype != q.dtype && q.out_dtype != NINETOOTHED_FLOAT32) return false;
+    return q.m >= 0 && q.n >= 0 && q.k >= 0;
+}
+
+template <typename T, typename TOut>
+hipError_t generic_launch_typed(const GemmProblem &q, hipStream_t stream) {
+    StridedProblem<T, TOut> prob;
+    prob.m = q.m;
+    prob.n = q.n;
+    prob.k = q.k;
+    prob.a = (const T *)q.a;
+    prob.b = (const T *)q.b;
+    prob.c = (TOut *)q.c;
+    prob.bias = (const T *)q.bias;
+    prob.sam = q.sam;
+    prob.sak = q.sak;
+    prob.sbk = q.sbk;
+    prob.sbn = q.sbn;
+    prob.scm = q.scm;
+    prob.scn = q.scn;
+    prob.sbm_ = q.sim;
+    prob.sbn_ = q.sin;
+    prob.alpha = q.alpha;
+    prob.beta = q.beta;
+    const int64_t tiles = (int64_t)ceil_div(q.m, kGenBM) * ceil_div(q.n, kGenBN);
+    if (tiles == 0) return hipSuccess;  // empty launch is legal
+    gemm_generic_kernel<StridedProblem<T, TOut>><<<dim3((unsigned)tiles), dim3(kGenThreads), 0, stream>>>(prob);
+    return hipGetLastError();
+}
+
+hipError_t generic_launch(const GemmProblem &q, hipStream_t stream) {
+    const bool f32out = q.out_dtype == NINETOOTHED_FLOAT32;
+    if (q.dtype == NINETOOTHED_FLOAT16)
+        return f32out ? generic_launch_typed<half_t, float>(q, stream) : generic_launch_typed<half_t, half_t>(q, stream);
+    return f32out ? generic_launch_typed<bf16_t, float>(q, stream) : generic_launch_typed<bf16_t, bf16_t>(q, stream);
+}
+
+// BM, BN, BK, wave grid WM x WN, LDS stages, waves per SIMD the register budget allows
+#define NT_FAST_INSTANCE(BM, BN, BK, WM, WN, ST, OCC) \
+    {#BM "x" #BN "x" #BK " waves " #WM "x" #WN " stages " #ST " lds-direct", BM, BN, BK, fast_accepts<BM, BN, BK, ST>, fast_launch<BM, BN, BK, WM, WN, ST, OCC>}
+
+const GemmInstance kInstances[] = {
+    {"128x128x32 waves 2x2 any-stride", kGenBM, kGenBN, kGenBK, generic_accepts, generic_launch},
+    NT_FAST_INSTANCE(256, 256, 32, 2, 4, 4, 2),
+    NT_FAST_INSTANCE(256, 256, 64, 2, 4, 2, 2),
+    NT_FAST_INSTANCE(128, 128, 64, 2, 2, 2, 2),
+#ifdef NT_GEMM_ABLATION
+#define NT_LOAD_INSTANCE(BM, BN, BK, WM, WN, ST, OCC, LD, AUX) \
+    {#BM "x" #BN "x" #BK " waves " #WM "x" #WN " stages " #ST " load " #LD " aux " #AUX, BM, BN, BK, fast_accepts<BM, BN, BK, ST>, fast_launch<BM, BN, BK, WM, WN, ST, OCC, 0, LD, AUX>}
+#define NT_ABLATED_INSTANCE(BM, BN, BK, WM, WN, ST, OCC, AB) \
+    {#BM "x" #BN "x" #BK " waves " #WM "x" #WN " stages " #ST " ABLATED " #AB " (wrong results)", BM, BN, BK, fast_accepts<BM, BN, BK, ST>, fast_launch<BM, BN, BK, WM, WN, ST, OCC, AB>}
+    NT_LOAD_INSTANCE(256, 256, 32, 2, 4, 5, 2, 1, 0),
+    NT_LOAD_INSTANCE(256, 256, 32, 2, 2, 4, 1, 1, 0),
+    NT_LOAD_INSTANCE(128, 256, 32, 2, 2, 4, 2, 1, 0),
+    NT_ABLATED_INSTANCE(256, 256, 32, 2, 4, 4, 2, 1),
+    NT_ABLATED_INSTANCE(256, 256, 32, 2, 4, 4, 2, 2),
+    NT_ABLATED_INSTANCE(256, 256, 32, 2, 4, 4, 2, 3),
+#endif
+};
+constexpr int kNumInstances = sizeof(kInstances) / sizeof(kInstances[0]);
+
+// ---- per-device cache of tuned choices (device, problem signature) -> instance ----
+struct TuneKey {
+    int device, dtype, out_dtype, m, n, k, addmm;
+    bool operator==(const TuneKey &o) const {
+        return device == o.device && dtype == o.dtype && out_dtype == o.out_dtype && m == o.m && n == o.n && k == o.k && addmm == o.addmm;
+    }
+};
+struct TuneKeyHash {
+    size_t operator()(const TuneKey &x) const {
+        size_t h = 1469598103934665603ull;
+        const int v[] = {x.device, x.dtype, x.out_dtype, x.m, x.n, x.k, x.addmm};
+        for (int e : v) h = (h ^ (size_t)(unsigned)e) * 1099511628211ull;
+        return h;
+    }
+};
+std::shared_mutex g_tune_mutex;
+std::unordered_map<TuneKey, int, TuneKeyHash> g_tuned;
+
+TuneKey make_key(const GemmProblem &q) {
+    int device = 0;
+    (void)hipGetDevice(&device);
+    return TuneKey{device, q.dtype, q.out_dtype, q.m, q.n, q.k, q.addmm() ? 1 : 0};
+}
+
+int lookup_tuned(const GemmProblem &q) {
+    const TuneKey key = make_key(q);
+    std::shared_lock<std::shared_mutex> lock(g_tune_mutex);
+    auto it = g_tuned.find(key);
+    return it == g_tuned.end() ? -1 : it->second;
+}
+
+// Untuned choice: the largest direct-to-LDS tile that still gives every CU a
+// tile (256 CUs), falling back to smaller tiles, then to the any-stride kernel.
+int heuristic_choice(const GemmProblem &q, int bm, int bn, int bk) {
+    if (bm > 0 && bn > 0) {  // caller fixed the blocks: nearest accepting instance
+        int best = -1;
+        long best_d = 0;
+        for (int i = 0; i < kNumInstances; ++i) {
+            if (!kInstances[i].accepts(q)) continue;
+            long d = labs(kInstances[i].bm - bm) + labs(kInstances[i].bn - bn) + (bk > 0 ? labs(kInstances[i].bk - bk) : 0);
+            if (best < 0 || d < best_d) {
+                best = i;
+                best_d = d;
+            }
+        }
+        return best;
+    }
+    const int order[] = {1, 2, 3};
+    for (int idx : order) {
+        const GemmInstance &inst = kInstances[idx];
+        if (!inst.accepts(q)) continue;
+        const int64_t tiles = (int64_t)(q.m / inst.bm) * (q.n / inst.bn);
+        if (tiles >= 256 || idx == 3) return idx;
+    }
+    return kInstances[0].accepts(q) ? 0 : -1;
+}
+
+bool read_matrix(const NineToothedTensor &t, uint64_t &d0, uint64_t &d1, int64_t &s0, int64_t &s1) {
+    if (t.shape == nullptr || t.strides == nullptr) return false;
+    d0 = t.shape[0];
+    d1 = t.shape[1];
+    s0 = t.strides[0];
+    s1 = t.strides[1];
+    return true;
+}
+
+int build_problem(GemmProblem &q, const NineToothedTensor *input, const NineToothedTensor &a, const NineToothedTensor &b,
+                  const NineToothedTensor *beta, const NineToothedTensor *alpha, const NineToothedTensor &c, int dtype,
+                  int out_dtype) {
+    uint64_t am, ak, bk, bn, cm, cn;
+    if (!read_matrix(a, am, ak, q.sam, q.sak) || !read_matrix(b, bk, bn, q.sbk, q.sbn) || !read_matrix(c, cm, cn, q.scm, q.scn))
+        return hipErrorInvalidValue;
+    if (ak != bk || am != cm || bn != cn) return hipErrorInvalidValue;
+    if (am > 0x7fffffffull || bn > 0x7fffffffull || ak > 0x7fffffffull) return NINETOOTHED_NO_KERNEL;
+    q.dtype = dtype;
+    q.out_dtype = out_dtype;
+    q.m = (int)am;
+    q.n = (int)bn;
+    q.k = (int)ak;
+    q.a = a.data;
+    q.b = b.data;
+    q.c = c.data;
+    q.bias = nullptr;
+    q.sim = q.sin = 0;
+    q.alpha = 1.0f;
+    q.beta = 0.0f;
+    if (input != nullptr && input->data != nullptr) {
+        uint64_t im, in_;
+        if (!read_matrix(*input, im, in_, q.sim, q.sin)) return hipErrorInvalidValue;
+        if (im != cm || in_ != cn) return hipErrorInvalidValue;
+        if (beta == nullptr || alpha == nullptr || beta->data == nullptr || alpha->data == nullptr) return hipErrorInvalidValue;
+        q.bias = input->data;
+        q.beta = (float)Scalar0d::as_double(*beta);
+        q.alpha = (float)Scalar0d::as_double(*alpha);
+    }
+    if ((q.m > 0 && q.n > 0) && (q.a == nullptr && q.k > 0)) return hipErrorInvalidValue;
+    return 0;
+}
+
+int run_gemm(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk) {
+    if (q.m == 0 || q.n == 0) return 0;
+    int choice = -1;
+    if (bm <= 0 || bn <= 0) choice = lookup_tuned(q);
+    if (choice < 0 || !kInstances[choice].accepts(q)) choice = heuristic_choice(q, bm, bn, bk);
+    if (choice < 0) return NINETOOTHED_NO_KERNEL;
+    return (int)kInstances[choice].launch(q, stream);
+}
+
+}  // namespace
+}  // namespace nt
+
+using namespace nt;
+
+extern "C" {
+
+NineToothedResult launch_nt_matmul(NineToothedStream stream, NineToothedTensor lhs, NineToothedTensor rhs,
+                                   NineToothedTensor output, int dtype, int output_dtype, int block_size_m,
+                                   int block_size_n, int block_size_k) {
+    GemmProblem q;
+    if (int err = build_problem(q, nullptr, lhs, rhs, nullptr, nullptr, output, dtype, output_dtype)) return err;
+    return run_gemm((hipStream_t)stream, q, block_size_m, block_size_n, block_size_k);
+}
+
+NineToothedResult launch_nt_addmm(NineToothedStream stream, NineToothedTensor input, NineToothedTensor mat1,
+                                  NineToothedTensor mat2, NineToothedTensor beta, NineToothedTensor alpha,
+                                  NineToothedTensor output, int dtype, int block_size_m, int block_size_n,
+                                  int block_size_k) {
+    if (input.data == nullptr) return hipErrorInvalidValue;
+    GemmProblem q;
+    if (int err = build_problem(q, &input, mat1, mat2, &beta, &alpha, output, dtype, dtype)) return err;
+    return run_gemm((hipStream_t)stream, q, block_size_m, block_size_n, block_size_k);
+}
+
+int nt_gemm_num_configs(void) { return kNumInstances; }
+
+NineToothedResult nt_gemm_config_name(int config, char *buffer, int size) {
+    if (config < 0 || config >= kNumInstances || buffer == nullptr || size <= 0) return NINETOOTHED_NO_KERNEL;
+    snprintf(buffer, (size_t)size, "%s", kInstances[config].name);
+    return 0;
+}
+
+NineToothedResult launch_nt_gemm_config(NineToothedStream stream, int config, NineToothedTensor input,
+                                        NineToothedTensor mat1, NineToothedTensor mat2, NineToothedTensor beta,
+                                        NineToothedTensor alpha, NineToothedTensor output, int dtype,
+                                        int output_dtype) {
+    if (config < 0 || config >= kNumInstances) return NINETOOTHED_NO_KERNEL;
+    GemmProblem q;
+    if (int err = build_problem(q, &input, mat1, mat2, &beta, &alpha, output, dtype, output_dtype)) return err;
+    if (q.m == 0 || q.n == 0) return 0;
+    if (!kInstances[config].accepts(q)) return NINETOOTHED_NO_KERNEL;
+    return (int)kInstances[config].launch(q, (hipStream_t)stream);
+}
+
+NineToothedResult nt_tune_gemm(NineToothedStream stream_, NineToothedTensor input, NineToothedTensor mat1,
+                               NineToothedTensor mat2, NineToothedTensor beta, NineToothedTensor alpha,
+                               NineToothedTensor output, int dtype, int output_dtype, int iters, int *best_config,
+                               float *best_ms) {
+    hipStream_t stream = (hipStream_t)stream_;
+    GemmProblem q;
+    if (int err = build_problem(q, &input, mat1, mat2, &beta, &alpha, output, dtype, output_dtype)) return err;
+    if (iters <= 0) iters = 5;
+    hipEvent_t start, stop;
+    hipError_t err;
+    if ((err = hipEventCreate(&start)) != hipSuccess) return (int)err;
+    if ((err = hipEventCreate(&stop)) != hipSuccess) {
+        (void)hipEventDestroy(start);
+        return (int)err;
+    }
+    int best = -1;
+    float best_time = 0.0f;
+    for (int i = 0; i < kNumInstances && err == hipSuccess; ++i) {
+        if (!kInstances[i].accepts(q)) continue;
+        for (int w = 0; w < 2 && err == hipSuccess; ++w) err = kInstances[i].launch(q, stream);
+        if (err != hipSuccess) break;
+        (void)hipEventRecord(start, stream);
+        for (int r = 0; r < iters && err == hipSuccess; ++r) err = kInstances[i].launch(q, stream);
+        (void)hipEventRecord(stop, stream);
+        if (err != hipSuccess) break;
+        if ((err = hipEventSynchronize(stop)) != hipSuccess) break;
+        float ms = 0.0f;
+        (void)hipEventElapsedTime(&ms, start, stop);
+        ms /= (float)iters;
+        if (best < 0 || ms < best_time) {
+            best = i;
+            best_time = ms;
+        }
+    }
+    (void)hipEventDestroy(start);
+    (void)hipEventDestroy(stop);
+    if (err != hipSuccess) return (int)err;
+    if (best < 0) return NINETOOTHED_NO_KERNEL;
+    {
+        std::unique_lock<std::shared_mutex> lock(g_tune_mutex);
+        g_tuned[make_key(q)] = best;
+    }
+    if (best_config) *best_config = best;
+    if (best_ms) *best_ms = best_time;
+    return 0;
+}
+
+NineToothedResult launch_nt_conv2d(NineToothedStream stream, NineToothedTensor input, NineToothedTensor filter,
+                                   NineToothedTensor output, int dtype, int padding_h, int padding_w, int block_size_m,
+                                   int block_size_n, int block_size_k) {
+    (void)block_size_m;
+    (void)block_size_n;
+    (void)block_size_k;
+    if (dtype != NINETOOTHED_FLOAT16 && dtype != NINETOOTHED_BFLOAT16) return NINETOOTHED_NO_KERNEL;
+    if (!input.shape || !filter.shape || !output.shape || !input.strides || !filter.strides || !output.strides)
+        return hipErrorInvalidValue;
+    if (padding_h < 0 || padding_w < 0) return hipErrorInvalidValue;
+    const int64_t N = (int64_t)input.shape[0], C = (int64_t)input.shape[1], H = (int64_t)input.shape[2], W = (int64_t)input.shape[3];
+    const int64_t K = (int64_t)filter.shape[0], R = (int64_t)filter.shape[2], S = (int64_t)filter.shape[3];
+    if ((int64_t)filter.shape[1] != C) return hipErrorInvalidValue;
+    const int64_t P = H + 2 * padding_h - R + 1, Q = W + 2 * padding_w - S + 1;
+    if ((int64_t)output.shape[0] != N || (int64_t)output.shape[1] != K) return hipErrorInvalidValue;
+    if ((int64_t)output.shape[2] != P || (int64_t)output.shape[3] != Q) return hipErrorInvalidValue;
+    if (P <= 0 || Q <= 0 || N == 0 || K == 0) return 0;  // nothing to write
+    const int64_t gm = N * P * Q, gk = C * R * S;
+    if (gm > 0x7fffffffll || gk > 0x7fffffffll || K > 0x7fffffffll) return NINETOOTHED_NO_KERNEL;
+    auto launch = [&](auto tag) -> hipError_t {
+        typedef decltype(tag) T;
+        Conv2dProblem<T> prob;
+        prob.m = (int)gm;
+        prob.n = (int)K;
+        prob.k = (int)gk;
+        prob.x = (const T *)input.data;
+        prob.w = (const T *)filter.data;
+        prob.y = (T *)output.data;
+        prob.C = (int)C;
+        prob.H = (int)H;
+        prob.W = (int)W;
+        prob.R = (int)R;
+        prob.S = (int)S;
+        prob.P = (int)P;
+        prob.Q = (int)Q;
+        prob.pad_h = padding_h;
+        prob.pad_w = padding_w;
+        for (int d = 0; d < 4; ++d) {
+            prob.xs[d] = input.strides[d];
+            prob.ws[d] = filter.strides[d];
+            prob.ys[d] = output.strides[d];
+        }
+        const int64_t tiles = (int64_t)ceil_div(prob.m, kGenBM) * ceil_div(prob.n, kGenBN);
+        gemm_generic_kernel<Conv2dProblem<T>><<<dim3((unsigned)tiles), dim3(kGenThreads), 0, (hipStream_t)stream>>>(prob);
+        return hipGetLastError();
+    };
+    if (dtype == NINETOOTHED_FLOAT16) return (int)launch(half_t());
+    return (int)launch(bf16_t());
+}
+
+#ifdef NT_GEMM_ABLATION
+void nt_debug_set_tile_order(int order) { g_tile_order = order; }
+#endif
+
+const char *nt_version(void) { return "nt_hip 0.1 gfx950"; }
+
+}  // extern "C"

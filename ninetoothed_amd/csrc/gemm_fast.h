@@ -1,0 +1,405 @@
+// Tiled GEMM for gfx950: C[M,N] = A[M,K] @ B[K,N] (+ addmm epilogue), fp16/bf16
+// inputs, fp32 accumulation on 32x32x16 MFMA.
+//
+// Fast path requirements (checked on the host before launch):
+//   A row-major with unit K stride, B row-major with unit N stride, C with unit
+//   N stride and the element type of A/B; M % BM == 0, N % BN == 0, K % BK == 0;
+//   row pitches and base addresses multiples of 16 bytes.
+//
+// Data movement per workgroup and K step:
+//   HBM/L2 --global_load_lds (16 B per lane, no registers)--> LDS stage
+//   LDS --ds_read_b128 (A) / ds_read_b64_tr_b16 (B)--> MFMA operand registers
+// LDS tiles are XOR-swizzled at 16-byte granularity so both the row-wise A
+// reads and the transposing B reads spread over all 64 banks.
+#pragma once
+
+#include <type_traits>
+
+#include "nt_common.h"
+
+namespace nt {
+
+struct GemmParams {
+    const void *a;
+    const void *b;
+    void *c;
+    const void *bias;  // addmm `input`; nullptr for plain matmul
+    int m, n, k;
+    int64_t lda, ldb, ldc;            // row pitches in elements
+    int64_t bias_stride_m, bias_stride_n;
+    float alpha, beta;
+    int tiles_m, tiles_n;
+    int bias_vector;  // addmm input readable with aligned 16-byte loads along N
+    int order;  // tile order: 0 = XCD-aware strips of 8 tile rows; other values are measurement aids
+};
+
+// A tile [BM][BK]: rows of BK * 2 bytes, split into 16-byte chunks.  Rows that
+// share a 256-byte bank window get different chunk permutations.
+template <int BK>
+NT_HOST_DEVICE constexpr int a_phys_chunk(int row, int chunk) {
+    constexpr int kChunksPerRow = BK / 8;
+    constexpr int kRowsPerWindow = (256 / (BK * 2)) > 0 ? (256 / (BK * 2)) : 1;
+    return chunk ^ ((row / kRowsPerWindow) % kChunksPerRow);
+}
+
+// B tile [BK][BN]: a transposing read touches 4 consecutive k rows x 64 bytes;
+// shifting each row by a different multiple of 64 bytes separates them.
+template <int BN>
+NT_HOST_DEVICE constexpr int b_phys_chunk(int krow, int chunk) {
+    constexpr int kChunksPerRow = BN / 8;
+    constexpr int kMask = (kChunksPerRow / 4 - 1) < 7 ? (kChunksPerRow / 4 - 1) : 7;
+    return chunk ^ ((krow & kMask) << 2);
+}
+
+// Maps the hardware workgroup id to an output tile.  Workgroup ids are dealt
+// round-robin to the 8 XCDs, so ids congruent mod 8 share an L2: give each
+// XCD a contiguous range of tile ids, ordered in column strips of kGroupM
+// tile-rows so that concurrently running tiles reuse A and B panels in L2.
+NT_DEVICE void map_tile(int tiles_m, int tiles_n, int order, int &tile_m, int &tile_n) {
+    int bid = blockIdx.x;
+    const int nblocks = gridDim.x;
+    // order: low 8 bits = tile rows per strip (0 -> 8), bit 8 = skip the XCD remap
+    const int group_m = (order & 0xff) ? (order & 0xff) : 8;
+    if ((nblocks & 7) == 0 && !(order & 0x100)) {
+        const int per_xcd = nblocks >> 3;
+        bid = (bid & 7) * per_xcd + (bid >> 3);
+    }
+    const int group_size = group_m * tiles_n;
+    const int group = bid / group_size;
+    const int first_m = group * group_m;
+    const int rows = min(tiles_m - first_m, group_m);
+    const int in_group = bid - group * group_size;
+    tile_m = first_m + in_group % rows;
+    tile_n = in_group / rows;
+}
+
+template <int I, int N, typename F>
+NT_DEVICE void static_for(F &&f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>());
+        static_for<I + 1, N>(f);
+    }
+}
+
+// Workgroup barrier for the LDS ring.  Written as an opaque statement with a
+// memory clobber: the compiler moves no LDS access across it, and -- unlike a
+// workgroup fence -- it does not make the wave wait for its outstanding
+// global -> LDS fills of later stages (they are waited for explicitly with
+// wait_vmcnt<N>()).  Every wave has consumed (waited for) its own LDS reads of
+// the stage that is refilled next before it arrives here, because the MFMAs
+// using them precede the barrier in program order.
+NT_DEVICE void lds_barrier() { asm volatile("s_barrier" ::: "memory"); }
+
+// kAblate is a measurement aid (bit 0: no global loads inside the K loop,
+// bit 1: operand fragments read from LDS only once); 0 in every shipped instance.
+template <typename T, int BM, int BN, int BK, int WM, int WN, int kStages, int kWavesPerSimd, bool kAddmm, int kAblate = 0, int kLoad = 0, int kAux = 0>
+__global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kernel(GemmParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only builtins; the host pass only needs the stub
+    typedef Elem<T> E;
+    typedef typename E::vec8 vec8;
+    constexpr int kWaves = WM * WN;
+    constexpr int kWaveM = BM / WM;   // rows of C per wave
+    constexpr int kWaveN = BN / WN;   // cols of C per wave
+    constexpr int TM = kWaveM / 32;   // 32x32 MFMA tiles per wave along M
+    constexpr int TN = kWaveN / 32;
+    constexpr int kStageA = BM * BK * 2;  // bytes
+    constexpr int kStageB = BK * BN * 2;
+    constexpr int kAChunksPerRow = BK / 8;
+    constexpr int kARowsPerInstr = 64 / kAChunksPerRow;
+    constexpr int kAInstr = kStageA / (kWaves * 1024);
+    constexpr int kBChunksPerRow = BN / 8;
+    constexpr int kBRowsPerInstr = 64 / kBChunksPerRow > 0 ? 64 / kBChunksPerRow : 1;
+    constexpr int kBInstr = kStageB / (kWaves * 1024);
+    constexpr int kLoadsPerTile = kAInstr + kBInstr;
+    static_assert(kStageA % (kWaves * 1024) == 0 && kStageB % (kWaves * 1024) == 0, "tile/wave mismatch");
+    static_assert(kBChunksPerRow <= 64, "BN too large for one-instruction rows");
+    static_assert(kWaveM % 32 == 0 && kWaveN % 32 == 0 && BK % 16 == 0, "wave tile");
+    static_assert(kStages >= 2 && kStages <= 5, "2..5 stages");
+    static_assert((kStages - 2) * kLoadsPerTile < 64, "vmcnt range");
+
+    // One array per stage and operand: distinct LDS objects let the compiler prove
+    // that the asynchronous fill of one stage does not alias reads of another,
+    // so it does not wait for the fill before the MFMA operand reads.
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_a0[kStageA];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_a1[kStageA];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_a2[kStages > 2 ? kStageA : 16];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_a3[kStages > 3 ? kStageA : 16];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_a4[kStages > 4 ? kStageA : 16];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_b0[kStageB];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_b1[kStageB];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_b2[kStages > 2 ? kStageB : 16];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_b3[kStages > 3 ? kStageB : 16];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_b4[kStages > 4 ? kStageB : 16];
+    auto stage_a = [&](auto tag) -> NT_LDS unsigned char * {
+        constexpr int i = decltype(tag)::value;
+        if constexpr (i == 0) return (NT_LDS unsigned char *)lds_a0;
+        else if constexpr (i == 1) return (NT_LDS unsigned char *)lds_a1;
+        else if constexpr (i == 2) return (NT_LDS unsigned char *)lds_a2;
+        else if constexpr (i == 3) return (NT_LDS unsigned char *)lds_a3;
+        else return (NT_LDS unsigned char *)lds_a4;
+    };
+    auto stage_b = [&](auto tag) -> NT_LDS unsigned char * {
+        constexpr int i = decltype(tag)::value;
+        if constexpr (i == 0) return (NT_LDS unsigned char *)lds_b0;
+        else if constexpr (i == 1) return (NT_LDS unsigned char *)lds_b1;
+        else if constexpr (i == 2) return (NT_LDS unsigned char *)lds_b2;
+        else if constexpr (i == 3) return (NT_LDS unsigned char *)lds_b3;
+        else return (NT_LDS unsigned char *)lds_b4;
+    };
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_m = wave / WN;
+    const int wave_n = wave % WN;
+
+    int tile_m, tile_n;
+    map_tile(p.tiles_m, p.tiles_n, p.order, tile_m, tile_n);
+    const int m0 = tile_m * BM;
+    const int n0 = tile_n * BN;
+
+    const T *A = (const T *)p.a;
+    const T *B = (const T *)p.b;
+
+    // ---- global -> LDS assignments (per lane, fixed over the K loop) ----
+    // Byte offsets relative to the tile's first A row / B column stay below
+    // 2^31 (checked on the host), so addresses are a uniform base + 32-bit lane offset.
+    // A: instruction j of this wave fills rows [(j*kWaves+wave)*kARowsPerInstr, +kARowsPerInstr)
+    const unsigned char *a_base = (const unsigned char *)(A + (int64_t)m0 * p.lda);
+    const unsigned char *b_base = (const unsigned char *)(B + n0);
+    unsigned a_src[kAInstr];
+#pragma unroll
+    for (int j = 0; j < kAInstr; ++j) {
+        const int row = (j * kWaves + wave) * kARowsPerInstr + lane / kAChunksPerRow;
+        const int phys = lane % kAChunksPerRow;
+        const int chunk = a_phys_chunk<BK>(row, phys);  // XOR is an involution
+        a_src[j] = (unsigned)(row * (int)p.lda + chunk * 8) * 2u;
+    }
+    unsigned b_src[kBInstr];
+#pragma unroll
+    for (int j = 0; j < kBInstr; ++j) {
+        const int krow = (j * kWaves + wave) * kBRowsPerInstr + lane / kBChunksPerRow;
+        const int phys = lane % kBChunksPerRow;
+        const int chunk = b_phys_chunk<BN>(krow, phys);
+        b_src[j] = (unsigned)(krow * (int)p.ldb + chunk * 8) * 2u;
+    }
+
+    // kLoad 0: global_load_lds (64-bit base + lane offset); 1: buffer_load ... lds
+    // (buffer resource on the tile panel, 32-bit lane offset, scalar K offset)
+    __amdgpu_buffer_rsrc_t a_rsrc, b_rsrc;
+    if constexpr (kLoad == 1) {
+        a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)a_base, 0, 0xffffffff, 0x00020000);
+        b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)b_base, 0, 0xffffffff, 0x00020000);
+    }
+    auto issue_loads = [&](auto stage_tag, int kt) {
+        NT_LDS unsigned char *sa = stage_a(stage_tag);
+        NT_LDS unsigned char *sb = stage_b(stage_tag);
+        if constexpr (kLoad == 1) {
+            const int a_k = kt * BK * 2;
+            const int b_k = kt * BK * (int)p.ldb * 2;
+#pragma unroll
+            for (int j = 0; j < kAInstr; ++j)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, sa + (j * kWaves + wave) * 1024, 16, a_src[j], a_k, 0, kAux);
+#pragma unroll
+            for (int j = 0; j < kBInstr; ++j)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, sb + (j * kWaves + wave) * 1024, 16, b_src[j], b_k, 0, kAux);
+        } else {
+            const unsigned char *a_tile = a_base + (int64_t)kt * BK * 2;
+            const unsigned char *b_tile = b_base + (int64_t)kt * BK * p.ldb * 2;
+#pragma unroll
+            for (int j = 0; j < kAInstr; ++j)
+                __builtin_amdgcn_global_load_lds((const NT_GLOBAL void *)(a_tile + a_src[j]), sa + (j * kWaves + wave) * 1024, 16, 0, kAux);
+#pragma unroll
+            for (int j = 0; j < kBInstr; ++j)
+                __builtin_amdgcn_global_load_lds((const NT_GLOBAL void *)(b_tile + b_src[j]), sb + (j * kWaves + wave) * 1024, 16, 0, kAux);
+        }
+    };
+
+    // ---- LDS -> register read offsets (bytes, within a stage) ----
+    const int g = lane >> 5;        // k half of the MFMA operand this lane holds
+    const int l32 = lane & 31;
+    int a_row_off[TM];              // byte offset of this lane's A row
+    int a_row_sw[TM];               // swizzle term of that row
+#pragma unroll
+    for (int ti = 0; ti < TM; ++ti) {
+        const int row = wave_m * kWaveM + ti * 32 + l32;
+        a_row_off[ti] = row * (BK * 2);
+        a_row_sw[ti] = a_phys_chunk<BK>(row, 0);
+    }
+    // B (transposing read): lane i of a 16-lane group addresses row i/4,
+    // columns 4*(i%4).. of the group's 4(k) x 16(n) block.
+    const int i16 = lane & 15;
+    const int nhalf = (lane >> 4) & 1;
+    const int b_krow = 8 * g + (i16 >> 2);  // + 16*ks (+4 for the upper half)
+    int b_col_chunk[TN];                    // 16-byte chunk index of the column
+    int b_col_in[TN];                       // byte offset inside the chunk
+#pragma unroll
+    for (int tj = 0; tj < TN; ++tj) {
+        const int ncol = wave_n * kWaveN + tj * 32 + nhalf * 16 + 4 * (i16 & 3);
+        b_col_chunk[tj] = ncol >> 3;
+        b_col_in[tj] = (ncol & 7) * 2;
+    }
+
+    float16_t acc[TM][TN];
+#pragma unroll
+    for (int ti = 0; ti < TM; ++ti)
+#pragma unroll
+        for (int tj = 0; tj < TN; ++tj)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[ti][tj][r] = 0.0f;
+
+    auto read_frags = [&](auto stage_tag, int ks, vec8 (&af)[TM], vec8 (&bf)[TN]) {
+        const NT_LDS unsigned char *sa = stage_a(stage_tag);
+        const NT_LDS unsigned char *sb = stage_b(stage_tag);
+#pragma unroll
+        for (int ti = 0; ti < TM; ++ti) {
+            const int chunk = (ks * 2 + g) ^ a_row_sw[ti];
+            af[ti] = *(const NT_LDS vec8 *)(sa + a_row_off[ti] + chunk * 16);
+        }
+#pragma unroll
+        for (int tj = 0; tj < TN; ++tj) {
+            const int k_lo = ks * 16 + b_krow;
+            const int k_hi = k_lo + 4;
+            const int c_lo = b_phys_chunk<BN>(k_lo, b_col_chunk[tj]);
+            const int c_hi = b_phys_chunk<BN>(k_hi, b_col_chunk[tj]);
+            short4_t lo = lds_read_tr16_b64(sb + k_lo * (BN * 2) + c_lo * 16 + b_col_in[tj]);
+            short4_t hi = lds_read_tr16_b64(sb + k_hi * (BN * 2) + c_hi * 16 + b_col_in[tj]);
+            short8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            bf[tj] = __builtin_bit_cast(vec8, both);
+        }
+    };
+
+    vec8 af_once[TM];
+    vec8 bf_once[TN];
+
+    auto multiply_stage = [&](auto stage_tag) {
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            vec8 af[TM];
+            vec8 bf[TN];
+            if constexpr (kAblate & 2) {
+#pragma unroll
+                for (int ti = 0; ti < TM; ++ti) af[ti] = af_once[ti];
+#pragma unroll
+                for (int tj = 0; tj < TN; ++tj) bf[tj] = bf_once[tj];
+            } else {
+                read_frags(stage_tag, ks, af, bf);
+            }
+#pragma unroll
+            for (int ti = 0; ti < TM; ++ti)
+#pragma unroll
+                for (int tj = 0; tj < TN; ++tj) acc[ti][tj] = E::mfma32(bf[tj], af[ti], acc[ti][tj]);  // transposed tile
+        }
+    };
+
+    // K loop, unrolled over the stages so every LDS array is named statically.
+    // Step for tile t: wait until tile t has landed, barrier (which also tells
+    // that all waves finished tile t-1), refill the stage tile t-1 used with
+    // tile t+kStages-1, multiply tile t.  Past the end the last tile is fetched
+    // again into a stage nobody reads, which keeps the outstanding-load count
+    // the same in every step.
+    const int num_k = p.k / BK;
+    const int last_k = num_k - 1;
+    const int main_k = num_k - num_k % kStages;
+
+    static_for<0, kStages - 1>([&](auto s) { issue_loads(s, min((int)decltype(s)::value, last_k)); });
+    if constexpr (kAblate & 2) {
+        wait_vmcnt<0>();
+        lds_barrier();
+        read_frags(std::integral_constant<int, 0>(), 0, af_once, bf_once);
+    }
+    auto step = [&](auto s, int kt) {
+        constexpr int kS = decltype(s)::value;
+        wait_vmcnt<(kAblate & 1) ? 0 : (kStages - 2) * kLoadsPerTile>();
+        lds_barrier();
+        if constexpr (!(kAblate & 1))
+            issue_loads(std::integral_constant<int, (kS + kStages - 1) % kStages>(), min(kt + kS + kStages - 1, last_k));
+        multiply_stage(s);
+    };
+    for (int kt = 0; kt < main_k; kt += kStages) {
+        static_for<0, kStages>([&](auto s) { step(s, kt); });
+    }
+    // remaining num_k % kStages tiles continue the stage rotation
+    static_for<0, kStages - 1>([&](auto s) {
+        if (main_k + (int)decltype(s)::value < num_k) step(s, main_k);
+    });
+
+    // ---- epilogue ----
+    // The accumulators hold C transposed per 32x32 tile: lane (l32, g) has, in
+    // registers 4*r4 .. 4*r4+3, the columns 8*r4 + 4*g .. +3 of row l32.  Each
+    // wave passes its tile through its own LDS slab 32 rows at a time, so that
+    // global stores (and addmm input loads) are 16 bytes per lane and cover
+    // whole 128-byte lines.  (All fills have landed and all waves are done with
+    // the stages before the slabs overwrite them.)
+    constexpr int kRowBytes = kWaveN * 2;
+    constexpr int kCChunks = kWaveN / 8;  // 16-byte chunks per slab row
+    constexpr int kCShift = kRowBytes >= 256 ? 0 : (kRowBytes == 128 ? 1 : 2);
+    // the slabs live in the (now idle) stage memory: A0, B0, A1, B1 in this order
+    constexpr int kSlabBytes = 32 * kRowBytes;
+    constexpr int kSlabsA = kStageA / kSlabBytes;
+    constexpr int kSlabsB = kStageB / kSlabBytes;
+    static_assert(kWaves <= 2 * (kSlabsA + kSlabsB), "epilogue slabs do not fit two stages");
+    wait_vmcnt<0>();
+    lds_barrier();
+    NT_LDS unsigned char *slab;
+    {
+        int w = wave;
+        if (w < kSlabsA) {
+            slab = (NT_LDS unsigned char *)lds_a0;
+        } else if ((w -= kSlabsA) < kSlabsB) {
+            slab = (NT_LDS unsigned char *)lds_b0;
+        } else if ((w -= kSlabsB) < kSlabsA) {
+            slab = (NT_LDS unsigned char *)lds_a1;
+        } else {
+            w -= kSlabsA;
+            slab = (NT_LDS unsigned char *)lds_b1;
+        }
+        slab += w * kSlabBytes;
+    }
+    T *C = (T *)p.c;
+    const T *bias = (const T *)p.bias;
+    const int slab_sw = (l32 >> kCShift) & (kCChunks - 1);
+#pragma unroll
+    for (int ti = 0; ti < TM; ++ti) {
+#pragma unroll
+        for (int tj = 0; tj < TN; ++tj) {
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                typedef T vec4 __attribute__((ext_vector_type(4)));
+                vec4 v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = E::from_float(acc[ti][tj][4 * r4 + e]);
+                const int chunk = (tj * 4 + r4) ^ slab_sw;
+                *(NT_LDS vec4 *)(slab + l32 * kRowBytes + chunk * 16 + 8 * g) = v;
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < kCChunks / 2; ++it) {
+            const int idx = it * 64 + lane;
+            const int row = idx / kCChunks;
+            const int phys = idx % kCChunks;
+            const int chunk = phys ^ ((row >> kCShift) & (kCChunks - 1));
+            vec8 v = *(const NT_LDS vec8 *)(slab + row * kRowBytes + phys * 16);
+            const int grow = m0 + wave_m * kWaveM + ti * 32 + row;
+            const int gcol = n0 + wave_n * kWaveN + chunk * 8;
+            if constexpr (kAddmm) {
+                // the matmul result was rounded to the element type; beta, alpha
+                // are fp32 scalars, so the combination happens in fp32
+                const T *src = bias + (int64_t)grow * p.bias_stride_m + (int64_t)gcol * p.bias_stride_n;
+                vec8 in;
+                if (p.bias_vector) {
+                    in = *(const vec8 *)src;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) in[e] = src[(int64_t)e * p.bias_stride_n];
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] = E::from_float(p.beta * E::to_float(in[e]) + p.alpha * E::to_float(v[e]));
+            }
+            *(vec8 *)(C + (int64_t)grow * p.ldc + gcol) = v;
+        }
+    }
+#endif
+}
+
+}  // namespace nt

@@ -1,0 +1,293 @@
+// Row softmax for gfx950.  Bandwidth-bound: every element is read once and
+// written once; a row (or row segment) lives in registers between the two.
+//
+// A "segment" is what one program of the arrange-and-apply softmax handles:
+// columns [s * block, min((s + 1) * block, N)) of one row.  With block >= N
+// (the usual call) a segment is a whole row.
+#include "nt_common.h"
+
+namespace nt {
+namespace {
+
+struct SoftmaxParams {
+    const void *in;
+    void *out;
+    int64_t rows, cols;
+    int64_t in_row_stride, in_col_stride, out_row_stride, out_col_stride;
+    int64_t block;      // segment length
+    int64_t segments;   // per row
+};
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+NT_DEVICE float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+NT_DEVICE float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+// Reduction over the kRowThreads threads that share a segment.  For 64 it is a
+// pure wave reduction; for more, partial results cross waves through LDS.
+template <int kRowThreads, bool kIsMax>
+NT_DEVICE float group_reduce(float v, float *scratch) {
+    v = kIsMax ? wave_max(v) : wave_sum(v);
+    if constexpr (kRowThreads > 64) {
+        constexpr int kWaves = kRowThreads / 64;
+        const int wave = threadIdx.x >> 6;
+        __syncthreads();  // scratch may still be read from a previous reduction
+        if ((threadIdx.x & 63) == 0) scratch[wave] = v;
+        __syncthreads();
+        v = scratch[0];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) v = kIsMax ? fmaxf(v, scratch[w]) : v + scratch[w];
+    }
+    return v;
+}
+
+template <typename T>
+struct Vec16 {  // 16 bytes of T
+    static constexpr int kWidth = 16 / sizeof(T);
+    typedef T type __attribute__((ext_vector_type(16 / sizeof(T))));
+};
+
+// Vector path: unit column strides, 16-byte aligned segments whose length is a
+// multiple of the vector width.  Thread t of a segment's group owns vectors
+// t, t + kRowThreads, ...  (coalesced 16-byte accesses).
+template <typename T, int kRowThreads, int kVecs>
+__global__ __launch_bounds__(256) void softmax_vec_kernel(SoftmaxParams p) {
+    typedef typename Vec16<T>::type vec_t;
+    constexpr int W = Vec16<T>::kWidth;
+    constexpr int kGroups = 256 / kRowThreads;  // segments per workgroup
+    __shared__ float scratch[4];
+
+    const int group = threadIdx.x / kRowThreads;
+    const int t = threadIdx.x % kRowThreads;
+    const int64_t seg = (int64_t)blockIdx.x * kGroups + group;
+    const int64_t total = p.rows * p.segments;
+    // whole groups leave together, so the barriers below stay uniform (kGroups == 1 when they exist)
+    const bool active = seg < total;
+    const int64_t row = active ? seg / p.segments : 0;
+    const int64_t start = active ? (seg % p.segments) * p.block : 0;
+    const int len = active ? (int)min(p.block, p.cols - start) : 0;
+    const int nvec = len / W;
+
+    const T *src = (const T *)p.in + row * p.in_row_stride + start;
+    T *dst = (T *)p.out + row * p.out_row_stride + start;
+
+    float x[kVecs][W];
+    float m = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < kVecs; ++j) {
+        const int v = j * kRowThreads + t;
+        if (v < nvec) {
+            vec_t raw = __builtin_nontemporal_load((const vec_t *)src + v);
+#pragma unroll
+            for (int e = 0; e < W; ++e) {
+                x[j][e] = (float)raw[e];
+                m = fmaxf(m, x[j][e]);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < W; ++e) x[j][e] = -INFINITY;
+        }
+    }
+    m = group_reduce<kRowThreads, true>(m, scratch);
+    const float shift = m * kLog2e;
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kVecs; ++j)
+#pragma unroll
+        for (int e = 0; e < W; ++e) {
+            // exp(x - m) as exp2(x * log2e - m * log2e); padding (-inf) gives 0
+            x[j][e] = __builtin_amdgcn_exp2f(fmaf(x[j][e], kLog2e, -shift));
+            s += x[j][e];
+        }
+    s = group_reduce<kRowThreads, false>(s, scratch);
+    const float inv = 1.0f / s;
+#pragma unroll
+    for (int j = 0; j < kVecs; ++j) {
+        const int v = j * kRowThreads + t;
+        if (v < nvec) {
+            vec_t o;
+#pragma unroll
+            for (int e = 0; e < W; ++e) o[e] = (T)(x[j][e] * inv);
+            __builtin_nontemporal_store(o, (vec_t *)dst + v);
+        }
+    }
+}
+
+// Element path: any strides / alignment / length up to kRowThreads * kElems.
+template <typename T, int kRowThreads, int kElems>
+__global__ __launch_bounds__(256) void softmax_elem_kernel(SoftmaxParams p) {
+    constexpr int kGroups = 256 / kRowThreads;
+    __shared__ float scratch[4];
+
+    const int group = threadIdx.x / kRowThreads;
+    const int t = threadIdx.x % kRowThreads;
+    const int64_t seg = (int64_t)blockIdx.x * kGroups + group;
+    const int64_t total = p.rows * p.segments;
+    const bool active = seg < total;
+    const int64_t row = active ? seg / p.segments : 0;
+    const int64_t start = active ? (seg % p.segments) * p.block : 0;
+    const int len = active ? (int)min(p.block, p.cols - start) : 0;
+
+    const T *src = (const T *)p.in + row * p.in_row_stride + start * p.in_col_stride;
+    T *dst = (T *)p.out + row * p.out_row_stride + start * p.out_col_stride;
+
+    float x[kElems];
+    float m = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < kElems; ++j) {
+        const int c = j * kRowThreads + t;
+        x[j] = c < len ? (float)src[(int64_t)c * p.in_col_stride] : -INFINITY;
+        m = fmaxf(m, x[j]);
+    }
+    m = group_reduce<kRowThreads, true>(m, scratch);
+    const float shift = m * kLog2e;
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kElems; ++j) {
+        x[j] = __builtin_amdgcn_exp2f(fmaf(x[j], kLog2e, -shift));
+        s += x[j];
+    }
+    s = group_reduce<kRowThreads, false>(s, scratch);
+    const float inv = 1.0f / s;
+#pragma unroll
+    for (int j = 0; j < kElems; ++j) {
+        const int c = j * kRowThreads + t;
+        if (c < len) dst[(int64_t)c * p.out_col_stride] = (T)(x[j] * inv);
+    }
+}
+
+// Long segments: one workgroup per segment, three sweeps over memory (max, sum,
+// write); the second and third sweeps hit L2 for segments that fit there.
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_loop_kernel(SoftmaxParams p) {
+    __shared__ float scratch[4];
+    const int64_t seg = blockIdx.x;
+    const int64_t row = seg / p.segments;
+    const int64_t start = (seg % p.segments) * p.block;
+    const int64_t len = min(p.block, p.cols - start);
+    const T *src = (const T *)p.in + row * p.in_row_stride + start * p.in_col_stride;
+    T *dst = (T *)p.out + row * p.out_row_stride + start * p.out_col_stride;
+
+    float m = -INFINITY;
+    for (int64_t c = threadIdx.x; c < len; c += 256) m = fmaxf(m, (float)src[c * p.in_col_stride]);
+    m = group_reduce<256, true>(m, scratch);
+    const float shift = m * kLog2e;
+    float s = 0.0f;
+    for (int64_t c = threadIdx.x; c < len; c += 256)
+        s += __builtin_amdgcn_exp2f(fmaf((float)src[c * p.in_col_stride], kLog2e, -shift));
+    s = group_reduce<256, false>(s, scratch);
+    const float inv = 1.0f / s;
+    for (int64_t c = threadIdx.x; c < len; c += 256)
+        dst[c * p.out_col_stride] = (T)(__builtin_amdgcn_exp2f(fmaf((float)src[c * p.in_col_stride], kLog2e, -shift)) * inv);
+}
+
+template <typename T, int kRowThreads>
+hipError_t launch_vec(const SoftmaxParams &p, int vecs_needed, hipStream_t stream) {
+    const int64_t total = p.rows * p.segments;
+    constexpr int kGroups = 256 / kRowThreads;
+    const dim3 grid((unsigned)((total + kGroups - 1) / kGroups)), block(256);
+    if (vecs_needed <= 1)
+        softmax_vec_kernel<T, kRowThreads, 1><<<grid, block, 0, stream>>>(p);
+    else if (vecs_needed <= 2)
+        softmax_vec_kernel<T, kRowThreads, 2><<<grid, block, 0, stream>>>(p);
+    else if (vecs_needed <= 4)
+        softmax_vec_kernel<T, kRowThreads, 4><<<grid, block, 0, stream>>>(p);
+    else if (vecs_needed <= 8)
+        softmax_vec_kernel<T, kRowThreads, 8><<<grid, block, 0, stream>>>(p);
+    else
+        softmax_vec_kernel<T, kRowThreads, 16><<<grid, block, 0, stream>>>(p);
+    return hipGetLastError();
+}
+
+template <typename T, int kRowThreads>
+hipError_t launch_elem(const SoftmaxParams &p, int elems_needed, hipStream_t stream) {
+    const int64_t total = p.rows * p.segments;
+    constexpr int kGroups = 256 / kRowThreads;
+    const dim3 grid((unsigned)((total + kGroups - 1) / kGroups)), block(256);
+    if (elems_needed <= 4)
+        softmax_elem_kernel<T, kRowThreads, 4><<<grid, block, 0, stream>>>(p);
+    else if (elems_needed <= 16)
+        softmax_elem_kernel<T, kRowThreads, 16><<<grid, block, 0, stream>>>(p);
+    else
+        softmax_elem_kernel<T, kRowThreads, 64><<<grid, block, 0, stream>>>(p);
+    return hipGetLastError();
+}
+
+// `variant`: 0 = library's choice, 1 = one wave per segment, 2 = one workgroup per segment
+template <typename T>
+int run_softmax(const SoftmaxParams &p, int variant, hipStream_t stream) {
+    constexpr int W = Vec16<T>::kWidth;
+    const int64_t total = p.rows * p.segments;
+    if (total == 0 || p.cols == 0) return 0;
+    if (total > 0x7fffffffll) return NINETOOTHED_NO_KERNEL;
+    const int64_t len = p.block < p.cols ? p.block : p.cols;
+    const bool vector_ok = p.in_col_stride == 1 && p.out_col_stride == 1 && p.cols % W == 0 &&
+                           (p.segments == 1 || p.block % W == 0) && p.in_row_stride % W == 0 &&
+                           p.out_row_stride % W == 0 && ((uintptr_t)p.in & 15) == 0 && ((uintptr_t)p.out & 15) == 0;
+    if (vector_ok && len <= (int64_t)256 * 16 * W) {
+        const bool wave_fits = len <= (int64_t)64 * 16 * W;
+        bool use_wave = wave_fits && len <= (int64_t)64 * 8 * W;  // default: keep <= 8 vectors per lane
+        if (variant == 1 && wave_fits) use_wave = true;
+        if (variant == 2) use_wave = false;
+        if (use_wave) return (int)launch_vec<T, 64>(p, (int)((len / W + 63) / 64), stream);
+        return (int)launch_vec<T, 256>(p, (int)((len / W + 255) / 256), stream);
+    }
+    if (len <= 64 * 16) return (int)launch_elem<T, 64>(p, (int)((len + 63) / 64), stream);
+    if (len <= 256 * 64) return (int)launch_elem<T, 256>(p, (int)((len + 255) / 256), stream);
+    softmax_loop_kernel<T><<<dim3((unsigned)total), dim3(256), 0, stream>>>(p);
+    return (int)hipGetLastError();
+}
+
+int softmax_entry(NineToothedStream stream, const NineToothedTensor &input, const NineToothedTensor &output, int dtype,
+                  int block_size, int variant) {
+    if (!input.shape || !output.shape || !input.strides || !output.strides) return hipErrorInvalidValue;
+    if (input.shape[0] != output.shape[0] || input.shape[1] != output.shape[1]) return hipErrorInvalidValue;
+    SoftmaxParams p;
+    p.in = input.data;
+    p.out = output.data;
+    p.rows = (int64_t)input.shape[0];
+    p.cols = (int64_t)input.shape[1];
+    p.in_row_stride = input.strides[0];
+    p.in_col_stride = input.strides[1];
+    p.out_row_stride = output.strides[0];
+    p.out_col_stride = output.strides[1];
+    p.block = block_size > 0 ? block_size : (p.cols > 0 ? p.cols : 1);
+    p.segments = p.cols > 0 ? (p.cols + p.block - 1) / p.block : 0;
+    switch (dtype) {
+        case NINETOOTHED_FLOAT32:
+            return run_softmax<float>(p, variant, (hipStream_t)stream);
+        case NINETOOTHED_FLOAT16:
+            return run_softmax<half_t>(p, variant, (hipStream_t)stream);
+        case NINETOOTHED_BFLOAT16:
+            return run_softmax<bf16_t>(p, variant, (hipStream_t)stream);
+        default:
+            return NINETOOTHED_NO_KERNEL;
+    }
+}
+
+}  // namespace
+}  // namespace nt
+
+extern "C" {
+
+NineToothedResult launch_nt_softmax(NineToothedStream stream, NineToothedTensor input, NineToothedTensor output,
+                                    int dtype, int block_size) {
+    return nt::softmax_entry(stream, input, output, dtype, block_size, 0);
+}
+
+NineToothedResult launch_nt_softmax_config(NineToothedStream stream, int config, NineToothedTensor input,
+                                           NineToothedTensor output, int dtype, int block_size) {
+    if (config < 0 || config > 2) return NINETOOTHED_NO_KERNEL;
+    return nt::softmax_entry(stream, input, output, dtype, block_size, config);
+}
+
+}  // extern "C"
