@@ -1,0 +1,330 @@
+"""``make`` and ``jit``: bind an arrangement to an application and return a
+callable on torch tensors.
+
+Same surface as the reference (src/ninetoothed/make.py:7-56,
+src/ninetoothed/jit.py:8-128): ``make(arrangement, application, tensors)`` runs
+the arrangement on the symbolic tensors and pairs its results with the
+application's parameters by position; ``jit`` takes them from the parameter
+annotations.  The returned kernel is called with one argument per application
+parameter, in order (torch tensors; Python numbers for zero-dimensional
+tensors) plus the arrangement's call-time constants by keyword (for example
+``BLOCK_SIZE=``, ``padding_h=``); it writes its outputs in place and returns
+``None`` (launch convention: src/ninetoothed/generation.py:518-600).
+
+Instead of generating and compiling code, the kernel object recognises the
+program (:mod:`ninetoothed_amd.recognition`) and, per distinct combination of
+shapes / strides / dtypes, prepares a launch plan for ``libnt_hip.so``.
+"""
+
+import hashlib
+import inspect
+import pathlib
+
+from ninetoothed_amd import recognition, runtime
+from ninetoothed_amd.recognition import UnsupportedProgram
+from ninetoothed_amd.symbol import Symbol
+from ninetoothed_amd.tensor import Tensor
+
+CACHE_DIR = pathlib.Path.home() / ".ninetoothed_amd"
+
+_TORCH_DTYPE_TAGS = None
+
+
+def _dtype_tag(torch_dtype):
+    global _TORCH_DTYPE_TAGS
+    if _TORCH_DTYPE_TAGS is None:
+        import torch
+
+        _TORCH_DTYPE_TAGS = {
+            torch.int8: "i8",
+            torch.int16: "i16",
+            torch.int32: "i32",
+            torch.int64: "i64",
+            torch.uint8: "u8",
+            torch.float16: "fp16",
+            torch.bfloat16: "bf16",
+            torch.float32: "fp32",
+            torch.float64: "fp64",
+        }
+    try:
+        return _TORCH_DTYPE_TAGS[torch_dtype]
+    except KeyError:
+        raise UnsupportedProgram(f"Element type `{torch_dtype}` is not supported.") from None
+
+
+def make(
+    arrangement,
+    application,
+    tensors,
+    caller="torch",
+    kernel_name=None,
+    output_dir=None,
+    num_warps=None,
+    num_stages=None,
+    max_num_configs=None,
+):
+    """Integrates the arrangement and the application of the tensors.
+
+    :param arrangement: The arrangement of the tensors.
+    :param application: The application of the tensors.
+    :param tensors: The tensors.
+    :param caller: Who will call the compute kernel; only ``"torch"``.
+    :param kernel_name: The name for the kernel.
+    :param output_dir: Unused (no files are generated for ``"torch"``).
+    :param num_warps: Accepted for compatibility; wave counts belong to the
+        hand-written kernels.
+    :param num_stages: Accepted for compatibility; see ``num_warps``.
+    :param max_num_configs: Accepted for compatibility; tile selection is
+        done inside the library.
+    :return: A handle to the compute kernel.
+    """
+
+    if caller != "torch":
+        raise NotImplementedError("Only `caller=\"torch\"` is supported; ahead-of-time packaging is not part of this build.")
+    types = arrangement(*tensors)
+    types = types if isinstance(types, tuple) else (types,)
+    return Kernel(application, types, kernel_name=kernel_name)
+
+
+def jit(func=None, *, caller="torch", kernel_name=None, num_warps=None, num_stages=None, max_num_configs=None, _prettify=False):
+    """A decorator that builds a kernel from a function whose parameter
+    annotations are arranged tensors."""
+
+    if caller != "torch":
+        raise NotImplementedError("Only `caller=\"torch\"` is supported.")
+
+    def wrapper(function):
+        annotations = inspect.get_annotations(function) if hasattr(inspect, "get_annotations") else function.__annotations__
+        parameters = inspect.signature(function).parameters
+        try:
+            types = tuple(annotations[name] for name in parameters)
+        except KeyError as error:
+            raise TypeError(f"Parameter `{error.args[0]}` has no arranged tensor as its annotation.") from None
+        return Kernel(function, types, kernel_name=kernel_name)
+
+    if func is None:
+        return wrapper
+    return wrapper(func)
+
+
+class Kernel:
+    """A compute kernel bound to hand-written gfx950 code."""
+
+    def __init__(self, application, types, kernel_name=None):
+        self.application = application
+        self.types = tuple(types)
+        self.kernel_name = kernel_name if kernel_name is not None else getattr(application, "__name__", "kernel")
+        self.kind, self.details, self.program = recognition.identify(application, self.types)
+        self.parameters = list(inspect.signature(application).parameters)
+        self.meta_symbols = recognition.unbound_meta_symbols(self.types)
+        self._plans = {}
+        self._source_path = None
+        self.last_plan = None  # description of the launch used by the latest call
+
+    # `_source` mirrors the reference handle's attribute (src/ninetoothed/jit.py:121-125):
+    # a path to a readable description of what runs
+    @property
+    def _source(self):
+        if self._source_path is None:
+            text = (
+                f"# kernel `{self.kernel_name}`: recognised as `{self.kind}` {self.details}\n"
+                f"# executed by libnt_hip.so ({runtime.LIBRARY_PATH})\n"
+                f"# dataflow graph of the application (digest {self.program.digest}):\n" + self.program.describe() + "\n"
+            )
+            CACHE_DIR.mkdir(parents=True, exist_ok=True)
+            path = CACHE_DIR / (hashlib.sha256(text.encode()).hexdigest() + ".txt")
+            if not path.exists():
+                path.write_text(text)
+            self._source_path = str(path)
+        return self._source_path
+
+    def __call__(self, *args, **kwargs):
+        if len(args) != len(self.types):
+            raise TypeError(f"`{self.kernel_name}` takes {len(self.types)} positional arguments but {len(args)} were given.")
+        key = self._signature(args, kwargs)
+        plan = self._plans.get(key)
+        if plan is None:
+            plan = self._plans[key] = self._prepare(args, kwargs)
+        self.last_plan = plan.description
+        plan(args)
+
+    # ---- plan construction ----------------------------------------------
+    def _signature(self, args, kwargs):
+        parts = []
+        for arg, tensor in zip(args, self.types):
+            if tensor.ndim == 0 and not isinstance(tensor.dtype, Tensor):
+                parts.append((type(arg).__name__, arg if tensor.constexpr else None))
+            else:
+                parts.append((tuple(arg.shape), tuple(arg.stride()), arg.dtype, arg.device.index))
+        return tuple(parts), tuple(sorted(kwargs.items()))
+
+    def _environment(self, args, kwargs):
+        import torch
+
+        env = {}
+        for name, arg, tensor in zip(self.parameters, args, self.types):
+            source = tensor.source
+            if tensor.ndim == 0 and not isinstance(tensor.dtype, Tensor):
+                if isinstance(arg, torch.Tensor):
+                    raise TypeError(f"`{name}` is a zero-dimensional tensor: pass a Python number.")
+                continue
+            if not isinstance(arg, torch.Tensor):
+                raise TypeError(f"`{name}` must be a torch tensor, not `{type(arg).__name__}`.")
+            if not arg.is_cuda:
+                raise RuntimeError(f"`{name}` lives on `{arg.device}`; this build only runs on the GPU (there is no CPU path).")
+            if arg.ndim != source.ndim:
+                raise ValueError(f"`{name}` must have {source.ndim} dimensions, got {arg.ndim}.")
+            for dim in range(source.ndim):
+                declared = source.shape[dim]
+                if not isinstance(declared, Symbol) and int(declared) != arg.shape[dim]:
+                    raise ValueError(f"Dimension {dim} of `{name}` was declared as {declared}, got {arg.shape[dim]}.")
+                if isinstance(declared, Symbol) and declared.is_name:
+                    env[declared.name] = arg.shape[dim]
+                env[source.size_string(dim)] = arg.shape[dim]
+                env[source.stride_string(dim)] = arg.stride(dim)
+        for name, value in kwargs.items():
+            env[name] = value
+        for name in self.meta_symbols:
+            env.setdefault(name, 1)  # index maps do not depend on block sizes; analyse with unit blocks
+        return env
+
+    def _prepare(self, args, kwargs):
+        env = self._environment(args, kwargs)
+        try:
+            builder = getattr(self, "_prepare_" + self.kind)
+            return builder(args, env)
+        except KeyError as error:
+            raise TypeError(f"`{self.kernel_name}` needs a value for {error.args[0]}; pass it by keyword.") from None
+
+    def _tensor_dtype(self, *tensors, allowed):
+        tags = {_dtype_tag(tensor.dtype) for tensor in tensors}
+        if len(tags) != 1:
+            raise UnsupportedProgram(f"Operands have different element types: {sorted(tags)}.")
+        (tag,) = tags
+        if tag not in allowed:
+            raise UnsupportedProgram(f"No `{self.kind}` kernel for element type `{tag}` (supported: {', '.join(allowed)}).")
+        return tag
+
+    def _prepare_matmul(self, args, env):
+        lhs, rhs, out = args
+        kind, info = recognition.analyze_gemm(self.types[0], self.types[1], self.types[2], env)
+        if kind == "empty":
+            return _Plan("empty launch", lambda call_args: None)
+        tag = self._tensor_dtype(lhs, rhs, allowed=("fp16", "bf16"))
+        out_tag = _dtype_tag(out.dtype)
+        cast = self.details.get("cast")
+        if kind == "conv2d":
+            if out_tag != tag or cast not in (None, tag):
+                raise UnsupportedProgram("conv2d needs input, filter and output of one element type.")
+            return self._conv2d_plan(info, tag)
+        if cast is not None and cast != out_tag:
+            raise UnsupportedProgram(f"The application rounds to `{cast}` but the output tensor holds `{out_tag}`.")
+        if out_tag not in (tag, "fp32"):
+            raise UnsupportedProgram(f"No matmul kernel writing `{out_tag}` from `{tag}` operands.")
+        return self._gemm_plan(info, tag, out_tag, positions=(None, 0, 1, None, None, 2))
+
+    def _prepare_addmm(self, args, env):
+        input, mat1, mat2, beta, alpha, out = args
+        kind, info = recognition.analyze_gemm(self.types[1], self.types[2], self.types[5], env, input_type=self.types[0])
+        if kind == "empty":
+            return _Plan("empty launch", lambda call_args: None)
+        tag = self._tensor_dtype(input, mat1, mat2, out, allowed=("fp16", "bf16"))
+        if self.details.get("cast") != tag:
+            raise UnsupportedProgram(f"The application rounds the product to `{self.details.get('cast')}` but the tensors hold `{tag}`.")
+        return self._gemm_plan(info, tag, tag, positions=(0, 1, 2, 3, 4, 5))
+
+    def _gemm_plan(self, info, tag, out_tag, positions):
+        lib = runtime.library()
+        itemsize = 2
+        out_itemsize = 4 if out_tag == "fp32" else 2
+        a, b, c, i = info["a"], info["b"], info["c"], info["input"]
+        m, n, k = info["m"], info["n"], info["k"]
+        blocks = [info["blocks"][axis] if info["blocks"][axis] > 1 else 0 for axis in ("m", "n", "k")]
+        dtype, out_dtype = runtime.DATA_TYPE_INDEX[tag], runtime.DATA_TYPE_INDEX[out_tag]
+        in_pos, a_pos, b_pos, beta_pos, alpha_pos, c_pos = positions
+        a_arg = runtime.ArgumentTensor.from_layout(0, (m, k), (a.row_stride, a.col_stride))
+        b_arg = runtime.ArgumentTensor.from_layout(0, (k, n), (b.row_stride, b.col_stride))
+        c_arg = runtime.ArgumentTensor.from_layout(0, (m, n), (c.row_stride, c.col_stride))
+        if i is not None:
+            i_arg = runtime.ArgumentTensor.from_layout(0, (m, n), (i.row_stride, i.col_stride))
+
+            def launch(call_args):
+                a_arg.data = call_args[a_pos].data_ptr() + a.base * itemsize
+                b_arg.data = call_args[b_pos].data_ptr() + b.base * itemsize
+                c_arg.data = call_args[c_pos].data_ptr() + c.base * out_itemsize
+                i_arg.data = call_args[in_pos].data_ptr() + i.base * itemsize
+                beta = runtime.ArgumentTensor.from_scalar(float(call_args[beta_pos]))
+                alpha = runtime.ArgumentTensor.from_scalar(float(call_args[alpha_pos]))
+                runtime.check(lib.launch_nt_addmm(runtime.current_stream(), i_arg, a_arg, b_arg, beta, alpha, c_arg, dtype, *blocks))
+
+            return _Plan(f"launch_nt_addmm {m}x{n}x{k} {tag} blocks {blocks}", launch)
+
+        def launch(call_args):
+            a_arg.data = call_args[a_pos].data_ptr() + a.base * itemsize
+            b_arg.data = call_args[b_pos].data_ptr() + b.base * itemsize
+            c_arg.data = call_args[c_pos].data_ptr() + c.base * out_itemsize
+            runtime.check(lib.launch_nt_matmul(runtime.current_stream(), a_arg, b_arg, c_arg, dtype, out_dtype, *blocks))
+
+        return _Plan(f"launch_nt_matmul {m}x{n}x{k} {tag}->{out_tag} blocks {blocks}", launch)
+
+    def _conv2d_plan(self, info, tag):
+        lib = runtime.library()
+        dtype = runtime.DATA_TYPE_INDEX[tag]
+        pad_h, pad_w = info["pad_h"], info["pad_w"]
+        blocks = [info["blocks"][axis] if info["blocks"][axis] > 1 else 0 for axis in ("m", "n", "k")]
+
+        def launch(call_args):
+            x, w, y = (runtime.ArgumentTensor.from_torch_tensor(tensor) for tensor in call_args)
+            runtime.check(lib.launch_nt_conv2d(runtime.current_stream(), x, w, y, dtype, pad_h, pad_w, *blocks))
+
+        return _Plan(f"launch_nt_conv2d gemm {info['m']}x{info['n']}x{info['k']} {tag} padding ({pad_h}, {pad_w})", launch)
+
+    def _prepare_softmax(self, args, env):
+        kind, info = recognition.analyze_softmax(self.types[0], self.types[1], env)
+        if kind == "empty":
+            return _Plan("empty launch", lambda call_args: None)
+        tag = self._tensor_dtype(*args, allowed=("fp32", "fp16", "bf16"))
+        lib = runtime.library()
+        dtype = runtime.DATA_TYPE_INDEX[tag]
+        block = info["input"]["block"]
+
+        def launch(call_args):
+            input, output = (runtime.ArgumentTensor.from_torch_tensor(tensor) for tensor in call_args)
+            runtime.check(lib.launch_nt_softmax(runtime.current_stream(), input, output, dtype, block))
+
+        return _Plan(f"launch_nt_softmax {info['input']['rows']}x{info['input']['cols']} {tag} block {block}", launch)
+
+    def _prepare_attention(self, args, env):
+        scaled = self.details["scale"]
+        if scaled:
+            q, k, v, is_causal, scale, o = args
+            q_t, k_t, v_t, o_t = self.types[0], self.types[1], self.types[2], self.types[5]
+        else:
+            q, k, v, is_causal, o = args
+            q_t, k_t, v_t, o_t = self.types[0], self.types[1], self.types[2], self.types[4]
+        kind, info = recognition.analyze_attention(q_t, k_t, v_t, o_t, env)
+        if kind == "empty":
+            return _Plan("empty launch", lambda call_args: None)
+        tag = self._tensor_dtype(q, k, v, o, allowed=("fp16", "bf16"))
+        lib = runtime.library()
+        dtype = runtime.DATA_TYPE_INDEX[tag]
+        o_pos = 5 if scaled else 4
+
+        def launch(call_args):
+            tensors = [runtime.ArgumentTensor.from_torch_tensor(call_args[p]) for p in (0, 1, 2, o_pos)]
+            causal = runtime.ArgumentTensor.from_scalar(int(bool(call_args[3])))
+            scale_arg = runtime.ArgumentTensor.from_scalar(float(call_args[4])) if scaled else runtime.ArgumentTensor.null()
+            runtime.check(lib.launch_nt_attention(runtime.current_stream(), tensors[0], tensors[1], tensors[2], causal, scale_arg, tensors[3], dtype, 0, 0))
+
+        return _Plan(f"launch_nt_attention q{info['q']['shape']} k{info['k']['shape']} {tag}", launch)
+
+
+class _Plan:
+    __slots__ = ("description", "launch")
+
+    def __init__(self, description, launch):
+        self.description = description
+        self.launch = launch
+
+    def __call__(self, args):
+        self.launch(args)

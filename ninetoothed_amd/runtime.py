@@ -1,0 +1,132 @@
+"""ctypes binding of ``libnt_hip.so`` (the C ABI declared in
+``include/ninetoothed_hip.h``).
+
+Follows the calling convention of the reference's AOT loader
+(src/ninetoothed/aot.py:704-751, 802-862): tensors are passed by value as
+``{data, shape, strides}`` structs with element strides, Python scalars as
+zero-dimensional tensors whose ``data`` points to a host ``double`` /
+``int64``, the launch happens on the caller's current stream, and a non-zero
+return value raises :class:`KernelLaunchError`.  There is no fallback: if the
+library is missing, loading fails.
+"""
+
+import ctypes
+import pathlib
+import threading
+
+LIBRARY_PATH = pathlib.Path(__file__).resolve().parent / "lib" / "libnt_hip.so"
+
+NO_KERNEL = 1
+
+# order of the reference's NineToothedDataType enum (src/ninetoothed/aot.py:524-537)
+DATA_TYPES = ("i8", "i16", "i32", "i64", "u8", "u16", "u32", "u64", "fp16", "bf16", "fp32", "fp64")
+DATA_TYPE_INDEX = {name: index for index, name in enumerate(DATA_TYPES)}
+
+
+class KernelLaunchError(RuntimeError):
+    def __init__(self, error_code):
+        self.error_code = error_code
+        super().__init__(f"Kernel launch failed with error code: {error_code}.")
+
+
+class ArgumentTensor(ctypes.Structure):
+    _fields_ = [
+        ("data", ctypes.c_void_p),
+        ("shape", ctypes.POINTER(ctypes.c_uint64)),
+        ("strides", ctypes.POINTER(ctypes.c_int64)),
+    ]
+
+    @staticmethod
+    def from_layout(data_ptr, shape, strides):
+        shape_array = (ctypes.c_uint64 * max(len(shape), 1))(*shape)
+        strides_array = (ctypes.c_int64 * max(len(strides), 1))(*strides)
+        tensor = ArgumentTensor(data_ptr, shape_array, strides_array)
+        tensor._keepalive = (shape_array, strides_array)
+        return tensor
+
+    @staticmethod
+    def from_torch_tensor(tensor):
+        argument = ArgumentTensor.from_layout(tensor.data_ptr(), tuple(tensor.shape), tuple(tensor.stride()))
+        argument._torch_tensor = tensor
+        return argument
+
+    @staticmethod
+    def from_scalar(value):
+        """A zero-dimensional tensor: host double for floats, host int64 otherwise."""
+        buffer = ctypes.c_double(value) if isinstance(value, float) else ctypes.c_int64(int(value))
+        argument = ArgumentTensor(ctypes.addressof(buffer), None, None)
+        argument._keepalive = buffer
+        return argument
+
+    @staticmethod
+    def null():
+        return ArgumentTensor(None, None, None)
+
+
+_T = ArgumentTensor
+_I = ctypes.c_int
+_S = ctypes.c_void_p
+
+_SIGNATURES = {
+    "launch_nt_matmul": (_S, _T, _T, _T, _I, _I, _I, _I, _I),
+    "launch_nt_addmm": (_S, _T, _T, _T, _T, _T, _T, _I, _I, _I, _I),
+    "launch_nt_softmax": (_S, _T, _T, _I, _I),
+    "launch_nt_softmax_config": (_S, _I, _T, _T, _I, _I),
+    "launch_nt_attention": (_S, _T, _T, _T, _T, _T, _T, _I, _I, _I),
+    "launch_nt_conv2d": (_S, _T, _T, _T, _I, _I, _I, _I, _I, _I),
+    "launch_nt_gemm_config": (_S, _I, _T, _T, _T, _T, _T, _T, _I, _I),
+    "nt_tune_gemm": (_S, _T, _T, _T, _T, _T, _T, _I, _I, _I, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_float)),
+    "nt_gemm_num_configs": (),
+    "nt_gemm_config_name": (_I, ctypes.c_char_p, _I),
+}
+
+_library = None
+_lock = threading.Lock()
+
+
+def library():
+    """Loads ``libnt_hip.so`` once; raises if it has not been built."""
+    global _library
+    if _library is not None:
+        return _library
+    with _lock:
+        if _library is None:
+            if not LIBRARY_PATH.exists():
+                raise RuntimeError(
+                    f"{LIBRARY_PATH} is missing: build it with `python -m ninetoothed_amd.build` (needs hipcc). "
+                    "There is no fallback path."
+                )
+            lib = ctypes.CDLL(str(LIBRARY_PATH))
+            for name, argtypes in _SIGNATURES.items():
+                function = getattr(lib, name)
+                function.argtypes = list(argtypes)
+                function.restype = ctypes.c_int
+            lib.nt_version.restype = ctypes.c_char_p
+            lib.nt_version.argtypes = []
+            _library = lib
+    return _library
+
+
+def exported_symbols():
+    return tuple(_SIGNATURES) + ("nt_version",)
+
+
+def check(result):
+    if result != 0:
+        raise KernelLaunchError(result)
+
+
+def current_stream():
+    import torch
+
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def gemm_config_names():
+    lib = library()
+    names = []
+    for index in range(lib.nt_gemm_num_configs()):
+        buffer = ctypes.create_string_buffer(160)
+        check(lib.nt_gemm_config_name(index, buffer, len(buffer)))
+        names.append(buffer.value.decode())
+    return names

@@ -1,0 +1,315 @@
+"""Parity of the HIP path (through ``ninetoothed_amd.make`` and the C ABI of
+libnt_hip.so) with the CPU oracle on the same seeded inputs, at sizes the
+oracle finishes in seconds, and with the torch ops the reference's own tests
+compare against.  Bars: rtol = atol = 1e-2 for fp16 / bf16 (the reference's
+tests/test_attention.py:102 states the same for fp16), 1e-5 for fp32 softmax."""
+
+import functools
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import ninetoothed_amd as ninetoothed
+from ninetoothed_amd import Tensor, programs
+from oracle import programs as oracle
+
+pytestmark = pytest.mark.gpu
+
+HALF_TOL = dict(rtol=1e-2, atol=1e-2)
+
+
+def _native_only(kernel, expected_prefix):
+    assert kernel.last_plan is not None and kernel.last_plan.startswith(expected_prefix), kernel.last_plan
+
+
+def _randn(*shape, dtype=torch.float16, scale=1.0):
+    return (torch.randn(*shape) * scale).to(dtype)
+
+
+# ---- matmul ---------------------------------------------------------------
+
+
+def _matmul_kernel(application=programs.matmul.application, **blocks):
+    arrangement = functools.partial(programs.matmul.arrangement, **blocks) if blocks else programs.matmul.arrangement
+    return ninetoothed.make(arrangement, application, (Tensor(2), Tensor(2), Tensor(2)))
+
+
+@pytest.mark.parametrize("m, n, k", ((512, 512, 512), (300, 200, 100), (64, 48, 8), (1, 1, 1), (257, 129, 65)))
+def test_matmul_against_oracle(m, n, k):
+    a, b = _randn(m, k), _randn(k, n)
+    out = torch.empty(m, n, dtype=torch.float16, device="cuda")
+    kernel = _matmul_kernel(programs.matmul.application_with_cast)
+    kernel(a.cuda(), b.cuda(), out)
+    _native_only(kernel, "launch_nt_matmul")
+    expected = oracle.matmul(a.numpy(), b.numpy(), 64, 64, 64)
+    assert np.allclose(out.cpu().float().numpy(), expected, **HALF_TOL)
+    assert torch.allclose(out, torch.matmul(a.cuda(), b.cuda()), **HALF_TOL)
+
+
+def test_matmul_readme_program_fixed_blocks_and_strides():
+    a, b = _randn(512, 384), _randn(384, 256)
+    kernel = _matmul_kernel(BLOCK_SIZE_M=64, BLOCK_SIZE_N=64, BLOCK_SIZE_K=64)
+    out = torch.empty(512, 256, dtype=torch.float16, device="cuda")
+    kernel(a.cuda(), b.cuda(), out)
+    assert torch.allclose(out, torch.matmul(a.cuda(), b.cuda()), **HALF_TOL)
+    # column-major rhs, row-strided lhs, strided output
+    bt = b.t().contiguous().cuda().t()
+    wide = torch.zeros(512, 512, dtype=torch.float16, device="cuda")
+    wide[:, :384] = a.cuda()
+    out2 = torch.zeros(512, 512, dtype=torch.float16, device="cuda")
+    kernel(wide[:, :384], bt, out2[:, ::2])
+    assert torch.allclose(out2[:, ::2], out, rtol=0, atol=0)
+    assert torch.count_nonzero(out2[:, 1::2]) == 0
+
+
+def test_matmul_bfloat16_and_float32_output():
+    a, b = _randn(256, 128, dtype=torch.bfloat16), _randn(128, 256, dtype=torch.bfloat16)
+    kernel = _matmul_kernel()
+    out = torch.empty(256, 256, dtype=torch.bfloat16, device="cuda")
+    kernel(a.cuda(), b.cuda(), out)
+    expected = oracle.matmul(a.float().numpy(), b.float().numpy(), 64, 64, 64, out_dtype="bf16")
+    assert np.allclose(out.cpu().float().numpy(), expected, rtol=2e-2, atol=2e-2)
+    out32 = torch.empty(256, 256, dtype=torch.float32, device="cuda")
+    kernel(a.cuda(), b.cuda(), out32)
+    assert torch.allclose(out32, a.cuda().float() @ b.cuda().float(), rtol=1e-4, atol=1e-3)
+
+
+def test_matmul_empty_and_errors():
+    kernel = _matmul_kernel()
+    out = torch.empty(0, 16, dtype=torch.float16, device="cuda")
+    kernel(torch.empty(0, 8, dtype=torch.float16, device="cuda"), torch.empty(8, 16, dtype=torch.float16, device="cuda"), out)
+    with pytest.raises(RuntimeError):
+        kernel(torch.empty(4, 4, dtype=torch.float16), torch.empty(4, 4, dtype=torch.float16), torch.empty(4, 4, dtype=torch.float16))
+    with pytest.raises(ninetoothed.UnsupportedProgram):
+        kernel(*(torch.empty(4, 4, dtype=torch.float64, device="cuda") for _ in range(3)))
+
+
+def test_matmul_large_properties():
+    # 8192^3: linearity and an identity block, properties that hold at any size
+    n = 8192
+    a = _randn(n, n).cuda()
+    b = _randn(n, n, scale=0.05).cuda()
+    kernel = _matmul_kernel()
+    out = torch.empty(n, n, dtype=torch.float16, device="cuda")
+    kernel(a, b, out)
+    _native_only(kernel, "launch_nt_matmul")
+    rows = torch.randint(0, n, (64,), device="cuda")
+    expected = (a[rows].float() @ b.float())
+    assert torch.allclose(out[rows].float(), expected, **HALF_TOL)
+    eye = torch.eye(n, dtype=torch.float16, device="cuda")
+    kernel(a, eye, out)
+    assert torch.equal(out, a)
+
+
+# ---- addmm ----------------------------------------------------------------
+
+
+def _addmm_kernel():
+    return ninetoothed.make(programs.addmm.arrangement, programs.addmm.application, programs.addmm.tensors())
+
+
+@pytest.mark.parametrize("m, n, k", ((512, 512, 512), (100, 36, 52)))
+def test_addmm_against_oracle(m, n, k):
+    input, mat1, mat2 = _randn(m, n), _randn(m, k), _randn(k, n)
+    beta, alpha = 0.37, 0.81
+    out = torch.empty(m, n, dtype=torch.float16, device="cuda")
+    kernel = _addmm_kernel()
+    kernel(input.cuda(), mat1.cuda(), mat2.cuda(), beta, alpha, out)
+    _native_only(kernel, "launch_nt_addmm")
+    expected = oracle.addmm(input.numpy(), mat1.numpy(), mat2.numpy(), beta, alpha, 64, 64, 64)
+    assert np.allclose(out.cpu().float().numpy(), expected, **HALF_TOL)
+    # the reference's own bar: tests/test_addmm.py:88-90, atol 0.075 against torch.addmm
+    reference = torch.addmm(input.cuda(), mat1.cuda(), mat2.cuda(), beta=beta, alpha=alpha)
+    assert torch.allclose(out, reference, atol=0.075)
+
+
+def test_addmm_large():
+    n = 8192
+    input, mat1, mat2 = _randn(n, n).cuda(), _randn(n, n).cuda(), _randn(n, n, scale=0.05).cuda()
+    out = torch.empty(n, n, dtype=torch.float16, device="cuda")
+    kernel = _addmm_kernel()
+    kernel(input, mat1, mat2, 0.5, 1.0, out)
+    rows = torch.randint(0, n, (64,), device="cuda")
+    expected = 0.5 * input[rows].float() + (mat1[rows].float() @ mat2.float()).half().float()
+    assert torch.allclose(out[rows].float(), expected, **HALF_TOL)
+
+
+# ---- softmax --------------------------------------------------------------
+
+
+def _softmax(x, block_size=None):
+    kernel = ninetoothed.make(programs.softmax.arrangement, programs.softmax.application, programs.softmax.tensors())
+    out = torch.empty_like(x)
+    kernel(x, out, BLOCK_SIZE=x.shape[-1] if block_size is None else block_size)
+    _native_only(kernel, "launch_nt_softmax")
+    return out
+
+
+@pytest.mark.parametrize("m, n", ((1823, 781), (64, 4096), (5, 1), (3, 17000), (33, 8192)))
+def test_softmax_against_oracle(m, n):
+    x = torch.rand(m, n) if n == 781 else torch.randn(m, n)
+    out = _softmax(x.cuda())
+    assert np.allclose(out.cpu().numpy(), oracle.softmax(x.numpy()), rtol=1e-5, atol=1e-5)
+    assert torch.allclose(out, torch.softmax(x.cuda(), dim=-1), rtol=1e-5, atol=1e-6)
+
+
+def test_softmax_jit_decorator_form():
+    # the decorator form with annotated parameters, as in the reference's tests/test_softmax.py:10-27
+    import ninetoothed_amd.language as ntl
+    from ninetoothed_amd import Symbol
+
+    BLOCK_SIZE = Symbol("BLOCK_SIZE", constexpr=True)
+
+    @ninetoothed.jit
+    def softmax_kernel(
+        input_row: Tensor(2, other=float("-inf")).tile((1, BLOCK_SIZE)),
+        output_row: Tensor(2).tile((1, BLOCK_SIZE)),
+    ):
+        row_minus_max = input_row - ntl.max(input_row)
+        numerator = ntl.exp(row_minus_max)
+        denominator = ntl.sum(numerator)
+        output_row = numerator / denominator  # noqa: F841
+
+    x = torch.rand(1823, 781, device="cuda")
+    out = torch.empty_like(x)
+    softmax_kernel(x, out, BLOCK_SIZE=x.shape[-1])
+    assert torch.allclose(out, torch.softmax(x, dim=-1))
+
+
+def test_softmax_half_blocks_and_strides():
+    x = torch.randn(128, 1000).to(torch.float16)
+    out = _softmax(x.cuda())
+    expected = torch.softmax(x.float(), dim=-1)
+    assert torch.allclose(out.cpu().float(), expected, rtol=1e-2, atol=1e-3)
+    y = torch.randn(16, 100)
+    out = _softmax(y.cuda(), block_size=32)
+    assert np.allclose(out.cpu().numpy(), oracle.softmax(y.numpy(), block_size=32), rtol=1e-5, atol=1e-6)
+    wide = torch.randn(64, 512, device="cuda")
+    view = wide[:, ::2]
+    out = _softmax(view)
+    assert torch.allclose(out, torch.softmax(view, dim=-1), rtol=1e-5, atol=1e-6)
+
+
+def test_softmax_baseline_shape_properties():
+    x = torch.randn(4096, 4096, device="cuda")
+    out = _softmax(x)
+    assert torch.allclose(out.sum(dim=-1), torch.ones(4096, device="cuda"), atol=1e-5)
+    assert torch.allclose(out, _softmax(x + 2.5), rtol=1e-4, atol=1e-7)  # shift invariance
+    assert torch.allclose(out, torch.softmax(x, dim=-1), rtol=1e-5, atol=1e-6)
+
+
+# ---- attention ------------------------------------------------------------
+
+
+def _attention(q, k, v, is_causal=False, scale=None):
+    o = torch.empty_like(q)
+    if scale is None:
+        kernel = ninetoothed.make(programs.attention.arrangement, programs.attention.application, programs.attention.tensors())
+        kernel(q, k, v, is_causal, o)
+    else:
+        kernel = ninetoothed.make(programs.attention.arrangement_with_scale, programs.attention.application_with_scale, programs.attention.tensors(True))
+        kernel(q, k, v, is_causal, scale, o)
+    _native_only(kernel, "launch_nt_attention")
+    return o
+
+
+@pytest.mark.parametrize("is_causal", (False, True))
+@pytest.mark.parametrize("seq_len, emb_dim", ((160, 64), (1, 64), (100, 128), (333, 32)))
+def test_attention_against_oracle(seq_len, emb_dim, is_causal):
+    q, k, v = (_randn(2, 2, seq_len, emb_dim) for _ in range(3))
+    out = _attention(q.cuda(), k.cuda(), v.cuda(), is_causal)
+    expected = oracle.attention(q.numpy(), k.numpy(), v.numpy(), is_causal=is_causal, bm=64, bn=32)
+    assert np.allclose(out.cpu().float().numpy(), expected, **HALF_TOL)
+
+
+@pytest.mark.parametrize("is_causal", (False, True))
+@pytest.mark.parametrize("seq_len", (1024, 1))
+def test_attention_reference_test_shapes(seq_len, is_causal):
+    # reference: tests/test_attention.py:99-117 -- [2, 4, {1024, 1}, 64] fp16, scale 1, rtol = atol = 0.01
+    q, k, v = (_randn(2, 4, seq_len, 64).cuda() for _ in range(3))
+    out = _attention(q, k, v, is_causal)
+    expected = F.scaled_dot_product_attention(q, k, v, is_causal=is_causal, scale=1)
+    assert torch.allclose(out, expected, **HALF_TOL)
+
+
+@pytest.mark.parametrize("is_causal", (False, True))
+def test_attention_scaled_head_dim_128_and_bfloat16(is_causal):
+    q, k, v = (_randn(1, 3, 1000, 128).cuda() for _ in range(3))
+    out = _attention(q, k, v, is_causal, scale=128**-0.5)
+    expected = F.scaled_dot_product_attention(q, k, v, is_causal=is_causal, scale=128**-0.5)
+    assert torch.allclose(out, expected, **HALF_TOL)
+    qb, kb, vb = (t.to(torch.bfloat16) for t in (q, k, v))
+    out = _attention(qb, kb, vb, is_causal, scale=128**-0.5)
+    expected = F.scaled_dot_product_attention(qb, kb, vb, is_causal=is_causal, scale=128**-0.5)
+    assert torch.allclose(out.float(), expected.float(), rtol=3e-2, atol=3e-2)
+
+
+def test_attention_closed_forms_and_layouts():
+    q, v = _randn(1, 2, 300, 64).cuda(), _randn(1, 2, 300, 64).cuda()
+    k = torch.zeros_like(q)
+    out = _attention(q, k, v)
+    assert torch.allclose(out.float(), v.float().mean(dim=2, keepdim=True).expand_as(out), atol=5e-3)
+    causal = _attention(q, k, v, True)
+    assert torch.allclose(causal[:, :, 0], v[:, :, 0], atol=1e-3)
+    # [batch, seq, heads, dim] storage viewed as [batch, heads, seq, dim]
+    packed = _randn(2, 200, 3, 64).cuda()
+    view = packed.permute(0, 2, 1, 3)
+    out = _attention(view, view, view)
+    expected = F.scaled_dot_product_attention(view, view, view, scale=1)
+    assert torch.allclose(out, expected, **HALF_TOL)
+
+
+@pytest.mark.parametrize("is_causal", (False, True))
+def test_attention_baseline_shape(is_causal):
+    q, k, v = (_randn(4, 32, 4096, 128).cuda() for _ in range(3))
+    out = _attention(q, k, v, is_causal, scale=128**-0.5)
+    expected = F.scaled_dot_product_attention(q[:1, :2], k[:1, :2], v[:1, :2], is_causal=is_causal, scale=128**-0.5)
+    assert torch.allclose(out[:1, :2], expected, **HALF_TOL)
+    assert torch.isfinite(out).all()
+
+
+# ---- conv2d ---------------------------------------------------------------
+
+
+def _conv2d(x, w, padding):
+    n, _, h, width = x.shape
+    k, _, r, s = w.shape
+    p, q = h + 2 * padding[0] - r + 1, width + 2 * padding[1] - s + 1
+    out = torch.empty(n, k, p, q, dtype=x.dtype, device=x.device)
+    kernel = ninetoothed.make(programs.conv2d.arrangement, programs.conv2d.application, programs.conv2d.tensors())
+    kernel(x, w, out, padding_h=padding[0], padding_w=padding[1])
+    _native_only(kernel, "launch_nt_conv2d")
+    return out
+
+
+@pytest.mark.parametrize("padding", ((0, 0), (1, 1), (0, 1), (2, 0)))
+def test_conv2d_against_oracle(padding):
+    x = torch.rand(2, 6, 9, 8).to(torch.float16)
+    w = torch.rand(5, 6, 3, 3).to(torch.float16)
+    out = _conv2d(x.cuda(), w.cuda(), padding)
+    expected = oracle.conv2d(x.numpy(), w.numpy(), padding=padding, bm=16, bn=4, bk=8)
+    assert np.allclose(out.cpu().float().numpy(), expected, **HALF_TOL)
+
+
+@pytest.mark.parametrize("padding", ((0, 0), (1, 1), (0, 1), (2, 0)))
+def test_conv2d_reference_test_shapes(padding):
+    # reference: tests/test_conv2d.py:116-133 -- N4 C64 H16 W16 K512 R3 S3, torch.rand, rtol = atol = 1e-3
+    x = torch.rand(4, 64, 16, 16, dtype=torch.float16, device="cuda")
+    w = torch.rand(512, 64, 3, 3, dtype=torch.float16, device="cuda")
+    out = _conv2d(x, w, padding)
+    expected = F.conv2d(x, w, padding=padding)
+    assert torch.allclose(out, expected, rtol=1e-3, atol=1e-3)
+
+
+def test_conv2d_baseline_shape_and_1x1():
+    x = _randn(32, 256, 56, 56, scale=0.1).cuda()
+    w = _randn(256, 256, 3, 3, scale=0.1).cuda()
+    out = _conv2d(x, w, (1, 1))
+    expected = F.conv2d(x[:2], w, padding=1)
+    assert torch.allclose(out[:2], expected, **HALF_TOL)
+    w1 = _randn(64, 256, 1, 1, scale=0.1).cuda()
+    out = _conv2d(x[:1], w1, (0, 0))
+    as_matmul = (x[:1].permute(0, 2, 3, 1).reshape(-1, 256).float() @ w1.reshape(64, 256).t().float()).reshape(1, 56, 56, 64).permute(0, 3, 1, 2)
+    assert torch.allclose(out.float(), as_matmul, **HALF_TOL)
