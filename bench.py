@@ -1,0 +1,249 @@
+"""Benchmark of the hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+
+A step is one launch of the workload's kernel through ``ninetoothed_amd.make``
+(i.e. through the C ABI of libnt_hip.so) on synthetic, seeded inputs that are
+already resident in HBM.  The default workload is the one the headline metric
+is quoted on: addmm, fp16, M = N = K = 8192, alpha = 1.0, beta = 0.5.  The other
+configurations of the baseline (512^3 matmul, 4096^2 fp32 softmax, SDPA forward
+[4, 32, 4096, 128] causal / non-causal, conv2d [32, 256, 56, 56] * [256, 256, 3, 3])
+are measured in the same run and reported under ``"others"``.
+
+Prints ONE JSON line.  ``roofline.achieved`` = algorithmic FLOP (or bytes) per
+launch / average launch time from device events on the launch stream.
+``cpu_baseline`` times the CPU oracle (oracle/programs.py, single thread) on a
+bounded sample of the same workload.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+PEAK_TFLOPS = 2500.0  # dense fp16 MFMA, MI355X
+PEAK_GBS = 8000.0     # HBM3E, MI355X
+
+METRIC = "TFLOP/s fp16 matmul 8192^3 + attention fwd on 1 MI355X; % of MFMA peak"
+
+
+def parse_args():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=20)
+    parser.add_argument("--warmup", type=int, default=5)
+    parser.add_argument("--workload", default="addmm_8192")
+    parser.add_argument("--only", action="store_true", help="measure only --workload")
+    parser.add_argument("--no-cpu-baseline", action="store_true")
+    return parser.parse_args()
+
+
+def build_workloads():
+    import torch
+
+    import ninetoothed_amd as ninetoothed
+    from ninetoothed_amd import programs
+
+    def seeded(*shape, dtype=torch.float16, scale=1.0, seed=0):
+        generator = torch.Generator().manual_seed(seed)
+        return (torch.randn(*shape, generator=generator) * scale).to(dtype)
+
+    workloads = {}
+
+    def addmm_8192():
+        n = 8192
+        input, mat1, mat2 = (seeded(n, n, seed=s).cuda() for s in (0, 1, 2))
+        out = torch.empty(n, n, dtype=torch.float16, device="cuda")
+        kernel = ninetoothed.make(programs.addmm.arrangement, programs.addmm.application, programs.addmm.tensors())
+        return dict(
+            step=lambda: kernel(input, mat1, mat2, 0.5, 1.0, out),
+            work=2.0 * n**3, bound="mfma", kernel=kernel,
+            describe={"workload": "addmm fp16 M=N=K=8192 alpha=1.0 beta=0.5", "inputs": "randn, seeded"},
+        )
+
+    def matmul_512():
+        n = 512
+        a, b = seeded(n, n, seed=0).cuda(), seeded(n, n, seed=1).cuda()
+        out = torch.empty(n, n, dtype=torch.float16, device="cuda")
+        kernel = ninetoothed.make(programs.matmul.arrangement, programs.matmul.application, programs.matmul.tensors())
+        return dict(step=lambda: kernel(a, b, out), work=2.0 * n**3, bound="mfma", kernel=kernel,
+                    describe={"workload": "matmul fp16 M=N=K=512 (README program)"})
+
+    def softmax_4096():
+        x = seeded(4096, 4096, dtype=torch.float32).cuda()
+        out = torch.empty_like(x)
+        kernel = ninetoothed.make(programs.softmax.arrangement, programs.softmax.application, programs.softmax.tensors())
+        return dict(step=lambda: kernel(x, out, BLOCK_SIZE=4096), work=2.0 * 4096 * 4096 * 4, bound="hbm", kernel=kernel,
+                    describe={"workload": "row softmax fp32 [4096, 4096]"})
+
+    def attention(is_causal):
+        def make():
+            q, k, v = (seeded(4, 32, 4096, 128, seed=s).cuda() for s in (0, 1, 2))
+            o = torch.empty_like(q)
+            kernel = ninetoothed.make(programs.attention.arrangement_with_scale, programs.attention.application_with_scale, programs.attention.tensors(True))
+            flops = 4.0 * 4 * 32 * 4096 * 4096 * 128 * (0.5 if is_causal else 1.0)
+            return dict(step=lambda: kernel(q, k, v, is_causal, 128**-0.5, o), work=flops, bound="mfma", kernel=kernel,
+                        describe={"workload": f"SDPA forward fp16 [4, 32, 4096, 128] scale=1/sqrt(128) causal={is_causal}"})
+        return make
+
+    def conv2d():
+        x = seeded(32, 256, 56, 56, scale=0.1, seed=0).cuda()
+        w = seeded(256, 256, 3, 3, scale=0.1, seed=1).cuda()
+        out = torch.empty(32, 256, 56, 56, dtype=torch.float16, device="cuda")
+        kernel = ninetoothed.make(programs.conv2d.arrangement, programs.conv2d.application, programs.conv2d.tensors())
+        return dict(step=lambda: kernel(x, w, out, padding_h=1, padding_w=1), work=2.0 * (32 * 56 * 56) * 256 * (256 * 9), bound="mfma", kernel=kernel,
+                    describe={"workload": "conv2d fp16 x[32,256,56,56] w[256,256,3,3] stride 1 padding 1 (implicit GEMM)"})
+
+    workloads["addmm_8192"] = addmm_8192
+    workloads["matmul_512"] = matmul_512
+    workloads["softmax_4096"] = softmax_4096
+    workloads["attention"] = attention(False)
+    workloads["attention_causal"] = attention(True)
+    workloads["conv2d"] = conv2d
+    return workloads
+
+
+def measure(workload, steps, warmup):
+    """Times exactly ``steps`` launches with device events on the launch stream."""
+    import torch
+
+    for _ in range(warmup):
+        workload["step"]()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    wall0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        workload["step"]()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - wall0) * 1e3 / steps
+    device_ms = start.elapsed_time(stop) / steps
+    return device_ms, wall
+
+
+def roofline(workload, device_ms, traffic):
+    if workload["bound"] == "mfma":
+        achieved = workload["work"] / (device_ms * 1e-3) / 1e12
+        return {"bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_TFLOPS, "traffic": traffic}
+    achieved = workload["work"] / (device_ms * 1e-3) / 1e9
+    return {"bound": "hbm", "achieved": achieved, "peak": PEAK_GBS, "unit": "GB/s", "frac": achieved / PEAK_GBS, "traffic": traffic}
+
+
+def cpu_baseline_addmm():
+    """The CPU oracle (tile-by-tile numpy restatement) on a 64-row band of the
+    8192^3 addmm: 64 x 8192 x 8192, one thread."""
+    import numpy as np
+    from threadpoolctl import threadpool_limits
+
+    from oracle import programs as oracle
+
+    rows, n = 64, 8192
+    rng = np.random.default_rng(0)
+    input = rng.standard_normal((rows, n), dtype=np.float32).astype(np.float16)
+    mat1 = rng.standard_normal((rows, n), dtype=np.float32).astype(np.float16)
+    mat2 = rng.standard_normal((n, n), dtype=np.float32).astype(np.float16)
+    with threadpool_limits(limits=1):
+        t0 = time.perf_counter()
+        oracle.addmm(input, mat1, mat2, 0.5, 1.0, bm=64, bn=64, bk=64)
+        seconds = time.perf_counter() - t0
+    flops = 2.0 * rows * n * n
+    return {
+        "value": flops / seconds / 1e12,
+        "unit": "TFLOP/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": f"oracle.addmm on a {rows}x{n}x{n} band of the workload (64x64x64 blocks), {seconds:.1f} s",
+    }
+
+
+def torch_cpu_addmm():
+    """torch.addmm on the host, all threads, on a 1024-row band (context only)."""
+    import torch
+
+    rows, n = 1024, 8192
+    generator = torch.Generator().manual_seed(0)
+    input = torch.randn(rows, n, generator=generator)
+    mat1 = torch.randn(rows, n, generator=generator)
+    mat2 = torch.randn(n, n, generator=generator)
+    t0 = time.perf_counter()
+    torch.addmm(input, mat1, mat2, beta=0.5, alpha=1.0)
+    seconds = time.perf_counter() - t0
+    return {"value": 2.0 * rows * n * n / seconds / 1e12, "unit": "TFLOP/s", "threads": torch.get_num_threads(),
+            "sample": f"torch.addmm fp32 {rows}x{n}x{n} on the host, {seconds:.2f} s"}
+
+
+def load_traffic():
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic.json")
+    if os.path.exists(path):
+        with open(path) as handle:
+            return json.load(handle)
+    return {}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this build has no multi-GPU path (asked for --gpus {args.gpus}).", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (there is no CPU path).", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+
+    workloads = build_workloads()
+    if args.workload not in workloads:
+        print(f"unknown workload `{args.workload}`; choose from {sorted(workloads)}", file=sys.stderr)
+        sys.exit(2)
+    traffic = load_traffic()
+
+    main_workload = workloads[args.workload]()
+    device_ms, wall_ms = measure(main_workload, args.steps, args.warmup)
+    main_roofline = roofline(main_workload, device_ms, traffic.get(args.workload))
+    launch_plan = main_workload["kernel"].last_plan
+    del main_workload["step"]
+
+    others = {}
+    if not args.only:
+        for name, factory in workloads.items():
+            if name == args.workload:
+                continue
+            workload = factory()
+            ms, _ = measure(workload, max(5, args.steps // 2), args.warmup)
+            entry = roofline(workload, ms, traffic.get(name))
+            entry["ms_per_step"] = ms
+            entry["config"] = workload["describe"]
+            others[name] = entry
+            del workload
+            torch.cuda.empty_cache()
+
+    result = {
+        "metric": METRIC,
+        "value": main_roofline["achieved"],
+        "unit": main_roofline["unit"],
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": device_ms,
+        "wall_ms_per_step": wall_ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16" if main_roofline["bound"] == "mfma" else "f32",
+        "data": "synthetic",
+        "config": dict(main_workload["describe"], launch=launch_plan),
+        "roofline": main_roofline,
+        "others": others,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline_addmm()
+        result["torch_cpu"] = torch_cpu_addmm()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
