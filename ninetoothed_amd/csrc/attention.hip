@@ -32,14 +32,14 @@ struct AttentionParams {
     int q_blocks;
 };
 
-constexpr int kAttnBN = 64;
 constexpr int kAttnWaves = 4;
 
-template <typename T, int D, int kQTiles>
-__global__ __launch_bounds__(kAttnWaves * 64) void attention_fwd_kernel(AttentionParams p) {
+// BN: key/value rows per block; kOcc: waves per SIMD the register budget is held to
+template <typename T, int D, int kQTiles, int BN, int kOcc>
+__global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(AttentionParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
     typedef Elem<T> E;
     typedef typename E::vec8 vec8;
-    constexpr int BN = kAttnBN;
     constexpr int BM = kAttnWaves * 32 * kQTiles;
     constexpr int KT = BN / 32;          // kv tiles of S^T per block
     constexpr int DT = D / 32;           // d tiles of O^T
@@ -71,9 +71,20 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attention_fwd_kernel(Attentio
     const int g = lane >> 5;
     const int l32 = lane & 31;
 
-    // workgroup -> (batch, head, query block); consecutive ids share K/V
-    const int qb = blockIdx.x % p.q_blocks;
-    const int bh = blockIdx.x / p.q_blocks;
+    // workgroup -> (batch, head, query block).  Non-causal: consecutive ids are
+    // the query blocks of one (batch, head) and share its K/V in L2.  Causal: the
+    // work of a query block grows with its index, so ids walk the (batch, head)
+    // pairs first and the query blocks from last (longest) to first; every CU then
+    // gets the same mix of long and short blocks.
+    int qb, bh;
+    if (p.causal) {
+        const int pairs = p.batch * p.heads;
+        qb = p.q_blocks - 1 - blockIdx.x / pairs;
+        bh = blockIdx.x % pairs;
+    } else {
+        qb = blockIdx.x % p.q_blocks;
+        bh = blockIdx.x / p.q_blocks;
+    }
     const int head = bh % p.heads;
     const int batch = bh / p.heads;
     const int q0 = qb * BM;
@@ -227,10 +238,14 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attention_fwd_kernel(Attentio
                     sum += pv;
                 }
             l_run[qt] = l_run[qt] * alpha + sum;
+            // the running maximum settles after a few blocks; skip the rescale of the
+            // output accumulators when no row of this wave's tile moved (wave-uniform)
+            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
+                for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) o_acc[dt][qt][r] *= alpha;
+                    for (int r = 0; r < 16; ++r) o_acc[dt][qt][r] *= alpha;
+            }
         }
 
         // O^T += V^T . P^T
@@ -298,23 +313,35 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attention_fwd_kernel(Attentio
                 }
         }
     }
+#endif
 }
 
-template <typename T, int D, int kQTiles>
+template <typename T, int D, int kQTiles, int BN, int kOcc>
 hipError_t launch_attention(AttentionParams &p, hipStream_t stream) {
     constexpr int BM = kAttnWaves * 32 * kQTiles;
     p.q_blocks = ceil_div(p.seq_q, BM);
     const int64_t grid = (int64_t)p.batch * p.heads * p.q_blocks;
     if (grid == 0) return hipSuccess;
-    attention_fwd_kernel<T, D, kQTiles><<<dim3((unsigned)grid), dim3(kAttnWaves * 64), 0, stream>>>(p);
+    attention_fwd_kernel<T, D, kQTiles, BN, kOcc><<<dim3((unsigned)grid), dim3(kAttnWaves * 64), 0, stream>>>(p);
     return hipGetLastError();
 }
 
+// variant: 0 = 128 query rows per workgroup, 64-key blocks, two workgroups per CU (default)
+//          1 = 256 query rows per workgroup, 64-key blocks, one workgroup per CU
+//          2 = 128 query rows per workgroup, 32-key blocks, three workgroups per CU
 template <typename T>
-int dispatch_attention(AttentionParams &p, int head_dim, int q_tiles, hipStream_t stream) {
-    if (head_dim == 128) return (int)(q_tiles == 1 ? launch_attention<T, 128, 1>(p, stream) : launch_attention<T, 128, 2>(p, stream));
-    if (head_dim == 64) return (int)(q_tiles == 1 ? launch_attention<T, 64, 1>(p, stream) : launch_attention<T, 64, 2>(p, stream));
-    if (head_dim == 32) return (int)launch_attention<T, 32, 1>(p, stream);
+int dispatch_attention(AttentionParams &p, int head_dim, int variant, hipStream_t stream) {
+    if (head_dim == 128) {
+        if (variant == 1) return (int)launch_attention<T, 128, 2, 64, 1>(p, stream);
+        if (variant == 2) return (int)launch_attention<T, 128, 1, 32, 3>(p, stream);
+        return (int)launch_attention<T, 128, 1, 64, 2>(p, stream);
+    }
+    if (head_dim == 64) {
+        if (variant == 1) return (int)launch_attention<T, 64, 2, 64, 1>(p, stream);
+        if (variant == 2) return (int)launch_attention<T, 64, 1, 32, 3>(p, stream);
+        return (int)launch_attention<T, 64, 1, 64, 2>(p, stream);
+    }
+    if (head_dim == 32) return (int)launch_attention<T, 32, 1, 64, 2>(p, stream);
     return NINETOOTHED_NO_KERNEL;
 }
 
@@ -327,7 +354,6 @@ extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineT
                                                  NineToothedTensor v, NineToothedTensor is_causal,
                                                  NineToothedTensor scale, NineToothedTensor o, int dtype,
                                                  int block_size_m, int block_size_n) {
-    (void)block_size_n;
     if (dtype != NINETOOTHED_FLOAT16 && dtype != NINETOOTHED_BFLOAT16) return NINETOOTHED_NO_KERNEL;
     const NineToothedTensor *ts[4] = {&q, &k, &v, &o};
     for (const NineToothedTensor *t : ts)
@@ -360,9 +386,9 @@ extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineT
     const double scale_value = scale.data ? Scalar0d::as_double(scale) : 1.0;
     p.q_scale = (float)(scale_value * 1.4426950408889634);
     p.causal = is_causal.data ? (Scalar0d::as_int64(is_causal) != 0) : 0;
-    // block_size_m <= 128 selects the 128-row workgroup, otherwise 256 rows (default
-    // for long sequences: half the K/V traffic through LDS per query row)
-    int q_tiles = block_size_m > 0 ? (block_size_m <= 128 ? 1 : 2) : (p.seq_q >= 1024 ? 2 : 1);
-    if (dtype == NINETOOTHED_FLOAT16) return dispatch_attention<half_t>(p, (int)head_dim, q_tiles, (hipStream_t)stream);
-    return dispatch_attention<bf16_t>(p, (int)head_dim, q_tiles, (hipStream_t)stream);
+    // block sizes are hints: 256 query rows select the one-workgroup-per-CU
+    // variant, 32-key blocks the three-workgroups-per-CU variant
+    const int variant = block_size_m >= 256 ? 1 : (block_size_n > 0 && block_size_n <= 32 ? 2 : 0);
+    if (dtype == NINETOOTHED_FLOAT16) return dispatch_attention<half_t>(p, (int)head_dim, variant, (hipStream_t)stream);
+    return dispatch_attention<bf16_t>(p, (int)head_dim, variant, (hipStream_t)stream);
 }
