@@ -95,12 +95,25 @@ def build_workloads():
         return dict(step=lambda: kernel(x, w, out, padding_h=1, padding_w=1), work=2.0 * (32 * 56 * 56) * 256 * (256 * 9), bound="mfma", kernel=kernel,
                     describe={"workload": "conv2d fp16 x[32,256,56,56] w[256,256,3,3] stride 1 padding 1 (implicit GEMM)"})
 
+    def copy_1gib():
+        # a plain device-to-device copy of known size: the calibration point for the
+        # HBM traffic counters (FETCH_SIZE / WRITE_SIZE) quoted in profiles/
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+
+        class _Copy:
+            last_plan = "torch copy_ (not part of the library)"
+
+        return dict(step=lambda: dst.copy_(src), work=2.0 * (1 << 30), bound="hbm", kernel=_Copy(),
+                    describe={"workload": "device copy of 1 GiB (2 GiB of traffic), counter calibration only"})
+
     workloads["addmm_8192"] = addmm_8192
     workloads["matmul_512"] = matmul_512
     workloads["softmax_4096"] = softmax_4096
     workloads["attention"] = attention(False)
     workloads["attention_causal"] = attention(True)
     workloads["conv2d"] = conv2d
+    workloads["copy_1gib"] = copy_1gib
     return workloads
 
 
@@ -210,7 +223,7 @@ def main():
     others = {}
     if not args.only:
         for name, factory in workloads.items():
-            if name == args.workload:
+            if name == args.workload or name == "copy_1gib":
                 continue
             workload = factory()
             ms, _ = measure(workload, max(5, args.steps // 2), args.warmup)

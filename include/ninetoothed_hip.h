@@ -102,6 +102,14 @@ NineToothedResult launch_nt_softmax(NineToothedStream stream,
                                     NineToothedTensor output,
                                     int dtype, int block_size);
 
+/* Same as launch_nt_softmax with the kernel variant fixed: 0 = library's
+ * choice, 1 = one wavefront per row segment, 2 = one workgroup per row segment
+ * (measurement aid of the tile selection; no counterpart in the reference). */
+NineToothedResult launch_nt_softmax_config(NineToothedStream stream, int config,
+                                           NineToothedTensor input,
+                                           NineToothedTensor output,
+                                           int dtype, int block_size);
+
 /* o = softmax(scale * q k^T [+ causal mask]) v for q,k,v,o of shape
  * [batch, heads, seq, head_dim] (k/v may have their own seq length).
  * Replaces the kernel generated for tests/test_attention.py:14-70; that

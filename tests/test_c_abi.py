@@ -1,0 +1,74 @@
+"""The C ABI library: it loads, exports every symbol include/ninetoothed_hip.h
+declares, and rejects bad requests without touching a GPU."""
+
+import ctypes
+import pathlib
+import re
+
+import pytest
+
+from ninetoothed_amd import runtime
+
+ROOT = pathlib.Path(__file__).resolve().parent.parent
+HEADER = ROOT / "include" / "ninetoothed_hip.h"
+
+
+def _declared_functions():
+    text = HEADER.read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = re.findall(r"\b(launch_nt_\w+|nt_\w+)\s*\(", text)
+    return sorted(set(names))
+
+
+def test_header_declares_the_entry_points():
+    names = _declared_functions()
+    for expected in ("launch_nt_matmul", "launch_nt_addmm", "launch_nt_softmax", "launch_nt_attention", "launch_nt_conv2d", "nt_tune_gemm"):
+        assert expected in names
+
+
+def test_library_exports_every_declared_symbol():
+    library = ctypes.CDLL(str(runtime.LIBRARY_PATH))
+    for name in _declared_functions():
+        assert hasattr(library, name), f"{name} is declared in the header but not exported"
+
+
+def test_python_binding_covers_the_header():
+    assert set(_declared_functions()) == set(runtime.exported_symbols())
+
+
+def test_version_and_instance_table():
+    library = runtime.library()
+    assert library.nt_version().decode().startswith("nt_hip")
+    names = runtime.gemm_config_names()
+    assert len(names) >= 3 and any("any-stride" in name for name in names)
+    buffer = ctypes.create_string_buffer(8)
+    assert library.nt_gemm_config_name(10_000, buffer, 8) == runtime.NO_KERNEL
+
+
+def test_struct_layout_matches_the_header():
+    # {void *data; uint64_t *shape; int64_t *strides;} passed by value
+    assert ctypes.sizeof(runtime.ArgumentTensor) == 3 * ctypes.sizeof(ctypes.c_void_p)
+    assert [name for name, _ in runtime.ArgumentTensor._fields_] == ["data", "shape", "strides"]
+    scalar = runtime.ArgumentTensor.from_scalar(0.25)
+    assert ctypes.cast(scalar.data, ctypes.POINTER(ctypes.c_double))[0] == 0.25
+    flag = runtime.ArgumentTensor.from_scalar(True)
+    assert ctypes.cast(flag.data, ctypes.POINTER(ctypes.c_int64))[0] == 1
+
+
+def test_launch_error_class():
+    with pytest.raises(runtime.KernelLaunchError, match="error code: 1"):
+        runtime.check(1)
+    runtime.check(0)
+
+
+def test_requests_without_a_kernel_are_refused_on_the_host():
+    # validation happens before any device call, so this runs without a GPU
+    library = runtime.library()
+    a = runtime.ArgumentTensor.from_layout(0, (4, 4), (4, 1))
+    fp64 = runtime.DATA_TYPE_INDEX["fp64"]
+    assert library.launch_nt_matmul(None, a, a, a, fp64, fp64, 0, 0, 0) == runtime.NO_KERNEL
+    assert library.launch_nt_softmax(None, a, a, runtime.DATA_TYPE_INDEX["i32"], 0) == runtime.NO_KERNEL
+    mismatched = runtime.ArgumentTensor.from_layout(0, (5, 4), (4, 1))
+    assert library.launch_nt_matmul(None, a, mismatched, a, runtime.DATA_TYPE_INDEX["fp16"], runtime.DATA_TYPE_INDEX["fp16"], 0, 0, 0) != 0  # hipErrorInvalidValue
+    empty = runtime.ArgumentTensor.from_layout(0, (0, 4), (4, 1))
+    assert library.launch_nt_softmax(None, empty, empty, runtime.DATA_TYPE_INDEX["fp32"], 0) == 0
