@@ -1,0 +1,22 @@
+// Shared between the conv2d entry point (gemm_api.hip) and the repacking
+// implicit-GEMM path (conv2d.hip).
+#pragma once
+
+#include "nt_common.h"
+
+namespace nt {
+
+struct Conv2dRequest {
+    int dtype;
+    const void *x;
+    const void *w;
+    void *y;
+    int N, C, H, W, K, R, S, P, Q, pad_h, pad_w;
+    int64_t xs[4], ws[4], ys[4];  // element strides of input, filter, output
+};
+
+// Runs the direct-to-LDS implicit GEMM when the request qualifies; returns
+// NINETOOTHED_NO_KERNEL when it does not (the caller then uses the gather kernel).
+int conv2d_fast(const Conv2dRequest &request, hipStream_t stream);
+
+}  // namespace nt

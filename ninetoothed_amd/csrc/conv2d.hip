@@ -1,0 +1,357 @@
+// conv2d (stride 1, dilation 1, zero padding) as implicit GEMM on the direct-to-LDS
+// MFMA main loop of gemm_fast.h.
+//
+//   GEMM row  m = (image, out_y, out_x)      M = N*P*Q
+//   GEMM col  j = output channel             K_out
+//   GEMM k    = (filter_y, filter_x, c)      R*S*C, channel fastest
+//
+// The MFMA operands need 8 consecutive k-values per lane, i.e. consecutive
+// CHANNELS of one input position, while NCHW keeps channels H*W elements apart.
+// Two stream-ordered pre-passes therefore repack the operands into temporaries
+// obtained with hipMallocAsync on the launch stream (freed with hipFreeAsync
+// right after the main kernel, so the call stays asynchronous and re-entrant):
+//   x[N,C,H,W]  -> xt[N,H,W,C]              (tiled transpose through LDS, 16-byte accesses)
+//   w[K,C,R,S]  -> wt[(r*S+s)*C + c, K]     (row-major K x N operand of the GEMM)
+// The main kernel then is the 256x256x32, 4-stage GEMM: a K step is 32 channels of
+// one filter tap (r, s); the A rows of a step are 64-byte runs of xt whose
+// addresses differ from step to step by a uniform offset; taps that fall into
+// the padding are fetched with an out-of-range buffer offset, which the
+// hardware returns as zeros.  The epilogue writes NCHW: per output channel the
+// GEMM rows of a tile are contiguous, so the accumulators go through an LDS slab
+// laid out [channel][row] and leave as 16-byte stores.
+//
+// Requirements of this path (anything else uses the any-stride gather kernel):
+// fp16/bf16, C % 32 == 0, K_out % 256 == 0, (P*Q) % 8 == 0, contiguous output.
+#include "conv2d.h"
+#include "gemm_fast.h"
+
+namespace nt {
+namespace {
+
+struct ConvParams {
+    const void *xt;
+    const void *wt;
+    void *y;
+    int N, C, H, W, K, R, S, P, Q, pad_h, pad_w;
+    int tiles_per_image, tiles_m, tiles_n;
+    unsigned xt_bytes;
+};
+
+// ---- pre-pass 1: NCHW (any strides) -> NHWC contiguous ----
+template <typename T>
+__global__ __launch_bounds__(256) void nchw_to_nhwc_kernel(const T *x, T *xt, int C, int HW, int W, int64_t s_n, int64_t s_c,
+                                                          int64_t s_h, int64_t s_w, int vector_ok) {
+    typedef typename Elem<T>::vec8 vec8;
+    constexpr int kPitch = 64 + 8;  // halfs; keeps 16-byte alignment of rows
+    __shared__ __attribute__((aligned(16))) T tile[64 * kPitch];
+    const int hw0 = blockIdx.x * 64, c0 = blockIdx.y * 64, n = blockIdx.z;
+    const int t = threadIdx.x;
+    const T *src = x + (int64_t)n * s_n;
+    // load: rows = channels, 8 consecutive positions per thread
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        const int c = pass * 32 + (t >> 3);
+        const int hw = hw0 + (t & 7) * 8;
+        vec8 v;
+        if (vector_ok && c0 + c < C && hw + 8 <= HW) {
+            v = *(const vec8 *)(src + (int64_t)(c0 + c) * s_c + hw);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int pos = hw + e;
+                v[e] = (c0 + c < C && pos < HW) ? src[(int64_t)(c0 + c) * s_c + (int64_t)(pos / W) * s_h + (int64_t)(pos % W) * s_w] : (T)0.0f;
+            }
+        }
+        *(vec8 *)&tile[c * kPitch + (t & 7) * 8] = v;
+    }
+    __syncthreads();
+    // store: rows = positions, 8 consecutive channels per thread
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        const int hw = pass * 32 + (t >> 3);
+        const int c = (t & 7) * 8;
+        if (hw0 + hw < HW && c0 + c < C) {  // C % 8 == 0 on this path
+            vec8 v;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = tile[(c + e) * kPitch + hw];
+            *(vec8 *)(xt + ((int64_t)n * HW + hw0 + hw) * C + c0 + c) = v;
+        }
+    }
+}
+
+// ---- pre-pass 2: w[K,C,R,S] (any strides) -> wt[(r*S+s)*C + c][K] ----
+template <typename T>
+__global__ __launch_bounds__(256) void filter_to_rsck_kernel(const T *w, T *wt, int K, int C, int R, int S, int64_t s_k,
+                                                            int64_t s_c, int64_t s_r, int64_t s_s) {
+    const int64_t total = (int64_t)K * C * R * S;
+    const int64_t index = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (index >= total) return;
+    const int k = (int)(index % K);
+    const int64_t row = index / K;
+    const int c = (int)(row % C);
+    const int rs = (int)(row / C);
+    wt[index] = w[(int64_t)k * s_k + (int64_t)c * s_c + (int64_t)(rs / S) * s_r + (int64_t)(rs % S) * s_s];
+}
+
+// ---- main kernel ----
+template <typename T>
+__global__ __launch_bounds__(512, 2) void conv2d_nhwc_kernel(ConvParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef Elem<T> E;
+    typedef typename E::vec8 vec8;
+    constexpr int BM = 256, BN = 256, BK = 32, WM = 2, WN = 4, kStages = 4;
+    constexpr int kWaves = WM * WN;
+    constexpr int kWaveM = BM / WM, kWaveN = BN / WN;
+    constexpr int TM = kWaveM / 32, TN = kWaveN / 32;
+    constexpr int kStageA = BM * BK * 2, kStageB = BK * BN * 2;
+    constexpr int kAChunksPerRow = BK / 8, kARowsPerInstr = 64 / kAChunksPerRow;
+    constexpr int kAInstr = kStageA / (kWaves * 1024);
+    constexpr int kBChunksPerRow = BN / 8, kBRowsPerInstr = 64 / kBChunksPerRow;
+    constexpr int kBInstr = kStageB / (kWaves * 1024);
+    constexpr int kLoadsPerTile = kAInstr + kBInstr;
+
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_a0[kStageA];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_a1[kStageA];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_a2[kStageA];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_a3[kStageA];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_b0[kStageB];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_b1[kStageB];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_b2[kStageB];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_b3[kStageB];
+    auto stage_a = [&](auto tag) -> NT_LDS unsigned char * {
+        constexpr int i = decltype(tag)::value;
+        if constexpr (i == 0) return (NT_LDS unsigned char *)lds_a0;
+        else if constexpr (i == 1) return (NT_LDS unsigned char *)lds_a1;
+        else if constexpr (i == 2) return (NT_LDS unsigned char *)lds_a2;
+        else return (NT_LDS unsigned char *)lds_a3;
+    };
+    auto stage_b = [&](auto tag) -> NT_LDS unsigned char * {
+        constexpr int i = decltype(tag)::value;
+        if constexpr (i == 0) return (NT_LDS unsigned char *)lds_b0;
+        else if constexpr (i == 1) return (NT_LDS unsigned char *)lds_b1;
+        else if constexpr (i == 2) return (NT_LDS unsigned char *)lds_b2;
+        else return (NT_LDS unsigned char *)lds_b3;
+    };
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_m = wave / WN, wave_n = wave % WN;
+
+    int tile_m, tile_n;
+    map_tile(p.tiles_m, p.tiles_n, 0, tile_m, tile_n);
+    const int image = tile_m / p.tiles_per_image;
+    const int pq0 = (tile_m % p.tiles_per_image) * BM;
+    const int n0 = tile_n * BN;
+    const int PQ = p.P * p.Q;
+
+    // ---- A: rows of the tile are output positions; per lane one 16-byte chunk of 8 channels ----
+    __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.xt, 0, p.xt_bytes, 0x00020000);
+    __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)((const T *)p.wt + n0), 0, 0xffffffff, 0x00020000);
+    int a_base[kAInstr], a_y[kAInstr], a_x[kAInstr];
+#pragma unroll
+    for (int j = 0; j < kAInstr; ++j) {
+        const int row = (j * kWaves + wave) * kARowsPerInstr + lane / kAChunksPerRow;
+        const int chunk = a_phys_chunk<BK>(row, lane % kAChunksPerRow);
+        const int pq = pq0 + row;
+        const int oy = pq / p.Q, ox = pq - oy * p.Q;
+        a_y[j] = pq < PQ ? oy - p.pad_h : -(1 << 20);  // rows past the image never pass the bounds test
+        a_x[j] = ox - p.pad_w;
+        a_base[j] = pq < PQ ? (((image * p.H + a_y[j]) * p.W + a_x[j]) * p.C + chunk * 8) * 2 : 0;
+    }
+    unsigned b_src[kBInstr];
+#pragma unroll
+    for (int j = 0; j < kBInstr; ++j) {
+        const int krow = (j * kWaves + wave) * kBRowsPerInstr + lane / kBChunksPerRow;
+        const int chunk = b_phys_chunk<BN>(krow, lane % kBChunksPerRow);
+        b_src[j] = (unsigned)(krow * p.K + chunk * 8) * 2u;
+    }
+    const int channel_blocks = p.C / BK;
+    auto issue_loads = [&](auto stage_tag, int kt) {
+        NT_LDS unsigned char *sa = stage_a(stage_tag);
+        NT_LDS unsigned char *sb = stage_b(stage_tag);
+        const int tap = kt / channel_blocks;
+        const int c0 = (kt - tap * channel_blocks) * BK;
+        const int fy = tap / p.S, fx = tap - fy * p.S;
+        const int delta = ((fy * p.W + fx) * p.C + c0) * 2;
+#pragma unroll
+        for (int j = 0; j < kAInstr; ++j) {
+            const bool inside = (unsigned)(a_y[j] + fy) < (unsigned)p.H && (unsigned)(a_x[j] + fx) < (unsigned)p.W;
+            const unsigned offset = inside ? (unsigned)(a_base[j] + delta) : 0x80000000u;  // beyond num_records: reads zeros
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, sa + (j * kWaves + wave) * 1024, 16, offset, 0, 0, 0);
+        }
+        const int b_k = kt * BK * p.K * 2;
+#pragma unroll
+        for (int j = 0; j < kBInstr; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, sb + (j * kWaves + wave) * 1024, 16, b_src[j], b_k, 0, 0);
+    };
+
+    // ---- LDS -> registers (as in gemm_fast.h) ----
+    const int g = lane >> 5, l32 = lane & 31;
+    int a_row_off[TM], a_row_sw[TM];
+#pragma unroll
+    for (int ti = 0; ti < TM; ++ti) {
+        const int row = wave_m * kWaveM + ti * 32 + l32;
+        a_row_off[ti] = row * (BK * 2);
+        a_row_sw[ti] = a_phys_chunk<BK>(row, 0);
+    }
+    const int i16 = lane & 15, nhalf = (lane >> 4) & 1;
+    const int b_krow = 8 * g + (i16 >> 2);
+    int b_col_chunk[TN], b_col_in[TN];
+#pragma unroll
+    for (int tj = 0; tj < TN; ++tj) {
+        const int ncol = wave_n * kWaveN + tj * 32 + nhalf * 16 + 4 * (i16 & 3);
+        b_col_chunk[tj] = ncol >> 3;
+        b_col_in[tj] = (ncol & 7) * 2;
+    }
+
+    float16_t acc[TM][TN];
+#pragma unroll
+    for (int ti = 0; ti < TM; ++ti)
+#pragma unroll
+        for (int tj = 0; tj < TN; ++tj)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[ti][tj][r] = 0.0f;
+
+    auto multiply_stage = [&](auto stage_tag) {
+        const NT_LDS unsigned char *sa = stage_a(stage_tag);
+        const NT_LDS unsigned char *sb = stage_b(stage_tag);
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            vec8 af[TM], bf[TN];
+#pragma unroll
+            for (int ti = 0; ti < TM; ++ti) {
+                const int chunk = (ks * 2 + g) ^ a_row_sw[ti];
+                af[ti] = *(const NT_LDS vec8 *)(sa + a_row_off[ti] + chunk * 16);
+            }
+#pragma unroll
+            for (int tj = 0; tj < TN; ++tj) {
+                const int k_lo = ks * 16 + b_krow, k_hi = k_lo + 4;
+                const int c_lo = b_phys_chunk<BN>(k_lo, b_col_chunk[tj]);
+                const int c_hi = b_phys_chunk<BN>(k_hi, b_col_chunk[tj]);
+                short4_t lo = lds_read_tr16_b64(sb + k_lo * (BN * 2) + c_lo * 16 + b_col_in[tj]);
+                short4_t hi = lds_read_tr16_b64(sb + k_hi * (BN * 2) + c_hi * 16 + b_col_in[tj]);
+                short8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                bf[tj] = __builtin_bit_cast(vec8, both);
+            }
+#pragma unroll
+            for (int ti = 0; ti < TM; ++ti)
+#pragma unroll
+                for (int tj = 0; tj < TN; ++tj) acc[ti][tj] = E::mfma32(af[ti], bf[tj], acc[ti][tj]);
+        }
+    };
+
+    const int num_k = p.R * p.S * channel_blocks;
+    const int last_k = num_k - 1;
+    const int main_k = num_k - num_k % kStages;
+    static_for<0, kStages - 1>([&](auto s) { issue_loads(s, min((int)decltype(s)::value, last_k)); });
+    auto step = [&](auto s, int kt) {
+        constexpr int kS = decltype(s)::value;
+        wait_vmcnt<(kStages - 2) * kLoadsPerTile>();
+        lds_barrier();
+        issue_loads(std::integral_constant<int, (kS + kStages - 1) % kStages>(), min(kt + kS + kStages - 1, last_k));
+        multiply_stage(s);
+    };
+    for (int kt = 0; kt < main_k; kt += kStages) static_for<0, kStages>([&](auto s) { step(s, kt); });
+    static_for<0, kStages - 1>([&](auto s) {
+        if (main_k + (int)decltype(s)::value < num_k) step(s, main_k);
+    });
+    wait_vmcnt<0>();
+    lds_barrier();
+
+    // ---- epilogue: lane holds, per 32x32 tile, output channel l32 and rows 8*(r/4) + 4*g + r%4 ----
+    // slab layout [32 channels][kWaveM rows], 16-byte chunks swizzled by channel; two slabs per stage array
+    constexpr int kRowBytes = kWaveM * 2;  // 256
+    constexpr int kSlabBytes = 32 * kRowBytes;
+    constexpr int kChunks = kWaveM / 8;    // 16
+    NT_LDS unsigned char *slab;
+    {
+        const int which = wave >> 1;
+        slab = which == 0 ? (NT_LDS unsigned char *)lds_a0
+               : which == 1 ? (NT_LDS unsigned char *)lds_b0
+               : which == 2 ? (NT_LDS unsigned char *)lds_a1
+                            : (NT_LDS unsigned char *)lds_b1;
+        slab += (wave & 1) * kSlabBytes;
+    }
+    T *Y = (T *)p.y + (int64_t)image * p.K * PQ;
+#pragma unroll
+    for (int tj = 0; tj < TN; ++tj) {
+#pragma unroll
+        for (int ti = 0; ti < TM; ++ti)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                typedef T vec4 __attribute__((ext_vector_type(4)));
+                vec4 v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = E::from_float(acc[ti][tj][4 * r4 + e]);
+                const int chunk = (ti * 4 + r4) ^ (l32 & (kChunks - 1));
+                *(NT_LDS vec4 *)(slab + l32 * kRowBytes + chunk * 16 + 8 * g) = v;
+            }
+#pragma unroll
+        for (int it = 0; it < (32 * kChunks) / 64; ++it) {
+            const int idx = it * 64 + lane;
+            const int channel = idx / kChunks;
+            const int phys = idx % kChunks;
+            const int chunk = phys ^ (channel & (kChunks - 1));
+            vec8 v = *(const NT_LDS vec8 *)(slab + channel * kRowBytes + phys * 16);
+            const int pq = pq0 + wave_m * kWaveM + chunk * 8;
+            const int out_channel = n0 + wave_n * kWaveN + tj * 32 + channel;
+            if (pq < PQ) *(vec8 *)(Y + (int64_t)out_channel * PQ + pq) = v;  // PQ % 8 == 0: chunks are all-in or all-out
+        }
+    }
+#endif
+}
+
+template <typename T>
+int run_fast(const Conv2dRequest &q, hipStream_t stream) {
+    const int64_t xt_bytes = (int64_t)q.N * q.H * q.W * q.C * 2;
+    const int64_t wt_bytes = (int64_t)q.K * q.C * q.R * q.S * 2;
+    void *xt = nullptr, *wt = nullptr;
+    hipError_t err = hipMallocAsync(&xt, (size_t)xt_bytes, stream);
+    if (err != hipSuccess) return NINETOOTHED_NO_KERNEL;  // no temporary: the caller falls back to the gather kernel
+    err = hipMallocAsync(&wt, (size_t)wt_bytes, stream);
+    if (err != hipSuccess) {
+        (void)hipFreeAsync(xt, stream);
+        return NINETOOTHED_NO_KERNEL;
+    }
+    const int HW = q.H * q.W;
+    const int vector_ok = q.xs[3] == 1 && q.xs[2] == q.W && HW % 8 == 0 && q.xs[1] % 8 == 0 && q.xs[0] % 8 == 0 && ((uintptr_t)q.x & 15) == 0;
+    nchw_to_nhwc_kernel<T><<<dim3(ceil_div(HW, 64), ceil_div(q.C, 64), q.N), dim3(256), 0, stream>>>(
+        (const T *)q.x, (T *)xt, q.C, HW, q.W, q.xs[0], q.xs[1], q.xs[2], q.xs[3], vector_ok);
+    const int64_t filter_elems = (int64_t)q.K * q.C * q.R * q.S;
+    filter_to_rsck_kernel<T><<<dim3((unsigned)((filter_elems + 255) / 256)), dim3(256), 0, stream>>>(
+        (const T *)q.w, (T *)wt, q.K, q.C, q.R, q.S, q.ws[0], q.ws[1], q.ws[2], q.ws[3]);
+    ConvParams p;
+    p.xt = xt;
+    p.wt = wt;
+    p.y = q.y;
+    p.N = q.N; p.C = q.C; p.H = q.H; p.W = q.W; p.K = q.K; p.R = q.R; p.S = q.S; p.P = q.P; p.Q = q.Q;
+    p.pad_h = q.pad_h; p.pad_w = q.pad_w;
+    p.tiles_per_image = ceil_div(q.P * q.Q, 256);
+    p.tiles_m = q.N * p.tiles_per_image;
+    p.tiles_n = q.K / 256;
+    p.xt_bytes = (unsigned)xt_bytes;
+    conv2d_nhwc_kernel<T><<<dim3(p.tiles_m * p.tiles_n), dim3(512), 0, stream>>>(p);
+    err = hipGetLastError();
+    (void)hipFreeAsync(xt, stream);
+    (void)hipFreeAsync(wt, stream);
+    return (int)err;
+}
+
+}  // namespace
+
+int conv2d_fast(const Conv2dRequest &q, hipStream_t stream) {
+    if (q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) return NINETOOTHED_NO_KERNEL;
+    if (q.C % 32 || q.K % 256 || (q.P * q.Q) % 8) return NINETOOTHED_NO_KERNEL;
+    if (q.ys[3] != 1 || q.ys[2] != q.Q || q.ys[1] != (int64_t)q.P * q.Q || q.ys[0] != (int64_t)q.K * q.P * q.Q) return NINETOOTHED_NO_KERNEL;
+    if (((uintptr_t)q.y & 15) != 0) return NINETOOTHED_NO_KERNEL;
+    const int64_t xt_bytes = (int64_t)q.N * q.H * q.W * q.C * 2;
+    const int64_t wt_bytes = (int64_t)q.K * q.C * q.R * q.S * 2;
+    if (xt_bytes >= (int64_t(1) << 31) || wt_bytes >= (int64_t(1) << 31)) return NINETOOTHED_NO_KERNEL;  // 32-bit buffer offsets
+    if ((int64_t)q.N * ceil_div(q.P * q.Q, 256) * (q.K / 256) > 0x7fffffffll) return NINETOOTHED_NO_KERNEL;
+    // enough work to amortise the two repacking passes
+    if ((int64_t)q.N * q.P * q.Q < 1024) return NINETOOTHED_NO_KERNEL;
+    return q.dtype == NINETOOTHED_FLOAT16 ? run_fast<half_t>(q, stream) : run_fast<bf16_t>(q, stream);
+}
+
+}  // namespace nt

@@ -7,6 +7,7 @@
 #include <cstdio>
 #include <cstring>
 
+#include "conv2d.h"
 #include "gemm_fast.h"
 #include "gemm_generic.h"
 
@@ -358,7 +359,6 @@ NineToothedResult nt_tune_gemm(NineToothedStream stream_, NineToothedTensor inpu
 NineToothedResult launch_nt_conv2d(NineToothedStream stream, NineToothedTensor input, NineToothedTensor filter,
                                    NineToothedTensor output, int dtype, int padding_h, int padding_w, int block_size_m,
                                    int block_size_n, int block_size_k) {
-    (void)block_size_m;
     (void)block_size_n;
     (void)block_size_k;
     if (dtype != NINETOOTHED_FLOAT16 && dtype != NINETOOTHED_BFLOAT16) return NINETOOTHED_NO_KERNEL;
@@ -374,6 +374,23 @@ NineToothedResult launch_nt_conv2d(NineToothedStream stream, NineToothedTensor i
     if (P <= 0 || Q <= 0 || N == 0 || K == 0) return 0;  // nothing to write
     const int64_t gm = N * P * Q, gk = C * R * S;
     if (gm > 0x7fffffffll || gk > 0x7fffffffll || K > 0x7fffffffll) return NINETOOTHED_NO_KERNEL;
+    {
+        Conv2dRequest request;
+        request.dtype = dtype;
+        request.x = input.data;
+        request.w = filter.data;
+        request.y = output.data;
+        request.N = (int)N; request.C = (int)C; request.H = (int)H; request.W = (int)W;
+        request.K = (int)K; request.R = (int)R; request.S = (int)S; request.P = (int)P; request.Q = (int)Q;
+        request.pad_h = padding_h; request.pad_w = padding_w;
+        for (int d = 0; d < 4; ++d) {
+            request.xs[d] = input.strides[d];
+            request.ws[d] = filter.strides[d];
+            request.ys[d] = output.strides[d];
+        }
+        const int fast = block_size_m == 1 ? NINETOOTHED_NO_KERNEL : conv2d_fast(request, (hipStream_t)stream);
+        if (fast != NINETOOTHED_NO_KERNEL) return fast;
+    }
     auto launch = [&](auto tag) -> hipError_t {
         typedef decltype(tag) T;
         Conv2dProblem<T> prob;
