@@ -34,8 +34,9 @@ struct AttentionParams {
 
 constexpr int kAttnWaves = 4;
 
-// BN: key/value rows per block; kOcc: waves per SIMD the register budget is held to
-template <typename T, int D, int kQTiles, int BN, int kOcc>
+// BN: key/value rows per block; kOcc: waves per SIMD the register budget is held to;
+// kPipelined: overlap the softmax of a block with the MFMAs of its neighbours
+template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined>
 __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(AttentionParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     typedef Elem<T> E;
@@ -56,11 +57,11 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
     __shared__ __attribute__((aligned(1024))) unsigned char lds_v0[kTileBytes];
     __shared__ __attribute__((aligned(1024))) unsigned char lds_k1[kTileBytes];
     __shared__ __attribute__((aligned(1024))) unsigned char lds_v1[kTileBytes];
-    auto stage_k = [&](auto tag) -> NT_LDS unsigned char * {
+    auto stage_k = [&](auto tag) __attribute__((always_inline)) -> NT_LDS unsigned char * {
         if constexpr (decltype(tag)::value == 0) return (NT_LDS unsigned char *)lds_k0;
         else return (NT_LDS unsigned char *)lds_k1;
     };
-    auto stage_v = [&](auto tag) -> NT_LDS unsigned char * {
+    auto stage_v = [&](auto tag) __attribute__((always_inline)) -> NT_LDS unsigned char * {
         if constexpr (decltype(tag)::value == 0) return (NT_LDS unsigned char *)lds_v0;
         else return (NT_LDS unsigned char *)lds_v1;
     };
@@ -118,43 +119,64 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
     const int last_block = num_blocks - 1;
 
     // ---- global -> LDS assignment ----
-    int ld_row[kInstr];
-    unsigned ld_k_col[kInstr], ld_v_col[kInstr];
-#pragma unroll
-    for (int j = 0; j < kInstr; ++j) {
-        const int row = (j * kAttnWaves + wave) * kRowsPerInstr + lane / kChunksPerRow;
+    // K and V of this (batch, head) are addressed through buffer descriptors that
+    // end with the last key row: the per-lane byte offset is fixed for the whole
+    // kernel, the block offset travels in a scalar register, and rows past the end
+    // of the sequence read as zeros (the range check covers the scalar offset too).
+    const unsigned k_bytes = (unsigned)((p.seq_k - 1) * p.k_strides[2] + D) * 2u;
+    const unsigned v_bytes = (unsigned)((p.seq_k - 1) * p.v_strides[2] + D) * 2u;
+    __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)K, 0, k_bytes, 0x00020000);
+    __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)V, 0, v_bytes, 0x00020000);
+    const unsigned k_block_bytes = (unsigned)(BN * p.k_strides[2]) * 2u;
+    const unsigned v_block_bytes = (unsigned)(BN * p.v_strides[2]) * 2u;
+    // load instruction j of a wave covers the rows kLoadRowStep * j further down; both
+    // swizzles repeat with that period, so one lane offset serves every j and the
+    // row step goes into the scalar offset as well
+    constexpr int kLoadRowStep = kAttnWaves * kRowsPerInstr;
+    static_assert(a_phys_chunk<D>(kLoadRowStep, 0) == 0 && b_phys_chunk<D>(kLoadRowStep, 0) == 0, "swizzle period");
+    const unsigned k_step_bytes = (unsigned)(kLoadRowStep * p.k_strides[2]) * 2u;
+    const unsigned v_step_bytes = (unsigned)(kLoadRowStep * p.v_strides[2]) * 2u;
+    unsigned ld_k_off, ld_v_off;
+    {
+        const int row = wave * kRowsPerInstr + lane / kChunksPerRow;
         const int phys = lane % kChunksPerRow;
-        ld_row[j] = row;
-        ld_k_col[j] = a_phys_chunk<D>(row, phys) * 8;
-        ld_v_col[j] = b_phys_chunk<D>(row, phys) * 8;
+        ld_k_off = ((unsigned)row * (unsigned)p.k_strides[2] + a_phys_chunk<D>(row, phys) * 8) * 2u;
+        ld_v_off = ((unsigned)row * (unsigned)p.v_strides[2] + b_phys_chunk<D>(row, phys) * 8) * 2u;
     }
-    auto issue_loads = [&](auto stage_tag, int blk) {
+    auto issue_k = [&](auto stage_tag, int blk) __attribute__((always_inline)) {
         NT_LDS unsigned char *sk = stage_k(stage_tag);
-        NT_LDS unsigned char *sv = stage_v(stage_tag);
+        const unsigned block_off = (unsigned)blk * k_block_bytes;
 #pragma unroll
-        for (int j = 0; j < kInstr; ++j) {
-            const int row = min(blk * BN + ld_row[j], p.seq_k - 1);  // rows past the end are masked later
-            global_to_lds_16(K + (int64_t)row * p.k_strides[2] + ld_k_col[j], sk + (j * kAttnWaves + wave) * 1024);
-            global_to_lds_16(V + (int64_t)row * p.v_strides[2] + ld_v_col[j], sv + (j * kAttnWaves + wave) * 1024);
-        }
+        for (int j = 0; j < kInstr; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, sk + (j * kAttnWaves + wave) * 1024, 16, ld_k_off, block_off + j * k_step_bytes, 0, 0);
+    };
+    auto issue_v = [&](auto stage_tag, int blk) __attribute__((always_inline)) {
+        NT_LDS unsigned char *sv = stage_v(stage_tag);
+        const unsigned block_off = (unsigned)blk * v_block_bytes;
+#pragma unroll
+        for (int j = 0; j < kInstr; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, sv + (j * kAttnWaves + wave) * 1024, 16, ld_v_off, block_off + j * v_step_bytes, 0, 0);
     };
 
     // ---- LDS read offsets ----
-    int k_row_off[KT], k_row_sw[KT];
+    // K: lane reads row kt * 32 + l32, 16-byte chunk 2 * ks + g.  The swizzle of a
+    // row repeats every 16 rows, so one offset per contraction step serves all kt
+    // (the tile offset is an immediate).
+    static_assert(a_phys_chunk<D>(32, 0) == 0, "K swizzle period");
+    int k_off[KS];
 #pragma unroll
-    for (int kt = 0; kt < KT; ++kt) {
-        const int row = kt * 32 + l32;
-        k_row_off[kt] = row * (D * 2);
-        k_row_sw[kt] = a_phys_chunk<D>(row, 0);
-    }
+    for (int ks = 0; ks < KS; ++ks) k_off[ks] = l32 * (D * 2) + a_phys_chunk<D>(l32, ks * 2 + g) * 16;
+    // V (transposing read): lane i of a 16-lane group addresses row 4g + i/4 (+ 16 per
+    // contraction step, + 8 for the upper slots), columns 4 * (i % 4) of the group's 16.
+    // The swizzle only looks at the row modulo 8 or less, so one offset per d tile.
+    static_assert(b_phys_chunk<D>(8, 0) == 0, "V swizzle period");
     const int i16 = lane & 15;
-    const int v_row = 4 * g + (i16 >> 2);  // + 16 * step (+ 8 for the upper slots)
-    int v_col_chunk[DT], v_col_in[DT];
+    int v_off[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
+        const int row = 4 * g + (i16 >> 2);
         const int col = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
-        v_col_chunk[dt] = col >> 3;
-        v_col_in[dt] = (col & 7) * 2;
+        v_off[dt] = row * (D * 2) + b_phys_chunk<D>(row, col >> 3) * 16 + (col & 7) * 2;
     }
 
     float16_t o_acc[DT][kQTiles];
@@ -171,12 +193,9 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
         l_run[qt] = 0.0f;
     }
 
-    auto process_block = [&](auto stage_tag, int blk) {
+    // S^T = K . Q'^T for the block held in a K stage
+    auto scores = [&](auto stage_tag, float16_t (&s_acc)[KT][kQTiles]) __attribute__((always_inline)) {
         const NT_LDS unsigned char *sk = stage_k(stage_tag);
-        const NT_LDS unsigned char *sv = stage_v(stage_tag);
-
-        // S^T = K . Q'^T
-        float16_t s_acc[KT][kQTiles];
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
@@ -187,35 +206,43 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
         for (int ks = 0; ks < KS; ++ks) {
             vec8 kf[KT];
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt) {
-                const int chunk = (ks * 2 + g) ^ k_row_sw[kt];
-                kf[kt] = *(const NT_LDS vec8 *)(sk + k_row_off[kt] + chunk * 16);
-            }
+            for (int kt = 0; kt < KT; ++kt) kf[kt] = *(const NT_LDS vec8 *)(sk + k_off[ks] + kt * (32 * D * 2));
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
                 for (int qt = 0; qt < kQTiles; ++qt) s_acc[kt][qt] = E::mfma32(kf[kt], qf[qt][ks], s_acc[kt][qt]);
         }
+    };
 
-        // masks: keys past the end of the sequence, and (causal) keys after the query
+    // masks of block `blk`: keys past the end of the sequence, and (causal) keys
+    // after the query.  Few blocks need them (the last one, the ones on the
+    // diagonal), so the callers branch on needs_masks (uniform over the wave) to a
+    // copy of the block's code with or without the masking arithmetic.
+    auto needs_masks = [&](int blk) __attribute__((always_inline)) -> bool {
         const int kv0 = blk * BN;
         const bool mask_tail = kv0 + BN > p.seq_k || blk > last_block;
         const bool mask_causal = p.causal && (kv0 + BN - 1 > q0 + wave * kQTiles * 32);
-        if (mask_tail || mask_causal) {
-            const int limit = blk > last_block ? 0 : p.seq_k;
+        return mask_tail || mask_causal;
+    };
+    auto apply_masks = [&](float16_t (&s_acc)[KT][kQTiles], int blk) __attribute__((always_inline)) {
+        const int kv0 = blk * BN;
+        const int limit = blk > last_block ? 0 : p.seq_k;
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt)
+        for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-                for (int qt = 0; qt < kQTiles; ++qt)
+            for (int qt = 0; qt < kQTiles; ++qt)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int kv = kv0 + kt * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
-                        const bool keep = kv < limit && (!p.causal || q_row[qt] >= kv);
-                        if (!keep) s_acc[kt][qt][r] = -INFINITY;
-                    }
-        }
+                for (int r = 0; r < 16; ++r) {
+                    const int kv = kv0 + kt * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+                    const bool keep = kv < limit && (!p.causal || q_row[qt] >= kv);
+                    if (!keep) s_acc[kt][qt][r] = -INFINITY;
+                }
+    };
 
-        // online softmax per query row (= per lane and q tile)
+    // online softmax: turns (masked) S^T into P^T operand fragments, updates the
+    // running maximum / sum, returns the factor the output has to be rescaled by
+    // (per q tile; 1 when the maximum did not move)
+    auto softmax = [&](float16_t (&s_acc)[KT][kQTiles], vec8 (&pf)[PS][kQTiles], float (&alpha)[kQTiles]) __attribute__((always_inline)) {
 #pragma unroll
         for (int qt = 0; qt < kQTiles; ++qt) {
             float mx = -INFINITY;
@@ -223,10 +250,14 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
             for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s_acc[kt][qt][r]);
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            {   // exchange with lane ^ 32 in registers (no LDS round trip)
+                const unsigned bits = __builtin_bit_cast(unsigned, mx);
+                auto halves = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+                mx = fmaxf(__builtin_bit_cast(float, (unsigned)halves[0]), __builtin_bit_cast(float, (unsigned)halves[1]));
+            }
             const float m_new = fmaxf(m_run[qt], mx);
             const float m_use = m_new == -INFINITY ? 0.0f : m_new;  // fully masked so far
-            const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_use);
+            alpha[qt] = __builtin_amdgcn_exp2f(m_run[qt] - m_use);
             m_run[qt] = m_new;
             float sum = 0.0f;
 #pragma unroll
@@ -237,61 +268,190 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
                     s_acc[kt][qt][r] = pv;
                     sum += pv;
                 }
-            l_run[qt] = l_run[qt] * alpha + sum;
-            // the running maximum settles after a few blocks; skip the rescale of the
-            // output accumulators when no row of this wave's tile moved (wave-uniform)
-            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) o_acc[dt][qt][r] *= alpha;
-            }
+            l_run[qt] = l_run[qt] * alpha[qt] + sum;
         }
-
-        // O^T += V^T . P^T
 #pragma unroll
-        for (int ps = 0; ps < PS; ++ps) {
-            vec8 pf[kQTiles];
+        for (int ps = 0; ps < PS; ++ps)
 #pragma unroll
             for (int qt = 0; qt < kQTiles; ++qt)
 #pragma unroll
-                for (int e = 0; e < 8; ++e) pf[qt][e] = E::from_float(s_acc[ps / 2][qt][8 * (ps & 1) + e]);
+                for (int e = 0; e < 8; ++e) pf[ps][qt][e] = E::from_float(s_acc[ps / 2][qt][8 * (ps & 1) + e]);
+    };
+
+    // the running maximum settles after a few blocks; skip the rescale of the
+    // output accumulators when no row of this wave's tile moved (wave-uniform)
+    auto rescale = [&](const float (&alpha)[kQTiles]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int qt = 0; qt < kQTiles; ++qt) {
+            if (__builtin_amdgcn_ballot_w64(alpha[qt] != 1.0f) != 0) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) o_acc[dt][qt][r] *= alpha[qt];
+            }
+        }
+    };
+
+    // O^T += V^T . P^T for the block held in a V stage
+    auto accumulate = [&](auto stage_tag, const vec8 (&pf)[PS][kQTiles]) __attribute__((always_inline)) {
+        const NT_LDS unsigned char *sv = stage_v(stage_tag);
+#pragma unroll
+        for (int ps = 0; ps < PS; ++ps) {
             vec8 vf[DT];
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-                const int r_lo = ps * 16 + v_row;
-                const int r_hi = r_lo + 8;
-                const int c_lo = b_phys_chunk<D>(r_lo, v_col_chunk[dt]);
-                const int c_hi = b_phys_chunk<D>(r_hi, v_col_chunk[dt]);
-                short4_t lo = lds_read_tr16_b64(sv + r_lo * (D * 2) + c_lo * 16 + v_col_in[dt]);
-                short4_t hi = lds_read_tr16_b64(sv + r_hi * (D * 2) + c_hi * 16 + v_col_in[dt]);
+                short4_t lo = lds_read_tr16_b64(sv + v_off[dt] + (ps * 16) * (D * 2));
+                short4_t hi = lds_read_tr16_b64(sv + v_off[dt] + (ps * 16 + 8) * (D * 2));
                 short8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
                 vf[dt] = __builtin_bit_cast(vec8, both);
             }
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-                for (int qt = 0; qt < kQTiles; ++qt) o_acc[dt][qt] = E::mfma32(vf[dt], pf[qt], o_acc[dt][qt]);
+                for (int qt = 0; qt < kQTiles; ++qt) o_acc[dt][qt] = E::mfma32(vf[dt], pf[ps][qt], o_acc[dt][qt]);
         }
     };
 
-    // two LDS stages, loop unrolled by two; an odd block count runs one fully
-    // masked extra block, whose loads re-fetch the last block
+    // A stage may be overwritten by the loads issued right after a barrier, so a wave
+    // only arrives at the barrier once its own reads of that stage have returned: an
+    // LDS read that is merely issued can still be queued behind other waves' reads
+    // when the (L2-fast) load of the next block lands.
+    auto stage_barrier = [&]() __attribute__((always_inline)) {
+        wait_lgkmcnt<0>();
+        lds_barrier();
+    };
     typedef std::integral_constant<int, 0> Stage0;
     typedef std::integral_constant<int, 1> Stage1;
-    if (num_blocks > 0) {
-        issue_loads(Stage0(), 0);
-        for (int blk = 0; blk < num_blocks; blk += 2) {
-            wait_vmcnt<0>();
-            lds_barrier();
-            issue_loads(Stage1(), min(blk + 1, last_block));
-            process_block(Stage0(), blk);
-            wait_vmcnt<0>();
-            lds_barrier();
-            issue_loads(Stage0(), min(blk + 2, last_block));
-            process_block(Stage1(), blk + 1);
+    if constexpr (!kPipelined) {
+        // two LDS stages, loop unrolled by two; an odd block count runs one fully
+        // masked extra block, whose loads re-fetch the last block
+        auto block = [&](auto stage_tag, int blk) __attribute__((always_inline)) {
+            float16_t s_acc[KT][kQTiles];
+            vec8 pf[PS][kQTiles];
+            float alpha[kQTiles];
+            scores(stage_tag, s_acc);
+            if (needs_masks(blk)) apply_masks(s_acc, blk);
+            softmax(s_acc, pf, alpha);
+            rescale(alpha);
+            accumulate(stage_tag, pf);
+        };
+        if (num_blocks > 0) {
+            issue_k(Stage0(), 0);
+            issue_v(Stage0(), 0);
+            for (int blk = 0; blk < num_blocks; blk += 2) {
+                wait_vmcnt<0>();
+                stage_barrier();
+                issue_k(Stage1(), min(blk + 1, last_block));
+                issue_v(Stage1(), min(blk + 1, last_block));
+                block(Stage0(), blk);
+                wait_vmcnt<0>();
+                stage_barrier();
+                issue_k(Stage0(), min(blk + 2, last_block));
+                issue_v(Stage0(), min(blk + 2, last_block));
+                block(Stage1(), blk + 1);
+            }
+            wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup ends
         }
-        wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup ends
+    } else {
+        // Software pipeline over key blocks.  Step j holds S(j) from the previous
+        // step and runs three mutually independent pieces that the instruction
+        // scheduler can interleave: the softmax of block j (VALU), the MFMAs of
+        // P(j-1) . V(j-1), and the MFMAs of K(j+1) . Q.  K(j+1) and V(j-1) sit in
+        // the stage opposite to the step's parity; K(j+2) and V(j) are requested
+        // into the step's own stage.  Past the end the last K block is fetched and
+        // multiplied again (its scores are never used), which keeps the steps uniform.
+        if (num_blocks > 0) {
+            // S(j) and P(j) live in the buffers of j's parity, so nothing is copied
+            float16_t s_buf[2][KT][kQTiles];
+            vec8 p_buf[2][PS][kQTiles];
+            float alpha[kQTiles];
+            issue_k(Stage0(), 0);
+            issue_k(Stage1(), min(1, last_block));
+            wait_vmcnt<kInstr>();
+            stage_barrier();
+            scores(Stage0(), s_buf[0]);
+            // step 0: nothing to accumulate yet
+            wait_vmcnt<0>();
+            stage_barrier();
+            issue_k(Stage0(), min(2, last_block));
+            issue_v(Stage0(), 0);
+            if (needs_masks(0)) apply_masks(s_buf[0], 0);
+            softmax(s_buf[0], p_buf[0], alpha);
+            scores(Stage1(), s_buf[1]);
+
+            auto step_body = [&](auto parity_tag, auto masked_tag, int j) __attribute__((always_inline)) {
+                constexpr int kParity = decltype(parity_tag)::value;
+                typedef std::integral_constant<int, kParity> Own;
+                typedef std::integral_constant<int, 1 - kParity> Other;
+                wait_vmcnt<0>();
+                stage_barrier();
+                issue_k(Own(), min(j + 2, last_block));
+                issue_v(Own(), j);
+                __builtin_amdgcn_sched_barrier(0);  // nothing of this step moves above the barrier
+                if constexpr (decltype(masked_tag)::value) apply_masks(s_buf[kParity], j);
+                softmax(s_buf[kParity], p_buf[kParity], alpha);
+                accumulate(Other(), p_buf[1 - kParity]);
+                scores(Other(), s_buf[1 - kParity]);
+                // desired issue order inside this region: one MFMA, then the LDS reads
+                // and softmax arithmetic that fit under it
+#ifndef NT_ATTN_SCHEDULE
+#define NT_ATTN_SCHEDULE 1
+#endif
+#if NT_ATTN_SCHEDULE
+                // Issue order asked of the scheduler: LDS reads run three MFMAs ahead; every
+                // MFMA (32 cycles in the matrix pipe) is followed by the operand reads of a
+                // later one and by at most 28 cycles of softmax arithmetic (4 per VALU
+                // instruction, 8 per exponential).  The first MFMAs overlap the running-max
+                // chain, the exponentials start once the maximum is known.
+                constexpr int kMfmaPerStep = (PS * DT + KS * KT) * kQTiles;
+                __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+                static_for<0, kMfmaPerStep>([&](auto i_tag) __attribute__((always_inline)) {
+                    constexpr int i = decltype(i_tag)::value;
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                    if constexpr (i < kMfmaPerStep / 8) {
+                        __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+                    } else {
+                        __builtin_amdgcn_sched_group_barrier(0x400, (i % 4 == 0) ? 2 : 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+                    }
+                });
+#endif
+                // P(j) and the row sums are only consumed in later steps; pin them here so
+                // that their arithmetic stays in this step, next to the MFMAs it overlaps with
+#pragma unroll
+                for (int ps = 0; ps < PS; ++ps)
+#pragma unroll
+                    for (int qt = 0; qt < kQTiles; ++qt) asm volatile("" : "+v"(p_buf[kParity][ps][qt]));
+#pragma unroll
+                for (int qt = 0; qt < kQTiles; ++qt) asm volatile("" : "+v"(l_run[qt]));
+                rescale(alpha);
+            };
+            // The blocks that need masks are the last ones.  A first loop runs the pairs
+            // of steps that lie entirely before them without the masking arithmetic, a
+            // second one the rest with it (masking a block that does not need it changes
+            // nothing).  The split differs between the waves of a workgroup; the number of
+            // steps, and with it the number of barriers, does not.
+            int unmasked = p.seq_k / BN;
+            if (p.causal) unmasked = min(unmasked, (q0 + wave * kQTiles * 32 + 1) / BN);
+            int j = 1;
+            for (; j + 1 < unmasked; j += 2) {
+                step_body(Stage1(), std::false_type(), j);
+                step_body(Stage0(), std::false_type(), j + 1);
+            }
+            for (; j + 1 < num_blocks; j += 2) {
+                step_body(Stage1(), std::true_type(), j);
+                step_body(Stage0(), std::true_type(), j + 1);
+            }
+            if (j < num_blocks) step_body(Stage1(), std::true_type(), j);
+            // drain: P(last) . V(last); V(last) was requested into the stage of its parity
+            wait_vmcnt<0>();
+            stage_barrier();
+            if ((num_blocks - 1) & 1)
+                accumulate(Stage1(), p_buf[1]);
+            else
+                accumulate(Stage0(), p_buf[0]);
+        }
     }
 
     // ---- epilogue: O[q, d] = O^T[d, q] / l ----
@@ -316,32 +476,37 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
 #endif
 }
 
-template <typename T, int D, int kQTiles, int BN, int kOcc>
+template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined>
 hipError_t launch_attention(AttentionParams &p, hipStream_t stream) {
     constexpr int BM = kAttnWaves * 32 * kQTiles;
     p.q_blocks = ceil_div(p.seq_q, BM);
     const int64_t grid = (int64_t)p.batch * p.heads * p.q_blocks;
     if (grid == 0) return hipSuccess;
-    attention_fwd_kernel<T, D, kQTiles, BN, kOcc><<<dim3((unsigned)grid), dim3(kAttnWaves * 64), 0, stream>>>(p);
+    attention_fwd_kernel<T, D, kQTiles, BN, kOcc, kPipelined><<<dim3((unsigned)grid), dim3(kAttnWaves * 64), 0, stream>>>(p);
     return hipGetLastError();
 }
 
 // variant: 0 = 128 query rows per workgroup, 64-key blocks, two workgroups per CU (default)
 //          1 = 256 query rows per workgroup, 64-key blocks, one workgroup per CU
 //          2 = 128 query rows per workgroup, 32-key blocks, three workgroups per CU
+//          3 = variant 0 with the software-pipelined main loop, 4 = variant 1 with it
 template <typename T>
 int dispatch_attention(AttentionParams &p, int head_dim, int variant, hipStream_t stream) {
     if (head_dim == 128) {
-        if (variant == 1) return (int)launch_attention<T, 128, 2, 64, 1>(p, stream);
-        if (variant == 2) return (int)launch_attention<T, 128, 1, 32, 3>(p, stream);
-        return (int)launch_attention<T, 128, 1, 64, 2>(p, stream);
+        if (variant == 3) return (int)launch_attention<T, 128, 1, 64, 2, true>(p, stream);
+        if (variant == 4) return (int)launch_attention<T, 128, 2, 64, 1, true>(p, stream);
+        if (variant == 1) return (int)launch_attention<T, 128, 2, 64, 1, false>(p, stream);
+        if (variant == 2) return (int)launch_attention<T, 128, 1, 32, 3, false>(p, stream);
+        return (int)launch_attention<T, 128, 1, 64, 2, false>(p, stream);
     }
     if (head_dim == 64) {
-        if (variant == 1) return (int)launch_attention<T, 64, 2, 64, 1>(p, stream);
-        if (variant == 2) return (int)launch_attention<T, 64, 1, 32, 3>(p, stream);
-        return (int)launch_attention<T, 64, 1, 64, 2>(p, stream);
+        if (variant == 3) return (int)launch_attention<T, 64, 1, 64, 2, true>(p, stream);
+        if (variant == 4) return (int)launch_attention<T, 64, 2, 64, 1, true>(p, stream);
+        if (variant == 1) return (int)launch_attention<T, 64, 2, 64, 1, false>(p, stream);
+        if (variant == 2) return (int)launch_attention<T, 64, 1, 32, 3, false>(p, stream);
+        return (int)launch_attention<T, 64, 1, 64, 2, false>(p, stream);
     }
-    if (head_dim == 32) return (int)launch_attention<T, 32, 1, 64, 2>(p, stream);
+    if (head_dim == 32) return (int)launch_attention<T, 32, 1, 64, 2, false>(p, stream);
     return NINETOOTHED_NO_KERNEL;
 }
 
@@ -371,6 +536,11 @@ extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineT
     }
     if (v.shape[2] != k.shape[2] || o.shape[2] != q.shape[2]) return hipErrorInvalidValue;
     if (q.shape[2] > 0x7fffffffull || k.shape[2] > 0x7fffffffull) return NINETOOTHED_NO_KERNEL;
+    // K and V of one (batch, head) are read through 32-bit buffer offsets
+    for (const NineToothedTensor *t : {&k, &v}) {
+        if (t->strides[2] < 0) return NINETOOTHED_NO_KERNEL;
+        if (((int64_t)t->shape[2] + 64) * t->strides[2] * 2 + 2 * head_dim > 0xffffffffll) return NINETOOTHED_NO_KERNEL;
+    }
     if (p.batch == 0 || p.heads == 0 || p.seq_q == 0) return 0;
     if (p.seq_k == 0) return NINETOOTHED_NO_KERNEL;  // softmax over nothing
     for (int d = 0; d < 3; ++d) {
@@ -388,7 +558,8 @@ extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineT
     p.causal = is_causal.data ? (Scalar0d::as_int64(is_causal) != 0) : 0;
     // block sizes are hints: 256 query rows select the one-workgroup-per-CU
     // variant, 32-key blocks the three-workgroups-per-CU variant
-    const int variant = block_size_m >= 256 ? 1 : (block_size_n > 0 && block_size_n <= 32 ? 2 : 0);
+    int variant = block_size_m >= 256 ? 1 : (block_size_n > 0 && block_size_n <= 32 ? 2 : 3);
+    if (block_size_n >= 1000) variant = block_size_n - 1000;  // measurement aid: explicit variant
     if (dtype == NINETOOTHED_FLOAT16) return dispatch_attention<half_t>(p, (int)head_dim, variant, (hipStream_t)stream);
     return dispatch_attention<bf16_t>(p, (int)head_dim, variant, (hipStream_t)stream);
 }
