@@ -312,14 +312,6 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
         }
     };
 
-    // A stage may be overwritten by the loads issued right after a barrier, so a wave
-    // only arrives at the barrier once its own reads of that stage have returned: an
-    // LDS read that is merely issued can still be queued behind other waves' reads
-    // when the (L2-fast) load of the next block lands.
-    auto stage_barrier = [&]() __attribute__((always_inline)) {
-        wait_lgkmcnt<0>();
-        lds_barrier();
-    };
     typedef std::integral_constant<int, 0> Stage0;
     typedef std::integral_constant<int, 1> Stage1;
     if constexpr (!kPipelined) {
@@ -340,12 +332,12 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
             issue_v(Stage0(), 0);
             for (int blk = 0; blk < num_blocks; blk += 2) {
                 wait_vmcnt<0>();
-                stage_barrier();
+                lds_barrier();
                 issue_k(Stage1(), min(blk + 1, last_block));
                 issue_v(Stage1(), min(blk + 1, last_block));
                 block(Stage0(), blk);
                 wait_vmcnt<0>();
-                stage_barrier();
+                lds_barrier();
                 issue_k(Stage0(), min(blk + 2, last_block));
                 issue_v(Stage0(), min(blk + 2, last_block));
                 block(Stage1(), blk + 1);
@@ -368,11 +360,11 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
             issue_k(Stage0(), 0);
             issue_k(Stage1(), min(1, last_block));
             wait_vmcnt<kInstr>();
-            stage_barrier();
+            lds_barrier();
             scores(Stage0(), s_buf[0]);
             // step 0: nothing to accumulate yet
             wait_vmcnt<0>();
-            stage_barrier();
+            lds_barrier();
             issue_k(Stage0(), min(2, last_block));
             issue_v(Stage0(), 0);
             if (needs_masks(0)) apply_masks(s_buf[0], 0);
@@ -384,7 +376,7 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
                 typedef std::integral_constant<int, kParity> Own;
                 typedef std::integral_constant<int, 1 - kParity> Other;
                 wait_vmcnt<0>();
-                stage_barrier();
+                lds_barrier();
                 issue_k(Own(), min(j + 2, last_block));
                 issue_v(Own(), j);
                 __builtin_amdgcn_sched_barrier(0);  // nothing of this step moves above the barrier
@@ -446,7 +438,7 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
             if (j < num_blocks) step_body(Stage1(), std::true_type(), j);
             // drain: P(last) . V(last); V(last) was requested into the stage of its parity
             wait_vmcnt<0>();
-            stage_barrier();
+            lds_barrier();
             if ((num_blocks - 1) & 1)
                 accumulate(Stage1(), p_buf[1]);
             else
@@ -557,8 +549,10 @@ extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineT
     p.q_scale = (float)(scale_value * 1.4426950408889634);
     p.causal = is_causal.data ? (Scalar0d::as_int64(is_causal) != 0) : 0;
     // block sizes are hints: 256 query rows select the one-workgroup-per-CU
-    // variant, 32-key blocks the three-workgroups-per-CU variant
-    int variant = block_size_m >= 256 ? 1 : (block_size_n > 0 && block_size_n <= 32 ? 2 : 3);
+    // variant, 32-key blocks the three-workgroups-per-CU variant.  Without a hint
+    // the pipelined variant runs non-causal problems; causal ones, whose waves
+    // spend a larger share of their blocks on masks, run the 32-key variant.
+    int variant = block_size_m >= 256 ? 1 : (block_size_n > 0 && block_size_n <= 32 ? 2 : (block_size_n >= 64 ? 0 : (p.causal ? 2 : 3)));
     if (block_size_n >= 1000) variant = block_size_n - 1000;  // measurement aid: explicit variant
     if (dtype == NINETOOTHED_FLOAT16) return dispatch_attention<half_t>(p, (int)head_dim, variant, (hipStream_t)stream);
     return dispatch_attention<bf16_t>(p, (int)head_dim, variant, (hipStream_t)stream);

@@ -85,10 +85,13 @@ NT_DEVICE void static_for(F &&f) {
 // memory clobber: the compiler moves no LDS access across it, and -- unlike a
 // workgroup fence -- it does not make the wave wait for its outstanding
 // global -> LDS fills of later stages (they are waited for explicitly with
-// wait_vmcnt<N>()).  Every wave has consumed (waited for) its own LDS reads of
-// the stage that is refilled next before it arrives here, because the MFMAs
-// using them precede the barrier in program order.
-NT_DEVICE void lds_barrier() { asm volatile("s_barrier" ::: "memory"); }
+// wait_vmcnt<N>()).  The stage that is refilled right after the barrier was
+// read just before it, and an LDS read that is merely issued can still sit in
+// the queue behind other waves' reads when the refill (an L2 hit) lands: the
+// MFMAs that consume it are not memory operations and may be scheduled below
+// the barrier, taking their wait with them.  So a wave first waits for its own
+// LDS reads and only then arrives at the barrier.
+NT_DEVICE void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // kAblate is a measurement aid (bit 0: no global loads inside the K loop,
 // bit 1: operand fragments read from LDS only once); 0 in every shipped instance.

@@ -204,7 +204,7 @@ def test_softmax_baseline_shape_properties():
 
 
 def _attention(q, k, v, is_causal=False, scale=None):
-    o = torch.empty_like(q)
+    o = torch.full_like(q, float("nan"))
     if scale is None:
         kernel = ninetoothed.make(programs.attention.arrangement, programs.attention.application, programs.attention.tensors())
         kernel(q, k, v, is_causal, o)
@@ -263,11 +263,42 @@ def test_attention_closed_forms_and_layouts():
 
 @pytest.mark.parametrize("is_causal", (False, True))
 def test_attention_baseline_shape(is_causal):
+    # every element of every (batch, head) is compared, on an output buffer that
+    # starts as NaN, twice: a synchronisation mistake in the kernel shows up as a
+    # few wrong rows in a few heads, not in every head
     q, k, v = (_randn(4, 32, 4096, 128).cuda() for _ in range(3))
-    out = _attention(q, k, v, is_causal, scale=128**-0.5)
-    expected = F.scaled_dot_product_attention(q[:1, :2], k[:1, :2], v[:1, :2], is_causal=is_causal, scale=128**-0.5)
-    assert torch.allclose(out[:1, :2], expected, **HALF_TOL)
-    assert torch.isfinite(out).all()
+    expected = torch.cat(
+        [F.scaled_dot_product_attention(q[b : b + 1], k[b : b + 1], v[b : b + 1], is_causal=is_causal, scale=128**-0.5) for b in range(4)]
+    )
+    kernel = ninetoothed.make(
+        programs.attention.arrangement_with_scale, programs.attention.application_with_scale, programs.attention.tensors(True)
+    )
+    for _ in range(2):
+        out = torch.full_like(q, float("nan"))
+        kernel(q, k, v, is_causal, 128**-0.5, out)
+        _native_only(kernel, "launch_nt_attention")
+        assert torch.allclose(out, expected, **HALF_TOL)
+
+
+@pytest.mark.parametrize("is_causal", (False, True))
+@pytest.mark.parametrize("emb_dim", (64, 128))
+@pytest.mark.parametrize("block_size_m, block_size_n", ((0, 0), (256, 0), (0, 32), (0, 64)))
+def test_attention_block_size_hints(block_size_m, block_size_n, emb_dim, is_causal):
+    # the block sizes of the arrangement reach the library as hints that pick the
+    # kernel variant; each variant is checked over the whole output, through the C ABI
+    from ninetoothed_amd import runtime
+
+    q, k, v = (_randn(2, 8, 2048 + 40, emb_dim).cuda() for _ in range(3))
+    out = torch.full_like(q, float("nan"))
+    tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (q, k, v, out)]
+    code = runtime.library().launch_nt_attention(
+        runtime.current_stream(), tensors[0], tensors[1], tensors[2],
+        runtime.ArgumentTensor.from_scalar(int(is_causal)), runtime.ArgumentTensor.from_scalar(float(emb_dim**-0.5)),
+        tensors[3], runtime.DATA_TYPE_INDEX["fp16"], block_size_m, block_size_n,
+    )
+    assert code == 0
+    expected = F.scaled_dot_product_attention(q, k, v, is_causal=is_causal, scale=emb_dim**-0.5)
+    assert torch.allclose(out, expected, **HALF_TOL)
 
 
 # ---- conv2d ---------------------------------------------------------------
