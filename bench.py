@@ -13,7 +13,12 @@ are measured in the same run and reported under ``"others"``.
 Prints ONE JSON line.  ``roofline.achieved`` = algorithmic FLOP (or bytes) per
 launch / average launch time from device events on the launch stream.
 ``cpu_baseline`` times the CPU oracle (oracle/programs.py, single thread) on a
-bounded sample of the same workload.
+bounded sample of the same workload.  ``vendor_gpu`` times the stock PyTorch
+operator of each workload (hipBLASLt / MIOpen / the built-in SDPA) on the same
+GPU and inputs, for context only.
+
+The GPU clock needs a few milliseconds of load to settle, so the default warm-up
+is 25 launches and the timed region 50.
 """
 
 import argparse
@@ -31,11 +36,12 @@ METRIC = "TFLOP/s fp16 matmul 8192^3 + attention fwd on 1 MI355X; % of MFMA peak
 def parse_args():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=20)
-    parser.add_argument("--warmup", type=int, default=5)
+    parser.add_argument("--steps", type=int, default=50)
+    parser.add_argument("--warmup", type=int, default=25)
     parser.add_argument("--workload", default="addmm_8192")
     parser.add_argument("--only", action="store_true", help="measure only --workload")
     parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--no-vendor", action="store_true", help="skip the stock PyTorch operators")
     return parser.parse_args()
 
 
@@ -58,6 +64,7 @@ def build_workloads():
         kernel = ninetoothed.make(programs.addmm.arrangement, programs.addmm.application, programs.addmm.tensors())
         return dict(
             step=lambda: kernel(input, mat1, mat2, 0.5, 1.0, out),
+            vendor=lambda: torch.addmm(input, mat1, mat2, beta=0.5, alpha=1.0, out=out),
             work=2.0 * n**3, bound="mfma", kernel=kernel,
             describe={"workload": "addmm fp16 M=N=K=8192 alpha=1.0 beta=0.5", "inputs": "randn, seeded"},
         )
@@ -67,14 +74,14 @@ def build_workloads():
         a, b = seeded(n, n, seed=0).cuda(), seeded(n, n, seed=1).cuda()
         out = torch.empty(n, n, dtype=torch.float16, device="cuda")
         kernel = ninetoothed.make(programs.matmul.arrangement, programs.matmul.application, programs.matmul.tensors())
-        return dict(step=lambda: kernel(a, b, out), work=2.0 * n**3, bound="mfma", kernel=kernel,
+        return dict(step=lambda: kernel(a, b, out), vendor=lambda: torch.matmul(a, b, out=out), work=2.0 * n**3, bound="mfma", kernel=kernel,
                     describe={"workload": "matmul fp16 M=N=K=512 (README program)"})
 
     def softmax_4096():
         x = seeded(4096, 4096, dtype=torch.float32).cuda()
         out = torch.empty_like(x)
         kernel = ninetoothed.make(programs.softmax.arrangement, programs.softmax.application, programs.softmax.tensors())
-        return dict(step=lambda: kernel(x, out, BLOCK_SIZE=4096), work=2.0 * 4096 * 4096 * 4, bound="hbm", kernel=kernel,
+        return dict(step=lambda: kernel(x, out, BLOCK_SIZE=4096), vendor=lambda: torch.softmax(x, dim=-1, out=out), work=2.0 * 4096 * 4096 * 4, bound="hbm", kernel=kernel,
                     describe={"workload": "row softmax fp32 [4096, 4096]"})
 
     def attention(is_causal):
@@ -83,7 +90,9 @@ def build_workloads():
             o = torch.empty_like(q)
             kernel = ninetoothed.make(programs.attention.arrangement_with_scale, programs.attention.application_with_scale, programs.attention.tensors(True))
             flops = 4.0 * 4 * 32 * 4096 * 4096 * 128 * (0.5 if is_causal else 1.0)
-            return dict(step=lambda: kernel(q, k, v, is_causal, 128**-0.5, o), work=flops, bound="mfma", kernel=kernel,
+            return dict(step=lambda: kernel(q, k, v, is_causal, 128**-0.5, o),
+                        vendor=lambda: torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=is_causal, scale=128**-0.5),
+                        work=flops, bound="mfma", kernel=kernel,
                         describe={"workload": f"SDPA forward fp16 [4, 32, 4096, 128] scale=1/sqrt(128) causal={is_causal}"})
         return make
 
@@ -92,7 +101,7 @@ def build_workloads():
         w = seeded(256, 256, 3, 3, scale=0.1, seed=1).cuda()
         out = torch.empty(32, 256, 56, 56, dtype=torch.float16, device="cuda")
         kernel = ninetoothed.make(programs.conv2d.arrangement, programs.conv2d.application, programs.conv2d.tensors())
-        return dict(step=lambda: kernel(x, w, out, padding_h=1, padding_w=1), work=2.0 * (32 * 56 * 56) * 256 * (256 * 9), bound="mfma", kernel=kernel,
+        return dict(step=lambda: kernel(x, w, out, padding_h=1, padding_w=1), vendor=lambda: torch.nn.functional.conv2d(x, w, padding=1), work=2.0 * (32 * 56 * 56) * 256 * (256 * 9), bound="mfma", kernel=kernel,
                     describe={"workload": "conv2d fp16 x[32,256,56,56] w[256,256,3,3] stride 1 padding 1 (implicit GEMM)"})
 
     def copy_1gib():
@@ -117,10 +126,11 @@ def build_workloads():
     return workloads
 
 
-def measure(workload, steps, warmup):
+def measure(workload, steps, warmup, which="step"):
     """Times exactly ``steps`` launches with device events on the launch stream."""
     import torch
 
+    workload = {"step": workload[which]}
     for _ in range(warmup):
         workload["step"]()
     torch.cuda.synchronize()
@@ -145,14 +155,14 @@ def roofline(workload, device_ms, traffic):
 
 
 def cpu_baseline_addmm():
-    """The CPU oracle (tile-by-tile numpy restatement) on a 64-row band of the
-    8192^3 addmm: 64 x 8192 x 8192, one thread."""
+    """The CPU oracle (tile-by-tile numpy restatement) on a 512-row band of the
+    8192^3 addmm: 512 x 8192 x 8192, one thread."""
     import numpy as np
     from threadpoolctl import threadpool_limits
 
     from oracle import programs as oracle
 
-    rows, n = 64, 8192
+    rows, n = 512, 8192
     rng = np.random.default_rng(0)
     input = rng.standard_normal((rows, n), dtype=np.float32).astype(np.float16)
     mat1 = rng.standard_normal((rows, n), dtype=np.float32).astype(np.float16)
@@ -218,6 +228,20 @@ def main():
     device_ms, wall_ms = measure(main_workload, args.steps, args.warmup)
     main_roofline = roofline(main_workload, device_ms, traffic.get(args.workload))
     launch_plan = main_workload["kernel"].last_plan
+    vendor = {}
+
+    def vendor_line(name, workload, steps):
+        if args.no_vendor or "vendor" not in workload:
+            return
+        try:
+            ms, _ = measure(workload, steps, args.warmup, which="vendor")
+        except Exception as error:  # a stock operator that is missing on this build is not this library's failure
+            vendor[name] = {"error": str(error).splitlines()[0][:120]}
+            return
+        entry = roofline(workload, ms, None)
+        vendor[name] = {"achieved": entry["achieved"], "unit": entry["unit"], "ms_per_step": ms}
+
+    vendor_line(args.workload, main_workload, args.steps)
     del main_workload["step"]
 
     others = {}
@@ -231,6 +255,7 @@ def main():
             entry["ms_per_step"] = ms
             entry["config"] = workload["describe"]
             others[name] = entry
+            vendor_line(name, workload, max(5, args.steps // 2))
             del workload
             torch.cuda.empty_cache()
 
@@ -251,6 +276,7 @@ def main():
         "config": dict(main_workload["describe"], launch=launch_plan),
         "roofline": main_roofline,
         "others": others,
+        "vendor_gpu": vendor,
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline_addmm()

@@ -259,16 +259,18 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
             const float m_use = m_new == -INFINITY ? 0.0f : m_new;  // fully masked so far
             alpha[qt] = __builtin_amdgcn_exp2f(m_run[qt] - m_use);
             m_run[qt] = m_new;
-            float sum = 0.0f;
+            // four independent partial sums: a single chain would tie every addition to
+            // the exponential right before it
+            float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const float pv = __builtin_amdgcn_exp2f(s_acc[kt][qt][r] - m_use);
                     s_acc[kt][qt][r] = pv;
-                    sum += pv;
+                    sum[r & 3] += pv;
                 }
-            l_run[qt] = l_run[qt] * alpha[qt] + sum;
+            l_run[qt] = l_run[qt] * alpha[qt] + ((sum[0] + sum[1]) + (sum[2] + sum[3]));
         }
 #pragma unroll
         for (int ps = 0; ps < PS; ++ps)
@@ -377,9 +379,9 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
                 typedef std::integral_constant<int, 1 - kParity> Other;
                 wait_vmcnt<0>();
                 lds_barrier();
+                __builtin_amdgcn_sched_barrier(0);  // nothing of this step moves above the barrier
                 issue_k(Own(), min(j + 2, last_block));
                 issue_v(Own(), j);
-                __builtin_amdgcn_sched_barrier(0);  // nothing of this step moves above the barrier
                 if constexpr (decltype(masked_tag)::value) apply_masks(s_buf[kParity], j);
                 softmax(s_buf[kParity], p_buf[kParity], alpha);
                 accumulate(Other(), p_buf[1 - kParity]);
@@ -396,7 +398,15 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
                 // instruction, 8 per exponential).  The first MFMAs overlap the running-max
                 // chain, the exponentials start once the maximum is known.
                 constexpr int kMfmaPerStep = (PS * DT + KS * KT) * kQTiles;
+#ifndef NT_ATTN_HEAD_VALU
+#define NT_ATTN_HEAD_VALU 12
+#endif
+                // first the operand reads of the first MFMAs, then the refills of this
+                // step's own stage and the head of the running-max chain while those reads
+                // are in flight
                 __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, 2 * kInstr, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, NT_ATTN_HEAD_VALU, 0);
                 static_for<0, kMfmaPerStep>([&](auto i_tag) __attribute__((always_inline)) {
                     constexpr int i = decltype(i_tag)::value;
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);

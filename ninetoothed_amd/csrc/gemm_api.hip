@@ -138,7 +138,7 @@ hipError_t generic_launch(const GemmProblem &q, hipStream_t stream) {
 
 const GemmInstance kInstances[] = {
     {"128x128x32 waves 2x2 any-stride", kGenBM, kGenBN, kGenBK, generic_accepts, generic_launch},
-    NT_FAST_INSTANCE(256, 256, 32, 2, 4, 4, 2),
+    NT_FAST_INSTANCE(256, 256, 32, 2, 4, 5, 2),  // 5 x 32 KiB: the whole LDS of a CU
     NT_FAST_INSTANCE(256, 256, 64, 2, 4, 2, 2),
     NT_FAST_INSTANCE(128, 128, 64, 2, 2, 2, 2),
 #ifdef NT_GEMM_ABLATION
@@ -146,7 +146,7 @@ const GemmInstance kInstances[] = {
     {#BM "x" #BN "x" #BK " waves " #WM "x" #WN " stages " #ST " load " #LD " aux " #AUX, BM, BN, BK, fast_accepts<BM, BN, BK, ST>, fast_launch<BM, BN, BK, WM, WN, ST, OCC, 0, LD, AUX>}
 #define NT_ABLATED_INSTANCE(BM, BN, BK, WM, WN, ST, OCC, AB) \
     {#BM "x" #BN "x" #BK " waves " #WM "x" #WN " stages " #ST " ABLATED " #AB " (wrong results)", BM, BN, BK, fast_accepts<BM, BN, BK, ST>, fast_launch<BM, BN, BK, WM, WN, ST, OCC, AB>}
-    NT_LOAD_INSTANCE(256, 256, 32, 2, 4, 5, 2, 1, 0),
+    NT_LOAD_INSTANCE(256, 256, 32, 2, 4, 4, 2, 1, 0),
     NT_LOAD_INSTANCE(256, 256, 32, 2, 2, 4, 1, 1, 0),
     NT_LOAD_INSTANCE(128, 256, 32, 2, 2, 4, 2, 1, 0),
     NT_ABLATED_INSTANCE(256, 256, 32, 2, 4, 4, 2, 1),
