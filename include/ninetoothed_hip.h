@@ -14,8 +14,11 @@
  * (floating point) or a HOST int64_t (integer / boolean), `shape` and
  * `strides` are not read (reference: src/ninetoothed/aot.py:725-733, 624-628).
  *
- * Launches are asynchronous on the given stream, never synchronise and never
- * allocate; the caller owns every buffer.  All functions are re-entrant.
+ * Launches are asynchronous on the given stream and never synchronise; the
+ * caller owns every tensor.  Only launch_nt_conv2d may take temporary device
+ * memory, from the stream-ordered allocator (hipMallocAsync / hipFreeAsync on
+ * the given stream, see there); every other launch allocates nothing.  All
+ * functions are re-entrant.
  */
 #ifndef NINETOOTHED_HIP_H
 #define NINETOOTHED_HIP_H
@@ -115,7 +118,13 @@ NineToothedResult launch_nt_softmax_config(NineToothedStream stream, int config,
  * Replaces the kernel generated for tests/test_attention.py:14-70; that
  * program has scale == 1, the scale tensor (0-d, host double) is this
  * library's extension for the 1/sqrt(head_dim) configuration.
- * is_causal is a 0-d tensor holding a host int64_t. */
+ * is_causal is a 0-d tensor holding a host int64_t.
+ * block_size_m / block_size_n are hints (0 = library's choice): block_size_m
+ * >= 256 selects 256 query rows per workgroup, block_size_n <= 32 the 32-key
+ * blocks with three workgroups per CU, block_size_n >= 64 the plain 64-key
+ * loop; without hints non-causal calls run the software-pipelined 64-key loop
+ * and causal calls the 32-key one.  K and V of one (batch, head) must span
+ * less than 4 GiB. */
 NineToothedResult launch_nt_attention(NineToothedStream stream,
                                       NineToothedTensor q,
                                       NineToothedTensor k,
@@ -129,7 +138,13 @@ NineToothedResult launch_nt_attention(NineToothedStream stream,
 /* output[N,K,P,Q] = conv2d(input[N,C,H,W], filter[K,C,R,S]) with stride 1,
  * dilation 1 and zero padding (padding_h, padding_w), computed as the implicit
  * GEMM [N*P*Q, C*R*S] x [C*R*S, K] the arrangement of
- * tests/test_conv2d.py:13-48 describes. */
+ * tests/test_conv2d.py:13-48 describes.
+ * When C % 32 == 0, K % 256 == 0, (P*Q) % 8 == 0, the output is contiguous and
+ * N*P*Q >= 1024, the call first repacks the input to channels-last and the
+ * filter to [R*S*C, K] in temporaries taken from and returned to the
+ * stream-ordered allocator on `stream` (N*C*H*W + K*C*R*S elements), then runs
+ * the direct-to-LDS main loop; block_size_m == 1 keeps the call on the
+ * allocation-free gather kernel, which also serves every other shape. */
 NineToothedResult launch_nt_conv2d(NineToothedStream stream,
                                    NineToothedTensor input,
                                    NineToothedTensor filter,
