@@ -13,7 +13,8 @@ are measured in the same run and reported under ``"others"``.
 Prints ONE JSON line.  ``roofline.achieved`` = algorithmic FLOP (or bytes) per
 launch / average launch time from device events on the launch stream.
 ``cpu_baseline`` times the CPU oracle (oracle/programs.py, single thread) on a
-bounded sample of the same workload.  ``vendor_gpu`` times the stock PyTorch
+bounded sample of the same workload; ``torch_cpu`` times the stock torch CPU
+operator of every configuration (all host threads, bounded samples).  ``vendor_gpu`` times the stock PyTorch
 operator of each workload (hipBLASLt / MIOpen / the built-in SDPA) on the same
 GPU and inputs, for context only.
 
@@ -146,6 +147,20 @@ def measure(workload, steps, warmup, which="step"):
     return device_ms, wall
 
 
+def per_launch(workload, launches=20):
+    """Median and minimum of single launches, each bracketed by its own pair of events."""
+    import torch
+
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(launches)]
+    for start, stop in events:
+        start.record()
+        workload["step"]()
+        stop.record()
+    torch.cuda.synchronize()
+    times = sorted(start.elapsed_time(stop) for start, stop in events)
+    return {"median_ms": times[len(times) // 2], "min_ms": times[0], "launches": launches}
+
+
 def roofline(workload, device_ms, traffic):
     if workload["bound"] == "mfma":
         achieved = workload["work"] / (device_ms * 1e-3) / 1e12
@@ -181,20 +196,47 @@ def cpu_baseline_addmm():
     }
 
 
-def torch_cpu_addmm():
-    """torch.addmm on the host, all threads, on a 1024-row band (context only)."""
+def torch_cpu_context():
+    """The stock torch CPU operator of each configuration on the host, all threads,
+    one warm-up and the median of three runs, on bounded samples (context only)."""
     import torch
+    import torch.nn.functional as F
 
-    rows, n = 1024, 8192
     generator = torch.Generator().manual_seed(0)
-    input = torch.randn(rows, n, generator=generator)
-    mat1 = torch.randn(rows, n, generator=generator)
-    mat2 = torch.randn(n, n, generator=generator)
-    t0 = time.perf_counter()
-    torch.addmm(input, mat1, mat2, beta=0.5, alpha=1.0)
-    seconds = time.perf_counter() - t0
-    return {"value": 2.0 * rows * n * n / seconds / 1e12, "unit": "TFLOP/s", "threads": torch.get_num_threads(),
-            "sample": f"torch.addmm fp32 {rows}x{n}x{n} on the host, {seconds:.2f} s"}
+
+    def randn(*shape, scale=1.0):
+        return torch.randn(*shape, generator=generator) * scale
+
+    def timed(fn, runs=3, warm=1):
+        for _ in range(warm):
+            fn()
+        times = []
+        for _ in range(runs):
+            t0 = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t0)
+        return sorted(times)[len(times) // 2]
+
+    out = {"threads": torch.get_num_threads(), "host_cpus": os.cpu_count()}
+    rows, n = 1024, 8192
+    input, mat1, mat2 = randn(rows, n), randn(rows, n), randn(n, n)
+    seconds = timed(lambda: torch.addmm(input, mat1, mat2, beta=0.5, alpha=1.0), runs=1, warm=0)
+    out["addmm_8192"] = {"value": 2.0 * rows * n * n / seconds / 1e12, "unit": "TFLOP/s", "sample": f"torch.addmm fp32 on a {rows}x{n}x{n} band, {seconds:.2f} s"}
+    a, b = randn(512, 512), randn(512, 512)
+    seconds = timed(lambda: torch.matmul(a, b))
+    out["matmul_512"] = {"value": 2.0 * 512**3 / seconds / 1e12, "unit": "TFLOP/s", "sample": f"torch.matmul fp32 512^3, {seconds * 1e3:.2f} ms"}
+    x = randn(4096, 4096)
+    seconds = timed(lambda: torch.softmax(x, dim=-1))
+    out["softmax_4096"] = {"value": 2.0 * 4096 * 4096 * 4 / seconds / 1e9, "unit": "GB/s", "sample": f"torch.softmax fp32 [4096, 4096], {seconds * 1e3:.1f} ms"}
+    q, k, v = (randn(1, 2, 4096, 128) for _ in range(3))
+    for causal, name in ((False, "attention"), (True, "attention_causal")):
+        seconds = timed(lambda: F.scaled_dot_product_attention(q, k, v, is_causal=causal, scale=128**-0.5), runs=1, warm=0)
+        flops = 4.0 * 2 * 4096 * 4096 * 128 * (0.5 if causal else 1.0)
+        out[name] = {"value": flops / seconds / 1e12, "unit": "TFLOP/s", "sample": f"F.scaled_dot_product_attention fp32 on 2 of the 128 (batch, head) pairs, {seconds:.2f} s"}
+    xc, wc = randn(2, 256, 56, 56, scale=0.1), randn(256, 256, 3, 3, scale=0.1)
+    seconds = timed(lambda: F.conv2d(xc, wc, padding=1), runs=1, warm=0)
+    out["conv2d"] = {"value": 2.0 * (2 * 56 * 56) * 256 * (256 * 9) / seconds / 1e12, "unit": "TFLOP/s", "sample": f"F.conv2d fp32 on 2 of the 32 images, {seconds:.2f} s"}
+    return out
 
 
 def load_traffic():
@@ -228,6 +270,7 @@ def main():
     device_ms, wall_ms = measure(main_workload, args.steps, args.warmup)
     main_roofline = roofline(main_workload, device_ms, traffic.get(args.workload))
     launch_plan = main_workload["kernel"].last_plan
+    single = per_launch(main_workload)
     vendor = {}
 
     def vendor_line(name, workload, steps):
@@ -275,12 +318,14 @@ def main():
         "data": "synthetic",
         "config": dict(main_workload["describe"], launch=launch_plan),
         "roofline": main_roofline,
+        "per_launch": single,
+        "l2": "not flushed between launches",
         "others": others,
         "vendor_gpu": vendor,
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline_addmm()
-        result["torch_cpu"] = torch_cpu_addmm()
+        result["torch_cpu"] = torch_cpu_context()
     print(json.dumps(result))
 
 
