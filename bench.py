@@ -105,6 +105,23 @@ def build_workloads():
         return dict(step=lambda: kernel(x, w, out, padding_h=1, padding_w=1), vendor=lambda: torch.nn.functional.conv2d(x, w, padding=1), work=2.0 * (32 * 56 * 56) * 256 * (256 * 9), bound="mfma", kernel=kernel,
                     describe={"workload": "conv2d fp16 x[32,256,56,56] w[256,256,3,3] stride 1 padding 1 (implicit GEMM)"})
 
+    def map_add():
+        # an element-wise program outside the five recognised ones: runs on the interpreter kernel
+        n = 1 << 26
+        lhs, rhs = seeded(n, dtype=torch.float32, seed=0).cuda(), seeded(n, dtype=torch.float32, seed=1).cuda()
+        out = torch.empty_like(lhs)
+        block = ninetoothed.Symbol("BLOCK_SIZE", meta=True)
+
+        def arrangement(lhs, rhs, output):
+            return lhs.tile((block,)), rhs.tile((block,)), output.tile((block,))
+
+        def application(lhs, rhs, output):
+            output = lhs + rhs  # noqa: F841
+
+        kernel = ninetoothed.make(arrangement, application, (ninetoothed.Tensor(1),) * 3)
+        return dict(step=lambda: kernel(lhs, rhs, out), vendor=lambda: torch.add(lhs, rhs, out=out), work=3.0 * n * 4, bound="hbm", kernel=kernel,
+                    describe={"workload": "element-wise add fp32, 2^26 elements (generic tile-map executor)"})
+
     def copy_1gib():
         # a plain device-to-device copy of known size: the calibration point for the
         # HBM traffic counters (FETCH_SIZE / WRITE_SIZE) quoted in profiles/
@@ -123,6 +140,7 @@ def build_workloads():
     workloads["attention"] = attention(False)
     workloads["attention_causal"] = attention(True)
     workloads["conv2d"] = conv2d
+    workloads["map_add"] = map_add
     workloads["copy_1gib"] = copy_1gib
     return workloads
 

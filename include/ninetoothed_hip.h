@@ -192,6 +192,115 @@ NineToothedResult nt_tune_gemm(NineToothedStream stream,
                                int dtype, int output_dtype, int iters,
                                int *best_config, float *best_ms);
 
+/*
+ * Element-wise / reducing tile programs that are none of the programs above.
+ *
+ * Replaces the Triton kernel the reference generates for an arbitrary
+ * arrange-and-apply pair (src/ninetoothed/generation.py:28-837) for the class
+ * of programs whose application is a map over tiles with an optional reduction
+ * (the programs of tests/test_add.py, test_clone.py, test_pad.py, test_pow.py,
+ * test_dropout.py, test_max_pool2d.py, test_generation.py:139-151 of the
+ * reference).  The host lowers the arrangement's index maps and the
+ * application's dataflow graph into two small stack programs; one kernel
+ * interprets them per output element:
+ *
+ *   - the iteration space is `num_vars` index variables with `extents`; the
+ *     first `num_vars - num_reduced` enumerate the output elements (the last of
+ *     them varies fastest across lanes), the rest the reduced positions;
+ *   - index code (one segment per operand, and per `.offsets()` use) computes a
+ *     flat element offset from the variables with + * // % by constants
+ *     (src/ninetoothed/tensor.py:258-274, 462-471, 555-556) and checks
+ *     0 <= index < size where the arrangement needs a mask
+ *     (src/ninetoothed/tensor.py:571-584); a masked load yields `other`, a
+ *     masked store is skipped (src/ninetoothed/generation.py:638-744);
+ *   - value code evaluates the expression in double precision with an explicit
+ *     rounding step after every operation whose result the reference holds in
+ *     a narrower type, so + - * / and sqrt are the correctly rounded fp16 /
+ *     bf16 / fp32 operations; `value_code[0 .. reduce_split)` runs per reduced
+ *     position, the rest once per output element on the reduced value.
+ *
+ * Code words are (opcode | argument << 8); the opcodes are the NT_MAP_I_* /
+ * NT_MAP_V_* values below.
+ *
+ * launch_nt_map specialises: the first launch of a program (same code, index
+ * constants, extents and element types) translates it to HIP source, compiles
+ * it with hipRTC (loaded on demand) and caches the kernel per device; later
+ * launches only pass pointers, `other` values and value constants.  Without
+ * hipRTC, or with NT_MAP_INTERPRET=1 in the environment, an interpreter kernel
+ * executes the same programs (the struct travels by value as its argument).
+ * No device memory is allocated either way.
+ */
+#define NT_MAP_MAX_OPERANDS 8
+#define NT_MAP_MAX_VARS 16
+#define NT_MAP_MAX_INDEX_CODE 320
+#define NT_MAP_MAX_INDEX_CONSTANTS 96
+#define NT_MAP_MAX_SEGMENTS 16
+#define NT_MAP_MAX_VALUE_CODE 128
+#define NT_MAP_MAX_VALUE_CONSTANTS 32
+
+enum NineToothedMapIndexOp {
+    NT_MAP_I_END,    /* the offset is on top of the stack */
+    NT_MAP_I_CONST,  /* push index_constants[arg] */
+    NT_MAP_I_VAR,    /* push variable arg */
+    NT_MAP_I_MULC,   /* top *= index_constants[arg] */
+    NT_MAP_I_ADD,    /* pop b; top += b */
+    NT_MAP_I_DIVC,   /* top = floor(top / index_constants[arg]) */
+    NT_MAP_I_MODC,   /* top = top - floor(top / c) * c */
+    NT_MAP_I_CHECK   /* pop v; valid &= 0 <= v < index_constants[arg] */
+};
+
+enum NineToothedMapValueOp {
+    NT_MAP_V_LOAD,      /* push operand arg at its offset (`other` when masked) */
+    NT_MAP_V_CONST,     /* push value_constants[arg] */
+    NT_MAP_V_OFFSET,    /* push the result of index segment arg */
+    NT_MAP_V_ADD, NT_MAP_V_SUB, NT_MAP_V_MUL, NT_MAP_V_DIV, NT_MAP_V_FLOORDIV, NT_MAP_V_MOD, NT_MAP_V_POW,
+    NT_MAP_V_MAX, NT_MAP_V_MIN,
+    NT_MAP_V_LT, NT_MAP_V_LE, NT_MAP_V_GT, NT_MAP_V_GE, NT_MAP_V_EQ, NT_MAP_V_NE, NT_MAP_V_AND, NT_MAP_V_OR,
+    NT_MAP_V_NEG, NT_MAP_V_NOT, NT_MAP_V_ABS, NT_MAP_V_EXP, NT_MAP_V_EXP2, NT_MAP_V_LOG, NT_MAP_V_LOG2,
+    NT_MAP_V_SQRT, NT_MAP_V_RSQRT, NT_MAP_V_SIGMOID, NT_MAP_V_TANH, NT_MAP_V_SIN, NT_MAP_V_COS, NT_MAP_V_FLOOR, NT_MAP_V_CEIL,
+    NT_MAP_V_WHERE,     /* pop b, a, c; push c ? a : b */
+    NT_MAP_V_ROUND,     /* round top to NineToothedDataType arg (integers truncate) */
+    NT_MAP_V_RAND       /* pop offset, seed; push the Philox-4x32-10 uniform float of (seed, offset) */
+};
+
+enum NineToothedMapReduceOp { NT_MAP_REDUCE_NONE, NT_MAP_REDUCE_MAX, NT_MAP_REDUCE_MIN, NT_MAP_REDUCE_SUM };
+
+typedef struct {
+    void *data;
+    int32_t dtype;    /* NineToothedDataType */
+    int32_t segment;  /* index segment that yields its element offset */
+    double other;     /* value of masked loads */
+} NineToothedMapOperand;
+
+typedef struct {
+    int32_t num_vars;
+    int32_t num_reduced;
+    int64_t extents[NT_MAP_MAX_VARS];
+    int32_t num_operands;
+    int32_t output;              /* operand that is stored */
+    NineToothedMapOperand operands[NT_MAP_MAX_OPERANDS];
+    int32_t num_segments;
+    int32_t segment_begin[NT_MAP_MAX_SEGMENTS];
+    int32_t index_code[NT_MAP_MAX_INDEX_CODE];
+    int64_t index_constants[NT_MAP_MAX_INDEX_CONSTANTS];
+    int32_t value_code_length;
+    int32_t reduce_split;
+    int32_t reduce_op;           /* NineToothedMapReduceOp */
+    int32_t reduce_dtype;        /* type the reduction accumulates in (sums of fp16 / bf16: FLOAT32) */
+    int32_t value_code[NT_MAP_MAX_VALUE_CODE];
+    double value_constants[NT_MAP_MAX_VALUE_CONSTANTS];
+} NineToothedMapProgram;
+
+/* Runs one store of such a program.  Returns NINETOOTHED_NO_KERNEL when the
+ * program does not fit the limits above or names an unknown opcode / type. */
+NineToothedResult launch_nt_map(NineToothedStream stream, const NineToothedMapProgram *program);
+
+/* Writes the HIP source launch_nt_map specialises `program` to (NUL terminated)
+ * into `buffer`; the counterpart of the generated source file the reference's
+ * handle exposes as `_source` (src/ninetoothed/jit.py:121-128).  Returns
+ * hipErrorInvalidValue when `size` is too small. */
+NineToothedResult nt_map_source(const NineToothedMapProgram *program, char *buffer, int size);
+
 /* Library version string, e.g. "nt_hip 0.1 gfx950". */
 const char *nt_version(void);
 

@@ -1,0 +1,748 @@
+// Interpreter kernel for element-wise / reducing tile programs (gfx950).
+//
+// The host lowers an arrangement's index maps and an application's dataflow
+// graph into two stack programs (see the NineToothedMapProgram comment in the
+// header); each lane walks output elements with a grid stride, evaluates the
+// index code of every operand it touches and the value code of the expression,
+// and stores one element.  Consecutive lanes take consecutive values of the last
+// output variable, which the host orders so that it is the innermost source
+// dimension: loads and stores of contiguous tensors coalesce.  The programs are
+// HBM-bound byte work; the interpreter's integer arithmetic hides behind the
+// memory latency as long as enough waves are resident (256 lanes per
+// workgroup, 8 workgroups per CU).
+//
+// launch_nt_map first tries a kernel specialised for the program: the two stack
+// programs are translated to straight-line HIP source (index constants, extents
+// and element types as literals, call-time scalars and pointers as arguments),
+// compiled once per distinct program with hipRTC and cached per device.  The
+// interpreter kernel below runs when hipRTC is not available (libhiprtc.so is
+// loaded on first use, not linked) or when NT_MAP_INTERPRET=1 is set; both
+// execute the same operations in the same order.
+#include <dlfcn.h>
+#include <hip/hip_runtime.h>
+#include <hip/hiprtc.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <sstream>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "nt_common.h"
+
+namespace nt {
+namespace {
+
+constexpr int kMapThreads = 256;
+constexpr int kIndexStack = 8;
+constexpr int kValueStack = 16;
+
+__device__ __forceinline__ int64_t floor_div(int64_t a, int64_t b) {
+    int64_t q = a / b;
+    if ((a % b != 0) && ((a < 0) != (b < 0))) --q;
+    return q;
+}
+
+// runs one index segment: returns the offset, clears `valid` when a check fails
+__device__ __forceinline__ int64_t run_index(const NineToothedMapProgram &p, int segment, const int64_t *vars, bool &valid) {
+    int64_t stack[kIndexStack];
+    int top = -1;
+    for (int pc = p.segment_begin[segment];; ++pc) {
+        const int word = p.index_code[pc];
+        const int op = word & 0xff;
+        const int arg = word >> 8;
+        switch (op) {
+            case NT_MAP_I_END: return top >= 0 ? stack[top] : 0;
+            case NT_MAP_I_CONST: stack[++top] = p.index_constants[arg]; break;
+            case NT_MAP_I_VAR: stack[++top] = vars[arg]; break;
+            case NT_MAP_I_MULC: stack[top] *= p.index_constants[arg]; break;
+            case NT_MAP_I_ADD: stack[top - 1] += stack[top]; --top; break;
+            case NT_MAP_I_DIVC: stack[top] = floor_div(stack[top], p.index_constants[arg]); break;
+            case NT_MAP_I_MODC: {
+                const int64_t c = p.index_constants[arg];
+                stack[top] -= floor_div(stack[top], c) * c;
+                break;
+            }
+            case NT_MAP_I_CHECK: {
+                const int64_t v = stack[top--];
+                valid = valid && v >= 0 && v < p.index_constants[arg];
+                break;
+            }
+            default: return 0;
+        }
+    }
+}
+
+__device__ __forceinline__ double load_element(const void *data, int dtype, int64_t offset) {
+    switch (dtype) {
+        case NINETOOTHED_INT8: return (double)((const int8_t *)data)[offset];
+        case NINETOOTHED_INT16: return (double)((const int16_t *)data)[offset];
+        case NINETOOTHED_INT32: return (double)((const int32_t *)data)[offset];
+        case NINETOOTHED_INT64: return (double)((const int64_t *)data)[offset];
+        case NINETOOTHED_UINT8: return (double)((const uint8_t *)data)[offset];
+        case NINETOOTHED_UINT16: return (double)((const uint16_t *)data)[offset];
+        case NINETOOTHED_UINT32: return (double)((const uint32_t *)data)[offset];
+        case NINETOOTHED_UINT64: return (double)((const uint64_t *)data)[offset];
+        case NINETOOTHED_FLOAT16: return (double)(float)((const half_t *)data)[offset];
+        case NINETOOTHED_BFLOAT16: return (double)(float)((const bf16_t *)data)[offset];
+        case NINETOOTHED_FLOAT32: return (double)((const float *)data)[offset];
+        default: return ((const double *)data)[offset];
+    }
+}
+
+__device__ __forceinline__ void store_element(void *data, int dtype, int64_t offset, double v) {
+    switch (dtype) {
+        case NINETOOTHED_INT8: ((int8_t *)data)[offset] = (int8_t)(int64_t)v; break;
+        case NINETOOTHED_INT16: ((int16_t *)data)[offset] = (int16_t)(int64_t)v; break;
+        case NINETOOTHED_INT32: ((int32_t *)data)[offset] = (int32_t)(int64_t)v; break;
+        case NINETOOTHED_INT64: ((int64_t *)data)[offset] = (int64_t)v; break;
+        case NINETOOTHED_UINT8: ((uint8_t *)data)[offset] = (uint8_t)(int64_t)v; break;
+        case NINETOOTHED_UINT16: ((uint16_t *)data)[offset] = (uint16_t)(int64_t)v; break;
+        case NINETOOTHED_UINT32: ((uint32_t *)data)[offset] = (uint32_t)(int64_t)v; break;
+        case NINETOOTHED_UINT64: ((uint64_t *)data)[offset] = (uint64_t)v; break;
+        case NINETOOTHED_FLOAT16: ((half_t *)data)[offset] = (half_t)(float)v; break;
+        case NINETOOTHED_BFLOAT16: ((bf16_t *)data)[offset] = (bf16_t)(float)v; break;
+        case NINETOOTHED_FLOAT32: ((float *)data)[offset] = (float)v; break;
+        default: ((double *)data)[offset] = v; break;
+    }
+}
+
+// the value as the reference would hold it in a tile of type `dtype`
+__device__ __forceinline__ double round_to(double v, int dtype) {
+    switch (dtype) {
+        case NINETOOTHED_FLOAT16: return (double)(float)(half_t)(float)v;
+        case NINETOOTHED_BFLOAT16: return (double)(float)(bf16_t)(float)v;
+        case NINETOOTHED_FLOAT32: return (double)(float)v;
+        case NINETOOTHED_FLOAT64: return v;
+        case NINETOOTHED_INT8: return (double)(int8_t)(int64_t)v;
+        case NINETOOTHED_INT16: return (double)(int16_t)(int64_t)v;
+        case NINETOOTHED_INT32: return (double)(int32_t)(int64_t)v;
+        case NINETOOTHED_UINT8: return (double)(uint8_t)(int64_t)v;
+        case NINETOOTHED_UINT16: return (double)(uint16_t)(int64_t)v;
+        case NINETOOTHED_UINT32: return (double)(uint32_t)(int64_t)v;
+        case NINETOOTHED_UINT64: return (double)(uint64_t)v;
+        default: return (double)(int64_t)v;
+    }
+}
+
+// Philox-4x32 with 10 rounds, counter (offset_lo, offset_hi, 0, 0), key = the two
+// halves of the seed; the first output word becomes a float in [0, 1): negative
+// values (as int32) are mirrored, then scaled by 2^-31.
+__device__ __forceinline__ double philox_uniform(uint64_t seed, uint64_t offset) {
+    uint32_t c0 = (uint32_t)offset, c1 = (uint32_t)(offset >> 32), c2 = 0, c3 = 0;
+    uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
+    for (int round = 0; round < 10; ++round) {
+        const uint32_t a = 0xD2511F53u, b = 0xCD9E8D57u;
+        const uint32_t p0 = c0, p2 = c2;
+        c0 = __umulhi(b, p2) ^ c1 ^ k0;
+        c2 = __umulhi(a, p0) ^ c3 ^ k1;
+        c1 = b * p2;
+        c3 = a * p0;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    int32_t x = (int32_t)c0;
+    if (x < 0) x = -x - 1;
+    return (double)((float)x * 4.6566127342e-10f);
+}
+
+// runs value_code[begin, end) on a stack that starts as `initial` (when `seeded`)
+__device__ __forceinline__ double run_value(const NineToothedMapProgram &p, int begin, int end, const int64_t *vars, bool seeded,
+                                             double initial) {
+    double stack[kValueStack];
+    int top = -1;
+    if (seeded) stack[++top] = initial;
+    for (int pc = begin; pc < end; ++pc) {
+        const int word = p.value_code[pc];
+        const int op = word & 0xff;
+        const int arg = word >> 8;
+        switch (op) {
+            case NT_MAP_V_LOAD: {
+                const NineToothedMapOperand &operand = p.operands[arg];
+                bool valid = true;
+                const int64_t offset = run_index(p, operand.segment, vars, valid);
+                stack[++top] = valid ? load_element(operand.data, operand.dtype, offset) : operand.other;
+                break;
+            }
+            case NT_MAP_V_CONST: stack[++top] = p.value_constants[arg]; break;
+            case NT_MAP_V_OFFSET: {
+                bool valid = true;
+                stack[++top] = (double)run_index(p, arg, vars, valid);
+                break;
+            }
+#define NT_BINARY(OP, EXPR)                          \
+    case OP: {                                       \
+        const double b = stack[top--];               \
+        const double a = stack[top];                 \
+        stack[top] = (EXPR);                         \
+        break;                                       \
+    }
+            NT_BINARY(NT_MAP_V_ADD, a + b)
+            NT_BINARY(NT_MAP_V_SUB, a - b)
+            NT_BINARY(NT_MAP_V_MUL, a * b)
+            NT_BINARY(NT_MAP_V_DIV, a / b)
+            NT_BINARY(NT_MAP_V_FLOORDIV, floor(a / b))
+            NT_BINARY(NT_MAP_V_MOD, a - floor(a / b) * b)
+            NT_BINARY(NT_MAP_V_POW, (double)powf((float)a, (float)b))
+            NT_BINARY(NT_MAP_V_MAX, (a != a || b != b) ? (a + b) : (a > b ? a : b))
+            NT_BINARY(NT_MAP_V_MIN, (a != a || b != b) ? (a + b) : (a < b ? a : b))
+            NT_BINARY(NT_MAP_V_LT, a < b ? 1.0 : 0.0)
+            NT_BINARY(NT_MAP_V_LE, a <= b ? 1.0 : 0.0)
+            NT_BINARY(NT_MAP_V_GT, a > b ? 1.0 : 0.0)
+            NT_BINARY(NT_MAP_V_GE, a >= b ? 1.0 : 0.0)
+            NT_BINARY(NT_MAP_V_EQ, a == b ? 1.0 : 0.0)
+            NT_BINARY(NT_MAP_V_NE, a != b ? 1.0 : 0.0)
+            NT_BINARY(NT_MAP_V_AND, (a != 0.0 && b != 0.0) ? 1.0 : 0.0)
+            NT_BINARY(NT_MAP_V_OR, (a != 0.0 || b != 0.0) ? 1.0 : 0.0)
+#undef NT_BINARY
+#define NT_UNARY(OP, EXPR)            \
+    case OP: {                        \
+        const double a = stack[top];  \
+        stack[top] = (EXPR);          \
+        break;                        \
+    }
+            NT_UNARY(NT_MAP_V_NEG, -a)
+            NT_UNARY(NT_MAP_V_NOT, a == 0.0 ? 1.0 : 0.0)
+            NT_UNARY(NT_MAP_V_ABS, fabs(a))
+            NT_UNARY(NT_MAP_V_EXP, (double)expf((float)a))
+            NT_UNARY(NT_MAP_V_EXP2, (double)exp2f((float)a))
+            NT_UNARY(NT_MAP_V_LOG, (double)logf((float)a))
+            NT_UNARY(NT_MAP_V_LOG2, (double)log2f((float)a))
+            NT_UNARY(NT_MAP_V_SQRT, sqrt(a))
+            NT_UNARY(NT_MAP_V_RSQRT, (double)(1.0f / sqrtf((float)a)))
+            NT_UNARY(NT_MAP_V_SIGMOID, (double)(1.0f / (1.0f + expf(-(float)a))))
+            NT_UNARY(NT_MAP_V_TANH, (double)tanhf((float)a))
+            NT_UNARY(NT_MAP_V_SIN, (double)sinf((float)a))
+            NT_UNARY(NT_MAP_V_COS, (double)cosf((float)a))
+            NT_UNARY(NT_MAP_V_FLOOR, floor(a))
+            NT_UNARY(NT_MAP_V_CEIL, ceil(a))
+#undef NT_UNARY
+            case NT_MAP_V_WHERE: {
+                const double b = stack[top--];
+                const double a = stack[top--];
+                stack[top] = stack[top] != 0.0 ? a : b;
+                break;
+            }
+            case NT_MAP_V_ROUND: stack[top] = round_to(stack[top], arg); break;
+            case NT_MAP_V_RAND: {
+                const double offset = stack[top--];
+                stack[top] = philox_uniform((uint64_t)(int64_t)stack[top], (uint64_t)(int64_t)offset);
+                break;
+            }
+            default: break;
+        }
+    }
+    return top >= 0 ? stack[top] : 0.0;
+}
+
+__global__ __launch_bounds__(kMapThreads) void map_kernel(const NineToothedMapProgram p, int64_t total_out, int64_t total_reduced) {
+    const int num_out = p.num_vars - p.num_reduced;
+    const int64_t stride = (int64_t)gridDim.x * kMapThreads;
+    for (int64_t element = (int64_t)blockIdx.x * kMapThreads + threadIdx.x; element < total_out; element += stride) {
+        int64_t vars[NT_MAP_MAX_VARS];
+        int64_t rest = element;
+        for (int v = num_out - 1; v >= 0; --v) {
+            const int64_t extent = p.extents[v];
+            vars[v] = rest % extent;
+            rest /= extent;
+        }
+        double value;
+        if (p.reduce_op == NT_MAP_REDUCE_NONE) {
+            value = run_value(p, 0, p.value_code_length, vars, false, 0.0);
+        } else {
+            double acc = p.reduce_op == NT_MAP_REDUCE_SUM ? 0.0 : (p.reduce_op == NT_MAP_REDUCE_MAX ? -INFINITY : INFINITY);
+            for (int64_t position = 0; position < total_reduced; ++position) {
+                int64_t inner = position;
+                for (int v = p.num_vars - 1; v >= num_out; --v) {
+                    const int64_t extent = p.extents[v];
+                    vars[v] = inner % extent;
+                    inner /= extent;
+                }
+                const double term = run_value(p, 0, p.reduce_split, vars, false, 0.0);
+                if (p.reduce_op == NT_MAP_REDUCE_SUM) {
+                    acc = round_to(acc + term, p.reduce_dtype);
+                } else if (term != term || acc != acc) {
+                    acc = acc + term;  // NaN propagates
+                } else if (p.reduce_op == NT_MAP_REDUCE_MAX) {
+                    acc = term > acc ? term : acc;
+                } else {
+                    acc = term < acc ? term : acc;
+                }
+            }
+            value = run_value(p, p.reduce_split, p.value_code_length, vars, true, acc);
+        }
+        const NineToothedMapOperand &out = p.operands[p.output];
+        bool valid = true;
+        const int64_t offset = run_index(p, out.segment, vars, valid);
+        if (valid) store_element(out.data, out.dtype, offset, value);
+    }
+}
+
+bool well_formed(const NineToothedMapProgram &p) {
+    if (p.num_vars < 0 || p.num_vars > NT_MAP_MAX_VARS || p.num_reduced < 0 || p.num_reduced > p.num_vars) return false;
+    if (p.num_operands < 1 || p.num_operands > NT_MAP_MAX_OPERANDS || p.output < 0 || p.output >= p.num_operands) return false;
+    if (p.num_segments < 1 || p.num_segments > NT_MAP_MAX_SEGMENTS) return false;
+    if (p.value_code_length < 0 || p.value_code_length > NT_MAP_MAX_VALUE_CODE) return false;
+    if (p.reduce_split < 0 || p.reduce_split > p.value_code_length) return false;
+    if (p.reduce_op < NT_MAP_REDUCE_NONE || p.reduce_op > NT_MAP_REDUCE_SUM) return false;
+    if ((p.reduce_op == NT_MAP_REDUCE_NONE) != (p.num_reduced == 0 && p.reduce_split == p.value_code_length)) return false;
+    for (int i = 0; i < p.num_operands; ++i) {
+        const NineToothedMapOperand &operand = p.operands[i];
+        if (operand.dtype < NINETOOTHED_INT8 || operand.dtype > NINETOOTHED_FLOAT64) return false;
+        if (operand.segment < 0 || operand.segment >= p.num_segments) return false;
+    }
+    // every segment must end inside the code array, use known opcodes, in-range
+    // arguments, and keep the stack within its bounds
+    for (int s = 0; s < p.num_segments; ++s) {
+        int pc = p.segment_begin[s];
+        if (pc < 0) return false;
+        int depth = 0;
+        for (;; ++pc) {
+            if (pc >= NT_MAP_MAX_INDEX_CODE) return false;
+            const int op = p.index_code[pc] & 0xff, arg = p.index_code[pc] >> 8;
+            if (op == NT_MAP_I_END) break;
+            if (op == NT_MAP_I_VAR) {
+                if (arg < 0 || arg >= p.num_vars) return false;
+                ++depth;
+            } else if (op == NT_MAP_I_ADD) {
+                if (depth < 2) return false;
+                --depth;
+            } else if (op == NT_MAP_I_CONST || op == NT_MAP_I_MULC || op == NT_MAP_I_DIVC || op == NT_MAP_I_MODC || op == NT_MAP_I_CHECK) {
+                if (arg < 0 || arg >= NT_MAP_MAX_INDEX_CONSTANTS) return false;
+                if ((op == NT_MAP_I_DIVC || op == NT_MAP_I_MODC) && p.index_constants[arg] == 0) return false;
+                if (op == NT_MAP_I_CONST) ++depth;
+                else if (depth < 1) return false;
+                if (op == NT_MAP_I_CHECK) --depth;
+            } else {
+                return false;
+            }
+            if (depth > kIndexStack) return false;
+        }
+    }
+    int depth = 0;
+    for (int pc = 0; pc < p.value_code_length; ++pc) {
+        if (pc == p.reduce_split && p.reduce_op != NT_MAP_REDUCE_NONE) {
+            if (depth != 1) return false;  // the per-position code leaves exactly the term
+        }
+        const int op = p.value_code[pc] & 0xff, arg = p.value_code[pc] >> 8;
+        if (op == NT_MAP_V_LOAD) {
+            if (arg < 0 || arg >= p.num_operands) return false;
+            ++depth;
+        } else if (op == NT_MAP_V_CONST) {
+            if (arg < 0 || arg >= NT_MAP_MAX_VALUE_CONSTANTS) return false;
+            ++depth;
+        } else if (op == NT_MAP_V_OFFSET) {
+            if (arg < 0 || arg >= p.num_segments) return false;
+            ++depth;
+        } else if (op >= NT_MAP_V_ADD && op <= NT_MAP_V_OR) {
+            if (depth < 2) return false;
+            --depth;
+        } else if (op >= NT_MAP_V_NEG && op <= NT_MAP_V_CEIL) {
+            if (depth < 1) return false;
+        } else if (op == NT_MAP_V_WHERE) {
+            if (depth < 3) return false;
+            depth -= 2;
+        } else if (op == NT_MAP_V_ROUND) {
+            if (depth < 1 || arg < NINETOOTHED_INT8 || arg > NINETOOTHED_FLOAT64) return false;
+        } else if (op == NT_MAP_V_RAND) {
+            if (depth < 2) return false;
+            --depth;
+        } else {
+            return false;
+        }
+        if (depth > kValueStack) return false;
+    }
+    if (p.reduce_op != NT_MAP_REDUCE_NONE && p.reduce_split == p.value_code_length && depth != 1) return false;
+    return depth == 1;
+}
+
+
+// ---- specialised kernels through hipRTC ----------------------------------------------
+
+struct MapJitArgs {
+    void *data[NT_MAP_MAX_OPERANDS];
+    double other[NT_MAP_MAX_OPERANDS];
+    double constants[NT_MAP_MAX_VALUE_CONSTANTS];
+    long long total_out;
+};
+
+const char *c_type(int dtype) {
+    switch (dtype) {
+        case NINETOOTHED_INT8: return "signed char";
+        case NINETOOTHED_INT16: return "short";
+        case NINETOOTHED_INT32: return "int";
+        case NINETOOTHED_INT64: return "long long";
+        case NINETOOTHED_UINT8: return "unsigned char";
+        case NINETOOTHED_UINT16: return "unsigned short";
+        case NINETOOTHED_UINT32: return "unsigned int";
+        case NINETOOTHED_UINT64: return "unsigned long long";
+        case NINETOOTHED_FLOAT16: return "_Float16";
+        case NINETOOTHED_BFLOAT16: return "__bf16";
+        case NINETOOTHED_FLOAT32: return "float";
+        default: return "double";
+    }
+}
+
+std::string round_expr(const std::string &v, int dtype) {
+    switch (dtype) {
+        case NINETOOTHED_FLOAT16: return "(double)(float)(_Float16)(float)(" + v + ")";
+        case NINETOOTHED_BFLOAT16: return "(double)(float)(__bf16)(float)(" + v + ")";
+        case NINETOOTHED_FLOAT32: return "(double)(float)(" + v + ")";
+        case NINETOOTHED_FLOAT64: return v;
+        case NINETOOTHED_UINT64: return "(double)(unsigned long long)(" + v + ")";
+        case NINETOOTHED_INT64: return "(double)(long long)(" + v + ")";
+        default: return std::string("(double)(") + c_type(dtype) + ")(long long)(" + v + ")";
+    }
+}
+
+std::string load_expr(const std::string &pointer, int dtype, const std::string &offset) {
+    const std::string element = std::string("((const ") + c_type(dtype) + " *)" + pointer + ")[" + offset + "]";
+    if (dtype == NINETOOTHED_FLOAT16 || dtype == NINETOOTHED_BFLOAT16) return "(double)(float)" + element;
+    return "(double)" + element;
+}
+
+std::string store_stmt(const std::string &pointer, int dtype, const std::string &offset, const std::string &v) {
+    const std::string target = std::string("((") + c_type(dtype) + " *)" + pointer + ")[" + offset + "]";
+    switch (dtype) {
+        case NINETOOTHED_FLOAT16:
+        case NINETOOTHED_BFLOAT16: return target + " = (" + c_type(dtype) + ")(float)(" + v + ");";
+        case NINETOOTHED_FLOAT32:
+        case NINETOOTHED_FLOAT64:
+        case NINETOOTHED_INT64:
+        case NINETOOTHED_UINT64: return target + " = (" + c_type(dtype) + ")(" + v + ");";
+        default: return target + " = (" + c_type(dtype) + ")(long long)(" + v + ");";
+    }
+}
+
+// Translates the programs into HIP source.  `counter` numbers temporaries.
+struct MapCodegen {
+    const NineToothedMapProgram &p;
+    std::ostringstream out;
+    int counter = 0;
+    std::string indent = "        ";
+
+    explicit MapCodegen(const NineToothedMapProgram &program) : p(program) {}
+
+    std::string fresh(const char *prefix) { return prefix + std::to_string(counter++); }
+
+    // emits the statements of one index segment; returns the offset expression and
+    // and-s the checks into `valid` (a declared bool variable) when it is not empty
+    std::string index_segment(int segment, const std::string &valid) {
+        std::vector<std::string> stack;
+        for (int pc = p.segment_begin[segment];; ++pc) {
+            const int op = p.index_code[pc] & 0xff, arg = p.index_code[pc] >> 8;
+            if (op == NT_MAP_I_END) break;
+            switch (op) {
+                case NT_MAP_I_CONST: stack.push_back(std::to_string((long long)p.index_constants[arg]) + "LL"); break;
+                case NT_MAP_I_VAR: stack.push_back("v" + std::to_string(arg)); break;
+                case NT_MAP_I_MULC: stack.back() = "(" + stack.back() + " * " + std::to_string((long long)p.index_constants[arg]) + "LL)"; break;
+                case NT_MAP_I_ADD: {
+                    const std::string b = stack.back();
+                    stack.pop_back();
+                    stack.back() = "(" + stack.back() + " + " + b + ")";
+                    break;
+                }
+                case NT_MAP_I_DIVC:
+                case NT_MAP_I_MODC: {
+                    const std::string name = fresh("i");
+                    const std::string c = std::to_string((long long)p.index_constants[arg]) + "LL";
+                    out << indent << "const long long " << name << " = " << (op == NT_MAP_I_DIVC ? "nt_floor_div(" : "nt_floor_mod(") << stack.back() << ", " << c << ");\n";
+                    stack.back() = name;
+                    break;
+                }
+                case NT_MAP_I_CHECK: {
+                    const std::string name = fresh("i");
+                    out << indent << "const long long " << name << " = " << stack.back() << ";\n";
+                    out << indent << valid << " = " << valid << " && " << name << " >= 0 && " << name << " < " << (long long)p.index_constants[arg] << "LL;\n";
+                    stack.pop_back();
+                    break;
+                }
+            }
+        }
+        const std::string name = fresh("i");
+        out << indent << "const long long " << name << " = " << (stack.empty() ? std::string("0LL") : stack.back()) << ";\n";
+        return name;
+    }
+
+    // emits value_code[begin, end); `seed` (if not empty) is the initial stack entry
+    std::string value_range(int begin, int end, const std::string &seed) {
+        std::vector<std::string> stack;
+        if (!seed.empty()) stack.push_back(seed);
+        auto define = [&](const std::string &expr) {
+            const std::string name = fresh("t");
+            out << indent << "const double " << name << " = " << expr << ";\n";
+            return name;
+        };
+        for (int pc = begin; pc < end; ++pc) {
+            const int op = p.value_code[pc] & 0xff, arg = p.value_code[pc] >> 8;
+            if (op == NT_MAP_V_LOAD) {
+                const NineToothedMapOperand &operand = p.operands[arg];
+                const std::string valid = fresh("ok");
+                out << indent << "bool " << valid << " = true;\n";
+                const std::string offset = index_segment(operand.segment, valid);
+                const std::string pointer = "a.data[" + std::to_string(arg) + "]";
+                stack.push_back(define(valid + " ? " + load_expr(pointer, operand.dtype, offset) + " : a.other[" + std::to_string(arg) + "]"));
+            } else if (op == NT_MAP_V_CONST) {
+                stack.push_back("a.constants[" + std::to_string(arg) + "]");
+            } else if (op == NT_MAP_V_OFFSET) {
+                const std::string valid = fresh("ok");
+                out << indent << "bool " << valid << " = true;\n";
+                stack.push_back(define("(double)" + index_segment(arg, valid)));
+            } else if (op >= NT_MAP_V_ADD && op <= NT_MAP_V_OR) {
+                const std::string b = stack.back();
+                stack.pop_back();
+                const std::string a = stack.back();
+                std::string e;
+                switch (op) {
+                    case NT_MAP_V_ADD: e = a + " + " + b; break;
+                    case NT_MAP_V_SUB: e = a + " - " + b; break;
+                    case NT_MAP_V_MUL: e = a + " * " + b; break;
+                    case NT_MAP_V_DIV: e = a + " / " + b; break;
+                    case NT_MAP_V_FLOORDIV: e = "floor(" + a + " / " + b + ")"; break;
+                    case NT_MAP_V_MOD: e = a + " - floor(" + a + " / " + b + ") * " + b; break;
+                    case NT_MAP_V_POW: e = "(double)powf((float)" + a + ", (float)" + b + ")"; break;
+                    case NT_MAP_V_MAX: e = "(" + a + " != " + a + " || " + b + " != " + b + ") ? (" + a + " + " + b + ") : (" + a + " > " + b + " ? " + a + " : " + b + ")"; break;
+                    case NT_MAP_V_MIN: e = "(" + a + " != " + a + " || " + b + " != " + b + ") ? (" + a + " + " + b + ") : (" + a + " < " + b + " ? " + a + " : " + b + ")"; break;
+                    case NT_MAP_V_LT: e = a + " < " + b + " ? 1.0 : 0.0"; break;
+                    case NT_MAP_V_LE: e = a + " <= " + b + " ? 1.0 : 0.0"; break;
+                    case NT_MAP_V_GT: e = a + " > " + b + " ? 1.0 : 0.0"; break;
+                    case NT_MAP_V_GE: e = a + " >= " + b + " ? 1.0 : 0.0"; break;
+                    case NT_MAP_V_EQ: e = a + " == " + b + " ? 1.0 : 0.0"; break;
+                    case NT_MAP_V_NE: e = a + " != " + b + " ? 1.0 : 0.0"; break;
+                    case NT_MAP_V_AND: e = "(" + a + " != 0.0 && " + b + " != 0.0) ? 1.0 : 0.0"; break;
+                    default: e = "(" + a + " != 0.0 || " + b + " != 0.0) ? 1.0 : 0.0"; break;
+                }
+                stack.back() = define(e);
+            } else if (op >= NT_MAP_V_NEG && op <= NT_MAP_V_CEIL) {
+                const std::string a = stack.back();
+                std::string e;
+                switch (op) {
+                    case NT_MAP_V_NEG: e = "-" + a; break;
+                    case NT_MAP_V_NOT: e = a + " == 0.0 ? 1.0 : 0.0"; break;
+                    case NT_MAP_V_ABS: e = "fabs(" + a + ")"; break;
+                    case NT_MAP_V_EXP: e = "(double)expf((float)" + a + ")"; break;
+                    case NT_MAP_V_EXP2: e = "(double)exp2f((float)" + a + ")"; break;
+                    case NT_MAP_V_LOG: e = "(double)logf((float)" + a + ")"; break;
+                    case NT_MAP_V_LOG2: e = "(double)log2f((float)" + a + ")"; break;
+                    case NT_MAP_V_SQRT: e = "sqrt(" + a + ")"; break;
+                    case NT_MAP_V_RSQRT: e = "(double)(1.0f / sqrtf((float)" + a + "))"; break;
+                    case NT_MAP_V_SIGMOID: e = "(double)(1.0f / (1.0f + expf(-(float)" + a + ")))"; break;
+                    case NT_MAP_V_TANH: e = "(double)tanhf((float)" + a + ")"; break;
+                    case NT_MAP_V_SIN: e = "(double)sinf((float)" + a + ")"; break;
+                    case NT_MAP_V_COS: e = "(double)cosf((float)" + a + ")"; break;
+                    case NT_MAP_V_FLOOR: e = "floor(" + a + ")"; break;
+                    default: e = "ceil(" + a + ")"; break;
+                }
+                stack.back() = define(e);
+            } else if (op == NT_MAP_V_WHERE) {
+                const std::string b = stack.back();
+                stack.pop_back();
+                const std::string a = stack.back();
+                stack.pop_back();
+                stack.back() = define(stack.back() + " != 0.0 ? " + a + " : " + b);
+            } else if (op == NT_MAP_V_ROUND) {
+                stack.back() = define(round_expr(stack.back(), arg));
+            } else if (op == NT_MAP_V_RAND) {
+                const std::string offset = stack.back();
+                stack.pop_back();
+                stack.back() = define("nt_philox_uniform((unsigned long long)(long long)" + stack.back() + ", (unsigned long long)(long long)" + offset + ")");
+            }
+        }
+        return stack.empty() ? std::string("0.0") : stack.back();
+    }
+
+    std::string generate() {
+        const int num_out = p.num_vars - p.num_reduced;
+        out << "struct MapJitArgs { void *data[" << NT_MAP_MAX_OPERANDS << "]; double other[" << NT_MAP_MAX_OPERANDS << "]; double constants["
+            << NT_MAP_MAX_VALUE_CONSTANTS << "]; long long total_out; };\n"
+            << "__device__ inline long long nt_floor_div(long long a, long long b) { long long q = a / b; if ((a % b != 0) && ((a < 0) != (b < 0))) --q; return q; }\n"
+            << "__device__ inline long long nt_floor_mod(long long a, long long b) { return a - nt_floor_div(a, b) * b; }\n"
+            << "__device__ inline double nt_philox_uniform(unsigned long long seed, unsigned long long offset) {\n"
+            << "    unsigned int c0 = (unsigned int)offset, c1 = (unsigned int)(offset >> 32), c2 = 0, c3 = 0;\n"
+            << "    unsigned int k0 = (unsigned int)seed, k1 = (unsigned int)(seed >> 32);\n"
+            << "    for (int round = 0; round < 10; ++round) {\n"
+            << "        const unsigned int ra = 0xD2511F53u, rb = 0xCD9E8D57u, p0 = c0, p2 = c2;\n"
+            << "        c0 = __umulhi(rb, p2) ^ c1 ^ k0; c2 = __umulhi(ra, p0) ^ c3 ^ k1; c1 = rb * p2; c3 = ra * p0;\n"
+            << "        k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;\n"
+            << "    }\n"
+            << "    int x = (int)c0; if (x < 0) x = -x - 1;\n"
+            << "    return (double)((float)x * 4.6566127342e-10f);\n"
+            << "}\n"
+            << "extern \"C\" __global__ __launch_bounds__(" << kMapThreads << ") void nt_map_specialised(const MapJitArgs a) {\n"
+            << "    const long long stride = (long long)gridDim.x * " << kMapThreads << ";\n"
+            << "    for (long long element = (long long)blockIdx.x * " << kMapThreads << " + threadIdx.x; element < a.total_out; element += stride) {\n"
+            << "        long long rest = element;\n";
+        for (int v = num_out - 1; v >= 0; --v) {
+            // 32-bit division when the extent allows it would be cheaper; the divisor is a literal either way
+            out << "        const long long v" << v << " = rest % " << (long long)p.extents[v] << "LL; rest /= " << (long long)p.extents[v] << "LL;\n";
+        }
+        std::string result;
+        if (p.reduce_op == NT_MAP_REDUCE_NONE) {
+            result = value_range(0, p.value_code_length, "");
+        } else {
+            const char *init = p.reduce_op == NT_MAP_REDUCE_SUM ? "0.0" : (p.reduce_op == NT_MAP_REDUCE_MAX ? "-__builtin_inf()" : "__builtin_inf()");
+            out << "        double acc = " << init << ";\n";
+            for (int v = num_out; v < p.num_vars; ++v) {
+                out << indent << "for (long long v" << v << " = 0; v" << v << " < " << (long long)p.extents[v] << "LL; ++v" << v << ") {\n";
+                indent += "    ";
+            }
+            const std::string term = value_range(0, p.reduce_split, "");
+            if (p.reduce_op == NT_MAP_REDUCE_SUM) {
+                out << indent << "acc = " << round_expr("acc + " + term, p.reduce_dtype) << ";\n";
+            } else {
+                const char *cmp = p.reduce_op == NT_MAP_REDUCE_MAX ? ">" : "<";
+                out << indent << "acc = (" << term << " != " << term << " || acc != acc) ? acc + " << term << " : (" << term << " " << cmp << " acc ? " << term << " : acc);\n";
+            }
+            for (int v = num_out; v < p.num_vars; ++v) {
+                indent.resize(indent.size() - 4);
+                out << indent << "}\n";
+            }
+            result = value_range(p.reduce_split, p.value_code_length, "acc");
+        }
+        const NineToothedMapOperand &target = p.operands[p.output];
+        out << indent << "bool store_ok = true;\n";
+        const std::string offset = index_segment(target.segment, "store_ok");
+        out << indent << "if (store_ok) " << store_stmt("a.data[" + std::to_string(p.output) + "]", target.dtype, offset, result) << "\n";
+        out << "    }\n}\n";
+        return out.str();
+    }
+};
+
+// hipRTC entry points, resolved at first use so that the library loads without it
+struct Hiprtc {
+    void *handle = nullptr;
+    hiprtcResult (*create)(hiprtcProgram *, const char *, const char *, int, const char **, const char **) = nullptr;
+    hiprtcResult (*compile)(hiprtcProgram, int, const char **) = nullptr;
+    hiprtcResult (*code_size)(hiprtcProgram, size_t *) = nullptr;
+    hiprtcResult (*code)(hiprtcProgram, char *) = nullptr;
+    hiprtcResult (*log_size)(hiprtcProgram, size_t *) = nullptr;
+    hiprtcResult (*log)(hiprtcProgram, char *) = nullptr;
+    hiprtcResult (*destroy)(hiprtcProgram *) = nullptr;
+    bool ok = false;
+
+    Hiprtc() {
+        for (const char *name : {"libhiprtc.so", "libhiprtc.so.7", "/opt/rocm/lib/libhiprtc.so"}) {
+            handle = dlopen(name, RTLD_NOW | RTLD_LOCAL);
+            if (handle) break;
+        }
+        if (!handle) return;
+        create = (decltype(create))dlsym(handle, "hiprtcCreateProgram");
+        compile = (decltype(compile))dlsym(handle, "hiprtcCompileProgram");
+        code_size = (decltype(code_size))dlsym(handle, "hiprtcGetCodeSize");
+        code = (decltype(code))dlsym(handle, "hiprtcGetCode");
+        log_size = (decltype(log_size))dlsym(handle, "hiprtcGetProgramLogSize");
+        log = (decltype(log))dlsym(handle, "hiprtcGetProgramLog");
+        destroy = (decltype(destroy))dlsym(handle, "hiprtcDestroyProgram");
+        ok = create && compile && code_size && code && log_size && log && destroy;
+    }
+};
+
+std::mutex g_jit_mutex;
+std::unordered_map<std::string, hipFunction_t> g_jit_cache;  // a null function = "do not try again"
+
+hipFunction_t specialised_kernel(const NineToothedMapProgram &p) {
+    static Hiprtc rtc;
+    if (!rtc.ok) return nullptr;
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) return nullptr;
+    // the key is everything the source depends on: all of the program but pointers,
+    // `other` values and value constants (those are kernel arguments)
+    NineToothedMapProgram shape = p;
+    for (int i = 0; i < NT_MAP_MAX_OPERANDS; ++i) {
+        shape.operands[i].data = nullptr;
+        shape.operands[i].other = 0.0;
+        if (i >= p.num_operands) shape.operands[i].dtype = shape.operands[i].segment = 0;
+    }
+    memset(shape.value_constants, 0, sizeof(shape.value_constants));
+    for (int v = p.num_vars; v < NT_MAP_MAX_VARS; ++v) shape.extents[v] = 0;
+    for (int i = p.num_segments; i < NT_MAP_MAX_SEGMENTS; ++i) shape.segment_begin[i] = 0;
+    for (int i = p.value_code_length; i < NT_MAP_MAX_VALUE_CODE; ++i) shape.value_code[i] = 0;
+    std::string key((const char *)&shape, sizeof(shape));
+    key.push_back((char)device);
+    std::lock_guard<std::mutex> lock(g_jit_mutex);
+    auto found = g_jit_cache.find(key);
+    if (found != g_jit_cache.end()) return found->second;
+    MapCodegen generator(p);
+    const std::string source = generator.generate();
+    hipFunction_t function = nullptr;
+    hiprtcProgram program = nullptr;
+    if (rtc.create(&program, source.c_str(), "nt_map_specialised.hip", 0, nullptr, nullptr) == HIPRTC_SUCCESS) {
+        // same code generation switches as the rest of the library: gfx950, packed FP32 off
+        const char *options[] = {"--offload-arch=gfx950", "-O3", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+        const hiprtcResult compiled = rtc.compile(program, 6, options);
+        if (compiled == HIPRTC_SUCCESS) {
+            size_t size = 0;
+            if (rtc.code_size(program, &size) == HIPRTC_SUCCESS && size > 0) {
+                std::vector<char> binary(size);
+                hipModule_t module = nullptr;
+                if (rtc.code(program, binary.data()) == HIPRTC_SUCCESS && hipModuleLoadData(&module, binary.data()) == hipSuccess) {
+                    if (hipModuleGetFunction(&function, module, "nt_map_specialised") != hipSuccess) function = nullptr;
+                }
+            }
+        } else if (getenv("NT_MAP_VERBOSE")) {
+            size_t size = 0;
+            rtc.log_size(program, &size);
+            std::vector<char> text(size + 1, 0);
+            rtc.log(program, text.data());
+            fprintf(stderr, "nt_hip: specialising a tile map failed:\n%s\n%s\n", text.data(), source.c_str());
+        }
+        rtc.destroy(&program);
+    }
+    g_jit_cache.emplace(key, function);
+    return function;
+}
+
+}  // namespace
+}  // namespace nt
+
+using namespace nt;
+
+extern "C" NineToothedResult launch_nt_map(NineToothedStream stream, const NineToothedMapProgram *program) {
+    if (program == nullptr) return hipErrorInvalidValue;
+    const NineToothedMapProgram &p = *program;
+    if (!well_formed(p)) return NINETOOTHED_NO_KERNEL;
+    int64_t total_out = 1, total_reduced = 1;
+    const int num_out = p.num_vars - p.num_reduced;
+    for (int v = 0; v < p.num_vars; ++v) {
+        if (p.extents[v] < 0) return hipErrorInvalidValue;
+        if (v < num_out) total_out *= p.extents[v];
+        else total_reduced *= p.extents[v];
+        if (total_out > (int64_t)1 << 46 || total_reduced > (int64_t)1 << 46) return NINETOOTHED_NO_KERNEL;
+    }
+    if (total_out == 0) return 0;  // empty launch is legal
+    for (int i = 0; i < p.num_operands; ++i)
+        if (p.operands[i].data == nullptr) return hipErrorInvalidValue;
+    // enough workgroups for 8 per CU; the grid stride covers the rest
+    int64_t blocks = (total_out + kMapThreads - 1) / kMapThreads;
+    if (blocks > 256 * 32) blocks = 256 * 32;
+    const char *interpret = getenv("NT_MAP_INTERPRET");
+    if (!(interpret && interpret[0] == '1')) {
+        if (hipFunction_t function = specialised_kernel(p)) {
+            MapJitArgs args;
+            for (int i = 0; i < NT_MAP_MAX_OPERANDS; ++i) {
+                args.data[i] = i < p.num_operands ? p.operands[i].data : nullptr;
+                args.other[i] = i < p.num_operands ? p.operands[i].other : 0.0;
+            }
+            memcpy(args.constants, p.value_constants, sizeof(args.constants));
+            args.total_out = total_out;
+            size_t size = sizeof(args);
+            void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+            return (int)hipModuleLaunchKernel(function, (unsigned)blocks, 1, 1, kMapThreads, 1, 1, 0, (hipStream_t)stream, nullptr, config);
+        }
+    }
+    map_kernel<<<dim3((unsigned)blocks), dim3(kMapThreads), 0, (hipStream_t)stream>>>(p, total_out, total_reduced);
+    return (int)hipGetLastError();
+}
+
+extern "C" NineToothedResult nt_map_source(const NineToothedMapProgram *program, char *buffer, int size) {
+    if (program == nullptr || buffer == nullptr || size <= 0) return hipErrorInvalidValue;
+    if (!well_formed(*program)) return NINETOOTHED_NO_KERNEL;
+    MapCodegen generator(*program);
+    const std::string source = generator.generate();
+    if ((int)source.size() + 1 > size) return hipErrorInvalidValue;
+    memcpy(buffer, source.c_str(), source.size() + 1);
+    return 0;
+}

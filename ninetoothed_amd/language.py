@@ -51,10 +51,27 @@ _FUNCTIONS = (
     "program_id",
     "rand",
     "cdiv",
+    "sin",
+    "cos",
+    "floor",
+    "ceil",
 )
 
 for _name in _FUNCTIONS:
     globals()[_name] = _Function(_name)
+
+
+class _LibDevice:
+    """``ninetoothed.language.libdevice``: math functions by name
+    (src/ninetoothed/language.py:1-26 re-exports Triton's ``libdevice``)."""
+
+    def __getattr__(self, name):
+        if name.startswith("_"):
+            raise AttributeError(name)
+        return _Function("libdevice." + name)
+
+
+libdevice = _LibDevice()
 
 int8 = _dtype.int8
 int16 = _dtype.int16

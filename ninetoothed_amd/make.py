@@ -45,6 +45,7 @@ def _dtype_tag(torch_dtype):
             torch.bfloat16: "bf16",
             torch.float32: "fp32",
             torch.float64: "fp64",
+            torch.bool: "u8",
         }
     try:
         return _TORCH_DTYPE_TAGS[torch_dtype]
@@ -131,6 +132,12 @@ class Kernel:
                 f"# executed by libnt_hip.so ({runtime.LIBRARY_PATH})\n"
                 f"# dataflow graph of the application (digest {self.program.digest}):\n" + self.program.describe() + "\n"
             )
+            for program in getattr(self, "_map_programs", ()):
+                import ctypes
+
+                buffer = ctypes.create_string_buffer(1 << 16)
+                if runtime.library().nt_map_source(ctypes.addressof(program), buffer, len(buffer)) == 0:
+                    text += "# HIP source of the latest prepared launch:\n" + buffer.value.decode() + "\n"
             CACHE_DIR.mkdir(parents=True, exist_ok=True)
             path = CACHE_DIR / (hashlib.sha256(text.encode()).hexdigest() + ".txt")
             if not path.exists():
@@ -158,7 +165,7 @@ class Kernel:
                 parts.append((tuple(arg.shape), tuple(arg.stride()), arg.dtype, arg.device.index))
         return tuple(parts), tuple(sorted(kwargs.items()))
 
-    def _environment(self, args, kwargs):
+    def _environment(self, args, kwargs, check_device=True):
         import torch
 
         env = {}
@@ -170,7 +177,7 @@ class Kernel:
                 continue
             if not isinstance(arg, torch.Tensor):
                 raise TypeError(f"`{name}` must be a torch tensor, not `{type(arg).__name__}`.")
-            if not arg.is_cuda:
+            if check_device and not arg.is_cuda:
                 raise RuntimeError(f"`{name}` lives on `{arg.device}`; this build only runs on the GPU (there is no CPU path).")
             if arg.ndim != source.ndim:
                 raise ValueError(f"`{name}` must have {source.ndim} dimensions, got {arg.ndim}.")
@@ -293,6 +300,37 @@ class Kernel:
             runtime.check(lib.launch_nt_softmax(runtime.current_stream(), input, output, dtype, block))
 
         return _Plan(f"launch_nt_softmax {info['input']['rows']}x{info['input']['cols']} {tag} block {block}", launch)
+
+    def _prepare_map(self, args, env):
+        """Element-wise / reducing programs: one interpreter launch per store."""
+        import ctypes
+
+        from ninetoothed_amd import mapping
+
+        lib = runtime.library()
+        tensor_params = [p for p, t in enumerate(self.types) if not (t.ndim == 0 and not isinstance(t.dtype, Tensor))]
+        for p in tensor_params:
+            if args[p].numel() > 0 and args[p].data_ptr() % args[p].element_size():
+                raise UnsupportedProgram("Tensor data must be aligned to its element size.")
+        launches = []
+        for store in self.program.stores:
+            built = mapping.build(store, self.types, args, env, lambda p: _dtype_tag(args[p].dtype), lambda p: args[p].data_ptr())
+            if built is not None:
+                launches.append(built)
+        if not launches:
+            return _Plan("empty launch", lambda call_args: None)
+
+        def launch(call_args):
+            stream = runtime.current_stream()
+            for program, _, scalar_slots, operand_params in launches:
+                for slot, param in enumerate(operand_params):
+                    program.operands[slot].data = call_args[param].data_ptr()
+                for index, param in scalar_slots:
+                    program.value_constants[index] = float(call_args[param])
+                runtime.check(lib.launch_nt_map(stream, ctypes.addressof(program)))
+
+        self._map_programs = [program for program, _, _, _ in launches]
+        return _Plan("launch_nt_map " + "; ".join(description for _, description, _, _ in launches), launch)
 
     def _prepare_attention(self, args, env):
         scaled = self.details["scale"]

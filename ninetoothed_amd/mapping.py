@@ -1,0 +1,569 @@
+"""Lowers element-wise / reducing tile programs to the interpreter kernel of
+``libnt_hip.so`` (``launch_nt_map``).
+
+The reference generates a Triton kernel for any arrange-and-apply pair
+(src/ninetoothed/generation.py:28-837).  Programs that are none of the
+recognised ones (matmul, addmm, softmax, attention, conv2d) run here if their
+application is a *tile map*: every store assigns, to a tile of an output
+parameter, an expression over whole tiles of the other parameters, call-time
+scalars and constants, with at most one ``ntl.max`` / ``ntl.min`` / ``ntl.sum``
+reduction (the programs of the reference's tests/test_add.py, test_clone.py
+(first application), test_pad.py, test_pow.py, test_dropout.py,
+test_max_pool2d.py, test_generation.py:139-151).
+
+Two lowerings happen per call signature:
+
+* every operand's index map (:meth:`Tensor.index_map`, normal form of
+  :mod:`ninetoothed_amd.affine`) becomes a stack program over shared index
+  variables -- the launch grid's dimensions, the output tile's dimensions, the
+  reduced dimensions -- with the arrangement's masks as range checks;
+* the dataflow graph of the stored value becomes a stack program over
+  doubles, with a rounding step wherever the reference holds the value in a
+  narrower type (type promotion as Triton applies it to the generated code: a
+  Python literal takes the tile's type, a run-time ``float`` argument is fp32,
+  mixed half types promote to fp32, ``/`` on integers gives fp32, sums of
+  fp16 / bf16 tiles accumulate in fp32).
+"""
+
+import ctypes
+
+from ninetoothed_amd import runtime
+from ninetoothed_amd.affine import Affine
+from ninetoothed_amd.recognition import Operand, UnsupportedProgram
+from ninetoothed_amd.tracing import ElementType, Node, ScalarParam, TensorRef
+
+MAX_OPERANDS = 8
+MAX_VARS = 16
+MAX_INDEX_CODE = 320
+MAX_INDEX_CONSTANTS = 96
+MAX_SEGMENTS = 16
+MAX_VALUE_CODE = 128
+MAX_VALUE_CONSTANTS = 32
+
+I_END, I_CONST, I_VAR, I_MULC, I_ADD, I_DIVC, I_MODC, I_CHECK = range(8)
+
+_VALUE_OPS = (
+    "LOAD CONST OFFSET ADD SUB MUL DIV FLOORDIV MOD POW MAX MIN LT LE GT GE EQ NE AND OR "
+    "NEG NOT ABS EXP EXP2 LOG LOG2 SQRT RSQRT SIGMOID TANH SIN COS FLOOR CEIL WHERE ROUND RAND"
+).split()
+V = {name: index for index, name in enumerate(_VALUE_OPS)}
+
+REDUCE = {"max": 1, "min": 2, "sum": 3}
+
+
+class MapOperand(ctypes.Structure):
+    _fields_ = [("data", ctypes.c_void_p), ("dtype", ctypes.c_int32), ("segment", ctypes.c_int32), ("other", ctypes.c_double)]
+
+
+class MapProgram(ctypes.Structure):
+    _fields_ = [
+        ("num_vars", ctypes.c_int32),
+        ("num_reduced", ctypes.c_int32),
+        ("extents", ctypes.c_int64 * MAX_VARS),
+        ("num_operands", ctypes.c_int32),
+        ("output", ctypes.c_int32),
+        ("operands", MapOperand * MAX_OPERANDS),
+        ("num_segments", ctypes.c_int32),
+        ("segment_begin", ctypes.c_int32 * MAX_SEGMENTS),
+        ("index_code", ctypes.c_int32 * MAX_INDEX_CODE),
+        ("index_constants", ctypes.c_int64 * MAX_INDEX_CONSTANTS),
+        ("value_code_length", ctypes.c_int32),
+        ("reduce_split", ctypes.c_int32),
+        ("reduce_op", ctypes.c_int32),
+        ("reduce_dtype", ctypes.c_int32),
+        ("value_code", ctypes.c_int32 * MAX_VALUE_CODE),
+        ("value_constants", ctypes.c_double * MAX_VALUE_CONSTANTS),
+    ]
+
+
+# ---- types of values -----------------------------------------------------------
+
+_FLOATS = ("fp16", "bf16", "fp32", "fp64")
+_INT_RANK = {"bool": 0, "i8": 1, "u8": 1, "i16": 2, "u16": 2, "i32": 3, "u32": 3, "i64": 4, "u64": 4}
+_LITERAL_INT, _LITERAL_FLOAT = "int literal", "float literal"
+
+
+def _promote(a, b, division=False):
+    """Result type of an arithmetic operation (Triton's rules for the generated code)."""
+    literals = (_LITERAL_INT, _LITERAL_FLOAT)
+    if a in literals and b in literals:
+        return _LITERAL_FLOAT if _LITERAL_FLOAT in (a, b) or division else _LITERAL_INT
+    if a in literals or b in literals:
+        literal, other = (a, b) if a in literals else (b, a)
+        if other in _FLOATS:
+            return other
+        return "fp32" if literal == _LITERAL_FLOAT or division else other
+    if a in _FLOATS and b in _FLOATS:
+        if a == b:
+            return a
+        if {a, b} == {"fp16", "bf16"}:
+            return "fp32"
+        return max(a, b, key=_FLOATS.index) if "fp64" in (a, b) or "fp32" in (a, b) else "fp32"
+    if a in _FLOATS or b in _FLOATS:
+        return a if a in _FLOATS else b
+    if division:
+        return "fp32"
+    return a if _INT_RANK[a] >= _INT_RANK[b] else b
+
+
+def _needs_rounding(dtype):
+    return dtype in ("fp16", "bf16", "fp32") or dtype in _INT_RANK and dtype != "bool"
+
+
+# ---- the application: which programs are tile maps ----------------------------------
+
+_BINARY = {
+    "add": "ADD", "sub": "SUB", "mul": "MUL", "div": "DIV", "floordiv": "FLOORDIV", "mod": "MOD", "pow": "POW",
+    "maximum": "MAX", "minimum": "MIN", "libdevice.pow": "POW",
+}
+_COMPARE = {"lt": "LT", "le": "LE", "gt": "GT", "ge": "GE", "eq": "EQ", "ne": "NE"}
+_LOGICAL = {"and": "AND", "or": "OR"}
+_UNARY_SAME = {"neg": "NEG", "abs": "ABS", "floor": "FLOOR", "ceil": "CEIL", "libdevice.floor": "FLOOR", "libdevice.ceil": "CEIL"}
+_UNARY_FLOAT = {
+    "exp": "EXP", "exp2": "EXP2", "log": "LOG", "log2": "LOG2", "sqrt": "SQRT", "rsqrt": "RSQRT", "sigmoid": "SIGMOID",
+    "libdevice.tanh": "TANH", "libdevice.sin": "SIN", "libdevice.cos": "COS", "libdevice.exp": "EXP", "libdevice.log": "LOG",
+    "libdevice.sqrt": "SQRT", "libdevice.rsqrt": "RSQRT", "sin": "SIN", "cos": "COS",
+}
+
+
+def _kwargs(node):
+    positional, named = [], {}
+    for arg in node.args:
+        if isinstance(arg, Node) and arg.op == "kwarg":
+            named[arg.args[0]] = arg.args[1]
+        else:
+            positional.append(arg)
+    return positional, named
+
+
+class _Lowering:
+    """One store of one call: collects operands, index segments and value code."""
+
+    def __init__(self, types, args, env, dtype_tag):
+        self.types, self.args, self.env, self.dtype_tag = types, args, env, dtype_tag
+        self.operands = []        # (param, Operand)
+        self.operand_slot = {}    # param -> slot
+        self.var_extent = []      # shared variables: grid dims first, then output tile dims, then reduced dims
+        self.grid = None          # list of variable ids of the launch grid
+        self.segments = []        # (operand slot, kind, dim)
+        self.segment_slot = {}
+        self.value_code = []
+        self.constants = []
+        self.reduce = None        # (op name, accumulate dtype)
+        self.reduce_split = None
+        self.num_reduced = 0
+        self.bindings = {}        # operand slot -> {operand variable name: shared variable id}
+        self.scalar_slots = []    # (constant index, parameter position): refreshed at every launch
+        self.reduced_vars = []
+
+    # -- variables ---------------------------------------------------------
+    def new_var(self, extent):
+        self.var_extent.append(int(extent))
+        return len(self.var_extent) - 1
+
+    def operand(self, param):
+        if param in self.operand_slot:
+            return self.operand_slot[param]
+        tensor = self.types[param]
+        operand = Operand(tensor, self.env)
+        if len(operand.names) > 2:
+            raise UnsupportedProgram(f"`{tensor.source.name}` has more than one level below the launch grid.")
+        grid_names = operand.names[0]
+        if self.grid is None:
+            self.grid = [self.new_var(operand.extents[name]) for name in grid_names]
+        if len(grid_names) != len(self.grid):
+            raise UnsupportedProgram("The arranged tensors disagree on the number of launch-grid dimensions.")
+        binding = {}
+        for name, var in zip(grid_names, self.grid):
+            if operand.extents[name] != self.var_extent[var]:
+                raise UnsupportedProgram(
+                    f"`{tensor.source.name}` has {operand.extents[name]} tiles along a grid dimension where another tensor has {self.var_extent[var]}."
+                )
+            binding[name] = var
+        slot = len(self.operands)
+        if slot >= MAX_OPERANDS:
+            raise UnsupportedProgram("Too many tensor operands for the element-wise executor.")
+        self.operands.append((param, operand))
+        self.operand_slot[param] = slot
+        self.bindings[slot] = binding
+        return slot
+
+    def bind_tile(self, slot, dims):
+        """Binds the operand's tile dimensions to the shared variables ``dims``."""
+        _, operand = self.operands[slot]
+        tile_names = operand.names[1] if len(operand.names) > 1 else []
+        if len(tile_names) != len(dims):
+            raise UnsupportedProgram(
+                f"A tile of `{operand.tensor.source.name}` has {len(tile_names)} dimensions where the expression needs {len(dims)}."
+            )
+        binding = self.bindings[slot]
+        for name, var in zip(tile_names, dims):
+            extent = operand.extents[name]
+            if self.var_extent[var] is None:
+                self.var_extent[var] = extent
+            elif self.var_extent[var] != extent:
+                raise UnsupportedProgram(
+                    f"Tiles of different shapes meet in one expression ({extent} against {self.var_extent[var]} elements); broadcasting tiles is not supported."
+                )
+            if binding.get(name, var) != var:
+                raise UnsupportedProgram(f"`{operand.tensor.source.name}` is used with two different tile layouts.")
+            binding[name] = var
+
+    # -- value code -----------------------------------------------------------
+    def emit(self, op, arg=0):
+        self.value_code.append(V[op] | (arg << 8))
+
+    def constant(self, value):
+        value = float(value)
+        scalars = {index for index, _ in self.scalar_slots}
+        for index, known in enumerate(self.constants):
+            if index not in scalars and (known == value or (known != known and value != value)):
+                return index
+        self.constants.append(value)
+        return len(self.constants) - 1
+
+    def round(self, dtype):
+        if _needs_rounding(dtype):
+            self.emit("ROUND", runtime.DATA_TYPE_INDEX[dtype])
+
+    def segment(self, slot, kind, dim=None):
+        key = (slot, kind, dim)
+        if key not in self.segment_slot:
+            self.segment_slot[key] = len(self.segments)
+            self.segments.append(key)
+        return self.segment_slot[key]
+
+    def lower(self, value, dims, inside_reduction):
+        """Emits code that leaves ``value`` on the stack; returns its type."""
+        if isinstance(value, bool):
+            self.emit("CONST", self.constant(1.0 if value else 0.0))
+            return "bool"
+        if isinstance(value, int):
+            self.emit("CONST", self.constant(value))
+            return _LITERAL_INT
+        if isinstance(value, float):
+            self.emit("CONST", self.constant(value))
+            return _LITERAL_FLOAT
+        if isinstance(value, ScalarParam):
+            arg = self.args[value.param]
+            self.constants.append(float(arg))  # a slot of its own: call-time scalars are refreshed per launch
+            self.scalar_slots.append((len(self.constants) - 1, value.param))
+            self.emit("CONST", len(self.constants) - 1)
+            if value.constexpr:
+                return "bool" if isinstance(arg, bool) else _LITERAL_INT if isinstance(arg, int) else _LITERAL_FLOAT
+            if isinstance(arg, bool):
+                return "bool"
+            if isinstance(arg, int):
+                return "i32" if -(2**31) <= arg < 2**31 else "i64"
+            self.round("fp32")
+            return "fp32"
+        if not isinstance(value, Node):
+            raise UnsupportedProgram(f"A value of type `{type(value).__name__}` cannot be stored by the element-wise executor.")
+
+        op = value.op
+        if op == "load":
+            ref = value.args[0]
+            self._check_ref(ref)
+            if self.reduce is not None and not inside_reduction:
+                raise UnsupportedProgram("Tiles may only be loaded below the reduction of the expression.")
+            slot = self.operand(ref.param)
+            self.bind_tile(slot, dims)
+            self.emit("LOAD", slot)
+            return self.dtype_tag(ref.param)
+        if op == "offsets":
+            ref, dim = value.args
+            self._check_ref(ref)
+            slot = self.operand(ref.param)
+            self.bind_tile(slot, dims)
+            self.emit("OFFSET", self.segment(slot, "offsets", dim))
+            return "i64" if dim is None else "i32"
+        if op in _BINARY or op in _COMPARE or op in _LOGICAL:
+            positional, _ = _kwargs(value)
+            if len(positional) != 2:
+                raise UnsupportedProgram(f"`{op}` takes two operands.")
+            # a Python literal (or a constexpr scalar) takes the type of the tile it meets
+            # before the operation, as a constant of that type would
+            literals = (_LITERAL_INT, _LITERAL_FLOAT)
+            a = self.lower(positional[0], dims, inside_reduction)
+            mark = len(self.value_code)
+            b = self.lower(positional[1], dims, inside_reduction)
+            if a in literals and b not in literals and _needs_rounding(_promote(a, b)):
+                self.value_code.insert(mark, V["ROUND"] | (runtime.DATA_TYPE_INDEX[_promote(a, b)] << 8))
+                if self.reduce_split is not None and self.reduce_split >= mark:
+                    self.reduce_split += 1
+            elif b in literals and a not in literals and _needs_rounding(_promote(a, b)):
+                self.emit("ROUND", runtime.DATA_TYPE_INDEX[_promote(a, b)])
+            if op in _COMPARE:
+                self.emit(_COMPARE[op])
+                return "bool"
+            if op in _LOGICAL:
+                self.emit(_LOGICAL[op])
+                return "bool"
+            result = _promote(a, b, division=op == "div")
+            if op in ("pow", "libdevice.pow") and result not in _FLOATS:
+                result = "fp32"
+            self.emit(_BINARY[op])
+            self.round(result)
+            return result
+        if op in _UNARY_SAME or op in _UNARY_FLOAT:
+            positional, _ = _kwargs(value)
+            a = self.lower(positional[0], dims, inside_reduction)
+            if op in _UNARY_FLOAT:
+                if a not in _FLOATS:
+                    a = "fp32"
+                self.emit(_UNARY_FLOAT[op])
+                self.round(a)
+            else:
+                self.emit(_UNARY_SAME[op])
+            return a
+        if op == "pos":
+            return self.lower(value.args[0], dims, inside_reduction)
+        if op == "not":
+            self.lower(value.args[0], dims, inside_reduction)
+            self.emit("NOT")
+            return "bool"
+        if op == "where":
+            positional, _ = _kwargs(value)
+            if len(positional) != 3:
+                raise UnsupportedProgram("`where` takes a condition and two values.")
+            self.lower(positional[0], dims, inside_reduction)
+            a = self.lower(positional[1], dims, inside_reduction)
+            b = self.lower(positional[2], dims, inside_reduction)
+            self.emit("WHERE")
+            result = _promote(a, b)
+            self.round(result)
+            return result
+        if op == "cast":
+            source, target = value.args
+            self.lower(source, dims, inside_reduction)
+            if isinstance(target, ElementType):
+                target = self.dtype_tag(target.param)
+            if not isinstance(target, str) or target not in runtime.DATA_TYPE_INDEX:
+                raise UnsupportedProgram(f"Cannot cast to `{target!r}`.")
+            self.emit("ROUND", runtime.DATA_TYPE_INDEX[target])
+            return target
+        if op == "rand":
+            positional, _ = _kwargs(value)
+            if len(positional) != 2:
+                raise UnsupportedProgram("`rand` takes a seed and offsets.")
+            self.lower(positional[0], dims, inside_reduction)
+            self.lower(positional[1], dims, inside_reduction)
+            self.emit("RAND")
+            return "fp32"
+        if op in REDUCE:
+            if self.reduce is not None or inside_reduction:
+                raise UnsupportedProgram("Only one reduction per stored expression is supported.")
+            positional, named = _kwargs(value)
+            axis = named.get("axis", positional[1] if len(positional) > 1 else None)
+            if axis is not None and not isinstance(axis, int):
+                raise UnsupportedProgram("The reduction axis must be an integer constant.")
+            if self.value_code:
+                raise UnsupportedProgram("A reduction must be the innermost tile operation of the stored expression.")
+            if axis is None:
+                if any(self.var_extent[var] != 1 for var in dims):
+                    raise UnsupportedProgram("A full reduction yields a scalar; the stored tile has more than one element.")
+                rank = self._tile_rank(positional[0])
+                inner = [self.new_var_deferred() for _ in range(rank)]
+                reduced = list(inner)
+            else:
+                rank = len(dims) + 1
+                axis %= rank
+                fresh = self.new_var_deferred()
+                inner = list(dims[:axis]) + [fresh] + list(dims[axis:])
+                reduced = [fresh]
+            self.reduced_vars = reduced
+            self.reduce = (op, None)
+            term = self.lower(positional[0], inner, True)
+            accumulate = "fp32" if op == "sum" and term in ("fp16", "bf16") else term
+            if term in (_LITERAL_INT, _LITERAL_FLOAT):
+                raise UnsupportedProgram("A reduction needs a tile operand.")
+            self.reduce = (op, accumulate)
+            self.reduce_split = len(self.value_code)
+            if accumulate != term:
+                self.round(term)
+            return term
+        raise UnsupportedProgram(f"`{op}` is not an element-wise operation this build can execute.")
+
+    def new_var_deferred(self):
+        self.var_extent.append(None)
+        return len(self.var_extent) - 1
+
+    def _tile_rank(self, value):
+        ranks = set()
+
+        def visit(item):
+            if isinstance(item, Node):
+                if item.op == "load":
+                    ref = item.args[0]
+                    tensor = self.types[ref.param]
+                    ranks.add(tensor.dtype.ndim if hasattr(tensor.dtype, "ndim") else 0)
+                for arg in item.args:
+                    visit(arg)
+            elif isinstance(item, (tuple, list)):
+                for arg in item:
+                    visit(arg)
+
+        visit(value)
+        if len(ranks) != 1:
+            raise UnsupportedProgram("The operand of a full reduction must be built from tiles of one rank.")
+        return ranks.pop()
+
+    def _check_ref(self, ref):
+        if not isinstance(ref, TensorRef) or ref.level != 1 or ref.indices or not ref.is_tile:
+            raise UnsupportedProgram("Only whole tiles directly below the launch grid can be used by the element-wise executor.")
+
+    # -- index code ----------------------------------------------------------------
+    def index_program(self, order):
+        """Returns (code words, constants, segment begins) for all segments, with the
+        shared variables renumbered by ``order`` (old id -> new id)."""
+        code, constants, begins = [], [], []
+
+        def const(value):
+            value = int(value)
+            if value not in constants:
+                constants.append(value)
+            return constants.index(value)
+
+        def emit_affine(expr, binding):
+            code.append(I_CONST | (const(expr.const) << 8))
+            for atom, coef in sorted(expr.terms.items(), key=repr):
+                if atom[0] == "var":
+                    if atom[1] not in binding:
+                        raise UnsupportedProgram(f"Index variable `{atom[1]}` is not part of the iteration space.")
+                    code.append(I_VAR | (order[binding[atom[1]]] << 8))
+                else:
+                    emit_affine(Affine.from_key(atom[1]), binding)
+                    code.append((I_DIVC if atom[0] == "div" else I_MODC) | (const(atom[2]) << 8))
+                if coef != 1:
+                    code.append(I_MULC | (const(coef) << 8))
+                code.append(I_ADD)
+
+        for slot, kind, dim in self.segments:
+            _, operand = self.operands[slot]
+            binding = self.bindings[slot]
+            begins.append(len(code))
+            if kind == "access":
+                for index, size in operand.constraints:
+                    emit_affine(index, binding)
+                    code.append(I_CHECK | (const(size) << 8))
+                emit_affine(operand.offset(), binding)
+            elif dim is None:
+                emit_affine(operand.offset(), binding)
+            else:
+                emit_affine(operand.indices[dim], binding)
+            code.append(I_END)
+        return code, constants, begins
+
+
+def _other_value(tensor):
+    other = tensor.source.other
+    return 0.0 if other is None else float(other)
+
+
+def build(program_store, types, args, env, dtype_tag, data_ptr):
+    """Builds the :class:`MapProgram` of one store for one call.  Returns
+    ``None`` when the launch is empty."""
+
+    ref, value = program_store
+    lowering = _Lowering(types, args, env, dtype_tag)
+    lowering._check_ref(ref)
+    out_slot = lowering.operand(ref.param)
+    _, out_operand = lowering.operands[out_slot]
+    tile_names = out_operand.names[1] if len(out_operand.names) > 1 else []
+    out_dims = [lowering.new_var(out_operand.extents[name]) for name in tile_names]
+    lowering.bind_tile(out_slot, out_dims)
+    result = lowering.lower(value, out_dims, False)
+    out_dtype = dtype_tag(ref.param)
+    if result != out_dtype:
+        lowering.emit("ROUND", runtime.DATA_TYPE_INDEX[out_dtype])
+    if lowering.reduce is None:
+        lowering.reduce_split = len(lowering.value_code)
+    for slot in range(len(lowering.operands)):
+        lowering.segment(slot, "access")
+    if any(operand.empty for _, operand in lowering.operands):
+        return None
+    if any(extent is None for extent in lowering.var_extent):
+        raise UnsupportedProgram("A reduced dimension is not covered by any tile.")
+
+    # variable order: grid and output-tile variables enumerate the output elements
+    # (the fastest one is chosen so that lanes walk the output contiguously), reduced ones follow
+    reduced = list(lowering.reduced_vars)
+    outer = [v for v in range(len(lowering.var_extent)) if v not in reduced]
+    out_binding = lowering.bindings[out_slot]
+    offset = out_operand.offset()
+    stride_of = {}
+    for name, var in out_binding.items():
+        stride_of[var] = abs(offset.coef(name)) if offset.is_linear() else None
+    if all(stride_of.get(v) is not None for v in outer):
+        outer.sort(key=lambda v: (-(stride_of[v] or 1 << 62) if lowering.var_extent[v] > 1 else -(1 << 62), v))
+    order = {old: new for new, old in enumerate(outer + reduced)}
+    if len(order) > MAX_VARS:
+        raise UnsupportedProgram("Too many index variables for the element-wise executor.")
+
+    code, constants, begins = lowering.index_program(order)
+    if len(code) > MAX_INDEX_CODE or len(constants) > MAX_INDEX_CONSTANTS or len(begins) > MAX_SEGMENTS:
+        raise UnsupportedProgram("The index maps are too long for the element-wise executor.")
+    if len(lowering.value_code) > MAX_VALUE_CODE or len(lowering.constants) > MAX_VALUE_CONSTANTS:
+        raise UnsupportedProgram("The expression is too long for the element-wise executor.")
+
+    program = MapProgram()
+    program.num_vars = len(order)
+    program.num_reduced = len(reduced)
+    for old, new in order.items():
+        program.extents[new] = lowering.var_extent[old]
+    program.num_operands = len(lowering.operands)
+    program.output = out_slot
+    for slot, (param, operand) in enumerate(lowering.operands):
+        program.operands[slot].data = data_ptr(param)
+        program.operands[slot].dtype = runtime.DATA_TYPE_INDEX[dtype_tag(param)]
+        program.operands[slot].segment = lowering.segment_slot[(slot, "access", None)]
+        program.operands[slot].other = _other_value(operand.tensor)
+    program.num_segments = len(begins)
+    for index, begin in enumerate(begins):
+        program.segment_begin[index] = begin
+    for index, word in enumerate(code):
+        program.index_code[index] = word
+    for index, value_ in enumerate(constants):
+        program.index_constants[index] = value_
+    program.value_code_length = len(lowering.value_code)
+    program.reduce_split = lowering.reduce_split
+    program.reduce_op = REDUCE[lowering.reduce[0]] if lowering.reduce else 0
+    program.reduce_dtype = runtime.DATA_TYPE_INDEX[lowering.reduce[1]] if lowering.reduce else 0
+    for index, word in enumerate(lowering.value_code):
+        program.value_code[index] = word
+    for index, value_ in enumerate(lowering.constants):
+        program.value_constants[index] = value_
+    description = (
+        f"{len(lowering.operands)} operands, {program.num_vars} index variables {[lowering.var_extent[old] for old in outer + reduced]}, "
+        f"{len(code)} index words, {len(lowering.value_code)} value words"
+        + (f", {lowering.reduce[0]} over {len(reduced)} dimension(s)" if lowering.reduce else "")
+    )
+    return program, description, list(lowering.scalar_slots), [param for param, _ in lowering.operands]
+
+
+def check_application(program):
+    """Raises :class:`UnsupportedProgram` unless every store has the shape the
+    executor handles (sizes are checked later, per call)."""
+
+    for ref, value in program.stores:
+        if not isinstance(ref, TensorRef) or ref.level != 1 or ref.indices or not ref.is_tile:
+            raise UnsupportedProgram("Stores must assign whole tiles directly below the launch grid.")
+        _scan(value)
+
+
+def _scan(value):
+    if isinstance(value, Node):
+        known = (
+            set(_BINARY) | set(_COMPARE) | set(_LOGICAL) | set(_UNARY_SAME) | set(_UNARY_FLOAT) | set(REDUCE)
+            | {"load", "offsets", "pos", "not", "where", "cast", "rand", "kwarg"}
+        )
+        if value.op not in known:
+            raise UnsupportedProgram(f"`{value.op}` is not an element-wise operation this build can execute.")
+        for arg in value.args:
+            _scan(arg)
+    elif isinstance(value, (tuple, list)):
+        for item in value:
+            _scan(item)
+    elif isinstance(value, TensorRef):
+        if value.level != 1 or value.indices or not value.is_tile:
+            raise UnsupportedProgram("Only whole tiles directly below the launch grid can be used by the element-wise executor.")

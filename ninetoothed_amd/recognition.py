@@ -62,10 +62,17 @@ def identify(application, types):
         raise UnsupportedProgram(f"The application could not be traced: {error}") from error
     entry = known_applications().get(program.digest)
     if entry is None:
-        raise UnsupportedProgram(
-            "The application is not one of the programs this build has kernels for "
-            "(matmul, addmm, row softmax, attention forward, conv2d as matmul).  Its dataflow graph:\n" + program.describe()
-        )
+        from ninetoothed_amd import mapping  # imports this module
+
+        try:
+            mapping.check_application(program)
+        except UnsupportedProgram as error:
+            raise UnsupportedProgram(
+                "The application is not one of the programs this build has kernels for "
+                "(matmul, addmm, row softmax, attention forward, conv2d as matmul) and not an element-wise / reducing "
+                f"tile map either ({error}).  Its dataflow graph:\n" + program.describe()
+            ) from error
+        return "map", {}, program
     return entry[0], entry[1], program
 
 

@@ -76,6 +76,8 @@ _SIGNATURES = {
     "launch_nt_conv2d": (_S, _T, _T, _T, _I, _I, _I, _I, _I, _I),
     "launch_nt_gemm_config": (_S, _I, _T, _T, _T, _T, _T, _T, _I, _I),
     "nt_tune_gemm": (_S, _T, _T, _T, _T, _T, _T, _I, _I, _I, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_float)),
+    "launch_nt_map": (_S, ctypes.c_void_p),
+    "nt_map_source": (ctypes.c_void_p, ctypes.c_char_p, _I),
     "nt_gemm_num_configs": (),
     "nt_gemm_config_name": (_I, ctypes.c_char_p, _I),
 }

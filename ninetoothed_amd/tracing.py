@@ -83,6 +83,17 @@ class TensorRef:
         return not isinstance(self.tensor.dtype, Tensor)
 
 
+class _Element:
+    """The level below the grid of an untiled tensor: one element, no dimensions."""
+
+    ndim = 0
+    shape = ()
+    dtype = None
+
+
+_ELEMENT = _Element()
+
+
 class ScalarParam:
     """A zero-dimensional tensor parameter (a call-time scalar)."""
 
@@ -315,9 +326,8 @@ class Tracer:
                 value = ScalarParam(position, bool(tensor.constexpr))
                 kinds.append(("scalar", tensor.constexpr))
             else:
-                if not isinstance(tensor.dtype, Tensor):
-                    raise TracingError(f"Parameter `{name}` is not tiled: it has no level below the launch grid.")
-                value = TensorRef(position, tensor.dtype, 1)
+                # an untiled tensor is a grid of single elements (every program gets a scalar)
+                value = TensorRef(position, tensor.dtype if isinstance(tensor.dtype, Tensor) else _ELEMENT, 1)
                 kinds.append(("tensor", False))
             frame.locals[name] = value
             self.param_values[name] = value

@@ -195,3 +195,70 @@ def conv2d(x, w, padding=(0, 0), bm=64, bn=64, bk=64, dtype="fp16"):
 
     _matmul_programs(x.reshape(-1), w.reshape(-1), lhs, rhs, out, store)
     return y.reshape(n, k, p, q)
+
+
+# ---- tile maps: element-wise / reducing programs ----------------------------------------
+
+
+def tile_map(application, inputs, out_flat, out_view):
+    """Runs a program whose application maps tiles to a tile, the way the
+    reference's generated kernel does (src/ninetoothed/generation.py:638-744):
+    one program per position of the launch grid (the outermost level, equal for
+    all operands); every program gathers its input tiles through the offset
+    tables (masked positions read ``other``), calls ``application(*tiles)``
+    and scatters the result through the output's table (masked positions are
+    skipped).
+
+    ``inputs`` is a list of ``(flat array, View, other)``; a view with a single
+    level is a grid of single elements.  Programs of the reference this
+    restates: tests/test_add.py:9-23, tests/test_clone.py:10-21,
+    tests/test_pad.py:9-15, tests/test_pow.py:10-20, tests/test_dropout.py:12-18,
+    tests/test_max_pool2d.py:13-40, tests/test_generation.py:139-151.
+    """
+
+    grid = out_view.level_shape(0)
+    grid_rank = len(grid)
+    for _, view, _ in inputs:
+        assert tuple(view.level_shape(0)) == tuple(grid), "operands disagree on the launch grid"
+    for program in np.ndindex(*grid):
+        tiles = [gather(flat, view.table[program], other) for flat, view, other in inputs]
+        result = application(*tiles)
+        table = out_view.table[program]
+        values = np.broadcast_to(np.asarray(result).astype(out_flat.dtype), table.shape)
+        scatter(out_flat, np.asarray(table), values)
+    assert grid_rank == len(grid)
+
+
+def philox4x32(counter, key, rounds=10):
+    """Philox-4x32 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3",
+    SC'11): ``counter`` = four uint32 arrays, ``key`` = two.  Pinned by the known
+    answers of the Random123 distribution (tests/test_oracle_programs.py)."""
+    mask = np.uint64(0xFFFFFFFF)
+    c = [np.asarray(word, dtype=np.uint64) & mask for word in counter]
+    k0, k1 = (np.asarray(word, dtype=np.uint64) & mask for word in key)
+    round_a, round_b = np.uint64(0xD2511F53), np.uint64(0xCD9E8D57)
+    for _ in range(rounds):
+        prev0, prev2 = c[0], c[2]
+        c[0] = ((round_b * prev2) >> np.uint64(32)) ^ c[1] ^ k0
+        c[2] = ((round_a * prev0) >> np.uint64(32)) ^ c[3] ^ k1
+        c[1] = (round_b * prev2) & mask
+        c[3] = (round_a * prev0) & mask
+        k0 = (k0 + np.uint64(0x9E3779B9)) & mask
+        k1 = (k1 + np.uint64(0xBB67AE85)) & mask
+    return c
+
+
+def triton_rand(seed, offsets):
+    """``tl.rand(seed, offsets)``: Philox-4x32 with 10 rounds on the counter
+    ``(offset_lo, offset_hi, 0, 0)`` keyed by the two halves of ``seed``; the
+    first output word, read as int32 and mirrored when negative, times 2^-31
+    (the published algorithm of Triton's ``language/random.py``, the package the
+    reference's ``ntl.rand`` resolves to, src/ninetoothed/generation.py:849-855)."""
+    offsets = np.asarray(offsets, dtype=np.int64).astype(np.uint64)
+    seed = np.uint64(seed)
+    mask = np.uint64(0xFFFFFFFF)
+    zeros = np.zeros_like(offsets)
+    words = philox4x32((offsets & mask, offsets >> np.uint64(32), zeros, zeros), (seed & mask, seed >> np.uint64(32)))
+    word = words[0].astype(np.uint32).view(np.int32).astype(np.int64)
+    word = np.where(word < 0, -word - 1, word)
+    return word.astype(np.float32) * np.float32(4.6566127342e-10)

@@ -1,0 +1,415 @@
+"""Element-wise / reducing tile programs (the reference's tests/test_add.py,
+test_clone.py, test_pad.py, test_pow.py, test_dropout.py, test_max_pool2d.py,
+test_generation.py:139-151) through the interpreter kernel.
+
+CPU tests check the lowering (index and value programs) by executing it with
+``oracle.map_machine`` against ``oracle.programs.tile_map``, which restates the
+reference's semantics with offset tables; GPU tests run ``launch_nt_map``
+through ``make`` / ``jit`` and compare with torch at the reference's test
+shapes and with the oracle on small ones.
+"""
+
+import functools
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import ninetoothed_amd as ninetoothed
+import ninetoothed_amd.language as ntl
+from ninetoothed_amd import Symbol, Tensor, block_size, mapping
+from ninetoothed_amd.language import libdevice
+from ninetoothed_amd.make import _dtype_tag
+from ninetoothed_amd.recognition import UnsupportedProgram
+from oracle import programs as oracle
+from oracle.arrangement import View
+from oracle.map_machine import Machine
+
+# ---- the programs, written as in the reference's tests ------------------------------------
+
+BLOCK_SIZE = Symbol("BLOCK_SIZE", meta=True)
+
+
+@ninetoothed.jit
+def add_kernel(
+    lhs: Tensor(1).tile((BLOCK_SIZE,)),
+    rhs: Tensor(1).tile((BLOCK_SIZE,)),
+    output: Tensor(1).tile((BLOCK_SIZE,)),
+):
+    output = lhs + rhs  # noqa: F841
+
+
+def clone_arrangement(input, output):
+    block_shape = (ninetoothed.block_size(), ninetoothed.block_size())
+    return input.tile(block_shape), output.tile(block_shape)
+
+
+def clone_application(input, output):
+    output = input  # noqa: F841
+
+
+def pad_arrangement(input, output, input_slices, output_slices):
+    return input[input_slices], output[output_slices]
+
+
+def pow_arrangement(input, exponent, output, BLOCK_SIZE=block_size()):
+    return input.tile((BLOCK_SIZE,)), exponent.tile((BLOCK_SIZE,)), output.tile((BLOCK_SIZE,))
+
+
+def pow_application(input, exponent, output):
+    output = libdevice.pow(input, exponent)  # noqa: F841
+
+
+def dropout_arrangement(input, p, seed, output, BLOCK_SIZE=block_size()):
+    return input.tile((BLOCK_SIZE,)), p, seed, output.tile((BLOCK_SIZE,))
+
+
+def dropout_application(input, p, seed, output):
+    output = ntl.where(ntl.rand(seed, input.offsets()) > p, input / (1 - p), 0)  # noqa: F841
+
+
+def max_pool2d_arrangement(input, output, ceil_mode=False):
+    BLOCK_SIZE = Symbol("BLOCK_SIZE", meta=True)
+    WINDOW_HEIGHT = Symbol("WINDOW_HEIGHT", constexpr=True, upper_bound=16)
+    WINDOW_WIDTH = Symbol("WINDOW_WIDTH", constexpr=True, upper_bound=16)
+    input_arranged = input.tile((1, 1, WINDOW_HEIGHT, WINDOW_WIDTH), floor_mode=not ceil_mode)
+    input_arranged = input_arranged.ravel()
+    input_arranged = input_arranged.flatten(end_dim=4).flatten(start_dim=1)
+    input_arranged = input_arranged.tile((BLOCK_SIZE, -1))
+    output_arranged = output.tile((1, 1, 1, 1))
+    output_arranged = output_arranged.ravel()
+    output_arranged = output_arranged.flatten(end_dim=4).flatten(start_dim=1)
+    output_arranged = output_arranged.tile((BLOCK_SIZE, -1))
+    output_arranged.dtype = output_arranged.dtype.squeeze(1)
+    return input_arranged, output_arranged
+
+
+def max_pool2d_application(input, output):
+    output = ntl.max(input, axis=1)  # noqa: F841
+
+
+def scalar_add_arrangement(input, other, output, block_size=ninetoothed.block_size()):
+    return input.tile((block_size,)), other, output.tile((block_size,))
+
+
+def scalar_add_application(input, other, output):
+    output = input + other  # noqa: F841
+
+
+def fused_arrangement(x, y, scale, output):
+    block_shape = (ninetoothed.block_size(), ninetoothed.block_size())
+    return x.tile(block_shape), y.tile(block_shape), scale, output.tile(block_shape)
+
+
+def fused_application(x, y, scale, output):
+    output = ntl.where(x > y, ntl.exp(x - y) * scale, ntl.maximum(x, 0.5) / y)  # noqa: F841
+
+
+def row_sum_arrangement(input, output):
+    return input.tile((1, -1)).squeeze(1), output.tile((1,))
+
+
+def row_sum_application(input, output):
+    output = ntl.sum(input) * 2  # noqa: F841
+
+
+def _pad_config(shape, pad):
+    """tests/test_pad.py:67-95 of the reference, restated."""
+    ndim = len(shape)
+    output_shape, input_slices, output_slices = list(shape), [], []
+    for i in range(ndim):
+        left, right = pad[2 * (ndim - 1 - i)], pad[2 * (ndim - 1 - i) + 1]
+        output_shape[i] += left + right
+        input_slices.append(slice(max(0, -left), min(shape[i], shape[i] + right)))
+        output_slices.append(slice(max(0, left), output_shape[i] - max(0, right)))
+    return output_shape, tuple(input_slices), tuple(output_slices)
+
+
+# ---- CPU: lowering executed by the numpy machine ------------------------------------------
+
+
+def _run_on_machine(kernel, args, kwargs=None):
+    kwargs = kwargs or {}
+    env = kernel._environment(args, kwargs, check_device=False)
+    flat = {}
+
+    def storage(p):
+        if p not in flat:
+            tensor = args[p]
+            size = 1 + sum((n - 1) * abs(s) for n, s in zip(tensor.shape, tensor.stride())) if tensor.numel() else 0
+            flat[p] = torch.as_strided(tensor, (size,), (1,)).numpy()
+        return flat[p]
+
+    for store in kernel.program.stores:
+        built = mapping.build(store, kernel.types, args, env, lambda p: _dtype_tag(args[p].dtype), lambda p: 0)
+        if built is None:
+            continue
+        program, _, _, operand_params = built
+        Machine(program, {slot: storage(p) for slot, p in enumerate(operand_params)}).run()
+
+
+def test_lowering_add():
+    lhs, rhs = torch.rand(1000), torch.rand(1000)
+    out = torch.empty(1000)
+    assert add_kernel.kind == "map"
+    _run_on_machine(add_kernel, (lhs, rhs, out))
+    assert torch.equal(out, lhs + rhs)
+
+
+def test_lowering_clone_strided_against_oracle():
+    kernel = ninetoothed.make(clone_arrangement, clone_application, (Tensor(2), Tensor(2)))
+    source = torch.randn(37 * 50)
+    input = torch.as_strided(source, (37, 23), (50, 2))
+    out = torch.zeros(37, 23)
+    _run_on_machine(kernel, (input, out))
+    # the oracle works on offset tables of the strided source
+    table = (np.arange(37)[:, None] * 50 + np.arange(23)[None, :] * 2).astype(np.intp)
+    expected = np.zeros(37 * 23, dtype=np.float32)
+    oracle.tile_map(lambda tile: tile, [(source.numpy(), View(table, [2]).tile((8, 16)), None)], expected, View.of_shape((37, 23)).tile((8, 16)))
+    assert np.array_equal(out.numpy().reshape(-1), expected)
+    assert torch.equal(out, input)
+
+
+@pytest.mark.parametrize("shape, pad_", (((20, 13), (-3, 2, 4, -1)), ((2, 3), (1, 1, 1, 2)), ((2, 3, 4), (1, 3, 1, 0, 0, 0)), ((2, 3), (-1, -1, 0, 0))))
+def test_lowering_pad(shape, pad_):
+    input = torch.randn(shape)
+    output_shape, input_slices, output_slices = _pad_config(shape, pad_)
+    out = torch.full(output_shape, 7.0)
+    kernel = ninetoothed.make(pad_arrangement, clone_application, (Tensor(len(shape)), Tensor(len(shape)), input_slices, output_slices))
+    _run_on_machine(kernel, (input, out))
+    assert torch.equal(out, F.pad(input, pad_, "constant", 7.0))
+
+
+@pytest.mark.parametrize("ceil_mode", (False, True))
+def test_lowering_max_pool2d_against_oracle(ceil_mode):
+    kernel = ninetoothed.make(
+        functools.partial(max_pool2d_arrangement, ceil_mode=ceil_mode), max_pool2d_application, (Tensor(4, other=float("-inf")), Tensor(4))
+    )
+    x = torch.randn(2, 3, 8, 7).half()
+    expected = F.max_pool2d(x.float(), (3, 3), ceil_mode=ceil_mode).half()
+    out = torch.zeros_like(expected)
+    _run_on_machine(kernel, (x, out), dict(WINDOW_HEIGHT=3, WINDOW_WIDTH=3))
+    assert torch.equal(out, expected)
+    # the same arrangement on offset tables
+    view_in = View.of_shape(x.shape).tile((1, 1, 3, 3), floor_mode=not ceil_mode).ravel().flatten(end_dim=4).flatten(start_dim=1).tile((4, -1))
+    view_out = View.of_shape(expected.shape).tile((1, 1, 1, 1)).ravel().flatten(end_dim=4).flatten(start_dim=1).tile((4, -1)).squeeze(1, level=1)
+    result = np.zeros(expected.numel(), dtype=np.float16)
+    oracle.tile_map(lambda tile: tile.max(axis=1), [(x.numpy().reshape(-1), view_in, -np.inf)], result, view_out)
+    assert np.array_equal(result, out.numpy().reshape(-1))
+
+
+def test_lowering_dropout_matches_published_philox():
+    kernel = ninetoothed.make(dropout_arrangement, dropout_application, (Tensor(1), Tensor(0), Tensor(0), Tensor(1)))
+    x = torch.randn(349).half()
+    out = torch.empty_like(x)
+    p, seed = 0.3, 123456789
+    _run_on_machine(kernel, (x, p, seed, out))
+    keep = oracle.triton_rand(seed, np.arange(349)) > np.float32(p)
+    scaled = (x.float().numpy() / np.float32(1 - p)).astype(np.float16)
+    assert np.array_equal(out.numpy(), np.where(keep, scaled, np.float16(0)))
+    assert abs(keep.mean() - 0.7) < 0.05
+
+
+def test_philox_known_answers():
+    # Random123's kat_vectors for philox4x32-10
+    f = 0xFFFFFFFF
+    assert [int(w) for w in oracle.philox4x32((0, 0, 0, 0), (0, 0))] == [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]
+    assert [int(w) for w in oracle.philox4x32((f, f, f, f), (f, f))] == [0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD]
+    assert [int(w) for w in oracle.philox4x32((0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344), (0xA4093822, 0x299F31D0))] == [
+        0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1,
+    ]
+
+
+def test_lowering_types_follow_the_reference_promotion():
+    kernel = ninetoothed.make(fused_arrangement, fused_application, (Tensor(2), Tensor(2), Tensor(0), Tensor(2)))
+    x, y = torch.randn(9, 11).half(), (torch.rand(9, 11) + 0.5).half()
+    out = torch.empty(9, 11).half()
+    _run_on_machine(kernel, (x, y, 1.5, out))
+    xf, yf = x.float(), y.float()
+    first = (torch.exp((x - y).float()).half().float() * 1.5)  # fp16 tile times run-time float: fp32
+    second = (torch.maximum(x, torch.tensor(0.5).half()).float() / yf).half().float()  # stays fp16
+    expected = torch.where(xf > yf, first, second).half()
+    assert torch.allclose(out.float(), expected.float(), rtol=2e-3, atol=2e-3)
+
+
+def test_lowering_full_reduction_and_post_operation():
+    kernel = ninetoothed.make(row_sum_arrangement, row_sum_application, (Tensor(2), Tensor(1)))
+    x = torch.randn(5, 33)
+    out = torch.empty(5)
+    _run_on_machine(kernel, (x, out))
+    assert torch.allclose(out, x.sum(dim=1) * 2, rtol=1e-5, atol=1e-5)
+
+
+def test_scalar_constexpr_and_empty_programs():
+    kernel = ninetoothed.make(scalar_add_arrangement, scalar_add_application, (Tensor(1), Tensor(0, constexpr=True), Tensor(1)))
+    x = torch.randn(1086)
+    out = torch.empty_like(x)
+    _run_on_machine(kernel, (x, math.pi, out))
+    assert torch.equal(out, x + math.pi)
+
+
+def test_programs_outside_the_class_are_reported():
+    def arrangement(input, output):
+        return input.tile((1, -1)), output.tile((1, -1))
+
+    def application(input, output):
+        output = ntl.dot(input, ntl.trans(input))  # noqa: F841
+
+    with pytest.raises(UnsupportedProgram):
+        ninetoothed.make(arrangement, application, (Tensor(2), Tensor(2)))
+
+
+# ---- GPU: the interpreter kernel through make / jit -------------------------------------------
+
+gpu = pytest.mark.gpu
+
+
+def _served_by_map(kernel):
+    assert kernel.last_plan.startswith("launch_nt_map"), kernel.last_plan
+
+
+@gpu
+def test_add():
+    lhs, rhs = torch.rand(98432, device="cuda"), torch.rand(98432, device="cuda")
+    out = torch.empty_like(lhs)
+    add_kernel(lhs, rhs, out)
+    _served_by_map(add_kernel)
+    assert torch.equal(out, lhs + rhs)
+
+
+@gpu
+def test_clone_strided():
+    input = torch.empty_strided((641, 280), (700, 300), device="cuda")
+    input.copy_(torch.randn(641, 280, device="cuda"))
+    out = torch.empty_like(input)
+    kernel = ninetoothed.make(clone_arrangement, clone_application, (Tensor(2), Tensor(2)))
+    kernel(input, out)
+    _served_by_map(kernel)
+    assert out.shape == input.shape and torch.equal(out, input)
+
+
+@gpu
+@pytest.mark.parametrize("dtype", (torch.float32, torch.float16))
+@pytest.mark.parametrize("value", (0, 1, -1, float("-inf"), math.pi))
+@pytest.mark.parametrize("shape, pad_", (((2026, 1207), (-100, 20, 99, -10)), ((2, 3), (1, 1, 1, 2)), ((2, 3, 4), (1, 3, 1, 0, 0, 0)), ((2, 3), (-1, -1, 0, 0))))
+def test_pad(shape, pad_, value, dtype):
+    input = torch.randn(shape, dtype=dtype, device="cuda")
+    output_shape, input_slices, output_slices = _pad_config(shape, pad_)
+    out = torch.full(output_shape, value, dtype=dtype, device="cuda")
+    kernel = ninetoothed.make(pad_arrangement, clone_application, (Tensor(len(shape)), Tensor(len(shape)), input_slices, output_slices))
+    kernel(input, out)
+    _served_by_map(kernel)
+    assert torch.equal(out, F.pad(input, pad_, "constant", value))
+
+
+@gpu
+def test_pow():
+    input, exponent = torch.rand(44925, device="cuda"), torch.rand(44925, device="cuda")
+    out = torch.empty_like(input)
+    kernel = ninetoothed.make(pow_arrangement, pow_application, (Tensor(1), Tensor(1), Tensor(1)))
+    kernel(input, exponent, out)
+    _served_by_map(kernel)
+    assert torch.allclose(out, torch.pow(input, exponent), equal_nan=True)
+
+
+@gpu
+def test_dropout():
+    x = torch.randn(349, dtype=torch.float16, device="cuda")
+    out = torch.empty_like(x)
+    kernel = ninetoothed.make(dropout_arrangement, dropout_application, (Tensor(1), Tensor(0), Tensor(0), Tensor(1)))
+    p = 0.3
+    for seed in (7, 2**31 - 5):  # a second call with another seed reuses the plan
+        kernel(x, p, seed, out)
+        _served_by_map(kernel)
+        keep = oracle.triton_rand(seed, np.arange(349)) > np.float32(p)
+        scaled = (x.float().cpu().numpy() / np.float32(1 - p)).astype(np.float16)
+        assert np.array_equal(out.cpu().numpy(), np.where(keep, scaled, np.float16(0)))
+    non_zero_ratio = out.nonzero().numel() / x.numel()
+    assert abs(non_zero_ratio - (1 - p)) < 0.05
+    assert torch.allclose(out[out != 0], (x[out != 0] / (1 - p)))
+
+
+@gpu
+@pytest.mark.parametrize("ceil_mode", (False, True))
+def test_max_pool2d(ceil_mode):
+    x = torch.randn(32, 3, 64, 64, dtype=torch.float16, device="cuda")
+    expected = F.max_pool2d(x, (3, 3), ceil_mode=ceil_mode)
+    out = torch.empty_like(expected)
+    kernel = ninetoothed.make(
+        functools.partial(max_pool2d_arrangement, ceil_mode=ceil_mode), max_pool2d_application, (Tensor(4, other=float("-inf")), Tensor(4))
+    )
+    kernel(x, out, WINDOW_HEIGHT=3, WINDOW_WIDTH=3)
+    _served_by_map(kernel)
+    assert torch.equal(out, expected)
+
+
+@gpu
+def test_non_int_constexpr():
+    x = torch.randn(1086, device="cuda")
+    out = torch.empty_like(x)
+    kernel = ninetoothed.make(scalar_add_arrangement, scalar_add_application, (Tensor(1), Tensor(0, constexpr=True), Tensor(1)))
+    kernel(x, math.pi, out)
+    _served_by_map(kernel)
+    assert torch.allclose(out, x + math.pi)
+
+
+@gpu
+def test_fused_expression_against_machine():
+    kernel = ninetoothed.make(fused_arrangement, fused_application, (Tensor(2), Tensor(2), Tensor(0), Tensor(2)))
+    x, y = torch.randn(130, 70).half(), (torch.rand(130, 70) + 0.5).half()
+    expected = torch.empty(130, 70).half()
+    _run_on_machine(kernel, (x, y, 1.5, expected))
+    out = torch.empty(130, 70, dtype=torch.float16, device="cuda")
+    kernel(x.cuda(), y.cuda(), 1.5, out)
+    _served_by_map(kernel)
+    assert torch.allclose(out.cpu().float(), expected.float(), rtol=2e-3, atol=2e-3)
+
+
+@gpu
+@pytest.mark.parametrize("interpret", ("0", "1"))
+def test_interpreter_and_specialised_kernels_agree(interpret, monkeypatch):
+    # NT_MAP_INTERPRET=1 keeps launch_nt_map on the interpreter kernel (the path taken when
+    # hipRTC is missing); both must produce the machine's result
+    monkeypatch.setenv("NT_MAP_INTERPRET", interpret)
+    kernel = ninetoothed.make(dropout_arrangement, dropout_application, (Tensor(1), Tensor(0), Tensor(0), Tensor(1)))
+    x = torch.randn(5000).half()
+    expected = torch.empty_like(x)
+    _run_on_machine(kernel, (x, 0.25, 99, expected))
+    out = torch.empty(5000, dtype=torch.float16, device="cuda")
+    kernel(x.cuda(), 0.25, 99, out)
+    assert torch.equal(out.cpu(), expected)
+    pool = ninetoothed.make(
+        functools.partial(max_pool2d_arrangement, ceil_mode=True), max_pool2d_application, (Tensor(4, other=float("-inf")), Tensor(4))
+    )
+    image = torch.randn(3, 5, 17, 19, dtype=torch.float16, device="cuda")
+    pooled = torch.empty(3, 5, 6, 7, dtype=torch.float16, device="cuda")
+    pool(image, pooled, WINDOW_HEIGHT=3, WINDOW_WIDTH=3)
+    assert torch.equal(pooled, F.max_pool2d(image, (3, 3), ceil_mode=True))
+    if interpret == "0":
+        assert "nt_map_specialised" in open(pool._source).read()
+
+
+@gpu
+def test_row_sum():
+    kernel = ninetoothed.make(row_sum_arrangement, row_sum_application, (Tensor(2), Tensor(1)))
+    x = torch.randn(300, 257, device="cuda")
+    out = torch.empty(300, device="cuda")
+    kernel(x, out)
+    _served_by_map(kernel)
+    assert torch.allclose(out, x.sum(dim=1) * 2, rtol=1e-4, atol=1e-4)
+
+
+@gpu
+def test_empty_tensor_and_no_store():
+    def arrangement(x):
+        return x.tile((ninetoothed.block_size(),)).unsqueeze(0)
+
+    def application(x):
+        x
+
+    kernel = ninetoothed.make(arrangement, application, (Tensor(1),))
+    kernel(torch.randn((0,), device="cuda"))
+    out = torch.empty(0, device="cuda")
+    add_kernel(torch.empty(0, device="cuda"), torch.empty(0, device="cuda"), out)
