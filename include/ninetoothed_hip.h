@@ -192,6 +192,18 @@ NineToothedResult nt_tune_gemm(NineToothedStream stream,
                                int dtype, int output_dtype, int iters,
                                int *best_config, float *best_ms);
 
+/* Persistence of the tuned choices in the line-pair CSV format of the
+ * reference's AutoTuningCache (src/ninetoothed/templates/auto_tuning_cache.h:27-75,
+ * writer src/ninetoothed/build.py:683-703): a line of integers for the problem
+ * (dtype, output dtype, M, N, K, addmm), then a line for the choice (block M,
+ * block N, block K, instance index); the first pair has an empty problem line
+ * and holds the default.  Both act on the cache of the current device. */
+NineToothedResult nt_tune_cache_save(const char *path);
+NineToothedResult nt_tune_cache_load(const char *path, int *entries);
+
+/* The cached instance for a problem, or -1. */
+int nt_tune_cache_lookup(int dtype, int output_dtype, int m, int n, int k, int addmm);
+
 /*
  * Element-wise / reducing tile programs that are none of the programs above.
  *

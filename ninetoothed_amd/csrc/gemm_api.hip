@@ -5,6 +5,7 @@
 #include <unordered_map>
 #include <vector>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include "conv2d.h"
@@ -357,6 +358,89 @@ NineToothedResult nt_tune_gemm(NineToothedStream stream_, NineToothedTensor inpu
     if (best_config) *best_config = best;
     if (best_ms) *best_ms = best_time;
     return 0;
+}
+
+// On-disk form of the tuned choices: the line-pair CSV the reference's AutoTuningCache reads
+// (src/ninetoothed/templates/auto_tuning_cache.h:27-75; written by src/ninetoothed/build.py:683-703):
+// a line of integers describing the problem, then a line of integers with the choice; the first
+// pair has an empty problem line and carries the default.  Problem = dtype, output dtype, M, N, K,
+// addmm flag; choice = block M, block N, block K, instance index.
+NineToothedResult nt_tune_cache_save(const char *path) {
+    if (path == nullptr) return hipErrorInvalidValue;
+    int device = 0;
+    (void)hipGetDevice(&device);
+    FILE *file = fopen(path, "w");
+    if (file == nullptr) return hipErrorInvalidValue;
+    const GemmInstance &fallback = kInstances[1];
+    fprintf(file, "\n%d,%d,%d,%d\n", fallback.bm, fallback.bn, fallback.bk, 1);
+    {
+        std::shared_lock<std::shared_mutex> lock(g_tune_mutex);
+        for (const auto &entry : g_tuned) {
+            const TuneKey &key = entry.first;
+            if (key.device != device || entry.second < 0 || entry.second >= kNumInstances) continue;
+            const GemmInstance &instance = kInstances[entry.second];
+            fprintf(file, "%d,%d,%d,%d,%d,%d\n%d,%d,%d,%d\n", key.dtype, key.out_dtype, key.m, key.n, key.k, key.addmm, instance.bm,
+                    instance.bn, instance.bk, entry.second);
+        }
+    }
+    return fclose(file) == 0 ? 0 : (int)hipErrorInvalidValue;
+}
+
+// Reads such a file into the cache of the current device.  *entries (may be NULL) receives the
+// number of choices taken over; lines that do not parse, or name an instance this build does not
+// have, are skipped.
+NineToothedResult nt_tune_cache_load(const char *path, int *entries) {
+    if (entries) *entries = 0;
+    if (path == nullptr) return hipErrorInvalidValue;
+    FILE *file = fopen(path, "r");
+    if (file == nullptr) return hipErrorInvalidValue;
+    int device = 0;
+    (void)hipGetDevice(&device);
+    auto parse = [](const char *line, std::vector<long> &values) {
+        values.clear();
+        const char *cursor = line;
+        while (*cursor) {
+            while (*cursor == ' ' || *cursor == '\t' || *cursor == '\r' || *cursor == '\n' || *cursor == ',') ++cursor;
+            if (!*cursor) break;
+            char *end = nullptr;
+            const long value = strtol(cursor, &end, 10);
+            if (end == cursor) return false;
+            values.push_back(value);
+            cursor = end;
+        }
+        return true;
+    };
+    char problem_line[512], choice_line[512];
+    std::vector<long> problem, choice;
+    bool first = true;
+    int taken = 0;
+    while (fgets(problem_line, sizeof(problem_line), file) && fgets(choice_line, sizeof(choice_line), file)) {
+        const bool parsed = parse(problem_line, problem) && parse(choice_line, choice);
+        if (first) {  // the default pair
+            first = false;
+            continue;
+        }
+        if (!parsed || problem.size() != 6 || choice.size() != 4) continue;
+        const int instance = (int)choice[3];
+        if (instance < 0 || instance >= kNumInstances) continue;
+        if (kInstances[instance].bm != choice[0] || kInstances[instance].bn != choice[1] || kInstances[instance].bk != choice[2]) continue;
+        TuneKey key{device, (int)problem[0], (int)problem[1], (int)problem[2], (int)problem[3], (int)problem[4], (int)problem[5]};
+        std::unique_lock<std::shared_mutex> lock(g_tune_mutex);
+        g_tuned[key] = instance;
+        ++taken;
+    }
+    fclose(file);
+    if (entries) *entries = taken;
+    return 0;
+}
+
+// The cached choice for a problem given by its sizes (no tensors needed): instance index, or -1.
+int nt_tune_cache_lookup(int dtype, int output_dtype, int m, int n, int k, int addmm) {
+    int device = 0;
+    (void)hipGetDevice(&device);
+    std::shared_lock<std::shared_mutex> lock(g_tune_mutex);
+    auto it = g_tuned.find(TuneKey{device, dtype, output_dtype, m, n, k, addmm ? 1 : 0});
+    return it == g_tuned.end() ? -1 : it->second;
 }
 
 NineToothedResult launch_nt_conv2d(NineToothedStream stream, NineToothedTensor input, NineToothedTensor filter,

@@ -252,6 +252,24 @@ class Kernel:
         a_arg = runtime.ArgumentTensor.from_layout(0, (m, k), (a.row_stride, a.col_stride))
         b_arg = runtime.ArgumentTensor.from_layout(0, (k, n), (b.row_stride, b.col_stride))
         c_arg = runtime.ArgumentTensor.from_layout(0, (m, n), (c.row_stride, c.col_stride))
+        # block sizes left to the tuner (all meta): like the reference's autotuned kernels, the
+        # first launch of a new problem times the candidates once (src/ninetoothed/generation.py:372-516)
+        from ninetoothed_amd import auto_tuner
+
+        state = {"tune": blocks == [0, 0, 0] and min(m, n, k) > 0 and auto_tuner.enabled()}
+        if state["tune"]:
+            auto_tuner.load_once()
+            state["tune"] = auto_tuner.lookup(dtype, out_dtype, m, n, k, i is not None) < 0
+
+        def maybe_tune(call_args, input_arg, beta, alpha):
+            state["tune"] = False
+            out = call_args[c_pos]
+            sources = [call_args[p] for p in (in_pos, a_pos, b_pos) if p is not None]
+            # timing launches rewrite the output; skip when it overlaps an operand
+            if any(t.untyped_storage().data_ptr() == out.untyped_storage().data_ptr() for t in sources):
+                return
+            auto_tuner.tune(input_arg, a_arg, b_arg, beta, alpha, c_arg, dtype, out_dtype)
+
         if i is not None:
             i_arg = runtime.ArgumentTensor.from_layout(0, (m, n), (i.row_stride, i.col_stride))
 
@@ -262,6 +280,8 @@ class Kernel:
                 i_arg.data = call_args[in_pos].data_ptr() + i.base * itemsize
                 beta = runtime.ArgumentTensor.from_scalar(float(call_args[beta_pos]))
                 alpha = runtime.ArgumentTensor.from_scalar(float(call_args[alpha_pos]))
+                if state["tune"]:
+                    maybe_tune(call_args, i_arg, beta, alpha)
                 runtime.check(lib.launch_nt_addmm(runtime.current_stream(), i_arg, a_arg, b_arg, beta, alpha, c_arg, dtype, *blocks))
 
             return _Plan(f"launch_nt_addmm {m}x{n}x{k} {tag} blocks {blocks}", launch)
@@ -270,6 +290,9 @@ class Kernel:
             a_arg.data = call_args[a_pos].data_ptr() + a.base * itemsize
             b_arg.data = call_args[b_pos].data_ptr() + b.base * itemsize
             c_arg.data = call_args[c_pos].data_ptr() + c.base * out_itemsize
+            if state["tune"]:
+                null = runtime.ArgumentTensor.null()
+                maybe_tune(call_args, null, null, null)
             runtime.check(lib.launch_nt_matmul(runtime.current_stream(), a_arg, b_arg, c_arg, dtype, out_dtype, *blocks))
 
         return _Plan(f"launch_nt_matmul {m}x{n}x{k} {tag}->{out_tag} blocks {blocks}", launch)

@@ -78,6 +78,9 @@ _SIGNATURES = {
     "nt_tune_gemm": (_S, _T, _T, _T, _T, _T, _T, _I, _I, _I, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_float)),
     "launch_nt_map": (_S, ctypes.c_void_p),
     "nt_map_source": (ctypes.c_void_p, ctypes.c_char_p, _I),
+    "nt_tune_cache_save": (ctypes.c_char_p,),
+    "nt_tune_cache_load": (ctypes.c_char_p, ctypes.POINTER(ctypes.c_int)),
+    "nt_tune_cache_lookup": (_I, _I, _I, _I, _I, _I),
     "nt_gemm_num_configs": (),
     "nt_gemm_config_name": (_I, ctypes.c_char_p, _I),
 }

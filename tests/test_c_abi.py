@@ -72,3 +72,39 @@ def test_requests_without_a_kernel_are_refused_on_the_host():
     assert library.launch_nt_matmul(None, a, mismatched, a, runtime.DATA_TYPE_INDEX["fp16"], runtime.DATA_TYPE_INDEX["fp16"], 0, 0, 0) != 0  # hipErrorInvalidValue
     empty = runtime.ArgumentTensor.from_layout(0, (0, 4), (4, 1))
     assert library.launch_nt_softmax(None, empty, empty, runtime.DATA_TYPE_INDEX["fp32"], 0) == 0
+
+
+def test_tuning_cache_reads_and_writes_the_reference_csv_format(tmp_path):
+    # the file layout of src/ninetoothed/build.py:683-703 (csv.writer rows: an empty row and the
+    # default first, then problem / choice pairs), read by templates/auto_tuning_cache.h:27-75
+    import csv
+    import ctypes
+
+    from ninetoothed_amd import runtime
+
+    lib = runtime.library()
+    names = runtime.gemm_config_names()
+    fast = next(index for index, name in enumerate(names) if name.startswith("256x256x32"))
+    fp16 = runtime.DATA_TYPE_INDEX["fp16"]
+    path = tmp_path / "cache.csv"
+    with open(path, "w") as handle:
+        writer = csv.writer(handle)
+        writer.writerow(())
+        writer.writerow((256, 256, 32, fast))
+        writer.writerow((fp16, fp16, 4096, 2048, 1024, 1))
+        writer.writerow((256, 256, 32, fast))
+        writer.writerow((fp16, fp16, 64, 64, 64, 0))
+        writer.writerow((7, 7, 7, 999))  # an instance this build does not have: skipped
+    entries = ctypes.c_int(-1)
+    assert lib.nt_tune_cache_load(str(path).encode(), ctypes.byref(entries)) == 0
+    assert entries.value == 1
+    assert lib.nt_tune_cache_lookup(fp16, fp16, 4096, 2048, 1024, 1) == fast
+    assert lib.nt_tune_cache_lookup(fp16, fp16, 64, 64, 64, 0) == -1
+    assert lib.nt_tune_cache_lookup(fp16, fp16, 4096, 2048, 1024, 0) == -1
+
+    saved = tmp_path / "saved.csv"
+    assert lib.nt_tune_cache_save(str(saved).encode()) == 0
+    rows = list(csv.reader(open(saved)))
+    assert rows[0] == [] and len(rows[1]) == 4  # the default pair
+    assert [str(v) for v in (fp16, fp16, 4096, 2048, 1024, 1)] in rows
+    assert lib.nt_tune_cache_load(str(tmp_path / "missing.csv").encode(), None) != 0

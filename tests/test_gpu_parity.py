@@ -344,3 +344,40 @@ def test_conv2d_baseline_shape_and_1x1():
     out = _conv2d(x[:1], w1, (0, 0))
     as_matmul = (x[:1].permute(0, 2, 3, 1).reshape(-1, 256).float() @ w1.reshape(64, 256).t().float()).reshape(1, 56, 56, 64).permute(0, 3, 1, 2)
     assert torch.allclose(out.float(), as_matmul, **HALF_TOL)
+
+
+# ---- tile selection -------------------------------------------------------------
+
+
+def test_first_launch_tunes_and_the_choice_persists(tmp_path, monkeypatch):
+    import ctypes
+
+    from ninetoothed_amd import auto_tuner, runtime
+
+    monkeypatch.setattr(auto_tuner, "CACHE_DIR", tmp_path)
+    lib = runtime.library()
+    fp16 = runtime.DATA_TYPE_INDEX["fp16"]
+    m, n, k = 768, 1280, 512  # a problem no other test uses
+    assert lib.nt_tune_cache_lookup(fp16, fp16, m, n, k, 0) == -1
+    a, b = _randn(m, k).cuda(), _randn(k, n).cuda()
+    out = torch.full((m, n), float("nan"), dtype=torch.float16, device="cuda")
+    kernel = ninetoothed.make(programs.matmul.arrangement, programs.matmul.application_with_cast, programs.matmul.tensors())
+    kernel(a, b, out)
+    assert torch.allclose(out, torch.matmul(a, b), **HALF_TOL)
+    choice = lib.nt_tune_cache_lookup(fp16, fp16, m, n, k, 0)
+    assert 0 <= choice < lib.nt_gemm_num_configs()
+    files = list(tmp_path.glob("gemm_*.csv"))
+    assert len(files) == 1
+    entries = ctypes.c_int(0)
+    assert lib.nt_tune_cache_load(str(files[0]).encode(), ctypes.byref(entries)) == 0 and entries.value >= 1
+    # every instance that accepts the problem gives the same answer as the tuned launch
+    null = runtime.ArgumentTensor.null()
+    for config in range(lib.nt_gemm_num_configs()):
+        other = torch.full_like(out, float("nan"))
+        code = lib.launch_nt_gemm_config(
+            runtime.current_stream(), config, null, runtime.ArgumentTensor.from_torch_tensor(a), runtime.ArgumentTensor.from_torch_tensor(b),
+            null, null, runtime.ArgumentTensor.from_torch_tensor(other), fp16, fp16,
+        )
+        assert code in (0, runtime.NO_KERNEL)
+        if code == 0:
+            assert torch.allclose(other, out, **HALF_TOL)
