@@ -49,7 +49,11 @@ enum NineToothedDataType {
     NINETOOTHED_FLOAT16,
     NINETOOTHED_BFLOAT16,
     NINETOOTHED_FLOAT32,
-    NINETOOTHED_FLOAT64
+    NINETOOTHED_FLOAT64,
+    /* extension beyond the reference's enum: 8-bit floating point with 5 exponent
+     * and 2 mantissa bits, the operand type of the second case of
+     * tests/test_matmul.py:61-88; accepted by launch_nt_matmul only */
+    NINETOOTHED_FLOAT8_E5M2
 };
 
 typedef struct {
@@ -73,7 +77,10 @@ typedef int NineToothedResult;
  * Replaces the kernel generated for tests/test_matmul.py:14-45 (== README.md:40-62):
  * generated launch function src/ninetoothed/generation.py:545-600.
  * `dtype` is the element type of lhs/rhs; `output_dtype` that of output
- * (FLOAT16, BFLOAT16 or FLOAT32).  Any strides are accepted. */
+ * (FLOAT16, BFLOAT16 or FLOAT32).  Any strides are accepted.
+ * FLOAT8_E5M2 operands (output FLOAT16 or FLOAT32) are widened to fp16 on the
+ * way into LDS -- exact, the format is the upper byte of fp16 -- and multiplied
+ * on the fp16 MFMA path with fp32 accumulation. */
 NineToothedResult launch_nt_matmul(NineToothedStream stream,
                                    NineToothedTensor lhs,
                                    NineToothedTensor rhs,

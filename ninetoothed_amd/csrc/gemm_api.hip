@@ -95,6 +95,8 @@ hipError_t fast_launch(const GemmProblem &q, hipStream_t stream) {
 }
 
 bool generic_accepts(const GemmProblem &q) {
+    if (q.dtype == NINETOOTHED_FLOAT8_E5M2)  // matmul only, widened to fp16
+        return !q.addmm() && (q.out_dtype == NINETOOTHED_FLOAT16 || q.out_dtype == NINETOOTHED_FLOAT32) && q.m >= 0 && q.n >= 0 && q.k >= 0;
     if (q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) return false;
     if (q.out_dtype != q.dtype && q.out_dtype != NINETOOTHED_FLOAT32) return false;
     return q.m >= 0 && q.n >= 0 && q.k >= 0;
@@ -126,8 +128,30 @@ hipError_t generic_launch_typed(const GemmProblem &q, hipStream_t stream) {
     return hipGetLastError();
 }
 
+template <typename TOut>
+hipError_t fp8_launch_typed(const GemmProblem &q, hipStream_t stream) {
+    Fp8E5m2Problem<TOut> prob;
+    prob.m = q.m;
+    prob.n = q.n;
+    prob.k = q.k;
+    prob.a = (const uint8_t *)q.a;
+    prob.b = (const uint8_t *)q.b;
+    prob.c = (TOut *)q.c;
+    prob.sam = q.sam;
+    prob.sak = q.sak;
+    prob.sbk = q.sbk;
+    prob.sbn = q.sbn;
+    prob.scm = q.scm;
+    prob.scn = q.scn;
+    const int64_t tiles = (int64_t)ceil_div(q.m, kGenBM) * ceil_div(q.n, kGenBN);
+    if (tiles == 0) return hipSuccess;
+    gemm_generic_kernel<Fp8E5m2Problem<TOut>><<<dim3((unsigned)tiles), dim3(kGenThreads), 0, stream>>>(prob);
+    return hipGetLastError();
+}
+
 hipError_t generic_launch(const GemmProblem &q, hipStream_t stream) {
     const bool f32out = q.out_dtype == NINETOOTHED_FLOAT32;
+    if (q.dtype == NINETOOTHED_FLOAT8_E5M2) return f32out ? fp8_launch_typed<float>(q, stream) : fp8_launch_typed<half_t>(q, stream);
     if (q.dtype == NINETOOTHED_FLOAT16)
         return f32out ? generic_launch_typed<half_t, float>(q, stream) : generic_launch_typed<half_t, half_t>(q, stream);
     return f32out ? generic_launch_typed<bf16_t, float>(q, stream) : generic_launch_typed<bf16_t, bf16_t>(q, stream);

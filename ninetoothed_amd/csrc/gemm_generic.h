@@ -176,6 +176,38 @@ struct StridedProblem {
     }
 };
 
+// ---- policy: fp8 (e5m2) operands, any strides ----
+// An e5m2 value is the upper byte of the fp16 value with the same sign and
+// exponent, so widening is a shift and the fp16 MFMA multiplies exactly.
+template <typename TOut>
+struct Fp8E5m2Problem {
+    typedef half_t elem;
+    int m, n, k;
+    const uint8_t *a;
+    const uint8_t *b;
+    TOut *c;
+    int64_t sam, sak, sbk, sbn, scm, scn;
+
+    static NT_DEVICE half_t widen(uint8_t byte) {
+        const unsigned short bits = (unsigned short)((unsigned short)byte << 8);
+        return __builtin_bit_cast(half_t, bits);
+    }
+
+    NT_DEVICE void load_a16(int row, int k0, half_t out[16]) const {
+        const uint8_t *src = a + (int64_t)row * sam + (int64_t)k0 * sak;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) out[i] = (row < m && k0 + i < k) ? widen(src[(int64_t)i * sak]) : (half_t)0.0f;
+    }
+
+    NT_DEVICE void load_b16(int col, int k0, half_t out[16]) const {
+        const uint8_t *src = b + (int64_t)k0 * sbk + (int64_t)col * sbn;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) out[i] = (col < n && k0 + i < k) ? widen(src[(int64_t)i * sbk]) : (half_t)0.0f;
+    }
+
+    NT_DEVICE void store_c(int row, int col, float v) const { c[(int64_t)row * scm + (int64_t)col * scn] = from_float<TOut>(v); }
+};
+
 // ---- policy: conv2d as implicit GEMM (stride 1, dilation 1, zero padding) ----
 // GEMM row  = (image, out_y, out_x), GEMM k = (channel, filter_y, filter_x),
 // GEMM col  = output channel.

@@ -47,6 +47,8 @@ def _dtype_tag(torch_dtype):
             torch.float64: "fp64",
             torch.bool: "u8",
         }
+        if hasattr(torch, "float8_e5m2"):
+            _TORCH_DTYPE_TAGS[torch.float8_e5m2] = "fp8e5m2"
     try:
         return _TORCH_DTYPE_TAGS[torch_dtype]
     except KeyError:
@@ -145,6 +147,15 @@ class Kernel:
             self._source_path = str(path)
         return self._source_path
 
+    # the reference's handle also carries `_kernel` (the compiled kernel) and `_launch`
+    # (the launch function `__call__` forwards to), src/ninetoothed/jit.py:121-128
+    @property
+    def _kernel(self):
+        return self
+
+    def _launch(self, *args, **kwargs):
+        return self(*args, **kwargs)
+
     def __call__(self, *args, **kwargs):
         if len(args) != len(self.types):
             raise TypeError(f"`{self.kernel_name}` takes {len(self.types)} positional arguments but {len(args)} were given.")
@@ -217,9 +228,13 @@ class Kernel:
         kind, info = recognition.analyze_gemm(self.types[0], self.types[1], self.types[2], env)
         if kind == "empty":
             return _Plan("empty launch", lambda call_args: None)
-        tag = self._tensor_dtype(lhs, rhs, allowed=("fp16", "bf16"))
+        tag = self._tensor_dtype(lhs, rhs, allowed=("fp16", "bf16", "fp8e5m2"))
         out_tag = _dtype_tag(out.dtype)
         cast = self.details.get("cast")
+        if tag == "fp8e5m2":  # the second case of the reference's tests/test_matmul.py:61-88
+            if kind == "conv2d" or out_tag not in ("fp16", "fp32") or cast not in (None, out_tag):
+                raise UnsupportedProgram("fp8 operands are supported for plain matmul into fp16 / fp32 only.")
+            return self._gemm_plan(info, tag, out_tag, positions=(None, 0, 1, None, None, 2))
         if kind == "conv2d":
             if out_tag != tag or cast not in (None, tag):
                 raise UnsupportedProgram("conv2d needs input, filter and output of one element type.")
@@ -242,7 +257,7 @@ class Kernel:
 
     def _gemm_plan(self, info, tag, out_tag, positions):
         lib = runtime.library()
-        itemsize = 2
+        itemsize = 1 if tag == "fp8e5m2" else 2
         out_itemsize = 4 if out_tag == "fp32" else 2
         a, b, c, i = info["a"], info["b"], info["c"], info["input"]
         m, n, k = info["m"], info["n"], info["k"]

@@ -19,7 +19,7 @@ LIBRARY_PATH = pathlib.Path(__file__).resolve().parent / "lib" / "libnt_hip.so"
 NO_KERNEL = 1
 
 # order of the reference's NineToothedDataType enum (src/ninetoothed/aot.py:524-537)
-DATA_TYPES = ("i8", "i16", "i32", "i64", "u8", "u16", "u32", "u64", "fp16", "bf16", "fp32", "fp64")
+DATA_TYPES = ("i8", "i16", "i32", "i64", "u8", "u16", "u32", "u64", "fp16", "bf16", "fp32", "fp64", "fp8e5m2")  # the last one extends the enum
 DATA_TYPE_INDEX = {name: index for index, name in enumerate(DATA_TYPES)}
 
 

@@ -381,3 +381,21 @@ def test_first_launch_tunes_and_the_choice_persists(tmp_path, monkeypatch):
         assert code in (0, runtime.NO_KERNEL)
         if code == 0:
             assert torch.allclose(other, out, **HALF_TOL)
+
+
+@pytest.mark.skipif(not hasattr(torch, "float8_e5m2"), reason="this torch has no float8_e5m2")
+@pytest.mark.parametrize("m, n, k", ((512, 512, 512), (130, 70, 45)))
+def test_matmul_float8_e5m2_operands(m, n, k):
+    # tests/test_matmul.py:61-88 of the reference: fp8 operands (the right one column-major), fp16 output,
+    # compared with the fp16 product of the widened operands at atol 0.125; widening is exact, so the
+    # oracle on the widened operands must agree to fp16 rounding as well
+    lhs = _randn(m, k).to(torch.float8_e5m2)
+    rhs = _randn(n, k).to(torch.float8_e5m2).T  # shape (k, n), strides (1, k)
+    out = torch.full((m, n), float("nan"), dtype=torch.float16, device="cuda")
+    kernel = ninetoothed.make(programs.matmul.arrangement, programs.matmul.application, programs.matmul.tensors())
+    kernel(lhs.cuda(), rhs.cuda(), out)
+    _native_only(kernel, "launch_nt_matmul")
+    expected = torch.matmul(lhs.to(torch.float16).cuda(), rhs.to(torch.float16).cuda())
+    assert torch.allclose(out, expected, atol=0.125)
+    reference = oracle.matmul(lhs.to(torch.float16).numpy(), np.ascontiguousarray(rhs.to(torch.float16).numpy()), bm=64, bn=64, bk=64)
+    assert np.allclose(out.cpu().float().numpy(), reference, **HALF_TOL)
