@@ -15,9 +15,10 @@
  * `strides` are not read (reference: src/ninetoothed/aot.py:725-733, 624-628).
  *
  * Launches are asynchronous on the given stream and never synchronise; the
- * caller owns every tensor.  Only launch_nt_conv2d may take temporary device
- * memory, from the stream-ordered allocator (hipMallocAsync / hipFreeAsync on
- * the given stream, see there); every other launch allocates nothing.  All
+ * caller owns every tensor.  Only launch_nt_conv2d and launch_nt_attention on
+ * FLOAT32 tensors take temporary device memory, from the stream-ordered
+ * allocator (hipMallocAsync / hipFreeAsync on the given stream, see there);
+ * every other launch allocates nothing.  All
  * functions are re-entrant.
  */
 #ifndef NINETOOTHED_HIP_H
@@ -52,7 +53,8 @@ enum NineToothedDataType {
     NINETOOTHED_FLOAT64,
     /* extension beyond the reference's enum: 8-bit floating point with 5 exponent
      * and 2 mantissa bits, the operand type of the second case of
-     * tests/test_matmul.py:61-88; accepted by launch_nt_matmul only */
+     * tests/test_matmul.py:61-88 and tests/test_addmm.py:57-90; accepted by
+     * launch_nt_matmul and launch_nt_addmm (input, mat1, mat2 fp8, output fp16) */
     NINETOOTHED_FLOAT8_E5M2
 };
 
@@ -126,6 +128,11 @@ NineToothedResult launch_nt_softmax_config(NineToothedStream stream, int config,
  * program has scale == 1, the scale tensor (0-d, host double) is this
  * library's extension for the 1/sqrt(head_dim) configuration.
  * is_causal is a 0-d tensor holding a host int64_t.
+ * dtype FLOAT16 / BFLOAT16, or FLOAT32 (the fp32 case of
+ * tests/test_attention.py:99-117, rtol = atol = 0.025 there): K and V are first
+ * narrowed to fp16 copies taken from the stream-ordered allocator on `stream`,
+ * Q is narrowed while it is scaled, the products run on the fp16 MFMA path with
+ * fp32 accumulation and O is written unrounded.
  * block_size_m / block_size_n are hints (0 = library's choice): block_size_m
  * >= 256 selects 256 query rows per workgroup, block_size_n <= 32 the 32-key
  * blocks with three workgroups per CU, block_size_n >= 64 the plain 64-key

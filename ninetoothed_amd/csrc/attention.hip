@@ -36,7 +36,9 @@ constexpr int kAttnWaves = 4;
 
 // BN: key/value rows per block; kOcc: waves per SIMD the register budget is held to;
 // kPipelined: overlap the softmax of a block with the MFMAs of its neighbours
-template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined>
+// TIO: element type of Q and O in memory -- T, or float for fp32 tensors (their K and V
+// are converted to T beforehand; Q is converted while it is scaled, O is stored unrounded)
+template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined, typename TIO = T>
 __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(AttentionParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     typedef Elem<T> E;
@@ -97,10 +99,10 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
     const int batch = bh / p.heads;
     const int q0 = qb * BM;
 
-    const T *Q = (const T *)p.q + batch * p.q_strides[0] + head * p.q_strides[1];
+    const TIO *Q = (const TIO *)p.q + batch * p.q_strides[0] + head * p.q_strides[1];
     const T *K = (const T *)p.k + batch * p.k_strides[0] + head * p.k_strides[1];
     const T *V = (const T *)p.v + batch * p.v_strides[0] + head * p.v_strides[1];
-    T *O = (T *)p.o + batch * p.o_strides[0] + head * p.o_strides[1];
+    TIO *O = (TIO *)p.o + batch * p.o_strides[0] + head * p.o_strides[1];
 
     // ---- Q' fragments (B operand of S^T): lane holds row l32 of its q tile, 8 d's per step ----
     vec8 qf[kQTiles][KS];
@@ -109,12 +111,23 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
     for (int qt = 0; qt < kQTiles; ++qt) {
         q_row[qt] = q0 + (wave * kQTiles + qt) * 32 + l32;
         const int row = min(q_row[qt], p.seq_q - 1);
-        const T *src = Q + (int64_t)row * p.q_strides[2];
+        const TIO *src = Q + (int64_t)row * p.q_strides[2];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            vec8 raw = *(const vec8 *)(src + ks * 16 + 8 * g);
+            vec8 raw;
+            if constexpr (std::is_same<TIO, float>::value) {
+                const float4_t lo = *(const float4_t *)(src + ks * 16 + 8 * g);
+                const float4_t hi = *(const float4_t *)(src + ks * 16 + 8 * g + 4);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) raw[e] = E::from_float(E::to_float(raw[e]) * p.q_scale);
+                for (int e = 0; e < 4; ++e) {
+                    raw[e] = E::from_float(lo[e] * p.q_scale);
+                    raw[4 + e] = E::from_float(hi[e] * p.q_scale);
+                }
+            } else {
+                raw = *(const vec8 *)(src + ks * 16 + 8 * g);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) raw[e] = E::from_float(E::to_float(raw[e]) * p.q_scale);
+            }
             qf[qt][ks] = raw;
         }
     }
@@ -469,15 +482,19 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
         const float l_total = l_run[qt] + __shfl_xor(l_run[qt], 32, 64);
         const float inv = 1.0f / l_total;
         if (q_row[qt] < p.seq_q) {
-            T *dst = O + (int64_t)q_row[qt] * p.o_strides[2];
+            TIO *dst = O + (int64_t)q_row[qt] * p.o_strides[2];
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
                 for (int r4 = 0; r4 < 4; ++r4) {
-                    typedef T vec4 __attribute__((ext_vector_type(4)));
+                    typedef TIO vec4 __attribute__((ext_vector_type(4)));
                     vec4 out;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) out[e] = E::from_float(o_acc[dt][qt][r4 * 4 + e] * inv);
+                    for (int e = 0; e < 4; ++e) {
+                        const float value = o_acc[dt][qt][r4 * 4 + e] * inv;
+                        if constexpr (std::is_same<TIO, float>::value) out[e] = value;
+                        else out[e] = E::from_float(value);
+                    }
                     *(vec4 *)(dst + dt * 32 + 8 * r4 + 4 * g) = out;
                 }
         }
@@ -485,14 +502,50 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
 #endif
 }
 
-template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined>
+template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined, typename TIO = T>
 hipError_t launch_attention(AttentionParams &p, hipStream_t stream) {
     constexpr int BM = kAttnWaves * 32 * kQTiles;
     p.q_blocks = ceil_div(p.seq_q, BM);
     const int64_t grid = (int64_t)p.batch * p.heads * p.q_blocks;
     if (grid == 0) return hipSuccess;
-    attention_fwd_kernel<T, D, kQTiles, BN, kOcc, kPipelined><<<dim3((unsigned)grid), dim3(kAttnWaves * 64), 0, stream>>>(p);
+    attention_fwd_kernel<T, D, kQTiles, BN, kOcc, kPipelined, TIO><<<dim3((unsigned)grid), dim3(kAttnWaves * 64), 0, stream>>>(p);
     return hipGetLastError();
+}
+
+// fp32 tensors: K and V become contiguous [batch, heads, seq, D] half-precision copies
+__global__ __launch_bounds__(256) void attention_narrow_kernel(const float *src, half_t *dst, int64_t total, int heads, int seq, int dim, int64_t s0,
+                                                               int64_t s1, int64_t s2, int64_t s3) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int d = (int)(i % dim);
+        int64_t rest = i / dim;
+        const int s = (int)(rest % seq);
+        rest /= seq;
+        const int h = (int)(rest % heads);
+        const int64_t b = rest / heads;
+        dst[i] = (half_t)src[b * s0 + h * s1 + s * s2 + d * s3];
+    }
+}
+
+int attention_float32(AttentionParams p, int head_dim, const NineToothedTensor &k, const NineToothedTensor &v, hipStream_t stream) {
+    const int64_t total = (int64_t)p.batch * p.heads * p.seq_k * head_dim;
+    half_t *narrow = nullptr;
+    hipError_t err = hipMallocAsync((void **)&narrow, (size_t)total * 2 * sizeof(half_t), stream);
+    if (err != hipSuccess) return (int)err;
+    const unsigned blocks = (unsigned)((total + 255) / 256 < 256 * 16 ? (total + 255) / 256 : 256 * 16);
+    attention_narrow_kernel<<<dim3(blocks), dim3(256), 0, stream>>>((const float *)k.data, narrow, total, p.heads, p.seq_k, head_dim, k.strides[0],
+                                                                  k.strides[1], k.strides[2], k.strides[3]);
+    attention_narrow_kernel<<<dim3(blocks), dim3(256), 0, stream>>>((const float *)v.data, narrow + total, total, p.heads, p.seq_k, head_dim,
+                                                                  v.strides[0], v.strides[1], v.strides[2], v.strides[3]);
+    p.k = narrow;
+    p.v = narrow + total;
+    const int64_t contiguous[3] = {(int64_t)p.heads * p.seq_k * head_dim, (int64_t)p.seq_k * head_dim, head_dim};
+    for (int d = 0; d < 3; ++d) p.k_strides[d] = p.v_strides[d] = contiguous[d];
+    int result = NINETOOTHED_NO_KERNEL;
+    if (head_dim == 128) result = (int)launch_attention<half_t, 128, 1, 64, 2, false, float>(p, stream);
+    else if (head_dim == 64) result = (int)launch_attention<half_t, 64, 1, 64, 2, false, float>(p, stream);
+    else if (head_dim == 32) result = (int)launch_attention<half_t, 32, 1, 64, 2, false, float>(p, stream);
+    const hipError_t released = hipFreeAsync(narrow, stream);
+    return result != 0 ? result : (int)released;
 }
 
 // variant: 0 = 128 query rows per workgroup, 64-key blocks, two workgroups per CU
@@ -526,7 +579,8 @@ extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineT
                                                  NineToothedTensor v, NineToothedTensor is_causal,
                                                  NineToothedTensor scale, NineToothedTensor o, int dtype,
                                                  int block_size_m, int block_size_n) {
-    if (dtype != NINETOOTHED_FLOAT16 && dtype != NINETOOTHED_BFLOAT16) return NINETOOTHED_NO_KERNEL;
+    if (dtype != NINETOOTHED_FLOAT16 && dtype != NINETOOTHED_BFLOAT16 && dtype != NINETOOTHED_FLOAT32) return NINETOOTHED_NO_KERNEL;
+    const bool float32 = dtype == NINETOOTHED_FLOAT32;
     const NineToothedTensor *ts[4] = {&q, &k, &v, &o};
     for (const NineToothedTensor *t : ts)
         if (!t->shape || !t->strides) return hipErrorInvalidValue;
@@ -538,13 +592,16 @@ extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineT
     const int64_t head_dim = (int64_t)q.shape[3];
     for (const NineToothedTensor *t : ts) {
         if (t->shape[0] != q.shape[0] || t->shape[1] != q.shape[1] || (int64_t)t->shape[3] != head_dim) return hipErrorInvalidValue;
+        if (float32 && (t == &k || t == &v)) continue;  // converted copies: any strides
         if (t->strides[3] != 1 && head_dim > 1) return NINETOOTHED_NO_KERNEL;
-        if (((uintptr_t)t->data & 15) || t->strides[0] % 8 || t->strides[1] % 8 || t->strides[2] % 8) return NINETOOTHED_NO_KERNEL;
+        const int lanes = float32 ? 4 : 8;  // elements per 16 bytes
+        if (((uintptr_t)t->data & 15) || t->strides[0] % lanes || t->strides[1] % lanes || t->strides[2] % lanes) return NINETOOTHED_NO_KERNEL;
     }
     if (v.shape[2] != k.shape[2] || o.shape[2] != q.shape[2]) return hipErrorInvalidValue;
     if (q.shape[2] > 0x7fffffffull || k.shape[2] > 0x7fffffffull) return NINETOOTHED_NO_KERNEL;
     // K and V of one (batch, head) are read through 32-bit buffer offsets
     for (const NineToothedTensor *t : {&k, &v}) {
+        if (float32) break;
         if (t->strides[2] < 0) return NINETOOTHED_NO_KERNEL;
         if (((int64_t)t->shape[2] + 64) * t->strides[2] * 2 + 2 * head_dim > 0xffffffffll) return NINETOOTHED_NO_KERNEL;
     }
@@ -563,6 +620,7 @@ extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineT
     const double scale_value = scale.data ? Scalar0d::as_double(scale) : 1.0;
     p.q_scale = (float)(scale_value * 1.4426950408889634);
     p.causal = is_causal.data ? (Scalar0d::as_int64(is_causal) != 0) : 0;
+    if (float32) return attention_float32(p, (int)head_dim, k, v, (hipStream_t)stream);
     // block sizes are hints: 256 query rows select the one-workgroup-per-CU
     // variant, 32-key blocks the three-workgroups-per-CU variant.  Without a hint
     // the pipelined variant runs non-causal problems; causal ones, whose waves

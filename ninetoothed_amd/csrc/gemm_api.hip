@@ -95,8 +95,8 @@ hipError_t fast_launch(const GemmProblem &q, hipStream_t stream) {
 }
 
 bool generic_accepts(const GemmProblem &q) {
-    if (q.dtype == NINETOOTHED_FLOAT8_E5M2)  // matmul only, widened to fp16
-        return !q.addmm() && (q.out_dtype == NINETOOTHED_FLOAT16 || q.out_dtype == NINETOOTHED_FLOAT32) && q.m >= 0 && q.n >= 0 && q.k >= 0;
+    if (q.dtype == NINETOOTHED_FLOAT8_E5M2)  // widened to fp16; addmm rounds its product to fp16, so it writes fp16
+        return (q.out_dtype == NINETOOTHED_FLOAT16 || (q.out_dtype == NINETOOTHED_FLOAT32 && !q.addmm())) && q.m >= 0 && q.n >= 0 && q.k >= 0;
     if (q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) return false;
     if (q.out_dtype != q.dtype && q.out_dtype != NINETOOTHED_FLOAT32) return false;
     return q.m >= 0 && q.n >= 0 && q.k >= 0;
@@ -143,6 +143,11 @@ hipError_t fp8_launch_typed(const GemmProblem &q, hipStream_t stream) {
     prob.sbn = q.sbn;
     prob.scm = q.scm;
     prob.scn = q.scn;
+    prob.bias = (const uint8_t *)q.bias;
+    prob.sbm_ = q.sim;
+    prob.sbn_ = q.sin;
+    prob.alpha = q.alpha;
+    prob.beta = q.beta;
     const int64_t tiles = (int64_t)ceil_div(q.m, kGenBM) * ceil_div(q.n, kGenBN);
     if (tiles == 0) return hipSuccess;
     gemm_generic_kernel<Fp8E5m2Problem<TOut>><<<dim3((unsigned)tiles), dim3(kGenThreads), 0, stream>>>(prob);
@@ -313,7 +318,8 @@ NineToothedResult launch_nt_addmm(NineToothedStream stream, NineToothedTensor in
                                   int block_size_k) {
     if (input.data == nullptr) return hipErrorInvalidValue;
     GemmProblem q;
-    if (int err = build_problem(q, &input, mat1, mat2, &beta, &alpha, output, dtype, dtype)) return err;
+    const int output_dtype = dtype == NINETOOTHED_FLOAT8_E5M2 ? NINETOOTHED_FLOAT16 : dtype;  // fp8 operands: the rounded product is fp16
+    if (int err = build_problem(q, &input, mat1, mat2, &beta, &alpha, output, dtype, output_dtype)) return err;
     return run_gemm((hipStream_t)stream, q, block_size_m, block_size_n, block_size_k);
 }
 

@@ -186,7 +186,9 @@ struct Fp8E5m2Problem {
     const uint8_t *a;
     const uint8_t *b;
     TOut *c;
-    int64_t sam, sak, sbk, sbn, scm, scn;
+    const uint8_t *bias;  // addmm input (fp8 as well), or null
+    int64_t sam, sak, sbk, sbn, scm, scn, sbm_, sbn_;
+    float alpha, beta;
 
     static NT_DEVICE half_t widen(uint8_t byte) {
         const unsigned short bits = (unsigned short)((unsigned short)byte << 8);
@@ -205,7 +207,14 @@ struct Fp8E5m2Problem {
         for (int i = 0; i < 16; ++i) out[i] = (col < n && k0 + i < k) ? widen(src[(int64_t)i * sbk]) : (half_t)0.0f;
     }
 
-    NT_DEVICE void store_c(int row, int col, float v) const { c[(int64_t)row * scm + (int64_t)col * scn] = from_float<TOut>(v); }
+    NT_DEVICE void store_c(int row, int col, float v) const {
+        if (bias != nullptr) {  // the product is rounded to fp16 first, the combination happens in fp32
+            const float mm = (float)(half_t)v;
+            const float in = (float)widen(bias[(int64_t)row * sbm_ + (int64_t)col * sbn_]);
+            v = beta * in + alpha * mm;
+        }
+        c[(int64_t)row * scm + (int64_t)col * scn] = from_float<TOut>(v);
+    }
 };
 
 // ---- policy: conv2d as implicit GEMM (stride 1, dilation 1, zero padding) ----

@@ -250,6 +250,11 @@ class Kernel:
         kind, info = recognition.analyze_gemm(self.types[1], self.types[2], self.types[5], env, input_type=self.types[0])
         if kind == "empty":
             return _Plan("empty launch", lambda call_args: None)
+        if _dtype_tag(mat1.dtype) == "fp8e5m2":  # the second case of the reference's tests/test_addmm.py:57-90
+            tag = self._tensor_dtype(input, mat1, mat2, allowed=("fp8e5m2",))
+            if self.details.get("cast") != "fp16" or _dtype_tag(out.dtype) != "fp16":
+                raise UnsupportedProgram("addmm on fp8 operands rounds the product to fp16 and writes an fp16 tensor.")
+            return self._gemm_plan(info, tag, "fp16", positions=(0, 1, 2, 3, 4, 5))
         tag = self._tensor_dtype(input, mat1, mat2, out, allowed=("fp16", "bf16"))
         if self.details.get("cast") != tag:
             raise UnsupportedProgram(f"The application rounds the product to `{self.details.get('cast')}` but the tensors hold `{tag}`.")
@@ -381,7 +386,7 @@ class Kernel:
         kind, info = recognition.analyze_attention(q_t, k_t, v_t, o_t, env)
         if kind == "empty":
             return _Plan("empty launch", lambda call_args: None)
-        tag = self._tensor_dtype(q, k, v, o, allowed=("fp16", "bf16"))
+        tag = self._tensor_dtype(q, k, v, o, allowed=("fp16", "bf16", "fp32"))
         lib = runtime.library()
         dtype = runtime.DATA_TYPE_INDEX[tag]
         o_pos = 5 if scaled else 4

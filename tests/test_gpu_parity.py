@@ -399,3 +399,36 @@ def test_matmul_float8_e5m2_operands(m, n, k):
     assert torch.allclose(out, expected, atol=0.125)
     reference = oracle.matmul(lhs.to(torch.float16).numpy(), np.ascontiguousarray(rhs.to(torch.float16).numpy()), bm=64, bn=64, bk=64)
     assert np.allclose(out.cpu().float().numpy(), reference, **HALF_TOL)
+
+
+@pytest.mark.skipif(not hasattr(torch, "float8_e5m2"), reason="this torch has no float8_e5m2")
+def test_addmm_float8_e5m2_operands():
+    # tests/test_addmm.py:57-90 of the reference: fp8 input, mat1, mat2 (the last column-major), fp16 output
+    m, n, k = 512, 512, 512
+    input = _randn(m, n).to(torch.float8_e5m2)
+    mat1 = _randn(m, k).to(torch.float8_e5m2)
+    mat2 = _randn(n, k).to(torch.float8_e5m2).T
+    beta, alpha = 0.37, 0.81
+    out = torch.full((m, n), float("nan"), dtype=torch.float16, device="cuda")
+    kernel = ninetoothed.make(programs.addmm.arrangement, programs.addmm.application, programs.addmm.tensors())
+    kernel(input.cuda(), mat1.cuda(), mat2.cuda(), beta, alpha, out)
+    _native_only(kernel, "launch_nt_addmm")
+    widened = [t.to(torch.float16) for t in (input, mat1, mat2)]
+    expected = torch.addmm(widened[0].cuda(), widened[1].cuda(), widened[2].cuda(), beta=beta, alpha=alpha)
+    assert torch.allclose(out, expected, atol=0.075)
+    reference = oracle.addmm(widened[0].numpy(), widened[1].numpy(), np.ascontiguousarray(widened[2].numpy()), beta, alpha)
+    assert np.allclose(out.cpu().float().numpy(), reference, **HALF_TOL)
+
+
+@pytest.mark.parametrize("is_causal", (False, True))
+@pytest.mark.parametrize("seq_len", (1024, 1))
+def test_attention_float32_tensors(seq_len, is_causal):
+    # the fp32 case of tests/test_attention.py:99-117 of the reference, with its tolerance
+    q, k, v = (torch.randn(2, 4, seq_len, 64, generator=torch.Generator().manual_seed(s)) for s in (0, 1, 2))
+    out = _attention(q.cuda(), k.cuda(), v.cuda(), is_causal)
+    expected = F.scaled_dot_product_attention(q.cuda(), k.cuda(), v.cuda(), is_causal=is_causal, scale=1)
+    assert out.dtype == torch.float32
+    assert torch.allclose(out, expected, rtol=0.025, atol=0.025)
+    # strided K / V (a transposed view) go through the same conversion
+    k_view = k.transpose(1, 2).contiguous().transpose(1, 2)
+    assert torch.allclose(_attention(q.cuda(), k_view.cuda(), v.cuda(), is_causal), expected, rtol=0.025, atol=0.025)
