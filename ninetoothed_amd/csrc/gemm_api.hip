@@ -171,6 +171,8 @@ const GemmInstance kInstances[] = {
     NT_FAST_INSTANCE(256, 256, 32, 2, 4, 5, 2),  // 5 x 32 KiB: the whole LDS of a CU
     NT_FAST_INSTANCE(256, 256, 64, 2, 4, 2, 2),
     NT_FAST_INSTANCE(128, 128, 64, 2, 2, 2, 2),
+    NT_FAST_INSTANCE(64, 64, 64, 2, 2, 4, 2),  // small problems: more, smaller tiles to occupy the CUs
+    NT_FAST_INSTANCE(128, 256, 32, 1, 4, 3, 2),  // two workgroups per CU: mid-size problems
 #ifdef NT_GEMM_ABLATION
 #define NT_LOAD_INSTANCE(BM, BN, BK, WM, WN, ST, OCC, LD, AUX) \
     {#BM "x" #BN "x" #BK " waves " #WM "x" #WN " stages " #ST " load " #LD " aux " #AUX, BM, BN, BK, fast_accepts<BM, BN, BK, ST>, fast_launch<BM, BN, BK, WM, WN, ST, OCC, 0, LD, AUX>}
@@ -236,12 +238,15 @@ int heuristic_choice(const GemmProblem &q, int bm, int bn, int bk) {
         }
         return best;
     }
-    const int order[] = {1, 2, 3};
-    for (int idx : order) {
-        const GemmInstance &inst = kInstances[idx];
+    // untuned preference (measured on square problems): 256x256 tiles from 256 tiles up,
+    // 128x256 from 128 tiles up, 128x128 from 256 tiles up, else the smallest tile that divides
+    struct Rule { int instance; int64_t min_tiles; };
+    const Rule rules[] = {{1, 256}, {2, 256}, {5, 128}, {3, 256}, {4, 1}, {3, 1}, {5, 1}, {2, 1}, {1, 1}};
+    for (const Rule &rule : rules) {
+        const GemmInstance &inst = kInstances[rule.instance];
         if (!inst.accepts(q)) continue;
         const int64_t tiles = (int64_t)(q.m / inst.bm) * (q.n / inst.bn);
-        if (tiles >= 256 || idx == 3) return idx;
+        if (tiles >= rule.min_tiles) return rule.instance;
     }
     return kInstances[0].accepts(q) ? 0 : -1;
 }

@@ -122,9 +122,14 @@ def check(result):
 
 
 def current_stream():
+    """The raw handle of torch's current stream on the current device (what the
+    reference's launcher passes, src/ninetoothed/aot.py:834-856)."""
     import torch
 
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    try:
+        return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(torch.cuda.current_device()))
+    except AttributeError:  # a torch without the private accessor
+        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
 def gemm_config_names():

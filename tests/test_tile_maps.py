@@ -413,3 +413,29 @@ def test_empty_tensor_and_no_store():
     kernel(torch.randn((0,), device="cuda"))
     out = torch.empty(0, device="cuda")
     add_kernel(torch.empty(0, device="cuda"), torch.empty(0, device="cuda"), out)
+
+
+def _expand_arrangement(x, BLOCK_SIZE=block_size()):
+    return (x.expand((BLOCK_SIZE,)).tile((BLOCK_SIZE,)),)
+
+
+def _no_store_application(x):
+    x
+
+
+def _single_tensor_arrangement(x):
+    return x.tile((ninetoothed.block_size(),))
+
+
+def test_programs_without_stores_are_accepted():
+    # tests/test_expand.py:9-23 and tests/test_generation.py:59-70 of the reference
+    assert ninetoothed.make(_expand_arrangement, _no_store_application, (Tensor(1),)).kind == "map"
+    assert ninetoothed.make(_single_tensor_arrangement, _no_store_application, (Tensor(1),)).kind == "map"
+
+
+@gpu
+def test_expand_on_an_empty_tensor():
+    kernel = ninetoothed.make(_expand_arrangement, _no_store_application, (Tensor(1),))
+    kernel(torch.empty((0,), device="cuda"))
+    kernel = ninetoothed.make(_single_tensor_arrangement, _no_store_application, (Tensor(1),))
+    kernel(torch.randn(100, device="cuda"))
