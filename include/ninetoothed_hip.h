@@ -233,6 +233,9 @@ int nt_tune_cache_lookup(int dtype, int output_dtype, int m, int n, int k, int a
  *   - the iteration space is `num_vars` index variables with `extents`; the
  *     first `num_vars - num_reduced` enumerate the output elements (the last of
  *     them varies fastest across lanes), the rest the reduced positions;
+ *     `num_dynamic` further variables take their value from the data
+ *     (`output[row] = input` with `row` loaded from a tensor,
+ *     tests/test_generation.py:72-115);
  *   - index code (one segment per operand, and per `.offsets()` use) computes a
  *     flat element offset from the variables with + * // % by constants
  *     (src/ninetoothed/tensor.py:258-274, 462-471, 555-556) and checks
@@ -286,7 +289,8 @@ enum NineToothedMapValueOp {
     NT_MAP_V_SQRT, NT_MAP_V_RSQRT, NT_MAP_V_SIGMOID, NT_MAP_V_TANH, NT_MAP_V_SIN, NT_MAP_V_COS, NT_MAP_V_FLOOR, NT_MAP_V_CEIL,
     NT_MAP_V_WHERE,     /* pop b, a, c; push c ? a : b */
     NT_MAP_V_ROUND,     /* round top to NineToothedDataType arg (integers truncate) */
-    NT_MAP_V_RAND       /* pop offset, seed; push the Philox-4x32-10 uniform float of (seed, offset) */
+    NT_MAP_V_RAND,      /* pop offset, seed; push the Philox-4x32-10 uniform float of (seed, offset) */
+    NT_MAP_V_SETVAR     /* pop v; dynamic variable arg = (integer) v: a data-dependent level index */
 };
 
 enum NineToothedMapReduceOp { NT_MAP_REDUCE_NONE, NT_MAP_REDUCE_MAX, NT_MAP_REDUCE_MIN, NT_MAP_REDUCE_SUM };
@@ -299,8 +303,10 @@ typedef struct {
 } NineToothedMapOperand;
 
 typedef struct {
-    int32_t num_vars;
+    int32_t num_vars;     /* enumerated variables: output elements, then reduced positions */
     int32_t num_reduced;
+    int32_t num_dynamic;  /* variables num_vars .. num_vars + num_dynamic - 1 are set by NT_MAP_V_SETVAR */
+    int32_t reserved;
     int64_t extents[NT_MAP_MAX_VARS];
     int32_t num_operands;
     int32_t output;              /* operand that is stored */

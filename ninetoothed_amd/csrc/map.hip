@@ -150,7 +150,7 @@ __device__ __forceinline__ double philox_uniform(uint64_t seed, uint64_t offset)
 }
 
 // runs value_code[begin, end) on a stack that starts as `initial` (when `seeded`)
-__device__ __forceinline__ double run_value(const NineToothedMapProgram &p, int begin, int end, const int64_t *vars, bool seeded,
+__device__ __forceinline__ double run_value(const NineToothedMapProgram &p, int begin, int end, int64_t *vars, bool seeded,
                                              double initial) {
     double stack[kValueStack];
     int top = -1;
@@ -232,6 +232,7 @@ __device__ __forceinline__ double run_value(const NineToothedMapProgram &p, int 
                 stack[top] = philox_uniform((uint64_t)(int64_t)stack[top], (uint64_t)(int64_t)offset);
                 break;
             }
+            case NT_MAP_V_SETVAR: vars[arg] = (int64_t)stack[top--]; break;
             default: break;
         }
     }
@@ -243,6 +244,7 @@ __global__ __launch_bounds__(kMapThreads) void map_kernel(const NineToothedMapPr
     const int64_t stride = (int64_t)gridDim.x * kMapThreads;
     for (int64_t element = (int64_t)blockIdx.x * kMapThreads + threadIdx.x; element < total_out; element += stride) {
         int64_t vars[NT_MAP_MAX_VARS];
+        for (int v = p.num_vars; v < p.num_vars + p.num_dynamic; ++v) vars[v] = 0;
         int64_t rest = element;
         for (int v = num_out - 1; v >= 0; --v) {
             const int64_t extent = p.extents[v];
@@ -283,6 +285,7 @@ __global__ __launch_bounds__(kMapThreads) void map_kernel(const NineToothedMapPr
 
 bool well_formed(const NineToothedMapProgram &p) {
     if (p.num_vars < 0 || p.num_vars > NT_MAP_MAX_VARS || p.num_reduced < 0 || p.num_reduced > p.num_vars) return false;
+    if (p.num_dynamic < 0 || p.num_vars + p.num_dynamic > NT_MAP_MAX_VARS) return false;
     if (p.num_operands < 1 || p.num_operands > NT_MAP_MAX_OPERANDS || p.output < 0 || p.output >= p.num_operands) return false;
     if (p.num_segments < 1 || p.num_segments > NT_MAP_MAX_SEGMENTS) return false;
     if (p.value_code_length < 0 || p.value_code_length > NT_MAP_MAX_VALUE_CODE) return false;
@@ -305,7 +308,7 @@ bool well_formed(const NineToothedMapProgram &p) {
             const int op = p.index_code[pc] & 0xff, arg = p.index_code[pc] >> 8;
             if (op == NT_MAP_I_END) break;
             if (op == NT_MAP_I_VAR) {
-                if (arg < 0 || arg >= p.num_vars) return false;
+                if (arg < 0 || arg >= p.num_vars + p.num_dynamic) return false;
                 ++depth;
             } else if (op == NT_MAP_I_ADD) {
                 if (depth < 2) return false;
@@ -349,6 +352,9 @@ bool well_formed(const NineToothedMapProgram &p) {
             if (depth < 1 || arg < NINETOOTHED_INT8 || arg > NINETOOTHED_FLOAT64) return false;
         } else if (op == NT_MAP_V_RAND) {
             if (depth < 2) return false;
+            --depth;
+        } else if (op == NT_MAP_V_SETVAR) {
+            if (depth < 1 || arg < p.num_vars || arg >= p.num_vars + p.num_dynamic) return false;
             --depth;
         } else {
             return false;
@@ -549,6 +555,9 @@ struct MapCodegen {
                 const std::string offset = stack.back();
                 stack.pop_back();
                 stack.back() = define("nt_philox_uniform((unsigned long long)(long long)" + stack.back() + ", (unsigned long long)(long long)" + offset + ")");
+            } else if (op == NT_MAP_V_SETVAR) {
+                out << indent << "v" << arg << " = (long long)(" << stack.back() << ");\n";
+                stack.pop_back();
             }
         }
         return stack.empty() ? std::string("0.0") : stack.back();
@@ -579,6 +588,7 @@ struct MapCodegen {
             // 32-bit division when the extent allows it would be cheaper; the divisor is a literal either way
             out << "        const long long v" << v << " = rest % " << (long long)p.extents[v] << "LL; rest /= " << (long long)p.extents[v] << "LL;\n";
         }
+        for (int v = p.num_vars; v < p.num_vars + p.num_dynamic; ++v) out << "        long long v" << v << " = 0;\n";
         std::string result;
         if (p.reduce_op == NT_MAP_REDUCE_NONE) {
             result = value_range(0, p.value_code_length, "");

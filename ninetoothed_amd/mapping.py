@@ -44,7 +44,7 @@ I_END, I_CONST, I_VAR, I_MULC, I_ADD, I_DIVC, I_MODC, I_CHECK = range(8)
 
 _VALUE_OPS = (
     "LOAD CONST OFFSET ADD SUB MUL DIV FLOORDIV MOD POW MAX MIN LT LE GT GE EQ NE AND OR "
-    "NEG NOT ABS EXP EXP2 LOG LOG2 SQRT RSQRT SIGMOID TANH SIN COS FLOOR CEIL WHERE ROUND RAND"
+    "NEG NOT ABS EXP EXP2 LOG LOG2 SQRT RSQRT SIGMOID TANH SIN COS FLOOR CEIL WHERE ROUND RAND SETVAR"
 ).split()
 V = {name: index for index, name in enumerate(_VALUE_OPS)}
 
@@ -59,6 +59,8 @@ class MapProgram(ctypes.Structure):
     _fields_ = [
         ("num_vars", ctypes.c_int32),
         ("num_reduced", ctypes.c_int32),
+        ("num_dynamic", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
         ("extents", ctypes.c_int64 * MAX_VARS),
         ("num_operands", ctypes.c_int32),
         ("output", ctypes.c_int32),
@@ -110,6 +112,10 @@ def _needs_rounding(dtype):
     return dtype in ("fp16", "bf16", "fp32") or dtype in _INT_RANK and dtype != "bool"
 
 
+def operand_param(lowering, slot):
+    return lowering.operands[slot][0]
+
+
 # ---- the application: which programs are tile maps ----------------------------------
 
 _BINARY = {
@@ -155,19 +161,25 @@ class _Lowering:
         self.bindings = {}        # operand slot -> {operand variable name: shared variable id}
         self.scalar_slots = []    # (constant index, parameter position): refreshed at every launch
         self.reduced_vars = []
+        self.dynamic_vars = []    # variables that take their value from the data (level indices)
+        self.levels_used = {}     # param -> level its tiles are taken from
 
     # -- variables ---------------------------------------------------------
     def new_var(self, extent):
         self.var_extent.append(int(extent))
         return len(self.var_extent) - 1
 
-    def operand(self, param):
+    def operand(self, param, level=1):
+        if self.levels_used.setdefault(param, level) != level:
+            raise UnsupportedProgram("A tensor is used at two different levels.")
         if param in self.operand_slot:
             return self.operand_slot[param]
         tensor = self.types[param]
         operand = Operand(tensor, self.env)
-        if len(operand.names) > 2:
-            raise UnsupportedProgram(f"`{tensor.source.name}` has more than one level below the launch grid.")
+        if len(operand.names) > level + 1:
+            raise UnsupportedProgram(f"`{tensor.source.name}` has a level below the tiles the application uses.")
+        if len(operand.names) < level:
+            raise UnsupportedProgram(f"`{tensor.source.name}` is indexed deeper than it is arranged.")
         grid_names = operand.names[0]
         if self.grid is None:
             self.grid = [self.new_var(operand.extents[name]) for name in grid_names]
@@ -191,7 +203,8 @@ class _Lowering:
     def bind_tile(self, slot, dims):
         """Binds the operand's tile dimensions to the shared variables ``dims``."""
         _, operand = self.operands[slot]
-        tile_names = operand.names[1] if len(operand.names) > 1 else []
+        level = self.levels_used[operand_param(self, slot)]
+        tile_names = operand.names[level] if len(operand.names) > level else []
         if len(tile_names) != len(dims):
             raise UnsupportedProgram(
                 f"A tile of `{operand.tensor.source.name}` has {len(tile_names)} dimensions where the expression needs {len(dims)}."
@@ -266,15 +279,13 @@ class _Lowering:
             self._check_ref(ref)
             if self.reduce is not None and not inside_reduction:
                 raise UnsupportedProgram("Tiles may only be loaded below the reduction of the expression.")
-            slot = self.operand(ref.param)
-            self.bind_tile(slot, dims)
+            slot = self.bind_ref(ref, dims, inside_reduction)
             self.emit("LOAD", slot)
             return self.dtype_tag(ref.param)
         if op == "offsets":
             ref, dim = value.args
             self._check_ref(ref)
-            slot = self.operand(ref.param)
-            self.bind_tile(slot, dims)
+            slot = self.bind_ref(ref, dims, inside_reduction)
             self.emit("OFFSET", self.segment(slot, "offsets", dim))
             return "i64" if dim is None else "i32"
         if op in _BINARY or op in _COMPARE or op in _LOGICAL:
@@ -409,8 +420,39 @@ class _Lowering:
         return ranks.pop()
 
     def _check_ref(self, ref):
-        if not isinstance(ref, TensorRef) or ref.level != 1 or ref.indices or not ref.is_tile:
-            raise UnsupportedProgram("Only whole tiles directly below the launch grid can be used by the element-wise executor.")
+        if not isinstance(ref, TensorRef) or ref.level not in (1, 2) or not ref.is_tile:
+            raise UnsupportedProgram("Only whole tiles one or two levels below the launch grid can be used by the element-wise executor.")
+
+    def bind_ref(self, ref, dims, inside_reduction):
+        """Registers the operand of ``ref``, binds its tile to ``dims`` and, for a tile taken
+        from a middle level (``tensor[i, j]``), emits the code that computes the level indices."""
+        slot = self.operand(ref.param, ref.level)
+        self.bind_tile(slot, dims)
+        if ref.level == 2:
+            _, operand = self.operands[slot]
+            names = operand.names[1]
+            if len(ref.indices) != len(names):
+                raise UnsupportedProgram("A level must be indexed with one index per dimension.")
+            binding = self.bindings[slot]
+            for name, index in zip(names, ref.indices):
+                if name in binding:
+                    raise UnsupportedProgram("A tensor may be indexed at a middle level only once per program.")
+                var = self.new_var(operand.extents[name])
+                self.dynamic_vars.append(var)
+                binding[name] = var
+                # the index is a scalar: a constant, a call-time scalar or a one-element tile
+                rank = self._tile_rank(index) if isinstance(index, Node) and self._has_load(index) else 0
+                unit = [self.new_var(1) for _ in range(rank)]
+                self.lower(index, unit, inside_reduction)
+                self.emit("SETVAR", var)
+        return slot
+
+    def _has_load(self, value):
+        if isinstance(value, Node):
+            return value.op == "load" or any(self._has_load(arg) for arg in value.args)
+        if isinstance(value, (tuple, list)):
+            return any(self._has_load(item) for item in value)
+        return False
 
     # -- index code ----------------------------------------------------------------
     def index_program(self, order):
@@ -443,6 +485,12 @@ class _Lowering:
             binding = self.bindings[slot]
             begins.append(len(code))
             if kind == "access":
+                # indices that come from the data are range-checked: an element outside its level
+                # is treated like a masked one (the reference would access out of bounds)
+                for name, var in binding.items():
+                    if var in self.dynamic_vars:
+                        code.append(I_VAR | (order[var] << 8))
+                        code.append(I_CHECK | (const(operand.extents[name]) << 8))
                 for index, size in operand.constraints:
                     emit_affine(index, binding)
                     code.append(I_CHECK | (const(size) << 8))
@@ -467,11 +515,11 @@ def build(program_store, types, args, env, dtype_tag, data_ptr):
     ref, value = program_store
     lowering = _Lowering(types, args, env, dtype_tag)
     lowering._check_ref(ref)
-    out_slot = lowering.operand(ref.param)
+    out_slot = lowering.operand(ref.param, ref.level)
     _, out_operand = lowering.operands[out_slot]
-    tile_names = out_operand.names[1] if len(out_operand.names) > 1 else []
+    tile_names = out_operand.names[ref.level] if len(out_operand.names) > ref.level else []
     out_dims = [lowering.new_var(out_operand.extents[name]) for name in tile_names]
-    lowering.bind_tile(out_slot, out_dims)
+    lowering.bind_ref(ref, out_dims, False)
     result = lowering.lower(value, out_dims, False)
     out_dtype = dtype_tag(ref.param)
     if result != out_dtype:
@@ -488,7 +536,8 @@ def build(program_store, types, args, env, dtype_tag, data_ptr):
     # variable order: grid and output-tile variables enumerate the output elements
     # (the fastest one is chosen so that lanes walk the output contiguously), reduced ones follow
     reduced = list(lowering.reduced_vars)
-    outer = [v for v in range(len(lowering.var_extent)) if v not in reduced]
+    dynamic = list(lowering.dynamic_vars)
+    outer = [v for v in range(len(lowering.var_extent)) if v not in reduced and v not in dynamic]
     out_binding = lowering.bindings[out_slot]
     offset = out_operand.offset()
     stride_of = {}
@@ -496,7 +545,11 @@ def build(program_store, types, args, env, dtype_tag, data_ptr):
         stride_of[var] = abs(offset.coef(name)) if offset.is_linear() else None
     if all(stride_of.get(v) is not None for v in outer):
         outer.sort(key=lambda v: (-(stride_of[v] or 1 << 62) if lowering.var_extent[v] > 1 else -(1 << 62), v))
-    order = {old: new for new, old in enumerate(outer + reduced)}
+    order = {old: new for new, old in enumerate(outer + reduced + dynamic)}
+    # SETVAR words were emitted with provisional ids: renumber them like the index code
+    for position, word in enumerate(lowering.value_code):
+        if word & 0xFF == V["SETVAR"]:
+            lowering.value_code[position] = V["SETVAR"] | (order[word >> 8] << 8)
     if len(order) > MAX_VARS:
         raise UnsupportedProgram("Too many index variables for the element-wise executor.")
 
@@ -507,8 +560,9 @@ def build(program_store, types, args, env, dtype_tag, data_ptr):
         raise UnsupportedProgram("The expression is too long for the element-wise executor.")
 
     program = MapProgram()
-    program.num_vars = len(order)
+    program.num_vars = len(outer) + len(reduced)
     program.num_reduced = len(reduced)
+    program.num_dynamic = len(dynamic)
     for old, new in order.items():
         program.extents[new] = lowering.var_extent[old]
     program.num_operands = len(lowering.operands)
@@ -535,6 +589,8 @@ def build(program_store, types, args, env, dtype_tag, data_ptr):
         program.value_constants[index] = value_
     description = (
         f"{len(lowering.operands)} operands, {program.num_vars} index variables {[lowering.var_extent[old] for old in outer + reduced]}, "
+        + (f"{len(dynamic)} data-dependent, " if dynamic else "")
+        + 
         f"{len(code)} index words, {len(lowering.value_code)} value words"
         + (f", {lowering.reduce[0]} over {len(reduced)} dimension(s)" if lowering.reduce else "")
     )
@@ -546,8 +602,9 @@ def check_application(program):
     executor handles (sizes are checked later, per call)."""
 
     for ref, value in program.stores:
-        if not isinstance(ref, TensorRef) or ref.level != 1 or ref.indices or not ref.is_tile:
-            raise UnsupportedProgram("Stores must assign whole tiles directly below the launch grid.")
+        if not isinstance(ref, TensorRef) or ref.level not in (1, 2) or not ref.is_tile:
+            raise UnsupportedProgram("Stores must assign whole tiles one or two levels below the launch grid.")
+        _scan(ref.indices)
         _scan(value)
 
 
@@ -565,5 +622,6 @@ def _scan(value):
         for item in value:
             _scan(item)
     elif isinstance(value, TensorRef):
-        if value.level != 1 or value.indices or not value.is_tile:
-            raise UnsupportedProgram("Only whole tiles directly below the launch grid can be used by the element-wise executor.")
+        if value.level not in (1, 2) or not value.is_tile:
+            raise UnsupportedProgram("Only whole tiles one or two levels below the launch grid can be used by the element-wise executor.")
+        _scan(value.indices)

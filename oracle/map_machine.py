@@ -148,6 +148,8 @@ class Machine:
                     offset = stack.pop()
                     seed = stack.pop()
                     stack.append(philox_uniform(seed.astype(np.int64), offset.astype(np.int64)))
+                elif op == "SETVAR":
+                    variables[arg] = np.broadcast_to(np.trunc(stack.pop()).astype(np.int64), shape)
                 else:
                     a = stack.pop()
                     f32 = a.astype(np.float32)
@@ -170,7 +172,7 @@ class Machine:
         if total == 0:
             return
         grids = np.unravel_index(np.arange(total), out_extents) if out_extents else ()
-        variables = [np.asarray(g) for g in grids] + [None] * p.num_reduced
+        variables = [np.asarray(g) for g in grids] + [None] * p.num_reduced + [np.zeros(total, dtype=np.int64)] * p.num_dynamic
         if p.reduce_op == 0:
             value = self.run_value(0, p.value_code_length, variables)
         else:

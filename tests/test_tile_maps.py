@@ -439,3 +439,94 @@ def test_expand_on_an_empty_tensor():
     kernel(torch.empty((0,), device="cuda"))
     kernel = ninetoothed.make(_single_tensor_arrangement, _no_store_application, (Tensor(1),))
     kernel(torch.randn(100, device="cuda"))
+
+
+# ---- data-dependent level indices (tests/test_generation.py:72-115 of the reference) ----------
+
+
+def _scatter_rows_arrangement(input, indices, output):
+    input_arranged = input.tile((1, -1)).squeeze(1)
+    input_arranged.dtype = input_arranged.dtype.squeeze(0)
+    indices_arranged = indices.tile((1,))
+    output_arranged = output.tile((1, -1)).tile((-1, -1)).squeeze(0).expand((input_arranged.shape[0],))
+    output_arranged.dtype = output_arranged.dtype.squeeze(1)
+    output_arranged.dtype.dtype = output_arranged.dtype.dtype.squeeze(0)
+    return input_arranged, indices_arranged, output_arranged
+
+
+def _scatter_rows_application(input, index, output):
+    row = index
+
+    output[row] = input
+
+
+def _gather_rows_arrangement(table, indices, output):
+    table_arranged = table.tile((1, -1)).tile((-1, -1)).squeeze(0).expand((indices.shape[0],))
+    table_arranged.dtype = table_arranged.dtype.squeeze(1)
+    table_arranged.dtype.dtype = table_arranged.dtype.dtype.squeeze(0)
+    indices_arranged = indices.tile((1,))
+    output_arranged = output.tile((1, -1)).squeeze(1)
+    output_arranged.dtype = output_arranged.dtype.squeeze(0)
+    return table_arranged, indices_arranged, output_arranged
+
+
+def _gather_rows_application(table, index, output):
+    output = table[index] * 2  # noqa: F841
+
+
+def _scatter_kernel():
+    options = {"constexpr": True}
+    tensors = (Tensor(2, shape_options=options), Tensor(1, shape_options=options), Tensor(2, shape_options=options))
+    return ninetoothed.make(_scatter_rows_arrangement, _scatter_rows_application, tensors)
+
+
+def test_lowering_scatter_rows_by_loaded_index():
+    kernel = _scatter_kernel()
+    input = torch.randn(10, 128)
+    indices = torch.randperm(1024)[:10]
+    out = torch.zeros(1024, 128)
+    expected = out.clone()
+    _run_on_machine(kernel, (input, indices, out))
+    expected[indices] = input
+    assert torch.equal(out, expected)
+
+
+def test_lowering_out_of_range_indices_are_skipped():
+    kernel = _scatter_kernel()
+    input = torch.randn(4, 8)
+    indices = torch.tensor([3, -1, 20, 0])
+    out = torch.zeros(20, 8)
+    _run_on_machine(kernel, (input, indices, out))
+    expected = torch.zeros(20, 8)
+    expected[3], expected[0] = input[0], input[3]
+    assert torch.equal(out, expected)
+
+
+def test_lowering_gather_rows_by_loaded_index():
+    kernel = ninetoothed.make(_gather_rows_arrangement, _gather_rows_application, (Tensor(2), Tensor(1), Tensor(2)))
+    table = torch.randn(50, 24)
+    indices = torch.randint(0, 50, (17,))
+    out = torch.zeros(17, 24)
+    _run_on_machine(kernel, (table, indices, out))
+    assert torch.equal(out, table[indices] * 2)
+
+
+@gpu
+@pytest.mark.parametrize("interpret", ("0", "1"))
+def test_rows_by_loaded_index(interpret, monkeypatch):
+    monkeypatch.setenv("NT_MAP_INTERPRET", interpret)
+    kernel = _scatter_kernel()
+    input = torch.randn(10, 128, device="cuda")
+    indices = torch.randperm(1024, device="cuda")[:10]
+    out = torch.empty(1024, 128, device="cuda").normal_()
+    expected = out.clone()
+    kernel(input, indices, out)
+    _served_by_map(kernel)
+    expected[indices] = input
+    assert torch.equal(out, expected)
+    gather = ninetoothed.make(_gather_rows_arrangement, _gather_rows_application, (Tensor(2), Tensor(1), Tensor(2)))
+    table = torch.randn(5000, 96, device="cuda")
+    picks = torch.randint(0, 5000, (333,), device="cuda")
+    rows = torch.empty(333, 96, device="cuda")
+    gather(table, picks, rows)
+    assert torch.equal(rows, table[picks] * 2)
