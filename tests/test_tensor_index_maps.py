@@ -148,3 +148,22 @@ def test_conv2d_arrangement_matches_oracle_and_unfold(padding):
     im2col = columns.permute(0, 2, 1).reshape(n * p * q, c * r * s).numpy()
     mine = np.where(x_view.table >= 0, x_view.table + 1, 0)
     assert np.array_equal(mine, im2col)
+
+
+def test_simulate_arrangement_matches_the_reference_vectors():
+    # reference: tests/test_debugging.py:12-239 (addmm arrangement, m=3, n=4, k=5, 2x2x2 blocks):
+    # six source tensors followed by six target tensors
+    import functools
+
+    from ninetoothed_amd import programs
+    from ninetoothed_amd.debugging import simulate_arrangement
+    from tests.golden_vectors import load
+
+    vectors = load("debugging_vectors.json")
+    arrangement = functools.partial(programs.addmm.arrangement, BLOCK_SIZE_M=2, BLOCK_SIZE_N=2, BLOCK_SIZE_K=2)
+    tensors = (Tensor(shape=(3, 4)), Tensor(shape=(3, 5)), Tensor(shape=(5, 4)), Tensor(0), Tensor(0), Tensor(shape=(3, 4)))
+    sources, targets = simulate_arrangement(arrangement, tensors, device="cpu")
+    assert len(sources) == len(targets) == 6
+    for position in range(6):
+        assert np.array_equal(sources[position].numpy(), vectors[position]), position
+        assert np.array_equal(targets[position].numpy(), vectors[6 + position]), position
