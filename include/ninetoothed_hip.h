@@ -137,7 +137,7 @@ NineToothedResult launch_nt_softmax_config(NineToothedStream stream, int config,
  * >= 256 selects 256 query rows per workgroup, block_size_n <= 32 the 32-key
  * blocks with three workgroups per CU, block_size_n >= 64 the plain 64-key
  * loop; without hints non-causal calls run the software-pipelined 64-key loop
- * and causal calls the 32-key one.  K and V of one (batch, head) must span
+ * and causal calls the plain one.  K and V of one (batch, head) must span
  * less than 4 GiB. */
 NineToothedResult launch_nt_attention(NineToothedStream stream,
                                       NineToothedTensor q,
