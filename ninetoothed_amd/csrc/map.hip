@@ -681,8 +681,9 @@ hipFunction_t specialised_kernel(const NineToothedMapProgram &p) {
     hiprtcProgram program = nullptr;
     if (rtc.create(&program, source.c_str(), "nt_map_specialised.hip", 0, nullptr, nullptr) == HIPRTC_SUCCESS) {
         // same code generation switches as the rest of the library: gfx950, packed FP32 off
-        const char *options[] = {"--offload-arch=gfx950", "-O3", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
-        const hiprtcResult compiled = rtc.compile(program, 6, options);
+        // and no contraction: every operation is rounded on its own, as the value program says
+        const char *options[] = {"--offload-arch=gfx950", "-O3", "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+        const hiprtcResult compiled = rtc.compile(program, 7, options);
         if (compiled == HIPRTC_SUCCESS) {
             size_t size = 0;
             if (rtc.code_size(program, &size) == HIPRTC_SUCCESS && size > 0) {

@@ -530,3 +530,23 @@ def test_rows_by_loaded_index(interpret, monkeypatch):
     rows = torch.empty(333, 96, device="cuda")
     gather(table, picks, rows)
     assert torch.equal(rows, table[picks] * 2)
+
+
+def _mul_add_arrangement(lhs, rhs, output, block=block_size()):
+    return lhs.tile((block,)), rhs.tile((block,)), output.tile((block,))
+
+
+def _mul_add_application(lhs, rhs, output):
+    output = lhs * rhs + 1  # noqa: F841
+
+
+@gpu
+@pytest.mark.parametrize("interpret", ("0", "1"))
+def test_operations_are_rounded_one_by_one(interpret, monkeypatch):
+    # a multiplication followed by an addition must not be contracted into a fused multiply-add
+    monkeypatch.setenv("NT_MAP_INTERPRET", interpret)
+    kernel = ninetoothed.make(_mul_add_arrangement, _mul_add_application, (Tensor(1),) * 3)
+    lhs, rhs = torch.randn(100000), torch.randn(100000)
+    out = torch.empty(100000, device="cuda")
+    kernel(lhs.cuda(), rhs.cuda(), out)
+    assert torch.equal(out.cpu(), lhs * rhs + 1)
