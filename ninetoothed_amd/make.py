@@ -71,9 +71,11 @@ def make(
     :param arrangement: The arrangement of the tensors.
     :param application: The application of the tensors.
     :param tensors: The tensors.
-    :param caller: Who will call the compute kernel; only ``"torch"``.
+    :param caller: Who will call the compute kernel: ``"torch"``, or ``"hip"``
+        (alias ``"cuda"``) to package the kernel ahead of time as
+        ``<output_dir>/<kernel_name>.{h,c,so}`` exporting ``launch_<kernel_name>``.
     :param kernel_name: The name for the kernel.
-    :param output_dir: Unused (no files are generated for ``"torch"``).
+    :param output_dir: Where the packaged files go (``"hip"`` only).
     :param num_warps: Accepted for compatibility; wave counts belong to the
         hand-written kernels.
     :param num_stages: Accepted for compatibility; see ``num_warps``.
@@ -82,8 +84,12 @@ def make(
     :return: A handle to the compute kernel.
     """
 
+    if caller in ("hip", "cuda"):  # ahead-of-time packaging (the reference's `caller="cuda"`, src/ninetoothed/make.py:38-56)
+        from ninetoothed_amd import aot
+
+        return aot.package(arrangement, application, tensors, kernel_name, output_dir)
     if caller != "torch":
-        raise NotImplementedError("Only `caller=\"torch\"` is supported; ahead-of-time packaging is not part of this build.")
+        raise NotImplementedError(f"Unknown caller `{caller}`: use \"torch\" or \"hip\".")
     types = arrangement(*tensors)
     types = types if isinstance(types, tuple) else (types,)
     return Kernel(application, types, kernel_name=kernel_name)
