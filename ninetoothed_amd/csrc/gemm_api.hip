@@ -42,7 +42,8 @@ bool fast_accepts(const GemmProblem &q) {
     if (q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) return false;
     if (q.out_dtype != q.dtype) return false;
     if (q.m <= 0 || q.n <= 0 || q.k <= 0) return false;
-    if (q.m % BM || q.n % BN || q.k % BK) return false;
+    // any number of rows: rows past M read as zeros and are not stored; N and K must fit the tile
+    if (q.n % BN || q.k % BK) return false;
     if (q.sak != 1 || q.sbn != 1 || q.scn != 1) return false;
     if (q.sam % 8 || q.sbk % 8 || q.sam < q.k || q.sbk < q.n || q.scm < q.n) return false;
     if (((uintptr_t)q.a & 15) || ((uintptr_t)q.b & 15) || ((uintptr_t)q.c & 15) || q.scm % 8) return false;
@@ -67,7 +68,7 @@ void fill_params(GemmParams &p, const GemmProblem &q, int bm, int bn) {
     p.bias_stride_n = q.sin;
     p.alpha = q.alpha;
     p.beta = q.beta;
-    p.tiles_m = q.m / bm;
+    p.tiles_m = (q.m + bm - 1) / bm;
     p.tiles_n = q.n / bn;
     p.order = g_tile_order;
     p.bias_vector = q.bias != nullptr && q.sin == 1 && q.sim % 8 == 0 && ((uintptr_t)q.bias & 15) == 0;
@@ -245,7 +246,7 @@ int heuristic_choice(const GemmProblem &q, int bm, int bn, int bk) {
     for (const Rule &rule : rules) {
         const GemmInstance &inst = kInstances[rule.instance];
         if (!inst.accepts(q)) continue;
-        const int64_t tiles = (int64_t)(q.m / inst.bm) * (q.n / inst.bn);
+        const int64_t tiles = (int64_t)((q.m + inst.bm - 1) / inst.bm) * (q.n / inst.bn);
         if (tiles >= rule.min_tiles) return rule.instance;
     }
     return kInstances[0].accepts(q) ? 0 : -1;

@@ -191,7 +191,10 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     // (buffer resource on the tile panel, 32-bit lane offset, scalar K offset)
     __amdgpu_buffer_rsrc_t a_rsrc, b_rsrc;
     if constexpr (kLoad == 1) {
-        a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)a_base, 0, 0xffffffff, 0x00020000);
+        // the A descriptor ends with the last row of the matrix: rows of the tile past M read as zeros
+        const int64_t a_rows = min((int64_t)BM, (int64_t)p.m - m0);
+        const unsigned a_bytes = (unsigned)(((a_rows - 1) * p.lda + p.k) * 2);
+        a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)a_base, 0, a_bytes, 0x00020000);
         b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)b_base, 0, 0xffffffff, 0x00020000);
     }
     auto issue_loads = [&](auto stage_tag, int kt) {
@@ -385,6 +388,7 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
             vec8 v = *(const NT_LDS vec8 *)(slab + row * kRowBytes + phys * 16);
             const int grow = m0 + wave_m * kWaveM + ti * 32 + row;
             const int gcol = n0 + wave_n * kWaveN + chunk * 8;
+            if (grow >= p.m) continue;  // a partial last tile of rows
             if constexpr (kAddmm) {
                 // the matmul result was rounded to the element type; beta, alpha
                 // are fp32 scalars, so the combination happens in fp32

@@ -432,3 +432,40 @@ def test_attention_float32_tensors(seq_len, is_causal):
     # strided K / V (a transposed view) go through the same conversion
     k_view = k.transpose(1, 2).contiguous().transpose(1, 2)
     assert torch.allclose(_attention(q.cuda(), k_view.cuda(), v.cuda(), is_causal), expected, rtol=0.025, atol=0.025)
+
+
+@pytest.mark.parametrize("m", (1, 100, 1000, 4097))
+@pytest.mark.parametrize("addmm", (False, True))
+def test_gemm_any_number_of_rows_on_the_direct_to_lds_path(m, addmm):
+    # M need not be a multiple of the tile: rows past the end read as zeros and are not stored
+    from ninetoothed_amd import runtime
+
+    n, k = 1024, 512
+    a, b = _randn(m, k).cuda(), _randn(k, n, scale=0.1).cuda()
+    guard = torch.full((m + 64, n), 7.0, dtype=torch.float16, device="cuda")  # rows after the output must stay untouched
+    out = guard[:m]
+    lib = runtime.library()
+    names = runtime.gemm_config_names()
+    fp16 = runtime.DATA_TYPE_INDEX["fp16"]
+    null = runtime.ArgumentTensor.null()
+    if addmm:
+        input = _randn(m, n).cuda()
+        expected = torch.addmm(input, a, b, beta=0.5, alpha=2.0)
+        extra = (runtime.ArgumentTensor.from_torch_tensor(input), runtime.ArgumentTensor.from_scalar(0.5), runtime.ArgumentTensor.from_scalar(2.0))
+    else:
+        expected = torch.matmul(a, b)
+        extra = (null, null, null)
+    ran = 0
+    for config, name in enumerate(names):
+        if "lds-direct" not in name:
+            continue
+        out.fill_(float("nan"))
+        code = lib.launch_nt_gemm_config(
+            runtime.current_stream(), config, extra[0], runtime.ArgumentTensor.from_torch_tensor(a), runtime.ArgumentTensor.from_torch_tensor(b),
+            extra[1], extra[2], runtime.ArgumentTensor.from_torch_tensor(out), fp16, fp16,
+        )
+        assert code == 0, name
+        assert torch.allclose(out, expected, rtol=2e-2, atol=2e-2), name
+        assert bool((guard[m:] == 7.0).all()), name
+        ran += 1
+    assert ran >= 4
