@@ -3,11 +3,12 @@
 //
 // Fast path requirements (checked on the host before launch):
 //   A row-major with unit K stride, B row-major with unit N stride, C with unit
-//   N stride and the element type of A/B; M % BM == 0, N % BN == 0, K % BK == 0;
-//   row pitches and base addresses multiples of 16 bytes.
+//   N stride and the element type of A/B; any M (rows of the last tile past M
+//   read as zeros through the A buffer descriptor and are not stored),
+//   N % BN == 0, K % BK == 0; row pitches and base addresses multiples of 16 bytes.
 //
 // Data movement per workgroup and K step:
-//   HBM/L2 --global_load_lds (16 B per lane, no registers)--> LDS stage
+//   HBM/L2 --buffer_load ... lds (16 B per lane, no registers)--> LDS stage
 //   LDS --ds_read_b128 (A) / ds_read_b64_tr_b16 (B)--> MFMA operand registers
 // LDS tiles are XOR-swizzled at 16-byte granularity so both the row-wise A
 // reads and the transposing B reads spread over all 64 banks.

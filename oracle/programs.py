@@ -19,7 +19,7 @@ Arithmetic conventions restated from the kernels the reference generates:
 ``ntl.dot`` multiplies fp16/bf16 tiles exactly and accumulates in fp32;
 ``.to(dtype)`` and stores into a narrower tensor round to nearest even;
 a tile times a Python float keeps the tile's dtype, a tile times a run-time
-fp32 scalar promotes to fp32 (SURVEY of Triton's promotion rules:
+fp32 scalar promotes to fp32 (Triton promotion rules:
 ``language/semantic.py`` of triton 3.6, binary arithmetic type checks).
 
 Pinned (tests/test_oracle_programs.py) against the library routines the
