@@ -5,6 +5,7 @@ executed by hand-written gfx950 (MI355X) kernels.
 Public names follow the reference package (src/ninetoothed/__init__.py:1-44).
 """
 
+from ninetoothed_amd.build import build
 from ninetoothed_amd.dtype import (
     bfloat16,
     float16,
@@ -44,6 +45,7 @@ __all__ = [
     "UnsupportedProgram",
     "bfloat16",
     "block_size",
+    "build",
     "eval",
     "float16",
     "float32",

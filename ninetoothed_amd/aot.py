@@ -13,7 +13,7 @@ point of the recognised program with the element type and block sizes fixed at
 packaging time, and ``<kernel_name>.so`` is built from it and linked against
 ``libnt_hip.so``.
 
-Only the five recognised programs can be packaged: tile maps are lowered per
+Only the recognised programs (matmul, addmm, softmax, attention, conv2d) can be packaged: tile maps are lowered per
 call from the sizes of the arguments (``ninetoothed_amd.mapping``), which a C
 dispatcher cannot do.
 """
@@ -72,10 +72,30 @@ def _probe_environment(kernel, sizes):
     return env
 
 
+def _conv2d_sample_sizes(kernel, constexprs):
+    """Sample x[N,C,H,W], w[K,C,R,S], y[N,K,P,Q]: declared sizes where the tensors fix them."""
+
+    def declared(tensor, defaults):
+        return [int(size) if not hasattr(size, "is_name") else default for size, default in zip(tensor.source.shape, defaults)]
+
+    n, c, h, w = declared(kernel.types[0], (2, 8, 10, 12))
+    k, _, r, s = declared(kernel.types[1], (16, c, 3, 3))
+    pad_h, pad_w = int(constexprs.get("padding_h", 0)), int(constexprs.get("padding_w", 0))
+    return (n, c, h, w), (k, c, r, s), (n, k, h + 2 * pad_h - r + 1, w + 2 * pad_w - s + 1)
+
+
 def _check_structure(kernel, constexprs):
     """Runs the call-time arrangement analysis on sample sizes: the dispatcher forwards whole
     tensors, which is only right if the arrangement is the program's canonical one."""
     kind = kernel.kind
+    if kind == "matmul" and kernel.types[0].source.ndim == 4:
+        sizes = _conv2d_sample_sizes(kernel, constexprs)
+        env = _probe_environment(kernel, sizes)
+        env.update(constexprs)
+        result, info = recognition.analyze_gemm(kernel.types[0], kernel.types[1], kernel.types[2], env)
+        if result != "conv2d":
+            raise UnsupportedProgram("The arrangement is not the implicit-GEMM view of a convolution the packaged dispatcher forwards.")
+        return {"conv2d": True, "pad_h": info["pad_h"], "pad_w": info["pad_w"], **info["blocks"]}
     if kind in ("matmul", "addmm"):
         m, n, k = 96, 160, 224
         if kind == "matmul":
@@ -119,7 +139,9 @@ def _dispatcher_source(kernel, name, dtype, out_dtype, blocks):
     signature = f"NineToothedResult launch_{name}(NineToothedStream stream, {parameters})"
     p = kernel.parameters
     bm, bn, bk = (blocks.get(axis, 0) if blocks.get(axis, 0) > 1 else 0 for axis in ("m", "n", "k"))
-    if kernel.kind == "matmul":
+    if blocks.get("conv2d"):
+        body = f"return launch_nt_conv2d(stream, {p[0]}, {p[1]}, {p[2]}, {_ENUM_NAMES[dtype]}, {blocks['pad_h']}, {blocks['pad_w']}, {bm}, {bn}, {bk});"
+    elif kernel.kind == "matmul":
         body = f"return launch_nt_matmul(stream, {p[0]}, {p[1]}, {p[2]}, {_ENUM_NAMES[dtype]}, {_ENUM_NAMES[out_dtype]}, {bm}, {bn}, {bk});"
     elif kernel.kind == "addmm":
         body = f"return launch_nt_addmm(stream, {p[0]}, {p[1]}, {p[2]}, {p[3]}, {p[4]}, {p[5]}, {_ENUM_NAMES[dtype]}, {bm}, {bn}, {bk});"
@@ -143,8 +165,11 @@ def _dispatcher_source(kernel, name, dtype, out_dtype, blocks):
     return header, source
 
 
-def package(arrangement, application, tensors, kernel_name, output_dir, constexprs=None):
-    """Writes ``<kernel_name>.h/.c``, builds ``<kernel_name>.so`` and returns a handle."""
+def generate(arrangement, application, tensors, kernel_name, output_dir, constexprs=None, block_hints=True):
+    """Writes ``<kernel_name>.h`` and ``<kernel_name>.c`` and returns the analysed kernel.
+
+    With ``block_hints=False`` the dispatcher passes no block sizes, which leaves the choice of
+    the GEMM instance to the library (its heuristic table and tuning cache)."""
     from ninetoothed_amd.make import Kernel
 
     if kernel_name is None or output_dir is None:
@@ -153,6 +178,8 @@ def package(arrangement, application, tensors, kernel_name, output_dir, constexp
     types = types if isinstance(types, tuple) else (types,)
     kernel = Kernel(application, types, kernel_name=kernel_name)
     blocks = _check_structure(kernel, dict(constexprs or {}))
+    if not block_hints:
+        blocks = {name: value for name, value in blocks.items() if name not in ("m", "n", "k")}
     tensor_types = [t for t in kernel.types if not (t.ndim == 0 and not isinstance(t.dtype, Tensor))]
     dtype = _element_type(tensor_types[0], kernel.parameters[0])
     out_dtype = _element_type(tensor_types[-1], kernel.parameters[-1])
@@ -164,18 +191,30 @@ def package(arrangement, application, tensors, kernel_name, output_dir, constexp
     output_dir.mkdir(parents=True, exist_ok=True)
     (output_dir / f"{kernel_name}.h").write_text(header)
     (output_dir / f"{kernel_name}.c").write_text(source)
-    library = output_dir / f"{kernel_name}.so"
+    return kernel
+
+
+def compile_library(sources, library, include_dirs):
+    """Builds a shared library from C sources, linked against ``libnt_hip.so``."""
     compiler = shutil.which("gcc") or shutil.which("cc") or shutil.which("hipcc")
     if compiler is None:
         raise RuntimeError("No C compiler found to build the packaged kernel.")
     lib_dir = runtime.LIBRARY_PATH.parent
     command = [
-        compiler, "-shared", "-fPIC", "-O2", f"-I{INCLUDE_DIR}", f"-I{output_dir}", str(output_dir / f"{kernel_name}.c"),
+        compiler, "-shared", "-fPIC", "-O2", f"-I{INCLUDE_DIR}", *(f"-I{path}" for path in include_dirs), *map(str, sources),
         f"-L{lib_dir}", "-lnt_hip", f"-Wl,-rpath,{lib_dir}", "-o", str(library),
     ]
     result = subprocess.run(command, capture_output=True, text=True)
     if result.returncode != 0:
         raise RuntimeError("Building the packaged kernel failed:\n" + " ".join(command) + "\n" + result.stderr)
+    return library
+
+
+def package(arrangement, application, tensors, kernel_name, output_dir, constexprs=None):
+    """Writes ``<kernel_name>.h/.c``, builds ``<kernel_name>.so`` and returns a handle."""
+    kernel = generate(arrangement, application, tensors, kernel_name, output_dir, constexprs)
+    output_dir = pathlib.Path(output_dir)
+    library = compile_library([output_dir / f"{kernel_name}.c"], output_dir / f"{kernel_name}.so", [output_dir])
     return PackagedKernel(library, kernel_name, kernel)
 
 
@@ -195,17 +234,22 @@ class PackagedKernel:
         self._source = str(pathlib.Path(self.library_path).with_suffix(".c"))
 
     def __call__(self, *args):
-        import torch
-
         if len(args) != len(self._scalar):
             raise TypeError(f"`{self.kernel_name}` takes {len(self._scalar)} arguments but {len(args)} were given.")
-        marshalled = []
-        for arg, scalar in zip(args, self._scalar):
-            if scalar:
-                value = arg.item() if isinstance(arg, torch.Tensor) else arg
-                marshalled.append(runtime.ArgumentTensor.from_scalar(float(value) if isinstance(value, float) else int(value)))
-            else:
-                if not arg.is_cuda:
-                    raise RuntimeError("Packaged kernels run on the GPU only (there is no CPU path).")
-                marshalled.append(runtime.ArgumentTensor.from_torch_tensor(arg))
-        runtime.check(self._function(runtime.current_stream(), *marshalled))
+        runtime.check(self._function(runtime.current_stream(), *marshal(args, self._scalar)))
+
+
+def marshal(args, scalar):
+    """Torch tensors and Python scalars as the ``NineToothedTensor`` values a packaged launch function takes."""
+    import torch
+
+    marshalled = []
+    for arg, is_scalar in zip(args, scalar):
+        if is_scalar:
+            value = arg.item() if isinstance(arg, torch.Tensor) else arg
+            marshalled.append(runtime.ArgumentTensor.from_scalar(float(value) if isinstance(value, float) else int(value)))
+        else:
+            if not arg.is_cuda:
+                raise RuntimeError("Packaged kernels run on the GPU only (there is no CPU path).")
+            marshalled.append(runtime.ArgumentTensor.from_torch_tensor(arg))
+    return marshalled

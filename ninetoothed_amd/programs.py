@@ -217,3 +217,15 @@ class conv2d:
     application = matmul.application_with_cast
 
     tensors = staticmethod(lambda: (Tensor(4), Tensor(4, shape_options={"constexpr": True}), Tensor(4)))
+
+    @staticmethod
+    def premake(n=None, c=None, h=None, w=None, k=None, r=None, s=None, dtype=None, block_size_m=64, block_size_n=64, block_size_k=64):
+        """The unpadded convolution with sizes fixed or left open, for ``build`` (after the
+        reference's tests/test_conv2d.py:51-87)."""
+        arrangement = functools.partial(
+            conv2d.arrangement, enable_padding=False, BLOCK_SIZE_M=block_size_m, BLOCK_SIZE_N=block_size_n, BLOCK_SIZE_K=block_size_k
+        )
+        p = h - r + 1 if h is not None and r is not None else None
+        q = w - s + 1 if w is not None and s is not None else None
+        tensors = (Tensor(shape=(n, c, h, w), dtype=dtype), Tensor(shape=(k, c, r, s), dtype=dtype), Tensor(shape=(n, k, p, q), dtype=dtype))
+        return arrangement, matmul.application, tensors

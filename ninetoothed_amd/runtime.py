@@ -98,7 +98,7 @@ def library():
         if _library is None:
             if not LIBRARY_PATH.exists():
                 raise RuntimeError(
-                    f"{LIBRARY_PATH} is missing: build it with `python -m ninetoothed_amd.build` (needs hipcc). "
+                    f"{LIBRARY_PATH} is missing: build it with `python -m ninetoothed_amd.build_library` (needs hipcc). "
                     "There is no fallback path."
                 )
             lib = ctypes.CDLL(str(LIBRARY_PATH))
