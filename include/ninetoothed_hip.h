@@ -235,7 +235,8 @@ int nt_tune_cache_lookup(int dtype, int output_dtype, int m, int n, int k, int a
  *     them varies fastest across lanes), the rest the reduced positions;
  *     `num_dynamic` further variables take their value from the data
  *     (`output[row] = input` with `row` loaded from a tensor,
- *     tests/test_generation.py:72-115);
+ *     tests/test_generation.py:72-115; `x.source[rows, columns]` and
+ *     `ntl.load(x.source.data_ptr() + offsets)`, tests/test_clone.py:23-37);
  *   - index code (one segment per operand, and per `.offsets()` use) computes a
  *     flat element offset from the variables with + * // % by constants
  *     (src/ninetoothed/tensor.py:258-274, 462-471, 555-556) and checks
@@ -295,6 +296,11 @@ enum NineToothedMapValueOp {
 
 enum NineToothedMapReduceOp { NT_MAP_REDUCE_NONE, NT_MAP_REDUCE_MAX, NT_MAP_REDUCE_MIN, NT_MAP_REDUCE_SUM };
 
+/* How the value reaches the output element: a plain store, or an atomic add
+ * (`ntl.atomic_add(pointer, value)`, tests/test_data_ptr.py:17-18; 32 / 64 bit
+ * integers, float and double only). */
+enum NineToothedMapStoreOp { NT_MAP_STORE_ASSIGN, NT_MAP_STORE_ATOMIC_ADD };
+
 typedef struct {
     void *data;
     int32_t dtype;    /* NineToothedDataType */
@@ -306,7 +312,7 @@ typedef struct {
     int32_t num_vars;     /* enumerated variables: output elements, then reduced positions */
     int32_t num_reduced;
     int32_t num_dynamic;  /* variables num_vars .. num_vars + num_dynamic - 1 are set by NT_MAP_V_SETVAR */
-    int32_t reserved;
+    int32_t store_op;     /* NineToothedMapStoreOp */
     int64_t extents[NT_MAP_MAX_VARS];
     int32_t num_operands;
     int32_t output;              /* operand that is stored */

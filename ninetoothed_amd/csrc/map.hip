@@ -110,6 +110,18 @@ __device__ __forceinline__ void store_element(void *data, int dtype, int64_t off
     }
 }
 
+__device__ __forceinline__ void atomic_add_element(void *data, int dtype, int64_t offset, double v) {
+    switch (dtype) {
+        case NINETOOTHED_INT32: atomicAdd((int *)data + offset, (int)(int64_t)v); break;
+        case NINETOOTHED_UINT32: atomicAdd((unsigned int *)data + offset, (unsigned int)(int64_t)v); break;
+        case NINETOOTHED_INT64: atomicAdd((unsigned long long *)data + offset, (unsigned long long)(int64_t)v); break;
+        case NINETOOTHED_UINT64: atomicAdd((unsigned long long *)data + offset, (unsigned long long)v); break;
+        case NINETOOTHED_FLOAT32: atomicAdd((float *)data + offset, (float)v); break;
+        case NINETOOTHED_FLOAT64: atomicAdd((double *)data + offset, v); break;
+        default: break;
+    }
+}
+
 // the value as the reference would hold it in a tile of type `dtype`
 __device__ __forceinline__ double round_to(double v, int dtype) {
     switch (dtype) {
@@ -279,7 +291,10 @@ __global__ __launch_bounds__(kMapThreads) void map_kernel(const NineToothedMapPr
         const NineToothedMapOperand &out = p.operands[p.output];
         bool valid = true;
         const int64_t offset = run_index(p, out.segment, vars, valid);
-        if (valid) store_element(out.data, out.dtype, offset, value);
+        if (valid) {
+            if (p.store_op == NT_MAP_STORE_ATOMIC_ADD) atomic_add_element(out.data, out.dtype, offset, value);
+            else store_element(out.data, out.dtype, offset, value);
+        }
     }
 }
 
@@ -287,6 +302,13 @@ bool well_formed(const NineToothedMapProgram &p) {
     if (p.num_vars < 0 || p.num_vars > NT_MAP_MAX_VARS || p.num_reduced < 0 || p.num_reduced > p.num_vars) return false;
     if (p.num_dynamic < 0 || p.num_vars + p.num_dynamic > NT_MAP_MAX_VARS) return false;
     if (p.num_operands < 1 || p.num_operands > NT_MAP_MAX_OPERANDS || p.output < 0 || p.output >= p.num_operands) return false;
+    if (p.store_op != NT_MAP_STORE_ASSIGN && p.store_op != NT_MAP_STORE_ATOMIC_ADD) return false;
+    if (p.store_op == NT_MAP_STORE_ATOMIC_ADD) {
+        const int dtype = p.operands[p.output].dtype;
+        if (dtype != NINETOOTHED_INT32 && dtype != NINETOOTHED_UINT32 && dtype != NINETOOTHED_INT64 && dtype != NINETOOTHED_UINT64 &&
+            dtype != NINETOOTHED_FLOAT32 && dtype != NINETOOTHED_FLOAT64)
+            return false;
+    }
     if (p.num_segments < 1 || p.num_segments > NT_MAP_MAX_SEGMENTS) return false;
     if (p.value_code_length < 0 || p.value_code_length > NT_MAP_MAX_VALUE_CODE) return false;
     if (p.reduce_split < 0 || p.reduce_split > p.value_code_length) return false;
@@ -421,6 +443,13 @@ std::string store_stmt(const std::string &pointer, int dtype, const std::string 
         case NINETOOTHED_UINT64: return target + " = (" + c_type(dtype) + ")(" + v + ");";
         default: return target + " = (" + c_type(dtype) + ")(long long)(" + v + ");";
     }
+}
+
+std::string atomic_add_stmt(const std::string &pointer, int dtype, const std::string &offset, const std::string &v) {
+    const char *type = dtype == NINETOOTHED_INT32 ? "int" : dtype == NINETOOTHED_UINT32 ? "unsigned int" : dtype == NINETOOTHED_FLOAT32 ? "float"
+                       : dtype == NINETOOTHED_FLOAT64 ? "double" : "unsigned long long";
+    const bool integer = dtype != NINETOOTHED_FLOAT32 && dtype != NINETOOTHED_FLOAT64 && dtype != NINETOOTHED_UINT64;
+    return std::string("atomicAdd((") + type + " *)" + pointer + " + " + offset + ", (" + type + ")" + (integer ? "(long long)" : "") + "(" + v + "));";
 }
 
 // Translates the programs into HIP source.  `counter` numbers temporaries.
@@ -615,7 +644,10 @@ struct MapCodegen {
         const NineToothedMapOperand &target = p.operands[p.output];
         out << indent << "bool store_ok = true;\n";
         const std::string offset = index_segment(target.segment, "store_ok");
-        out << indent << "if (store_ok) " << store_stmt("a.data[" + std::to_string(p.output) + "]", target.dtype, offset, result) << "\n";
+        const std::string pointer = "a.data[" + std::to_string(p.output) + "]";
+        out << indent << "if (store_ok) "
+            << (p.store_op == NT_MAP_STORE_ATOMIC_ADD ? atomic_add_stmt(pointer, target.dtype, offset, result) : store_stmt(pointer, target.dtype, offset, result))
+            << "\n";
         out << "    }\n}\n";
         return out.str();
     }

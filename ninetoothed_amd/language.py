@@ -55,6 +55,9 @@ _FUNCTIONS = (
     "cos",
     "floor",
     "ceil",
+    "load",
+    "store",
+    "atomic_add",
 )
 
 for _name in _FUNCTIONS:

@@ -7,9 +7,14 @@ recognised ones (matmul, addmm, softmax, attention, conv2d) run here if their
 application is a *tile map*: every store assigns, to a tile of an output
 parameter, an expression over whole tiles of the other parameters, call-time
 scalars and constants, with at most one ``ntl.max`` / ``ntl.min`` / ``ntl.sum``
-reduction (the programs of the reference's tests/test_add.py, test_clone.py
-(first application), test_pad.py, test_pow.py, test_dropout.py,
-test_max_pool2d.py, test_generation.py:139-151).
+reduction (the programs of the reference's tests/test_add.py, test_clone.py,
+test_pad.py, test_pow.py, test_dropout.py, test_max_pool2d.py,
+test_generation.py:139-151).  Besides tiles, a value may be read from, and a
+store may go to, elements of a whole tensor picked by computed indices
+(``x.source[rows, columns]``, masked to the tensor's bounds as
+src/ninetoothed/tensor.py:571-584 does) or by a raw pointer
+(``ntl.load / ntl.store / ntl.atomic_add`` on ``x.source.data_ptr() + offsets``,
+unmasked) -- tests/test_clone.py:23-37 and tests/test_data_ptr.py:17-18.
 
 Two lowerings happen per call signature:
 
@@ -30,7 +35,7 @@ import ctypes
 from ninetoothed_amd import runtime
 from ninetoothed_amd.affine import Affine
 from ninetoothed_amd.recognition import Operand, UnsupportedProgram
-from ninetoothed_amd.tracing import ElementType, Node, ScalarParam, TensorRef
+from ninetoothed_amd.tracing import ElementType, Node, ScalarParam, SourceDim, SourceStride, TensorRef
 
 MAX_OPERANDS = 8
 MAX_VARS = 16
@@ -60,7 +65,7 @@ class MapProgram(ctypes.Structure):
         ("num_vars", ctypes.c_int32),
         ("num_reduced", ctypes.c_int32),
         ("num_dynamic", ctypes.c_int32),
-        ("reserved", ctypes.c_int32),
+        ("store_op", ctypes.c_int32),
         ("extents", ctypes.c_int64 * MAX_VARS),
         ("num_operands", ctypes.c_int32),
         ("output", ctypes.c_int32),
@@ -140,6 +145,74 @@ def _kwargs(node):
         else:
             positional.append(arg)
     return positional, named
+
+
+class _RawOperand:
+    """A whole tensor addressed by computed indices (``x.source[i, j]``) or by a computed
+    element offset (a raw pointer): ``terms`` lists (dynamic variable, stride, size or None)."""
+
+    empty = False
+
+    def __init__(self, tensor):
+        self.tensor = tensor
+        self.terms = []
+
+
+def _affine_names(expr):
+    """The index variables an affine index expression depends on."""
+    names = set()
+    for atom, coef in expr.terms.items():
+        if coef == 0:
+            continue
+        if atom[0] == "var":
+            names.add(atom[1])
+        else:
+            names |= _affine_names(Affine.from_key(atom[1]))
+    return names
+
+
+def _split_pointer(expr):
+    """``x.source.data_ptr() + offsets`` -> (parameter of x, offsets in elements)."""
+    found = []
+
+    def strip(item):
+        if isinstance(item, Node) and item.op == "data_ptr":
+            found.append(item.args[0].param)
+            return None
+        if isinstance(item, Node) and item.op == "add":
+            a, b = strip(item.args[0]), strip(item.args[1])
+            if a is None or b is None:
+                return b if a is None else a
+            return Node("add", a, b)
+        return item
+
+    rest = strip(expr)
+    if len(found) != 1:
+        raise UnsupportedProgram("A pointer must be `tensor.source.data_ptr()` plus element offsets.")
+    return found[0], 0 if rest is None else rest
+
+
+_REDUCTIONS = ("max", "min", "sum")
+
+
+def _first_tile_ref(value):
+    """The first tile a value is built from outside of reductions: it fixes the shape of a store
+    that goes through computed indices or a pointer."""
+    if isinstance(value, Node):
+        if value.op in _REDUCTIONS:
+            return None
+        if value.op in ("load", "offsets") and isinstance(value.args[0], TensorRef):
+            return value.args[0]
+        for arg in value.args:
+            found = _first_tile_ref(arg)
+            if found is not None:
+                return found
+    elif isinstance(value, (tuple, list)):
+        for item in value:
+            found = _first_tile_ref(item)
+            if found is not None:
+                return found
+    return None
 
 
 class _Lowering:
@@ -270,10 +343,30 @@ class _Lowering:
                 return "i32" if -(2**31) <= arg < 2**31 else "i64"
             self.round("fp32")
             return "fp32"
+        if isinstance(value, (SourceDim, SourceStride)):
+            source = self.types[value.param].source
+            name = source.size_string(value.dim) if isinstance(value, SourceDim) else source.stride_string(value.dim)
+            self.emit("CONST", self.constant(int(self.env[name])))
+            return _LITERAL_INT
         if not isinstance(value, Node):
             raise UnsupportedProgram(f"A value of type `{type(value).__name__}` cannot be stored by the element-wise executor.")
 
         op = value.op
+        if op == "load" and not isinstance(value.args[0], TensorRef):  # `ntl.load(pointer)`
+            positional, named = _kwargs(value)
+            if len(positional) != 1 or named:
+                raise UnsupportedProgram("`ntl.load` of a pointer takes no mask here; index `tensor.source[...]` for a masked load.")
+            param, offset = _split_pointer(positional[0])
+            slot = self.raw_access(param, None, dims, inside_reduction, element_offset=offset)
+            self.emit("LOAD", slot)
+            return self.dtype_tag(param)
+        if op == "source_at":
+            source, indices = value.args
+            slot = self.raw_access(source.param, indices, dims, inside_reduction)
+            self.emit("LOAD", slot)
+            return self.dtype_tag(source.param)
+        if op == "index":
+            return self.lower_oriented_offsets(value, dims, inside_reduction)
         if op == "load":
             ref = value.args[0]
             self._check_ref(ref)
@@ -395,6 +488,60 @@ class _Lowering:
             return term
         raise UnsupportedProgram(f"`{op}` is not an element-wise operation this build can execute.")
 
+    def lower_oriented_offsets(self, value, dims, inside_reduction):
+        """``x.offsets(d)[:, None]``: the indices along source dimension ``d`` laid along one
+        dimension of the tile (src/ninetoothed/generation.py:212-230).  Values are computed per
+        tile element here, so this is the plain ``offsets(d)`` provided that index really only
+        varies along the dimension the subscript names."""
+        base, keys = value.args
+        plain = isinstance(base, Node) and base.op == "offsets" and base.args[1] is not None
+        if not plain or not all(key is None or key == slice(None) for key in keys):
+            raise UnsupportedProgram("Only `.offsets(dim)` can be subscripted, with `:` and `None`.")
+        along = [position for position, key in enumerate(keys) if key is not None]
+        if len(along) != 1 or len(keys) != len(dims):
+            raise UnsupportedProgram("A subscript of `.offsets(dim)` needs one `:` and as many entries as the tile has dimensions.")
+        ref, dim = base.args
+        self._check_ref(ref)
+        slot = self.bind_ref(ref, dims, inside_reduction)
+        _, operand = self.operands[slot]
+        binding = self.bindings[slot]
+        allowed = {dims[along[0]]} | set(self.grid) | set(self.dynamic_vars)
+        for name in _affine_names(operand.indices[dim]):
+            if binding.get(name) not in allowed and operand.extents.get(name, 1) != 1:
+                raise UnsupportedProgram("`.offsets(dim)` varies along another tile dimension than the one its subscript names.")
+        self.emit("OFFSET", self.segment(slot, "offsets", dim))
+        return "i32"
+
+    def raw_access(self, param, indices, dims, inside_reduction, element_offset=None):
+        """Registers an operand addressed by computed values; emits the code that computes them."""
+        slot = len(self.operands)
+        if slot >= MAX_OPERANDS:
+            raise UnsupportedProgram("Too many tensor operands for the element-wise executor.")
+        tensor = self.types[param]
+        if tensor.ndim == 0 and not hasattr(tensor.dtype, "ndim"):
+            raise UnsupportedProgram("Scalars have no elements to address.")
+        raw = _RawOperand(tensor)
+        self.operands.append((param, raw))
+        self.bindings[slot] = {}
+
+        def dynamic(value, size):
+            var = self.new_var(max(int(size), 1) if size is not None else 1)
+            self.dynamic_vars.append(var)
+            self.lower(value, dims, inside_reduction)
+            self.emit("SETVAR", var)
+            return var
+
+        source = tensor.source
+        if element_offset is not None:
+            raw.terms.append((dynamic(element_offset, None), 1, None))
+        else:
+            if len(indices) != source.ndim:
+                raise UnsupportedProgram("A source tensor needs one index per dimension.")
+            for dim, index in enumerate(indices):
+                size = int(self.env[source.size_string(dim)])
+                raw.terms.append((dynamic(index, size), int(self.env[source.stride_string(dim)]), size))
+        return slot
+
     def new_var_deferred(self):
         self.var_extent.append(None)
         return len(self.var_extent) - 1
@@ -404,7 +551,7 @@ class _Lowering:
 
         def visit(item):
             if isinstance(item, Node):
-                if item.op == "load":
+                if item.op == "load" and isinstance(item.args[0], TensorRef):
                     ref = item.args[0]
                     tensor = self.types[ref.param]
                     ranks.add(tensor.dtype.ndim if hasattr(tensor.dtype, "ndim") else 0)
@@ -449,7 +596,7 @@ class _Lowering:
 
     def _has_load(self, value):
         if isinstance(value, Node):
-            return value.op == "load" or any(self._has_load(arg) for arg in value.args)
+            return (value.op == "load" and isinstance(value.args[0], TensorRef)) or any(self._has_load(arg) for arg in value.args)
         if isinstance(value, (tuple, list)):
             return any(self._has_load(item) for item in value)
         return False
@@ -484,7 +631,18 @@ class _Lowering:
             _, operand = self.operands[slot]
             binding = self.bindings[slot]
             begins.append(len(code))
-            if kind == "access":
+            if kind == "raw":
+                for var, _, size in operand.terms:
+                    if size is not None:
+                        code.append(I_VAR | (order[var] << 8))
+                        code.append(I_CHECK | (const(size) << 8))
+                code.append(I_CONST | (const(0) << 8))
+                for var, stride, _ in operand.terms:
+                    code.append(I_VAR | (order[var] << 8))
+                    if stride != 1:
+                        code.append(I_MULC | (const(stride) << 8))
+                    code.append(I_ADD)
+            elif kind == "access":
                 # indices that come from the data are range-checked: an element outside its level
                 # is treated like a masked one (the reference would access out of bounds)
                 for name, var in binding.items():
@@ -514,20 +672,45 @@ def build(program_store, types, args, env, dtype_tag, data_ptr):
 
     ref, value = program_store
     lowering = _Lowering(types, args, env, dtype_tag)
-    lowering._check_ref(ref)
-    out_slot = lowering.operand(ref.param, ref.level)
-    _, out_operand = lowering.operands[out_slot]
-    tile_names = out_operand.names[ref.level] if len(out_operand.names) > ref.level else []
-    out_dims = [lowering.new_var(out_operand.extents[name]) for name in tile_names]
-    lowering.bind_ref(ref, out_dims, False)
-    result = lowering.lower(value, out_dims, False)
-    out_dtype = dtype_tag(ref.param)
-    if result != out_dtype:
-        lowering.emit("ROUND", runtime.DATA_TYPE_INDEX[out_dtype])
+    store_op = 0
+    if isinstance(ref, TensorRef):
+        lowering._check_ref(ref)
+        out_slot = order_slot = lowering.operand(ref.param, ref.level)
+        _, out_operand = lowering.operands[out_slot]
+        tile_names = out_operand.names[ref.level] if len(out_operand.names) > ref.level else []
+        out_dims = [lowering.new_var(out_operand.extents[name]) for name in tile_names]
+        lowering.bind_ref(ref, out_dims, False)
+        result = lowering.lower(value, out_dims, False)
+        out_dtype = dtype_tag(ref.param)
+        if result != out_dtype:
+            lowering.emit("ROUND", runtime.DATA_TYPE_INDEX[out_dtype])
+    else:
+        # a store through computed indices or a pointer: the first tile of the expression gives the shape
+        anchor = _first_tile_ref((ref.args, value))
+        order_slot, out_dims = None, []
+        if anchor is not None:
+            lowering._check_ref(anchor)
+            order_slot = lowering.operand(anchor.param, anchor.level)
+            _, anchor_operand = lowering.operands[order_slot]
+            tile_names = anchor_operand.names[anchor.level] if len(anchor_operand.names) > anchor.level else []
+            out_dims = [lowering.new_var(anchor_operand.extents[name]) for name in tile_names]
+            lowering.bind_ref(anchor, out_dims, False)
+        if ref.op == "source_at":
+            out_param, indices, offset = ref.args[0].param, ref.args[1], None
+        else:
+            (out_param, offset), indices = _split_pointer(ref.args[0]), None
+            store_op = 1 if ref.op == "pointer_atomic_add" else 0
+        result = lowering.lower(value, out_dims, False)
+        if lowering.grid is None:
+            raise UnsupportedProgram("The stored value is not built from any arranged tensor.")
+        out_dtype = dtype_tag(out_param)
+        if result != out_dtype:
+            lowering.emit("ROUND", runtime.DATA_TYPE_INDEX[out_dtype])
+        out_slot = lowering.raw_access(out_param, indices, out_dims, False, element_offset=offset)
     if lowering.reduce is None:
         lowering.reduce_split = len(lowering.value_code)
-    for slot in range(len(lowering.operands)):
-        lowering.segment(slot, "access")
+    for slot, (_, operand) in enumerate(lowering.operands):
+        lowering.segment(slot, "raw" if isinstance(operand, _RawOperand) else "access")
     if any(operand.empty for _, operand in lowering.operands):
         return None
     if any(extent is None for extent in lowering.var_extent):
@@ -538,12 +721,12 @@ def build(program_store, types, args, env, dtype_tag, data_ptr):
     reduced = list(lowering.reduced_vars)
     dynamic = list(lowering.dynamic_vars)
     outer = [v for v in range(len(lowering.var_extent)) if v not in reduced and v not in dynamic]
-    out_binding = lowering.bindings[out_slot]
-    offset = out_operand.offset()
     stride_of = {}
-    for name, var in out_binding.items():
-        stride_of[var] = abs(offset.coef(name)) if offset.is_linear() else None
-    if all(stride_of.get(v) is not None for v in outer):
+    if order_slot is not None:
+        offset = lowering.operands[order_slot][1].offset()
+        for name, var in lowering.bindings[order_slot].items():
+            stride_of[var] = abs(offset.coef(name)) if offset.is_linear() else None
+    if order_slot is not None and all(stride_of.get(v) is not None for v in outer):
         outer.sort(key=lambda v: (-(stride_of[v] or 1 << 62) if lowering.var_extent[v] > 1 else -(1 << 62), v))
     order = {old: new for new, old in enumerate(outer + reduced + dynamic)}
     # SETVAR words were emitted with provisional ids: renumber them like the index code
@@ -565,12 +748,13 @@ def build(program_store, types, args, env, dtype_tag, data_ptr):
     program.num_dynamic = len(dynamic)
     for old, new in order.items():
         program.extents[new] = lowering.var_extent[old]
+    program.store_op = store_op
     program.num_operands = len(lowering.operands)
     program.output = out_slot
     for slot, (param, operand) in enumerate(lowering.operands):
         program.operands[slot].data = data_ptr(param)
         program.operands[slot].dtype = runtime.DATA_TYPE_INDEX[dtype_tag(param)]
-        program.operands[slot].segment = lowering.segment_slot[(slot, "access", None)]
+        program.operands[slot].segment = lowering.segment_slot[(slot, "raw" if isinstance(operand, _RawOperand) else "access", None)]
         program.operands[slot].other = _other_value(operand.tensor)
     program.num_segments = len(begins)
     for index, begin in enumerate(begins):
@@ -602,6 +786,10 @@ def check_application(program):
     executor handles (sizes are checked later, per call)."""
 
     for ref, value in program.stores:
+        if isinstance(ref, Node) and ref.op in ("source_at", "pointer_store", "pointer_atomic_add"):
+            _scan(ref.args)
+            _scan(value)
+            continue
         if not isinstance(ref, TensorRef) or ref.level not in (1, 2) or not ref.is_tile:
             raise UnsupportedProgram("Stores must assign whole tiles one or two levels below the launch grid.")
         _scan(ref.indices)
@@ -612,7 +800,7 @@ def _scan(value):
     if isinstance(value, Node):
         known = (
             set(_BINARY) | set(_COMPARE) | set(_LOGICAL) | set(_UNARY_SAME) | set(_UNARY_FLOAT) | set(REDUCE)
-            | {"load", "offsets", "pos", "not", "where", "cast", "rand", "kwarg"}
+            | {"load", "offsets", "pos", "not", "where", "cast", "rand", "kwarg", "index", "source_at", "data_ptr"}
         )
         if value.op not in known:
             raise UnsupportedProgram(f"`{value.op}` is not an element-wise operation this build can execute.")

@@ -129,6 +129,15 @@ class SourceDim:
         self.param, self.dim = param, dim
 
 
+class SourceStride:
+    """The stride (in elements) of one dimension of a parameter's source tensor."""
+
+    __slots__ = ("param", "dim")
+
+    def __init__(self, param, dim):
+        self.param, self.dim = param, dim
+
+
 class ElementType:
     """The element type of a parameter's source tensor."""
 
@@ -172,6 +181,10 @@ def _digest_of(value):
         return f"dim[{value.param},{value.level},{value.dim}]"
     if isinstance(value, SourceDim):
         return f"srcdim[{value.param},{value.dim}]"
+    if isinstance(value, SourceStride):
+        return f"srcstride[{value.param},{value.dim}]"
+    if isinstance(value, SourceRef):
+        return f"source[{value.param}]"
     if isinstance(value, ElementType):
         return f"elemtype[{value.param}]"
     if isinstance(value, LoopVar):
@@ -378,6 +391,9 @@ class Tracer:
                 self._assign(element, item, frame)
         elif isinstance(target, ast.Subscript):
             ref = self._eval(_as_load(target), frame)
+            if isinstance(ref, Node) and ref.op == "source_at":
+                self.stores.append((ref, self._value(value)))
+                return
             if not isinstance(ref, TensorRef) or not ref.is_tile:
                 raise TracingError("Only tiles of tensor parameters can be assigned through a subscript.")
             self.stores.append((ref, self._value(value)))
@@ -567,6 +583,8 @@ class Tracer:
                 return _SourceShape(base.param, self.types[base.param].source.ndim)
             if attr == "ndim":
                 return self.types[base.param].source.ndim
+            if attr in ("data_ptr", "stride"):
+                return _BoundMethod(base, attr)
             raise TracingError(f"`.source` has no attribute `{attr}`.")
         if isinstance(base, Node):
             if attr == "to":
@@ -593,6 +611,8 @@ class Tracer:
             if len(keys) != base.tensor.ndim:
                 raise TracingError(f"A level with {base.tensor.ndim} dimensions needs {base.tensor.ndim} indices, got {len(keys)}.")
             return TensorRef(base.param, base.tensor.dtype, base.level + 1, base.indices + tuple(self._value(k) for k in keys))
+        if isinstance(base, SourceRef):  # `x.source[rows, columns]`: elements of the whole tensor by index
+            return Node("source_at", base, self._source_indices(base, key))
         if isinstance(base, _SourceShape):
             if not isinstance(key, int):
                 raise TracingError("Source shapes are indexed with integer constants.")
@@ -606,6 +626,13 @@ class Tracer:
             return base[key]
         raise TracingError("Unsupported subscript in an application.")
 
+    def _source_indices(self, source, key):
+        keys = key if isinstance(key, tuple) else (key,)
+        ndim = self.types[source.param].source.ndim
+        if len(keys) != ndim:
+            raise TracingError(f"A source tensor with {ndim} dimensions needs {ndim} indices, got {len(keys)}.")
+        return tuple(self._value(k) for k in keys)
+
     def _eval_Call(self, node, frame):
         func = self._eval(node.func, frame)
         args = [self._eval(arg, frame) for arg in node.args]
@@ -613,6 +640,12 @@ class Tracer:
         if any(keyword.arg is None for keyword in node.keywords):
             raise TracingError("`**kwargs` is not supported in an application.")
 
+        if language.is_function(func) and func.name in ("store", "atomic_add"):
+            # `ntl.store(pointer, value)` / `ntl.atomic_add(pointer, value)`: a store through a raw pointer
+            if len(args) != 2 or kwargs:
+                raise TracingError(f"`ntl.{func.name}` takes a pointer and a value.")
+            self.stores.append((Node("pointer_" + func.name, self._value(args[0])), self._value(args[1])))
+            return None
         if language.is_function(func):
             items = tuple(self._value(arg) for arg in args)
             named = tuple(sorted((name, self._value(value)) for name, value in kwargs.items()))
@@ -645,6 +678,14 @@ class Tracer:
             if not isinstance(dim, int):
                 raise TracingError("`.offsets(dim)` needs an integer constant.")
             return Node("offsets", base, dim % source_ndim)
+        if name == "data_ptr":
+            if not isinstance(base, SourceRef) or args or kwargs:
+                raise TracingError("`.data_ptr()` applies to `tensor.source`.")
+            return Node("data_ptr", base)
+        if name == "stride":
+            if not isinstance(base, SourceRef) or len(args) != 1 or not isinstance(args[0], int):
+                raise TracingError("`.source.stride(dim)` needs an integer constant.")
+            return SourceStride(base.param, args[0] % self.types[base.param].source.ndim)
         raise TracingError(f"Method `{name}` is not supported in an application.")
 
     def _inline(self, func, call, args, kwargs, frame):

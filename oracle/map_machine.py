@@ -195,6 +195,10 @@ class Machine:
         value = np.broadcast_to(value, valid.shape)
         tag = runtime.DATA_TYPES[out.dtype]
         if tag.startswith("fp") or tag == "bf16":
-            target[offset[valid]] = value[valid].astype(target.dtype)
+            stored = value[valid].astype(target.dtype)
         else:
-            target[offset[valid]] = np.trunc(value[valid]).astype(np.int64).astype(target.dtype)
+            stored = np.trunc(value[valid]).astype(np.int64).astype(target.dtype)
+        if p.store_op == 1:  # atomic add: every output element adds its value
+            np.add.at(target, offset[valid], stored)
+        else:
+            target[offset[valid]] = stored

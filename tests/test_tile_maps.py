@@ -550,3 +550,104 @@ def test_operations_are_rounded_one_by_one(interpret, monkeypatch):
     out = torch.empty(100000, device="cuda")
     kernel(lhs.cuda(), rhs.cuda(), out)
     assert torch.equal(out.cpu(), lhs * rhs + 1)
+
+
+# ---- elements of whole tensors by computed indices / raw pointers -----------------------------
+# (the other three applications of the reference's tests/test_clone.py:23-37 and the atomic sum of
+#  tests/test_data_ptr.py:11-18)
+
+
+def _clone_by_pointer(input, output):
+    output = ntl.load(  # noqa: F841
+        input.source.data_ptr() + input.offsets(0)[:, None] * input.source.stride(0) + input.offsets(1)[None, :] * input.source.stride(1)
+    )
+
+
+def _clone_by_source_load(input, output):
+    output = input.source[input.offsets(0)[:, None], input.offsets(1)[None, :]]  # noqa: F841
+
+
+def _clone_by_source_store(input, output):
+    output.source[output.offsets(0)[:, None], output.offsets(1)[None, :]] = input
+
+
+_CLONES = (_clone_by_pointer, _clone_by_source_load, _clone_by_source_store)
+
+
+def _transposed_gather(input, output):
+    output = input.source[input.offsets(0)[None, :], input.offsets(1)[:, None]]  # noqa: F841
+
+
+def _sum_arrangement(input, output, BLOCK_SIZE=1024):
+    input_arranged = input.tile((BLOCK_SIZE,))
+    return input_arranged, output.tile((-1,)).expand(input_arranged.shape)
+
+
+def _sum_application(input, output):
+    ntl.atomic_add(output.source.data_ptr(), ntl.sum(input))
+
+
+def _strided_matrix(rows, cols, row_stride, col_stride, device="cpu"):
+    storage = torch.randn(rows * row_stride, device=device)
+    return torch.as_strided(storage, (rows, cols), (row_stride, col_stride))
+
+
+@pytest.mark.parametrize("application", _CLONES)
+def test_lowering_clone_through_indices_and_pointers(application):
+    kernel = ninetoothed.make(clone_arrangement, application, (Tensor(2), Tensor(2)))
+    assert kernel.kind == "map"
+    input = _strided_matrix(41, 28, 30, 1)
+    out = torch.full((41, 28), float("nan"))
+    _run_on_machine(kernel, (input, out))
+    assert torch.equal(out, input)
+
+
+def test_lowering_rejects_offsets_laid_along_the_wrong_dimension():
+    def arrangement(input, output):
+        return input.tile((8, 8)), output.tile((8, 8))
+
+    kernel = ninetoothed.make(arrangement, _transposed_gather, (Tensor(2), Tensor(2)))
+    with pytest.raises(UnsupportedProgram):
+        _run_on_machine(kernel, (torch.randn(16, 16), torch.empty(16, 16)))
+
+
+def test_lowering_atomic_sum_through_a_pointer():
+    kernel = ninetoothed.make(_sum_arrangement, _sum_application, (Tensor(1), Tensor(1, shape_options={"constexpr": True})))
+    input = torch.randn(5000, dtype=torch.float64)
+    out = torch.zeros(1, dtype=torch.float64)
+    _run_on_machine(kernel, (input, out))
+    # one partial sum per tile of 1024, added in tile order
+    expected = sum(float(chunk.sum()) for chunk in input.split(1024))
+    assert abs(out.item() - expected) < 1e-9
+    assert abs(out.item() - input.sum().item()) < 1e-9
+
+
+@gpu
+@pytest.mark.parametrize("interpret", ("0", "1"))
+@pytest.mark.parametrize("application", _CLONES)
+def test_clone_through_indices_and_pointers(application, interpret, monkeypatch):
+    """tests/test_clone.py:55-69 of the reference: a 641 x 280 matrix with strides (700, 300)."""
+    monkeypatch.setenv("NT_MAP_INTERPRET", interpret)
+    kernel = ninetoothed.make(clone_arrangement, application, (Tensor(2), Tensor(2)))
+    input = torch.empty_strided((641, 280), (700, 300), device="cuda")
+    input.copy_(torch.randn(641, 280))
+    out = torch.full((641, 280), float("nan"), device="cuda")
+    kernel(input, out)
+    _served_by_map(kernel)
+    assert torch.equal(out, input)
+
+
+@gpu
+@pytest.mark.parametrize("interpret", ("0", "1"))
+def test_atomic_sum_through_a_pointer(interpret, monkeypatch):
+    """tests/test_data_ptr.py:34-42 of the reference."""
+    monkeypatch.setenv("NT_MAP_INTERPRET", interpret)
+    kernel = ninetoothed.make(_sum_arrangement, _sum_application, (Tensor(1), Tensor(1, shape_options={"constexpr": True})))
+    input = torch.randn(64180, device="cuda")
+    for _ in range(2):
+        out = torch.zeros(1, device="cuda")
+        kernel(input, out)
+        assert torch.allclose(out[0], torch.sum(input))
+    counts = torch.zeros(1, dtype=torch.int32, device="cuda")
+    kernel(torch.ones(64180, dtype=torch.int32, device="cuda"), counts)
+    assert counts.item() == 64180
