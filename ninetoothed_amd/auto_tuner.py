@@ -72,3 +72,106 @@ def tune(input, mat1, mat2, beta, alpha, output, dtype, out_dtype, iters=5):
     except OSError:
         pass  # a read-only home directory only costs the persistence
     return best.value, best_ms.value
+
+
+class AutoTuner:
+    """Picks the fastest of several callables per argument signature and keeps the timings on
+    disk, in the files the reference's ``AutoTuner`` writes (src/ninetoothed/auto_tuner.py:11-118):
+
+    * ``<sha256(str(key))>.json`` per callable: ``{argument key: milliseconds}``;
+    * ``<sha256(str(tuple(keys)))>.json`` for the tuner: ``{argument key: [milliseconds per callable]}``
+      (plus one empty object per callable key, as the reference initialises it).
+
+    An argument key is ``"tensor(shape=(..), dtype=float16), 3, name=value"``.  A callable that
+    raises :class:`runtime.KernelLaunchError` is timed as infinity.  Timing is wall clock around
+    repeated calls, each batch closed by a device synchronisation when a GPU is in use.
+    """
+
+    def __init__(self, funcs, keys, cache_dir=None, repetitions=5):
+        import json
+
+        self._json = json
+        self._funcs = tuple(funcs)
+        self._keys = tuple(keys)
+        self._func_to_key = dict(zip(self._funcs, self._keys))
+        self._repetitions = repetitions
+        self._cache_dir = pathlib.Path(cache_dir) if cache_dir is not None else CACHE_DIR / _project_key()
+        self._cache_dir.mkdir(parents=True, exist_ok=True)
+        self._cache_path = self._cache_dir / (hashlib.sha256(str(self._keys).encode()).hexdigest() + ".json")
+        if self._cache_path.exists():
+            self._timings = json.loads(self._cache_path.read_text())
+        else:
+            self._timings = {key: {} for key in self._keys}
+        self._best_func = {}
+
+    def __call__(self, *args, **kwargs):
+        arg_key = self._make_arg_key(args, kwargs)
+        if arg_key not in self._best_func:
+            timings = self._get_timings(args, kwargs)
+            self._best_func[arg_key] = self._funcs[timings.index(min(timings))]
+        return self._best_func[arg_key](*args, **kwargs)
+
+    def _get_timings(self, args, kwargs):
+        arg_key = self._make_arg_key(args, kwargs)
+        if arg_key in self._timings:
+            return self._timings[arg_key]
+        timings = [self._get_timing(func, args, kwargs) for func in self._funcs]
+        self._timings[arg_key] = timings
+        self._cache_path.write_text(self._json.dumps(self._timings))
+        return timings
+
+    def _get_timing(self, func, args, kwargs):
+        data = self._timings.setdefault(self._func_to_key[func], {})
+        arg_key = self._make_arg_key(args, kwargs)
+        cache_path = self._get_func_cache_path(func)
+        if arg_key not in data and cache_path.exists():
+            data.update(self._json.loads(cache_path.read_text()))
+        if arg_key in data:
+            return data[arg_key]
+        try:
+            timing = self._measure(lambda: func(*args, **kwargs))
+        except runtime.KernelLaunchError:
+            timing = float("inf")
+        data[arg_key] = timing
+        cache_path.write_text(self._json.dumps(data))
+        return timing
+
+    def _measure(self, call):
+        import time
+
+        try:
+            import torch
+
+            synchronize = torch.cuda.synchronize if torch.cuda.is_available() else (lambda: None)
+        except ImportError:
+            synchronize = lambda: None  # noqa: E731
+        call()  # warm-up: first-launch work (plans, specialisation) is not the kernel's time
+        synchronize()
+        best = float("inf")
+        for _ in range(self._repetitions):
+            start = time.perf_counter()
+            call()
+            synchronize()
+            best = min(best, (time.perf_counter() - start) * 1e3)
+        return best
+
+    def _get_func_cache_path(self, func):
+        return self._cache_dir / (hashlib.sha256(str(self._func_to_key[func]).encode()).hexdigest() + ".json")
+
+    @staticmethod
+    def _make_arg_key(args, kwargs):
+        def make_key(arg):
+            if hasattr(arg, "shape") and hasattr(arg, "dtype"):
+                return f"tensor(shape={tuple(arg.shape)}, dtype={str(arg.dtype).split('.')[-1]})"
+            return str(arg)
+
+        return ", ".join([make_key(arg) for arg in args] + [f"{name}={make_key(arg)}" for name, arg in sorted(kwargs.items())])
+
+
+def _project_key():
+    """Timings belong to one build of the kernels: the key is the library's instance list and version."""
+    try:
+        names = "|".join(runtime.gemm_config_names()) + "|" + runtime.library().nt_version().decode()
+    except Exception:
+        names = "no-library"
+    return "timings_" + hashlib.sha256(names.encode()).hexdigest()[:16]

@@ -108,3 +108,66 @@ def test_tuning_cache_reads_and_writes_the_reference_csv_format(tmp_path):
     assert rows[0] == [] and len(rows[1]) == 4  # the default pair
     assert [str(v) for v in (fp16, fp16, 4096, 2048, 1024, 1)] in rows
     assert lib.nt_tune_cache_load(str(tmp_path / "missing.csv").encode(), None) != 0
+
+
+def test_auto_tuner_json_caches(tmp_path):
+    """The reference's tests/test_auto_tuner.py:9-80: callables with known delays, the two kinds of
+    JSON files, and a second call that no longer measures."""
+    import json
+    import time
+
+    from ninetoothed_amd.auto_tuner import AutoTuner
+
+    def delay_foo(*args, **kwargs):
+        return 0.001 * (2 * len(args) + len(kwargs))
+
+    def delay_bar(*args, **kwargs):
+        return 0.001 * (len(args) + 2 * len(kwargs))
+
+    def foo(*args, **kwargs):
+        time.sleep(delay_foo(*args, **kwargs))
+
+    def bar(*args, **kwargs):
+        time.sleep(delay_bar(*args, **kwargs))
+
+    for args, kwargs in (((1,), {"a": 2, "b": 4, "c": 6, "d": 8}), ((1, 3, 5), {"a": 2})):
+        tuner = AutoTuner((foo, bar), ("foo", "bar"), cache_dir=tmp_path / f"cache{len(args)}")
+        assert not tuner._cache_path.exists() and not tuner._get_func_cache_path(foo).exists()
+        start = time.perf_counter()
+        tuner(*args, **kwargs)
+        first = time.perf_counter() - start
+        assert tuner._cache_path.exists() and tuner._get_func_cache_path(foo).exists() and tuner._get_func_cache_path(bar).exists()
+        start = time.perf_counter()
+        tuner(*args, **kwargs)
+        assert time.perf_counter() - start < first
+        key = tuner._make_arg_key(args, kwargs)
+        assert key == ", ".join([str(a) for a in args] + [f"{k}={v}" for k, v in sorted(kwargs.items())])
+        expected = foo if delay_foo(*args, **kwargs) < delay_bar(*args, **kwargs) else bar
+        assert tuner._best_func[key] is expected
+        # the files hold what the reference's reader expects
+        per_func = json.loads(tuner._get_func_cache_path(foo).read_text())
+        assert list(per_func) == [key] and per_func[key] >= delay_foo(*args, **kwargs) * 1e3
+        whole = json.loads(tuner._cache_path.read_text())
+        assert set(whole) == {"foo", "bar", key} and len(whole[key]) == 2
+        # a new tuner over the same directory starts from the files and measures nothing
+        again = AutoTuner((foo, bar), ("foo", "bar"), cache_dir=tmp_path / f"cache{len(args)}")
+        assert again._get_timings(args, kwargs) == whole[key]
+
+
+def test_auto_tuner_tensor_keys_and_failed_launches(tmp_path):
+    import torch
+
+    from ninetoothed_amd.auto_tuner import AutoTuner
+    from ninetoothed_amd.runtime import KernelLaunchError
+
+    def refuses(x):
+        raise KernelLaunchError(1)
+
+    def works(x):
+        return x
+
+    tuner = AutoTuner((refuses, works), ("refuses", "works"), cache_dir=tmp_path)
+    x = torch.zeros(3, 4, dtype=torch.float16)
+    assert tuner(x) is x
+    assert tuner._make_arg_key((x,), {}) == "tensor(shape=(3, 4), dtype=float16)"
+    assert tuner._timings["tensor(shape=(3, 4), dtype=float16)"][0] == float("inf")
