@@ -178,6 +178,8 @@ class Kernel:
         for arg, tensor in zip(args, self.types):
             if tensor.ndim == 0 and not isinstance(tensor.dtype, Tensor):
                 parts.append((type(arg).__name__, arg if tensor.constexpr else None))
+            elif getattr(arg, "is_nested", False):
+                parts.append(_jagged_layout(arg) + (arg.dtype, arg.device.index))
             else:
                 parts.append((tuple(arg.shape), tuple(arg.stride()), arg.dtype, arg.device.index))
         return tuple(parts), tuple(sorted(kwargs.items()))
@@ -198,6 +200,23 @@ class Kernel:
                 raise RuntimeError(f"`{name}` lives on `{arg.device}`; this build only runs on the GPU (there is no CPU path).")
             if arg.ndim != source.ndim:
                 raise ValueError(f"`{name}` must have {source.ndim} dimensions, got {arg.ndim}.")
+            if (source.jagged_dim is not None) != bool(getattr(arg, "is_nested", False)):
+                raise TypeError(f"`{name}` is {'declared jagged: pass a `torch.jagged` nested tensor' if source.jagged_dim is not None else 'not declared jagged: pass a dense tensor'}.")
+            if source.jagged_dim is not None:
+                # sizes as the launch sees them (src/ninetoothed/tensor.py:621-637, generation.py:686-704):
+                # the longest sequence along the jagged dimension, no stride along the batch
+                if self.kind != "map":
+                    raise UnsupportedProgram("Jagged tensors are only supported by the element-wise executor.")
+                if arg._ragged_idx != source.jagged_dim:
+                    raise ValueError(f"`{name}` is jagged along dimension {arg._ragged_idx}, declared along {source.jagged_dim}.")
+                shape, strides = _jagged_layout(arg)
+                for dim in range(source.ndim):
+                    declared = source.shape[dim]
+                    if isinstance(declared, Symbol) and declared.is_name:
+                        env[declared.name] = shape[dim]
+                    env[source.size_string(dim)] = shape[dim]
+                    env[source.stride_string(dim)] = strides[dim]
+                continue
             for dim in range(source.ndim):
                 declared = source.shape[dim]
                 if not isinstance(declared, Symbol) and int(declared) != arg.shape[dim]:
@@ -359,11 +378,11 @@ class Kernel:
         lib = runtime.library()
         tensor_params = [p for p, t in enumerate(self.types) if not (t.ndim == 0 and not isinstance(t.dtype, Tensor))]
         for p in tensor_params:
-            if args[p].numel() > 0 and args[p].data_ptr() % args[p].element_size():
+            if args[p].numel() > 0 and _storage(args, p).data_ptr() % args[p].element_size():
                 raise UnsupportedProgram("Tensor data must be aligned to its element size.")
         launches = []
         for store in self.program.stores:
-            built = mapping.build(store, self.types, args, env, lambda p: _dtype_tag(args[p].dtype), lambda p: args[p].data_ptr())
+            built = mapping.build(store, self.types, args, env, lambda p: _dtype_tag(_storage(args, p).dtype), lambda p: _storage(args, p).data_ptr())
             if built is not None:
                 launches.append(built)
         if not launches:
@@ -373,7 +392,7 @@ class Kernel:
             stream = runtime.current_stream()
             for program, _, scalar_slots, operand_params in launches:
                 for slot, param in enumerate(operand_params):
-                    program.operands[slot].data = call_args[param].data_ptr()
+                    program.operands[slot].data = _storage(call_args, param).data_ptr()
                 for index, param in scalar_slots:
                     program.value_constants[index] = float(call_args[param])
                 runtime.check(lib.launch_nt_map(stream, ctypes.addressof(program)))
@@ -404,6 +423,27 @@ class Kernel:
             runtime.check(lib.launch_nt_attention(runtime.current_stream(), tensors[0], tensors[1], tensors[2], causal, scale_arg, tensors[3], dtype, 0, 0))
 
         return _Plan(f"launch_nt_attention q{info['q']['shape']} k{info['k']['shape']} {tag}", launch)
+
+
+def _storage(args, param):
+    """The dense tensor behind an operand of a tile map: the argument itself, the values of a
+    jagged argument, or (``(position, "offsets")``) the sequence offsets of a jagged argument."""
+    if isinstance(param, tuple):
+        return args[param[0]].offsets()
+    arg = args[param]
+    return arg.values() if getattr(arg, "is_nested", False) else arg
+
+
+def _jagged_layout(arg):
+    """(shape, strides) a jagged nested tensor is launched with: batch entries of the longest
+    length, laid over the values with no stride along the batch (the reference reads the
+    longest length the same way at every call, src/ninetoothed/torchifier.py:33-36)."""
+    values, offsets = arg.values(), arg.offsets()
+    jagged_dim = arg._ragged_idx
+    longest = int(offsets.diff().max().item()) if offsets.numel() > 1 else 0
+    shape = [offsets.numel() - 1] + [longest if dim == jagged_dim else values.shape[dim - 1] for dim in range(1, arg.ndim)]
+    strides = [0] + [values.stride(dim - 1) for dim in range(1, arg.ndim)]
+    return tuple(shape), tuple(strides)
 
 
 class _Plan:

@@ -236,6 +236,7 @@ class _Lowering:
         self.reduced_vars = []
         self.dynamic_vars = []    # variables that take their value from the data (level indices)
         self.levels_used = {}     # param -> level its tiles are taken from
+        self.jagged = {}          # operand slot -> (variable of the sequence start, variable of its end)
 
     # -- variables ---------------------------------------------------------
     def new_var(self, extent):
@@ -517,9 +518,11 @@ class _Lowering:
         slot = len(self.operands)
         if slot >= MAX_OPERANDS:
             raise UnsupportedProgram("Too many tensor operands for the element-wise executor.")
-        tensor = self.types[param]
-        if tensor.ndim == 0 and not hasattr(tensor.dtype, "ndim"):
+        tensor = None if isinstance(param, tuple) else self.types[param]  # (position, "offsets"): sequence offsets of a jagged tensor
+        if tensor is not None and tensor.ndim == 0 and not hasattr(tensor.dtype, "ndim"):
             raise UnsupportedProgram("Scalars have no elements to address.")
+        if tensor is not None and tensor.source.jagged_dim is not None:
+            raise UnsupportedProgram("Jagged tensors cannot be addressed by computed indices or pointers.")
         raw = _RawOperand(tensor)
         self.operands.append((param, raw))
         self.bindings[slot] = {}
@@ -531,15 +534,15 @@ class _Lowering:
             self.emit("SETVAR", var)
             return var
 
-        source = tensor.source
         if element_offset is not None:
             raw.terms.append((dynamic(element_offset, None), 1, None))
-        else:
-            if len(indices) != source.ndim:
-                raise UnsupportedProgram("A source tensor needs one index per dimension.")
-            for dim, index in enumerate(indices):
-                size = int(self.env[source.size_string(dim)])
-                raw.terms.append((dynamic(index, size), int(self.env[source.stride_string(dim)]), size))
+            return slot
+        source = tensor.source
+        if len(indices) != source.ndim:
+            raise UnsupportedProgram("A source tensor needs one index per dimension.")
+        for dim, index in enumerate(indices):
+            size = int(self.env[source.size_string(dim)])
+            raw.terms.append((dynamic(index, size), int(self.env[source.stride_string(dim)]), size))
         return slot
 
     def new_var_deferred(self):
@@ -575,6 +578,8 @@ class _Lowering:
         from a middle level (``tensor[i, j]``), emits the code that computes the level indices."""
         slot = self.operand(ref.param, ref.level)
         self.bind_tile(slot, dims)
+        if self.types[ref.param].source.jagged_dim is not None and slot not in self.jagged:
+            self.bind_sequence(slot, ref, dims, inside_reduction)
         if ref.level == 2:
             _, operand = self.operands[slot]
             names = operand.names[1]
@@ -593,6 +598,21 @@ class _Lowering:
                 self.lower(index, unit, inside_reduction)
                 self.emit("SETVAR", var)
         return slot
+
+    def bind_sequence(self, slot, ref, dims, inside_reduction):
+        """A jagged tensor: loads where the batch entry's sequence starts and ends in the values
+        (``offsets[batch]``, ``offsets[batch + 1]``; src/ninetoothed/generation.py:686-704) into
+        two variables the index program of the operand uses."""
+        if ref.level != 1:
+            raise UnsupportedProgram("Jagged tensors are supported with tiles directly below the launch grid.")
+        start, end = self.new_var(1), self.new_var(1)
+        self.dynamic_vars += [start, end]
+        self.jagged[slot] = (start, end)
+        batch = Node("offsets", ref, 0)
+        for var, position in ((start, batch), (end, Node("add", batch, 1))):
+            bounds = self.raw_access((ref.param, "offsets"), None, dims, inside_reduction, element_offset=position)
+            self.emit("LOAD", bounds)
+            self.emit("SETVAR", var)
 
     def _has_load(self, value):
         if isinstance(value, Node):
@@ -627,6 +647,13 @@ class _Lowering:
                     code.append(I_MULC | (const(coef) << 8))
                 code.append(I_ADD)
 
+        def emit_sequence_start(slot, operand):
+            if slot in self.jagged:
+                source = operand.tensor.source
+                code.append(I_VAR | (order[self.jagged[slot][0]] << 8))
+                code.append(I_MULC | (const(int(self.env[source.stride_string(source.jagged_dim)])) << 8))
+                code.append(I_ADD)
+
         for slot, kind, dim in self.segments:
             _, operand = self.operands[slot]
             binding = self.bindings[slot]
@@ -652,9 +679,29 @@ class _Lowering:
                 for index, size in operand.constraints:
                     emit_affine(index, binding)
                     code.append(I_CHECK | (const(size) << 8))
+                if slot in self.jagged:
+                    # inside the sequence: 0 <= end - 1 - start - index (its lower bound is the tile mask above,
+                    # or holds by construction); the values are then addressed from the sequence's start
+                    start, end = self.jagged[slot]
+                    jagged_dim = operand.tensor.source.jagged_dim
+                    code.append(I_VAR | (order[end] << 8))
+                    code.append(I_CONST | (const(-1) << 8))
+                    code.append(I_ADD)
+                    for term in (None, operand.indices[jagged_dim]):
+                        if term is None:
+                            code.append(I_VAR | (order[start] << 8))
+                        else:
+                            emit_affine(term, binding)
+                        code.append(I_MULC | (const(-1) << 8))
+                        code.append(I_ADD)
+                    code.append(I_CHECK | (const(1 << 62) << 8))
+                    emit_affine(operand.indices[jagged_dim], binding)
+                    code.append(I_CHECK | (const(1 << 62) << 8))
                 emit_affine(operand.offset(), binding)
+                emit_sequence_start(slot, operand)
             elif dim is None:
                 emit_affine(operand.offset(), binding)
+                emit_sequence_start(slot, operand)
             else:
                 emit_affine(operand.indices[dim], binding)
             code.append(I_END)
@@ -662,6 +709,8 @@ class _Lowering:
 
 
 def _other_value(tensor):
+    if tensor is None:
+        return 0.0
     other = tensor.source.other
     return 0.0 if other is None else float(other)
 

@@ -99,8 +99,9 @@ class Tensor:
     :param ndim: The number of dimensions.
     :param shape: The shape; ``None`` entries become size symbols.
     :param dtype: The element type, or the next inner level.
-    :param jagged_dim: Accepted for interface compatibility; jagged tensors
-        are not supported by this build.
+    :param jagged_dim: The dimension whose length differs per batch entry (a
+        ``torch.jagged`` nested tensor is passed at call time; the batch is
+        dimension 0).
     :param other: The value out-of-bounds positions read as.
     :param shape_options: Options for the size symbols (one dict, or one per dim).
     :param constexpr: Whether a zero-dimensional tensor is a call-time constant.
@@ -126,11 +127,8 @@ class Tensor:
         target_dims=None,
         _links=None,
     ):
-        if jagged_dim is not None:
-            raise NotImplementedError("Jagged tensors are not supported.")
-
         self.dtype = dtype
-        self.jagged_dim = None
+        self.jagged_dim = jagged_dim
 
         if name is not None:
             self.name = name
@@ -143,6 +141,8 @@ class Tensor:
             ndim = len(shape)
         if shape is None:
             shape = (None,) * ndim
+        if jagged_dim is not None and not 1 <= jagged_dim < ndim:
+            raise ValueError("`jagged_dim` must name a dimension after the batch dimension.")
 
         if shape_options is None:
             shape_options = tuple({} for _ in range(ndim))

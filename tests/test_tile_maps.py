@@ -21,7 +21,7 @@ import ninetoothed_amd as ninetoothed
 import ninetoothed_amd.language as ntl
 from ninetoothed_amd import Symbol, Tensor, block_size, mapping
 from ninetoothed_amd.language import libdevice
-from ninetoothed_amd.make import _dtype_tag
+from ninetoothed_amd.make import _dtype_tag, _storage
 from ninetoothed_amd.recognition import UnsupportedProgram
 from oracle import programs as oracle
 from oracle.arrangement import View
@@ -137,13 +137,13 @@ def _run_on_machine(kernel, args, kwargs=None):
 
     def storage(p):
         if p not in flat:
-            tensor = args[p]
+            tensor = _storage(args, p)
             size = 1 + sum((n - 1) * abs(s) for n, s in zip(tensor.shape, tensor.stride())) if tensor.numel() else 0
             flat[p] = torch.as_strided(tensor, (size,), (1,)).numpy()
         return flat[p]
 
     for store in kernel.program.stores:
-        built = mapping.build(store, kernel.types, args, env, lambda p: _dtype_tag(args[p].dtype), lambda p: 0)
+        built = mapping.build(store, kernel.types, args, env, lambda p: _dtype_tag(_storage(args, p).dtype), lambda p: 0)
         if built is None:
             continue
         program, _, _, operand_params = built
@@ -651,3 +651,88 @@ def test_atomic_sum_through_a_pointer(interpret, monkeypatch):
     counts = torch.zeros(1, dtype=torch.int32, device="cuda")
     kernel(torch.ones(64180, dtype=torch.int32, device="cuda"), counts)
     assert counts.item() == 64180
+
+
+# ---- jagged tensors (the reference's tests/test_jagged.py) --------------------------------------
+
+_JAGGED_BLOCK = Symbol("block_size", constexpr=True)
+
+
+def _to_padded_arrangement(input, output, block_size=_JAGGED_BLOCK):
+    tile_shape = (1,) + tuple(block_size for _ in range(1, input.ndim))
+    return input.tile(tile_shape), output.tile(tile_shape)
+
+
+def _jagged_copy_arrangement(dst, src, jagged_dim, block_size=_JAGGED_BLOCK):
+    tile_shape = (1,) + tuple(block_size for _ in range(1, dst.ndim))
+    return dst.tile(tile_shape), src.expand(tuple(-1 if dim != jagged_dim else dst.shape[dim] for dim in range(src.ndim))).tile(tile_shape)
+
+
+def _jagged_copy_application(dst, src):
+    dst = src  # noqa: F841
+
+
+def _jagged_batches(jagged_dim, lengths, batch_shape, device="cpu"):
+    batches = tuple(torch.randn(batch_shape[: jagged_dim - 1] + (n,) + batch_shape[jagged_dim:], device=device) for n in lengths)
+    return torch.nested.nested_tensor(batches, layout=torch.jagged)
+
+
+@pytest.mark.parametrize("jagged_dim", (1, 2))
+def test_lowering_jagged_to_padded_and_expand(jagged_dim):
+    nested = _jagged_batches(jagged_dim, (3, 6, 1, 9), (5, 7))
+    kernel = ninetoothed.make(_to_padded_arrangement, clone_application, (Tensor(3, jagged_dim=jagged_dim, other=-1), Tensor(3)))
+    expected = torch.nested.to_padded_tensor(nested, -1.0)
+    out = torch.full(expected.shape, float("nan"))
+    _run_on_machine(kernel, (nested, out), {"block_size": 4})
+    assert torch.equal(out, expected)
+
+    # a dense row / column written into every entry of a jagged destination
+    copy = ninetoothed.make(functools.partial(_jagged_copy_arrangement, jagged_dim=jagged_dim), _jagged_copy_application, (Tensor(3, jagged_dim=jagged_dim), Tensor(3)))
+    src = torch.randn(tuple(size if dim != jagged_dim else 1 for dim, size in enumerate(expected.shape)))
+    before = nested.values().clone()
+    _run_on_machine(copy, (nested, src), {"block_size": 4})
+    assert not torch.equal(nested.values(), before)
+    padded = torch.nested.to_padded_tensor(nested, float("nan"))
+    inside = ~torch.isnan(padded)
+    assert inside.sum().item() == nested.values().numel()
+    assert torch.equal(padded[inside], src.expand_as(padded)[inside])
+
+
+def test_jagged_arguments_are_checked():
+    kernel = ninetoothed.make(_to_padded_arrangement, clone_application, (Tensor(3, jagged_dim=1, other=-1), Tensor(3)))
+    nested = _jagged_batches(2, (3, 4), (5, 7))
+    with pytest.raises(ValueError):  # jagged along another dimension than declared
+        kernel._environment((nested, torch.empty(2, 5, 4)), {"block_size": 4}, check_device=False)
+    with pytest.raises(TypeError):  # a dense tensor where a jagged one is declared
+        kernel._environment((torch.empty(2, 5, 4), torch.empty(2, 5, 4)), {"block_size": 4}, check_device=False)
+    with pytest.raises(ValueError):
+        Tensor(3, jagged_dim=0)
+
+
+@gpu
+@pytest.mark.parametrize("interpret", ("0", "1"))
+@pytest.mark.parametrize("num_batches", (2, 7, 16))
+@pytest.mark.parametrize("jagged_dim", (1, 2))
+def test_jagged_to_padded_tensor_and_expand(jagged_dim, num_batches, interpret, monkeypatch):
+    """tests/test_jagged.py:55-158 of the reference (ndim 3, padding -1, block size 32)."""
+    import random
+
+    monkeypatch.setenv("NT_MAP_INTERPRET", interpret)
+    generator = random.Random(17 * num_batches + jagged_dim)
+    batch_shape = (generator.randint(1, 300), generator.randint(1, 300))
+    lengths = [generator.randint(1, 300) for _ in range(num_batches)]
+    nested = _jagged_batches(jagged_dim, lengths, batch_shape, device="cuda")
+    kernel = ninetoothed.make(_to_padded_arrangement, clone_application, (Tensor(3, jagged_dim=jagged_dim, other=-1), Tensor(3)))
+    expected = torch.nested.to_padded_tensor(nested, -1.0)
+    out = torch.full(expected.shape, float("nan"), device="cuda")
+    kernel(nested, out, block_size=32)
+    _served_by_map(kernel)
+    assert torch.equal(out, expected)
+
+    copy = ninetoothed.make(functools.partial(_jagged_copy_arrangement, jagged_dim=jagged_dim), _jagged_copy_application, (Tensor(3, jagged_dim=jagged_dim), Tensor(3)))
+    src = torch.randn(tuple(size if dim != jagged_dim else 1 for dim, size in enumerate(expected.shape)), device="cuda")
+    copy(nested, src, block_size=32)
+    padded = torch.nested.to_padded_tensor(nested, float("nan"))
+    inside = ~torch.isnan(padded)
+    assert inside.sum().item() == nested.values().numel()
+    assert torch.equal(padded[inside], src.expand_as(padded)[inside])
