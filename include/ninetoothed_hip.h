@@ -16,10 +16,12 @@
  *
  * Launches are asynchronous on the given stream and never synchronise; the
  * caller owns every tensor.  Only launch_nt_conv2d and launch_nt_attention on
- * FLOAT32 tensors take temporary device memory, from the stream-ordered
- * allocator (hipMallocAsync / hipFreeAsync on the given stream, see there);
- * every other launch allocates nothing.  All
- * functions are re-entrant.
+ * FLOAT32 tensors use scratch device memory: one buffer per (device, stream,
+ * purpose) that the library allocates (hipMalloc) the first time a call needs
+ * it, grows (hipFree + hipMalloc, which wait for the device) when a later call
+ * needs more, and otherwise reuses, so that steady-state calls allocate
+ * nothing; nt_release_workspaces frees them.  Every other launch allocates
+ * nothing.  All functions may be called from several host threads.
  */
 #ifndef NINETOOTHED_HIP_H
 #define NINETOOTHED_HIP_H
@@ -130,7 +132,7 @@ NineToothedResult launch_nt_softmax_config(NineToothedStream stream, int config,
  * is_causal is a 0-d tensor holding a host int64_t.
  * dtype FLOAT16 / BFLOAT16, or FLOAT32 (the fp32 case of
  * tests/test_attention.py:99-117, rtol = atol = 0.025 there): K and V are first
- * narrowed to fp16 copies taken from the stream-ordered allocator on `stream`,
+ * narrowed to fp16 copies in the library's scratch buffer of `stream`,
  * Q is narrowed while it is scaled, the products run on the fp16 MFMA path with
  * fp32 accumulation and O is written unrounded.
  * block_size_m / block_size_n are hints (0 = library's choice): block_size_m
@@ -155,10 +157,11 @@ NineToothedResult launch_nt_attention(NineToothedStream stream,
  * tests/test_conv2d.py:13-48 describes.
  * When C % 32 == 0, K % 256 == 0, (P*Q) % 8 == 0, the output is contiguous and
  * N*P*Q >= 1024, the call first repacks the input to channels-last and the
- * filter to [R*S*C, K] in temporaries taken from and returned to the
- * stream-ordered allocator on `stream` (N*C*H*W + K*C*R*S elements), then runs
- * the direct-to-LDS main loop; block_size_m == 1 keeps the call on the
- * allocation-free gather kernel, which also serves every other shape. */
+ * filter to [R*S*C, K] in the library's scratch buffers of `stream`
+ * (N*C*H*W + K*C*R*S elements), then runs the direct-to-LDS main loop;
+ * block_size_m == 1 keeps the call on the scratch-free gather kernel, which
+ * also serves every other shape and calls whose scratch cannot be allocated
+ * (out of memory; a stream under graph capture that has no buffer yet). */
 NineToothedResult launch_nt_conv2d(NineToothedStream stream,
                                    NineToothedTensor input,
                                    NineToothedTensor filter,
@@ -341,6 +344,10 @@ NineToothedResult nt_map_source(const NineToothedMapProgram *program, char *buff
 
 /* Library version string, e.g. "nt_hip 0.1 gfx950". */
 const char *nt_version(void);
+
+/* Frees every scratch buffer the library holds (see the introduction).  Waits
+ * for the device.  No counterpart in the reference, whose kernels need none. */
+void nt_release_workspaces(void);
 
 #ifdef __cplusplus
 }

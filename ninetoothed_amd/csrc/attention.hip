@@ -18,6 +18,7 @@
 #include <type_traits>
 
 #include "gemm_fast.h"  // swizzle helpers, static_for, lds_barrier
+#include "workspace.h"
 
 namespace nt {
 namespace {
@@ -539,9 +540,9 @@ __global__ __launch_bounds__(256) void attention_narrow_kernel(const float *src,
 
 int attention_float32(AttentionParams p, int head_dim, const NineToothedTensor &k, const NineToothedTensor &v, hipStream_t stream) {
     const int64_t total = (int64_t)p.batch * p.heads * p.seq_k * head_dim;
-    half_t *narrow = nullptr;
-    hipError_t err = hipMallocAsync((void **)&narrow, (size_t)total * 2 * sizeof(half_t), stream);
-    if (err != hipSuccess) return (int)err;
+    WorkspaceLease lease(stream);
+    half_t *narrow = (half_t *)lease.get(kWorkspaceAttentionNarrow, (size_t)total * 2 * sizeof(half_t));
+    if (narrow == nullptr) return (int)hipErrorOutOfMemory;
     const unsigned blocks = (unsigned)((total + 255) / 256 < 256 * 16 ? (total + 255) / 256 : 256 * 16);
     attention_narrow_kernel<<<dim3(blocks), dim3(256), 0, stream>>>((const float *)k.data, narrow, total, p.heads, p.seq_k, head_dim, k.strides[0],
                                                                   k.strides[1], k.strides[2], k.strides[3]);
@@ -555,8 +556,7 @@ int attention_float32(AttentionParams p, int head_dim, const NineToothedTensor &
     if (head_dim == 128) result = (int)launch_attention<half_t, 128, 1, 64, 2, false, float>(p, stream);
     else if (head_dim == 64) result = (int)launch_attention<half_t, 64, 1, 64, 2, false, float>(p, stream);
     else if (head_dim == 32) result = (int)launch_attention<half_t, 32, 1, 64, 2, false, float>(p, stream);
-    const hipError_t released = hipFreeAsync(narrow, stream);
-    return result != 0 ? result : (int)released;
+    return result;
 }
 
 // variant: 0 = 128 query rows per workgroup, 64-key blocks, two workgroups per CU

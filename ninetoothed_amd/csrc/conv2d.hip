@@ -7,9 +7,9 @@
 //
 // The MFMA operands need 8 consecutive k-values per lane, i.e. consecutive
 // CHANNELS of one input position, while NCHW keeps channels H*W elements apart.
-// Two stream-ordered pre-passes therefore repack the operands into temporaries
-// obtained with hipMallocAsync on the launch stream (freed with hipFreeAsync
-// right after the main kernel, so the call stays asynchronous and re-entrant):
+// A pre-pass on the launch stream therefore repacks both operands into scratch
+// buffers the library keeps per stream between calls (workspace.h; the call stays
+// asynchronous, and allocates only when a call needs more than any before it):
 //   x[N,C,H,W]  -> xt[N,H,W,C]              (tiled transpose through LDS, 16-byte accesses)
 //   w[K,C,R,S]  -> wt[(r*S+s)*C + c, K]     (row-major K x N operand of the GEMM)
 // The main kernel then is the 256x256x32, 4-stage GEMM: a K step is 32 channels of
@@ -24,6 +24,7 @@
 // fp16/bf16, C % 32 == 0, K_out % 256 == 0, (P*Q) % 8 == 0, contiguous output.
 #include "conv2d.h"
 #include "gemm_fast.h"
+#include "workspace.h"
 
 namespace nt {
 namespace {
@@ -37,15 +38,39 @@ struct ConvParams {
     unsigned xt_bytes;
 };
 
-// ---- pre-pass 1: NCHW (any strides) -> NHWC contiguous ----
+// ---- pre-pass: one launch, two jobs ----
+// grid layer  z == 0: w[K,C,R,S] (any strides) -> wt[(r*S+s)*C + c][K], grid-stride over the layer's threads
+//                     (first, so that its scattered reads overlap the streaming layers behind it)
+// grid layers z >= 1: x[z-1] NCHW (any strides) -> xt[z-1] NHWC contiguous (64 x 64 tiles through LDS)
+struct FilterRepack {
+    const void *w;
+    void *wt;
+    int K, C, R, S;
+    int64_t s_k, s_c, s_r, s_s;
+};
+
 template <typename T>
-__global__ __launch_bounds__(256) void nchw_to_nhwc_kernel(const T *x, T *xt, int C, int HW, int W, int64_t s_n, int64_t s_c,
-                                                          int64_t s_h, int64_t s_w, int vector_ok) {
+__global__ __launch_bounds__(256) void conv2d_repack_kernel(const T *x, T *xt, int C, int HW, int W, int64_t s_n, int64_t s_c, int64_t s_h,
+                                                           int64_t s_w, int vector_ok, FilterRepack f) {
     typedef typename Elem<T>::vec8 vec8;
     constexpr int kPitch = 64 + 8;  // halfs; keeps 16-byte alignment of rows
     __shared__ __attribute__((aligned(16))) T tile[64 * kPitch];
-    const int hw0 = blockIdx.x * 64, c0 = blockIdx.y * 64, n = blockIdx.z;
     const int t = threadIdx.x;
+    if (blockIdx.z == 0) {
+        const T *w = (const T *)f.w;
+        T *wt = (T *)f.wt;
+        const int64_t total = (int64_t)f.K * f.C * f.R * f.S;
+        const int64_t layer_threads = (int64_t)gridDim.x * gridDim.y * 256;
+        for (int64_t index = ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * 256 + t; index < total; index += layer_threads) {
+            const int k = (int)(index % f.K);
+            const int64_t row = index / f.K;
+            const int c = (int)(row % f.C);
+            const int rs = (int)(row / f.C);
+            wt[index] = w[(int64_t)k * f.s_k + (int64_t)c * f.s_c + (int64_t)(rs / f.S) * f.s_r + (int64_t)(rs % f.S) * f.s_s];
+        }
+        return;
+    }
+    const int hw0 = blockIdx.x * 64, c0 = blockIdx.y * 64, n = blockIdx.z - 1;
     const T *src = x + (int64_t)n * s_n;
     // load: rows = channels, 8 consecutive positions per thread
 #pragma unroll
@@ -77,20 +102,6 @@ __global__ __launch_bounds__(256) void nchw_to_nhwc_kernel(const T *x, T *xt, in
             *(vec8 *)(xt + ((int64_t)n * HW + hw0 + hw) * C + c0 + c) = v;
         }
     }
-}
-
-// ---- pre-pass 2: w[K,C,R,S] (any strides) -> wt[(r*S+s)*C + c][K] ----
-template <typename T>
-__global__ __launch_bounds__(256) void filter_to_rsck_kernel(const T *w, T *wt, int K, int C, int R, int S, int64_t s_k,
-                                                            int64_t s_c, int64_t s_r, int64_t s_s) {
-    const int64_t total = (int64_t)K * C * R * S;
-    const int64_t index = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (index >= total) return;
-    const int k = (int)(index % K);
-    const int64_t row = index / K;
-    const int c = (int)(row % C);
-    const int rs = (int)(row / C);
-    wt[index] = w[(int64_t)k * s_k + (int64_t)c * s_c + (int64_t)(rs / S) * s_r + (int64_t)(rs % S) * s_s];
 }
 
 // ---- main kernel ----
@@ -306,21 +317,19 @@ template <typename T>
 int run_fast(const Conv2dRequest &q, hipStream_t stream) {
     const int64_t xt_bytes = (int64_t)q.N * q.H * q.W * q.C * 2;
     const int64_t wt_bytes = (int64_t)q.K * q.C * q.R * q.S * 2;
-    void *xt = nullptr, *wt = nullptr;
-    hipError_t err = hipMallocAsync(&xt, (size_t)xt_bytes, stream);
-    if (err != hipSuccess) return NINETOOTHED_NO_KERNEL;  // no temporary: the caller falls back to the gather kernel
-    err = hipMallocAsync(&wt, (size_t)wt_bytes, stream);
-    if (err != hipSuccess) {
-        (void)hipFreeAsync(xt, stream);
-        return NINETOOTHED_NO_KERNEL;
-    }
+    WorkspaceLease lease(stream);
+    void *xt = lease.get(kWorkspaceConvInput, (size_t)xt_bytes);
+    void *wt = lease.get(kWorkspaceConvFilter, (size_t)wt_bytes);
+    if (xt == nullptr || wt == nullptr) return NINETOOTHED_NO_KERNEL;  // no scratch: the caller falls back to the gather kernel
     const int HW = q.H * q.W;
     const int vector_ok = q.xs[3] == 1 && q.xs[2] == q.W && HW % 8 == 0 && q.xs[1] % 8 == 0 && q.xs[0] % 8 == 0 && ((uintptr_t)q.x & 15) == 0;
-    nchw_to_nhwc_kernel<T><<<dim3(ceil_div(HW, 64), ceil_div(q.C, 64), q.N), dim3(256), 0, stream>>>(
-        (const T *)q.x, (T *)xt, q.C, HW, q.W, q.xs[0], q.xs[1], q.xs[2], q.xs[3], vector_ok);
-    const int64_t filter_elems = (int64_t)q.K * q.C * q.R * q.S;
-    filter_to_rsck_kernel<T><<<dim3((unsigned)((filter_elems + 255) / 256)), dim3(256), 0, stream>>>(
-        (const T *)q.w, (T *)wt, q.K, q.C, q.R, q.S, q.ws[0], q.ws[1], q.ws[2], q.ws[3]);
+    FilterRepack f;
+    f.w = q.w;
+    f.wt = wt;
+    f.K = q.K; f.C = q.C; f.R = q.R; f.S = q.S;
+    f.s_k = q.ws[0]; f.s_c = q.ws[1]; f.s_r = q.ws[2]; f.s_s = q.ws[3];
+    conv2d_repack_kernel<T><<<dim3(ceil_div(HW, 64), ceil_div(q.C, 64), q.N + 1), dim3(256), 0, stream>>>(
+        (const T *)q.x, (T *)xt, q.C, HW, q.W, q.xs[0], q.xs[1], q.xs[2], q.xs[3], vector_ok, f);
     ConvParams p;
     p.xt = xt;
     p.wt = wt;
@@ -332,10 +341,7 @@ int run_fast(const Conv2dRequest &q, hipStream_t stream) {
     p.tiles_n = q.K / 256;
     p.xt_bytes = (unsigned)xt_bytes;
     conv2d_nhwc_kernel<T><<<dim3(p.tiles_m * p.tiles_n), dim3(512), 0, stream>>>(p);
-    err = hipGetLastError();
-    (void)hipFreeAsync(xt, stream);
-    (void)hipFreeAsync(wt, stream);
-    return (int)err;
+    return (int)hipGetLastError();
 }
 
 }  // namespace
@@ -349,7 +355,8 @@ int conv2d_fast(const Conv2dRequest &q, hipStream_t stream) {
     const int64_t wt_bytes = (int64_t)q.K * q.C * q.R * q.S * 2;
     if (xt_bytes >= (int64_t(1) << 31) || wt_bytes >= (int64_t(1) << 31)) return NINETOOTHED_NO_KERNEL;  // 32-bit buffer offsets
     if ((int64_t)q.N * ceil_div(q.P * q.Q, 256) * (q.K / 256) > 0x7fffffffll) return NINETOOTHED_NO_KERNEL;
-    // enough work to amortise the two repacking passes
+    if (q.N >= 65535 || ceil_div(q.C, 64) > 65535) return NINETOOTHED_NO_KERNEL;  // grid of the repacking pass: (positions, channels, images + 1)
+    // enough work to amortise the repacking pass
     if ((int64_t)q.N * q.P * q.Q < 1024) return NINETOOTHED_NO_KERNEL;
     return q.dtype == NINETOOTHED_FLOAT16 ? run_fast<half_t>(q, stream) : run_fast<bf16_t>(q, stream);
 }

@@ -108,12 +108,14 @@ def library():
                 function.restype = ctypes.c_int
             lib.nt_version.restype = ctypes.c_char_p
             lib.nt_version.argtypes = []
+            lib.nt_release_workspaces.restype = None
+            lib.nt_release_workspaces.argtypes = []
             _library = lib
     return _library
 
 
 def exported_symbols():
-    return tuple(_SIGNATURES) + ("nt_version",)
+    return tuple(_SIGNATURES) + ("nt_version", "nt_release_workspaces")
 
 
 def check(result):

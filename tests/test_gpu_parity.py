@@ -346,6 +346,33 @@ def test_conv2d_baseline_shape_and_1x1():
     assert torch.allclose(out.float(), as_matmul, **HALF_TOL)
 
 
+def test_scratch_buffers_are_reused_grown_and_released():
+    """conv2d's repacked operands and fp32 attention's narrowed K / V live in buffers the library
+    keeps per stream: a smaller call after a larger one, a larger one after that, another stream and
+    a call after nt_release_workspaces all have to give the same results."""
+    from ninetoothed_amd import runtime
+
+    def conv_case(n, c, hw, k):
+        x, w = _randn(n, c, hw, hw, scale=0.1).cuda(), _randn(k, c, 3, 3, scale=0.1).cuda()
+        return x, w, F.conv2d(x.float(), w.float(), padding=1).half()
+
+    cases = [conv_case(4, 64, 16, 256), conv_case(2, 32, 8, 256), conv_case(8, 64, 24, 512)]
+    side = torch.cuda.Stream()
+    for round_ in range(2):
+        for x, w, expected in cases:
+            assert torch.allclose(_conv2d(x, w, (1, 1)), expected, **HALF_TOL)
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            x, w, expected = cases[0]
+            assert torch.allclose(_conv2d(x, w, (1, 1)), expected, **HALF_TOL)
+        side.synchronize()
+        q, k, v = (torch.randn(1, 2, 300 - 100 * round_, 64, device="cuda") for _ in range(3))
+        o = _attention(q, k, v, scale=0.125)
+        assert torch.allclose(o, F.scaled_dot_product_attention(q, k, v, scale=0.125), rtol=0.025, atol=0.025)
+        torch.cuda.synchronize()
+        runtime.library().nt_release_workspaces()
+
+
 # ---- tile selection -------------------------------------------------------------
 
 
