@@ -459,9 +459,67 @@ struct MapCodegen {
     int counter = 0;
     std::string indent = "        ";
 
-    explicit MapCodegen(const NineToothedMapProgram &program) : p(program) {}
+    bool narrow;  // index arithmetic in 32 bits: every index value provably fits
+
+    explicit MapCodegen(const NineToothedMapProgram &program) : p(program), narrow(fits_int32(program)) {}
 
     std::string fresh(const char *prefix) { return prefix + std::to_string(counter++); }
+
+    const char *idx() const { return narrow ? "int" : "long long"; }
+    std::string lit(long long value) const { return std::to_string(value) + (narrow ? "" : "LL"); }
+    std::string ulit(long long value) const { return std::to_string(value) + (narrow ? "u" : "ULL"); }
+
+    // Interval evaluation of the index programs over the variables' ranges: true when the element
+    // count, every constant and every intermediate value stay within 31 bits (then `int` arithmetic
+    // computes the same offsets with a fraction of the instructions of 64-bit arithmetic).
+    static bool fits_int32(const NineToothedMapProgram &q) {
+        typedef __int128 wide;
+        const wide limit = (wide)1 << 31;
+        if (q.num_dynamic != 0) return false;
+        wide total = 1;
+        for (int v = 0; v < q.num_vars; ++v) {
+            if (q.extents[v] < 0 || (wide)q.extents[v] >= limit) return false;
+            if (v < q.num_vars - q.num_reduced) total *= q.extents[v] > 0 ? q.extents[v] : 1;
+            if (total >= ((wide)1 << 30)) return false;  // leaves room for the loop increment
+        }
+        for (int segment = 0; segment < q.num_segments; ++segment) {
+            std::vector<std::pair<wide, wide>> stack;
+            for (int pc = q.segment_begin[segment];; ++pc) {
+                const int op = q.index_code[pc] & 0xff, arg = q.index_code[pc] >> 8;
+                if (op == NT_MAP_I_END) break;
+                const wide c = op == NT_MAP_I_VAR ? 0 : (wide)q.index_constants[arg];
+                if (op != NT_MAP_I_VAR && op != NT_MAP_I_ADD && (c >= limit || c < -limit)) return false;
+                switch (op) {
+                    case NT_MAP_I_CONST: stack.push_back({c, c}); break;
+                    case NT_MAP_I_VAR: stack.push_back({0, q.extents[arg] > 0 ? (wide)q.extents[arg] - 1 : 0}); break;
+                    case NT_MAP_I_MULC: {
+                        const wide a = stack.back().first * c, b = stack.back().second * c;
+                        stack.back() = {a < b ? a : b, a < b ? b : a};
+                        break;
+                    }
+                    case NT_MAP_I_ADD: {
+                        const std::pair<wide, wide> b = stack.back();
+                        stack.pop_back();
+                        stack.back().first += b.first;
+                        stack.back().second += b.second;
+                        break;
+                    }
+                    case NT_MAP_I_DIVC:
+                    case NT_MAP_I_MODC: {  // never larger in magnitude than the operand (and the divisor)
+                        wide bound = stack.back().first < 0 ? -stack.back().first : stack.back().first;
+                        const wide other = stack.back().second < 0 ? -stack.back().second : stack.back().second;
+                        if (other > bound) bound = other;
+                        stack.back() = {-bound - 1, bound + 1};
+                        break;
+                    }
+                    case NT_MAP_I_CHECK: stack.pop_back(); break;
+                    default: return false;
+                }
+                if (!stack.empty() && (stack.back().first < -limit || stack.back().second >= limit)) return false;
+            }
+        }
+        return true;
+    }
 
     // emits the statements of one index segment; returns the offset expression and
     // and-s the checks into `valid` (a declared bool variable) when it is not empty
@@ -471,9 +529,9 @@ struct MapCodegen {
             const int op = p.index_code[pc] & 0xff, arg = p.index_code[pc] >> 8;
             if (op == NT_MAP_I_END) break;
             switch (op) {
-                case NT_MAP_I_CONST: stack.push_back(std::to_string((long long)p.index_constants[arg]) + "LL"); break;
+                case NT_MAP_I_CONST: stack.push_back(lit((long long)p.index_constants[arg])); break;
                 case NT_MAP_I_VAR: stack.push_back("v" + std::to_string(arg)); break;
-                case NT_MAP_I_MULC: stack.back() = "(" + stack.back() + " * " + std::to_string((long long)p.index_constants[arg]) + "LL)"; break;
+                case NT_MAP_I_MULC: stack.back() = "(" + stack.back() + " * " + lit((long long)p.index_constants[arg]) + ")"; break;
                 case NT_MAP_I_ADD: {
                     const std::string b = stack.back();
                     stack.pop_back();
@@ -483,22 +541,22 @@ struct MapCodegen {
                 case NT_MAP_I_DIVC:
                 case NT_MAP_I_MODC: {
                     const std::string name = fresh("i");
-                    const std::string c = std::to_string((long long)p.index_constants[arg]) + "LL";
-                    out << indent << "const long long " << name << " = " << (op == NT_MAP_I_DIVC ? "nt_floor_div(" : "nt_floor_mod(") << stack.back() << ", " << c << ");\n";
+                    const std::string c = lit((long long)p.index_constants[arg]);
+                    out << indent << "const " << idx() << " " << name << " = " << (op == NT_MAP_I_DIVC ? "nt_floor_div(" : "nt_floor_mod(") << stack.back() << ", " << c << ");\n";
                     stack.back() = name;
                     break;
                 }
                 case NT_MAP_I_CHECK: {
                     const std::string name = fresh("i");
-                    out << indent << "const long long " << name << " = " << stack.back() << ";\n";
-                    out << indent << valid << " = " << valid << " && " << name << " >= 0 && " << name << " < " << (long long)p.index_constants[arg] << "LL;\n";
+                    out << indent << "const " << idx() << " " << name << " = " << stack.back() << ";\n";
+                    out << indent << valid << " = " << valid << " && " << name << " >= 0 && " << name << " < " << lit((long long)p.index_constants[arg]) << ";\n";
                     stack.pop_back();
                     break;
                 }
             }
         }
         const std::string name = fresh("i");
-        out << indent << "const long long " << name << " = " << (stack.empty() ? std::string("0LL") : stack.back()) << ";\n";
+        out << indent << "const " << idx() << " " << name << " = " << (stack.empty() ? lit(0) : stack.back()) << ";\n";
         return name;
     }
 
@@ -585,7 +643,7 @@ struct MapCodegen {
                 stack.pop_back();
                 stack.back() = define("nt_philox_uniform((unsigned long long)(long long)" + stack.back() + ", (unsigned long long)(long long)" + offset + ")");
             } else if (op == NT_MAP_V_SETVAR) {
-                out << indent << "v" << arg << " = (long long)(" << stack.back() << ");\n";
+                out << indent << "v" << arg << " = (nt_idx)(" << stack.back() << ");\n";
                 stack.pop_back();
             }
         }
@@ -596,8 +654,10 @@ struct MapCodegen {
         const int num_out = p.num_vars - p.num_reduced;
         out << "struct MapJitArgs { void *data[" << NT_MAP_MAX_OPERANDS << "]; double other[" << NT_MAP_MAX_OPERANDS << "]; double constants["
             << NT_MAP_MAX_VALUE_CONSTANTS << "]; long long total_out; };\n"
-            << "__device__ inline long long nt_floor_div(long long a, long long b) { long long q = a / b; if ((a % b != 0) && ((a < 0) != (b < 0))) --q; return q; }\n"
-            << "__device__ inline long long nt_floor_mod(long long a, long long b) { return a - nt_floor_div(a, b) * b; }\n"
+            << "typedef " << idx() << " nt_idx;\n"
+            << "typedef unsigned " << idx() << " nt_uidx;  // element numbers are decoded unsigned: no sign fix-ups in the divisions\n"
+            << "__device__ inline nt_idx nt_floor_div(nt_idx a, nt_idx b) { nt_idx q = a / b; if ((a % b != 0) && ((a < 0) != (b < 0))) --q; return q; }\n"
+            << "__device__ inline nt_idx nt_floor_mod(nt_idx a, nt_idx b) { return a - nt_floor_div(a, b) * b; }\n"
             << "__device__ inline double nt_philox_uniform(unsigned long long seed, unsigned long long offset) {\n"
             << "    unsigned int c0 = (unsigned int)offset, c1 = (unsigned int)(offset >> 32), c2 = 0, c3 = 0;\n"
             << "    unsigned int k0 = (unsigned int)seed, k1 = (unsigned int)(seed >> 32);\n"
@@ -610,14 +670,13 @@ struct MapCodegen {
             << "    return (double)((float)x * 4.6566127342e-10f);\n"
             << "}\n"
             << "extern \"C\" __global__ __launch_bounds__(" << kMapThreads << ") void nt_map_specialised(const MapJitArgs a) {\n"
-            << "    const long long stride = (long long)gridDim.x * " << kMapThreads << ";\n"
-            << "    for (long long element = (long long)blockIdx.x * " << kMapThreads << " + threadIdx.x; element < a.total_out; element += stride) {\n"
-            << "        long long rest = element;\n";
-        for (int v = num_out - 1; v >= 0; --v) {
-            // 32-bit division when the extent allows it would be cheaper; the divisor is a literal either way
-            out << "        const long long v" << v << " = rest % " << (long long)p.extents[v] << "LL; rest /= " << (long long)p.extents[v] << "LL;\n";
-        }
-        for (int v = p.num_vars; v < p.num_vars + p.num_dynamic; ++v) out << "        long long v" << v << " = 0;\n";
+            << "    const nt_idx stride = (nt_idx)gridDim.x * " << kMapThreads << ";\n"
+            << "    const nt_idx total_out = (nt_idx)a.total_out;\n";
+        out << "    for (nt_idx element = (nt_idx)blockIdx.x * " << kMapThreads << " + threadIdx.x; element < total_out; element += stride) {\n"
+            << "        nt_uidx rest = (nt_uidx)element;\n";
+        for (int v = num_out - 1; v >= 0; --v)
+            out << "        const nt_idx v" << v << " = (nt_idx)(rest % " << ulit((long long)p.extents[v]) << "); rest /= " << ulit((long long)p.extents[v]) << ";\n";
+        for (int v = p.num_vars; v < p.num_vars + p.num_dynamic; ++v) out << "        nt_idx v" << v << " = 0;\n";
         std::string result;
         if (p.reduce_op == NT_MAP_REDUCE_NONE) {
             result = value_range(0, p.value_code_length, "");
@@ -625,7 +684,7 @@ struct MapCodegen {
             const char *init = p.reduce_op == NT_MAP_REDUCE_SUM ? "0.0" : (p.reduce_op == NT_MAP_REDUCE_MAX ? "-__builtin_inf()" : "__builtin_inf()");
             out << "        double acc = " << init << ";\n";
             for (int v = num_out; v < p.num_vars; ++v) {
-                out << indent << "for (long long v" << v << " = 0; v" << v << " < " << (long long)p.extents[v] << "LL; ++v" << v << ") {\n";
+                out << indent << "for (nt_idx v" << v << " = 0; v" << v << " < " << lit((long long)p.extents[v]) << "; ++v" << v << ") {\n";
                 indent += "    ";
             }
             const std::string term = value_range(0, p.reduce_split, "");

@@ -736,3 +736,18 @@ def test_jagged_to_padded_tensor_and_expand(jagged_dim, num_batches, interpret, 
     inside = ~torch.isnan(padded)
     assert inside.sum().item() == nested.values().numel()
     assert torch.equal(padded[inside], src.expand_as(padded)[inside])
+
+
+@gpu
+def test_offsets_beyond_32_bits():
+    """Specialised kernels compute offsets in 32 bits when every index provably fits; this one does not."""
+    kernel = ninetoothed.make(scalar_add_arrangement, scalar_add_application, (Tensor(1), Tensor(0), Tensor(1)))
+    n = (1 << 31) + 4096
+    input = torch.zeros(n, dtype=torch.int8, device="cuda")
+    input[-5:] = torch.arange(5, dtype=torch.int8, device="cuda")
+    input[:3] = 7
+    out = torch.full((n,), -1, dtype=torch.int8, device="cuda")
+    kernel(input, 1, out)
+    _served_by_map(kernel)
+    assert out[:4].tolist() == [8, 8, 8, 1] and out[-5:].tolist() == [1, 2, 3, 4, 5]
+    assert int(out.to(torch.int32).sum().item()) == n + 21 + 10
