@@ -433,7 +433,8 @@ class Tensor:
             env.update(_shape_environment(self.source, self.source.shape))
 
         levels, index_symbols, source_indices, constraints = self.index_map()
-        shape = [int(evaluate(size, env)) for level in levels for size in level.shape]
+        # a tile larger than its tensor, stepped by less than its size, has a negative count: no tiles
+        shape = [max(int(evaluate(size, env)), 0) for level in levels for size in level.shape]
         flat_symbols = [symbol for symbols in index_symbols for symbol in symbols]
         grids = np.ogrid[tuple(slice(0, extent) for extent in shape)] if shape else []
         for symbol, grid in zip(flat_symbols, grids):
