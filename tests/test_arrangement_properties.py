@@ -10,6 +10,7 @@ A random chain of meta-operations is applied, step by step, to a symbolic ``Tens
 """
 
 import numpy as np
+import pytest
 import torch
 from hypothesis import HealthCheck, assume, given, settings
 from hypothesis import strategies as st
@@ -120,6 +121,16 @@ def _clone_application(input, output):
     output = input  # noqa: F841
 
 
+def _run_machine(kernel, args):
+    env = kernel._environment(args, {}, check_device=False)
+    flat = {p: arg.reshape(-1).numpy() for p, arg in enumerate(args)}
+    for store in kernel.program.stores:
+        built = mapping.build(store, kernel.types, args, env, lambda p: _dtype_tag(_storage(args, p).dtype), lambda p: 0)
+        if built is not None:
+            program, _, _, operand_params = built
+            Machine(program, {slot: flat[p] for slot, p in enumerate(operand_params)}).run()
+
+
 @settings(max_examples=400, deadline=None, suppress_health_check=[HealthCheck.too_slow, HealthCheck.data_too_large, HealthCheck.filter_too_much])
 @given(shape=_shapes, data=st.data())
 def test_lowered_clone_copies_what_the_table_names(shape, data):
@@ -137,18 +148,50 @@ def test_lowered_clone_copies_what_the_table_names(shape, data):
         assume(False)
     source = torch.arange(1, int(np.prod(shape)) + 1, dtype=torch.float32).reshape(shape)
     out = torch.zeros(shape)
-    args = (source, out)
-    env = kernel._environment(args, {}, check_device=False)
-    flat = {0: source.reshape(-1).numpy(), 1: out.reshape(-1).numpy()}
     try:
-        for store in kernel.program.stores:
-            built = mapping.build(store, kernel.types, args, env, lambda p: _dtype_tag(_storage(args, p).dtype), lambda p: 0)
-            if built is not None:
-                program, _, _, operand_params = built
-                Machine(program, {slot: flat[p] for slot, p in enumerate(operand_params)}).run()
+        _run_machine(kernel, (source, out))
     except UnsupportedProgram:
         assume(False)  # limits of the executor (variables, code length), not wrong results
     named = view.table[view.table >= 0]
     expected = np.zeros(int(np.prod(shape)), dtype=np.float32)
     expected[named] = named + 1
     assert np.array_equal(out.reshape(-1).numpy(), expected), chain
+
+
+@pytest.mark.gpu
+@settings(max_examples=60, deadline=None, derandomize=True, suppress_health_check=list(HealthCheck))
+@given(shape=_shapes, data=st.data())
+def test_clone_on_the_gpu_copies_what_the_table_names(shape, data):
+    """The same property through ``launch_nt_map`` (specialised kernel and interpreter).  The numpy
+    machine runs first: the device only sees index programs that stayed in bounds there."""
+    import os
+
+    chain = _draw_chain(data, shape)
+    _, view = _arranged(chain, shape)
+    assume(len(view.levels) <= 2 and view.table.size > 0 and len(view.level_shape(0)) > 0)
+
+    def arrangement(input, output):
+        return _arranged(chain, shape, input)[0], _arranged(chain, shape, output)[0]
+
+    try:
+        kernel = ninetoothed.make(arrangement, _clone_application, (Tensor(len(shape)), Tensor(len(shape))))
+    except UnsupportedProgram:
+        assume(False)
+    source = torch.arange(1, int(np.prod(shape)) + 1, dtype=torch.float32).reshape(shape)
+    named = view.table[view.table >= 0]
+    expected = np.zeros(int(np.prod(shape)), dtype=np.float32)
+    expected[named] = named + 1
+    host_out = torch.zeros(shape)
+    try:
+        _run_machine(kernel, (source, host_out))
+    except UnsupportedProgram:
+        assume(False)
+    assert np.array_equal(host_out.reshape(-1).numpy(), expected), chain
+    for interpret in ("0", "1"):
+        os.environ["NT_MAP_INTERPRET"] = interpret
+        try:
+            out = torch.zeros(shape, device="cuda")
+            kernel(source.cuda(), out)
+            assert np.array_equal(out.cpu().reshape(-1).numpy(), expected), (interpret, chain)
+        finally:
+            os.environ.pop("NT_MAP_INTERPRET", None)
