@@ -708,6 +708,29 @@ class _Lowering:
         return code, constants, begins
 
 
+def _as_element(value, tag):
+    """``value`` as an element of type ``tag`` holds it (a masked load yields a tile of the
+    tensor's type, so `other` is rounded like any constant of that type)."""
+    import struct
+
+    if value != value or value in (float("inf"), float("-inf")):
+        return value
+    if tag == "fp16":
+        import numpy as np
+
+        with np.errstate(over="ignore"):
+            return float(np.float16(value))
+    if tag == "bf16":
+        bits = struct.unpack("<I", struct.pack("<f", value))[0]
+        bits = (bits + 0x7FFF + ((bits >> 16) & 1)) & 0xFFFF0000
+        return struct.unpack("<f", struct.pack("<I", bits & 0xFFFFFFFF))[0]
+    if tag == "fp32":
+        return struct.unpack("<f", struct.pack("<f", value))[0]
+    if tag == "fp64":
+        return float(value)
+    return float(int(value))
+
+
 def _other_value(tensor):
     if tensor is None:
         return 0.0
@@ -804,7 +827,7 @@ def build(program_store, types, args, env, dtype_tag, data_ptr):
         program.operands[slot].data = data_ptr(param)
         program.operands[slot].dtype = runtime.DATA_TYPE_INDEX[dtype_tag(param)]
         program.operands[slot].segment = lowering.segment_slot[(slot, "raw" if isinstance(operand, _RawOperand) else "access", None)]
-        program.operands[slot].other = _other_value(operand.tensor)
+        program.operands[slot].other = _as_element(_other_value(operand.tensor), dtype_tag(param))
     program.num_segments = len(begins)
     for index, begin in enumerate(begins):
         program.segment_begin[index] = begin
