@@ -647,9 +647,24 @@ class Tracer:
             self.stores.append((Node("pointer_" + func.name, self._value(args[0])), self._value(args[1])))
             return None
         if language.is_function(func):
+            # one spelling per call: trailing positional arguments that have a name become keywords,
+            # `dot(a, b, acc)` is `acc + dot(a, b)` (so equivalent applications share a digest)
+            args, kwargs = list(args), dict(kwargs)
+            names = _TRAILING_PARAMETERS.get(func.name)
+            if names is not None:
+                first, trailing = names
+                for name, value in zip(trailing, args[first:]):
+                    if name in kwargs:
+                        raise TracingError(f"`ntl.{func.name}` got `{name}` twice.")
+                    kwargs[name] = value
+                del args[first:]
+            accumulator = kwargs.pop("acc", None) if func.name == "dot" else None
             items = tuple(self._value(arg) for arg in args)
-            named = tuple(sorted((name, self._value(value)) for name, value in kwargs.items()))
-            return Node(func.name, *items, *[Node("kwarg", name, value) for name, value in named])
+            named = tuple(sorted((name, self._value(value)) for name, value in kwargs.items() if not (name == "keep_dims" and value is False) and not (name == "axis" and value is None)))
+            node = Node(func.name, *items, *[Node("kwarg", name, value) for name, value in named])
+            if accumulator is not None:
+                node = Node("add", self._value(accumulator), node)
+            return node
         if isinstance(func, _BoundMethod):
             return self._call_method(func, args, kwargs)
         if func is range:
@@ -706,6 +721,17 @@ class Tracer:
                 callee.aliases[keyword.arg] = (frame, keyword.value.id)
         self._exec_body(_function_tree(func).body, callee)
         return callee.returned[0] if callee.returned is not None else None
+
+
+# language functions whose trailing positional parameters have names: (leading positional count, names)
+_TRAILING_PARAMETERS = {
+    "zeros": (1, ("dtype",)),
+    "full": (2, ("dtype",)),
+    "sum": (1, ("axis", "keep_dims")),
+    "max": (1, ("axis", "keep_dims")),
+    "min": (1, ("axis", "keep_dims")),
+    "dot": (2, ("acc",)),
+}
 
 
 class _BoundMethod:

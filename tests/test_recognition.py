@@ -181,3 +181,32 @@ def test_kernel_call_checks_arguments_before_any_launch():
         kernel(torch.zeros(2, 2))
     with pytest.raises(RuntimeError, match="no CPU path"):
         kernel(torch.zeros(2, 2), torch.zeros(2, 2), BLOCK_SIZE=2)
+
+
+def test_equivalent_spellings_of_an_application_share_its_digest():
+    """`ntl.dot(a, b, acc)`, positional dtypes / axes and `+=` are spellings, not other programs."""
+
+    def with_accumulator_argument(lhs, rhs, output):
+        accumulator = ntl.zeros(output.shape, dtype=ntl.float32)
+        for k in range(lhs.shape[0]):
+            accumulator = ntl.dot(lhs[k], rhs[k], accumulator)
+        output = accumulator  # noqa: F841
+
+    def with_positional_dtype(lhs, rhs, output):
+        acc = ntl.zeros(output.shape, ntl.float32)
+        for k in range(lhs.shape[0]):
+            acc = acc + ntl.dot(lhs[k], rhs[k])
+        output = acc  # noqa: F841
+
+    def softmax_with_positional_axis(input, output):
+        input_loaded = input
+        row_minus_max = input_loaded - ntl.max(input_loaded, None)
+        numerator = ntl.exp(row_minus_max)
+        denominator = ntl.sum(numerator, None, False)
+        output = numerator / denominator  # noqa: F841
+
+    for application in (with_accumulator_argument, with_positional_dtype):
+        kernel = ninetoothed.make(programs.matmul.arrangement, application, programs.matmul.tensors())
+        assert kernel.kind == "matmul"
+    kernel = ninetoothed.make(programs.softmax.arrangement, softmax_with_positional_axis, programs.softmax.tensors())
+    assert kernel.kind == "softmax"
