@@ -270,6 +270,7 @@ int nt_tune_cache_lookup(int dtype, int output_dtype, int m, int n, int k, int a
 #define NT_MAP_MAX_SEGMENTS 16
 #define NT_MAP_MAX_VALUE_CODE 128
 #define NT_MAP_MAX_VALUE_CONSTANTS 32
+#define NT_MAP_MAX_PHASES 4
 
 enum NineToothedMapIndexOp {
     NT_MAP_I_END,    /* the offset is on top of the stack */
@@ -294,7 +295,8 @@ enum NineToothedMapValueOp {
     NT_MAP_V_WHERE,     /* pop b, a, c; push c ? a : b */
     NT_MAP_V_ROUND,     /* round top to NineToothedDataType arg (integers truncate) */
     NT_MAP_V_RAND,      /* pop offset, seed; push the Philox-4x32-10 uniform float of (seed, offset) */
-    NT_MAP_V_SETVAR     /* pop v; dynamic variable arg = (integer) v: a data-dependent level index */
+    NT_MAP_V_SETVAR,    /* pop v; dynamic variable arg = (integer) v: a data-dependent level index */
+    NT_MAP_V_REDUCED    /* tile mode: push the result of reduction phase arg (arg < the phase being computed) */
 };
 
 enum NineToothedMapReduceOp { NT_MAP_REDUCE_NONE, NT_MAP_REDUCE_MAX, NT_MAP_REDUCE_MIN, NT_MAP_REDUCE_SUM };
@@ -330,6 +332,19 @@ typedef struct {
     int32_t reduce_dtype;        /* type the reduction accumulates in (sums of fp16 / bf16: FLOAT32) */
     int32_t value_code[NT_MAP_MAX_VALUE_CODE];
     double value_constants[NT_MAP_MAX_VALUE_CONSTANTS];
+    /* Tile mode (num_phases > 0; needs reduce_op == NONE, num_reduced == num_dynamic == 0, a plain
+     * store): whole-tile reductions whose results the stored expression uses on every element of
+     * the tile (normalisations: `x / ntl.sum(x)`, `(x - mean) * ntl.rsqrt(var + eps)`, ...).  The
+     * first num_grid variables enumerate the tiles, the others the elements of a tile.  One
+     * workgroup takes a tile: for k = 0 .. num_phases - 1 it reduces, over the tile's elements,
+     * the term value_code[phase_end[k-1] .. phase_end[k]) (phase_end[-1] = 0) with phase_op[k],
+     * accumulating in phase_dtype[k]; then value_code[phase_end[num_phases-1] .. value_code_length)
+     * is evaluated and stored per element.  NT_MAP_V_REDUCED reads an earlier phase's result. */
+    int32_t num_phases;
+    int32_t num_grid;
+    int32_t phase_end[NT_MAP_MAX_PHASES];
+    int32_t phase_op[NT_MAP_MAX_PHASES];     /* NineToothedMapReduceOp, not NONE */
+    int32_t phase_dtype[NT_MAP_MAX_PHASES];
 } NineToothedMapProgram;
 
 /* Runs one store of such a program.  Returns NINETOOTHED_NO_KERNEL when the

@@ -163,7 +163,7 @@ __device__ __forceinline__ double philox_uniform(uint64_t seed, uint64_t offset)
 
 // runs value_code[begin, end) on a stack that starts as `initial` (when `seeded`)
 __device__ __forceinline__ double run_value(const NineToothedMapProgram &p, int begin, int end, int64_t *vars, bool seeded,
-                                             double initial) {
+                                             double initial, const double *reduced = nullptr) {
     double stack[kValueStack];
     int top = -1;
     if (seeded) stack[++top] = initial;
@@ -245,6 +245,7 @@ __device__ __forceinline__ double run_value(const NineToothedMapProgram &p, int 
                 break;
             }
             case NT_MAP_V_SETVAR: vars[arg] = (int64_t)stack[top--]; break;
+            case NT_MAP_V_REDUCED: stack[++top] = reduced[arg]; break;
             default: break;
         }
     }
@@ -298,6 +299,70 @@ __global__ __launch_bounds__(kMapThreads) void map_kernel(const NineToothedMapPr
     }
 }
 
+// acc (op) term with the rounding / NaN rules of the element kernel's reductions
+__device__ __forceinline__ double reduce_combine(int op, int dtype, double acc, double term) {
+    if (op == NT_MAP_REDUCE_SUM) return round_to(acc + term, dtype);
+    if (term != term || acc != acc) return acc + term;  // NaN propagates
+    if (op == NT_MAP_REDUCE_MAX) return term > acc ? term : acc;
+    return term < acc ? term : acc;
+}
+
+__device__ __forceinline__ double reduce_identity(int op) {
+    return op == NT_MAP_REDUCE_SUM ? 0.0 : (op == NT_MAP_REDUCE_MAX ? -INFINITY : INFINITY);
+}
+
+// all threads of the workgroup get the combination of everybody's `value`
+__device__ __forceinline__ double block_reduce(int op, int dtype, double value, double *scratch) {
+    for (int offset = 32; offset > 0; offset >>= 1) value = reduce_combine(op, dtype, value, __shfl_xor(value, offset, 64));
+    constexpr int kWaves = kMapThreads / 64;
+    __syncthreads();  // scratch may still be read from the previous phase
+    if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = value;
+    __syncthreads();
+    value = scratch[0];
+    for (int w = 1; w < kWaves; ++w) value = reduce_combine(op, dtype, value, scratch[w]);
+    return value;
+}
+
+// Tile mode: one workgroup per tile; phases of whole-tile reductions, then the stored expression.
+__global__ __launch_bounds__(kMapThreads) void map_tile_kernel(const NineToothedMapProgram p, int64_t tiles, int64_t tile_elements) {
+    __shared__ double scratch[kMapThreads / 64];
+    for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+        int64_t vars[NT_MAP_MAX_VARS];
+        int64_t rest = tile;
+        for (int v = p.num_grid - 1; v >= 0; --v) {
+            const int64_t extent = p.extents[v];
+            vars[v] = rest % extent;
+            rest /= extent;
+        }
+        auto decode = [&](int64_t element) {
+            for (int v = p.num_vars - 1; v >= p.num_grid; --v) {
+                const int64_t extent = p.extents[v];
+                vars[v] = element % extent;
+                element /= extent;
+            }
+        };
+        double reduced[NT_MAP_MAX_PHASES];
+        int begin = 0;
+        for (int k = 0; k < p.num_phases; ++k) {
+            double acc = reduce_identity(p.phase_op[k]);
+            for (int64_t element = threadIdx.x; element < tile_elements; element += kMapThreads) {
+                decode(element);
+                acc = reduce_combine(p.phase_op[k], p.phase_dtype[k], acc, run_value(p, begin, p.phase_end[k], vars, false, 0.0, reduced));
+            }
+            reduced[k] = block_reduce(p.phase_op[k], p.phase_dtype[k], acc, scratch);
+            begin = p.phase_end[k];
+        }
+        const NineToothedMapOperand &out = p.operands[p.output];
+        for (int64_t element = threadIdx.x; element < tile_elements; element += kMapThreads) {
+            decode(element);
+            const double value = run_value(p, begin, p.value_code_length, vars, false, 0.0, reduced);
+            bool valid = true;
+            const int64_t offset = run_index(p, out.segment, vars, valid);
+            if (valid) store_element(out.data, out.dtype, offset, value);
+        }
+    }
+}
+
 bool well_formed(const NineToothedMapProgram &p) {
     if (p.num_vars < 0 || p.num_vars > NT_MAP_MAX_VARS || p.num_reduced < 0 || p.num_reduced > p.num_vars) return false;
     if (p.num_dynamic < 0 || p.num_vars + p.num_dynamic > NT_MAP_MAX_VARS) return false;
@@ -347,8 +412,26 @@ bool well_formed(const NineToothedMapProgram &p) {
             if (depth > kIndexStack) return false;
         }
     }
+    if (p.num_phases < 0 || p.num_phases > NT_MAP_MAX_PHASES) return false;
+    if (p.num_phases > 0) {
+        if (p.reduce_op != NT_MAP_REDUCE_NONE || p.num_dynamic != 0 || p.store_op != NT_MAP_STORE_ASSIGN) return false;
+        if (p.num_grid < 0 || p.num_grid > p.num_vars) return false;
+        int previous = 0;
+        for (int k = 0; k < p.num_phases; ++k) {
+            if (p.phase_end[k] <= previous || p.phase_end[k] >= p.value_code_length) return false;
+            if (p.phase_op[k] < NT_MAP_REDUCE_MAX || p.phase_op[k] > NT_MAP_REDUCE_SUM) return false;
+            if (p.phase_dtype[k] < NINETOOTHED_INT8 || p.phase_dtype[k] > NINETOOTHED_FLOAT64) return false;
+            previous = p.phase_end[k];
+        }
+    }
     int depth = 0;
+    int phase = 0;  // the phase the code at `pc` belongs to (num_phases: the stored expression)
     for (int pc = 0; pc < p.value_code_length; ++pc) {
+        if (phase < p.num_phases && pc == p.phase_end[phase]) {
+            if (depth != 1) return false;  // a phase leaves exactly its term
+            depth = 0;
+            ++phase;
+        }
         if (pc == p.reduce_split && p.reduce_op != NT_MAP_REDUCE_NONE) {
             if (depth != 1) return false;  // the per-position code leaves exactly the term
         }
@@ -378,6 +461,9 @@ bool well_formed(const NineToothedMapProgram &p) {
         } else if (op == NT_MAP_V_SETVAR) {
             if (depth < 1 || arg < p.num_vars || arg >= p.num_vars + p.num_dynamic) return false;
             --depth;
+        } else if (op == NT_MAP_V_REDUCED) {
+            if (arg < 0 || arg >= phase) return false;
+            ++depth;
         } else {
             return false;
         }
@@ -645,9 +731,63 @@ struct MapCodegen {
             } else if (op == NT_MAP_V_SETVAR) {
                 out << indent << "v" << arg << " = (nt_idx)(" << stack.back() << ");\n";
                 stack.pop_back();
+            } else if (op == NT_MAP_V_REDUCED) {
+                stack.push_back("r" + std::to_string(arg));
             }
         }
         return stack.empty() ? std::string("0.0") : stack.back();
+    }
+
+    std::string combine_expr(int op, int dtype, const std::string &acc, const std::string &term) {
+        if (op == NT_MAP_REDUCE_SUM) return round_expr(acc + " + " + term, dtype);
+        const char *cmp = op == NT_MAP_REDUCE_MAX ? ">" : "<";
+        return "(" + term + " != " + term + " || " + acc + " != " + acc + ") ? " + acc + " + " + term + " : (" + term + " " + cmp + " " + acc + " ? " + term + " : " + acc + ")";
+    }
+
+    void decode_tile_variables() {
+        out << indent << "nt_uidx rest = (nt_uidx)element;\n";
+        for (int v = p.num_vars - 1; v >= p.num_grid; --v)
+            out << indent << "const nt_idx v" << v << " = (nt_idx)(rest % " << ulit((long long)p.extents[v]) << "); rest /= " << ulit((long long)p.extents[v]) << ";\n";
+    }
+
+    // one workgroup per tile: reduction phases, then the stored expression (see the tile mode of the header)
+    std::string generate_tile() {
+        long long tiles = 1, tile_elements = 1;
+        for (int v = 0; v < p.num_vars; ++v) (v < p.num_grid ? tiles : tile_elements) *= (long long)p.extents[v];
+        out << "    __shared__ double scratch[" << kMapThreads / 64 << "];\n"
+            << "    for (nt_idx tile = (nt_idx)blockIdx.x; tile < " << lit(tiles) << "; tile += (nt_idx)gridDim.x) {\n"
+            << "        nt_uidx tile_rest = (nt_uidx)tile;\n";
+        for (int v = p.num_grid - 1; v >= 0; --v)
+            out << "        const nt_idx v" << v << " = (nt_idx)(tile_rest % " << ulit((long long)p.extents[v]) << "); tile_rest /= " << ulit((long long)p.extents[v]) << ";\n";
+        int begin = 0;
+        for (int k = 0; k < p.num_phases; ++k) {
+            const int op = p.phase_op[k], dtype = p.phase_dtype[k];
+            const char *init = op == NT_MAP_REDUCE_SUM ? "0.0" : (op == NT_MAP_REDUCE_MAX ? "-__builtin_inf()" : "__builtin_inf()");
+            out << "        double r" << k << ";\n        {\n            double acc = " << init << ";\n"
+                << "            for (nt_idx element = threadIdx.x; element < " << lit(tile_elements) << "; element += " << kMapThreads << ") {\n";
+            indent = "                ";
+            decode_tile_variables();
+            const std::string term = value_range(begin, p.phase_end[k], "");
+            out << indent << "acc = " << combine_expr(op, dtype, "acc", term) << ";\n"
+                << "            }\n"
+                << "            for (int offset = 32; offset > 0; offset >>= 1) { const double other = __shfl_xor(acc, offset, 64); acc = "
+                << combine_expr(op, dtype, "acc", "other") << "; }\n"
+                << "            __syncthreads();\n            if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = acc;\n            __syncthreads();\n"
+                << "            acc = scratch[0];\n"
+                << "            for (int w = 1; w < " << kMapThreads / 64 << "; ++w) { const double other = scratch[w]; acc = " << combine_expr(op, dtype, "acc", "other")
+                << "; }\n            r" << k << " = acc;\n        }\n";
+            begin = p.phase_end[k];
+        }
+        const NineToothedMapOperand &target = p.operands[p.output];
+        out << "        for (nt_idx element = threadIdx.x; element < " << lit(tile_elements) << "; element += " << kMapThreads << ") {\n";
+        indent = "            ";
+        decode_tile_variables();
+        const std::string result = value_range(begin, p.value_code_length, "");
+        out << indent << "bool store_ok = true;\n";
+        const std::string offset = index_segment(target.segment, "store_ok");
+        out << indent << "if (store_ok) " << store_stmt("a.data[" + std::to_string(p.output) + "]", target.dtype, offset, result) << "\n"
+            << "        }\n    }\n}\n";
+        return out.str();
     }
 
     std::string generate() {
@@ -672,6 +812,7 @@ struct MapCodegen {
             << "extern \"C\" __global__ __launch_bounds__(" << kMapThreads << ") void nt_map_specialised(const MapJitArgs a) {\n"
             << "    const nt_idx stride = (nt_idx)gridDim.x * " << kMapThreads << ";\n"
             << "    const nt_idx total_out = (nt_idx)a.total_out;\n";
+        if (p.num_phases > 0) return generate_tile();
         out << "    for (nt_idx element = (nt_idx)blockIdx.x * " << kMapThreads << " + threadIdx.x; element < total_out; element += stride) {\n"
             << "        nt_uidx rest = (nt_uidx)element;\n";
         for (int v = num_out - 1; v >= 0; --v)
@@ -761,6 +902,8 @@ hipFunction_t specialised_kernel(const NineToothedMapProgram &p) {
     for (int v = p.num_vars; v < NT_MAP_MAX_VARS; ++v) shape.extents[v] = 0;
     for (int i = p.num_segments; i < NT_MAP_MAX_SEGMENTS; ++i) shape.segment_begin[i] = 0;
     for (int i = p.value_code_length; i < NT_MAP_MAX_VALUE_CODE; ++i) shape.value_code[i] = 0;
+    for (int k = p.num_phases; k < NT_MAP_MAX_PHASES; ++k) shape.phase_end[k] = shape.phase_op[k] = shape.phase_dtype[k] = 0;
+    if (p.num_phases == 0) shape.num_grid = 0;
     std::string key((const char *)&shape, sizeof(shape));
     key.push_back((char)device);
     std::lock_guard<std::mutex> lock(g_jit_mutex);
@@ -820,6 +963,11 @@ extern "C" NineToothedResult launch_nt_map(NineToothedStream stream, const NineT
     // enough workgroups for 8 per CU; the grid stride covers the rest
     int64_t blocks = (total_out + kMapThreads - 1) / kMapThreads;
     if (blocks > 256 * 32) blocks = 256 * 32;
+    int64_t tiles = 1, tile_elements = 1;
+    if (p.num_phases > 0) {  // tile mode: one workgroup per tile
+        for (int v = 0; v < p.num_vars; ++v) (v < p.num_grid ? tiles : tile_elements) *= p.extents[v];
+        blocks = tiles < 256 * 32 ? tiles : 256 * 32;
+    }
     const char *interpret = getenv("NT_MAP_INTERPRET");
     if (!(interpret && interpret[0] == '1')) {
         if (hipFunction_t function = specialised_kernel(p)) {
@@ -835,7 +983,10 @@ extern "C" NineToothedResult launch_nt_map(NineToothedStream stream, const NineT
             return (int)hipModuleLaunchKernel(function, (unsigned)blocks, 1, 1, kMapThreads, 1, 1, 0, (hipStream_t)stream, nullptr, config);
         }
     }
-    map_kernel<<<dim3((unsigned)blocks), dim3(kMapThreads), 0, (hipStream_t)stream>>>(p, total_out, total_reduced);
+    if (p.num_phases > 0)
+        map_tile_kernel<<<dim3((unsigned)blocks), dim3(kMapThreads), 0, (hipStream_t)stream>>>(p, tiles, tile_elements);
+    else
+        map_kernel<<<dim3((unsigned)blocks), dim3(kMapThreads), 0, (hipStream_t)stream>>>(p, total_out, total_reduced);
     return (int)hipGetLastError();
 }
 

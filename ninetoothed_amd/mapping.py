@@ -35,7 +35,8 @@ import ctypes
 from ninetoothed_amd import runtime
 from ninetoothed_amd.affine import Affine
 from ninetoothed_amd.recognition import Operand, UnsupportedProgram
-from ninetoothed_amd.tracing import ElementType, Node, ScalarParam, SourceDim, SourceStride, TensorRef
+from ninetoothed_amd.symbol import evaluate
+from ninetoothed_amd.tracing import Dim, ElementType, Node, ScalarParam, SourceDim, SourceStride, TensorRef
 
 MAX_OPERANDS = 8
 MAX_VARS = 16
@@ -44,12 +45,13 @@ MAX_INDEX_CONSTANTS = 96
 MAX_SEGMENTS = 16
 MAX_VALUE_CODE = 128
 MAX_VALUE_CONSTANTS = 32
+MAX_PHASES = 4
 
 I_END, I_CONST, I_VAR, I_MULC, I_ADD, I_DIVC, I_MODC, I_CHECK = range(8)
 
 _VALUE_OPS = (
     "LOAD CONST OFFSET ADD SUB MUL DIV FLOORDIV MOD POW MAX MIN LT LE GT GE EQ NE AND OR "
-    "NEG NOT ABS EXP EXP2 LOG LOG2 SQRT RSQRT SIGMOID TANH SIN COS FLOOR CEIL WHERE ROUND RAND SETVAR"
+    "NEG NOT ABS EXP EXP2 LOG LOG2 SQRT RSQRT SIGMOID TANH SIN COS FLOOR CEIL WHERE ROUND RAND SETVAR REDUCED"
 ).split()
 V = {name: index for index, name in enumerate(_VALUE_OPS)}
 
@@ -80,6 +82,11 @@ class MapProgram(ctypes.Structure):
         ("reduce_dtype", ctypes.c_int32),
         ("value_code", ctypes.c_int32 * MAX_VALUE_CODE),
         ("value_constants", ctypes.c_double * MAX_VALUE_CONSTANTS),
+        ("num_phases", ctypes.c_int32),
+        ("num_grid", ctypes.c_int32),
+        ("phase_end", ctypes.c_int32 * MAX_PHASES),
+        ("phase_op", ctypes.c_int32 * MAX_PHASES),
+        ("phase_dtype", ctypes.c_int32 * MAX_PHASES),
     ]
 
 
@@ -218,8 +225,13 @@ def _first_tile_ref(value):
 class _Lowering:
     """One store of one call: collects operands, index segments and value code."""
 
-    def __init__(self, types, args, env, dtype_tag):
+    def __init__(self, types, args, env, dtype_tag, tile_mode=False):
         self.types, self.args, self.env, self.dtype_tag = types, args, env, dtype_tag
+        # tile mode: whole-tile reductions become phases whose results the expression may use on
+        # every element of the tile; `phases` holds (operation, accumulate type, term code)
+        self.tile_mode = tile_mode
+        self.phases = []
+        self.phase_of = {}        # digest of a reduction -> (phase, type of its term, type it accumulates in)
         self.operands = []        # (param, Operand)
         self.operand_slot = {}    # param -> slot
         self.var_extent = []      # shared variables: grid dims first, then output tile dims, then reduced dims
@@ -349,6 +361,10 @@ class _Lowering:
             name = source.size_string(value.dim) if isinstance(value, SourceDim) else source.stride_string(value.dim)
             self.emit("CONST", self.constant(int(self.env[name])))
             return _LITERAL_INT
+        if isinstance(value, Dim):  # `x.shape[d]` of a level: a call-time integer
+            level = self.types[value.param].levels()[value.level]
+            self.emit("CONST", self.constant(int(evaluate(level.shape[value.dim], self.env))))
+            return _LITERAL_INT
         if not isinstance(value, Node):
             raise UnsupportedProgram(f"A value of type `{type(value).__name__}` cannot be stored by the element-wise executor.")
 
@@ -455,6 +471,36 @@ class _Lowering:
             self.lower(positional[1], dims, inside_reduction)
             self.emit("RAND")
             return "fp32"
+        if op in REDUCE and self.tile_mode:
+            positional, named = _kwargs(value)
+            axis = named.get("axis", positional[1] if len(positional) > 1 else None)
+            if axis is not None:
+                raise UnsupportedProgram("Only reductions over a whole tile can be combined with the elements of the tile.")
+            if self._tile_rank(positional[0]) != len(dims):
+                raise UnsupportedProgram("A reduction whose result is used on a tile must run over tiles of that tile's shape.")
+            if value.digest in self.phase_of:  # the same reduction used again: one phase serves every use
+                k, term, accumulate = self.phase_of[value.digest]
+                self.emit("REDUCED", k)
+                if accumulate != term:
+                    self.round(term)
+                return term
+            outer_code, self.value_code = self.value_code, []
+            try:
+                term = self.lower(positional[0], dims, inside_reduction)
+                code = self.value_code
+            finally:
+                self.value_code = outer_code
+            if term in (_LITERAL_INT, _LITERAL_FLOAT):
+                raise UnsupportedProgram("A reduction needs a tile operand.")
+            if len(self.phases) >= MAX_PHASES:
+                raise UnsupportedProgram("Too many reductions in one stored expression.")
+            accumulate = "fp32" if op == "sum" and term in ("fp16", "bf16") else term
+            self.phases.append((op, accumulate, code))
+            self.phase_of[value.digest] = (len(self.phases) - 1, term, accumulate)
+            self.emit("REDUCED", len(self.phases) - 1)
+            if accumulate != term:
+                self.round(term)
+            return term
         if op in REDUCE:
             if self.reduce is not None or inside_reduction:
                 raise UnsupportedProgram("Only one reduction per stored expression is supported.")
@@ -738,12 +784,36 @@ def _other_value(tensor):
     return 0.0 if other is None else float(other)
 
 
+def _has_whole_tile_reduction(value):
+    if isinstance(value, Node):
+        if value.op in REDUCE:
+            positional, named = _kwargs(value)
+            if named.get("axis", positional[1] if len(positional) > 1 else None) is None:
+                return True
+        return any(_has_whole_tile_reduction(arg) for arg in value.args)
+    if isinstance(value, (tuple, list)):
+        return any(_has_whole_tile_reduction(item) for item in value)
+    return False
+
+
 def build(program_store, types, args, env, dtype_tag, data_ptr):
     """Builds the :class:`MapProgram` of one store for one call.  Returns
-    ``None`` when the launch is empty."""
+    ``None`` when the launch is empty.
 
+    A reduction is first tried as the innermost operation of the expression (one result per
+    output element); when the expression does not have that form but reduces whole tiles, the
+    program is built in tile mode (reductions as phases of a workgroup that owns the tile)."""
+    try:
+        return _build(program_store, types, args, env, dtype_tag, data_ptr, False)
+    except UnsupportedProgram:
+        if not isinstance(program_store[0], TensorRef) or not _has_whole_tile_reduction(program_store[1]):
+            raise
+        return _build(program_store, types, args, env, dtype_tag, data_ptr, True)
+
+
+def _build(program_store, types, args, env, dtype_tag, data_ptr, tile_mode):
     ref, value = program_store
-    lowering = _Lowering(types, args, env, dtype_tag)
+    lowering = _Lowering(types, args, env, dtype_tag, tile_mode)
     store_op = 0
     if isinstance(ref, TensorRef):
         lowering._check_ref(ref)
@@ -779,6 +849,16 @@ def build(program_store, types, args, env, dtype_tag, data_ptr):
         if result != out_dtype:
             lowering.emit("ROUND", runtime.DATA_TYPE_INDEX[out_dtype])
         out_slot = lowering.raw_access(out_param, indices, out_dims, False, element_offset=offset)
+    if tile_mode:
+        if lowering.dynamic_vars or lowering.reduce is not None or not lowering.phases or store_op != 0:
+            raise UnsupportedProgram("Whole-tile reductions cannot be combined with data-dependent indices or atomic stores.")
+        # phases first (in the order they were completed: a phase only uses earlier ones), then the stored expression
+        final_code, lowering.value_code = lowering.value_code, []
+        phase_ends = []
+        for _, _, code in lowering.phases:
+            lowering.value_code += code
+            phase_ends.append(len(lowering.value_code))
+        lowering.value_code += final_code
     if lowering.reduce is None:
         lowering.reduce_split = len(lowering.value_code)
     for slot, (_, operand) in enumerate(lowering.operands):
@@ -800,6 +880,9 @@ def build(program_store, types, args, env, dtype_tag, data_ptr):
             stride_of[var] = abs(offset.coef(name)) if offset.is_linear() else None
     if order_slot is not None and all(stride_of.get(v) is not None for v in outer):
         outer.sort(key=lambda v: (-(stride_of[v] or 1 << 62) if lowering.var_extent[v] > 1 else -(1 << 62), v))
+    if tile_mode:  # the variables that enumerate tiles first, then those of the tile (fastest last, as sorted)
+        grid_vars = [v for v in outer if v in lowering.grid]
+        outer = grid_vars + [v for v in outer if v not in lowering.grid]
     order = {old: new for new, old in enumerate(outer + reduced + dynamic)}
     # SETVAR words were emitted with provisional ids: renumber them like the index code
     for position, word in enumerate(lowering.value_code):
@@ -821,6 +904,13 @@ def build(program_store, types, args, env, dtype_tag, data_ptr):
     for old, new in order.items():
         program.extents[new] = lowering.var_extent[old]
     program.store_op = store_op
+    if tile_mode:
+        program.num_phases = len(lowering.phases)
+        program.num_grid = len(grid_vars)
+        for k, (op, accumulate, _) in enumerate(lowering.phases):
+            program.phase_end[k] = phase_ends[k]
+            program.phase_op[k] = REDUCE[op]
+            program.phase_dtype[k] = runtime.DATA_TYPE_INDEX[accumulate]
     program.num_operands = len(lowering.operands)
     program.output = out_slot
     for slot, (param, operand) in enumerate(lowering.operands):
@@ -849,6 +939,7 @@ def build(program_store, types, args, env, dtype_tag, data_ptr):
         + 
         f"{len(code)} index words, {len(lowering.value_code)} value words"
         + (f", {lowering.reduce[0]} over {len(reduced)} dimension(s)" if lowering.reduce else "")
+        + (f", {len(lowering.phases)} whole-tile reduction(s), one workgroup per tile" if tile_mode else "")
     )
     return program, description, list(lowering.scalar_slots), [param for param, _ in lowering.operands]
 

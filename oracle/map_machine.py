@@ -104,7 +104,7 @@ class Machine:
             else:
                 raise ValueError(f"unknown index opcode {op}")
 
-    def run_value(self, begin, end, variables, initial=None):
+    def run_value(self, begin, end, variables, initial=None, reduced=()):
         p = self.p
         V = mapping.V
         names = {index: name for name, index in V.items()}
@@ -150,6 +150,8 @@ class Machine:
                     stack.append(philox_uniform(seed.astype(np.int64), offset.astype(np.int64)))
                 elif op == "SETVAR":
                     variables[arg] = np.broadcast_to(np.trunc(stack.pop()).astype(np.int64), shape)
+                elif op == "REDUCED":
+                    stack.append(reduced[arg])
                 else:
                     a = stack.pop()
                     f32 = a.astype(np.float32)
@@ -164,8 +166,37 @@ class Machine:
                     }[op]())
         return stack[-1]
 
+    def run_tiles(self):
+        """Tile mode: whole-tile reductions as phases, then the stored expression on every element."""
+        p = self.p
+        grid_extents = [p.extents[v] for v in range(p.num_grid)]
+        tile_extents = [p.extents[v] for v in range(p.num_grid, p.num_vars)]
+        tiles = int(np.prod(grid_extents)) if grid_extents else 1
+        elements = int(np.prod(tile_extents)) if tile_extents else 1
+        if tiles == 0 or elements == 0:
+            return
+        tile_number, element_number = np.divmod(np.arange(tiles * elements), elements)
+        variables = [np.asarray(g) for g in (np.unravel_index(tile_number, grid_extents) if grid_extents else ())]
+        variables += [np.asarray(g) for g in (np.unravel_index(element_number, tile_extents) if tile_extents else ())]
+        reduced = []
+        begin = 0
+        for k in range(p.num_phases):
+            term = np.broadcast_to(self.run_value(begin, p.phase_end[k], variables, reduced=reduced), (tiles * elements,)).reshape(tiles, elements)
+            if p.phase_op[k] == 3:
+                result = round_to(term.sum(axis=1), p.phase_dtype[k])  # any summation order is as good as the kernel's tree
+            elif p.phase_op[k] == 1:
+                result = term.max(axis=1)
+            else:
+                result = term.min(axis=1)
+            reduced.append(np.repeat(result, elements))
+            begin = p.phase_end[k]
+        value = self.run_value(begin, p.value_code_length, variables, reduced=reduced)
+        self._store(value, variables)
+
     def run(self):
         p = self.p
+        if p.num_phases:
+            return self.run_tiles()
         num_out = p.num_vars - p.num_reduced
         out_extents = [p.extents[v] for v in range(num_out)]
         total = int(np.prod(out_extents)) if out_extents else 1
@@ -189,6 +220,10 @@ class Machine:
                 else:
                     acc = np.minimum(acc, term)
             value = self.run_value(p.reduce_split, p.value_code_length, variables, initial=acc)
+        self._store(value, variables)
+
+    def _store(self, value, variables):
+        p = self.p
         out = p.operands[p.output]
         offset, valid = self.run_index(out.segment, variables)
         target = self.arrays[p.output]

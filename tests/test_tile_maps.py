@@ -751,3 +751,89 @@ def test_offsets_beyond_32_bits():
     _served_by_map(kernel)
     assert out[:4].tolist() == [8, 8, 8, 1] and out[-5:].tolist() == [1, 2, 3, 4, 5]
     assert int(out.to(torch.int32).sum().item()) == n + 21 + 10
+
+
+# ---- whole-tile reductions used on the elements of the tile (normalisations) ---------------------
+
+
+def _rows(tensor):
+    arranged = tensor.tile((1, -1)).squeeze(1)
+    arranged.dtype = arranged.dtype.squeeze(0)
+    return arranged
+
+
+def _row_arrangement(input, output):
+    return _rows(input), _rows(output)
+
+
+def _row_weight_arrangement(input, weight, output):
+    return _rows(input), weight.tile((-1,)).expand((input.shape[0],)), _rows(output)
+
+
+def _scaled_softmax_application(input, output):
+    shifted = input * 2 - ntl.max(input * 2)
+    numerator = ntl.exp(shifted)
+    output = numerator / ntl.sum(numerator)  # noqa: F841
+
+
+def _rms_norm_application(input, weight, output):
+    mean_square = ntl.sum(input * input) / input.shape[-1]
+    output = input * ntl.rsqrt(mean_square + 1e-6) * weight  # noqa: F841
+
+
+def _layer_norm_application(input, weight, output):
+    mean = ntl.sum(input) / input.shape[-1]
+    centred = input - mean
+    variance = ntl.sum(centred * centred) / input.shape[-1]
+    output = centred * ntl.rsqrt(variance + 1e-5) * weight  # noqa: F841
+
+
+def _normalisation_cases(device, dtype=torch.float32, rows=7, cols=300):
+    x = torch.randn(rows, cols, device=device, dtype=dtype)
+    w = torch.randn(cols, device=device, dtype=dtype)
+    xf, wf = x.float(), w.float()
+    softmax = ninetoothed.make(_row_arrangement, _scaled_softmax_application, (Tensor(2), Tensor(2)))
+    rms_norm = ninetoothed.make(_row_weight_arrangement, _rms_norm_application, (Tensor(2), Tensor(1), Tensor(2)))
+    layer_norm = ninetoothed.make(_row_weight_arrangement, _layer_norm_application, (Tensor(2), Tensor(1), Tensor(2)))
+    return (
+        (softmax, (x,), torch.softmax(xf * 2, -1)),
+        (rms_norm, (x, w), xf * torch.rsqrt((xf * xf).mean(-1, keepdim=True) + 1e-6) * wf),
+        (layer_norm, (x, w), F.layer_norm(xf, (cols,), wf, None, 1e-5)),
+    )
+
+
+def test_lowering_whole_tile_reductions_in_tile_mode():
+    for kernel, inputs, expected in _normalisation_cases("cpu"):
+        assert kernel.kind == "map"
+        out = torch.full_like(inputs[0], float("nan"))
+        _run_on_machine(kernel, (*inputs, out))
+        assert torch.allclose(out, expected, rtol=1e-5, atol=1e-6)
+
+
+def test_tile_mode_program_layout():
+    kernel, inputs, _ = _normalisation_cases("cpu")[2]
+    out = torch.empty_like(inputs[0])
+    args = (*inputs, out)
+    env = kernel._environment(args, {}, check_device=False)
+    program, description, _, _ = mapping.build(kernel.program.stores[0], kernel.types, args, env, lambda p: _dtype_tag(args[p].dtype), lambda p: 0)
+    assert program.num_phases == 2 and program.num_grid == 1 and program.reduce_op == 0
+    assert 0 < program.phase_end[0] < program.phase_end[1] < program.value_code_length
+    assert "whole-tile reduction" in description
+    # the second phase (variance) reads the first one (mean); nothing reads a later phase
+    words = [program.value_code[i] for i in range(program.value_code_length)]
+    reduced = [(i, w >> 8) for i, w in enumerate(words) if w & 0xFF == mapping.V["REDUCED"]]
+    assert any(program.phase_end[0] <= i < program.phase_end[1] and k == 0 for i, k in reduced)
+    assert all(k < sum(i >= program.phase_end[j] for j in range(program.num_phases)) for i, k in reduced)
+
+
+@gpu
+@pytest.mark.parametrize("interpret", ("0", "1"))
+@pytest.mark.parametrize("dtype, tolerance", ((torch.float32, 1e-5), (torch.float16, 1e-2)))
+def test_whole_tile_reductions_on_the_gpu(dtype, tolerance, interpret, monkeypatch):
+    monkeypatch.setenv("NT_MAP_INTERPRET", interpret)
+    for rows, cols in ((7, 300), (64, 4096), (3, 1)):
+        for kernel, inputs, expected in _normalisation_cases("cuda", dtype, rows, cols):
+            out = torch.full_like(inputs[0], float("nan"))
+            kernel(*inputs, out)
+            _served_by_map(kernel)
+            assert torch.allclose(out.float(), expected, rtol=tolerance, atol=tolerance), (rows, cols, kernel.kernel_name)
