@@ -541,9 +541,17 @@ class _Lowering:
         tile element here, so this is the plain ``offsets(d)`` provided that index really only
         varies along the dimension the subscript names."""
         base, keys = value.args
+        if not all(key is None or key == slice(None) for key in keys):
+            raise UnsupportedProgram("Tiles and `.offsets(dim)` can only be subscripted with `:` and `None`.")
+        if isinstance(base, Node) and base.op == "load" and isinstance(base.args[0], TensorRef):
+            # `bias[None, :]`: a tile of lower rank laid along the dimensions the `:` entries name;
+            # every element of the result reads the element of the tile at those coordinates
+            if len(keys) != len(dims):
+                raise UnsupportedProgram("A broadcast subscript needs as many entries as the expression's tiles have dimensions.")
+            return self.lower(base, [dim for dim, key in zip(dims, keys) if key is not None], inside_reduction)
         plain = isinstance(base, Node) and base.op == "offsets" and base.args[1] is not None
-        if not plain or not all(key is None or key == slice(None) for key in keys):
-            raise UnsupportedProgram("Only `.offsets(dim)` can be subscripted, with `:` and `None`.")
+        if not plain:
+            raise UnsupportedProgram("Only tiles and `.offsets(dim)` can be subscripted with `:` and `None`.")
         along = [position for position, key in enumerate(keys) if key is not None]
         if len(along) != 1 or len(keys) != len(dims):
             raise UnsupportedProgram("A subscript of `.offsets(dim)` needs one `:` and as many entries as the tile has dimensions.")

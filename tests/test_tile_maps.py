@@ -837,3 +837,38 @@ def test_whole_tile_reductions_on_the_gpu(dtype, tolerance, interpret, monkeypat
             kernel(*inputs, out)
             _served_by_map(kernel)
             assert torch.allclose(out.float(), expected, rtol=tolerance, atol=tolerance), (rows, cols, kernel.kernel_name)
+
+
+# ---- a tile of lower rank broadcast along a tile of the expression (`bias[None, :]`) -------------
+
+
+def _bias_arrangement(input, row_bias, column_bias, output):
+    block_m, block_n = ninetoothed.block_size(), ninetoothed.block_size()
+    tiled = input.tile((block_m, block_n))
+    rows = row_bias.tile((block_n,)).unsqueeze(0).expand((tiled.shape[0], -1))
+    columns = column_bias.tile((block_m,)).unsqueeze(1).expand((-1, tiled.shape[1]))
+    return tiled, rows, columns, output.tile((block_m, block_n))
+
+
+def _bias_application(input, row_bias, column_bias, output):
+    output = input + row_bias[None, :] + column_bias[:, None] * 2  # noqa: F841
+
+
+def test_lowering_broadcast_subscripts_on_tiles():
+    kernel = ninetoothed.make(_bias_arrangement, _bias_application, (Tensor(2), Tensor(1), Tensor(1), Tensor(2)))
+    x, r, c = torch.randn(37, 50), torch.randn(50), torch.randn(37)
+    out = torch.full_like(x, float("nan"))
+    _run_on_machine(kernel, (x, r, c, out), {name: 8 for name in kernel.meta_symbols})
+    assert torch.equal(out, x + r[None, :] + c[:, None] * 2)
+
+
+@gpu
+@pytest.mark.parametrize("interpret", ("0", "1"))
+def test_broadcast_subscripts_on_tiles(interpret, monkeypatch):
+    monkeypatch.setenv("NT_MAP_INTERPRET", interpret)
+    kernel = ninetoothed.make(_bias_arrangement, _bias_application, (Tensor(2), Tensor(1), Tensor(1), Tensor(2)))
+    x, r, c = torch.randn(641, 280, device="cuda"), torch.randn(280, device="cuda"), torch.randn(641, device="cuda")
+    out = torch.full_like(x, float("nan"))
+    kernel(x, r, c, out)
+    _served_by_map(kernel)
+    assert torch.equal(out, x + r[None, :] + c[:, None] * 2)
