@@ -361,7 +361,10 @@ NineToothedResult nt_map_source(const NineToothedMapProgram *program, char *buff
 const char *nt_version(void);
 
 /* Frees every scratch buffer the library holds (see the introduction).  Waits
- * for the device.  No counterpart in the reference, whose kernels need none. */
+ * for the device.  A HIP graph captured from a call that used such a buffer
+ * refers to it by address: do not release the buffers, or let a larger call on
+ * the same stream replace them, while that graph is still replayed.
+ * No counterpart in the reference, whose kernels need none. */
 void nt_release_workspaces(void);
 
 #ifdef __cplusplus
