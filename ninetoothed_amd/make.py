@@ -400,6 +400,57 @@ class Kernel:
         self._map_programs = [program for program, _, _, _ in launches]
         return _Plan("launch_nt_map " + "; ".join(description for _, description, _, _ in launches), launch)
 
+    def _prepare_gemm_epilogue(self, args, env):
+        """A matmul accumulator followed by element-wise work (bias, activation, scaling, residual):
+        the product goes to an fp32 scratch tensor laid out like the output (what the reference
+        holds in the accumulator tile), then the rest runs as a tile map over it."""
+        import ctypes
+
+        import torch
+
+        from ninetoothed_amd import mapping
+
+        lib = runtime.library()
+        details = self.details
+        lhs_pos, rhs_pos, out_pos = details["lhs"], details["rhs"], details["output"]
+        kind, info = recognition.analyze_gemm(self.types[lhs_pos], self.types[rhs_pos], self.types[out_pos], env)
+        if kind == "empty":
+            return _Plan("empty launch", lambda call_args: None)
+        if kind != "strided":
+            raise UnsupportedProgram("A product with an element-wise epilogue needs plain strided matrices.")
+        tag = self._tensor_dtype(args[lhs_pos], args[rhs_pos], allowed=("fp16", "bf16"))
+        out = args[out_pos]
+        if out.numel() and not (out.is_contiguous() or out.t().is_contiguous()):
+            raise UnsupportedProgram("The output of a product with an epilogue must be a dense matrix.")
+        scratch_pos = len(args)
+        gemm = self._gemm_plan(info, tag, "fp32", positions=(None, lhs_pos, rhs_pos, None, None, scratch_pos))
+
+        def with_scratch(call_args):
+            target = call_args[out_pos]
+            scratch = torch.empty_strided(target.shape, target.stride(), dtype=torch.float32, device=target.device)
+            return tuple(call_args) + (scratch,)
+
+        types = self.types + (self.types[out_pos],)
+        sample = with_scratch(args)
+        built = mapping.build(
+            details["epilogue"].stores[0], types, sample, env, lambda p: _dtype_tag(_storage(sample, p).dtype), lambda p: _storage(sample, p).data_ptr()
+        )
+        if built is None:
+            return _Plan("empty launch", lambda call_args: None)
+        program, description, scalar_slots, operand_params = built
+
+        def launch(call_args):
+            extended = with_scratch(call_args)  # from torch's stream-ordered allocator: free again once both launches are queued
+            gemm(extended)
+            for slot, param in enumerate(operand_params):
+                program.operands[slot].data = _storage(extended, param).data_ptr()
+            for index, param in scalar_slots:
+                program.value_constants[index] = float(extended[param])
+            runtime.check(lib.launch_nt_map(runtime.current_stream(), ctypes.addressof(program)))
+
+        self._map_programs = [program]
+        return _Plan(f"{gemm.description}; launch_nt_map {description}", launch)
+
     def _prepare_attention(self, args, env):
         scaled = self.details["scale"]
         if scaled:

@@ -22,7 +22,7 @@ from ninetoothed_amd import programs
 from ninetoothed_amd.affine import Affine, NotAffine, Ranges
 from ninetoothed_amd.symbol import Symbol, evaluate
 from ninetoothed_amd.tensor import Tensor
-from ninetoothed_amd.tracing import TracingError, trace
+from ninetoothed_amd.tracing import Carried, Dim, LoopVar, Node, Program, TensorRef, TracingError, trace
 
 
 class UnsupportedProgram(NotImplementedError):
@@ -67,6 +67,9 @@ def identify(application, types):
         try:
             mapping.check_application(program)
         except UnsupportedProgram as error:
+            fused = match_gemm_with_epilogue(program, types)
+            if fused is not None:
+                return "gemm_epilogue", fused, program
             raise UnsupportedProgram(
                 "The application is not one of the programs this build has kernels for "
                 "(matmul, addmm, row softmax, attention forward, conv2d as matmul) and not an element-wise / reducing "
@@ -74,6 +77,93 @@ def identify(application, types):
             ) from error
         return "map", {}, program
     return entry[0], entry[1], program
+
+
+# ---- a matrix product followed by element-wise work on the accumulator ---------------------------
+
+
+def _is_accumulation(node):
+    """``loop_out`` of `acc = zeros(...); for k in range(lhs.shape[0]): acc += dot(lhs[k], rhs[k])`:
+    returns the parameter positions (lhs, rhs), or None."""
+    if not (isinstance(node, Node) and node.op == "loop_out" and node.args[1] == 0):
+        return None
+    loop = node.args[0]
+    if not (isinstance(loop, Node) and loop.op == "loop" and len(loop.args[1]) == 1 and len(loop.args[2]) == 1):
+        return None
+    init, body = loop.args[1][0], loop.args[2][0]
+    if not (isinstance(init, Node) and init.op == "zeros"):
+        return None
+    if not (isinstance(body, Node) and body.op == "add" and len(body.args) == 2):
+        return None
+    carried = [arg for arg in body.args if isinstance(arg, Carried)]
+    products = [arg for arg in body.args if isinstance(arg, Node) and arg.op == "dot" and len(arg.args) == 2]
+    if len(carried) != 1 or len(products) != 1:
+        return None
+    operands = []
+    for factor in products[0].args:
+        if not (isinstance(factor, Node) and factor.op == "load" and isinstance(factor.args[0], TensorRef)):
+            return None
+        ref = factor.args[0]
+        if ref.level != 2 or len(ref.indices) != 1 or not isinstance(ref.indices[0], LoopVar):
+            return None
+        operands.append(ref.param)
+    extent = loop.args[0]
+    if not (isinstance(extent, Dim) and extent.param == operands[0] and extent.level == 1 and extent.dim == 0):
+        return None
+    return tuple(operands)
+
+
+def match_gemm_with_epilogue(program, types):
+    """A single store whose value is element-wise work on one matmul accumulator (bias, activation,
+    scaling, a residual ...).  Returns ``{"lhs", "rhs", "output", "accumulator"}`` (parameter
+    positions and the accumulator node) when, with the accumulator replaced by a tile of a new
+    tensor arranged like the output, the rest is a tile map; else None."""
+    from ninetoothed_amd import mapping
+
+    if len(program.stores) != 1 or not isinstance(program.stores[0][0], TensorRef):
+        return None
+    ref, value = program.stores[0]
+    found = {}
+
+    def visit(item):
+        if isinstance(item, Node):
+            operands = _is_accumulation(item)
+            if operands is not None:
+                found[item.digest] = (item, operands)
+                return
+            for arg in item.args:
+                visit(arg)
+        elif isinstance(item, (tuple, list)):
+            for arg in item:
+                visit(arg)
+
+    visit(value)
+    if len(found) != 1:
+        return None
+    (accumulator, (lhs, rhs)), = found.values()
+    if ref.level != 1 or not ref.is_tile or ref.param in (lhs, rhs):
+        return None
+    stand_in = TensorRef(len(types), ref.tensor, 1)
+    epilogue = substitute(value, accumulator.digest, Node("load", stand_in))
+    candidate = Program(program.params + [("tensor", False)], [(ref, epilogue)])
+    try:
+        mapping.check_application(candidate)
+    except UnsupportedProgram:
+        return None
+    return {"lhs": lhs, "rhs": rhs, "output": ref.param, "epilogue": candidate}
+
+
+def substitute(value, digest, replacement):
+    """``value`` with every node of that digest replaced."""
+    if isinstance(value, Node):
+        if value.digest == digest:
+            return replacement
+        return Node(value.op, *[substitute(arg, digest, replacement) for arg in value.args])
+    if isinstance(value, tuple):
+        return tuple(substitute(item, digest, replacement) for item in value)
+    if isinstance(value, list):
+        return [substitute(item, digest, replacement) for item in value]
+    return value
 
 
 # ---- arrangement analysis -------------------------------------------------------
