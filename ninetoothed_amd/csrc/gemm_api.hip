@@ -40,7 +40,8 @@ struct GemmInstance {
 template <int BM, int BN, int BK, int kStages>
 bool fast_accepts(const GemmProblem &q) {
     if (q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) return false;
-    if (q.out_dtype != q.dtype) return false;
+    // the element type, or fp32 for a plain product (the accumulators as they are)
+    if (q.out_dtype != q.dtype && !(q.out_dtype == NINETOOTHED_FLOAT32 && !q.addmm())) return false;
     if (q.m <= 0 || q.n <= 0 || q.k <= 0) return false;
     // any number of rows: rows past M read as zeros and are not stored; N and K must fit the tile
     if (q.n % BN || q.k % BK) return false;
@@ -79,7 +80,10 @@ hipError_t fast_launch_typed(const GemmProblem &q, hipStream_t stream) {
     GemmParams p;
     fill_params(p, q, BM, BN);
     const dim3 grid(p.tiles_m * p.tiles_n), block(WM * WN * 64);
-    if (q.addmm()) {
+    if (q.out_dtype == NINETOOTHED_FLOAT32) {
+        auto kernel = gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, false, kAblate, kLoad, kAux, true>;
+        kernel<<<grid, block, 0, stream>>>(p);
+    } else if (q.addmm()) {
         auto kernel = gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, true, kAblate, kLoad, kAux>;
         kernel<<<grid, block, 0, stream>>>(p);
     } else {

@@ -96,7 +96,8 @@ NT_DEVICE void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" 
 
 // kAblate is a measurement aid (bit 0: no global loads inside the K loop,
 // bit 1: operand fragments read from LDS only once); 0 in every shipped instance.
-template <typename T, int BM, int BN, int BK, int WM, int WN, int kStages, int kWavesPerSimd, bool kAddmm, int kAblate = 0, int kLoad = 0, int kAux = 0>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int kStages, int kWavesPerSimd, bool kAddmm, int kAblate = 0, int kLoad = 0, int kAux = 0,
+          bool kFloatOut = false>
 __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kernel(GemmParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only builtins; the host pass only needs the stub
     typedef Elem<T> E;
@@ -338,6 +339,31 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     // global stores (and addmm input loads) are 16 bytes per lane and cover
     // whole 128-byte lines.  (All fills have landed and all waves are done with
     // the stages before the slabs overwrite them.)
+    if constexpr (kFloatOut) {
+        // fp32 output (matmul only): a lane's four registers of one r4 group are four consecutive
+        // columns of its row, i.e. one 16-byte store; the two halves of a wave complete 32 bytes
+        // and the four groups a 128-byte line, which the L2 merges
+        static_assert(!kAddmm, "the fp32 output path has no addmm epilogue");
+        wait_vmcnt<0>();
+        float *C32 = (float *)p.c;
+#pragma unroll
+        for (int ti = 0; ti < TM; ++ti) {
+            const int grow = m0 + wave_m * kWaveM + ti * 32 + l32;
+            if (grow >= p.m) continue;
+#pragma unroll
+            for (int tj = 0; tj < TN; ++tj)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    typedef float float4_t __attribute__((ext_vector_type(4)));
+                    float4_t v;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = acc[ti][tj][4 * r4 + e];
+                    const int gcol = n0 + wave_n * kWaveN + tj * 32 + 8 * r4 + 4 * g;
+                    *(float4_t *)(C32 + (int64_t)grow * p.ldc + gcol) = v;
+                }
+        }
+        return;
+    }
     constexpr int kRowBytes = kWaveN * 2;
     constexpr int kCChunks = kWaveN / 8;  // 16-byte chunks per slab row
     constexpr int kCShift = kRowBytes >= 256 ? 0 : (kRowBytes == 128 ? 1 : 2);

@@ -76,6 +76,37 @@ def test_matmul_bfloat16_and_float32_output():
     assert torch.allclose(out32, a.cuda().float() @ b.cuda().float(), rtol=1e-4, atol=1e-3)
 
 
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
+@pytest.mark.parametrize("m, n, k", ((512, 512, 512), (1000, 768, 1024), (4096, 2048, 4096)))
+def test_matmul_float32_output_on_the_fast_instances(m, n, k, dtype):
+    """fp32 output of a plain product = the accumulators as they are; every instance that takes the
+    shape has to write all of them (NaN-poisoned output, whole-output comparison with an fp32 product
+    of the same rounded operands)."""
+    from ninetoothed_amd import runtime
+
+    lib = runtime.library()
+    a = torch.randn(m, k, dtype=dtype, device="cuda")
+    b = torch.randn(k, n, dtype=dtype, device="cuda")
+    expected = a.float() @ b.float()
+    kernel = _matmul_kernel()
+    out = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
+    kernel(a, b, out)
+    assert torch.allclose(out, expected, rtol=1e-3, atol=1e-2 * (k / 512) ** 0.5)
+    tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (a, b, out)]
+    null = runtime.ArgumentTensor.null()
+    tag = runtime.DATA_TYPE_INDEX["fp16" if dtype == torch.float16 else "bf16"]
+    served = 0
+    for instance in range(lib.nt_gemm_num_configs()):
+        out.fill_(float("nan"))
+        result = lib.launch_nt_gemm_config(runtime.current_stream(), instance, null, tensors[0], tensors[1], null, null, tensors[2], tag, runtime.DATA_TYPE_INDEX["fp32"])
+        if result == 1:
+            continue
+        assert result == 0
+        served += 1
+        assert torch.allclose(out, expected, rtol=1e-3, atol=1e-2 * (k / 512) ** 0.5), runtime.gemm_config_names()[instance]
+    assert served >= 2
+
+
 def test_matmul_empty_and_errors():
     kernel = _matmul_kernel()
     out = torch.empty(0, 16, dtype=torch.float16, device="cuda")
