@@ -37,6 +37,9 @@ struct GemmInstance {
     LaunchFn launch;
 };
 
+// the fast instances take B row-major ([K, N], unit column stride) or transposed ([N, K] storage, unit k stride)
+bool b_is_transposed(const GemmProblem &q) { return q.sbn != 1 && q.sbk == 1; }
+
 template <int BM, int BN, int BK, int kStages>
 bool fast_accepts(const GemmProblem &q) {
     if (q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) return false;
@@ -45,12 +48,18 @@ bool fast_accepts(const GemmProblem &q) {
     if (q.m <= 0 || q.n <= 0 || q.k <= 0) return false;
     // any number of rows: rows past M read as zeros and are not stored; N and K must fit the tile
     if (q.n % BN || q.k % BK) return false;
-    if (q.sak != 1 || q.sbn != 1 || q.scn != 1) return false;
-    if (q.sam % 8 || q.sbk % 8 || q.sam < q.k || q.sbk < q.n || q.scm < q.n) return false;
+    if (q.sak != 1 || q.scn != 1) return false;
+    if (q.sam % 8 || q.sam < q.k || q.scm < q.n) return false;
     if (((uintptr_t)q.a & 15) || ((uintptr_t)q.b & 15) || ((uintptr_t)q.c & 15) || q.scm % 8) return false;
     // per-lane 32-bit byte offsets inside one tile panel
     if ((int64_t)BM * q.sam * 2 >= (int64_t(1) << 31)) return false;
-    if ((int64_t)q.k * q.sbk * 2 >= (int64_t(1) << 31)) return false;
+    if (b_is_transposed(q)) {  // B as [N, K] with K contiguous (`x @ w.T`)
+        if (q.sbn % 8 || q.sbn < q.k) return false;
+        if ((int64_t)BN * q.sbn * 2 >= (int64_t(1) << 31)) return false;
+    } else {
+        if (q.sbn != 1 || q.sbk % 8 || q.sbk < q.n) return false;
+        if ((int64_t)q.k * q.sbk * 2 >= (int64_t(1) << 31)) return false;
+    }
     return true;
 }
 
@@ -63,7 +72,7 @@ void fill_params(GemmParams &p, const GemmProblem &q, int bm, int bn) {
     p.n = q.n;
     p.k = q.k;
     p.lda = q.sam;
-    p.ldb = q.sbk;
+    p.ldb = b_is_transposed(q) ? q.sbn : q.sbk;
     p.ldc = q.scm;
     p.bias_stride_m = q.sim;
     p.bias_stride_n = q.sin;
@@ -80,15 +89,15 @@ hipError_t fast_launch_typed(const GemmProblem &q, hipStream_t stream) {
     GemmParams p;
     fill_params(p, q, BM, BN);
     const dim3 grid(p.tiles_m * p.tiles_n), block(WM * WN * 64);
-    if (q.out_dtype == NINETOOTHED_FLOAT32) {
-        auto kernel = gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, false, kAblate, kLoad, kAux, true>;
-        kernel<<<grid, block, 0, stream>>>(p);
-    } else if (q.addmm()) {
-        auto kernel = gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, true, kAblate, kLoad, kAux>;
-        kernel<<<grid, block, 0, stream>>>(p);
+    const bool f32 = q.out_dtype == NINETOOTHED_FLOAT32, addmm = q.addmm();
+    if (b_is_transposed(q)) {
+        if (f32) gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, false, kAblate, kLoad, kAux, true, true><<<grid, block, 0, stream>>>(p);
+        else if (addmm) gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, true, kAblate, kLoad, kAux, false, true><<<grid, block, 0, stream>>>(p);
+        else gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, false, kAblate, kLoad, kAux, false, true><<<grid, block, 0, stream>>>(p);
     } else {
-        auto kernel = gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, false, kAblate, kLoad, kAux>;
-        kernel<<<grid, block, 0, stream>>>(p);
+        if (f32) gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, false, kAblate, kLoad, kAux, true><<<grid, block, 0, stream>>>(p);
+        else if (addmm) gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, true, kAblate, kLoad, kAux><<<grid, block, 0, stream>>>(p);
+        else gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, false, kAblate, kLoad, kAux><<<grid, block, 0, stream>>>(p);
     }
     return hipGetLastError();
 }

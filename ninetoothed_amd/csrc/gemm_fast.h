@@ -97,7 +97,7 @@ NT_DEVICE void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" 
 // kAblate is a measurement aid (bit 0: no global loads inside the K loop,
 // bit 1: operand fragments read from LDS only once); 0 in every shipped instance.
 template <typename T, int BM, int BN, int BK, int WM, int WN, int kStages, int kWavesPerSimd, bool kAddmm, int kAblate = 0, int kLoad = 0, int kAux = 0,
-          bool kFloatOut = false>
+          bool kFloatOut = false, bool kBT = false>
 __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kernel(GemmParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only builtins; the host pass only needs the stub
     typedef Elem<T> E;
@@ -171,7 +171,9 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     // 2^31 (checked on the host), so addresses are a uniform base + 32-bit lane offset.
     // A: instruction j of this wave fills rows [(j*kWaves+wave)*kARowsPerInstr, +kARowsPerInstr)
     const unsigned char *a_base = (const unsigned char *)(A + (int64_t)m0 * p.lda);
-    const unsigned char *b_base = (const unsigned char *)(B + n0);
+    // kBT: B is given as [N, K] with K contiguous (`x @ w.T`): its tile is staged and read exactly
+    // like A's (rows = columns of C, 16-byte chunks of 8 consecutive k), no transposing read
+    const unsigned char *b_base = (const unsigned char *)(kBT ? B + (int64_t)n0 * p.ldb : B + n0);
     unsigned a_src[kAInstr];
 #pragma unroll
     for (int j = 0; j < kAInstr; ++j) {
@@ -183,10 +185,16 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     unsigned b_src[kBInstr];
 #pragma unroll
     for (int j = 0; j < kBInstr; ++j) {
-        const int krow = (j * kWaves + wave) * kBRowsPerInstr + lane / kBChunksPerRow;
-        const int phys = lane % kBChunksPerRow;
-        const int chunk = b_phys_chunk<BN>(krow, phys);
-        b_src[j] = (unsigned)(krow * (int)p.ldb + chunk * 8) * 2u;
+        if constexpr (kBT) {
+            const int row = (j * kWaves + wave) * kARowsPerInstr + lane / kAChunksPerRow;
+            const int chunk = a_phys_chunk<BK>(row, lane % kAChunksPerRow);
+            b_src[j] = (unsigned)(row * (int)p.ldb + chunk * 8) * 2u;
+        } else {
+            const int krow = (j * kWaves + wave) * kBRowsPerInstr + lane / kBChunksPerRow;
+            const int phys = lane % kBChunksPerRow;
+            const int chunk = b_phys_chunk<BN>(krow, phys);
+            b_src[j] = (unsigned)(krow * (int)p.ldb + chunk * 8) * 2u;
+        }
     }
 
     // kLoad 0: global_load_lds (64-bit base + lane offset); 1: buffer_load ... lds
@@ -204,7 +212,7 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         NT_LDS unsigned char *sb = stage_b(stage_tag);
         if constexpr (kLoad == 1) {
             const int a_k = kt * BK * 2;
-            const int b_k = kt * BK * (int)p.ldb * 2;
+            const int b_k = kBT ? a_k : kt * BK * (int)p.ldb * 2;
 #pragma unroll
             for (int j = 0; j < kAInstr; ++j)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, sa + (j * kWaves + wave) * 1024, 16, a_src[j], a_k, 0, kAux);
@@ -213,7 +221,7 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, sb + (j * kWaves + wave) * 1024, 16, b_src[j], b_k, 0, kAux);
         } else {
             const unsigned char *a_tile = a_base + (int64_t)kt * BK * 2;
-            const unsigned char *b_tile = b_base + (int64_t)kt * BK * p.ldb * 2;
+            const unsigned char *b_tile = b_base + (kBT ? (int64_t)kt * BK * 2 : (int64_t)kt * BK * p.ldb * 2);
 #pragma unroll
             for (int j = 0; j < kAInstr; ++j)
                 __builtin_amdgcn_global_load_lds((const NT_GLOBAL void *)(a_tile + a_src[j]), sa + (j * kWaves + wave) * 1024, 16, 0, kAux);
@@ -248,6 +256,14 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         b_col_in[tj] = (ncol & 7) * 2;
     }
 
+    int bt_row_off[TN], bt_row_sw[TN];  // kBT: this lane's B row (a column of C), as for A
+#pragma unroll
+    for (int tj = 0; tj < TN; ++tj) {
+        const int row = wave_n * kWaveN + tj * 32 + l32;
+        bt_row_off[tj] = row * (BK * 2);
+        bt_row_sw[tj] = a_phys_chunk<BK>(row, 0);
+    }
+
     float16_t acc[TM][TN];
 #pragma unroll
     for (int ti = 0; ti < TM; ++ti)
@@ -266,14 +282,19 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         }
 #pragma unroll
         for (int tj = 0; tj < TN; ++tj) {
-            const int k_lo = ks * 16 + b_krow;
-            const int k_hi = k_lo + 4;
-            const int c_lo = b_phys_chunk<BN>(k_lo, b_col_chunk[tj]);
-            const int c_hi = b_phys_chunk<BN>(k_hi, b_col_chunk[tj]);
-            short4_t lo = lds_read_tr16_b64(sb + k_lo * (BN * 2) + c_lo * 16 + b_col_in[tj]);
-            short4_t hi = lds_read_tr16_b64(sb + k_hi * (BN * 2) + c_hi * 16 + b_col_in[tj]);
-            short8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            bf[tj] = __builtin_bit_cast(vec8, both);
+            if constexpr (kBT) {
+                const int chunk = (ks * 2 + g) ^ bt_row_sw[tj];
+                bf[tj] = *(const NT_LDS vec8 *)(sb + bt_row_off[tj] + chunk * 16);
+            } else {
+                const int k_lo = ks * 16 + b_krow;
+                const int k_hi = k_lo + 4;
+                const int c_lo = b_phys_chunk<BN>(k_lo, b_col_chunk[tj]);
+                const int c_hi = b_phys_chunk<BN>(k_hi, b_col_chunk[tj]);
+                short4_t lo = lds_read_tr16_b64(sb + k_lo * (BN * 2) + c_lo * 16 + b_col_in[tj]);
+                short4_t hi = lds_read_tr16_b64(sb + k_hi * (BN * 2) + c_hi * 16 + b_col_in[tj]);
+                short8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                bf[tj] = __builtin_bit_cast(vec8, both);
+            }
         }
     };
 

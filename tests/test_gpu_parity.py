@@ -107,6 +107,46 @@ def test_matmul_float32_output_on_the_fast_instances(m, n, k, dtype):
     assert served >= 2
 
 
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
+@pytest.mark.parametrize("m, n, k", ((512, 512, 512), (1000, 768, 1024), (4096, 2048, 4096)))
+def test_transposed_rhs_on_the_fast_instances(m, n, k, dtype):
+    """`x @ w.T` with `w` stored [N, K]: the rhs reaches the kernels with a unit k stride.  Every
+    instance that takes it, matmul (both output types) and addmm, whole output, NaN-poisoned."""
+    from ninetoothed_amd import runtime
+
+    lib = runtime.library()
+    a = torch.randn(m, k, dtype=dtype, device="cuda")
+    w = torch.randn(n, k + 8, dtype=dtype, device="cuda")[:, :k]  # rows padded: a row stride that is not k
+    b = w.t()
+    bias = torch.randn(m, n, dtype=dtype, device="cuda")
+    product = a.float() @ b.float()
+    tag = runtime.DATA_TYPE_INDEX["fp16" if dtype == torch.float16 else "bf16"]
+    null = runtime.ArgumentTensor.null()
+    beta, alpha = runtime.ArgumentTensor.from_scalar(0.5), runtime.ArgumentTensor.from_scalar(2.0)
+    tolerance = dict(rtol=2e-2, atol=2e-2 * (k / 512) ** 0.5) if dtype == torch.bfloat16 else dict(rtol=1e-2, atol=1e-2 * (k / 512) ** 0.5)
+    for out_dtype, with_bias in ((dtype, False), (torch.float32, False), (dtype, True)):
+        out = torch.empty(m, n, dtype=out_dtype, device="cuda")
+        tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (bias, a, b, out)]
+        expected = 0.5 * bias.float() + 2.0 * product.to(dtype).float() if with_bias else product
+        served = 0
+        for instance in range(lib.nt_gemm_num_configs()):
+            out.fill_(float("nan"))
+            result = lib.launch_nt_gemm_config(
+                runtime.current_stream(), instance, tensors[0] if with_bias else null, tensors[1], tensors[2], beta if with_bias else null,
+                alpha if with_bias else null, tensors[3], tag, runtime.DATA_TYPE_INDEX["fp32" if out_dtype == torch.float32 else ("fp16" if dtype == torch.float16 else "bf16")],
+            )
+            if result == 1:
+                continue
+            assert result == 0
+            served += 1
+            assert torch.allclose(out.float(), expected, **tolerance), (runtime.gemm_config_names()[instance], out_dtype, with_bias)
+        assert served >= 2
+    # and through `make`
+    out = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+    _matmul_kernel()(a, b, out)
+    assert torch.allclose(out.float(), product, **tolerance)
+
+
 def test_matmul_empty_and_errors():
     kernel = _matmul_kernel()
     out = torch.empty(0, 16, dtype=torch.float16, device="cuda")
