@@ -139,7 +139,8 @@ NineToothedResult launch_nt_softmax_config(NineToothedStream stream, int config,
  * >= 256 selects 256 query rows per workgroup, block_size_n <= 32 the 32-key
  * blocks with three workgroups per CU, block_size_n >= 64 the plain 64-key
  * loop; without hints non-causal calls run the software-pipelined 64-key loop
- * and causal calls the plain one.  K and V of one (batch, head) must span
+ * (with 256 query rows and eight waves per workgroup when that still fills the
+ * chip twice) and causal calls the plain one.  K and V of one (batch, head) must span
  * less than 4 GiB. */
 NineToothedResult launch_nt_attention(NineToothedStream stream,
                                       NineToothedTensor q,

@@ -39,12 +39,12 @@ constexpr int kAttnWaves = 4;
 // kPipelined: overlap the softmax of a block with the MFMAs of its neighbours
 // TIO: element type of Q and O in memory -- T, or float for fp32 tensors (their K and V
 // are converted to T beforehand; Q is converted while it is scaled, O is stored unrounded)
-template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined, typename TIO = T>
-__global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(AttentionParams p) {
+template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined, typename TIO = T, int kWaves = kAttnWaves>
+__global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(AttentionParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     typedef Elem<T> E;
     typedef typename E::vec8 vec8;
-    constexpr int BM = kAttnWaves * 32 * kQTiles;
+    constexpr int BM = kWaves * 32 * kQTiles;
     constexpr int KT = BN / 32;          // kv tiles of S^T per block
     constexpr int DT = D / 32;           // d tiles of O^T
     constexpr int KS = D / 16;           // contraction steps of S^T
@@ -52,9 +52,9 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
     constexpr int kTileBytes = BN * D * 2;
     constexpr int kChunksPerRow = D / 8;
     constexpr int kRowsPerInstr = 64 / kChunksPerRow;
-    constexpr int kInstr = kTileBytes / (kAttnWaves * 1024);
+    constexpr int kInstr = kTileBytes / (kWaves * 1024);
     static_assert(D % 32 == 0 && D >= 32 && D <= 256, "head dim");
-    static_assert(kTileBytes % (kAttnWaves * 1024) == 0, "tile/wave mismatch");
+    static_assert(kTileBytes % (kWaves * 1024) == 0, "tile/wave mismatch");
 
     __shared__ __attribute__((aligned(1024))) unsigned char lds_k0[kTileBytes];
     __shared__ __attribute__((aligned(1024))) unsigned char lds_v0[kTileBytes];
@@ -164,7 +164,7 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
     // load instruction j of a wave covers the rows kLoadRowStep * j further down; both
     // swizzles repeat with that period, so one lane offset serves every j and the
     // row step goes into the scalar offset as well
-    constexpr int kLoadRowStep = kAttnWaves * kRowsPerInstr;
+    constexpr int kLoadRowStep = kWaves * kRowsPerInstr;
     static_assert(a_phys_chunk<D>(kLoadRowStep, 0) == 0 && b_phys_chunk<D>(kLoadRowStep, 0) == 0, "swizzle period");
     const unsigned k_step_bytes = (unsigned)(kLoadRowStep * p.k_strides[2]) * 2u;
     const unsigned v_step_bytes = (unsigned)(kLoadRowStep * p.v_strides[2]) * 2u;
@@ -180,14 +180,14 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
         const unsigned block_off = (unsigned)blk * k_block_bytes;
 #pragma unroll
         for (int j = 0; j < kInstr; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, sk + (j * kAttnWaves + wave) * 1024, 16, ld_k_off, block_off + j * k_step_bytes, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, sk + (j * kWaves + wave) * 1024, 16, ld_k_off, block_off + j * k_step_bytes, 0, 0);
     };
     auto issue_v = [&](auto stage_tag, int blk) __attribute__((always_inline)) {
         NT_LDS unsigned char *sv = stage_v(stage_tag);
         const unsigned block_off = (unsigned)blk * v_block_bytes;
 #pragma unroll
         for (int j = 0; j < kInstr; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, sv + (j * kAttnWaves + wave) * 1024, 16, ld_v_off, block_off + j * v_step_bytes, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, sv + (j * kWaves + wave) * 1024, 16, ld_v_off, block_off + j * v_step_bytes, 0, 0);
     };
 
     // ---- LDS read offsets ----
@@ -514,13 +514,13 @@ __global__ __launch_bounds__(kAttnWaves * 64, kOcc) void attention_fwd_kernel(At
 #endif
 }
 
-template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined, typename TIO = T>
+template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined, typename TIO = T, int kWaves = kAttnWaves>
 hipError_t launch_attention(AttentionParams &p, hipStream_t stream) {
-    constexpr int BM = kAttnWaves * 32 * kQTiles;
+    constexpr int BM = kWaves * 32 * kQTiles;
     p.q_blocks = ceil_div(p.seq_q, BM);
     const int64_t grid = (int64_t)p.batch * p.heads * p.q_blocks;
     if (grid == 0) return hipSuccess;
-    attention_fwd_kernel<T, D, kQTiles, BN, kOcc, kPipelined, TIO><<<dim3((unsigned)grid), dim3(kAttnWaves * 64), 0, stream>>>(p);
+    attention_fwd_kernel<T, D, kQTiles, BN, kOcc, kPipelined, TIO, kWaves><<<dim3((unsigned)grid), dim3(kWaves * 64), 0, stream>>>(p);
     return hipGetLastError();
 }
 
@@ -563,15 +563,21 @@ int attention_float32(AttentionParams p, int head_dim, const NineToothedTensor &
 //          1 = 256 query rows per workgroup, 64-key blocks, one workgroup per CU
 //          2 = 128 query rows per workgroup, 32-key blocks, three workgroups per CU
 //          3 = variant 0 with the software-pipelined main loop
+//          4 = variant 3 with eight waves (256 query rows) per workgroup, one workgroup per CU
 template <typename T>
 int dispatch_attention(AttentionParams &p, int head_dim, int variant, hipStream_t stream) {
     if (head_dim == 128) {
+        if (variant == 4) return (int)launch_attention<T, 128, 1, 64, 2, true, T, 8>(p, stream);
+#ifdef NT_MEASUREMENT_AIDS
+        if (variant == 5) return (int)launch_attention<T, 128, 1, 64, 2, false, T, 8>(p, stream);
+#endif
         if (variant == 3) return (int)launch_attention<T, 128, 1, 64, 2, true>(p, stream);
         if (variant == 1) return (int)launch_attention<T, 128, 2, 64, 1, false>(p, stream);
         if (variant == 2) return (int)launch_attention<T, 128, 1, 32, 3, false>(p, stream);
         return (int)launch_attention<T, 128, 1, 64, 2, false>(p, stream);
     }
     if (head_dim == 64) {
+        if (variant == 4) return (int)launch_attention<T, 64, 1, 64, 2, true, T, 8>(p, stream);
         if (variant == 3) return (int)launch_attention<T, 64, 1, 64, 2, true>(p, stream);
         if (variant == 1) return (int)launch_attention<T, 64, 2, 64, 1, false>(p, stream);
         if (variant == 2) return (int)launch_attention<T, 64, 1, 32, 3, false>(p, stream);
@@ -635,8 +641,12 @@ extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineT
     // block sizes are hints: 256 query rows select the one-workgroup-per-CU
     // variant, 32-key blocks the three-workgroups-per-CU variant.  Without a hint
     // the pipelined variant runs non-causal problems and the plain 64-key loop causal
-    // ones (measured at [4, 32, 4096, 128]: 0.94 against 0.92 and 0.90 PFLOP/s).
+    // ones (measured at [4, 32, 4096, 128]: 0.94 against 0.92 and 0.90 PFLOP/s); non-causal
+    // problems with enough 256-row blocks to fill the chip twice run the pipelined loop with
+    // eight waves per workgroup, which loads every K / V block once for 256 query rows
+    // (1.02 against 0.99 PFLOP/s).
     int variant = block_size_m >= 256 ? 1 : (block_size_n > 0 && block_size_n <= 32 ? 2 : (block_size_n >= 64 || p.causal ? 0 : 3));
+    if (variant == 3 && block_size_m == 0 && head_dim >= 64 && (int64_t)p.batch * p.heads * ceil_div(p.seq_q, 256) >= 512) variant = 4;
 #ifdef NT_MEASUREMENT_AIDS
     if (block_size_n >= 1000) variant = block_size_n - 1000;  // explicit variant, for timing harnesses only
 #endif

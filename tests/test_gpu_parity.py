@@ -372,6 +372,24 @@ def test_attention_block_size_hints(block_size_m, block_size_n, emb_dim, is_caus
     assert torch.allclose(out, expected, **HALF_TOL)
 
 
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
+@pytest.mark.parametrize("emb_dim", (64, 128))
+def test_attention_many_short_sequences(emb_dim, dtype):
+    # enough 256-row query blocks for the eight-wave loop (512 of them), with ragged ends on both
+    # the query side (300 = 256 + 44) and the key side (333), and keys of another length than queries
+    q = _randn(8, 32, 300, emb_dim, dtype=dtype).cuda()
+    k, v = (_randn(8, 32, 333, emb_dim, dtype=dtype).cuda() for _ in range(2))
+    kernel = ninetoothed.make(
+        programs.attention.arrangement_with_scale, programs.attention.application_with_scale, programs.attention.tensors(True)
+    )
+    expected = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), scale=emb_dim**-0.5)
+    for _ in range(2):
+        out = torch.full_like(q, float("nan"))
+        kernel(q, k, v, False, emb_dim**-0.5, out)
+        _native_only(kernel, "launch_nt_attention")
+        assert torch.allclose(out.float(), expected, rtol=2e-2, atol=2e-2)
+
+
 # ---- conv2d ---------------------------------------------------------------
 
 
