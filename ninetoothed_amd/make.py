@@ -498,11 +498,18 @@ def _jagged_layout(arg):
 
 
 class _Plan:
-    __slots__ = ("description", "launch")
+    """A prepared launch.  Its argument structs are filled in per call, so calls from several
+    host threads take turns (the launches themselves are asynchronous)."""
+
+    __slots__ = ("description", "launch", "_lock")
 
     def __init__(self, description, launch):
+        import threading
+
         self.description = description
         self.launch = launch
+        self._lock = threading.Lock()
 
     def __call__(self, args):
-        self.launch(args)
+        with self._lock:
+            self.launch(args)

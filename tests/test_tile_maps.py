@@ -19,7 +19,7 @@ import torch.nn.functional as F
 
 import ninetoothed_amd as ninetoothed
 import ninetoothed_amd.language as ntl
-from ninetoothed_amd import Symbol, Tensor, block_size, mapping
+from ninetoothed_amd import Symbol, Tensor, block_size, mapping, programs
 from ninetoothed_amd.language import libdevice
 from ninetoothed_amd.make import _dtype_tag, _storage
 from ninetoothed_amd.recognition import UnsupportedProgram
@@ -872,3 +872,35 @@ def test_broadcast_subscripts_on_tiles(interpret, monkeypatch):
     kernel(x, r, c, out)
     _served_by_map(kernel)
     assert torch.equal(out, x + r[None, :] + c[:, None] * 2)
+
+
+@gpu
+def test_one_kernel_called_from_several_threads():
+    """Calls with one signature share a prepared launch whose argument structs are filled per call."""
+    import threading
+
+    n = 1 << 16
+    matmul = ninetoothed.make(programs.matmul.arrangement, programs.matmul.application, programs.matmul.tensors())
+    failures = []
+
+    def worker(seed):
+        generator = torch.Generator(device="cuda").manual_seed(seed)
+        lhs = torch.randn(n, device="cuda", generator=generator)
+        rhs = torch.randn(n, device="cuda", generator=generator)
+        a = torch.randn(256, 128, device="cuda", generator=generator).half()
+        b = torch.randn(128, 256, device="cuda", generator=generator).half()
+        for _ in range(100):
+            out = torch.empty(n, device="cuda")
+            add_kernel(lhs, rhs, out, BLOCK_SIZE=1024)
+            c = torch.empty(256, 256, dtype=torch.float16, device="cuda")
+            matmul(a, b, c)
+            if not torch.equal(out, lhs + rhs) or not torch.allclose(c, a @ b, rtol=1e-2, atol=1e-2):
+                failures.append(seed)
+                return
+
+    threads = [threading.Thread(target=worker, args=(seed,)) for seed in range(4)]
+    for thread in threads:
+        thread.start()
+    for thread in threads:
+        thread.join()
+    assert not failures
