@@ -232,6 +232,8 @@ class _Lowering:
         self.tile_mode = tile_mode
         self.phases = []
         self.phase_of = {}        # digest of a reduction -> (phase, type of its term, type it accumulates in)
+        self.tile_axis = None     # axis of the tile the phases reduce over (None: the whole tile)
+        self.axis_subscript_seen = False
         self.operands = []        # (param, Operand)
         self.operand_slot = {}    # param -> slot
         self.var_extent = []      # shared variables: grid dims first, then output tile dims, then reduced dims
@@ -474,10 +476,21 @@ class _Lowering:
         if op in REDUCE and self.tile_mode:
             positional, named = _kwargs(value)
             axis = named.get("axis", positional[1] if len(positional) > 1 else None)
-            if axis is not None:
-                raise UnsupportedProgram("Only reductions over a whole tile can be combined with the elements of the tile.")
             if self._tile_rank(positional[0]) != len(dims):
                 raise UnsupportedProgram("A reduction whose result is used on a tile must run over tiles of that tile's shape.")
+            # every reduction of the expression runs over the same part of the tile: all of it, or one
+            # axis (then the other tile dimensions enumerate "rows", each reduced on its own, and the
+            # result is laid back over the tile with a `None` subscript at that axis)
+            if axis is not None:
+                if not isinstance(axis, int) or not -len(dims) <= axis < len(dims):
+                    raise UnsupportedProgram("The reduction axis must be an integer constant within the tile's dimensions.")
+                axis %= len(dims)
+                if not self.axis_subscript_seen:
+                    raise UnsupportedProgram("Subscript the result of an axis reduction with `None` at that axis to use it on the tile.")
+                self.axis_subscript_seen = False
+            if self.phases and self.tile_axis != axis:
+                raise UnsupportedProgram("All reductions of one stored expression must run over the same axis.")
+            self.tile_axis = axis
             if value.digest in self.phase_of:  # the same reduction used again: one phase serves every use
                 k, term, accumulate = self.phase_of[value.digest]
                 self.emit("REDUCED", k)
@@ -543,6 +556,17 @@ class _Lowering:
         base, keys = value.args
         if not all(key is None or key == slice(None) for key in keys):
             raise UnsupportedProgram("Tiles and `.offsets(dim)` can only be subscripted with `:` and `None`.")
+        if isinstance(base, Node) and base.op in REDUCE and self.tile_mode:
+            # `ntl.max(x, axis=1)[:, None]`: one value per row of the tile, laid back over the tile
+            positional, named = _kwargs(base)
+            axis = named.get("axis", positional[1] if len(positional) > 1 else None)
+            if not isinstance(axis, int) or len(keys) != len(dims):
+                raise UnsupportedProgram("Only the result of an axis reduction of the tile can be subscripted with `None`.")
+            expected = tuple(None if position == axis % len(dims) else slice(None) for position in range(len(dims)))
+            if tuple(keys) != expected:
+                raise UnsupportedProgram("The `None` of the subscript must stand at the reduced axis.")
+            self.axis_subscript_seen = True
+            return self.lower(base, dims, inside_reduction)
         if isinstance(base, Node) and base.op == "load" and isinstance(base.args[0], TensorRef):
             # `bias[None, :]`: a tile of lower rank laid along the dimensions the `:` entries name;
             # every element of the result reads the element of the tile at those coordinates
@@ -793,11 +817,14 @@ def _other_value(tensor):
 
 
 def _has_whole_tile_reduction(value):
+    """Whether the expression reduces whole tiles, or uses an axis reduction on the tile (`m[:, None]`)."""
     if isinstance(value, Node):
         if value.op in REDUCE:
             positional, named = _kwargs(value)
             if named.get("axis", positional[1] if len(positional) > 1 else None) is None:
                 return True
+        if value.op == "index" and isinstance(value.args[0], Node) and value.args[0].op in REDUCE:
+            return True
         return any(_has_whole_tile_reduction(arg) for arg in value.args)
     if isinstance(value, (tuple, list)):
         return any(_has_whole_tile_reduction(item) for item in value)
@@ -888,9 +915,10 @@ def _build(program_store, types, args, env, dtype_tag, data_ptr, tile_mode):
             stride_of[var] = abs(offset.coef(name)) if offset.is_linear() else None
     if order_slot is not None and all(stride_of.get(v) is not None for v in outer):
         outer.sort(key=lambda v: (-(stride_of[v] or 1 << 62) if lowering.var_extent[v] > 1 else -(1 << 62), v))
-    if tile_mode:  # the variables that enumerate tiles first, then those of the tile (fastest last, as sorted)
-        grid_vars = [v for v in outer if v in lowering.grid]
-        outer = grid_vars + [v for v in outer if v not in lowering.grid]
+    if tile_mode:  # the variables that enumerate tiles (or rows of tiles) first, then the reduced ones (fastest last, as sorted)
+        reduced_over = set(out_dims) if lowering.tile_axis is None else {out_dims[lowering.tile_axis]}
+        grid_vars = [v for v in outer if v not in reduced_over]
+        outer = grid_vars + [v for v in outer if v in reduced_over]
     order = {old: new for new, old in enumerate(outer + reduced + dynamic)}
     # SETVAR words were emitted with provisional ids: renumber them like the index code
     for position, word in enumerate(lowering.value_code):

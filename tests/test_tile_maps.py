@@ -904,3 +904,55 @@ def test_one_kernel_called_from_several_threads():
     for thread in threads:
         thread.join()
     assert not failures
+
+
+# ---- axis reductions laid back over the tile (`ntl.max(x, 1)[:, None]`) ---------------------------
+
+
+def _row_block_arrangement(input, output):
+    return input.tile((8, -1)), output.tile((8, -1))
+
+
+def _row_block_softmax_application(input, output):
+    shifted = input - ntl.max(input, 1)[:, None]
+    numerator = ntl.exp(shifted)
+    output = numerator / ntl.sum(numerator, axis=1)[:, None]  # noqa: F841
+
+
+def _column_normalise_application(input, output):
+    output = input / ntl.sum(input * input, axis=0)[None, :]  # noqa: F841
+
+
+def test_lowering_axis_reductions_used_on_the_tile():
+    x = torch.randn(37, 50)
+    kernel = ninetoothed.make(_row_block_arrangement, _row_block_softmax_application, (Tensor(2, other=float("-inf")), Tensor(2)))
+    out = torch.full_like(x, float("nan"))
+    _run_on_machine(kernel, (x, out))
+    assert torch.allclose(out, torch.softmax(x, -1), rtol=1e-5, atol=1e-7)
+
+    def columns(input, output):
+        return input.tile((-1, 4)), output.tile((-1, 4))
+
+    kernel = ninetoothed.make(columns, _column_normalise_application, (Tensor(2), Tensor(2)))
+    out = torch.full_like(x, float("nan"))
+    _run_on_machine(kernel, (x, out))
+    assert torch.allclose(out, x / (x * x).sum(0, keepdim=True), rtol=1e-5, atol=1e-7)
+
+    def mixed(input, output):
+        output = input - ntl.max(input, 1)[:, None] - ntl.max(input)  # noqa: F841
+
+    kernel = ninetoothed.make(_row_block_arrangement, mixed, (Tensor(2, other=float("-inf")), Tensor(2)))
+    with pytest.raises(UnsupportedProgram):
+        _run_on_machine(kernel, (x, torch.empty_like(x)))
+
+
+@gpu
+@pytest.mark.parametrize("interpret", ("0", "1"))
+def test_axis_reductions_used_on_the_tile(interpret, monkeypatch):
+    monkeypatch.setenv("NT_MAP_INTERPRET", interpret)
+    x = torch.randn(641, 1000, device="cuda")
+    kernel = ninetoothed.make(_row_block_arrangement, _row_block_softmax_application, (Tensor(2, other=float("-inf")), Tensor(2)))
+    out = torch.full_like(x, float("nan"))
+    kernel(x, out)
+    _served_by_map(kernel)
+    assert torch.allclose(out, torch.softmax(x, -1), rtol=1e-5, atol=1e-7)
