@@ -15,13 +15,14 @@ can be compared or pattern-matched structurally.
 """
 
 from ninetoothed_amd.symbol import Symbol
+from ninetoothed_amd.symbolic_int import integer, is_symbolic
 
 
 class Affine:
     __slots__ = ("const", "terms")
 
     def __init__(self, const=0, terms=None):
-        self.const = int(const)
+        self.const = integer(const)
         self.terms = {atom: coef for atom, coef in (terms or {}).items() if coef != 0}
 
     # atoms: ("var", name) | ("div", key, c) | ("mod", key, c); `key` = Affine.key()
@@ -117,7 +118,8 @@ def _split(expr, c):
     ``remainder`` not divisible by ``c`` and its constant in ``[0, c)``."""
     quotient_terms, remainder_terms = {}, {}
     for atom, coef in expr.terms.items():
-        if coef % c == 0:
+        # sizes only known at launch: any term may stay in the remainder, so nothing is decided from the sample
+        if not is_symbolic(coef, c) and coef % c == 0:
             quotient_terms[atom] = coef // c
         else:
             remainder_terms[atom] = coef
@@ -165,13 +167,13 @@ class Ranges:
         expr = _wrap(expr)
         if c <= 0:
             raise NotAffine("division by a non-positive constant")
-        if c == 1:
+        if not is_symbolic(c) and c == 1:
             return expr
         quotient, remainder = _split(expr, c)
         if remainder.is_const():
             return quotient + remainder.const // c
         lo, hi = self.interval(remainder)
-        if lo // c == hi // c:
+        if not is_symbolic(lo, hi, c) and lo // c == hi // c:
             return quotient + lo // c
         if len(remainder.terms) == 1 and remainder.const == 0:
             (atom, coef), = remainder.terms.items()
@@ -183,17 +185,17 @@ class Ranges:
         expr = _wrap(expr)
         if c <= 0:
             raise NotAffine("modulo by a non-positive constant")
-        if c == 1:
+        if not is_symbolic(c) and c == 1:
             return Affine(0)
         _, remainder = _split(expr, c)
         if remainder.is_const():
             return Affine(remainder.const % c)
         lo, hi = self.interval(remainder)
-        if lo // c == hi // c:
+        if not is_symbolic(lo, hi, c) and lo // c == hi // c:
             return remainder - (lo // c) * c
         if len(remainder.terms) == 1 and remainder.const == 0:
             (atom, coef), = remainder.terms.items()
-            if coef == 1 and atom[0] == "mod" and atom[2] % c == 0:  # (x % a) % c == x % c when c | a
+            if coef == 1 and atom[0] == "mod" and not is_symbolic(atom[2], c) and atom[2] % c == 0:  # (x % a) % c == x % c when c | a
                 return self.mod(Affine.from_key(atom[1]), c)
         return Affine(0, {("mod", remainder.key(), c): 1})
 
@@ -211,11 +213,11 @@ class Ranges:
         if expr.is_name:
             name = expr.name
             if name in env:
-                return Affine(int(env[name]))
+                return Affine(integer(env[name]))
             if name not in self.bounds:
                 raise NotAffine(f"unknown symbol `{name}`")
             lo, hi = self.bounds[name]
-            return Affine(lo) if lo == hi else Affine.var(name)
+            return Affine(lo) if not is_symbolic(lo, hi) and lo == hi else Affine.var(name)
         op = expr.op
         lhs = self.convert(expr.operands[0], env)
         rhs = self.convert(expr.operands[1], env)

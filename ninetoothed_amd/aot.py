@@ -13,9 +13,13 @@ point of the recognised program with the element type and block sizes fixed at
 packaging time, and ``<kernel_name>.so`` is built from it and linked against
 ``libnt_hip.so``.
 
-Only the recognised programs (matmul, addmm, softmax, attention, conv2d) can be packaged: tile maps are lowered per
-call from the sizes of the arguments (``ninetoothed_amd.mapping``), which a C
-dispatcher cannot do.
+Element-wise and reducing programs (tile maps) are lowered from the sizes of a call
+(``ninetoothed_amd.mapping``).  For a package that lowering runs once, on sample sizes that
+remember how every number was computed (``ninetoothed_amd.symbolic_int``): the C launch
+function holds the lowered ``NineToothedMapProgram`` as a constant, checks the recorded
+decisions against the sizes it is called with (returning 1, "no kernel", when one comes out
+differently), recomputes the size-dependent fields and calls ``launch_nt_map``.  Declared
+sizes (``Tensor(shape=(4096,))``) are plain numbers: nothing is left to check but the sizes.
 """
 
 import ctypes
@@ -134,6 +138,196 @@ def _check_structure(kernel, constexprs):
     raise UnsupportedProgram(f"Programs of kind `{kind}` cannot be packaged ahead of time.")
 
 
+# sample sizes for dimensions that are only known at launch, innermost first: odd, so that no
+# tile size divides them (bounds checks stay in), and pairwise different
+_SAMPLE_SIZES = (1000003, 1009, 101, 11, 7, 5, 3, 3)
+
+
+def _c_double(value):
+    if value != value:
+        return "NAN"
+    if value in (float("inf"), float("-inf")):
+        return "INFINITY" if value > 0 else "-INFINITY"
+    return float(value).hex()
+
+
+def _c_initialiser(structure, indent="    "):
+    """A ctypes structure as a C designated initialiser (zero fields and array tails left out)."""
+    parts = []
+    for field, kind in structure._fields_:
+        value = getattr(structure, field)
+        if isinstance(value, ctypes.Array):
+            items = list(value)
+            if items and isinstance(items[0], ctypes.Structure):
+                texts = [_c_initialiser(item, indent + "    ") for item in items]
+                while texts and texts[-1] == "{0}":
+                    texts.pop()
+            else:
+                while items and items[-1] == 0 and not (isinstance(items[-1], float) and str(items[-1]) == "-0.0"):
+                    items.pop()
+                texts = [_c_double(item) if isinstance(item, float) else str(item) for item in items]
+            if texts:
+                parts.append(f".{field} = {{{', '.join(texts)}}}")
+        elif isinstance(value, float):
+            if value != 0 or str(value) == "-0.0":
+                parts.append(f".{field} = {_c_double(value)}")
+        elif value:
+            parts.append(f".{field} = {value}")
+    if not parts:
+        return "{0}"
+    return "{" + ", ".join(parts) + "}"
+
+
+_FLOAT_TAGS = ("fp16", "bf16", "fp32", "fp64")
+
+
+class MapPackage:
+    """A tile-map program lowered on sample sizes: the programs, the size expressions of their
+    call-dependent fields, and the decisions (guards) under which they hold."""
+
+    def __init__(self, kernel, constexprs):
+        from ninetoothed_amd import mapping
+        from ninetoothed_amd.symbol import Symbol
+        from ninetoothed_amd.symbolic_int import Recorder, SymInt
+
+        self.parameters = list(kernel.parameters)
+        self.declared = []       # (parameter, dimension, size) fixed by the tensors' declarations
+        self.scalar_dtypes = {}  # parameter position -> element type of a call-time scalar
+        env, tags, sample_args = {}, {}, []
+        # a dimension some tensor declares is the sample for the undeclared ones at the same place
+        # (counted from the innermost), so that tensors of one shape stay of one shape
+        samples = {}
+        for tensor in kernel.types:
+            for dim, declared in enumerate(tensor.source.shape):
+                if not isinstance(declared, Symbol):
+                    samples.setdefault(tensor.source.ndim - 1 - dim, int(declared))
+        for position, (parameter, tensor) in enumerate(zip(self.parameters, kernel.types)):
+            source = tensor.source
+            if tensor.ndim == 0 and not isinstance(tensor.dtype, Tensor):
+                if tensor.constexpr:
+                    raise UnsupportedProgram("Compile-time scalars of a packaged element-wise program are not supported: declare a plain `Tensor(0)`.")
+                declared = source.dtype if isinstance(source.dtype, str) else "fp64"
+                if declared not in _ENUM_NAMES:
+                    raise UnsupportedProgram(f"Scalar `{parameter}` has no packaged representation for type `{declared}`.")
+                self.scalar_dtypes[position] = declared
+                sample_args.append(1.0 if declared in _FLOAT_TAGS else 1)
+                continue
+            if source.jagged_dim is not None:
+                raise UnsupportedProgram("Jagged tensors cannot be packaged ahead of time.")
+            tags[position] = _element_type(tensor, parameter)
+            sample_args.append(None)
+            shape, sample_shape = [], []
+            for dim, declared in enumerate(source.shape):
+                if isinstance(declared, Symbol):
+                    sample = samples.get(source.ndim - 1 - dim, _SAMPLE_SIZES[source.ndim - 1 - dim])
+                    shape.append(SymInt.symbol(f"{parameter}.shape[{dim}]", sample))
+                else:
+                    sample = int(declared)
+                    shape.append(sample)
+                    self.declared.append((parameter, dim, sample))
+                sample_shape.append(sample)
+            stride = 1
+            for dim in reversed(range(source.ndim)):
+                env[source.stride_string(dim)] = SymInt.symbol(f"{parameter}.strides[{dim}]", stride)
+                stride *= sample_shape[dim]
+            for dim, declared in enumerate(source.shape):
+                if isinstance(declared, Symbol) and declared.is_name:
+                    env[declared.name] = shape[dim]
+                env[source.size_string(dim)] = shape[dim]
+        env.update(constexprs)
+        for symbol in kernel.meta_symbols:
+            env.setdefault(symbol, 1)
+
+        with Recorder() as recorder:
+            self.launches = []  # (program, scalar slots, operand parameters)
+            for store in kernel.program.stores:
+                built = mapping.build(store, kernel.types, sample_args, env, lambda p: tags[p], lambda p: 0, self.scalar_dtypes)
+                if built is None:
+                    raise UnsupportedProgram("The sample sizes give an empty launch: the program cannot be packaged.")
+                program, _, scalar_slots, operand_params = built
+                if any(isinstance(param, tuple) for param in operand_params):
+                    raise UnsupportedProgram("Jagged tensors cannot be packaged ahead of time.")
+                self.launches.append((program, scalar_slots, operand_params))
+        self.guards = dict(recorder.guards)
+
+    def instantiate(self, shapes, strides, scalars):
+        """What the packaged C code computes for one call, in Python: the list of programs (data
+        pointers left at zero), or ``None`` when a declared size or a guard does not hold.
+        ``shapes`` / ``strides`` / ``scalars``: by parameter name."""
+        from ninetoothed_amd import mapping
+        from ninetoothed_amd.symbolic_int import evaluate, holds
+
+        if any(shapes[parameter][dim] != size for parameter, dim, size in self.declared):
+            return None
+        symbols = {}
+        for parameter, shape in shapes.items():
+            for dim, size in enumerate(shape):
+                symbols[f"{parameter}.shape[{dim}]"] = size
+                symbols[f"{parameter}.strides[{dim}]"] = strides[parameter][dim]
+        for key, outcome in self.guards.items():
+            if not holds(key, outcome, symbols):
+                return None
+        programs = []
+        for template, scalar_slots, _ in self.launches:
+            program = mapping.MapProgram.from_buffer_copy(bytes(template))
+            for field, value in template.patches:
+                name, index = field[:-1].split("[")
+                getattr(program, name)[int(index)] = evaluate(value.expr, symbols)
+            for index, param in scalar_slots:
+                program.value_constants[index] = float(scalars[self.parameters[param]])
+            programs.append(program)
+        return programs
+
+    def c_source(self, name):
+        """Header and source of ``launch_<name>``."""
+        from ninetoothed_amd.symbolic_int import C_HELPERS, CWriter
+
+        parameters = self.parameters
+        writer = CWriter()
+        body = []
+        if self.declared:
+            body.append("/* sizes the tensors were declared with */")
+            checks = " || ".join(f"{parameter}.shape[{dim}] != {size}ULL" for parameter, dim, size in self.declared)
+            body.append(f"if ({checks})\n        return 1;")
+        if self.guards:
+            body.append("/* decisions the lowering took on its sample sizes: the programs below hold for calls that repeat them */")
+        for key, outcome in self.guards.items():
+            failure = writer.failure(key, outcome)
+            body.extend(writer.take_lines())
+            body.append(f"if ({failure})\n        return 1;")
+        templates = []
+        for number, (program, scalar_slots, operand_params) in enumerate(self.launches):
+            templates.append(f"static const NineToothedMapProgram {name}_program_{number} = {_c_initialiser(program)};")
+            block = [f"NineToothedMapProgram program = {name}_program_{number};"]
+            for field, value in program.patches:
+                text = writer.value(value.expr)
+                body.extend(writer.take_lines())
+                block.append(f"program.{field} = {'(double)' if field.startswith('value_constants') else ''}{text};")
+            for slot, param in enumerate(operand_params):
+                block.append(f"program.operands[{slot}].data = {parameters[param]}.data;")
+            for index, param in scalar_slots:
+                read = "*(const double *)" if self.scalar_dtypes[param] in _FLOAT_TAGS else "(double)*(const int64_t *)"
+                block.append(f"program.value_constants[{index}] = {read}{parameters[param]}.data;")
+            block.append("NineToothedResult result = launch_nt_map(stream, &program);")
+            block.append("if (result != 0)\n            return result;")
+            body.append("{\n        " + "\n        ".join(block) + "\n    }")
+        body.append("return 0;")
+
+        arguments = ", ".join(f"NineToothedTensor {parameter}" for parameter in parameters)
+        signature = f"NineToothedResult launch_{name}(NineToothedStream stream, {arguments})"
+        header = (
+            f"/* launch_{name}: packaged element-wise program ({len(self.launches)} launch(es) of launch_nt_map in libnt_hip.so). */\n"
+            f"#ifndef NINETOOTHED_{name.upper()}_H\n#define NINETOOTHED_{name.upper()}_H\n\n"
+            '#include "ninetoothed_hip.h"\n\n#ifdef __cplusplus\nextern "C" {\n#endif\n\n'
+            f"{signature};\n\n#ifdef __cplusplus\n}}\n#endif\n\n#endif\n"
+        )
+        source = (
+            f'#include "{name}.h"\n\n#include <math.h>\n#include <stdint.h>\n\n' + C_HELPERS + "\n" + "\n".join(templates)
+            + f"\n\n{signature} {{\n    " + "\n    ".join(body) + "\n}\n"
+        )
+        return header, source
+
+
 def _dispatcher_source(kernel, name, dtype, out_dtype, blocks):
     parameters = ", ".join(f"NineToothedTensor {parameter}" for parameter in kernel.parameters)
     signature = f"NineToothedResult launch_{name}(NineToothedStream stream, {parameters})"
@@ -177,6 +371,14 @@ def generate(arrangement, application, tensors, kernel_name, output_dir, constex
     types = arrangement(*tensors)
     types = types if isinstance(types, tuple) else (types,)
     kernel = Kernel(application, types, kernel_name=kernel_name)
+    output_dir = pathlib.Path(output_dir)
+    if kernel.kind == "map":
+        kernel.map_package = MapPackage(kernel, dict(constexprs or {}))
+        header, source = kernel.map_package.c_source(kernel_name)
+        output_dir.mkdir(parents=True, exist_ok=True)
+        (output_dir / f"{kernel_name}.h").write_text(header)
+        (output_dir / f"{kernel_name}.c").write_text(source)
+        return kernel
     blocks = _check_structure(kernel, dict(constexprs or {}))
     if not block_hints:
         blocks = {name: value for name, value in blocks.items() if name not in ("m", "n", "k")}
@@ -187,7 +389,6 @@ def generate(arrangement, application, tensors, kernel_name, output_dir, constex
         if _element_type(tensor, "an operand") != dtype:
             raise UnsupportedProgram("Operands of a packaged kernel must share one element type.")
     header, source = _dispatcher_source(kernel, kernel_name, dtype, out_dtype, blocks)
-    output_dir = pathlib.Path(output_dir)
     output_dir.mkdir(parents=True, exist_ok=True)
     (output_dir / f"{kernel_name}.h").write_text(header)
     (output_dir / f"{kernel_name}.c").write_text(source)
@@ -226,7 +427,7 @@ class PackagedKernel:
         self.library_path = str(library_path)
         self.kernel_name = kernel_name
         self.kind = kernel.kind
-        self._scalar = [t.ndim == 0 and not isinstance(t.dtype, Tensor) for t in kernel.types]
+        self._scalar = scalar_kinds(kernel)
         self._library = ctypes.CDLL(self.library_path)
         self._function = getattr(self._library, f"launch_{kernel_name}")
         self._function.argtypes = [ctypes.c_void_p] + [runtime.ArgumentTensor] * len(kernel.types)
@@ -239,15 +440,34 @@ class PackagedKernel:
         runtime.check(self._function(runtime.current_stream(), *marshal(args, self._scalar)))
 
 
+def scalar_kinds(kernel):
+    """Per application parameter: ``None`` for a tensor, else how the launch function reads the
+    zero-dimensional tensor -- ``"float"`` (a host double) or ``"int"`` (a host int64).  The
+    declared element type decides (src/ninetoothed/aot.py:234-283, 610-630); undeclared scalars
+    are doubles, except the causal flag of the attention program."""
+    kinds = []
+    for position, tensor in enumerate(kernel.types):
+        if not (tensor.ndim == 0 and not isinstance(tensor.dtype, Tensor)):
+            kinds.append(None)
+        elif isinstance(tensor.source.dtype, str):
+            kinds.append("float" if tensor.source.dtype in _FLOAT_TAGS else "int")
+        else:
+            kinds.append("int" if kernel.kind == "attention" and position == 3 else "float")
+    return kinds
+
+
 def marshal(args, scalar):
-    """Torch tensors and Python scalars as the ``NineToothedTensor`` values a packaged launch function takes."""
+    """Torch tensors and Python scalars as the ``NineToothedTensor`` values a packaged launch function
+    takes; ``scalar``: per argument ``None`` / ``False`` (a tensor), ``"float"``, ``"int"`` or ``True``
+    (by the type of the Python value)."""
     import torch
 
     marshalled = []
-    for arg, is_scalar in zip(args, scalar):
-        if is_scalar:
+    for arg, kind in zip(args, scalar):
+        if kind:
             value = arg.item() if isinstance(arg, torch.Tensor) else arg
-            marshalled.append(runtime.ArgumentTensor.from_scalar(float(value) if isinstance(value, float) else int(value)))
+            is_float = isinstance(value, float) if kind is True else kind == "float"
+            marshalled.append(runtime.ArgumentTensor.from_scalar(float(value) if is_float else int(value)))
         else:
             if not arg.is_cuda:
                 raise RuntimeError("Packaged kernels run on the GPU only (there is no CPU path).")

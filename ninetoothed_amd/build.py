@@ -99,7 +99,11 @@ def _build(premake, configs, meta_parameters, caller, kernel_name, output_dir):
 
     tensor_parameters = max((c.parameters for c in configurations), key=len)
     config_parameters = tuple(dict.fromkeys(name for key in branches for name, _ in key))
-    scalar = [t.ndim == 0 and not isinstance(t.dtype, Tensor) for t in configurations[0].tensors]
+    # scalars travel as host doubles / int64s: by the declared element type, else by the Python value's type
+    scalar = [
+        (("float" if t.dtype in aot._FLOAT_TAGS else "int") if isinstance(t.dtype, str) else True) if t.ndim == 0 and not isinstance(t.dtype, Tensor) else None
+        for t in configurations[0].tensors
+    ]
 
     if not (library.exists() and fingerprint_path.exists() and fingerprint_path.read_text().strip() == fingerprint):
         sources, includes, launches = [], [], []

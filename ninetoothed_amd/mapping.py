@@ -36,6 +36,7 @@ from ninetoothed_amd import runtime
 from ninetoothed_amd.affine import Affine
 from ninetoothed_amd.recognition import Operand, UnsupportedProgram
 from ninetoothed_amd.symbol import evaluate
+from ninetoothed_amd.symbolic_int import integer, is_symbolic, plain, same
 from ninetoothed_amd.tracing import Dim, ElementType, Node, ScalarParam, SourceDim, SourceStride, TensorRef
 
 MAX_OPERANDS = 8
@@ -225,8 +226,11 @@ def _first_tile_ref(value):
 class _Lowering:
     """One store of one call: collects operands, index segments and value code."""
 
-    def __init__(self, types, args, env, dtype_tag, tile_mode=False):
+    def __init__(self, types, args, env, dtype_tag, tile_mode=False, scalar_dtypes=None):
         self.types, self.args, self.env, self.dtype_tag = types, args, env, dtype_tag
+        # packaged kernels: a scalar has the element type it was declared with, whatever Python number
+        # stands in for it (the reference's AOT signature, src/ninetoothed/aot.py:234-283)
+        self.scalar_dtypes = scalar_dtypes or {}
         # tile mode: whole-tile reductions become phases whose results the expression may use on
         # every element of the tile; `phases` holds (operation, accumulate type, term code)
         self.tile_mode = tile_mode
@@ -247,6 +251,7 @@ class _Lowering:
         self.num_reduced = 0
         self.bindings = {}        # operand slot -> {operand variable name: shared variable id}
         self.scalar_slots = []    # (constant index, parameter position): refreshed at every launch
+        self.symbolic_constants = {}  # constant index -> size expression (packaging only)
         self.reduced_vars = []
         self.dynamic_vars = []    # variables that take their value from the data (level indices)
         self.levels_used = {}     # param -> level its tiles are taken from
@@ -254,7 +259,7 @@ class _Lowering:
 
     # -- variables ---------------------------------------------------------
     def new_var(self, extent):
-        self.var_extent.append(int(extent))
+        self.var_extent.append(integer(extent))
         return len(self.var_extent) - 1
 
     def operand(self, param, level=1):
@@ -315,8 +320,12 @@ class _Lowering:
         self.value_code.append(V[op] | (arg << 8))
 
     def constant(self, value):
+        if is_symbolic(value):  # a size of the call used as a value: its own slot, filled in per launch by packaged code
+            self.constants.append(float(plain(value)))
+            self.symbolic_constants[len(self.constants) - 1] = value
+            return len(self.constants) - 1
         value = float(value)
-        scalars = {index for index, _ in self.scalar_slots}
+        scalars = {index for index, _ in self.scalar_slots} | set(self.symbolic_constants)
         for index, known in enumerate(self.constants):
             if index not in scalars and (known == value or (known != known and value != value)):
                 return index
@@ -350,6 +359,9 @@ class _Lowering:
             self.constants.append(float(arg))  # a slot of its own: call-time scalars are refreshed per launch
             self.scalar_slots.append((len(self.constants) - 1, value.param))
             self.emit("CONST", len(self.constants) - 1)
+            if value.param in self.scalar_dtypes:
+                self.round(self.scalar_dtypes[value.param])
+                return self.scalar_dtypes[value.param]
             if value.constexpr:
                 return "bool" if isinstance(arg, bool) else _LITERAL_INT if isinstance(arg, int) else _LITERAL_FLOAT
             if isinstance(arg, bool):
@@ -361,11 +373,11 @@ class _Lowering:
         if isinstance(value, (SourceDim, SourceStride)):
             source = self.types[value.param].source
             name = source.size_string(value.dim) if isinstance(value, SourceDim) else source.stride_string(value.dim)
-            self.emit("CONST", self.constant(int(self.env[name])))
+            self.emit("CONST", self.constant(integer(self.env[name])))
             return _LITERAL_INT
         if isinstance(value, Dim):  # `x.shape[d]` of a level: a call-time integer
             level = self.types[value.param].levels()[value.level]
-            self.emit("CONST", self.constant(int(evaluate(level.shape[value.dim], self.env))))
+            self.emit("CONST", self.constant(integer(evaluate(level.shape[value.dim], self.env))))
             return _LITERAL_INT
         if not isinstance(value, Node):
             raise UnsupportedProgram(f"A value of type `{type(value).__name__}` cannot be stored by the element-wise executor.")
@@ -606,7 +618,7 @@ class _Lowering:
         self.bindings[slot] = {}
 
         def dynamic(value, size):
-            var = self.new_var(max(int(size), 1) if size is not None else 1)
+            var = self.new_var(max(integer(size), 1) if size is not None else 1)
             self.dynamic_vars.append(var)
             self.lower(value, dims, inside_reduction)
             self.emit("SETVAR", var)
@@ -619,8 +631,8 @@ class _Lowering:
         if len(indices) != source.ndim:
             raise UnsupportedProgram("A source tensor needs one index per dimension.")
         for dim, index in enumerate(indices):
-            size = int(self.env[source.size_string(dim)])
-            raw.terms.append((dynamic(index, size), int(self.env[source.stride_string(dim)]), size))
+            size = integer(self.env[source.size_string(dim)])
+            raw.terms.append((dynamic(index, size), integer(self.env[source.stride_string(dim)]), size))
         return slot
 
     def new_var_deferred(self):
@@ -706,10 +718,12 @@ class _Lowering:
         code, constants, begins = [], [], []
 
         def const(value):
-            value = int(value)
-            if value not in constants:
-                constants.append(value)
-            return constants.index(value)
+            value = integer(value)
+            for index, known in enumerate(constants):
+                if same(known, value):
+                    return index
+            constants.append(value)
+            return len(constants) - 1
 
         def emit_affine(expr, binding):
             code.append(I_CONST | (const(expr.const) << 8))
@@ -721,7 +735,7 @@ class _Lowering:
                 else:
                     emit_affine(Affine.from_key(atom[1]), binding)
                     code.append((I_DIVC if atom[0] == "div" else I_MODC) | (const(atom[2]) << 8))
-                if coef != 1:
+                if is_symbolic(coef) or coef != 1:
                     code.append(I_MULC | (const(coef) << 8))
                 code.append(I_ADD)
 
@@ -729,7 +743,7 @@ class _Lowering:
             if slot in self.jagged:
                 source = operand.tensor.source
                 code.append(I_VAR | (order[self.jagged[slot][0]] << 8))
-                code.append(I_MULC | (const(int(self.env[source.stride_string(source.jagged_dim)])) << 8))
+                code.append(I_MULC | (const(integer(self.env[source.stride_string(source.jagged_dim)])) << 8))
                 code.append(I_ADD)
 
         for slot, kind, dim in self.segments:
@@ -744,7 +758,7 @@ class _Lowering:
                 code.append(I_CONST | (const(0) << 8))
                 for var, stride, _ in operand.terms:
                     code.append(I_VAR | (order[var] << 8))
-                    if stride != 1:
+                    if is_symbolic(stride) or stride != 1:
                         code.append(I_MULC | (const(stride) << 8))
                     code.append(I_ADD)
             elif kind == "access":
@@ -831,7 +845,7 @@ def _has_whole_tile_reduction(value):
     return False
 
 
-def build(program_store, types, args, env, dtype_tag, data_ptr):
+def build(program_store, types, args, env, dtype_tag, data_ptr, scalar_dtypes=None):
     """Builds the :class:`MapProgram` of one store for one call.  Returns
     ``None`` when the launch is empty.
 
@@ -839,16 +853,16 @@ def build(program_store, types, args, env, dtype_tag, data_ptr):
     output element); when the expression does not have that form but reduces whole tiles, the
     program is built in tile mode (reductions as phases of a workgroup that owns the tile)."""
     try:
-        return _build(program_store, types, args, env, dtype_tag, data_ptr, False)
+        return _build(program_store, types, args, env, dtype_tag, data_ptr, False, scalar_dtypes)
     except UnsupportedProgram:
         if not isinstance(program_store[0], TensorRef) or not _has_whole_tile_reduction(program_store[1]):
             raise
-        return _build(program_store, types, args, env, dtype_tag, data_ptr, True)
+        return _build(program_store, types, args, env, dtype_tag, data_ptr, True, scalar_dtypes)
 
 
-def _build(program_store, types, args, env, dtype_tag, data_ptr, tile_mode):
+def _build(program_store, types, args, env, dtype_tag, data_ptr, tile_mode, scalar_dtypes=None):
     ref, value = program_store
-    lowering = _Lowering(types, args, env, dtype_tag, tile_mode)
+    lowering = _Lowering(types, args, env, dtype_tag, tile_mode, scalar_dtypes)
     store_op = 0
     if isinstance(ref, TensorRef):
         lowering._check_ref(ref)
@@ -912,9 +926,10 @@ def _build(program_store, types, args, env, dtype_tag, data_ptr, tile_mode):
     if order_slot is not None:
         offset = lowering.operands[order_slot][1].offset()
         for name, var in lowering.bindings[order_slot].items():
-            stride_of[var] = abs(offset.coef(name)) if offset.is_linear() else None
+            stride_of[var] = abs(plain(offset.coef(name))) if offset.is_linear() else None
     if order_slot is not None and all(stride_of.get(v) is not None for v in outer):
-        outer.sort(key=lambda v: (-(stride_of[v] or 1 << 62) if lowering.var_extent[v] > 1 else -(1 << 62), v))
+        # (plain values: the order is a layout choice that no size of a call can make wrong)
+        outer.sort(key=lambda v: (-(stride_of[v] or 1 << 62) if plain(lowering.var_extent[v]) > 1 else -(1 << 62), v))
     if tile_mode:  # the variables that enumerate tiles (or rows of tiles) first, then the reduced ones (fastest last, as sorted)
         reduced_over = set(out_dims) if lowering.tile_axis is None else {out_dims[lowering.tile_axis]}
         grid_vars = [v for v in outer if v not in reduced_over]
@@ -934,11 +949,18 @@ def _build(program_store, types, args, env, dtype_tag, data_ptr, tile_mode):
         raise UnsupportedProgram("The expression is too long for the element-wise executor.")
 
     program = MapProgram()
+    patches = []  # (C lvalue inside the program, size expression): what packaged code recomputes per launch
+
+    def number(field, value):
+        if is_symbolic(value):
+            patches.append((field, value))
+        return plain(value)
+
     program.num_vars = len(outer) + len(reduced)
     program.num_reduced = len(reduced)
     program.num_dynamic = len(dynamic)
     for old, new in order.items():
-        program.extents[new] = lowering.var_extent[old]
+        program.extents[new] = number(f"extents[{new}]", lowering.var_extent[old])
     program.store_op = store_op
     if tile_mode:
         program.num_phases = len(lowering.phases)
@@ -960,7 +982,7 @@ def _build(program_store, types, args, env, dtype_tag, data_ptr, tile_mode):
     for index, word in enumerate(code):
         program.index_code[index] = word
     for index, value_ in enumerate(constants):
-        program.index_constants[index] = value_
+        program.index_constants[index] = number(f"index_constants[{index}]", value_)
     program.value_code_length = len(lowering.value_code)
     program.reduce_split = lowering.reduce_split
     program.reduce_op = REDUCE[lowering.reduce[0]] if lowering.reduce else 0
@@ -969,14 +991,17 @@ def _build(program_store, types, args, env, dtype_tag, data_ptr, tile_mode):
         program.value_code[index] = word
     for index, value_ in enumerate(lowering.constants):
         program.value_constants[index] = value_
+    for index, value_ in lowering.symbolic_constants.items():
+        patches.append((f"value_constants[{index}]", value_))
     description = (
-        f"{len(lowering.operands)} operands, {program.num_vars} index variables {[lowering.var_extent[old] for old in outer + reduced]}, "
+        f"{len(lowering.operands)} operands, {program.num_vars} index variables {[plain(lowering.var_extent[old]) for old in outer + reduced]}, "
         + (f"{len(dynamic)} data-dependent, " if dynamic else "")
         + 
         f"{len(code)} index words, {len(lowering.value_code)} value words"
         + (f", {lowering.reduce[0]} over {len(reduced)} dimension(s)" if lowering.reduce else "")
         + (f", {len(lowering.phases)} whole-tile reduction(s), one workgroup per tile" if tile_mode else "")
     )
+    program.patches = patches
     return program, description, list(lowering.scalar_slots), [param for param, _ in lowering.operands]
 
 

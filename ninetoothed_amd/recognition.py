@@ -21,6 +21,7 @@ import functools
 from ninetoothed_amd import programs
 from ninetoothed_amd.affine import Affine, NotAffine, Ranges
 from ninetoothed_amd.symbol import Symbol, evaluate
+from ninetoothed_amd.symbolic_int import constant_difference, integer, is_symbolic, same_structure
 from ninetoothed_amd.tensor import Tensor
 from ninetoothed_amd.tracing import Carried, Dim, LoopVar, Node, Program, TensorRef, TracingError, trace
 
@@ -181,16 +182,16 @@ class Operand:
         extents = {}
         for level, level_names in zip(levels, self.names):
             for name, size in zip(level_names, level.shape):
-                extents[name] = int(evaluate(size, env))
+                extents[name] = integer(evaluate(size, env))
         self.extents = extents
         self.empty = any(extent <= 0 for extent in extents.values())
         self.ranges = Ranges({name: max(extent, 1) for name, extent in extents.items()})
         source = tensor.source
-        self.source_shape = [int(evaluate(size, env)) for size in source.shape]
-        self.source_strides = [int(env[source.stride_string(d)]) for d in range(source.ndim)]
+        self.source_shape = [integer(evaluate(size, env)) for size in source.shape]
+        self.source_strides = [integer(env[source.stride_string(d)]) for d in range(source.ndim)]
         try:
             self.indices = [self.ranges.convert(index, env) for index in source_indices]
-            self.constraints = [(self.ranges.convert(index, env), int(evaluate(size, env))) for index, size in constraints]
+            self.constraints = [(self.ranges.convert(index, env), integer(evaluate(size, env))) for index, size in constraints]
         except NotAffine as error:
             raise UnsupportedProgram(f"Index map of `{source.name}` is not div/mod-affine: {error}") from error
         self._prune()
@@ -200,7 +201,14 @@ class Operand:
         remaining = []
         for index, size in self.constraints:
             lo, hi = self.ranges.interval(index)
-            if (lo < 0 or hi >= size) and (index, size) not in remaining:
+            # sizes only known at launch: the check stays unless the bounds show for every call that it holds
+            if is_symbolic(lo, hi, size):
+                below, above = constant_difference(lo, 0), constant_difference(hi, size)
+                if below is not None and below >= 0 and above is not None and above < 0:
+                    continue
+                if not any(same_structure((index.key(), size), (known.key(), bound)) for known, bound in remaining):
+                    remaining.append((index, size))
+            elif (lo < 0 or hi >= size) and (index, size) not in remaining:
                 remaining.append((index, size))
         self.constraints = remaining
 

@@ -43,7 +43,7 @@ def test_packaging_writes_header_source_and_library(tmp_path):
     assert subprocess.run(command, capture_output=True, text=True).returncode == 0
 
 
-def test_packaging_needs_element_types_and_a_recognised_program(tmp_path):
+def test_packaging_needs_element_types(tmp_path):
     with pytest.raises(UnsupportedProgram):
         _package(tmp_path, "untyped", programs.matmul.arrangement, programs.matmul.application, programs.matmul.tensors())
 
@@ -54,7 +54,7 @@ def test_packaging_needs_element_types_and_a_recognised_program(tmp_path):
         y = x + 1  # noqa: F841
 
     with pytest.raises(UnsupportedProgram):
-        _package(tmp_path, "add_one", arrangement, application, (Tensor(1, dtype=ninetoothed.float32), Tensor(1, dtype=ninetoothed.float32)))
+        _package(tmp_path, "add_one", arrangement, application, (Tensor(1), Tensor(1, dtype=ninetoothed.float32)))
 
 
 @pytest.mark.gpu
