@@ -40,14 +40,15 @@ struct GemmInstance {
 // the fast instances take B row-major ([K, N], unit column stride) or transposed ([N, K] storage, unit k stride)
 bool b_is_transposed(const GemmProblem &q) { return q.sbn != 1 && q.sbk == 1; }
 
-template <int BM, int BN, int BK, int kStages>
+template <int BM, int BN, int BK, int kStages, bool kTail = false>
 bool fast_accepts(const GemmProblem &q) {
     if (q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) return false;
     // the element type, or fp32 for a plain product (the accumulators as they are)
     if (q.out_dtype != q.dtype && !(q.out_dtype == NINETOOTHED_FLOAT32 && !q.addmm())) return false;
     if (q.m <= 0 || q.n <= 0 || q.k <= 0) return false;
-    // any number of rows: rows past M read as zeros and are not stored; N and K must fit the tile
-    if (q.n % BN || q.k % BK) return false;
+    // any number of rows: rows past M read as zeros and are not stored; N and K must fit the tile,
+    // or, for the instances with tails, be multiples of 8 (whole 16-byte chunks)
+    if (kTail ? (q.n % 8 || q.k % 8) : (q.n % BN || q.k % BK)) return false;
     if (q.sak != 1 || q.scn != 1) return false;
     if (q.sam % 8 || q.sam < q.k || q.scm < q.n) return false;
     if (((uintptr_t)q.a & 15) || ((uintptr_t)q.b & 15) || ((uintptr_t)q.c & 15) || q.scm % 8) return false;
@@ -79,33 +80,33 @@ void fill_params(GemmParams &p, const GemmProblem &q, int bm, int bn) {
     p.alpha = q.alpha;
     p.beta = q.beta;
     p.tiles_m = (q.m + bm - 1) / bm;
-    p.tiles_n = q.n / bn;
+    p.tiles_n = (q.n + bn - 1) / bn;
     p.order = g_tile_order;
     p.bias_vector = q.bias != nullptr && q.sin == 1 && q.sim % 8 == 0 && ((uintptr_t)q.bias & 15) == 0;
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int kStages, int kOcc, int kAblate, int kLoad, int kAux>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int kStages, int kOcc, int kAblate, int kLoad, int kAux, bool kTail>
 hipError_t fast_launch_typed(const GemmProblem &q, hipStream_t stream) {
     GemmParams p;
     fill_params(p, q, BM, BN);
     const dim3 grid(p.tiles_m * p.tiles_n), block(WM * WN * 64);
     const bool f32 = q.out_dtype == NINETOOTHED_FLOAT32, addmm = q.addmm();
     if (b_is_transposed(q)) {
-        if (f32) gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, false, kAblate, kLoad, kAux, true, true><<<grid, block, 0, stream>>>(p);
-        else if (addmm) gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, true, kAblate, kLoad, kAux, false, true><<<grid, block, 0, stream>>>(p);
-        else gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, false, kAblate, kLoad, kAux, false, true><<<grid, block, 0, stream>>>(p);
+        if (f32) gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, false, kAblate, kLoad, kAux, true, true, kTail><<<grid, block, 0, stream>>>(p);
+        else if (addmm) gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, true, kAblate, kLoad, kAux, false, true, kTail><<<grid, block, 0, stream>>>(p);
+        else gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, false, kAblate, kLoad, kAux, false, true, kTail><<<grid, block, 0, stream>>>(p);
     } else {
-        if (f32) gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, false, kAblate, kLoad, kAux, true><<<grid, block, 0, stream>>>(p);
-        else if (addmm) gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, true, kAblate, kLoad, kAux><<<grid, block, 0, stream>>>(p);
-        else gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, false, kAblate, kLoad, kAux><<<grid, block, 0, stream>>>(p);
+        if (f32) gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, false, kAblate, kLoad, kAux, true, false, kTail><<<grid, block, 0, stream>>>(p);
+        else if (addmm) gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, true, kAblate, kLoad, kAux, false, false, kTail><<<grid, block, 0, stream>>>(p);
+        else gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, false, kAblate, kLoad, kAux, false, false, kTail><<<grid, block, 0, stream>>>(p);
     }
     return hipGetLastError();
 }
 
-template <int BM, int BN, int BK, int WM, int WN, int kStages, int kOcc, int kAblate = 0, int kLoad = 1, int kAux = 0>
+template <int BM, int BN, int BK, int WM, int WN, int kStages, int kOcc, int kAblate = 0, int kLoad = 1, int kAux = 0, bool kTail = false>
 hipError_t fast_launch(const GemmProblem &q, hipStream_t stream) {
-    if (q.dtype == NINETOOTHED_FLOAT16) return fast_launch_typed<half_t, BM, BN, BK, WM, WN, kStages, kOcc, kAblate, kLoad, kAux>(q, stream);
-    return fast_launch_typed<bf16_t, BM, BN, BK, WM, WN, kStages, kOcc, kAblate, kLoad, kAux>(q, stream);
+    if (q.dtype == NINETOOTHED_FLOAT16) return fast_launch_typed<half_t, BM, BN, BK, WM, WN, kStages, kOcc, kAblate, kLoad, kAux, kTail>(q, stream);
+    return fast_launch_typed<bf16_t, BM, BN, BK, WM, WN, kStages, kOcc, kAblate, kLoad, kAux, kTail>(q, stream);
 }
 
 bool generic_accepts(const GemmProblem &q) {
@@ -180,6 +181,10 @@ hipError_t generic_launch(const GemmProblem &q, hipStream_t stream) {
 #define NT_FAST_INSTANCE(BM, BN, BK, WM, WN, ST, OCC) \
     {#BM "x" #BN "x" #BK " waves " #WM "x" #WN " stages " #ST " lds-direct", BM, BN, BK, fast_accepts<BM, BN, BK, ST>, fast_launch<BM, BN, BK, WM, WN, ST, OCC>}
 
+// the same kernels with partial last tiles along N and K (both multiples of 8)
+#define NT_TAIL_INSTANCE(BM, BN, BK, WM, WN, ST, OCC) \
+    {#BM "x" #BN "x" #BK " waves " #WM "x" #WN " stages " #ST " lds-direct tails", BM, BN, BK, fast_accepts<BM, BN, BK, ST, true>, fast_launch<BM, BN, BK, WM, WN, ST, OCC, 0, 1, 0, true>}
+
 const GemmInstance kInstances[] = {
     {"128x128x32 waves 2x2 any-stride", kGenBM, kGenBN, kGenBK, generic_accepts, generic_launch},
     NT_FAST_INSTANCE(256, 256, 32, 2, 4, 5, 2),  // 5 x 32 KiB: the whole LDS of a CU
@@ -187,6 +192,10 @@ const GemmInstance kInstances[] = {
     NT_FAST_INSTANCE(128, 128, 64, 2, 2, 2, 2),
     NT_FAST_INSTANCE(64, 64, 64, 2, 2, 4, 2),  // small problems: more, smaller tiles to occupy the CUs
     NT_FAST_INSTANCE(128, 256, 32, 1, 4, 3, 2),  // two workgroups per CU: mid-size problems
+    NT_TAIL_INSTANCE(256, 256, 32, 2, 4, 5, 2),
+    NT_TAIL_INSTANCE(128, 256, 32, 1, 4, 3, 2),
+    NT_TAIL_INSTANCE(128, 128, 64, 2, 2, 2, 2),
+    NT_TAIL_INSTANCE(64, 64, 64, 2, 2, 4, 2),
 #ifdef NT_GEMM_ABLATION
 #define NT_LOAD_INSTANCE(BM, BN, BK, WM, WN, ST, OCC, LD, AUX) \
     {#BM "x" #BN "x" #BK " waves " #WM "x" #WN " stages " #ST " load " #LD " aux " #AUX, BM, BN, BK, fast_accepts<BM, BN, BK, ST>, fast_launch<BM, BN, BK, WM, WN, ST, OCC, 0, LD, AUX>}
@@ -255,11 +264,12 @@ int heuristic_choice(const GemmProblem &q, int bm, int bn, int bk) {
     // untuned preference (measured on square problems): 256x256 tiles from 256 tiles up,
     // 128x256 from 128 tiles up, 128x128 from 256 tiles up, else the smallest tile that divides
     struct Rule { int instance; int64_t min_tiles; };
-    const Rule rules[] = {{1, 256}, {2, 256}, {5, 128}, {3, 256}, {4, 1}, {3, 1}, {5, 1}, {2, 1}, {1, 1}};
+    // (instances 6..9 are 1, 5, 3, 4 with tails: they accept what those accept, so they come after them)
+    const Rule rules[] = {{1, 256}, {2, 256}, {5, 128}, {3, 256}, {4, 1}, {3, 1}, {5, 1}, {2, 1}, {1, 1}, {6, 256}, {7, 128}, {8, 256}, {9, 1}, {8, 1}, {7, 1}, {6, 1}};
     for (const Rule &rule : rules) {
         const GemmInstance &inst = kInstances[rule.instance];
         if (!inst.accepts(q)) continue;
-        const int64_t tiles = (int64_t)((q.m + inst.bm - 1) / inst.bm) * (q.n / inst.bn);
+        const int64_t tiles = (int64_t)((q.m + inst.bm - 1) / inst.bm) * ((q.n + inst.bn - 1) / inst.bn);
         if (tiles >= rule.min_tiles) return rule.instance;
     }
     return kInstances[0].accepts(q) ? 0 : -1;

@@ -97,7 +97,7 @@ NT_DEVICE void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" 
 // kAblate is a measurement aid (bit 0: no global loads inside the K loop,
 // bit 1: operand fragments read from LDS only once); 0 in every shipped instance.
 template <typename T, int BM, int BN, int BK, int WM, int WN, int kStages, int kWavesPerSimd, bool kAddmm, int kAblate = 0, int kLoad = 0, int kAux = 0,
-          bool kFloatOut = false, bool kBT = false>
+          bool kFloatOut = false, bool kBT = false, bool kTail = false>
 __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kernel(GemmParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only builtins; the host pass only needs the stub
     typedef Elem<T> E;
@@ -116,6 +116,12 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     constexpr int kBRowsPerInstr = 64 / kBChunksPerRow > 0 ? 64 / kBChunksPerRow : 1;
     constexpr int kBInstr = kStageB / (kWaves * 1024);
     constexpr int kLoadsPerTile = kAInstr + kBInstr;
+    // kTail: N and K need not fit the tile (multiples of 8 elements, so that 16-byte chunks stay whole).
+    // Columns of B past N feed only columns of C that are not stored; the k positions past K of the last
+    // tile must read as zeros in both operands (a stray Inf times a zero would be a NaN): rows of a
+    // row-major B past K lie behind the end of its descriptor, and lanes whose chunk of a k-contiguous
+    // row (A, transposed B) starts past K get an offset behind the end of theirs.
+    static_assert(!kTail || kLoad == 1, "tails rely on the range check of buffer loads");
     static_assert(kStageA % (kWaves * 1024) == 0 && kStageB % (kWaves * 1024) == 0, "tile/wave mismatch");
     static_assert(kBChunksPerRow <= 64, "BN too large for one-instruction rows");
     static_assert(kWaveM % 32 == 0 && kWaveN % 32 == 0 && BK % 16 == 0, "wave tile");
@@ -205,14 +211,42 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         const int64_t a_rows = min((int64_t)BM, (int64_t)p.m - m0);
         const unsigned a_bytes = (unsigned)(((a_rows - 1) * p.lda + p.k) * 2);
         a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)a_base, 0, a_bytes, 0x00020000);
-        b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)b_base, 0, 0xffffffff, 0x00020000);
+        unsigned b_bytes = 0xffffffff;
+        if constexpr (kTail) {
+            const int64_t b_cols = (int64_t)p.n - n0;  // > 0
+            b_bytes = kBT ? (unsigned)(((min((int64_t)BN, b_cols) - 1) * p.ldb + p.k) * 2) : (unsigned)((((int64_t)p.k - 1) * p.ldb + b_cols) * 2);
+        }
+        b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)b_base, 0, b_bytes, 0x00020000);
     }
+    const int num_k = kTail ? (p.k + BK - 1) / BK : p.k / BK;
+    const int last_k = num_k - 1;
+    // 16-byte chunks of the last k tile that lie inside K (all of them without a tail)
+    const int tail_chunks = kTail ? (p.k - last_k * BK) / 8 : kAChunksPerRow;
     auto issue_loads = [&](auto stage_tag, int kt) {
         NT_LDS unsigned char *sa = stage_a(stage_tag);
         NT_LDS unsigned char *sb = stage_b(stage_tag);
         if constexpr (kLoad == 1) {
             const int a_k = kt * BK * 2;
             const int b_k = kBT ? a_k : kt * BK * (int)p.ldb * 2;
+            if (kTail && kt == last_k && tail_chunks < kAChunksPerRow) {  // uniform: the partial last k tile
+                constexpr unsigned kBehind = 0x7fffffffu;  // behind every descriptor (their sizes stay below 2^31)
+#pragma unroll
+                for (int j = 0; j < kAInstr; ++j) {
+                    const int row = (j * kWaves + wave) * kARowsPerInstr + lane / kAChunksPerRow;
+                    const bool inside = a_phys_chunk<BK>(row, lane % kAChunksPerRow) < tail_chunks;
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, sa + (j * kWaves + wave) * 1024, 16, inside ? a_src[j] : kBehind, a_k, 0, kAux);
+                }
+#pragma unroll
+                for (int j = 0; j < kBInstr; ++j) {
+                    bool inside = true;
+                    if constexpr (kBT) {
+                        const int row = (j * kWaves + wave) * kARowsPerInstr + lane / kAChunksPerRow;
+                        inside = a_phys_chunk<BK>(row, lane % kAChunksPerRow) < tail_chunks;
+                    }
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, sb + (j * kWaves + wave) * 1024, 16, inside ? b_src[j] : kBehind, b_k, 0, kAux);
+                }
+                return;
+            }
 #pragma unroll
             for (int j = 0; j < kAInstr; ++j)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, sa + (j * kWaves + wave) * 1024, 16, a_src[j], a_k, 0, kAux);
@@ -327,8 +361,6 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     // tile t+kStages-1, multiply tile t.  Past the end the last tile is fetched
     // again into a stage nobody reads, which keeps the outstanding-load count
     // the same in every step.
-    const int num_k = p.k / BK;
-    const int last_k = num_k - 1;
     const int main_k = num_k - num_k % kStages;
 
     static_for<0, kStages - 1>([&](auto s) { issue_loads(s, min((int)decltype(s)::value, last_k)); });
@@ -380,6 +412,7 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
 #pragma unroll
                     for (int e = 0; e < 4; ++e) v[e] = acc[ti][tj][4 * r4 + e];
                     const int gcol = n0 + wave_n * kWaveN + tj * 32 + 8 * r4 + 4 * g;
+                    if (kTail && gcol >= p.n) continue;  // a partial last tile of columns
                     *(float4_t *)(C32 + (int64_t)grow * p.ldc + gcol) = v;
                 }
         }
@@ -437,6 +470,7 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
             const int grow = m0 + wave_m * kWaveM + ti * 32 + row;
             const int gcol = n0 + wave_n * kWaveN + chunk * 8;
             if (grow >= p.m) continue;  // a partial last tile of rows
+            if (kTail && gcol >= p.n) continue;  // ... of columns (whole chunks: N is a multiple of 8)
             if constexpr (kAddmm) {
                 // the matmul result was rounded to the element type; beta, alpha
                 // are fp32 scalars, so the combination happens in fp32

@@ -585,3 +585,55 @@ def test_gemm_any_number_of_rows_on_the_direct_to_lds_path(m, addmm):
         assert bool((guard[m:] == 7.0).all()), name
         ran += 1
     assert ran >= 4
+
+
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
+@pytest.mark.parametrize("m, n, k", ((300, 200, 104), (1000, 1000, 1000), (257, 264, 72), (512, 520, 8), (2100, 3000, 2056)))
+def test_gemm_partial_tiles_along_n_and_k(m, n, k, dtype):
+    """N and K that do not fit the tile (multiples of 8) stay on the direct-to-LDS kernels: the
+    instances with tails, row-major and transposed rhs, element-type / fp32 / addmm epilogues.
+    Whole output, NaN-poisoned, inside a wider buffer whose extra columns must stay untouched.
+    What lies next to the operands in memory is Inf: the element after a row's end (the next
+    row's first), rows of the rhs past K -- none of it may reach the result."""
+    from ninetoothed_amd import runtime
+
+    lib = runtime.library()
+    names = runtime.gemm_config_names()
+    tag = runtime.DATA_TYPE_INDEX["fp16" if dtype == torch.float16 else "bf16"]
+    null = runtime.ArgumentTensor.null()
+    beta, alpha = runtime.ArgumentTensor.from_scalar(0.5), runtime.ArgumentTensor.from_scalar(2.0)
+    tolerance = dict(rtol=2e-2, atol=2e-2 * max(k / 512, 1) ** 0.5) if dtype == torch.bfloat16 else dict(rtol=1e-2, atol=1e-2 * max(k / 512, 1) ** 0.5)
+    a = torch.randn(m, k, dtype=dtype, device="cuda")
+    a[1, 0] = float("inf")  # follows row 0 in memory: only row 1 of the result may see it
+    tall = torch.randn(k + 8, n, dtype=dtype, device="cuda")
+    tall[k:] = float("inf")
+    wide = torch.randn(n, k, dtype=dtype, device="cuda")
+    wide[1, 0] = float("inf")  # transposed rhs: follows column 0's k range, belongs to column 1
+    bias = torch.randn(m, n, dtype=dtype, device="cuda")
+    for b, clean_rows, clean_cols in ((tall[:k], [r for r in range(m) if r != 1], slice(None)), (wide.t(), [r for r in range(m) if r != 1], [c for c in range(n) if c != 1])):
+        product = (a.float() @ b.float())[clean_rows][:, clean_cols]
+        assert bool(torch.isfinite(product).all())
+        for out_dtype, with_bias in ((dtype, False), (torch.float32, False), (dtype, True)):
+            buffer = torch.full((m, n + 24), 7.0, dtype=out_dtype, device="cuda")
+            out = buffer[:, :n]
+            tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (bias, a, b, out)]
+            expected = 0.5 * bias.float()[clean_rows][:, clean_cols] + 2.0 * product.to(dtype).float() if with_bias else product
+            out_tag = runtime.DATA_TYPE_INDEX["fp32"] if out_dtype == torch.float32 else tag
+            served = 0
+            for instance, name in enumerate(names):
+                if "tails" not in name:
+                    continue
+                out.fill_(float("nan"))
+                result = lib.launch_nt_gemm_config(
+                    runtime.current_stream(), instance, tensors[0] if with_bias else null, tensors[1], tensors[2], beta if with_bias else null,
+                    alpha if with_bias else null, tensors[3], tag, out_tag,
+                )
+                assert result == 0, name
+                served += 1
+                assert torch.allclose(out.float()[clean_rows][:, clean_cols], expected, **tolerance), (name, out_dtype, with_bias)
+                assert bool((buffer[:, n:] == 7.0).all()), name
+            assert served >= 3
+        # through `make`: the heuristic picks an instance with tails instead of the any-stride kernel
+        out = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+        _matmul_kernel()(a, b, out)
+        assert torch.allclose(out.float()[clean_rows][:, clean_cols], product, **tolerance)
