@@ -156,7 +156,7 @@ NineToothedResult launch_nt_attention(NineToothedStream stream,
  * dilation 1 and zero padding (padding_h, padding_w), computed as the implicit
  * GEMM [N*P*Q, C*R*S] x [C*R*S, K] the arrangement of
  * tests/test_conv2d.py:13-48 describes.
- * When C % 32 == 0, K % 256 == 0, (P*Q) % 8 == 0, the output is contiguous and
+ * When C % 32 == 0, K % 64 == 0, the output is contiguous and
  * N*P*Q >= 1024, the call first repacks the input to channels-last and the
  * filter to [R*S*C, K] in the library's scratch buffers of `stream`
  * (N*C*H*W + K*C*R*S elements), then runs the direct-to-LDS main loop;

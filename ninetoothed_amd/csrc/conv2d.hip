@@ -12,16 +12,21 @@
 // asynchronous, and allocates only when a call needs more than any before it):
 //   x[N,C,H,W]  -> xt[N,H,W,C]              (tiled transpose through LDS, 16-byte accesses)
 //   w[K,C,R,S]  -> wt[(r*S+s)*C + c, K]     (row-major K x N operand of the GEMM)
-// The main kernel then is the 256x256x32, 4-stage GEMM: a K step is 32 channels of
+// The main kernel then is the direct-to-LDS GEMM loop (256x256x32 tiles for wide layers,
+// 256x128 and 128x64 for layers with fewer output channels): a K step is 32 channels of
 // one filter tap (r, s); the A rows of a step are 64-byte runs of xt whose
 // addresses differ from step to step by a uniform offset; taps that fall into
 // the padding are fetched with an out-of-range buffer offset, which the
-// hardware returns as zeros.  The epilogue writes NCHW: per output channel the
-// GEMM rows of a tile are contiguous, so the accumulators go through an LDS slab
-// laid out [channel][row] and leave as 16-byte stores.
+// hardware returns as zeros.  GEMM rows run over all images (a tile may span
+// several small ones).  The epilogue writes NCHW: per output channel the
+// GEMM rows of an image are contiguous, so the accumulators go through an LDS slab
+// laid out [channel][row] and leave as 16-byte stores when P*Q is a multiple of 8
+// (8 consecutive rows then lie in one image, aligned), element by element otherwise.
 //
 // Requirements of this path (anything else uses the any-stride gather kernel):
-// fp16/bf16, C % 32 == 0, K_out % 256 == 0, (P*Q) % 8 == 0, contiguous output.
+// fp16/bf16, C % 32 == 0, K_out % 64 == 0, contiguous output.
+#include <algorithm>
+
 #include "conv2d.h"
 #include "gemm_fast.h"
 #include "workspace.h"
@@ -34,19 +39,21 @@ struct ConvParams {
     const void *wt;
     void *y;
     int N, C, H, W, K, R, S, P, Q, pad_h, pad_w;
-    int tiles_per_image, tiles_m, tiles_n;
+    int M, tiles_m, tiles_n;  // M = N*P*Q rows
     unsigned xt_bytes;
 };
 
 // ---- pre-pass: one launch, two jobs ----
-// grid layer  z == 0: w[K,C,R,S] (any strides) -> wt[(r*S+s)*C + c][K], grid-stride over the layer's threads
-//                     (first, so that its scattered reads overlap the streaming layers behind it)
-// grid layers z >= 1: x[z-1] NCHW (any strides) -> xt[z-1] NHWC contiguous (64 x 64 tiles through LDS)
+// grid layers z <  f.layers: w[K,C,R,S] (any strides) -> wt[(r*S+s)*C + c][K], grid-stride over these layers' threads
+//                     (first, so that its scattered reads overlap the streaming layers behind it; as many
+//                     layers as give the filter a few hundred workgroups, whatever the image size)
+// grid layers z >= f.layers: x[z - f.layers] NCHW (any strides) -> xt NHWC contiguous (64 x 64 tiles through LDS)
 struct FilterRepack {
     const void *w;
     void *wt;
     int K, C, R, S;
     int64_t s_k, s_c, s_r, s_s;
+    int layers;
 };
 
 template <typename T>
@@ -56,12 +63,12 @@ __global__ __launch_bounds__(256) void conv2d_repack_kernel(const T *x, T *xt, i
     constexpr int kPitch = 64 + 8;  // halfs; keeps 16-byte alignment of rows
     __shared__ __attribute__((aligned(16))) T tile[64 * kPitch];
     const int t = threadIdx.x;
-    if (blockIdx.z == 0) {
+    if ((int)blockIdx.z < f.layers) {
         const T *w = (const T *)f.w;
         T *wt = (T *)f.wt;
         const int64_t total = (int64_t)f.K * f.C * f.R * f.S;
-        const int64_t layer_threads = (int64_t)gridDim.x * gridDim.y * 256;
-        for (int64_t index = ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * 256 + t; index < total; index += layer_threads) {
+        const int64_t layer_threads = (int64_t)gridDim.x * gridDim.y * 256 * f.layers;
+        for (int64_t index = (((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 256 + t; index < total; index += layer_threads) {
             const int k = (int)(index % f.K);
             const int64_t row = index / f.K;
             const int c = (int)(row % f.C);
@@ -70,7 +77,7 @@ __global__ __launch_bounds__(256) void conv2d_repack_kernel(const T *x, T *xt, i
         }
         return;
     }
-    const int hw0 = blockIdx.x * 64, c0 = blockIdx.y * 64, n = blockIdx.z - 1;
+    const int hw0 = blockIdx.x * 64, c0 = blockIdx.y * 64, n = blockIdx.z - f.layers;
     const T *src = x + (int64_t)n * s_n;
     // load: rows = channels, 8 consecutive positions per thread
 #pragma unroll
@@ -105,12 +112,12 @@ __global__ __launch_bounds__(256) void conv2d_repack_kernel(const T *x, T *xt, i
 }
 
 // ---- main kernel ----
-template <typename T>
-__global__ __launch_bounds__(512, 2) void conv2d_nhwc_kernel(ConvParams p) {
+template <typename T, int BM, int BN, int WM, int WN, int kStages, int kOcc>
+__global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     typedef Elem<T> E;
     typedef typename E::vec8 vec8;
-    constexpr int BM = 256, BN = 256, BK = 32, WM = 2, WN = 4, kStages = 4;
+    constexpr int BK = 32;
     constexpr int kWaves = WM * WN;
     constexpr int kWaveM = BM / WM, kWaveN = BN / WN;
     constexpr int TM = kWaveM / 32, TN = kWaveN / 32;
@@ -120,15 +127,18 @@ __global__ __launch_bounds__(512, 2) void conv2d_nhwc_kernel(ConvParams p) {
     constexpr int kBChunksPerRow = BN / 8, kBRowsPerInstr = 64 / kBChunksPerRow;
     constexpr int kBInstr = kStageB / (kWaves * 1024);
     constexpr int kLoadsPerTile = kAInstr + kBInstr;
+    static_assert(kStageA % (kWaves * 1024) == 0 && kStageB % (kWaves * 1024) == 0, "every wave issues whole load instructions");
+    static_assert(kWaveM % 32 == 0 && kWaveN % 32 == 0, "wave tile");
+    static_assert(kStages >= 3 && kStages <= 4 && kStages >= WN, "stages (the epilogue slabs of all waves live in the A stages)");
 
     __shared__ __attribute__((aligned(1024))) unsigned char lds_a0[kStageA];
     __shared__ __attribute__((aligned(1024))) unsigned char lds_a1[kStageA];
     __shared__ __attribute__((aligned(1024))) unsigned char lds_a2[kStageA];
-    __shared__ __attribute__((aligned(1024))) unsigned char lds_a3[kStageA];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_a3[kStages > 3 ? kStageA : 16];
     __shared__ __attribute__((aligned(1024))) unsigned char lds_b0[kStageB];
     __shared__ __attribute__((aligned(1024))) unsigned char lds_b1[kStageB];
     __shared__ __attribute__((aligned(1024))) unsigned char lds_b2[kStageB];
-    __shared__ __attribute__((aligned(1024))) unsigned char lds_b3[kStageB];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_b3[kStages > 3 ? kStageB : 16];
     auto stage_a = [&](auto tag) -> NT_LDS unsigned char * {
         constexpr int i = decltype(tag)::value;
         if constexpr (i == 0) return (NT_LDS unsigned char *)lds_a0;
@@ -151,8 +161,7 @@ __global__ __launch_bounds__(512, 2) void conv2d_nhwc_kernel(ConvParams p) {
 
     int tile_m, tile_n;
     map_tile(p.tiles_m, p.tiles_n, 0, tile_m, tile_n);
-    const int image = tile_m / p.tiles_per_image;
-    const int pq0 = (tile_m % p.tiles_per_image) * BM;
+    const int m0 = tile_m * BM;
     const int n0 = tile_n * BN;
     const int PQ = p.P * p.Q;
 
@@ -164,11 +173,12 @@ __global__ __launch_bounds__(512, 2) void conv2d_nhwc_kernel(ConvParams p) {
     for (int j = 0; j < kAInstr; ++j) {
         const int row = (j * kWaves + wave) * kARowsPerInstr + lane / kAChunksPerRow;
         const int chunk = a_phys_chunk<BK>(row, lane % kAChunksPerRow);
-        const int pq = pq0 + row;
+        const int m = m0 + row;
+        const int image = m / PQ, pq = m - image * PQ;
         const int oy = pq / p.Q, ox = pq - oy * p.Q;
-        a_y[j] = pq < PQ ? oy - p.pad_h : -(1 << 20);  // rows past the image never pass the bounds test
+        a_y[j] = m < p.M ? oy - p.pad_h : -(1 << 20);  // rows past the last image never pass the bounds test
         a_x[j] = ox - p.pad_w;
-        a_base[j] = pq < PQ ? (((image * p.H + a_y[j]) * p.W + a_x[j]) * p.C + chunk * 8) * 2 : 0;
+        a_base[j] = m < p.M ? (((image * p.H + a_y[j]) * p.W + a_x[j]) * p.C + chunk * 8) * 2 : 0;
     }
     unsigned b_src[kBInstr];
 #pragma unroll
@@ -271,20 +281,22 @@ __global__ __launch_bounds__(512, 2) void conv2d_nhwc_kernel(ConvParams p) {
     lds_barrier();
 
     // ---- epilogue: lane holds, per 32x32 tile, output channel l32 and rows 8*(r/4) + 4*g + r%4 ----
-    // slab layout [32 channels][kWaveM rows], 16-byte chunks swizzled by channel; two slabs per stage array
-    constexpr int kRowBytes = kWaveM * 2;  // 256
+    // slab layout [32 channels][kWaveM rows], 16-byte chunks swizzled by channel; an A stage holds WM slabs
+    constexpr int kRowBytes = kWaveM * 2;
     constexpr int kSlabBytes = 32 * kRowBytes;
-    constexpr int kChunks = kWaveM / 8;    // 16
+    constexpr int kChunks = kWaveM / 8;
+    static_assert(kStageA == WM * kSlabBytes, "slabs per A stage");
     NT_LDS unsigned char *slab;
     {
-        const int which = wave >> 1;
+        const int which = wave / WM;
         slab = which == 0 ? (NT_LDS unsigned char *)lds_a0
-               : which == 1 ? (NT_LDS unsigned char *)lds_b0
-               : which == 2 ? (NT_LDS unsigned char *)lds_a1
-                            : (NT_LDS unsigned char *)lds_b1;
-        slab += (wave & 1) * kSlabBytes;
+               : which == 1 ? (NT_LDS unsigned char *)lds_a1
+               : which == 2 ? (NT_LDS unsigned char *)lds_a2
+                            : (NT_LDS unsigned char *)lds_a3;
+        slab += (wave % WM) * kSlabBytes;
     }
-    T *Y = (T *)p.y + (int64_t)image * p.K * PQ;
+    T *Y = (T *)p.y;
+    const bool whole_chunks = PQ % 8 == 0;
 #pragma unroll
     for (int tj = 0; tj < TN; ++tj) {
 #pragma unroll
@@ -305,9 +317,22 @@ __global__ __launch_bounds__(512, 2) void conv2d_nhwc_kernel(ConvParams p) {
             const int phys = idx % kChunks;
             const int chunk = phys ^ (channel & (kChunks - 1));
             vec8 v = *(const NT_LDS vec8 *)(slab + channel * kRowBytes + phys * 16);
-            const int pq = pq0 + wave_m * kWaveM + chunk * 8;
+            const int m = m0 + wave_m * kWaveM + chunk * 8;
+            if (m >= p.M) continue;
             const int out_channel = n0 + wave_n * kWaveN + tj * 32 + channel;
-            if (pq < PQ) *(vec8 *)(Y + (int64_t)out_channel * PQ + pq) = v;  // PQ % 8 == 0: chunks are all-in or all-out
+            int image = m / PQ, pq = m - image * PQ;
+            if (whole_chunks) {  // the 8 rows lie in one image and start at a multiple of 8
+                *(vec8 *)(Y + ((int64_t)image * p.K + out_channel) * PQ + pq) = v;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    if (m + e < p.M) Y[((int64_t)image * p.K + out_channel) * PQ + pq] = v[e];
+                    if (++pq == PQ) {
+                        pq = 0;
+                        ++image;
+                    }
+                }
+            }
         }
     }
 #endif
@@ -328,7 +353,11 @@ int run_fast(const Conv2dRequest &q, hipStream_t stream) {
     f.wt = wt;
     f.K = q.K; f.C = q.C; f.R = q.R; f.S = q.S;
     f.s_k = q.ws[0]; f.s_c = q.ws[1]; f.s_r = q.ws[2]; f.s_s = q.ws[3];
-    conv2d_repack_kernel<T><<<dim3(ceil_div(HW, 64), ceil_div(q.C, 64), q.N + 1), dim3(256), 0, stream>>>(
+    // about 512 workgroups for the filter, or one thread per element if that is less
+    const int64_t per_layer = (int64_t)ceil_div(HW, 64) * ceil_div(q.C, 64);
+    const int64_t wanted = std::min<int64_t>(512, ceil_div((int64_t)q.K * q.C * q.R * q.S, (int64_t)256));
+    f.layers = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(wanted, per_layer), 512));
+    conv2d_repack_kernel<T><<<dim3(ceil_div(HW, 64), ceil_div(q.C, 64), q.N + f.layers), dim3(256), 0, stream>>>(
         (const T *)q.x, (T *)xt, q.C, HW, q.W, q.xs[0], q.xs[1], q.xs[2], q.xs[3], vector_ok, f);
     ConvParams p;
     p.xt = xt;
@@ -336,11 +365,19 @@ int run_fast(const Conv2dRequest &q, hipStream_t stream) {
     p.y = q.y;
     p.N = q.N; p.C = q.C; p.H = q.H; p.W = q.W; p.K = q.K; p.R = q.R; p.S = q.S; p.P = q.P; p.Q = q.Q;
     p.pad_h = q.pad_h; p.pad_w = q.pad_w;
-    p.tiles_per_image = ceil_div(q.P * q.Q, 256);
-    p.tiles_m = q.N * p.tiles_per_image;
-    p.tiles_n = q.K / 256;
+    p.M = q.N * q.P * q.Q;
     p.xt_bytes = (unsigned)xt_bytes;
-    conv2d_nhwc_kernel<T><<<dim3(p.tiles_m * p.tiles_n), dim3(512), 0, stream>>>(p);
+    // tile by the number of output channels: 256 wide when they fill it and there are enough tiles for the
+    // chip, else 128 (two workgroups per CU), else 128 x 64 tiles of four waves
+    const auto launch = [&](auto kernel, int bm, int bn, int threads) {
+        p.tiles_m = ceil_div(p.M, bm);
+        p.tiles_n = q.K / bn;
+        kernel<<<dim3(p.tiles_m * p.tiles_n), dim3(threads), 0, stream>>>(p);
+    };
+    const int64_t tiles_256 = (int64_t)ceil_div(p.M, 256) * (q.K / 256);
+    if (q.K % 256 == 0 && tiles_256 >= 192) launch(conv2d_nhwc_kernel<T, 256, 256, 2, 4, 4, 2>, 256, 256, 512);
+    else if (q.K % 128 == 0 && (int64_t)ceil_div(p.M, 256) * (q.K / 128) >= 192) launch(conv2d_nhwc_kernel<T, 256, 128, 4, 2, 3, 4>, 256, 128, 512);
+    else launch(conv2d_nhwc_kernel<T, 128, 64, 2, 2, 4, 3>, 128, 64, 256);
     return (int)hipGetLastError();
 }
 
@@ -348,14 +385,14 @@ int run_fast(const Conv2dRequest &q, hipStream_t stream) {
 
 int conv2d_fast(const Conv2dRequest &q, hipStream_t stream) {
     if (q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) return NINETOOTHED_NO_KERNEL;
-    if (q.C % 32 || q.K % 256 || (q.P * q.Q) % 8) return NINETOOTHED_NO_KERNEL;
+    if (q.C % 32 || q.K % 64) return NINETOOTHED_NO_KERNEL;
     if (q.ys[3] != 1 || q.ys[2] != q.Q || q.ys[1] != (int64_t)q.P * q.Q || q.ys[0] != (int64_t)q.K * q.P * q.Q) return NINETOOTHED_NO_KERNEL;
     if (((uintptr_t)q.y & 15) != 0) return NINETOOTHED_NO_KERNEL;
     const int64_t xt_bytes = (int64_t)q.N * q.H * q.W * q.C * 2;
     const int64_t wt_bytes = (int64_t)q.K * q.C * q.R * q.S * 2;
     if (xt_bytes >= (int64_t(1) << 31) || wt_bytes >= (int64_t(1) << 31)) return NINETOOTHED_NO_KERNEL;  // 32-bit buffer offsets
-    if ((int64_t)q.N * ceil_div(q.P * q.Q, 256) * (q.K / 256) > 0x7fffffffll) return NINETOOTHED_NO_KERNEL;
-    if (q.N >= 65535 || ceil_div(q.C, 64) > 65535) return NINETOOTHED_NO_KERNEL;  // grid of the repacking pass: (positions, channels, images + 1)
+    if ((int64_t)q.N * q.P * q.Q > 0x7fffffffll || (int64_t)ceil_div(q.N * q.P * q.Q, 128) * (q.K / 64) > 0x7fffffffll) return NINETOOTHED_NO_KERNEL;
+    if (q.N >= 65535 - 512 || ceil_div(q.C, 64) > 65535) return NINETOOTHED_NO_KERNEL;  // grid of the repacking pass: (positions, channels, filter layers + images)
     // enough work to amortise the repacking pass
     if ((int64_t)q.N * q.P * q.Q < 1024) return NINETOOTHED_NO_KERNEL;
     return q.dtype == NINETOOTHED_FLOAT16 ? run_fast<half_t>(q, stream) : run_fast<bf16_t>(q, stream);

@@ -435,6 +435,40 @@ def test_conv2d_baseline_shape_and_1x1():
     assert torch.allclose(out.float(), as_matmul, **HALF_TOL)
 
 
+@pytest.mark.parametrize(
+    "n, c, h, w, k, r, s, padding",
+    (
+        (4, 64, 56, 56, 64, 3, 3, (1, 1)),     # 64 output channels: 128 x 64 tiles
+        (4, 128, 28, 28, 128, 3, 3, (1, 1)),
+        (8, 256, 14, 14, 256, 3, 3, (1, 1)),   # 196 positions per image: tiles span images, P*Q % 8 != 0
+        (8, 512, 7, 7, 512, 3, 3, (1, 1)),     # 49 positions per image
+        (5, 64, 56, 56, 256, 1, 1, (0, 0)),
+        (16, 256, 28, 28, 128, 3, 3, (1, 1)),  # 256 x 128 tiles
+        (2, 320, 16, 16, 320, 3, 3, (1, 1)),
+        (3, 32, 9, 11, 192, 3, 2, (1, 0)),     # odd sizes all round
+        (40, 96, 7, 5, 64, 2, 3, (0, 2)),
+    ),
+)
+def test_conv2d_layer_shapes_on_the_direct_to_lds_path(n, c, h, w, k, r, s, padding):
+    """Layers other than the baseline's stay on the implicit-GEMM kernel: fewer output channels
+    (narrower tiles), small images (GEMM rows run across images, stores element by element when
+    P*Q is not a multiple of 8).  Whole NaN-poisoned output against an fp32 convolution of the
+    same rounded operands (MIOpen's own half kernels deviate by more than the tolerance)."""
+    dtype = torch.float16  # the program rounds its product to float16 (tests/test_conv2d.py:44-48)
+    x = (torch.randn(n, c, h, w, device="cuda") * 0.5).to(dtype)
+    weight = (torch.randn(k, c, r, s, device="cuda") * 0.1).to(dtype)
+    p_out, q_out = h + 2 * padding[0] - r + 1, w + 2 * padding[1] - s + 1
+    guard = torch.full((n * k * p_out * q_out + 64,), 7.0, dtype=dtype, device="cuda")
+    out = guard[: n * k * p_out * q_out].view(n, k, p_out, q_out)
+    out.fill_(float("nan"))
+    kernel = ninetoothed.make(programs.conv2d.arrangement, programs.conv2d.application, programs.conv2d.tensors())
+    kernel(x, weight, out, padding_h=padding[0], padding_w=padding[1])
+    assert "implicit" in kernel.last_plan or "gemm" in kernel.last_plan
+    expected = F.conv2d(x.float(), weight.float(), padding=padding)
+    assert torch.allclose(out.float(), expected, rtol=1e-2, atol=1e-2)
+    assert bool((guard[n * k * p_out * q_out :] == 7.0).all())
+
+
 def test_scratch_buffers_are_reused_grown_and_released():
     """conv2d's repacked operands and fp32 attention's narrowed K / V live in buffers the library
     keeps per stream: a smaller call after a larger one, a larger one after that, another stream and
