@@ -141,7 +141,11 @@ NineToothedResult launch_nt_softmax_config(NineToothedStream stream, int config,
  * loop; without hints non-causal calls run the software-pipelined 64-key loop
  * (with 256 query rows and eight waves per workgroup when that still fills the
  * chip twice) and causal calls the plain one.  K and V of one (batch, head) must span
- * less than 4 GiB. */
+ * less than 4 GiB.
+ * head_dim: 32, 64, 128 and 256 have kernels of their size; any other multiple of
+ * 8 up to 256 runs on the next of these sizes with the missing columns read as
+ * zeros (K and V of one (batch, head) then span less than 2 GiB); anything else
+ * returns NINETOOTHED_NO_KERNEL. */
 NineToothedResult launch_nt_attention(NineToothedStream stream,
                                       NineToothedTensor q,
                                       NineToothedTensor k,

@@ -17,6 +17,8 @@
 // difference to the running row maximum.
 #include <type_traits>
 
+#include <algorithm>
+
 #include "gemm_fast.h"  // swizzle helpers, static_for, lds_barrier
 #include "workspace.h"
 
@@ -31,6 +33,7 @@ struct AttentionParams {
     float q_scale;  // scale * log2(e)
     int causal;
     int q_blocks;
+    int head_dim;  // elements per row in memory (a multiple of 8; the kernel's D when it is not padded)
 };
 
 constexpr int kAttnWaves = 4;
@@ -39,7 +42,9 @@ constexpr int kAttnWaves = 4;
 // kPipelined: overlap the softmax of a block with the MFMAs of its neighbours
 // TIO: element type of Q and O in memory -- T, or float for fp32 tensors (their K and V
 // are converted to T beforehand; Q is converted while it is scaled, O is stored unrounded)
-template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined, typename TIO = T, int kWaves = kAttnWaves>
+// kPadded: the head dimension in memory (p.head_dim, a multiple of 8) is smaller than D: the missing
+// columns of Q, K and V read as zeros (scores and the stored columns are unchanged by them)
+template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined, typename TIO = T, int kWaves = kAttnWaves, bool kPadded = false>
 __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(AttentionParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     typedef Elem<T> E;
@@ -127,7 +132,10 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             vec8 raw;
-            if constexpr (std::is_same<TIO, float>::value) {
+            if (kPadded && ks * 16 + 8 * g >= p.head_dim) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) raw[e] = E::from_float(0.0f);
+            } else if constexpr (std::is_same<TIO, float>::value) {
                 const float4_t lo = *(const float4_t *)(src + ks * 16 + 8 * g);
                 const float4_t hi = *(const float4_t *)(src + ks * 16 + 8 * g + 4);
 #pragma unroll
@@ -155,32 +163,50 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
     // end with the last key row: the per-lane byte offset is fixed for the whole
     // kernel, the block offset travels in a scalar register, and rows past the end
     // of the sequence read as zeros (the range check covers the scalar offset too).
-    const unsigned k_bytes = (unsigned)((p.seq_k - 1) * p.k_strides[2] + D) * 2u;
-    const unsigned v_bytes = (unsigned)((p.seq_k - 1) * p.v_strides[2] + D) * 2u;
+    const int row_elements = kPadded ? p.head_dim : D;
+    const unsigned k_bytes = (unsigned)((p.seq_k - 1) * p.k_strides[2] + row_elements) * 2u;
+    const unsigned v_bytes = (unsigned)((p.seq_k - 1) * p.v_strides[2] + row_elements) * 2u;
     __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)K, 0, k_bytes, 0x00020000);
     __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)V, 0, v_bytes, 0x00020000);
     const unsigned k_block_bytes = (unsigned)(BN * p.k_strides[2]) * 2u;
     const unsigned v_block_bytes = (unsigned)(BN * p.v_strides[2]) * 2u;
-    // load instruction j of a wave covers the rows kLoadRowStep * j further down; both
-    // swizzles repeat with that period, so one lane offset serves every j and the
-    // row step goes into the scalar offset as well
+    // load instruction j of a wave covers the rows kLoadRowStep * j further down; where the
+    // swizzle repeats with that period, one lane offset serves every j and the
+    // row step goes into the scalar offset as well (K rows of 256 elements: one offset per j).
+    // Padded rows: a lane whose 16-byte chunk starts past the row's end gets an offset behind the
+    // descriptor (these stay below 2^31 bytes, checked on the host) and so fetches zeros.
     constexpr int kLoadRowStep = kWaves * kRowsPerInstr;
-    static_assert(a_phys_chunk<D>(kLoadRowStep, 0) == 0 && b_phys_chunk<D>(kLoadRowStep, 0) == 0, "swizzle period");
+    constexpr bool kPeriodicK = a_phys_chunk<D>(kLoadRowStep, 0) == 0;
+    constexpr int kOffsetsK = kPeriodicK ? 1 : kInstr;
+    static_assert(b_phys_chunk<D>(kLoadRowStep, 0) == 0, "swizzle period");
     const unsigned k_step_bytes = (unsigned)(kLoadRowStep * p.k_strides[2]) * 2u;
     const unsigned v_step_bytes = (unsigned)(kLoadRowStep * p.v_strides[2]) * 2u;
-    unsigned ld_k_off, ld_v_off;
+    constexpr unsigned kBehind = 0x80000000u;
+    unsigned ld_k_off[kOffsetsK], ld_v_off;
     {
-        const int row = wave * kRowsPerInstr + lane / kChunksPerRow;
         const int phys = lane % kChunksPerRow;
-        ld_k_off = ((unsigned)row * (unsigned)p.k_strides[2] + a_phys_chunk<D>(row, phys) * 8) * 2u;
-        ld_v_off = ((unsigned)row * (unsigned)p.v_strides[2] + b_phys_chunk<D>(row, phys) * 8) * 2u;
+#pragma unroll
+        for (int j = 0; j < kOffsetsK; ++j) {
+            const int row = (j * kWaves + wave) * kRowsPerInstr + lane / kChunksPerRow;
+            const int chunk = a_phys_chunk<D>(row, phys);
+            ld_k_off[j] = ((unsigned)row * (unsigned)p.k_strides[2] + chunk * 8) * 2u;
+            if (kPadded && chunk * 8 >= p.head_dim) ld_k_off[j] = kBehind;
+        }
+        const int row = wave * kRowsPerInstr + lane / kChunksPerRow;
+        const int chunk = b_phys_chunk<D>(row, phys);
+        ld_v_off = ((unsigned)row * (unsigned)p.v_strides[2] + chunk * 8) * 2u;
+        if (kPadded && chunk * 8 >= p.head_dim) ld_v_off = kBehind;
     }
     auto issue_k = [&](auto stage_tag, int blk) __attribute__((always_inline)) {
         NT_LDS unsigned char *sk = stage_k(stage_tag);
         const unsigned block_off = (unsigned)blk * k_block_bytes;
 #pragma unroll
-        for (int j = 0; j < kInstr; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, sk + (j * kWaves + wave) * 1024, 16, ld_k_off, block_off + j * k_step_bytes, 0, 0);
+        for (int j = 0; j < kInstr; ++j) {
+            if constexpr (kPeriodicK)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, sk + (j * kWaves + wave) * 1024, 16, ld_k_off[0], block_off + j * k_step_bytes, 0, 0);
+            else
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, sk + (j * kWaves + wave) * 1024, 16, ld_k_off[j], block_off, 0, 0);
+        }
     };
     auto issue_v = [&](auto stage_tag, int blk) __attribute__((always_inline)) {
         NT_LDS unsigned char *sv = stage_v(stage_tag);
@@ -507,6 +533,7 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
                         if constexpr (std::is_same<TIO, float>::value) out[e] = value;
                         else out[e] = E::from_float(value);
                     }
+                    if (kPadded && dt * 32 + 8 * r4 + 4 * g >= p.head_dim) continue;
                     *(vec4 *)(dst + dt * 32 + 8 * r4 + 4 * g) = out;
                 }
         }
@@ -514,14 +541,29 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
 #endif
 }
 
-template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined, typename TIO = T, int kWaves = kAttnWaves>
+template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined, typename TIO = T, int kWaves = kAttnWaves, bool kPadded = false>
 hipError_t launch_attention(AttentionParams &p, hipStream_t stream) {
     constexpr int BM = kWaves * 32 * kQTiles;
     p.q_blocks = ceil_div(p.seq_q, BM);
     const int64_t grid = (int64_t)p.batch * p.heads * p.q_blocks;
     if (grid == 0) return hipSuccess;
-    attention_fwd_kernel<T, D, kQTiles, BN, kOcc, kPipelined, TIO, kWaves><<<dim3((unsigned)grid), dim3(kWaves * 64), 0, stream>>>(p);
+    attention_fwd_kernel<T, D, kQTiles, BN, kOcc, kPipelined, TIO, kWaves, kPadded><<<dim3((unsigned)grid), dim3(kWaves * 64), 0, stream>>>(p);
     return hipGetLastError();
+}
+
+// Head dimensions other than 32, 64 and 128: 256 as it is (one workgroup of four waves per CU: its
+// accumulators and Q fragments take most of the register file), other multiples of 8 on the next of
+// these sizes with the missing columns read as zeros.
+template <typename T, typename TIO>
+int launch_other_head_dim(AttentionParams &p, int head_dim, hipStream_t stream) {
+    if (head_dim <= 0 || head_dim > 256 || head_dim % 8) return NINETOOTHED_NO_KERNEL;
+    if (head_dim == 256) return (int)launch_attention<T, 256, 1, 64, 1, false, TIO>(p, stream);
+    // padded rows are fetched through offsets that must lie behind the K / V descriptors
+    if ((((int64_t)p.seq_k + 64) * std::max(p.k_strides[2], p.v_strides[2]) + head_dim) * 2 >= (int64_t(1) << 31)) return NINETOOTHED_NO_KERNEL;
+    if (head_dim > 128) return (int)launch_attention<T, 256, 1, 64, 1, false, TIO, kAttnWaves, true>(p, stream);
+    if (head_dim > 64) return (int)launch_attention<T, 128, 1, 64, 2, false, TIO, kAttnWaves, true>(p, stream);
+    if (head_dim > 32) return (int)launch_attention<T, 64, 1, 64, 2, false, TIO, kAttnWaves, true>(p, stream);
+    return (int)launch_attention<T, 32, 1, 64, 2, false, TIO, kAttnWaves, true>(p, stream);
 }
 
 // fp32 tensors: K and V become contiguous [batch, heads, seq, D] half-precision copies
@@ -556,6 +598,7 @@ int attention_float32(AttentionParams p, int head_dim, const NineToothedTensor &
     if (head_dim == 128) result = (int)launch_attention<half_t, 128, 1, 64, 2, false, float>(p, stream);
     else if (head_dim == 64) result = (int)launch_attention<half_t, 64, 1, 64, 2, false, float>(p, stream);
     else if (head_dim == 32) result = (int)launch_attention<half_t, 32, 1, 64, 2, false, float>(p, stream);
+    else result = launch_other_head_dim<half_t, float>(p, head_dim, stream);
     return result;
 }
 
@@ -584,7 +627,7 @@ int dispatch_attention(AttentionParams &p, int head_dim, int variant, hipStream_
         return (int)launch_attention<T, 64, 1, 64, 2, false>(p, stream);
     }
     if (head_dim == 32) return (int)launch_attention<T, 32, 1, 64, 2, false>(p, stream);
-    return NINETOOTHED_NO_KERNEL;
+    return launch_other_head_dim<T, T>(p, head_dim, stream);
 }
 
 }  // namespace
@@ -630,6 +673,7 @@ extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineT
         p.v_strides[d] = v.strides[d];
         p.o_strides[d] = o.strides[d];
     }
+    p.head_dim = (int)head_dim;
     p.q = q.data;
     p.k = k.data;
     p.v = v.data;

@@ -317,6 +317,43 @@ def test_attention_scaled_head_dim_128_and_bfloat16(is_causal):
     assert torch.allclose(out.float(), expected.float(), rtol=3e-2, atol=3e-2)
 
 
+def _attention_reference(q, k, v, is_causal, scale):
+    """fp32 attention on the given (already rounded) operands."""
+    scores = (q.float() * scale) @ k.float().transpose(-1, -2)
+    if is_causal:
+        mask = torch.ones(q.shape[-2], k.shape[-2], dtype=torch.bool, device=q.device).tril()
+        scores = scores.masked_fill(~mask, float("-inf"))
+    return torch.softmax(scores, dim=-1) @ v.float()
+
+
+@pytest.mark.parametrize("is_causal", (False, True))
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16, torch.float32))
+@pytest.mark.parametrize("emb_dim", (8, 40, 80, 96, 160, 192, 256))
+def test_attention_other_head_dims(emb_dim, dtype, is_causal):
+    """Head dimensions other than 32 / 64 / 128: 256 has a kernel of its own, other multiples of 8
+    run on the next size up with the missing columns of Q, K and V read as zeros.  K and V lie
+    inside larger Inf-filled rows, the output inside sentinel-filled ones: nothing past a row's
+    end may be read into the result or written."""
+    batch, heads, seq = 2, 3, 333
+    pitch = emb_dim + 8
+    def padded(fill):
+        storage = torch.full((batch, heads, seq, pitch), fill, dtype=dtype, device="cuda")
+        return storage, storage[..., :emb_dim]
+    (_, q), (_, k), (_, v) = (padded(float("inf")) for _ in range(3))
+    for t in (q, k, v):
+        t.copy_(torch.randn(batch, heads, seq, emb_dim, device="cuda") * 0.5)
+    o_storage, o = padded(7.0)
+    o.fill_(float("nan"))
+    scale = emb_dim**-0.5
+    kernel = ninetoothed.make(programs.attention.arrangement_with_scale, programs.attention.application_with_scale, programs.attention.tensors(True))
+    kernel(q, k, v, is_causal, scale, o)
+    _native_only(kernel, "launch_nt_attention")
+    expected = _attention_reference(q, k, v, is_causal, scale)
+    tolerance = {torch.float16: 1e-2, torch.bfloat16: 3e-2, torch.float32: 1e-2}[dtype]
+    assert torch.allclose(o.float(), expected, rtol=tolerance, atol=tolerance)
+    assert bool((o_storage[..., emb_dim:] == 7.0).all())
+
+
 def test_attention_closed_forms_and_layouts():
     q, v = _randn(1, 2, 300, 64).cuda(), _randn(1, 2, 300, 64).cuda()
     k = torch.zeros_like(q)
