@@ -520,17 +520,22 @@ std::string load_expr(const std::string &pointer, int dtype, const std::string &
     return "(double)" + element;
 }
 
+// Stores are non-temporal: the output of a streaming kernel is not read again by it, and the hint lets
+// the stores of a wave leave as whole lines (2^26-element add: fp32 5.65 -> 5.85 TB/s, fp16 3.98 -> 6.66;
+// row normalisations 5-18 % faster).  Loads stay plain: non-temporal loads cost 7-20 % in the softmax kernel.
 std::string store_stmt(const std::string &pointer, int dtype, const std::string &offset, const std::string &v) {
     const std::string target = std::string("((") + c_type(dtype) + " *)" + pointer + ")[" + offset + "]";
+    std::string value;
     switch (dtype) {
         case NINETOOTHED_FLOAT16:
-        case NINETOOTHED_BFLOAT16: return target + " = (" + c_type(dtype) + ")(float)(" + v + ");";
+        case NINETOOTHED_BFLOAT16: value = std::string("(") + c_type(dtype) + ")(float)(" + v + ")"; break;
         case NINETOOTHED_FLOAT32:
         case NINETOOTHED_FLOAT64:
         case NINETOOTHED_INT64:
-        case NINETOOTHED_UINT64: return target + " = (" + c_type(dtype) + ")(" + v + ");";
-        default: return target + " = (" + c_type(dtype) + ")(long long)(" + v + ");";
+        case NINETOOTHED_UINT64: value = std::string("(") + c_type(dtype) + ")(" + v + ")"; break;
+        default: value = std::string("(") + c_type(dtype) + ")(long long)(" + v + ")"; break;
     }
+    return "__builtin_nontemporal_store(" + value + ", &" + target + ");";
 }
 
 std::string atomic_add_stmt(const std::string &pointer, int dtype, const std::string &offset, const std::string &v) {

@@ -20,23 +20,27 @@ struct SoftmaxParams {
 
 constexpr float kLog2e = 1.4426950408889634f;
 
+// reductions over aligned groups of kLanes lanes of a wave
+template <int kLanes = 64>
 NT_DEVICE float wave_max(float v) {
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    for (int off = kLanes / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
     return v;
 }
 
+template <int kLanes = 64>
 NT_DEVICE float wave_sum(float v) {
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    for (int off = kLanes / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
     return v;
 }
 
-// Reduction over the kRowThreads threads that share a segment.  For 64 it is a
+// Reduction over the kRowThreads threads that share a segment.  Up to 64 it is a
 // pure wave reduction; for more, partial results cross waves through LDS.
 template <int kRowThreads, bool kIsMax>
 NT_DEVICE float group_reduce(float v, float *scratch) {
-    v = kIsMax ? wave_max(v) : wave_sum(v);
+    constexpr int kLanes = kRowThreads < 64 ? kRowThreads : 64;
+    v = kIsMax ? wave_max<kLanes>(v) : wave_sum<kLanes>(v);
     if constexpr (kRowThreads > 64) {
         constexpr int kWaves = kRowThreads / 64;
         const int wave = threadIdx.x >> 6;
@@ -60,11 +64,11 @@ struct Vec16 {  // 16 bytes of T
 // multiple of the vector width.  Thread t of a segment's group owns vectors
 // t, t + kRowThreads, ...  (coalesced 16-byte accesses).
 template <typename T, int kRowThreads, int kVecs>
-__global__ __launch_bounds__(256) void softmax_vec_kernel(SoftmaxParams p) {
+__global__ __launch_bounds__(kRowThreads > 256 ? kRowThreads : 256) void softmax_vec_kernel(SoftmaxParams p) {
     typedef typename Vec16<T>::type vec_t;
     constexpr int W = Vec16<T>::kWidth;
-    constexpr int kGroups = 256 / kRowThreads;  // segments per workgroup
-    __shared__ float scratch[4];
+    constexpr int kGroups = kRowThreads > 256 ? 1 : 256 / kRowThreads;  // segments per workgroup
+    __shared__ float scratch[16];
 
     const int group = threadIdx.x / kRowThreads;
     const int t = threadIdx.x % kRowThreads;
@@ -86,7 +90,7 @@ __global__ __launch_bounds__(256) void softmax_vec_kernel(SoftmaxParams p) {
     for (int j = 0; j < kVecs; ++j) {
         const int v = j * kRowThreads + t;
         if (v < nvec) {
-            vec_t raw = __builtin_nontemporal_load((const vec_t *)src + v);
+            vec_t raw = *((const vec_t *)src + v);  // (a non-temporal load here costs 7-20 % of the rate; the non-temporal store below gains)
 #pragma unroll
             for (int e = 0; e < W; ++e) {
                 x[j][e] = (float)raw[e];
@@ -126,7 +130,7 @@ __global__ __launch_bounds__(256) void softmax_vec_kernel(SoftmaxParams p) {
 template <typename T, int kRowThreads, int kElems>
 __global__ __launch_bounds__(256) void softmax_elem_kernel(SoftmaxParams p) {
     constexpr int kGroups = 256 / kRowThreads;
-    __shared__ float scratch[4];
+    __shared__ float scratch[16];
 
     const int group = threadIdx.x / kRowThreads;
     const int t = threadIdx.x % kRowThreads;
@@ -165,11 +169,15 @@ __global__ __launch_bounds__(256) void softmax_elem_kernel(SoftmaxParams p) {
     }
 }
 
-// Long segments: one workgroup per segment, three sweeps over memory (max, sum,
-// write); the second and third sweeps hit L2 for segments that fit there.
+// Long segments: one workgroup of 1024 threads per segment, two sweeps over memory: running
+// maximum and sum together (a thread rescales its sum once per round of eight independent loads),
+// then the write; the second sweep hits L2 for segments that fit there.
+constexpr int kLoopThreads = 1024;
+constexpr int kLoopUnroll = 8;
+
 template <typename T>
-__global__ __launch_bounds__(256) void softmax_loop_kernel(SoftmaxParams p) {
-    __shared__ float scratch[4];
+__global__ __launch_bounds__(kLoopThreads) void softmax_loop_kernel(SoftmaxParams p) {
+    __shared__ float scratch[kLoopThreads / 64];
     const int64_t seg = blockIdx.x;
     const int64_t row = seg / p.segments;
     const int64_t start = (seg % p.segments) * p.block;
@@ -177,24 +185,52 @@ __global__ __launch_bounds__(256) void softmax_loop_kernel(SoftmaxParams p) {
     const T *src = (const T *)p.in + row * p.in_row_stride + start * p.in_col_stride;
     T *dst = (T *)p.out + row * p.out_row_stride + start * p.out_col_stride;
 
-    float m = -INFINITY;
-    for (int64_t c = threadIdx.x; c < len; c += 256) m = fmaxf(m, (float)src[c * p.in_col_stride]);
-    m = group_reduce<256, true>(m, scratch);
-    const float shift = m * kLog2e;
-    float s = 0.0f;
-    for (int64_t c = threadIdx.x; c < len; c += 256)
-        s += __builtin_amdgcn_exp2f(fmaf((float)src[c * p.in_col_stride], kLog2e, -shift));
-    s = group_reduce<256, false>(s, scratch);
+    float m = -INFINITY, s = 0.0f;
+    for (int64_t base = threadIdx.x; base < len; base += kLoopThreads * kLoopUnroll) {
+        float x[kLoopUnroll];
+        float round_max = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < kLoopUnroll; ++u) {
+            const int64_t c = base + (int64_t)u * kLoopThreads;
+            x[u] = c < len ? (float)src[c * p.in_col_stride] : -INFINITY;
+            round_max = fmaxf(round_max, x[u]);
+        }
+        if (round_max > m) {  // (a first round of -inf only leaves m at -inf and s at 0)
+            s *= __builtin_amdgcn_exp2f((m - round_max) * kLog2e);
+            m = round_max;
+        }
+        if (m > -INFINITY) {
+            const float shift = m * kLog2e;
+#pragma unroll
+            for (int u = 0; u < kLoopUnroll; ++u) s += __builtin_amdgcn_exp2f(fmaf(x[u], kLog2e, -shift));
+        }
+    }
+    const float total_max = group_reduce<kLoopThreads, true>(m, scratch);
+    // every thread's sum is relative to its own maximum
+    s = m > -INFINITY ? s * __builtin_amdgcn_exp2f((m - total_max) * kLog2e) : 0.0f;
+    s = group_reduce<kLoopThreads, false>(s, scratch);
     const float inv = 1.0f / s;
-    for (int64_t c = threadIdx.x; c < len; c += 256)
-        dst[c * p.out_col_stride] = (T)(__builtin_amdgcn_exp2f(fmaf((float)src[c * p.in_col_stride], kLog2e, -shift)) * inv);
+    const float shift = total_max * kLog2e;
+    for (int64_t base = threadIdx.x; base < len; base += kLoopThreads * kLoopUnroll) {
+        float x[kLoopUnroll];
+#pragma unroll
+        for (int u = 0; u < kLoopUnroll; ++u) {
+            const int64_t c = base + (int64_t)u * kLoopThreads;
+            x[u] = c < len ? (float)src[c * p.in_col_stride] : -INFINITY;
+        }
+#pragma unroll
+        for (int u = 0; u < kLoopUnroll; ++u) {
+            const int64_t c = base + (int64_t)u * kLoopThreads;
+            if (c < len) dst[c * p.out_col_stride] = (T)(__builtin_amdgcn_exp2f(fmaf(x[u], kLog2e, -shift)) * inv);
+        }
+    }
 }
 
 template <typename T, int kRowThreads>
 hipError_t launch_vec(const SoftmaxParams &p, int vecs_needed, hipStream_t stream) {
     const int64_t total = p.rows * p.segments;
-    constexpr int kGroups = 256 / kRowThreads;
-    const dim3 grid((unsigned)((total + kGroups - 1) / kGroups)), block(256);
+    constexpr int kGroups = kRowThreads > 256 ? 1 : 256 / kRowThreads;
+    const dim3 grid((unsigned)((total + kGroups - 1) / kGroups)), block(kRowThreads > 256 ? kRowThreads : 256);
     if (vecs_needed <= 1)
         softmax_vec_kernel<T, kRowThreads, 1><<<grid, block, 0, stream>>>(p);
     else if (vecs_needed <= 2)
@@ -233,17 +269,28 @@ int run_softmax(const SoftmaxParams &p, int variant, hipStream_t stream) {
     const bool vector_ok = p.in_col_stride == 1 && p.out_col_stride == 1 && p.cols % W == 0 &&
                            (p.segments == 1 || p.block % W == 0) && p.in_row_stride % W == 0 &&
                            p.out_row_stride % W == 0 && ((uintptr_t)p.in & 15) == 0 && ((uintptr_t)p.out & 15) == 0;
-    if (vector_ok && len <= (int64_t)256 * 16 * W) {
+    if (vector_ok && len <= (int64_t)1024 * 16 * W) {
         const bool wave_fits = len <= (int64_t)64 * 16 * W;
         bool use_wave = wave_fits && len <= (int64_t)64 * 8 * W;  // default: keep <= 8 vectors per lane
+        // few segments: a workgroup each, so that more of the chip has something to fetch
+        if (use_wave && len > (int64_t)64 * W && total < 4096) use_wave = false;
         if (variant == 1 && wave_fits) use_wave = true;
         if (variant == 2) use_wave = false;
-        if (use_wave) return (int)launch_vec<T, 64>(p, (int)((len / W + 63) / 64), stream);
-        return (int)launch_vec<T, 256>(p, (int)((len / W + 255) / 256), stream);
+        const int64_t nvec = len / W;
+        if (variant == 0 && p.segments == 1) {  // short rows: 8, 16 or 32 lanes each, one vector per lane
+            if (nvec <= 8) return (int)launch_vec<T, 8>(p, 1, stream);
+            if (nvec <= 16) return (int)launch_vec<T, 16>(p, 1, stream);
+            if (nvec <= 32) return (int)launch_vec<T, 32>(p, 1, stream);
+        }
+        if (use_wave) return (int)launch_vec<T, 64>(p, (int)((nvec + 63) / 64), stream);
+        // more than 8 vectors per thread of a 256-thread workgroup: 1024 threads (registers per thread, not LDS, hold the row)
+        if (nvec > 256 * 8 && variant != 2) return (int)launch_vec<T, 1024>(p, (int)((nvec + 1023) / 1024), stream);
+        if (nvec > 256 * 16) return (int)launch_vec<T, 1024>(p, (int)((nvec + 1023) / 1024), stream);
+        return (int)launch_vec<T, 256>(p, (int)((nvec + 255) / 256), stream);
     }
     if (len <= 64 * 16) return (int)launch_elem<T, 64>(p, (int)((len + 63) / 64), stream);
     if (len <= 256 * 64) return (int)launch_elem<T, 256>(p, (int)((len + 255) / 256), stream);
-    softmax_loop_kernel<T><<<dim3((unsigned)total), dim3(256), 0, stream>>>(p);
+    softmax_loop_kernel<T><<<dim3((unsigned)total), dim3(kLoopThreads), 0, stream>>>(p);
     return (int)hipGetLastError();
 }
 

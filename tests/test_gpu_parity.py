@@ -226,6 +226,31 @@ def test_softmax_against_oracle(m, n):
     assert torch.allclose(out, torch.softmax(x.cuda(), dim=-1), rtol=1e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("dtype", (torch.float32, torch.float16, torch.bfloat16))
+@pytest.mark.parametrize(
+    "m, n",
+    ((100000, 32), (4099, 8), (7001, 64), (3000, 128), (513, 256), (1000, 1000), (128, 50257), (3, 200000), (9, 16385), (2, 70000)),
+)
+def test_softmax_short_rows_few_rows_and_long_rows(m, n, dtype):
+    """Rows of a few vectors share a wave (8, 16 or 32 lanes each); few rows get a workgroup
+    each; rows too long for registers take the two-sweep loop (running maximum and sum).
+    The output lies in a sentinel-filled buffer with a row pitch of its own."""
+    x = torch.randn(m, n, device="cuda").to(dtype)
+    x[0, 0] = 30.0  # one dominant element
+    if m > 1:
+        x[1, n // 2 :] = float("-inf")  # a row whose second half is masked out
+    pitch = n + (8 if n % 8 == 0 else 3)
+    buffer = torch.full((m, pitch), 7.0, dtype=dtype, device="cuda")
+    out = buffer[:, :n]
+    kernel = ninetoothed.make(programs.softmax.arrangement, programs.softmax.application, programs.softmax.tensors())
+    kernel(x, out, BLOCK_SIZE=1 << (n - 1).bit_length() if n > 1 else 1)
+    _native_only(kernel, "launch_nt_softmax")
+    expected = torch.softmax(x.float(), dim=-1)
+    tolerance = {torch.float32: dict(rtol=1e-5, atol=1e-6), torch.float16: dict(rtol=2e-3, atol=1e-4), torch.bfloat16: dict(rtol=1.6e-2, atol=1e-3)}[dtype]
+    assert torch.allclose(out.float(), expected, **tolerance)
+    assert bool((buffer[:, n:] == 7.0).all())
+
+
 def test_softmax_jit_decorator_form():
     # the decorator form with annotated parameters, as in the reference's tests/test_softmax.py:10-27
     import ninetoothed_amd.language as ntl
