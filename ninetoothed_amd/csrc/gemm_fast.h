@@ -413,7 +413,7 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
                     for (int e = 0; e < 4; ++e) v[e] = acc[ti][tj][4 * r4 + e];
                     const int gcol = n0 + wave_n * kWaveN + tj * 32 + 8 * r4 + 4 * g;
                     if (kTail && gcol >= p.n) continue;  // a partial last tile of columns
-                    *(float4_t *)(C32 + (int64_t)grow * p.ldc + gcol) = v;
+                    __builtin_nontemporal_store(v, (float4_t *)(C32 + (int64_t)grow * p.ldc + gcol));
                 }
         }
         return;
@@ -485,7 +485,9 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
 #pragma unroll
                 for (int e = 0; e < 8; ++e) v[e] = E::from_float(p.beta * E::to_float(in[e]) + p.alpha * E::to_float(v[e]));
             }
-            *(vec8 *)(C + (int64_t)grow * p.ldc + gcol) = v;
+            // non-temporal: C is not read again, and its lines then do not displace A / B panels in L2
+            // (4096^3 addmm +3 %, 8192^3 +0.3 %)
+            __builtin_nontemporal_store(v, (vec8 *)(C + (int64_t)grow * p.ldc + gcol));
         }
     }
 #endif
