@@ -15,8 +15,10 @@
  * `strides` are not read (reference: src/ninetoothed/aot.py:725-733, 624-628).
  *
  * Launches are asynchronous on the given stream and never synchronise; the
- * caller owns every tensor.  Only launch_nt_conv2d and launch_nt_attention on
- * FLOAT32 tensors use scratch device memory: one buffer per (device, stream,
+ * caller owns every tensor.  Only launch_nt_conv2d, launch_nt_attention on
+ * FLOAT32 tensors, and launch_nt_matmul / launch_nt_addmm on problems with few
+ * output tiles and a long K (split-K: parts x M x N floats, at most 64 MiB; not
+ * when the caller passes block sizes) use scratch device memory: one buffer per (device, stream,
  * purpose) that the library allocates (hipMalloc) the first time a call needs
  * it, grows (hipFree + hipMalloc, which wait for the device) when a later call
  * needs more, and otherwise reuses, so that steady-state calls allocate

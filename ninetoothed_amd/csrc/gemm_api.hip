@@ -1,6 +1,8 @@
 // C ABI for the GEMM family: launch_nt_matmul, launch_nt_addmm,
 // launch_nt_conv2d and the tile-selection entry points.
+#include <algorithm>
 #include <mutex>
+#include <type_traits>
 #include <shared_mutex>
 #include <unordered_map>
 #include <vector>
@@ -11,6 +13,7 @@
 #include "conv2d.h"
 #include "gemm_fast.h"
 #include "gemm_generic.h"
+#include "workspace.h"
 
 namespace nt {
 namespace {
@@ -109,6 +112,100 @@ hipError_t fast_launch(const GemmProblem &q, hipStream_t stream) {
     return fast_launch_typed<bf16_t, BM, BN, BK, WM, WN, kStages, kOcc, kAblate, kLoad, kAux, kTail>(q, stream);
 }
 
+// ---- split-K: problems with too few output tiles for 256 CUs (a few rows, or small M x N with a long K) ----
+// The k range is cut into parts, each (tile, part) is a workgroup that writes an fp32 tile to scratch
+// memory of the stream, and a second kernel sums the parts and applies the epilogue.
+
+// number of parts for tiles of bm x bn x bk, 1 = do not split
+int split_parts(const GemmProblem &q, int bm, int bn, int bk, int *kt_per_part) {
+    const int64_t tiles = (int64_t)((q.m + bm - 1) / bm) * ((q.n + bn - 1) / bn);
+    const int num_kt = (q.k + bk - 1) / bk;
+    if (tiles >= 192) return 1;
+    int64_t parts = (512 + tiles - 1) / tiles;                    // about two workgroups per CU
+    parts = std::min<int64_t>(parts, num_kt / 2);                  // at least two k tiles each
+    parts = std::min<int64_t>(parts, 256);
+    while (parts >= 2 && parts * q.m * q.n * 4 > (int64_t(64) << 20)) --parts;  // scratch of at most 64 MiB
+    if (parts < 2) return 1;
+    const int per_part = (int)((num_kt + parts - 1) / parts);
+    if (kt_per_part) *kt_per_part = per_part;
+    return (num_kt + per_part - 1) / per_part;                      // every part has at least one k tile
+}
+
+template <int BM, int BN, int BK, int kStages>
+bool split_accepts(const GemmProblem &q) {
+    // the operands, outputs and epilogues of the one-pass instances with tails (the second kernel writes
+    // four consecutive elements of C at a time, which their alignment rules cover)
+    return fast_accepts<BM, BN, BK, kStages, true>(q) && split_parts(q, BM, BN, BK, nullptr) >= 2;
+}
+
+// out[m][n] = epilogue(sum over parts): four consecutive columns per thread (N is a multiple of 8)
+template <typename T, typename TOut, bool kAddmm>
+__global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float *parts, int num_parts, int m, int n, TOut *c, int64_t ldc, const T *bias,
+                                                               int64_t bias_stride_m, int64_t bias_stride_n, float alpha, float beta) {
+    typedef float float4_t __attribute__((ext_vector_type(4)));
+    typedef TOut out4_t __attribute__((ext_vector_type(4)));
+    const int groups = n / 4;
+    const int64_t total = (int64_t)m * groups;
+    for (int64_t index = (int64_t)blockIdx.x * 256 + threadIdx.x; index < total; index += (int64_t)gridDim.x * 256) {
+        const int row = (int)(index / groups);
+        const int col = (int)(index - (int64_t)row * groups) * 4;
+        const float *src = parts + (int64_t)row * n + col;
+        float4_t sum = *(const float4_t *)src;
+        for (int part = 1; part < num_parts; ++part) sum += *(const float4_t *)(src + (int64_t)part * m * n);
+        out4_t out;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if constexpr (kAddmm) {
+                // as in the one-pass kernels: the product is rounded to the element type, then combined in fp32
+                const float product = Elem<T>::to_float(Elem<T>::from_float(sum[e]));
+                const float input = Elem<T>::to_float(bias[(int64_t)row * bias_stride_m + (int64_t)(col + e) * bias_stride_n]);
+                out[e] = Elem<T>::from_float(beta * input + alpha * product);
+            } else if constexpr (std::is_same<TOut, float>::value) {
+                out[e] = sum[e];
+            } else {
+                out[e] = Elem<T>::from_float(sum[e]);
+            }
+        }
+        __builtin_nontemporal_store(out, (out4_t *)(c + (int64_t)row * ldc + col));
+    }
+}
+
+template <typename T, int BM, int BN, int BK, int WM, int WN, int kStages, int kOcc>
+hipError_t split_launch_typed(const GemmProblem &q, hipStream_t stream) {
+    int kt_per_part = 0;
+    const int parts = split_parts(q, BM, BN, BK, &kt_per_part);
+    if (parts < 2) return (hipError_t)NINETOOTHED_NO_KERNEL;
+    WorkspaceLease lease(stream);
+    float *scratch = (float *)lease.get(kWorkspaceGemmParts, (size_t)parts * q.m * q.n * sizeof(float));
+    if (scratch == nullptr) return (hipError_t)NINETOOTHED_NO_KERNEL;  // no scratch (graph capture, out of memory): the caller takes a one-pass instance
+    GemmParams p;
+    fill_params(p, q, BM, BN);
+    p.c = scratch;
+    p.ldc = q.n;
+    p.bias = nullptr;
+    p.kt_per_split = kt_per_part;
+    const dim3 grid(p.tiles_m * p.tiles_n * parts), block(WM * WN * 64);
+    if (b_is_transposed(q)) gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, false, 0, 1, 0, true, true, true, true><<<grid, block, 0, stream>>>(p);
+    else gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, false, 0, 1, 0, true, false, true, true><<<grid, block, 0, stream>>>(p);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return err;
+    const int64_t groups = (int64_t)q.m * (q.n / 4);
+    const dim3 reduce_grid((unsigned)std::min<int64_t>((groups + 255) / 256, 256 * 8));
+    if (q.addmm())
+        gemm_split_reduce_kernel<T, T, true><<<reduce_grid, dim3(256), 0, stream>>>(scratch, parts, q.m, q.n, (T *)q.c, q.scm, (const T *)q.bias, q.sim, q.sin, q.alpha, q.beta);
+    else if (q.out_dtype == NINETOOTHED_FLOAT32)
+        gemm_split_reduce_kernel<T, float, false><<<reduce_grid, dim3(256), 0, stream>>>(scratch, parts, q.m, q.n, (float *)q.c, q.scm, nullptr, 0, 0, 1.0f, 0.0f);
+    else
+        gemm_split_reduce_kernel<T, T, false><<<reduce_grid, dim3(256), 0, stream>>>(scratch, parts, q.m, q.n, (T *)q.c, q.scm, nullptr, 0, 0, 1.0f, 0.0f);
+    return hipGetLastError();
+}
+
+template <int BM, int BN, int BK, int WM, int WN, int kStages, int kOcc>
+hipError_t split_launch(const GemmProblem &q, hipStream_t stream) {
+    if (q.dtype == NINETOOTHED_FLOAT16) return split_launch_typed<half_t, BM, BN, BK, WM, WN, kStages, kOcc>(q, stream);
+    return split_launch_typed<bf16_t, BM, BN, BK, WM, WN, kStages, kOcc>(q, stream);
+}
+
 bool generic_accepts(const GemmProblem &q) {
     if (q.dtype == NINETOOTHED_FLOAT8_E5M2)  // widened to fp16; addmm rounds its product to fp16, so it writes fp16
         return (q.out_dtype == NINETOOTHED_FLOAT16 || (q.out_dtype == NINETOOTHED_FLOAT32 && !q.addmm())) && q.m >= 0 && q.n >= 0 && q.k >= 0;
@@ -185,6 +282,9 @@ hipError_t generic_launch(const GemmProblem &q, hipStream_t stream) {
 #define NT_TAIL_INSTANCE(BM, BN, BK, WM, WN, ST, OCC) \
     {#BM "x" #BN "x" #BK " waves " #WM "x" #WN " stages " #ST " lds-direct tails", BM, BN, BK, fast_accepts<BM, BN, BK, ST, true>, fast_launch<BM, BN, BK, WM, WN, ST, OCC, 0, 1, 0, true>}
 
+#define NT_SPLIT_INSTANCE(BM, BN, BK, WM, WN, ST, OCC) \
+    {#BM "x" #BN "x" #BK " waves " #WM "x" #WN " stages " #ST " lds-direct tails split-k", BM, BN, BK, split_accepts<BM, BN, BK, ST>, split_launch<BM, BN, BK, WM, WN, ST, OCC>}
+
 const GemmInstance kInstances[] = {
     {"128x128x32 waves 2x2 any-stride", kGenBM, kGenBN, kGenBK, generic_accepts, generic_launch},
     NT_FAST_INSTANCE(256, 256, 32, 2, 4, 5, 2),  // 5 x 32 KiB: the whole LDS of a CU
@@ -196,6 +296,8 @@ const GemmInstance kInstances[] = {
     NT_TAIL_INSTANCE(128, 256, 32, 1, 4, 3, 2),
     NT_TAIL_INSTANCE(128, 128, 64, 2, 2, 2, 2),
     NT_TAIL_INSTANCE(64, 64, 64, 2, 2, 4, 2),
+    NT_SPLIT_INSTANCE(64, 64, 64, 2, 2, 4, 2),
+    NT_SPLIT_INSTANCE(128, 128, 64, 2, 2, 2, 2),
 #ifdef NT_GEMM_ABLATION
 #define NT_LOAD_INSTANCE(BM, BN, BK, WM, WN, ST, OCC, LD, AUX) \
     {#BM "x" #BN "x" #BK " waves " #WM "x" #WN " stages " #ST " load " #LD " aux " #AUX, BM, BN, BK, fast_accepts<BM, BN, BK, ST>, fast_launch<BM, BN, BK, WM, WN, ST, OCC, 0, LD, AUX>}
@@ -264,6 +366,10 @@ int heuristic_choice(const GemmProblem &q, int bm, int bn, int bk) {
     // untuned preference (measured on square problems): 256x256 tiles from 256 tiles up,
     // 128x256 from 128 tiles up, 128x128 from 256 tiles up, else the smallest tile that divides
     struct Rule { int instance; int64_t min_tiles; };
+    // too few tiles for the chip: split K (64-row tiles for up to 64 rows, else 128 x 128)
+    if (q.m <= 64 && kInstances[10].accepts(q)) return 10;
+    if (kInstances[11].accepts(q)) return 11;
+    if (kInstances[10].accepts(q)) return 10;
     // (instances 6..9 are 1, 5, 3, 4 with tails: they accept what those accept, so they come after them)
     const Rule rules[] = {{1, 256}, {2, 256}, {5, 128}, {3, 256}, {4, 1}, {3, 1}, {5, 1}, {2, 1}, {1, 1}, {6, 256}, {7, 128}, {8, 256}, {9, 1}, {8, 1}, {7, 1}, {6, 1}};
     for (const Rule &rule : rules) {
@@ -323,7 +429,12 @@ int run_gemm(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk) {
     if (bm <= 0 || bn <= 0) choice = lookup_tuned(q);
     if (choice < 0 || !kInstances[choice].accepts(q)) choice = heuristic_choice(q, bm, bn, bk);
     if (choice < 0) return NINETOOTHED_NO_KERNEL;
-    return (int)kInstances[choice].launch(q, stream);
+    int result = (int)kInstances[choice].launch(q, stream);
+    if (result == NINETOOTHED_NO_KERNEL && (choice == 10 || choice == 11)) {  // a split-K instance without scratch memory
+        for (int fallback : {9, 8, 6, 0})
+            if (kInstances[fallback].accepts(q)) return (int)kInstances[fallback].launch(q, stream);
+    }
+    return result;
 }
 
 }  // namespace

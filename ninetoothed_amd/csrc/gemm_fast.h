@@ -32,6 +32,7 @@ struct GemmParams {
     int tiles_m, tiles_n;
     int bias_vector;  // addmm input readable with aligned 16-byte loads along N
     int order;  // tile order: 0 = XCD-aware strips of 8 tile rows; other values are measurement aids
+    int kt_per_split;  // split-K instances: k tiles per part (the grid holds tiles * parts workgroups)
 };
 
 // A tile [BM][BK]: rows of BK * 2 bytes, split into 16-byte chunks.  Rows that
@@ -56,9 +57,7 @@ NT_HOST_DEVICE constexpr int b_phys_chunk(int krow, int chunk) {
 // round-robin to the 8 XCDs, so ids congruent mod 8 share an L2: give each
 // XCD a contiguous range of tile ids, ordered in column strips of kGroupM
 // tile-rows so that concurrently running tiles reuse A and B panels in L2.
-NT_DEVICE void map_tile(int tiles_m, int tiles_n, int order, int &tile_m, int &tile_n) {
-    int bid = blockIdx.x;
-    const int nblocks = gridDim.x;
+NT_DEVICE void map_tile(int tiles_m, int tiles_n, int order, int &tile_m, int &tile_n, int bid = blockIdx.x, int nblocks = gridDim.x) {
     // order: low 8 bits = tile rows per strip (0 -> 8), bit 8 = skip the XCD remap
     const int group_m = (order & 0xff) ? (order & 0xff) : 8;
     if ((nblocks & 7) == 0 && !(order & 0x100)) {
@@ -97,7 +96,7 @@ NT_DEVICE void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" 
 // kAblate is a measurement aid (bit 0: no global loads inside the K loop,
 // bit 1: operand fragments read from LDS only once); 0 in every shipped instance.
 template <typename T, int BM, int BN, int BK, int WM, int WN, int kStages, int kWavesPerSimd, bool kAddmm, int kAblate = 0, int kLoad = 0, int kAux = 0,
-          bool kFloatOut = false, bool kBT = false, bool kTail = false>
+          bool kFloatOut = false, bool kBT = false, bool kTail = false, bool kSplit = false>
 __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kernel(GemmParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only builtins; the host pass only needs the stub
     typedef Elem<T> E;
@@ -122,6 +121,10 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     // row-major B past K lie behind the end of its descriptor, and lanes whose chunk of a k-contiguous
     // row (A, transposed B) starts past K get an offset behind the end of theirs.
     static_assert(!kTail || kLoad == 1, "tails rely on the range check of buffer loads");
+    // kSplit: the grid holds tiles x parts workgroups; part s multiplies k tiles [s * kt_per_split, ...) and
+    // writes its fp32 accumulators to slice s of a [parts][M][N] scratch tensor (p.c, pitch p.ldc), which a
+    // second kernel sums -- for problems with too few output tiles to occupy the chip
+    static_assert(!kSplit || (kFloatOut && kTail && !kAddmm), "split-K parts are fp32 tiles with tails");
     static_assert(kStageA % (kWaves * 1024) == 0 && kStageB % (kWaves * 1024) == 0, "tile/wave mismatch");
     static_assert(kBChunksPerRow <= 64, "BN too large for one-instruction rows");
     static_assert(kWaveM % 32 == 0 && kWaveN % 32 == 0 && BK % 16 == 0, "wave tile");
@@ -165,7 +168,10 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     const int wave_n = wave % WN;
 
     int tile_m, tile_n;
-    map_tile(p.tiles_m, p.tiles_n, p.order, tile_m, tile_n);
+    const int tiles = p.tiles_m * p.tiles_n;
+    const int part = kSplit ? blockIdx.x / tiles : 0;
+    if constexpr (kSplit) map_tile(p.tiles_m, p.tiles_n, p.order, tile_m, tile_n, blockIdx.x - part * tiles, tiles);
+    else map_tile(p.tiles_m, p.tiles_n, p.order, tile_m, tile_n);
     const int m0 = tile_m * BM;
     const int n0 = tile_n * BN;
 
@@ -218,17 +224,20 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         }
         b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)b_base, 0, b_bytes, 0x00020000);
     }
-    const int num_k = kTail ? (p.k + BK - 1) / BK : p.k / BK;
+    const int all_k = kTail ? (p.k + BK - 1) / BK : p.k / BK;  // k tiles of the problem
+    const int k_first = kSplit ? part * p.kt_per_split : 0;     // this workgroup's first
+    const int num_k = kSplit ? min(p.kt_per_split, all_k - k_first) : all_k;
     const int last_k = num_k - 1;
-    // 16-byte chunks of the last k tile that lie inside K (all of them without a tail)
-    const int tail_chunks = kTail ? (p.k - last_k * BK) / 8 : kAChunksPerRow;
+    // 16-byte chunks of the problem's last k tile that lie inside K (all of them without a tail)
+    const int tail_chunks = kTail ? (p.k - (all_k - 1) * BK) / 8 : kAChunksPerRow;
     auto issue_loads = [&](auto stage_tag, int kt) {
         NT_LDS unsigned char *sa = stage_a(stage_tag);
         NT_LDS unsigned char *sb = stage_b(stage_tag);
+        kt += k_first;
         if constexpr (kLoad == 1) {
             const int a_k = kt * BK * 2;
             const int b_k = kBT ? a_k : kt * BK * (int)p.ldb * 2;
-            if (kTail && kt == last_k && tail_chunks < kAChunksPerRow) {  // uniform: the partial last k tile
+            if (kTail && kt == all_k - 1 && tail_chunks < kAChunksPerRow) {  // uniform: the partial last k tile
                 constexpr unsigned kBehind = 0x7fffffffu;  // behind every descriptor (their sizes stay below 2^31)
 #pragma unroll
                 for (int j = 0; j < kAInstr; ++j) {
@@ -398,7 +407,7 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         // and the four groups a 128-byte line, which the L2 merges
         static_assert(!kAddmm, "the fp32 output path has no addmm epilogue");
         wait_vmcnt<0>();
-        float *C32 = (float *)p.c;
+        float *C32 = (float *)p.c + (kSplit ? (int64_t)part * p.m * p.ldc : 0);
 #pragma unroll
         for (int ti = 0; ti < TM; ++ti) {
             const int grow = m0 + wave_m * kWaveM + ti * 32 + l32;

@@ -1,7 +1,7 @@
 // Device scratch buffers that outlive a call.
 //
-// conv2d's repacked operands and the narrowed K / V of fp32 attention are temporaries of
-// tens of megabytes.  Taking them from the stream-ordered allocator at every call leaves the
+// conv2d's repacked operands, the narrowed K / V of fp32 attention and the partial products of
+// split-K GEMMs are temporaries of up to tens of megabytes.  Taking them from the stream-ordered allocator at every call leaves the
 // GPU idle for ~10 us between calls (the allocation that follows a pending free is not handed
 // out before the free has executed).  Instead the library keeps one buffer per (device, stream,
 // purpose), grows it when a call needs more, and reuses it otherwise: work on one stream
@@ -15,7 +15,7 @@
 
 namespace nt {
 
-enum WorkspacePurpose { kWorkspaceConvInput, kWorkspaceConvFilter, kWorkspaceAttentionNarrow, kWorkspacePurposes };
+enum WorkspacePurpose { kWorkspaceConvInput, kWorkspaceConvFilter, kWorkspaceAttentionNarrow, kWorkspaceGemmParts, kWorkspacePurposes };
 
 // Holds the registry lock from construction to destruction: create it, take the buffers,
 // enqueue every kernel that uses them, then let it go.  Two host threads that launch on the

@@ -294,9 +294,17 @@ class Kernel:
         blocks = [info["blocks"][axis] if info["blocks"][axis] > 1 else 0 for axis in ("m", "n", "k")]
         dtype, out_dtype = runtime.DATA_TYPE_INDEX[tag], runtime.DATA_TYPE_INDEX[out_tag]
         in_pos, a_pos, b_pos, beta_pos, alpha_pos, c_pos = positions
-        a_arg = runtime.ArgumentTensor.from_layout(0, (m, k), (a.row_stride, a.col_stride))
-        b_arg = runtime.ArgumentTensor.from_layout(0, (k, n), (b.row_stride, b.col_stride))
-        c_arg = runtime.ArgumentTensor.from_layout(0, (m, n), (c.row_stride, c.col_stride))
+
+        def layout(matrix, rows, cols):
+            # a dimension of one element has no coefficient in the index map (stride 0): give it the
+            # stride of a dense matrix, so that a single row or column stays on the fast kernels
+            col_stride = matrix.col_stride if cols > 1 or matrix.col_stride else 1
+            row_stride = matrix.row_stride if rows > 1 or matrix.row_stride else (cols if col_stride == 1 else 1)
+            return (rows, cols), (row_stride, col_stride)
+
+        a_arg = runtime.ArgumentTensor.from_layout(0, *layout(a, m, k))
+        b_arg = runtime.ArgumentTensor.from_layout(0, *layout(b, k, n))
+        c_arg = runtime.ArgumentTensor.from_layout(0, *layout(c, m, n))
         # block sizes left to the tuner (all meta): like the reference's autotuned kernels, the
         # first launch of a new problem times the candidates once (src/ninetoothed/generation.py:372-516)
         from ninetoothed_amd import auto_tuner
@@ -316,7 +324,7 @@ class Kernel:
             auto_tuner.tune(input_arg, a_arg, b_arg, beta, alpha, c_arg, dtype, out_dtype)
 
         if i is not None:
-            i_arg = runtime.ArgumentTensor.from_layout(0, (m, n), (i.row_stride, i.col_stride))
+            i_arg = runtime.ArgumentTensor.from_layout(0, (m, n), (i.row_stride, i.col_stride))  # (a stride of 0 is a broadcast here)
 
             def launch(call_args):
                 a_arg.data = call_args[a_pos].data_ptr() + a.base * itemsize

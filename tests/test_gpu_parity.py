@@ -676,6 +676,8 @@ def test_gemm_any_number_of_rows_on_the_direct_to_lds_path(m, addmm):
             runtime.current_stream(), config, extra[0], runtime.ArgumentTensor.from_torch_tensor(a), runtime.ArgumentTensor.from_torch_tensor(b),
             extra[1], extra[2], runtime.ArgumentTensor.from_torch_tensor(out), fp16, fp16,
         )
+        if code == 1 and "split-k" in name:  # only takes problems with few output tiles
+            continue
         assert code == 0, name
         assert torch.allclose(out, expected, rtol=2e-2, atol=2e-2), name
         assert bool((guard[m:] == 7.0).all()), name
@@ -717,7 +719,7 @@ def test_gemm_partial_tiles_along_n_and_k(m, n, k, dtype):
             out_tag = runtime.DATA_TYPE_INDEX["fp32"] if out_dtype == torch.float32 else tag
             served = 0
             for instance, name in enumerate(names):
-                if "tails" not in name:
+                if "tails" not in name or "split-k" in name:
                     continue
                 out.fill_(float("nan"))
                 result = lib.launch_nt_gemm_config(
@@ -733,3 +735,51 @@ def test_gemm_partial_tiles_along_n_and_k(m, n, k, dtype):
         out = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
         _matmul_kernel()(a, b, out)
         assert torch.allclose(out.float()[clean_rows][:, clean_cols], product, **tolerance)
+
+
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
+@pytest.mark.parametrize("m, n, k", ((1, 2048, 4096), (16, 1024, 8192), (64, 520, 2056), (300, 200, 4104), (512, 512, 16384), (129, 136, 256)))
+def test_gemm_split_k(m, n, k, dtype):
+    """Few output tiles, long K: the k range is cut into parts that run as workgroups of their own
+    and a second kernel sums them (fp32) and applies the epilogue.  Both rhs layouts, element-type /
+    fp32 / addmm outputs, NaN-poisoned output with sentinel columns beside it; twice in a row
+    (the scratch tensor of the stream is reused)."""
+    from ninetoothed_amd import runtime
+
+    lib = runtime.library()
+    names = runtime.gemm_config_names()
+    tag = runtime.DATA_TYPE_INDEX["fp16" if dtype == torch.float16 else "bf16"]
+    null = runtime.ArgumentTensor.null()
+    beta, alpha = runtime.ArgumentTensor.from_scalar(0.5), runtime.ArgumentTensor.from_scalar(2.0)
+    tolerance = dict(rtol=2e-2, atol=2e-2 * max(k / 512, 1) ** 0.5) if dtype == torch.bfloat16 else dict(rtol=1e-2, atol=1e-2 * max(k / 512, 1) ** 0.5)
+    a = torch.randn(m, k, dtype=dtype, device="cuda")
+    bias = torch.randn(m, n, dtype=dtype, device="cuda")
+    for b in (torch.randn(k, n, dtype=dtype, device="cuda"), torch.randn(n, k, dtype=dtype, device="cuda").t()):
+        product = a.float() @ b.float()
+        for out_dtype, with_bias in ((dtype, False), (torch.float32, False), (dtype, True)):
+            buffer = torch.full((m, n + 8), 7.0, dtype=out_dtype, device="cuda")
+            out = buffer[:, :n]
+            tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (bias, a, b, out)]
+            expected = 0.5 * bias.float() + 2.0 * product.to(dtype).float() if with_bias else product
+            out_tag = runtime.DATA_TYPE_INDEX["fp32"] if out_dtype == torch.float32 else tag
+            served = 0
+            for instance, name in enumerate(names):
+                if "split-k" not in name:
+                    continue
+                for _ in range(2):
+                    out.fill_(float("nan"))
+                    result = lib.launch_nt_gemm_config(
+                        runtime.current_stream(), instance, tensors[0] if with_bias else null, tensors[1], tensors[2], beta if with_bias else null,
+                        alpha if with_bias else null, tensors[3], tag, out_tag,
+                    )
+                    if result == 1:
+                        break
+                    assert result == 0, name
+                    assert torch.allclose(out.float(), expected, **tolerance), (name, out_dtype, with_bias)
+                    assert bool((buffer[:, n:] == 7.0).all()), name
+                else:
+                    served += 1
+            assert served >= 1
+        out = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+        _matmul_kernel()(a, b, out)
+        assert torch.allclose(out.float(), product, **tolerance)
