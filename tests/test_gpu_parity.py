@@ -379,6 +379,19 @@ def test_attention_other_head_dims(emb_dim, dtype, is_causal):
     assert bool((o_storage[..., emb_dim:] == 7.0).all())
 
 
+@pytest.mark.parametrize("batch, heads, seq_q, seq_k, emb_dim", ((32, 32, 1, 2048, 128), (8, 32, 128, 8192, 128), (2, 8, 4096, 512, 64), (1, 8, 16, 65536, 128), (3, 5, 77, 1000, 64)))
+def test_attention_with_its_own_key_length(batch, heads, seq_q, seq_k, emb_dim):
+    """Queries against a longer (decoding, cross attention) or shorter key / value sequence."""
+    q = _randn(batch, heads, seq_q, emb_dim).cuda()
+    k, v = _randn(batch, heads, seq_k, emb_dim).cuda(), _randn(batch, heads, seq_k, emb_dim).cuda()
+    o = torch.full_like(q, float("nan"))
+    scale = emb_dim**-0.5
+    kernel = ninetoothed.make(programs.attention.arrangement_with_scale, programs.attention.application_with_scale, programs.attention.tensors(True))
+    kernel(q, k, v, False, scale, o)
+    _native_only(kernel, "launch_nt_attention")
+    assert torch.allclose(o.float(), _attention_reference(q, k, v, False, scale), **HALF_TOL)
+
+
 def test_attention_closed_forms_and_layouts():
     q, v = _randn(1, 2, 300, 64).cuda(), _randn(1, 2, 300, 64).cuda()
     k = torch.zeros_like(q)
