@@ -16,7 +16,9 @@
  *
  * Launches are asynchronous on the given stream and never synchronise; the
  * caller owns every tensor.  Only launch_nt_conv2d, launch_nt_attention on
- * FLOAT32 tensors, and launch_nt_matmul / launch_nt_addmm on problems with few
+ * FLOAT32 tensors or on few query blocks against many keys (split key range:
+ * parts x batch x heads x seq_q x (head_dim + 1) floats; not when the caller
+ * passes block sizes), and launch_nt_matmul / launch_nt_addmm on problems with few
  * output tiles and a long K (split-K: parts x M x N floats, at most 64 MiB; not
  * when the caller passes block sizes) use scratch device memory: one buffer per (device, stream,
  * purpose) that the library allocates (hipMalloc) the first time a call needs

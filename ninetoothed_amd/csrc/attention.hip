@@ -34,6 +34,12 @@ struct AttentionParams {
     int causal;
     int q_blocks;
     int head_dim;  // elements per row in memory (a multiple of 8; the kernel's D when it is not padded)
+    // split key range: the grid holds `parts` workgroups per (batch, head, query block); part s takes key
+    // blocks [s * blocks_per_part, ...) and writes a normalised fp32 partial output and the base-2
+    // logarithm of its softmax denominator (times 2^max) to scratch memory, which a second kernel merges
+    int parts, blocks_per_part;
+    float *part_o;    // [parts][batch * heads][seq_q][D]
+    float *part_lse;  // [parts][batch * heads][seq_q]
 };
 
 constexpr int kAttnWaves = 4;
@@ -44,8 +50,9 @@ constexpr int kAttnWaves = 4;
 // are converted to T beforehand; Q is converted while it is scaled, O is stored unrounded)
 // kPadded: the head dimension in memory (p.head_dim, a multiple of 8) is smaller than D: the missing
 // columns of Q, K and V read as zeros (scores and the stored columns are unchanged by them)
-template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined, typename TIO = T, int kWaves = kAttnWaves, bool kPadded = false>
+template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined, typename TIO = T, int kWaves = kAttnWaves, bool kPadded = false, bool kSplitKV = false>
 __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(AttentionParams p) {
+    static_assert(!kSplitKV || !kPipelined, "the key range is split in the plain loop only");
 #if defined(__HIP_DEVICE_COMPILE__)
     typedef Elem<T> E;
     typedef typename E::vec8 vec8;
@@ -91,8 +98,9 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
     // short blocks while only the K/V of one group (plus the next one's beginning)
     // is live in the XCD's L2.  Other pair counts fall back to walking all pairs.
     constexpr int kCausalGroup = 4;
-    int wg = blockIdx.x;
-    const int total = gridDim.x;
+    const int total = kSplitKV ? gridDim.x / p.parts : gridDim.x;
+    const int part = kSplitKV ? blockIdx.x / total : 0;
+    int wg = kSplitKV ? blockIdx.x - part * total : blockIdx.x;
     const bool renumber = total % 8 == 0;
     if (renumber) wg = (wg & 7) * (total >> 3) + (wg >> 3);
     int qb, bh;
@@ -105,8 +113,8 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
             qb = p.q_blocks - 1 - in_group / kCausalGroup;
             bh = group * kCausalGroup + in_group % kCausalGroup;
         } else {
-            qb = p.q_blocks - 1 - blockIdx.x / pairs;
-            bh = blockIdx.x % pairs;
+            qb = p.q_blocks - 1 - wg / pairs;
+            bh = wg % pairs;
         }
     } else {
         qb = wg % p.q_blocks;
@@ -155,7 +163,12 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
     // ---- number of kv blocks this query block needs ----
     int kv_end = p.seq_k;
     if (p.causal) kv_end = min(kv_end, q0 + BM);  // keys beyond the last query row are masked for all rows
-    const int num_blocks = ceil_div(kv_end, BN);
+    int num_blocks = ceil_div(kv_end, BN);  // one past the last key block of this workgroup
+    int first_block = 0;
+    if constexpr (kSplitKV) {
+        first_block = part * p.blocks_per_part;
+        num_blocks = min(num_blocks, first_block + p.blocks_per_part);  // may leave nothing (causal: parts past the diagonal)
+    }
     const int last_block = num_blocks - 1;
 
     // ---- global -> LDS assignment ----
@@ -387,10 +400,10 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
             rescale(alpha);
             accumulate(stage_tag, pf);
         };
-        if (num_blocks > 0) {
-            issue_k(Stage0(), 0);
-            issue_v(Stage0(), 0);
-            for (int blk = 0; blk < num_blocks; blk += 2) {
+        if (num_blocks > first_block) {
+            issue_k(Stage0(), first_block);
+            issue_v(Stage0(), first_block);
+            for (int blk = first_block; blk < num_blocks; blk += 2) {
                 wait_vmcnt<0>();
                 lds_barrier();
                 issue_k(Stage1(), min(blk + 1, last_block));
@@ -515,6 +528,29 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
     }
 
     // ---- epilogue: O[q, d] = O^T[d, q] / l ----
+    if constexpr (kSplitKV) {
+#pragma unroll
+        for (int qt = 0; qt < kQTiles; ++qt) {
+            const float l_total = l_run[qt] + __shfl_xor(l_run[qt], 32, 64);
+            const float inv = l_total > 0.0f ? 1.0f / l_total : 0.0f;  // a part without keys contributes nothing
+            if (q_row[qt] < p.seq_q) {
+                const int64_t row = ((int64_t)part * p.batch * p.heads + bh) * p.seq_q + q_row[qt];
+                float *dst = p.part_o + row * D;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int r4 = 0; r4 < 4; ++r4) {
+                        typedef float float4_t __attribute__((ext_vector_type(4)));
+                        float4_t out;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) out[e] = o_acc[dt][qt][r4 * 4 + e] * inv;
+                        *(float4_t *)(dst + dt * 32 + 8 * r4 + 4 * g) = out;
+                    }
+                if (g == 0) p.part_lse[row] = l_total > 0.0f ? m_run[qt] + __builtin_amdgcn_logf(l_total) : -INFINITY;
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int qt = 0; qt < kQTiles; ++qt) {
         const float l_total = l_run[qt] + __shfl_xor(l_run[qt], 32, 64);
@@ -539,6 +575,71 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
         }
     }
 #endif
+}
+
+// merges the parts of a split key range: O = sum_s w_s O_s / sum_s w_s with w_s = 2^(lse_s - max lse);
+// one thread per row and four consecutive columns
+template <typename TIO, int D>
+__global__ __launch_bounds__(256) void attention_merge_kernel(AttentionParams p) {
+    typedef float float4_t __attribute__((ext_vector_type(4)));
+    constexpr int kGroups = D / 4;
+    const int64_t rows = (int64_t)p.batch * p.heads * p.seq_q;
+    const int64_t index = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (index >= rows * kGroups) return;
+    const int64_t row = index / kGroups;
+    const int col = (int)(index - row * kGroups) * 4;
+    if (col >= p.head_dim) return;
+    float top = -INFINITY;
+    for (int s = 0; s < p.parts; ++s) top = fmaxf(top, p.part_lse[s * rows + row]);
+    float4_t sum = {0.0f, 0.0f, 0.0f, 0.0f};
+    float weights = 0.0f;
+    for (int s = 0; s < p.parts; ++s) {
+        const float lse = p.part_lse[s * rows + row];
+        if (lse == -INFINITY) continue;
+        const float w = __builtin_amdgcn_exp2f(lse - top);
+        weights += w;
+        sum += w * *(const float4_t *)(p.part_o + (s * rows + row) * D + col);
+    }
+    const float inv = 1.0f / weights;
+    const int64_t q_in_head = row % p.seq_q;
+    const int64_t bh = row / p.seq_q;
+    TIO *dst = (TIO *)p.o + (bh / p.heads) * p.o_strides[0] + (bh % p.heads) * p.o_strides[1] + q_in_head * p.o_strides[2] + col;
+    typedef TIO out4_t __attribute__((ext_vector_type(4)));
+    out4_t out;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        if constexpr (std::is_same<TIO, float>::value) out[e] = sum[e] * inv;
+        else out[e] = Elem<TIO>::from_float(sum[e] * inv);
+    }
+    *(out4_t *)dst = out;
+}
+
+// Few (batch, head, query block) workgroups and a long key sequence (decoding): the key range is split
+// so that about 512 workgroups run; returns NINETOOTHED_NO_KERNEL when that does not apply.
+template <typename T, int D>
+int launch_split_keys(AttentionParams &p, hipStream_t stream) {
+    constexpr int BM = kAttnWaves * 32, BN = 64;
+    p.q_blocks = ceil_div(p.seq_q, BM);
+    const int64_t groups = (int64_t)p.batch * p.heads * p.q_blocks;
+    const int key_blocks = ceil_div(p.seq_k, BN);
+    if (groups == 0 || groups >= 128 || key_blocks < 8) return NINETOOTHED_NO_KERNEL;
+    const int64_t parts = std::min<int64_t>((512 + groups - 1) / groups, key_blocks / 4);  // at least four key blocks each
+    if (parts < 2) return NINETOOTHED_NO_KERNEL;
+    p.blocks_per_part = ceil_div(key_blocks, (int)parts);
+    p.parts = ceil_div(key_blocks, p.blocks_per_part);
+    const int64_t rows = (int64_t)p.batch * p.heads * p.seq_q;
+    const size_t bytes = (size_t)p.parts * rows * (D + 1) * sizeof(float);
+    if (bytes > (size_t(256) << 20)) return NINETOOTHED_NO_KERNEL;
+    WorkspaceLease lease(stream);
+    float *scratch = (float *)lease.get(kWorkspaceAttentionParts, bytes);
+    if (scratch == nullptr) return NINETOOTHED_NO_KERNEL;  // (graph capture without a buffer, out of memory): one pass
+    p.part_o = scratch;
+    p.part_lse = scratch + (size_t)p.parts * rows * D;
+    attention_fwd_kernel<T, D, 1, BN, 2, false, T, kAttnWaves, false, true><<<dim3((unsigned)(groups * p.parts)), dim3(kAttnWaves * 64), 0, stream>>>(p);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return (int)err;
+    attention_merge_kernel<T, D><<<dim3((unsigned)((rows * (D / 4) + 255) / 256)), dim3(256), 0, stream>>>(p);
+    return (int)hipGetLastError();
 }
 
 template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined, typename TIO = T, int kWaves = kAttnWaves, bool kPadded = false>
@@ -645,6 +746,9 @@ extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineT
     for (const NineToothedTensor *t : ts)
         if (!t->shape || !t->strides) return hipErrorInvalidValue;
     AttentionParams p;
+    p.parts = 1;
+    p.blocks_per_part = 0;
+    p.part_o = p.part_lse = nullptr;
     p.batch = (int)q.shape[0];
     p.heads = (int)q.shape[1];
     p.seq_q = (int)q.shape[2];
@@ -694,6 +798,14 @@ extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineT
 #ifdef NT_MEASUREMENT_AIDS
     if (block_size_n >= 1000) variant = block_size_n - 1000;  // explicit variant, for timing harnesses only
 #endif
+    if (block_size_m == 0 && block_size_n == 0 && (head_dim == 128 || head_dim == 64)) {  // no hints: decoding-like shapes split the keys
+        int result;
+        if (dtype == NINETOOTHED_FLOAT16)
+            result = head_dim == 128 ? launch_split_keys<half_t, 128>(p, (hipStream_t)stream) : launch_split_keys<half_t, 64>(p, (hipStream_t)stream);
+        else
+            result = head_dim == 128 ? launch_split_keys<bf16_t, 128>(p, (hipStream_t)stream) : launch_split_keys<bf16_t, 64>(p, (hipStream_t)stream);
+        if (result != NINETOOTHED_NO_KERNEL) return result;
+    }
     if (dtype == NINETOOTHED_FLOAT16) return dispatch_attention<half_t>(p, (int)head_dim, variant, (hipStream_t)stream);
     return dispatch_attention<bf16_t>(p, (int)head_dim, variant, (hipStream_t)stream);
 }

@@ -15,7 +15,7 @@
 
 namespace nt {
 
-enum WorkspacePurpose { kWorkspaceConvInput, kWorkspaceConvFilter, kWorkspaceAttentionNarrow, kWorkspaceGemmParts, kWorkspacePurposes };
+enum WorkspacePurpose { kWorkspaceConvInput, kWorkspaceConvFilter, kWorkspaceAttentionNarrow, kWorkspaceGemmParts, kWorkspaceAttentionParts, kWorkspacePurposes };
 
 // Holds the registry lock from construction to destruction: create it, take the buffers,
 // enqueue every kernel that uses them, then let it go.  Two host threads that launch on the

@@ -392,6 +392,28 @@ def test_attention_with_its_own_key_length(batch, heads, seq_q, seq_k, emb_dim):
     assert torch.allclose(o.float(), _attention_reference(q, k, v, False, scale), **HALF_TOL)
 
 
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
+@pytest.mark.parametrize("is_causal", (False, True))
+@pytest.mark.parametrize("batch, heads, seq_q, seq_k, emb_dim", ((1, 32, 1, 32768, 128), (2, 4, 130, 5000, 64), (1, 2, 1024, 1024, 64), (1, 1, 300, 4097, 128), (3, 1, 7, 600, 64)))
+def test_attention_split_key_range(batch, heads, seq_q, seq_k, emb_dim, is_causal, dtype):
+    """Few (batch, head, query block) groups and many keys: parts of the key range run as
+    workgroups of their own and a second kernel merges them.  With a causal mask, parts past
+    the diagonal have no keys at all.  Twice in a row on the same scratch memory."""
+    if is_causal and seq_q != seq_k:
+        pytest.skip("the causal mask of the program assumes equal lengths")
+    q = _randn(batch, heads, seq_q, emb_dim).cuda().to(dtype)
+    k, v = _randn(batch, heads, seq_k, emb_dim).cuda().to(dtype), _randn(batch, heads, seq_k, emb_dim).cuda().to(dtype)
+    scale = emb_dim**-0.5
+    kernel = ninetoothed.make(programs.attention.arrangement_with_scale, programs.attention.application_with_scale, programs.attention.tensors(True))
+    expected = _attention_reference(q, k, v, is_causal, scale)
+    tolerance = HALF_TOL if dtype == torch.float16 else dict(rtol=3e-2, atol=3e-2)
+    for _ in range(2):
+        o = torch.full_like(q, float("nan"))
+        kernel(q, k, v, is_causal, scale, o)
+        assert torch.allclose(o.float(), expected, **tolerance)
+    _native_only(kernel, "launch_nt_attention")
+
+
 def test_attention_closed_forms_and_layouts():
     q, v = _randn(1, 2, 300, 64).cuda(), _randn(1, 2, 300, 64).cuda()
     k = torch.zeros_like(q)
