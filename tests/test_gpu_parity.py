@@ -593,6 +593,49 @@ def test_scratch_buffers_are_reused_grown_and_released():
         runtime.library().nt_release_workspaces()
 
 
+@pytest.mark.parametrize("warm_on_capture_stream", (False, True))
+def test_calls_that_use_scratch_memory_inside_a_captured_graph(warm_on_capture_stream):
+    """A split-K product, a decoding attention and a convolution captured into a HIP graph.  Warmed
+    up on the capture stream, the stream's scratch buffers exist and the captured kernels reuse them
+    on every replay; warmed up elsewhere, nothing may be allocated during capture and the calls take
+    their scratch-free kernels.  Replayed three times with eager work in between, each replay
+    checked against the eager results."""
+    a, b = _randn(16, 4096).cuda(), _randn(4096, 1024, scale=0.1).cuda()
+    q, k, v = _randn(1, 4, 1, 64).cuda(), _randn(1, 4, 4096, 64).cuda(), _randn(1, 4, 4096, 64).cuda()
+    x, w = _randn(2, 64, 16, 16, scale=0.1).cuda(), _randn(64, 64, 3, 3, scale=0.1).cuda()
+    c = torch.empty(16, 1024, dtype=torch.float16, device="cuda")
+    o = torch.empty_like(q)
+    y = torch.empty(2, 64, 16, 16, dtype=torch.float16, device="cuda")
+    matmul = _matmul_kernel()
+    attention = ninetoothed.make(programs.attention.arrangement, programs.attention.application, programs.attention.tensors())
+    conv = ninetoothed.make(programs.conv2d.arrangement, programs.conv2d.application, programs.conv2d.tensors())
+
+    def run():
+        matmul(a, b, c)
+        attention(q, k, v, False, o)
+        conv(x, w, y, padding_h=1, padding_w=1)
+
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream if warm_on_capture_stream else torch.cuda.current_stream()):
+        run()  # also lets the first-launch tuner (which synchronises) finish outside the capture
+    torch.cuda.synchronize()
+    expected = (a.float() @ b.float(), _attention_reference(q, k, v, False, 1.0), F.conv2d(x.float(), w.float(), padding=1))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        run()
+    for replay in range(3):
+        for t in (c, o, y):
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.allclose(c.float(), expected[0], **HALF_TOL), replay
+        assert torch.allclose(o.float(), expected[1], **HALF_TOL), replay
+        assert torch.allclose(y.float(), expected[2], **HALF_TOL), replay
+        run()  # eager work between the replays
+        torch.cuda.synchronize()
+
+
 # ---- tile selection -------------------------------------------------------------
 
 
