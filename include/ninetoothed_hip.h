@@ -164,10 +164,11 @@ NineToothedResult launch_nt_attention(NineToothedStream stream,
  * dilation 1 and zero padding (padding_h, padding_w), computed as the implicit
  * GEMM [N*P*Q, C*R*S] x [C*R*S, K] the arrangement of
  * tests/test_conv2d.py:13-48 describes.
- * When C % 32 == 0, K % 64 == 0, the output is contiguous and
+ * When K % 64 == 0, C >= 2, the output is contiguous and
  * N*P*Q >= 1024, the call first repacks the input to channels-last and the
- * filter to [R*S*C, K] in the library's scratch buffers of `stream`
- * (N*C*H*W + K*C*R*S elements), then runs the direct-to-LDS main loop;
+ * filter to [R*S*C', K] (C' = C rounded up to a multiple of 32, zero filled)
+ * in the library's scratch buffers of `stream`
+ * (N*C'*H*W + K*C'*R*S elements), then runs the direct-to-LDS main loop;
  * block_size_m == 1 keeps the call on the scratch-free gather kernel, which
  * also serves every other shape and calls whose scratch cannot be allocated
  * (out of memory; a stream under graph capture that has no buffer yet). */

@@ -24,7 +24,9 @@
 // (8 consecutive rows then lie in one image, aligned), element by element otherwise.
 //
 // Requirements of this path (anything else uses the any-stride gather kernel):
-// fp16/bf16, C % 32 == 0, K_out % 64 == 0, contiguous output.
+// fp16/bf16, K_out % 64 == 0, contiguous output.  The repacked operands hold C rounded up to a
+// multiple of 32 channels, the extra ones zero (a 3-channel stem layer multiplies ten times the
+// useful work and is still twice as fast as the gather kernel).
 #include <algorithm>
 
 #include "conv2d.h"
@@ -54,6 +56,7 @@ struct FilterRepack {
     int K, C, R, S;
     int64_t s_k, s_c, s_r, s_s;
     int layers;
+    int Cp;  // channels of the repacked operands: C rounded up to the k step, the extra ones zero
 };
 
 template <typename T>
@@ -66,14 +69,14 @@ __global__ __launch_bounds__(256) void conv2d_repack_kernel(const T *x, T *xt, i
     if ((int)blockIdx.z < f.layers) {
         const T *w = (const T *)f.w;
         T *wt = (T *)f.wt;
-        const int64_t total = (int64_t)f.K * f.C * f.R * f.S;
+        const int64_t total = (int64_t)f.K * f.Cp * f.R * f.S;
         const int64_t layer_threads = (int64_t)gridDim.x * gridDim.y * 256 * f.layers;
         for (int64_t index = (((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 256 + t; index < total; index += layer_threads) {
             const int k = (int)(index % f.K);
             const int64_t row = index / f.K;
-            const int c = (int)(row % f.C);
-            const int rs = (int)(row / f.C);
-            wt[index] = w[(int64_t)k * f.s_k + (int64_t)c * f.s_c + (int64_t)(rs / f.S) * f.s_r + (int64_t)(rs % f.S) * f.s_s];
+            const int c = (int)(row % f.Cp);
+            const int rs = (int)(row / f.Cp);
+            wt[index] = c < f.C ? w[(int64_t)k * f.s_k + (int64_t)c * f.s_c + (int64_t)(rs / f.S) * f.s_r + (int64_t)(rs % f.S) * f.s_s] : (T)0.0f;
         }
         return;
     }
@@ -102,11 +105,11 @@ __global__ __launch_bounds__(256) void conv2d_repack_kernel(const T *x, T *xt, i
     for (int pass = 0; pass < 2; ++pass) {
         const int hw = pass * 32 + (t >> 3);
         const int c = (t & 7) * 8;
-        if (hw0 + hw < HW && c0 + c < C) {  // C % 8 == 0 on this path
+        if (hw0 + hw < HW && c0 + c < f.Cp) {  // Cp % 8 == 0; channels from C on were loaded as zeros
             vec8 v;
 #pragma unroll
             for (int e = 0; e < 8; ++e) v[e] = tile[(c + e) * kPitch + hw];
-            *(vec8 *)(xt + ((int64_t)n * HW + hw0 + hw) * C + c0 + c) = v;
+            *(vec8 *)(xt + ((int64_t)n * HW + hw0 + hw) * f.Cp + c0 + c) = v;
         }
     }
 }
@@ -340,8 +343,9 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
 
 template <typename T>
 int run_fast(const Conv2dRequest &q, hipStream_t stream) {
-    const int64_t xt_bytes = (int64_t)q.N * q.H * q.W * q.C * 2;
-    const int64_t wt_bytes = (int64_t)q.K * q.C * q.R * q.S * 2;
+    const int Cp = ceil_div(q.C, 32) * 32;
+    const int64_t xt_bytes = (int64_t)q.N * q.H * q.W * Cp * 2;
+    const int64_t wt_bytes = (int64_t)q.K * Cp * q.R * q.S * 2;
     WorkspaceLease lease(stream);
     void *xt = lease.get(kWorkspaceConvInput, (size_t)xt_bytes);
     void *wt = lease.get(kWorkspaceConvFilter, (size_t)wt_bytes);
@@ -351,19 +355,19 @@ int run_fast(const Conv2dRequest &q, hipStream_t stream) {
     FilterRepack f;
     f.w = q.w;
     f.wt = wt;
-    f.K = q.K; f.C = q.C; f.R = q.R; f.S = q.S;
+    f.K = q.K; f.C = q.C; f.R = q.R; f.S = q.S; f.Cp = Cp;
     f.s_k = q.ws[0]; f.s_c = q.ws[1]; f.s_r = q.ws[2]; f.s_s = q.ws[3];
     // about 512 workgroups for the filter, or one thread per element if that is less
-    const int64_t per_layer = (int64_t)ceil_div(HW, 64) * ceil_div(q.C, 64);
-    const int64_t wanted = std::min<int64_t>(512, ceil_div((int64_t)q.K * q.C * q.R * q.S, (int64_t)256));
+    const int64_t per_layer = (int64_t)ceil_div(HW, 64) * ceil_div(Cp, 64);
+    const int64_t wanted = std::min<int64_t>(512, ((int64_t)q.K * Cp * q.R * q.S + 255) / 256);
     f.layers = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(wanted, per_layer), 512));
-    conv2d_repack_kernel<T><<<dim3(ceil_div(HW, 64), ceil_div(q.C, 64), q.N + f.layers), dim3(256), 0, stream>>>(
+    conv2d_repack_kernel<T><<<dim3(ceil_div(HW, 64), ceil_div(Cp, 64), q.N + f.layers), dim3(256), 0, stream>>>(
         (const T *)q.x, (T *)xt, q.C, HW, q.W, q.xs[0], q.xs[1], q.xs[2], q.xs[3], vector_ok, f);
     ConvParams p;
     p.xt = xt;
     p.wt = wt;
     p.y = q.y;
-    p.N = q.N; p.C = q.C; p.H = q.H; p.W = q.W; p.K = q.K; p.R = q.R; p.S = q.S; p.P = q.P; p.Q = q.Q;
+    p.N = q.N; p.C = Cp; p.H = q.H; p.W = q.W; p.K = q.K; p.R = q.R; p.S = q.S; p.P = q.P; p.Q = q.Q;
     p.pad_h = q.pad_h; p.pad_w = q.pad_w;
     p.M = q.N * q.P * q.Q;
     p.xt_bytes = (unsigned)xt_bytes;
@@ -385,11 +389,12 @@ int run_fast(const Conv2dRequest &q, hipStream_t stream) {
 
 int conv2d_fast(const Conv2dRequest &q, hipStream_t stream) {
     if (q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) return NINETOOTHED_NO_KERNEL;
-    if (q.C % 32 || q.K % 64) return NINETOOTHED_NO_KERNEL;
+    // channels are padded to the k step of 32 with zeros; below a sixteenth of useful work the gather kernel is as good
+    if (q.K % 64 || q.C < 2) return NINETOOTHED_NO_KERNEL;
     if (q.ys[3] != 1 || q.ys[2] != q.Q || q.ys[1] != (int64_t)q.P * q.Q || q.ys[0] != (int64_t)q.K * q.P * q.Q) return NINETOOTHED_NO_KERNEL;
     if (((uintptr_t)q.y & 15) != 0) return NINETOOTHED_NO_KERNEL;
-    const int64_t xt_bytes = (int64_t)q.N * q.H * q.W * q.C * 2;
-    const int64_t wt_bytes = (int64_t)q.K * q.C * q.R * q.S * 2;
+    const int64_t xt_bytes = (int64_t)q.N * q.H * q.W * ceil_div(q.C, 32) * 32 * 2;
+    const int64_t wt_bytes = (int64_t)q.K * ceil_div(q.C, 32) * 32 * q.R * q.S * 2;
     if (xt_bytes >= (int64_t(1) << 31) || wt_bytes >= (int64_t(1) << 31)) return NINETOOTHED_NO_KERNEL;  // 32-bit buffer offsets
     if ((int64_t)q.N * q.P * q.Q > 0x7fffffffll || (int64_t)ceil_div(q.N * q.P * q.Q, 128) * (q.K / 64) > 0x7fffffffll) return NINETOOTHED_NO_KERNEL;
     if (q.N >= 65535 - 512 || ceil_div(q.C, 64) > 65535) return NINETOOTHED_NO_KERNEL;  // grid of the repacking pass: (positions, channels, filter layers + images)

@@ -544,6 +544,10 @@ def test_conv2d_baseline_shape_and_1x1():
         (2, 320, 16, 16, 320, 3, 3, (1, 1)),
         (3, 32, 9, 11, 192, 3, 2, (1, 0)),     # odd sizes all round
         (40, 96, 7, 5, 64, 2, 3, (0, 2)),
+        (4, 3, 64, 64, 64, 7, 7, (3, 3)),      # channels padded to the k step of 32: a stem convolution
+        (4, 16, 20, 20, 128, 3, 3, (1, 1)),
+        (3, 40, 12, 12, 64, 3, 3, (1, 1)),
+        (2, 200, 9, 9, 64, 1, 1, (0, 0)),
     ),
 )
 def test_conv2d_layer_shapes_on_the_direct_to_lds_path(n, c, h, w, k, r, s, padding):
