@@ -164,7 +164,7 @@ NineToothedResult launch_nt_attention(NineToothedStream stream,
  * dilation 1 and zero padding (padding_h, padding_w), computed as the implicit
  * GEMM [N*P*Q, C*R*S] x [C*R*S, K] the arrangement of
  * tests/test_conv2d.py:13-48 describes.
- * When K % 64 == 0, C >= 2, the output is contiguous and
+ * When K % 8 == 0, C >= 2, the output is contiguous and
  * N*P*Q >= 1024, the call first repacks the input to channels-last and the
  * filter to [R*S*C', K] (C' = C rounded up to a multiple of 32, zero filled)
  * in the library's scratch buffers of `stream`

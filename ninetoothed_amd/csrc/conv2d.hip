@@ -24,7 +24,7 @@
 // (8 consecutive rows then lie in one image, aligned), element by element otherwise.
 //
 // Requirements of this path (anything else uses the any-stride gather kernel):
-// fp16/bf16, K_out % 64 == 0, contiguous output.  The repacked operands hold C rounded up to a
+// fp16/bf16, K_out % 8 == 0, contiguous output.  The repacked operands hold C rounded up to a
 // multiple of 32 channels, the extra ones zero (a 3-channel stem layer multiplies ten times the
 // useful work and is still twice as fast as the gather kernel).
 #include <algorithm>
@@ -42,7 +42,7 @@ struct ConvParams {
     void *y;
     int N, C, H, W, K, R, S, P, Q, pad_h, pad_w;
     int M, tiles_m, tiles_n;  // M = N*P*Q rows
-    unsigned xt_bytes;
+    unsigned xt_bytes, wt_bytes;
 };
 
 // ---- pre-pass: one launch, two jobs ----
@@ -170,7 +170,9 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
 
     // ---- A: rows of the tile are output positions; per lane one 16-byte chunk of 8 channels ----
     __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.xt, 0, p.xt_bytes, 0x00020000);
-    __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)((const T *)p.wt + n0), 0, 0xffffffff, 0x00020000);
+    // the filter descriptor ends with the matrix: a partial last tile of output channels reads the next
+    // row's values (they only feed channels that are not stored) and, in the last row, zeros
+    __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)((const T *)p.wt + n0), 0, p.wt_bytes - (unsigned)n0 * 2u, 0x00020000);
     int a_base[kAInstr], a_y[kAInstr], a_x[kAInstr];
 #pragma unroll
     for (int j = 0; j < kAInstr; ++j) {
@@ -323,6 +325,7 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
             const int m = m0 + wave_m * kWaveM + chunk * 8;
             if (m >= p.M) continue;
             const int out_channel = n0 + wave_n * kWaveN + tj * 32 + channel;
+            if (out_channel >= p.K) continue;  // a partial last tile of output channels
             int image = m / PQ, pq = m - image * PQ;
             if (whole_chunks) {  // the 8 rows lie in one image and start at a multiple of 8
                 __builtin_nontemporal_store(v, (vec8 *)(Y + ((int64_t)image * p.K + out_channel) * PQ + pq));  // +2 % over a plain store
@@ -371,16 +374,21 @@ int run_fast(const Conv2dRequest &q, hipStream_t stream) {
     p.pad_h = q.pad_h; p.pad_w = q.pad_w;
     p.M = q.N * q.P * q.Q;
     p.xt_bytes = (unsigned)xt_bytes;
+    p.wt_bytes = (unsigned)wt_bytes;
     // tile by the number of output channels: 256 wide when they fill it and there are enough tiles for the
     // chip, else 128 (two workgroups per CU), else 128 x 64 tiles of four waves
     const auto launch = [&](auto kernel, int bm, int bn, int threads) {
         p.tiles_m = ceil_div(p.M, bm);
-        p.tiles_n = q.K / bn;
+        p.tiles_n = ceil_div(q.K, bn);
         kernel<<<dim3(p.tiles_m * p.tiles_n), dim3(threads), 0, stream>>>(p);
     };
-    const int64_t tiles_256 = (int64_t)ceil_div(p.M, 256) * (q.K / 256);
-    if (q.K % 256 == 0 && tiles_256 >= 192) launch(conv2d_nhwc_kernel<T, 256, 256, 2, 4, 4, 2>, 256, 256, 512);
-    else if (q.K % 128 == 0 && (int64_t)ceil_div(p.M, 256) * (q.K / 128) >= 192) launch(conv2d_nhwc_kernel<T, 256, 128, 4, 2, 3, 4>, 256, 128, 512);
+    // the widest tile that is at least 4/5 full of output channels and leaves enough tiles for the chip
+    const auto fits = [&](int bm, int bn) {
+        const int64_t tiles = (int64_t)ceil_div(p.M, bm) * ceil_div(q.K, bn);
+        return q.K * 5 >= ceil_div(q.K, bn) * bn * 4 && tiles >= 192;
+    };
+    if (fits(256, 256)) launch(conv2d_nhwc_kernel<T, 256, 256, 2, 4, 4, 2>, 256, 256, 512);
+    else if (fits(256, 128)) launch(conv2d_nhwc_kernel<T, 256, 128, 4, 2, 3, 4>, 256, 128, 512);
     else launch(conv2d_nhwc_kernel<T, 128, 64, 2, 2, 4, 3>, 128, 64, 256);
     return (int)hipGetLastError();
 }
@@ -390,13 +398,13 @@ int run_fast(const Conv2dRequest &q, hipStream_t stream) {
 int conv2d_fast(const Conv2dRequest &q, hipStream_t stream) {
     if (q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) return NINETOOTHED_NO_KERNEL;
     // channels are padded to the k step of 32 with zeros; below a sixteenth of useful work the gather kernel is as good
-    if (q.K % 64 || q.C < 2) return NINETOOTHED_NO_KERNEL;
+    if (q.K % 8 || q.C < 2) return NINETOOTHED_NO_KERNEL;  // (rows of the repacked filter are read in 16-byte pieces)
     if (q.ys[3] != 1 || q.ys[2] != q.Q || q.ys[1] != (int64_t)q.P * q.Q || q.ys[0] != (int64_t)q.K * q.P * q.Q) return NINETOOTHED_NO_KERNEL;
     if (((uintptr_t)q.y & 15) != 0) return NINETOOTHED_NO_KERNEL;
     const int64_t xt_bytes = (int64_t)q.N * q.H * q.W * ceil_div(q.C, 32) * 32 * 2;
     const int64_t wt_bytes = (int64_t)q.K * ceil_div(q.C, 32) * 32 * q.R * q.S * 2;
     if (xt_bytes >= (int64_t(1) << 31) || wt_bytes >= (int64_t(1) << 31)) return NINETOOTHED_NO_KERNEL;  // 32-bit buffer offsets
-    if ((int64_t)q.N * q.P * q.Q > 0x7fffffffll || (int64_t)ceil_div(q.N * q.P * q.Q, 128) * (q.K / 64) > 0x7fffffffll) return NINETOOTHED_NO_KERNEL;
+    if ((int64_t)q.N * q.P * q.Q > 0x7fffffffll || (int64_t)ceil_div(q.N * q.P * q.Q, 128) * ceil_div(q.K, 64) > 0x7fffffffll) return NINETOOTHED_NO_KERNEL;
     if (q.N >= 65535 - 512 || ceil_div(q.C, 64) > 65535) return NINETOOTHED_NO_KERNEL;  // grid of the repacking pass: (positions, channels, filter layers + images)
     // enough work to amortise the repacking pass
     if ((int64_t)q.N * q.P * q.Q < 1024) return NINETOOTHED_NO_KERNEL;

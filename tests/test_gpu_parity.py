@@ -548,6 +548,10 @@ def test_conv2d_baseline_shape_and_1x1():
         (4, 16, 20, 20, 128, 3, 3, (1, 1)),
         (3, 40, 12, 12, 64, 3, 3, (1, 1)),
         (2, 200, 9, 9, 64, 1, 1, (0, 0)),
+        (4, 64, 16, 16, 96, 3, 3, (1, 1)),     # partial last tiles of output channels
+        (4, 32, 32, 32, 24, 3, 3, (1, 1)),
+        (16, 64, 32, 32, 1000, 1, 1, (0, 0)),
+        (2, 64, 20, 20, 328, 3, 3, (1, 1)),
     ),
 )
 def test_conv2d_layer_shapes_on_the_direct_to_lds_path(n, c, h, w, k, r, s, padding):
