@@ -51,10 +51,13 @@ bool fast_accepts(const GemmProblem &q) {
     if (q.m <= 0 || q.n <= 0 || q.k <= 0) return false;
     // any number of rows: rows past M read as zeros and are not stored; N and K must fit the tile,
     // or, for the instances with tails, be multiples of 8 (whole 16-byte chunks)
-    if (kTail ? (q.n % 8 || q.k % 8) : (q.n % BN || q.k % BK)) return false;
+    // (K: whole 16-byte chunks of the k-contiguous rows; N: only where rows of B run along it.  With a
+    // transposed B any N goes: C is then stored element by element when its rows are not 16-byte aligned)
+    if (kTail ? (q.k % 8 || (q.n % 8 && !b_is_transposed(q))) : (q.n % BN || q.k % BK)) return false;
     if (q.sak != 1 || q.scn != 1) return false;
     if (q.sam % 8 || q.sam < q.k || q.scm < q.n) return false;
-    if (((uintptr_t)q.a & 15) || ((uintptr_t)q.b & 15) || ((uintptr_t)q.c & 15) || q.scm % 8) return false;
+    if (((uintptr_t)q.a & 15) || ((uintptr_t)q.b & 15)) return false;
+    if (!kTail && (((uintptr_t)q.c & 15) || q.scm % 8)) return false;
     // per-lane 32-bit byte offsets inside one tile panel
     if ((int64_t)BM * q.sam * 2 >= (int64_t(1) << 31)) return false;
     if (b_is_transposed(q)) {  // B as [N, K] with K contiguous (`x @ w.T`)
@@ -85,7 +88,9 @@ void fill_params(GemmParams &p, const GemmProblem &q, int bm, int bn) {
     p.tiles_m = (q.m + bm - 1) / bm;
     p.tiles_n = (q.n + bn - 1) / bn;
     p.order = g_tile_order;
-    p.bias_vector = q.bias != nullptr && q.sin == 1 && q.sim % 8 == 0 && ((uintptr_t)q.bias & 15) == 0;
+    p.bias_vector = q.bias != nullptr && q.sin == 1 && q.sim % 8 == 0 && ((uintptr_t)q.bias & 15) == 0 && q.n % 8 == 0;
+    p.c_vector = ((uintptr_t)q.c & 15) == 0 && q.scm % 8 == 0 && q.n % 8 == 0;
+    p.kt_per_split = 0;
 }
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, int kStages, int kOcc, int kAblate, int kLoad, int kAux, bool kTail>
@@ -135,6 +140,7 @@ template <int BM, int BN, int BK, int kStages>
 bool split_accepts(const GemmProblem &q) {
     // the operands, outputs and epilogues of the one-pass instances with tails (the second kernel writes
     // four consecutive elements of C at a time, which their alignment rules cover)
+    if (q.n % 8 || q.scm % 8 || ((uintptr_t)q.c & 15)) return false;
     return fast_accepts<BM, BN, BK, kStages, true>(q) && split_parts(q, BM, BN, BK, nullptr) >= 2;
 }
 
@@ -182,6 +188,7 @@ hipError_t split_launch_typed(const GemmProblem &q, hipStream_t stream) {
     fill_params(p, q, BM, BN);
     p.c = scratch;
     p.ldc = q.n;
+    p.c_vector = 1;  // (N is a multiple of 8 here and the scratch tensor is aligned)
     p.bias = nullptr;
     p.kt_per_split = kt_per_part;
     const dim3 grid(p.tiles_m * p.tiles_n * parts), block(WM * WN * 64);

@@ -33,6 +33,7 @@ struct GemmParams {
     int bias_vector;  // addmm input readable with aligned 16-byte loads along N
     int order;  // tile order: 0 = XCD-aware strips of 8 tile rows; other values are measurement aids
     int kt_per_split;  // split-K instances: k tiles per part (the grid holds tiles * parts workgroups)
+    int c_vector;      // rows of C take aligned 16-byte stores (else, in the instances with tails: element stores)
 };
 
 // A tile [BM][BK]: rows of BK * 2 bytes, split into 16-byte chunks.  Rows that
@@ -422,6 +423,12 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
                     for (int e = 0; e < 4; ++e) v[e] = acc[ti][tj][4 * r4 + e];
                     const int gcol = n0 + wave_n * kWaveN + tj * 32 + 8 * r4 + 4 * g;
                     if (kTail && gcol >= p.n) continue;  // a partial last tile of columns
+                    if (kTail && !p.c_vector) {  // N or the row pitch of C no multiple of 4: element by element
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (gcol + e < p.n) C32[(int64_t)grow * p.ldc + gcol + e] = v[e];
+                        continue;
+                    }
                     __builtin_nontemporal_store(v, (float4_t *)(C32 + (int64_t)grow * p.ldc + gcol));
                 }
         }
@@ -489,10 +496,16 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
                     in = *(const vec8 *)src;
                 } else {
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) in[e] = src[(int64_t)e * p.bias_stride_n];
+                    for (int e = 0; e < 8; ++e) in[e] = (!kTail || gcol + e < p.n) ? src[(int64_t)e * p.bias_stride_n] : E::from_float(0.0f);
                 }
 #pragma unroll
                 for (int e = 0; e < 8; ++e) v[e] = E::from_float(p.beta * E::to_float(in[e]) + p.alpha * E::to_float(v[e]));
+            }
+            if (kTail && !p.c_vector) {  // N or the row pitch of C no multiple of 8: element by element
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (gcol + e < p.n) C[(int64_t)grow * p.ldc + gcol + e] = v[e];
+                continue;
             }
             // non-temporal: C is not read again, and its lines then do not displace A / B panels in L2
             // (4096^3 addmm +3 %, 8192^3 +0.3 %)

@@ -824,6 +824,50 @@ def test_gemm_partial_tiles_along_n_and_k(m, n, k, dtype):
 
 
 @pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
+@pytest.mark.parametrize("m, n, k", ((300, 1001, 512), (64, 50257, 256), (1000, 77, 1032), (5, 3, 8)))
+def test_gemm_transposed_rhs_any_number_of_columns(m, n, k, dtype):
+    """`x @ w.T` with any number of rows of `w` (an odd vocabulary size): the operands still stream
+    through LDS in 16-byte pieces, C -- whose rows are then not 16-byte aligned -- is stored
+    element by element.  Every instance with tails, element-type / fp32 / addmm (any-stride input)."""
+    from ninetoothed_amd import runtime
+
+    lib = runtime.library()
+    names = runtime.gemm_config_names()
+    tag = runtime.DATA_TYPE_INDEX["fp16" if dtype == torch.float16 else "bf16"]
+    null = runtime.ArgumentTensor.null()
+    beta, alpha = runtime.ArgumentTensor.from_scalar(0.5), runtime.ArgumentTensor.from_scalar(2.0)
+    tolerance = dict(rtol=2e-2, atol=2e-2 * max(k / 512, 1) ** 0.5) if dtype == torch.bfloat16 else dict(rtol=1e-2, atol=1e-2 * max(k / 512, 1) ** 0.5)
+    a = torch.randn(m, k, dtype=dtype, device="cuda")
+    w = torch.randn(n, k, dtype=dtype, device="cuda")
+    b = w.t()
+    bias = torch.randn(m, n, dtype=dtype, device="cuda")
+    product = a.float() @ b.float()
+    for out_dtype, with_bias in ((dtype, False), (torch.float32, False), (dtype, True)):
+        buffer = torch.full((m * n + 16,), 7.0, dtype=out_dtype, device="cuda")
+        out = buffer[: m * n].view(m, n)
+        tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (bias, a, b, out)]
+        expected = 0.5 * bias.float() + 2.0 * product.to(dtype).float() if with_bias else product
+        out_tag = runtime.DATA_TYPE_INDEX["fp32"] if out_dtype == torch.float32 else tag
+        served = 0
+        for instance, name in enumerate(names):
+            if "tails" not in name or "split-k" in name:
+                continue
+            out.fill_(float("nan"))
+            result = lib.launch_nt_gemm_config(
+                runtime.current_stream(), instance, tensors[0] if with_bias else null, tensors[1], tensors[2], beta if with_bias else null,
+                alpha if with_bias else null, tensors[3], tag, out_tag,
+            )
+            assert result == 0, name
+            served += 1
+            assert torch.allclose(out.float(), expected, **tolerance), (name, out_dtype, with_bias)
+            assert bool((buffer[m * n :] == 7.0).all()), name
+        assert served >= 3
+    out = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+    _matmul_kernel()(a, b, out)
+    assert torch.allclose(out.float(), product, **tolerance)
+
+
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
 @pytest.mark.parametrize("m, n, k", ((1, 2048, 4096), (16, 1024, 8192), (64, 520, 2056), (300, 200, 4104), (512, 512, 16384), (129, 136, 256)))
 def test_gemm_split_k(m, n, k, dtype):
     """Few output tiles, long K: the k range is cut into parts that run as workgroups of their own
