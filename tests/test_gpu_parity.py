@@ -229,7 +229,8 @@ def test_softmax_against_oracle(m, n):
 @pytest.mark.parametrize("dtype", (torch.float32, torch.float16, torch.bfloat16))
 @pytest.mark.parametrize(
     "m, n",
-    ((100000, 32), (4099, 8), (7001, 64), (3000, 128), (513, 256), (1000, 1000), (128, 50257), (3, 200000), (9, 16385), (2, 70000)),
+    ((100000, 32), (4099, 8), (7001, 64), (3000, 128), (513, 256), (1000, 1000), (128, 50257), (3, 200000), (9, 16385), (2, 70000),
+     (3000, 29), (2000, 101), (700, 1001), (300, 4099), (50, 12289), (40, 7000)),
 )
 def test_softmax_short_rows_few_rows_and_long_rows(m, n, dtype):
     """Rows of a few vectors share a wave (8, 16 or 32 lanes each); few rows get a workgroup
