@@ -546,6 +546,70 @@ std::string atomic_add_stmt(const std::string &pointer, int dtype, const std::st
 }
 
 // Translates the programs into HIP source.  `counter` numbers temporaries.
+// value of an index segment at one point of the variables (checks ignored)
+long long segment_offset_at(const NineToothedMapProgram &q, int segment, const long long *vars) {
+    std::vector<long long> stack;
+    for (int pc = q.segment_begin[segment];; ++pc) {
+        const int op = q.index_code[pc] & 0xff, arg = q.index_code[pc] >> 8;
+        if (op == NT_MAP_I_END) break;
+        switch (op) {
+            case NT_MAP_I_CONST: stack.push_back((long long)q.index_constants[arg]); break;
+            case NT_MAP_I_VAR: stack.push_back(vars[arg]); break;
+            case NT_MAP_I_MULC: stack.back() *= (long long)q.index_constants[arg]; break;
+            case NT_MAP_I_ADD: {
+                const long long b = stack.back();
+                stack.pop_back();
+                stack.back() += b;
+                break;
+            }
+            case NT_MAP_I_DIVC:
+            case NT_MAP_I_MODC: {
+                const long long c = (long long)q.index_constants[arg], a = stack.back();
+                if (c == 0) return 0;
+                long long quotient = a / c;
+                if ((a % c != 0) && ((a < 0) != (c < 0))) --quotient;
+                stack.back() = op == NT_MAP_I_DIVC ? quotient : a - quotient * c;
+                break;
+            }
+            case NT_MAP_I_CHECK: stack.pop_back(); break;
+            default: return 0;
+        }
+    }
+    return stack.empty() ? 0 : stack.back();
+}
+
+// Reductions whose reduced positions lie closer together in memory than the outputs do (row sums of a
+// row-major matrix) run with one wave per output element: the lanes stride the reduced positions, so
+// a wave reads consecutive elements, and combine their partial results with shuffles.  With one thread
+// per output the lanes of a wave would read a row each.  Returns the lanes per output element: 64 or 1.
+int cooperative_lanes(const NineToothedMapProgram &q) {
+    const int num_out = q.num_vars - q.num_reduced;
+    if (q.num_phases != 0 || q.reduce_op == NT_MAP_REDUCE_NONE || q.num_dynamic != 0 || q.num_reduced == 0 || q.store_op != NT_MAP_STORE_ASSIGN) return 1;
+    long long reduced = 1;
+    for (int v = num_out; v < q.num_vars; ++v) reduced *= q.extents[v];
+    if (reduced < 128) return 1;
+    int operand = -1;  // the first tensor the reduced term loads
+    for (int pc = 0; pc < q.reduce_split && operand < 0; ++pc)
+        if ((q.value_code[pc] & 0xff) == NT_MAP_V_LOAD) operand = q.value_code[pc] >> 8;
+    if (operand < 0 || operand >= q.num_operands) return 1;
+    const int segment = q.operands[operand].segment;
+    long long vars[NT_MAP_MAX_VARS] = {0};
+    const long long base = segment_offset_at(q, segment, vars);
+    const int inner_reduced = q.num_vars - 1;
+    if (q.extents[inner_reduced] < 2) return 1;
+    vars[inner_reduced] = 1;
+    const long long step_reduced = std::llabs(segment_offset_at(q, segment, vars) - base);
+    vars[inner_reduced] = 0;
+    long long step_out = 0;
+    for (int v = num_out - 1; v >= 0 && step_out == 0; --v) {  // the fastest output variable that moves this tensor
+        if (q.extents[v] < 2) continue;
+        vars[v] = 1;
+        step_out = std::llabs(segment_offset_at(q, segment, vars) - base);
+        vars[v] = 0;
+    }
+    return step_reduced != 0 && (step_out == 0 || step_reduced < step_out) ? 64 : 1;
+}
+
 struct MapCodegen {
     const NineToothedMapProgram &p;
     std::ostringstream out;
@@ -553,6 +617,7 @@ struct MapCodegen {
     std::string indent = "        ";
 
     bool narrow;  // index arithmetic in 32 bits: every index value provably fits
+    int lanes;    // lanes per output element (cooperative_lanes)
     // Tile mode with small tiles: a thread's elements stay in registers between the phases.
     // `kept` lists the operands whose loaded values an earlier phase left in `ld<slot>[e]`,
     // `in_body` maps operands already loaded in the loop body being emitted to their temporaries.
@@ -560,7 +625,7 @@ struct MapCodegen {
     std::vector<bool> kept = std::vector<bool>(NT_MAP_MAX_OPERANDS, false);
     std::map<int, std::string> in_body;
 
-    explicit MapCodegen(const NineToothedMapProgram &program) : p(program), narrow(fits_int32(program)) {}
+    explicit MapCodegen(const NineToothedMapProgram &program) : p(program), narrow(fits_int32(program)), lanes(cooperative_lanes(program)) {}
 
     std::string fresh(const char *prefix) { return prefix + std::to_string(counter++); }
 
@@ -864,6 +929,11 @@ struct MapCodegen {
             << "    const nt_idx stride = (nt_idx)gridDim.x * " << kMapThreads << ";\n"
             << "    const nt_idx total_out = (nt_idx)a.total_out;\n";
         if (p.num_phases > 0) return generate_tile();
+        if (lanes > 1)
+            out << "    const nt_idx lane = threadIdx.x & " << lanes - 1 << ";\n"
+                << "    for (nt_idx element = ((nt_idx)blockIdx.x * " << kMapThreads << " + threadIdx.x) / " << lanes << "; element < total_out; element += stride / " << lanes << ") {\n"
+                << "        nt_uidx rest = (nt_uidx)element;\n";
+        else
         out << "    for (nt_idx element = (nt_idx)blockIdx.x * " << kMapThreads << " + threadIdx.x; element < total_out; element += stride) {\n"
             << "        nt_uidx rest = (nt_uidx)element;\n";
         for (int v = num_out - 1; v >= 0; --v)
@@ -875,6 +945,15 @@ struct MapCodegen {
         } else {
             const char *init = p.reduce_op == NT_MAP_REDUCE_SUM ? "0.0" : (p.reduce_op == NT_MAP_REDUCE_MAX ? "-__builtin_inf()" : "__builtin_inf()");
             out << "        double acc = " << init << ";\n";
+            long long reduced_total = 1;
+            for (int v = num_out; v < p.num_vars; ++v) reduced_total *= p.extents[v];
+            if (lanes > 1) {  // the lanes of a wave stride the reduced positions
+                out << indent << "for (nt_idx position = lane; position < " << lit(reduced_total) << "; position += " << lanes << ") {\n";
+                indent += "    ";
+                out << indent << "nt_uidx inner = (nt_uidx)position;\n";
+                for (int v = p.num_vars - 1; v >= num_out; --v)
+                    out << indent << "const nt_idx v" << v << " = (nt_idx)(inner % " << ulit((long long)p.extents[v]) << "); inner /= " << ulit((long long)p.extents[v]) << ";\n";
+            } else
             for (int v = num_out; v < p.num_vars; ++v) {
                 out << indent << "for (nt_idx v" << v << " = 0; v" << v << " < " << lit((long long)p.extents[v]) << "; ++v" << v << ") {\n";
                 indent += "    ";
@@ -886,6 +965,12 @@ struct MapCodegen {
                 const char *cmp = p.reduce_op == NT_MAP_REDUCE_MAX ? ">" : "<";
                 out << indent << "acc = (" << term << " != " << term << " || acc != acc) ? acc + " << term << " : (" << term << " " << cmp << " acc ? " << term << " : acc);\n";
             }
+            if (lanes > 1) {
+                indent.resize(indent.size() - 4);
+                out << indent << "}\n";
+                for (int offset = lanes / 2; offset > 0; offset >>= 1)
+                    out << indent << "{ const double other = __shfl_xor(acc, " << offset << ", 64); acc = " << combine_expr(p.reduce_op, p.reduce_dtype, "acc", "other") << "; }\n";
+            } else
             for (int v = num_out; v < p.num_vars; ++v) {
                 indent.resize(indent.size() - 4);
                 out << indent << "}\n";
@@ -896,7 +981,7 @@ struct MapCodegen {
         out << indent << "bool store_ok = true;\n";
         const std::string offset = index_segment(target.segment, "store_ok");
         const std::string pointer = "a.data[" + std::to_string(p.output) + "]";
-        out << indent << "if (store_ok) "
+        out << indent << (lanes > 1 ? "if (store_ok && lane == 0) " : "if (store_ok) ")
             << (p.store_op == NT_MAP_STORE_ATOMIC_ADD ? atomic_add_stmt(pointer, target.dtype, offset, result) : store_stmt(pointer, target.dtype, offset, result))
             << "\n";
         out << "    }\n}\n";
@@ -1012,7 +1097,8 @@ extern "C" NineToothedResult launch_nt_map(NineToothedStream stream, const NineT
     for (int i = 0; i < p.num_operands; ++i)
         if (p.operands[i].data == nullptr) return hipErrorInvalidValue;
     // enough workgroups for 8 per CU; the grid stride covers the rest
-    int64_t blocks = (total_out + kMapThreads - 1) / kMapThreads;
+    const int lanes = cooperative_lanes(p);  // (the interpreter kernels below run one thread per element regardless)
+    int64_t blocks = (total_out * lanes + kMapThreads - 1) / kMapThreads;
     if (blocks > 256 * 32) blocks = 256 * 32;
     int64_t tiles = 1, tile_elements = 1;
     if (p.num_phases > 0) {  // tile mode: one workgroup per tile

@@ -956,3 +956,53 @@ def test_axis_reductions_used_on_the_tile(interpret, monkeypatch):
     kernel(x, out)
     _served_by_map(kernel)
     assert torch.allclose(out, torch.softmax(x, -1), rtol=1e-5, atol=1e-7)
+
+
+@gpu
+@pytest.mark.parametrize("dtype", (torch.float32, torch.float16))
+@pytest.mark.parametrize("shape", ((1000, 128), (37, 5000), (4096, 1000), (64, 127)))
+def test_reductions_over_the_contiguous_dimension_share_a_wave(shape, dtype):
+    """Row reductions of a row-major matrix: the generated kernel gives an output element to a wave,
+    whose lanes stride the row (one thread per row would make a wave read 64 rows at once).
+    Column reductions and short rows keep one thread per output.  Sums, maxima with a NaN, two
+    reduced dimensions."""
+    rows, cols = shape
+    x = torch.randn(rows, cols, device="cuda").to(dtype)
+    out = torch.full((rows,), float("nan"), dtype=dtype, device="cuda")
+    kernel = ninetoothed.make(row_sum_arrangement, row_sum_application, (Tensor(2), Tensor(1)))
+    kernel(x, out)
+    _served_by_map(kernel)
+    tolerance = dict(rtol=1e-4, atol=1e-3) if dtype == torch.float32 else dict(rtol=1e-2, atol=0.25)
+    assert torch.allclose(out.float(), x.float().sum(dim=1) * 2, **tolerance)
+    shared = "position += 64" in open(kernel._source).read()
+    assert shared == (cols >= 128)
+
+    def row_max_application(input, output):
+        output = ntl.max(input)  # noqa: F841
+
+    x[1, cols // 2] = float("nan")
+    kernel = ninetoothed.make(row_sum_arrangement, row_max_application, (Tensor(2), Tensor(1)))
+    kernel(x, out)
+    expected = x.max(dim=1).values
+    assert torch.isnan(out[1]) and torch.equal(out[[0] + list(range(2, rows))], expected[[0] + list(range(2, rows))])
+
+    # columns: the outputs are the contiguous ones, a thread each
+    def column_arrangement(input, output):
+        return input.tile((-1, 1)).squeeze(0), output.tile((1,))
+
+    x = torch.randn(rows, cols, device="cuda").to(dtype)
+    column_out = torch.full((cols,), float("nan"), dtype=dtype, device="cuda")
+    kernel = ninetoothed.make(column_arrangement, row_sum_application, (Tensor(2), Tensor(1)))
+    kernel(x, column_out)
+    assert torch.allclose(column_out.float(), x.float().sum(dim=0) * 2, **tolerance)
+    assert "position += 64" not in open(kernel._source).read()
+
+    # two reduced dimensions
+    def plane_arrangement(input, output):
+        return input.tile((1, -1, -1)).squeeze(2).squeeze(1), output.tile((1,))
+
+    planes = torch.randn(9, rows // 8 + 1, 40, device="cuda").to(dtype)
+    plane_out = torch.full((9,), float("nan"), dtype=dtype, device="cuda")
+    kernel = ninetoothed.make(plane_arrangement, row_sum_application, (Tensor(3), Tensor(1)))
+    kernel(planes, plane_out)
+    assert torch.allclose(plane_out.float(), planes.float().sum(dim=(1, 2)) * 2, rtol=1e-2 if dtype == torch.float16 else 1e-4, atol=1.0 if dtype == torch.float16 else 1e-2)
