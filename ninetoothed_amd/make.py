@@ -127,6 +127,7 @@ class Kernel:
         self.parameters = list(inspect.signature(application).parameters)
         self.meta_symbols = recognition.unbound_meta_symbols(self.types)
         self._plans = {}
+        self._scalar_flags = tuple((t.ndim == 0 and not isinstance(t.dtype, Tensor), bool(t.constexpr)) for t in self.types)
         self._source_path = None
         self.last_plan = None  # description of the launch used by the latest call
 
@@ -174,15 +175,19 @@ class Kernel:
 
     # ---- plan construction ----------------------------------------------
     def _signature(self, args, kwargs):
+        # on the path of every call: torch.Size, the stride tuple, dtype and device are hashable as they are
         parts = []
-        for arg, tensor in zip(args, self.types):
-            if tensor.ndim == 0 and not isinstance(tensor.dtype, Tensor):
-                parts.append((type(arg).__name__, arg if tensor.constexpr else None))
+        for arg, (is_scalar, constexpr) in zip(args, self._scalar_flags):
+            if is_scalar:
+                parts.append((type(arg), arg if constexpr else None))
             elif getattr(arg, "is_nested", False):
-                parts.append(_jagged_layout(arg) + (arg.dtype, arg.device.index))
+                parts.append(_jagged_layout(arg) + (arg.dtype, arg.device))
             else:
-                parts.append((tuple(arg.shape), tuple(arg.stride()), arg.dtype, arg.device.index))
-        return tuple(parts), tuple(sorted(kwargs.items()))
+                try:
+                    parts.append((arg.shape, arg.stride(), arg.dtype, arg.device))
+                except AttributeError:  # not a tensor: `_environment` says so
+                    parts.append((type(arg), None))
+        return tuple(parts), (tuple(sorted(kwargs.items())) if kwargs else ())
 
     def _environment(self, args, kwargs, check_device=True):
         import torch
