@@ -125,7 +125,7 @@ hipError_t fast_launch(const GemmProblem &q, hipStream_t stream) {
 int split_parts(const GemmProblem &q, int bm, int bn, int bk, int *kt_per_part) {
     const int64_t tiles = (int64_t)((q.m + bm - 1) / bm) * ((q.n + bn - 1) / bn);
     const int num_kt = (q.k + bk - 1) / bk;
-    if (tiles >= 192) return 1;
+    if (tiles >= 320) return 1;  // (the untuned choice only splits below 192 tiles; between, the tuner decides)
     int64_t parts = (512 + tiles - 1) / tiles;                    // about two workgroups per CU
     parts = std::min<int64_t>(parts, num_kt / 2);                  // at least two k tiles each
     parts = std::min<int64_t>(parts, 256);
@@ -374,9 +374,13 @@ int heuristic_choice(const GemmProblem &q, int bm, int bn, int bk) {
     // 128x256 from 128 tiles up, 128x128 from 256 tiles up, else the smallest tile that divides
     struct Rule { int instance; int64_t min_tiles; };
     // too few tiles for the chip: split K (64-row tiles for up to 64 rows, else 128 x 128)
-    if (q.m <= 64 && kInstances[10].accepts(q)) return 10;
-    if (kInstances[11].accepts(q)) return 11;
-    if (kInstances[10].accepts(q)) return 10;
+    const auto few_tiles = [&](int instance) {
+        const GemmInstance &inst = kInstances[instance];
+        return (int64_t)((q.m + inst.bm - 1) / inst.bm) * ((q.n + inst.bn - 1) / inst.bn) < 192 && inst.accepts(q);
+    };
+    if (q.m <= 64 && few_tiles(10)) return 10;
+    if (few_tiles(11)) return 11;
+    if (few_tiles(10)) return 10;
     // (instances 6..9 are 1, 5, 3, 4 with tails: they accept what those accept, so they come after them)
     const Rule rules[] = {{1, 256}, {2, 256}, {5, 128}, {3, 256}, {4, 1}, {3, 1}, {5, 1}, {2, 1}, {1, 1}, {6, 256}, {7, 128}, {8, 256}, {9, 1}, {8, 1}, {7, 1}, {6, 1}};
     for (const Rule &rule : rules) {
