@@ -312,6 +312,7 @@ const GemmInstance kInstances[] = {
     {#BM "x" #BN "x" #BK " waves " #WM "x" #WN " stages " #ST " ABLATED " #AB " (wrong results)", BM, BN, BK, fast_accepts<BM, BN, BK, ST>, fast_launch<BM, BN, BK, WM, WN, ST, OCC, AB>}
     NT_LOAD_INSTANCE(256, 256, 32, 2, 4, 4, 2, 1, 0),
     NT_LOAD_INSTANCE(256, 256, 32, 2, 2, 4, 1, 1, 0),
+    NT_LOAD_INSTANCE(256, 256, 64, 2, 2, 2, 1, 1, 0),
     NT_LOAD_INSTANCE(128, 256, 32, 2, 2, 4, 2, 1, 0),
     NT_LOAD_INSTANCE(128, 256, 32, 2, 2, 3, 2, 1, 0),
     NT_LOAD_INSTANCE(256, 128, 32, 2, 2, 3, 2, 1, 0),
