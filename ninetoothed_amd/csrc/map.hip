@@ -788,13 +788,14 @@ struct MapCodegen {
                     case NT_MAP_V_NEG: e = "-" + a; break;
                     case NT_MAP_V_NOT: e = a + " == 0.0 ? 1.0 : 0.0"; break;
                     case NT_MAP_V_ABS: e = "fabs(" + a + ")"; break;
-                    case NT_MAP_V_EXP: e = "(double)expf((float)" + a + ")"; break;
+                    // exponentials and the sigmoid through the hardware's 2^x, as Triton's `tl.exp` / `tl.sigmoid` do
+                    case NT_MAP_V_EXP: e = "(double)__expf((float)" + a + ")"; break;
                     case NT_MAP_V_EXP2: e = "(double)exp2f((float)" + a + ")"; break;
                     case NT_MAP_V_LOG: e = "(double)logf((float)" + a + ")"; break;
                     case NT_MAP_V_LOG2: e = "(double)log2f((float)" + a + ")"; break;
                     case NT_MAP_V_SQRT: e = "sqrt(" + a + ")"; break;
                     case NT_MAP_V_RSQRT: e = "(double)(1.0f / sqrtf((float)" + a + "))"; break;
-                    case NT_MAP_V_SIGMOID: e = "(double)(1.0f / (1.0f + expf(-(float)" + a + ")))"; break;
+                    case NT_MAP_V_SIGMOID: e = "(double)__fdividef(1.0f, 1.0f + __expf(-(float)" + a + "))"; break;
                     case NT_MAP_V_TANH: e = "(double)tanhf((float)" + a + ")"; break;
                     case NT_MAP_V_SIN: e = "(double)sinf((float)" + a + ")"; break;
                     case NT_MAP_V_COS: e = "(double)cosf((float)" + a + ")"; break;
