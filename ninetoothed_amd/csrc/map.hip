@@ -622,6 +622,11 @@ struct MapCodegen {
     // `kept` lists the operands whose loaded values an earlier phase left in `ld<slot>[e]`,
     // `in_body` maps operands already loaded in the loop body being emitted to their temporaries.
     bool keep_loads = false;
+    // a masked element takes the operand's `other`, which the host rounds to the element type: a float holds both
+    bool kept_as_float(int slot) const {
+        const int dtype = p.operands[slot].dtype;
+        return dtype == NINETOOTHED_FLOAT16 || dtype == NINETOOTHED_BFLOAT16 || dtype == NINETOOTHED_FLOAT32;
+    }
     std::vector<bool> kept = std::vector<bool>(NT_MAP_MAX_OPERANDS, false);
     std::map<int, std::string> in_body;
 
@@ -736,7 +741,7 @@ struct MapCodegen {
         for (int pc = begin; pc < end; ++pc) {
             const int op = p.value_code[pc] & 0xff, arg = p.value_code[pc] >> 8;
             if (op == NT_MAP_V_LOAD && keep_loads && kept[arg]) {
-                stack.push_back("ld" + std::to_string(arg) + "[e]");
+                stack.push_back(kept_as_float(arg) ? "(double)ld" + std::to_string(arg) + "[e]" : "ld" + std::to_string(arg) + "[e]");
             } else if (op == NT_MAP_V_LOAD && keep_loads && in_body.count(arg)) {
                 stack.push_back(in_body[arg]);
             } else if (op == NT_MAP_V_LOAD) {
@@ -747,7 +752,7 @@ struct MapCodegen {
                 const std::string pointer = "a.data[" + std::to_string(arg) + "]";
                 stack.push_back(define(valid + " ? " + load_expr(pointer, operand.dtype, offset) + " : a.other[" + std::to_string(arg) + "]"));
                 if (keep_loads) {
-                    out << indent << "ld" << arg << "[e] = " << stack.back() << ";\n";
+                    out << indent << "ld" << arg << "[e] = " << (kept_as_float(arg) ? "(float)" : "") << stack.back() << ";\n";
                     in_body[arg] = stack.back();
                 }
             } else if (op == NT_MAP_V_CONST) {
@@ -860,11 +865,11 @@ struct MapCodegen {
     std::string generate_tile() {
         long long tiles = 1, tile_elements = 1;
         for (int v = 0; v < p.num_vars; ++v) (v < p.num_grid ? tiles : tile_elements) *= (long long)p.extents[v];
-        // up to 8 elements per thread: every operand is read from memory once and kept in registers
-        // (4096 rows of fp32: softmax(2x) 1024 wide 13 us against 16, 2048 wide 20 against 27; with 16
-        // per thread the two-phase programs got slower, 4096 wide rms norm 39 us against 33)
+        // up to 16 elements per thread: every operand is read from memory once and kept in registers
+        // (4096 rows of fp32: softmax(2x) 1024 wide 13 us against 16, 2048 wide 20 against 27, 4096 wide 33
+        // against 42; 32 per thread spills: 8192 wide rms norm 97 us against 62)
         const int per_thread = (int)((tile_elements + kMapThreads - 1) / kMapThreads);
-        keep_loads = tile_elements <= (long long)kMapThreads * 8;
+        keep_loads = tile_elements <= (long long)kMapThreads * 16;
         out << "    __shared__ double scratch[" << kMapThreads / 64 << "];\n"
             << "    for (nt_idx tile = (nt_idx)blockIdx.x; tile < " << lit(tiles) << "; tile += (nt_idx)gridDim.x) {\n"
             << "        nt_uidx tile_rest = (nt_uidx)tile;\n";
@@ -872,7 +877,8 @@ struct MapCodegen {
             out << "        const nt_idx v" << v << " = (nt_idx)(tile_rest % " << ulit((long long)p.extents[v]) << "); tile_rest /= " << ulit((long long)p.extents[v]) << ";\n";
         if (keep_loads) {
             std::fill(kept.begin(), kept.end(), false);
-            for (int slot = 0; slot < p.num_operands; ++slot) out << "        double ld" << slot << "[" << per_thread << "];\n";
+            // (values of 16- and 32-bit floating-point tensors are kept as floats: half the registers)
+            for (int slot = 0; slot < p.num_operands; ++slot) out << "        " << (kept_as_float(slot) ? "float" : "double") << " ld" << slot << "[" << per_thread << "];\n";
         }
         int begin = 0;
         for (int k = 0; k < p.num_phases; ++k) {
