@@ -192,12 +192,15 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
         const int chunk = b_phys_chunk<BN>(krow, lane % kBChunksPerRow);
         b_src[j] = (unsigned)(krow * p.K + chunk * 8) * 2u;
     }
-    const int channel_blocks = p.C / BK;
     auto issue_loads = [&](auto stage_tag, int kt) {
         NT_LDS unsigned char *sa = stage_a(stage_tag);
         NT_LDS unsigned char *sb = stage_b(stage_tag);
-        const int tap = kt / channel_blocks;
-        const int c0 = (kt - tap * channel_blocks) * BK;
+        // k order: channel block outer, filter taps inner -- the R*S taps of a block of 32 channels read the
+        // same pixels shifted by a row or a column, so they hit in L2 while the lines are still there
+        const int taps = p.R * p.S;
+        const int cb = kt / taps;
+        const int tap = kt - cb * taps;
+        const int c0 = cb * BK;
         const int fy = tap / p.S, fx = tap - fy * p.S;
         const int delta = ((fy * p.W + fx) * p.C + c0) * 2;
 #pragma unroll
@@ -206,7 +209,7 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
             const unsigned offset = inside ? (unsigned)(a_base[j] + delta) : 0x80000000u;  // beyond num_records: reads zeros
             __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, sa + (j * kWaves + wave) * 1024, 16, offset, 0, 0, 0);
         }
-        const int b_k = kt * BK * p.K * 2;
+        const int b_k = (tap * p.C + c0) * p.K * 2;
 #pragma unroll
         for (int j = 0; j < kBInstr; ++j)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, sb + (j * kWaves + wave) * 1024, 16, b_src[j], b_k, 0, 0);
@@ -267,7 +270,7 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
         }
     };
 
-    const int num_k = p.R * p.S * channel_blocks;
+    const int num_k = p.R * p.S * (p.C / BK);
     const int last_k = num_k - 1;
     const int main_k = num_k - num_k % kStages;
     static_for<0, kStages - 1>([&](auto s) { issue_loads(s, min((int)decltype(s)::value, last_k)); });
