@@ -292,6 +292,12 @@ hipError_t generic_launch(const GemmProblem &q, hipStream_t stream) {
 #define NT_SPLIT_INSTANCE(BM, BN, BK, WM, WN, ST, OCC) \
     {#BM "x" #BN "x" #BK " waves " #WM "x" #WN " stages " #ST " lds-direct tails split-k", BM, BN, BK, split_accepts<BM, BN, BK, ST>, split_launch<BM, BN, BK, WM, WN, ST, OCC>}
 
+// positions in kInstances (the tuning cache and the heuristics refer to instances by position)
+enum InstanceIndex {
+    kAnyStride, k256x256x32, k256x256x64, k128x128x64, k64x64x64, k128x256x32,
+    kTail256x256x32, kTail128x256x32, kTail128x128x64, kTail64x64x64, kSplit64x64x64, kSplit128x128x64,
+};
+
 const GemmInstance kInstances[] = {
     {"128x128x32 waves 2x2 any-stride", kGenBM, kGenBN, kGenBK, generic_accepts, generic_launch},
     NT_FAST_INSTANCE(256, 256, 32, 2, 4, 5, 2),  // 5 x 32 KiB: the whole LDS of a CU
@@ -323,6 +329,7 @@ const GemmInstance kInstances[] = {
 #endif
 };
 constexpr int kNumInstances = sizeof(kInstances) / sizeof(kInstances[0]);
+static_assert(kNumInstances > kSplit128x128x64, "InstanceIndex names the first instances of the table");
 
 // ---- per-device cache of tuned choices (device, problem signature) -> instance ----
 struct TuneKey {
@@ -379,18 +386,20 @@ int heuristic_choice(const GemmProblem &q, int bm, int bn, int bk) {
         const GemmInstance &inst = kInstances[instance];
         return (int64_t)((q.m + inst.bm - 1) / inst.bm) * ((q.n + inst.bn - 1) / inst.bn) < 192 && inst.accepts(q);
     };
-    if (q.m <= 64 && few_tiles(10)) return 10;
-    if (few_tiles(11)) return 11;
-    if (few_tiles(10)) return 10;
-    // (instances 6..9 are 1, 5, 3, 4 with tails: they accept what those accept, so they come after them)
-    const Rule rules[] = {{1, 256}, {2, 256}, {5, 128}, {3, 256}, {4, 1}, {3, 1}, {5, 1}, {2, 1}, {1, 1}, {6, 256}, {7, 128}, {8, 256}, {9, 1}, {8, 1}, {7, 1}, {6, 1}};
+    if (q.m <= 64 && few_tiles(kSplit64x64x64)) return kSplit64x64x64;
+    if (few_tiles(kSplit128x128x64)) return kSplit128x128x64;
+    if (few_tiles(kSplit64x64x64)) return kSplit64x64x64;
+    // (the instances with tails accept what their plain forms accept, so they come after them)
+    const Rule rules[] = {{k256x256x32, 256}, {k256x256x64, 256}, {k128x256x32, 128}, {k128x128x64, 256}, {k64x64x64, 1}, {k128x128x64, 1},
+                          {k128x256x32, 1}, {k256x256x64, 1}, {k256x256x32, 1}, {kTail256x256x32, 256}, {kTail128x256x32, 128}, {kTail128x128x64, 256},
+                          {kTail64x64x64, 1}, {kTail128x128x64, 1}, {kTail128x256x32, 1}, {kTail256x256x32, 1}};
     for (const Rule &rule : rules) {
         const GemmInstance &inst = kInstances[rule.instance];
         if (!inst.accepts(q)) continue;
         const int64_t tiles = (int64_t)((q.m + inst.bm - 1) / inst.bm) * ((q.n + inst.bn - 1) / inst.bn);
         if (tiles >= rule.min_tiles) return rule.instance;
     }
-    return kInstances[0].accepts(q) ? 0 : -1;
+    return kInstances[kAnyStride].accepts(q) ? kAnyStride : -1;
 }
 
 bool read_matrix(const NineToothedTensor &t, uint64_t &d0, uint64_t &d1, int64_t &s0, int64_t &s1) {
@@ -442,8 +451,8 @@ int run_gemm(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk) {
     if (choice < 0 || !kInstances[choice].accepts(q)) choice = heuristic_choice(q, bm, bn, bk);
     if (choice < 0) return NINETOOTHED_NO_KERNEL;
     int result = (int)kInstances[choice].launch(q, stream);
-    if (result == NINETOOTHED_NO_KERNEL && (choice == 10 || choice == 11)) {  // a split-K instance without scratch memory
-        for (int fallback : {9, 8, 6, 0})
+    if (result == NINETOOTHED_NO_KERNEL && (choice == kSplit64x64x64 || choice == kSplit128x128x64)) {  // a split-K instance without scratch memory
+        for (int fallback : {(int)kTail64x64x64, (int)kTail128x128x64, (int)kTail256x256x32, (int)kAnyStride})
             if (kInstances[fallback].accepts(q)) return (int)kInstances[fallback].launch(q, stream);
     }
     return result;
@@ -553,8 +562,8 @@ NineToothedResult nt_tune_cache_save(const char *path) {
     (void)hipGetDevice(&device);
     FILE *file = fopen(path, "w");
     if (file == nullptr) return hipErrorInvalidValue;
-    const GemmInstance &fallback = kInstances[1];
-    fprintf(file, "\n%d,%d,%d,%d\n", fallback.bm, fallback.bn, fallback.bk, 1);
+    const GemmInstance &fallback = kInstances[k256x256x32];
+    fprintf(file, "\n%d,%d,%d,%d\n", fallback.bm, fallback.bn, fallback.bk, (int)k256x256x32);
     {
         std::shared_lock<std::shared_mutex> lock(g_tune_mutex);
         for (const auto &entry : g_tuned) {
