@@ -169,6 +169,8 @@ NineToothedResult launch_nt_attention(NineToothedStream stream,
  * filter to [R*S*C', K] (C' = C rounded up to a multiple of 32, zero filled)
  * in the library's scratch buffers of `stream`
  * (N*C'*H*W + K*C'*R*S elements), then runs the direct-to-LDS main loop;
+ * 1 x 1 filters without padding (P*Q and C multiples of 8) run as one batched
+ * launch of the GEMM kernels on the tensors as they lie, without scratch;
  * block_size_m == 1 keeps the call on the scratch-free gather kernel, which
  * also serves every other shape and calls whose scratch cannot be allocated
  * (out of memory; a stream under graph capture that has no buffer yet). */

@@ -25,6 +25,8 @@ struct GemmProblem {
     void *c;
     int64_t sam, sak, sbk, sbn, scm, scn, sim, sin;
     float alpha, beta;
+    int batch = 1;  // independent products that share the shapes; operands move by these element strides
+    int64_t a_batch = 0, b_batch = 0, c_batch = 0, bias_batch = 0;
     bool addmm() const { return bias != nullptr; }
 };
 
@@ -58,6 +60,7 @@ bool fast_accepts(const GemmProblem &q) {
     if (q.sam % 8 || q.sam < q.k || q.scm < q.n) return false;
     if (((uintptr_t)q.a & 15) || ((uintptr_t)q.b & 15)) return false;
     if (!kTail && (((uintptr_t)q.c & 15) || q.scm % 8)) return false;
+    if (q.batch > 1 && ((q.a_batch | q.b_batch | q.c_batch) % 8 || (int64_t)((q.m + BM - 1) / BM) * ((q.n + BN - 1) / BN) * q.batch > 0x7fffffffll)) return false;
     // per-lane 32-bit byte offsets inside one tile panel
     if ((int64_t)BM * q.sam * 2 >= (int64_t(1) << 31)) return false;
     if (b_is_transposed(q)) {  // B as [N, K] with K contiguous (`x @ w.T`)
@@ -91,13 +94,18 @@ void fill_params(GemmParams &p, const GemmProblem &q, int bm, int bn) {
     p.bias_vector = q.bias != nullptr && q.sin == 1 && q.sim % 8 == 0 && ((uintptr_t)q.bias & 15) == 0 && q.n % 8 == 0;
     p.c_vector = ((uintptr_t)q.c & 15) == 0 && q.scm % 8 == 0 && q.n % 8 == 0;
     p.kt_per_split = 0;
+    p.batch = q.batch;
+    p.a_batch = q.a_batch;
+    p.b_batch = q.b_batch;
+    p.c_batch = q.c_batch;
+    p.bias_batch = q.bias_batch;
 }
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, int kStages, int kOcc, int kAblate, int kLoad, int kAux, bool kTail>
 hipError_t fast_launch_typed(const GemmProblem &q, hipStream_t stream) {
     GemmParams p;
     fill_params(p, q, BM, BN);
-    const dim3 grid(p.tiles_m * p.tiles_n), block(WM * WN * 64);
+    const dim3 grid(p.tiles_m * p.tiles_n * q.batch), block(WM * WN * 64);
     const bool f32 = q.out_dtype == NINETOOTHED_FLOAT32, addmm = q.addmm();
     if (b_is_transposed(q)) {
         if (f32) gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, false, kAblate, kLoad, kAux, true, true, kTail><<<grid, block, 0, stream>>>(p);
@@ -140,7 +148,7 @@ template <int BM, int BN, int BK, int kStages>
 bool split_accepts(const GemmProblem &q) {
     // the operands, outputs and epilogues of the one-pass instances with tails (the second kernel writes
     // four consecutive elements of C at a time, which their alignment rules cover)
-    if (q.n % 8 || q.scm % 8 || ((uintptr_t)q.c & 15)) return false;
+    if (q.n % 8 || q.scm % 8 || ((uintptr_t)q.c & 15) || q.batch != 1) return false;
     return fast_accepts<BM, BN, BK, kStages, true>(q) && split_parts(q, BM, BN, BK, nullptr) >= 2;
 }
 
@@ -214,6 +222,7 @@ hipError_t split_launch(const GemmProblem &q, hipStream_t stream) {
 }
 
 bool generic_accepts(const GemmProblem &q) {
+    if (q.batch != 1) return false;
     if (q.dtype == NINETOOTHED_FLOAT8_E5M2)  // widened to fp16; addmm rounds its product to fp16, so it writes fp16
         return (q.out_dtype == NINETOOTHED_FLOAT16 || (q.out_dtype == NINETOOTHED_FLOAT32 && !q.addmm())) && q.m >= 0 && q.n >= 0 && q.k >= 0;
     if (q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) return false;
@@ -389,14 +398,15 @@ int heuristic_choice(const GemmProblem &q, int bm, int bn, int bk) {
     if (q.m <= 64 && few_tiles(kSplit64x64x64)) return kSplit64x64x64;
     if (few_tiles(kSplit128x128x64)) return kSplit128x128x64;
     if (few_tiles(kSplit64x64x64)) return kSplit64x64x64;
-    // (the instances with tails accept what their plain forms accept, so they come after them)
-    const Rule rules[] = {{k256x256x32, 256}, {k256x256x64, 256}, {k128x256x32, 128}, {k128x128x64, 256}, {k64x64x64, 1}, {k128x128x64, 1},
-                          {k128x256x32, 1}, {k256x256x64, 1}, {k256x256x32, 1}, {kTail256x256x32, 256}, {kTail128x256x32, 128}, {kTail128x128x64, 256},
-                          {kTail64x64x64, 1}, {kTail128x128x64, 1}, {kTail128x256x32, 1}, {kTail256x256x32, 1}};
+    // (an instance with tails accepts what its plain form accepts, so it comes right after it: a partial
+    // last tile costs less than a smaller tile everywhere)
+    const Rule rules[] = {{k256x256x32, 256}, {k256x256x64, 256}, {kTail256x256x32, 256}, {k128x256x32, 128}, {kTail128x256x32, 128},
+                          {k128x128x64, 256}, {kTail128x128x64, 256}, {k64x64x64, 1}, {kTail64x64x64, 1}, {k128x128x64, 1}, {kTail128x128x64, 1},
+                          {k128x256x32, 1}, {kTail128x256x32, 1}, {k256x256x64, 1}, {k256x256x32, 1}, {kTail256x256x32, 1}};
     for (const Rule &rule : rules) {
         const GemmInstance &inst = kInstances[rule.instance];
         if (!inst.accepts(q)) continue;
-        const int64_t tiles = (int64_t)((q.m + inst.bm - 1) / inst.bm) * ((q.n + inst.bn - 1) / inst.bn);
+        const int64_t tiles = (int64_t)((q.m + inst.bm - 1) / inst.bm) * ((q.n + inst.bn - 1) / inst.bn) * q.batch;
         if (tiles >= rule.min_tiles) return rule.instance;
     }
     return kInstances[kAnyStride].accepts(q) ? kAnyStride : -1;
@@ -665,6 +675,31 @@ NineToothedResult launch_nt_conv2d(NineToothedStream stream, NineToothedTensor i
             request.xs[d] = input.strides[d];
             request.ws[d] = filter.strides[d];
             request.ys[d] = output.strides[d];
+        }
+        // 1 x 1 filters without padding: per image Y[K, P*Q] = W[K, C] . X[C, P*Q], a batch of row-major
+        // products on the tensors as they lie (no repacking, no scratch memory)
+        if (block_size_m != 1 && R == 1 && S == 1 && padding_h == 0 && padding_w == 0 && input.strides[3] == 1 && input.strides[2] == W &&
+            output.strides[3] == 1 && output.strides[2] == Q && filter.strides[1] == 1 && N <= 0x7fffffffll) {
+            GemmProblem q;
+            q.dtype = q.out_dtype = dtype;
+            q.m = (int)K;
+            q.n = (int)(P * Q);
+            q.k = (int)C;
+            q.a = filter.data;
+            q.b = input.data;
+            q.c = output.data;
+            q.bias = nullptr;
+            q.sam = filter.strides[0]; q.sak = 1;
+            q.sbk = input.strides[1]; q.sbn = 1;
+            q.scm = output.strides[1]; q.scn = 1;
+            q.sim = q.sin = 0;
+            q.alpha = 1.0f; q.beta = 0.0f;
+            q.batch = (int)N;
+            q.a_batch = 0;
+            q.b_batch = input.strides[0];
+            q.c_batch = output.strides[0];
+            const int choice = heuristic_choice(q, 0, 0, 0);
+            if (choice > kAnyStride && choice != kSplit64x64x64 && choice != kSplit128x128x64) return (int)kInstances[choice].launch(q, (hipStream_t)stream);
         }
         const int fast = block_size_m == 1 ? NINETOOTHED_NO_KERNEL : conv2d_fast(request, (hipStream_t)stream);
         if (fast != NINETOOTHED_NO_KERNEL) return fast;

@@ -34,6 +34,9 @@ struct GemmParams {
     int order;  // tile order: 0 = XCD-aware strips of 8 tile rows; other values are measurement aids
     int kt_per_split;  // split-K instances: k tiles per part (the grid holds tiles * parts workgroups)
     int c_vector;      // rows of C take aligned 16-byte stores (else, in the instances with tails: element stores)
+    // batch > 1: the grid holds tiles * batch workgroups; product b uses the operands moved by these element strides
+    int batch;
+    int64_t a_batch, b_batch, c_batch, bias_batch;
 };
 
 // A tile [BM][BK]: rows of BK * 2 bytes, split into 16-byte chunks.  Rows that
@@ -171,13 +174,14 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     int tile_m, tile_n;
     const int tiles = p.tiles_m * p.tiles_n;
     const int part = kSplit ? blockIdx.x / tiles : 0;
-    if constexpr (kSplit) map_tile(p.tiles_m, p.tiles_n, p.order, tile_m, tile_n, blockIdx.x - part * tiles, tiles);
+    const int batch = !kSplit && p.batch > 1 ? blockIdx.x / tiles : 0;
+    if (kSplit || p.batch > 1) map_tile(p.tiles_m, p.tiles_n, p.order, tile_m, tile_n, blockIdx.x - (part + batch) * tiles, tiles);
     else map_tile(p.tiles_m, p.tiles_n, p.order, tile_m, tile_n);
     const int m0 = tile_m * BM;
     const int n0 = tile_n * BN;
 
-    const T *A = (const T *)p.a;
-    const T *B = (const T *)p.b;
+    const T *A = (const T *)p.a + batch * p.a_batch;
+    const T *B = (const T *)p.b + batch * p.b_batch;
 
     // ---- global -> LDS assignments (per lane, fixed over the K loop) ----
     // Byte offsets relative to the tile's first A row / B column stay below
@@ -408,7 +412,7 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         // and the four groups a 128-byte line, which the L2 merges
         static_assert(!kAddmm, "the fp32 output path has no addmm epilogue");
         wait_vmcnt<0>();
-        float *C32 = (float *)p.c + (kSplit ? (int64_t)part * p.m * p.ldc : 0);
+        float *C32 = (float *)p.c + (kSplit ? (int64_t)part * p.m * p.ldc : batch * p.c_batch);
 #pragma unroll
         for (int ti = 0; ti < TM; ++ti) {
             const int grow = m0 + wave_m * kWaveM + ti * 32 + l32;
@@ -461,8 +465,8 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         }
         slab += w * kSlabBytes;
     }
-    T *C = (T *)p.c;
-    const T *bias = (const T *)p.bias;
+    T *C = (T *)p.c + batch * p.c_batch;
+    const T *bias = (const T *)p.bias + batch * p.bias_batch;
     const int slab_sw = (l32 >> kCShift) & (kCChunks - 1);
 #pragma unroll
     for (int ti = 0; ti < TM; ++ti) {
