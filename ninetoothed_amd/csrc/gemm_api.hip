@@ -393,7 +393,8 @@ int heuristic_choice(const GemmProblem &q, int bm, int bn, int bk) {
     // too few tiles for the chip: split K (64-row tiles for up to 64 rows, else 128 x 128)
     const auto few_tiles = [&](int instance) {
         const GemmInstance &inst = kInstances[instance];
-        return (int64_t)((q.m + inst.bm - 1) / inst.bm) * ((q.n + inst.bn - 1) / inst.bn) < 192 && inst.accepts(q);
+        // (with a short K the second kernel costs more than the idle CUs: 512^3 8 us split, 5 in one pass)
+        return q.k >= 2048 && (int64_t)((q.m + inst.bm - 1) / inst.bm) * ((q.n + inst.bn - 1) / inst.bn) < 192 && inst.accepts(q);
     };
     if (q.m <= 64 && few_tiles(kSplit64x64x64)) return kSplit64x64x64;
     if (few_tiles(kSplit128x128x64)) return kSplit128x128x64;
