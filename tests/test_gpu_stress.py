@@ -110,3 +110,57 @@ def test_softmax_baseline_whole_output():
         out = torch.full_like(x, float("nan"))
         kernel(x, out, BLOCK_SIZE=4096)
         assert torch.allclose(out, expected, rtol=1e-5, atol=1e-6)
+
+
+def test_gemm_instances_on_random_shapes():
+    """Every instance on 48 seeded random problems: any M, N and K with and without the divisibility the
+    direct-to-LDS kernels ask for, both rhs layouts, padded row pitches, element-type / fp32 / addmm
+    outputs.  An instance either declines (1) or writes the whole NaN-poisoned output correctly and
+    leaves the sentinels around it alone."""
+    import random
+
+    lib = runtime.library()
+    names = runtime.gemm_config_names()
+    null = runtime.ArgumentTensor.null()
+    fp16, fp32 = runtime.DATA_TYPE_INDEX["fp16"], runtime.DATA_TYPE_INDEX["fp32"]
+    beta, alpha = runtime.ArgumentTensor.from_scalar(-0.75), runtime.ArgumentTensor.from_scalar(1.5)
+    rng = random.Random(20240607)
+    served = {name: 0 for name in names}
+    for case in range(48):
+        m = rng.choice((1, 3, 16, 64, 100, 129, 256, 300, 513, 700))
+        n = rng.choice((8, 24, 64, 72, 128, 200, 256, 264, 520, 1000)) + rng.choice((0, 0, 0, 1, 5))
+        k = rng.choice((8, 16, 64, 72, 256, 520, 1024, 2056, 4096)) + rng.choice((0, 0, 0, 3))
+        transposed = rng.random() < 0.5
+        pad_a, pad_b, pad_c = (rng.choice((0, 0, 8, 24)) for _ in range(3))
+        a = torch.randn(m, k + pad_a, dtype=torch.float16, device="cuda")[:, :k]
+        if transposed:
+            b = torch.randn(n, k + pad_b, dtype=torch.float16, device="cuda")[:, :k].t()
+        else:
+            b = torch.randn(k, n + pad_b, dtype=torch.float16, device="cuda")[:, :n]
+        bias = torch.randn(m, n, dtype=torch.float16, device="cuda")
+        product = a.float() @ b.float()
+        mode = rng.choice(("plain", "fp32", "addmm"))
+        out_dtype = torch.float32 if mode == "fp32" else torch.float16
+        buffer = torch.full((m + 1, n + pad_c + 8), 7.0, dtype=out_dtype, device="cuda")
+        out = buffer[:m, :n]
+        expected = -0.75 * bias.float() + 1.5 * product.half().float() if mode == "addmm" else product
+        tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (bias, a, b, out)]
+        tolerance = dict(rtol=1e-2, atol=1e-2 * max(k / 512, 1) ** 0.5 * (2.0 if mode == "addmm" else 1.0))
+        ran = 0
+        for instance, name in enumerate(names):
+            out.fill_(float("nan"))
+            code = lib.launch_nt_gemm_config(
+                runtime.current_stream(), instance, tensors[0] if mode == "addmm" else null, tensors[1], tensors[2],
+                beta if mode == "addmm" else null, alpha if mode == "addmm" else null, tensors[3], fp16, fp32 if mode == "fp32" else fp16,
+            )
+            if code == 1:
+                continue
+            description = (case, m, n, k, transposed, mode, name)
+            assert code == 0, description
+            assert torch.allclose(out.float(), expected, **tolerance), description
+            assert bool((buffer[:m, n:] == 7.0).all()) and bool((buffer[m] == 7.0).all()), description
+            served[name] += 1
+            ran += 1
+        assert ran >= 1, (case, m, n, k, transposed, mode)
+    # (the instances without tails need N and K to fit their tiles; test_every_gemm_instance_whole_output covers them)
+    assert all(count > 0 for name, count in served.items() if "tails" in name or "any-stride" in name), served
