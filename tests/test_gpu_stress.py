@@ -164,3 +164,68 @@ def test_gemm_instances_on_random_shapes():
         assert ran >= 1, (case, m, n, k, transposed, mode)
     # (the instances without tails need N and K to fit their tiles; test_every_gemm_instance_whole_output covers them)
     assert all(count > 0 for name, count in served.items() if "tails" in name or "any-stride" in name), served
+
+
+def test_conv2d_on_random_layers():
+    """40 seeded random layers: channel counts with and without the multiples the implicit-GEMM kernel
+    likes, odd feature maps, filters from 1 x 1 to 5 x 3, every padding that leaves an output; the
+    whole NaN-poisoned output against an fp32 convolution, sentinels behind it untouched."""
+    import random
+
+    rng = random.Random(777)
+    kernel = ninetoothed.make(programs.conv2d.arrangement, programs.conv2d.application, programs.conv2d.tensors())
+    for case in range(40):
+        n = rng.choice((1, 2, 3, 8, 33))
+        c = rng.choice((1, 3, 8, 16, 32, 40, 64, 96, 136))
+        k = rng.choice((8, 16, 24, 64, 72, 128, 200, 256, 320)) + rng.choice((0, 0, 0, 4))
+        h, w = rng.choice((7, 8, 13, 14, 28, 31)), rng.choice((7, 8, 12, 14, 28, 33))
+        r, s = rng.choice((1, 1, 2, 3, 3, 5)), rng.choice((1, 1, 3, 3))
+        pad = (rng.choice((0, 1, 2)), rng.choice((0, 1, 2)))
+        if h + 2 * pad[0] < r or w + 2 * pad[1] < s:
+            continue
+        x = (torch.randn(n, c, h, w, device="cuda") * 0.5).half()
+        weight = (torch.randn(k, c, r, s, device="cuda") * 0.1).half()
+        p_out, q_out = h + 2 * pad[0] - r + 1, w + 2 * pad[1] - s + 1
+        count = n * k * p_out * q_out
+        guard = torch.full((count + 64,), 7.0, dtype=torch.float16, device="cuda")
+        out = guard[:count].view(n, k, p_out, q_out)
+        out.fill_(float("nan"))
+        kernel(x, weight, out, padding_h=pad[0], padding_w=pad[1])
+        expected = F.conv2d(x.float(), weight.float(), padding=pad)
+        description = (case, n, c, h, w, k, r, s, pad)
+        assert torch.allclose(out.float(), expected, rtol=1e-2, atol=1e-2), description
+        assert bool((guard[count:] == 7.0).all()), description
+
+
+def test_attention_on_random_shapes():
+    """40 seeded random problems: head dimensions that are any multiple of 8 up to 256, query and key
+    lengths from 1 to a few thousand (few or many groups, so with and without a split key range),
+    causal where the lengths agree, fp16 and bf16, strided layouts."""
+    import random
+
+    rng = random.Random(4242)
+    kernel = ninetoothed.make(programs.attention.arrangement_with_scale, programs.attention.application_with_scale, programs.attention.tensors(True))
+    for case in range(40):
+        batch, heads = rng.choice((1, 1, 2, 5)), rng.choice((1, 2, 3, 16))
+        emb_dim = rng.choice((8, 32, 40, 64, 64, 96, 128, 128, 160, 256))
+        seq_k = rng.choice((1, 17, 64, 200, 513, 1024, 3000, 6000))
+        seq_q = seq_k if rng.random() < 0.5 else rng.choice((1, 5, 130, 700))
+        is_causal = seq_q == seq_k and rng.random() < 0.5
+        dtype = rng.choice((torch.float16, torch.bfloat16))
+        packed = rng.random() < 0.3  # [batch, seq, heads, dim] storage viewed as [batch, heads, seq, dim]
+
+        def tensor(seq):
+            if packed:
+                return (torch.randn(batch, seq, heads, emb_dim, device="cuda") * 0.5).to(dtype).permute(0, 2, 1, 3)
+            return (torch.randn(batch, heads, seq, emb_dim, device="cuda") * 0.5).to(dtype)
+
+        q, k, v = tensor(seq_q), tensor(seq_k), tensor(seq_k)
+        o = torch.full((batch, heads, seq_q, emb_dim), float("nan"), dtype=dtype, device="cuda")
+        scale = emb_dim**-0.5
+        kernel(q, k, v, is_causal, scale, o)
+        scores = (q.float() * scale) @ k.float().transpose(-1, -2)
+        if is_causal:
+            scores = scores.masked_fill(~torch.ones(seq_q, seq_k, dtype=torch.bool, device="cuda").tril(), float("-inf"))
+        expected = torch.softmax(scores, dim=-1) @ v.float()
+        tolerance = 1e-2 if dtype == torch.float16 else 3e-2
+        assert torch.allclose(o.float(), expected, rtol=tolerance, atol=tolerance), (case, batch, heads, seq_q, seq_k, emb_dim, is_causal, dtype, packed)
