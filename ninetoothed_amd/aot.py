@@ -193,6 +193,7 @@ class MapPackage:
         self.parameters = list(kernel.parameters)
         self.declared = []       # (parameter, dimension, size) fixed by the tensors' declarations
         self.scalar_dtypes = {}  # parameter position -> element type of a call-time scalar
+        self.ranks = [tensor.source.ndim for tensor in kernel.types]
         env, tags, sample_args = {}, {}, []
         # a dimension some tensor declares is the sample for the undeclared ones at the same place
         # (counted from the innermost), so that tensors of one shape stay of one shape
@@ -259,6 +260,8 @@ class MapPackage:
 
         if any(shapes[parameter][dim] != size for parameter, dim, size in self.declared):
             return None
+        if any(size == 0 for shape in shapes.values() for size in shape):
+            return []  # an empty tensor: nothing to launch, like the launch-time path
         symbols = {}
         for parameter, shape in shapes.items():
             for dim, size in enumerate(shape):
@@ -289,6 +292,13 @@ class MapPackage:
             body.append("/* sizes the tensors were declared with */")
             checks = " || ".join(f"{parameter}.shape[{dim}] != {size}ULL" for parameter, dim, size in self.declared)
             body.append(f"if ({checks})\n        return 1;")
+        empty = " || ".join(
+            f"{parameter}.shape[{dim}] == 0" for position, parameter in enumerate(parameters) if position not in self.scalar_dtypes
+            for dim in range(self.ranks[position])
+        )
+        if empty:
+            body.append("/* an empty tensor: nothing to launch */")
+            body.append(f"if ({empty})\n        return 0;")
         if self.guards:
             body.append("/* decisions the lowering took on its sample sizes: the programs below hold for calls that repeat them */")
         for key, outcome in self.guards.items():
