@@ -406,42 +406,12 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     // global stores (and addmm input loads) are 16 bytes per lane and cover
     // whole 128-byte lines.  (All fills have landed and all waves are done with
     // the stages before the slabs overwrite them.)
-    if constexpr (kFloatOut) {
-        // fp32 output (matmul only): a lane's four registers of one r4 group are four consecutive
-        // columns of its row, i.e. one 16-byte store; the two halves of a wave complete 32 bytes
-        // and the four groups a 128-byte line, which the L2 merges
-        static_assert(!kAddmm, "the fp32 output path has no addmm epilogue");
-        wait_vmcnt<0>();
-        float *C32 = (float *)p.c + (kSplit ? (int64_t)part * p.m * p.ldc : batch * p.c_batch);
-#pragma unroll
-        for (int ti = 0; ti < TM; ++ti) {
-            const int grow = m0 + wave_m * kWaveM + ti * 32 + l32;
-            if (grow >= p.m) continue;
-#pragma unroll
-            for (int tj = 0; tj < TN; ++tj)
-#pragma unroll
-                for (int r4 = 0; r4 < 4; ++r4) {
-                    typedef float float4_t __attribute__((ext_vector_type(4)));
-                    float4_t v;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] = acc[ti][tj][4 * r4 + e];
-                    const int gcol = n0 + wave_n * kWaveN + tj * 32 + 8 * r4 + 4 * g;
-                    if (kTail && gcol >= p.n) continue;  // a partial last tile of columns
-                    if (kTail && !p.c_vector) {  // N or the row pitch of C no multiple of 4: element by element
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (gcol + e < p.n) C32[(int64_t)grow * p.ldc + gcol + e] = v[e];
-                        continue;
-                    }
-                    // a plain store: the 32-byte pieces of a line arrive from four instructions and merge in L2
-                    // (as non-temporal stores they cost 20-60 %: 4096^3 156 us against 127)
-                    *(float4_t *)(C32 + (int64_t)grow * p.ldc + gcol) = v;
-                }
-        }
-        return;
-    }
-    constexpr int kRowBytes = kWaveN * 2;
-    constexpr int kCChunks = kWaveN / 8;  // 16-byte chunks per slab row
+    // (fp32 output, matmul and split-K parts only, takes the same route with rows twice as long.)
+    static_assert(!(kFloatOut && kAddmm), "the fp32 output path has no addmm epilogue");
+    using TOut = std::conditional_t<kFloatOut, float, T>;
+    constexpr int kChunkElems = 16 / (int)sizeof(TOut);
+    constexpr int kRowBytes = kWaveN * (int)sizeof(TOut);
+    constexpr int kCChunks = kRowBytes / 16;  // 16-byte chunks per slab row
     constexpr int kCShift = kRowBytes >= 256 ? 0 : (kRowBytes == 128 ? 1 : 2);
     // the slabs live in the (now idle) stage memory: A0, B0, A1, B1 in this order
     constexpr int kSlabBytes = 32 * kRowBytes;
@@ -465,8 +435,9 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         }
         slab += w * kSlabBytes;
     }
-    T *C = (T *)p.c + batch * p.c_batch;
+    TOut *C = (TOut *)p.c + (kSplit ? (int64_t)part * p.m * p.ldc : batch * p.c_batch);
     const T *bias = (const T *)p.bias + batch * p.bias_batch;
+    typedef TOut vec_out __attribute__((ext_vector_type(kChunkElems)));
     const int slab_sw = (l32 >> kCShift) & (kCChunks - 1);
 #pragma unroll
     for (int ti = 0; ti < TM; ++ti) {
@@ -474,12 +445,19 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         for (int tj = 0; tj < TN; ++tj) {
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
-                typedef T vec4 __attribute__((ext_vector_type(4)));
+                typedef TOut vec4 __attribute__((ext_vector_type(4)));
                 vec4 v;
+                if constexpr (kFloatOut) {  // four columns are one chunk
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = E::from_float(acc[ti][tj][4 * r4 + e]);
-                const int chunk = (tj * 4 + r4) ^ slab_sw;
-                *(NT_LDS vec4 *)(slab + l32 * kRowBytes + chunk * 16 + 8 * g) = v;
+                    for (int e = 0; e < 4; ++e) v[e] = acc[ti][tj][4 * r4 + e];
+                    const int chunk = (2 * (tj * 4 + r4) + g) ^ slab_sw;
+                    *(NT_LDS vec4 *)(slab + l32 * kRowBytes + chunk * 16) = v;
+                } else {  // ... half a chunk
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = E::from_float(acc[ti][tj][4 * r4 + e]);
+                    const int chunk = (tj * 4 + r4) ^ slab_sw;
+                    *(NT_LDS vec4 *)(slab + l32 * kRowBytes + chunk * 16 + 8 * g) = v;
+                }
             }
         }
 #pragma unroll
@@ -488,11 +466,11 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
             const int row = idx / kCChunks;
             const int phys = idx % kCChunks;
             const int chunk = phys ^ ((row >> kCShift) & (kCChunks - 1));
-            vec8 v = *(const NT_LDS vec8 *)(slab + row * kRowBytes + phys * 16);
+            vec_out v = *(const NT_LDS vec_out *)(slab + row * kRowBytes + phys * 16);
             const int grow = m0 + wave_m * kWaveM + ti * 32 + row;
-            const int gcol = n0 + wave_n * kWaveN + chunk * 8;
+            const int gcol = n0 + wave_n * kWaveN + chunk * kChunkElems;
             if (grow >= p.m) continue;  // a partial last tile of rows
-            if (kTail && gcol >= p.n) continue;  // ... of columns (whole chunks: N is a multiple of 8)
+            if (kTail && gcol >= p.n) continue;  // ... of columns (with vector stores N is a multiple of 8: whole chunks)
             if constexpr (kAddmm) {
                 // the matmul result was rounded to the element type; beta, alpha
                 // are fp32 scalars, so the combination happens in fp32
@@ -509,13 +487,13 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
             }
             if (kTail && !p.c_vector) {  // N or the row pitch of C no multiple of 8: element by element
 #pragma unroll
-                for (int e = 0; e < 8; ++e)
+                for (int e = 0; e < kChunkElems; ++e)
                     if (gcol + e < p.n) C[(int64_t)grow * p.ldc + gcol + e] = v[e];
                 continue;
             }
             // non-temporal: C is not read again, and its lines then do not displace A / B panels in L2
             // (4096^3 addmm +3 %, 8192^3 +0.3 %)
-            __builtin_nontemporal_store(v, (vec8 *)(C + (int64_t)grow * p.ldc + gcol));
+            __builtin_nontemporal_store(v, (vec_out *)(C + (int64_t)grow * p.ldc + gcol));
         }
     }
 #endif
