@@ -134,7 +134,8 @@ int split_parts(const GemmProblem &q, int bm, int bn, int bk, int *kt_per_part) 
     const int64_t tiles = (int64_t)((q.m + bm - 1) / bm) * ((q.n + bn - 1) / bn);
     const int num_kt = (q.k + bk - 1) / bk;
     if (tiles >= 320) return 1;  // (the untuned choice only splits below 192 tiles; between, the tuner decides)
-    int64_t parts = (512 + tiles - 1) / tiles;                    // about two workgroups per CU
+    // about two workgroups per CU; of 256 x 256 tiles a CU holds one, so there all of them should run at once
+    int64_t parts = bm * bn >= 256 * 256 ? 256 / tiles : (512 + tiles - 1) / tiles;
     parts = std::min<int64_t>(parts, num_kt / 2);                  // at least two k tiles each
     parts = std::min<int64_t>(parts, 256);
     while (parts >= 2 && parts * q.m * q.n * 4 > (int64_t(64) << 20)) --parts;  // scratch of at most 64 MiB
@@ -305,6 +306,7 @@ hipError_t generic_launch(const GemmProblem &q, hipStream_t stream) {
 enum InstanceIndex {
     kAnyStride, k256x256x32, k256x256x64, k128x128x64, k64x64x64, k128x256x32,
     kTail256x256x32, kTail128x256x32, kTail128x128x64, kTail64x64x64, kSplit64x64x64, kSplit128x128x64,
+    kSplit128x256x32, kSplit256x256x32,
 };
 
 const GemmInstance kInstances[] = {
@@ -320,6 +322,8 @@ const GemmInstance kInstances[] = {
     NT_TAIL_INSTANCE(64, 64, 64, 2, 2, 4, 2),
     NT_SPLIT_INSTANCE(64, 64, 64, 2, 2, 4, 2),
     NT_SPLIT_INSTANCE(128, 128, 64, 2, 2, 2, 2),
+    NT_SPLIT_INSTANCE(128, 256, 32, 1, 4, 3, 2),  // a few hundred rows against a wide rhs: 64 to 160 large tiles
+    NT_SPLIT_INSTANCE(256, 256, 32, 2, 4, 5, 2),
 #ifdef NT_GEMM_ABLATION
 #define NT_LOAD_INSTANCE(BM, BN, BK, WM, WN, ST, OCC, LD, AUX) \
     {#BM "x" #BN "x" #BK " waves " #WM "x" #WN " stages " #ST " load " #LD " aux " #AUX, BM, BN, BK, fast_accepts<BM, BN, BK, ST>, fast_launch<BM, BN, BK, WM, WN, ST, OCC, 0, LD, AUX>}
@@ -338,7 +342,9 @@ const GemmInstance kInstances[] = {
 #endif
 };
 constexpr int kNumInstances = sizeof(kInstances) / sizeof(kInstances[0]);
-static_assert(kNumInstances > kSplit128x128x64, "InstanceIndex names the first instances of the table");
+static_assert(kNumInstances > kSplit256x256x32, "InstanceIndex names the first instances of the table");
+
+inline bool is_split(int instance) { return instance >= kSplit64x64x64 && instance <= kSplit256x256x32; }
 
 // ---- per-device cache of tuned choices (device, problem signature) -> instance ----
 struct TuneKey {
@@ -462,7 +468,7 @@ int run_gemm(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk) {
     if (choice < 0 || !kInstances[choice].accepts(q)) choice = heuristic_choice(q, bm, bn, bk);
     if (choice < 0) return NINETOOTHED_NO_KERNEL;
     int result = (int)kInstances[choice].launch(q, stream);
-    if (result == NINETOOTHED_NO_KERNEL && (choice == kSplit64x64x64 || choice == kSplit128x128x64)) {  // a split-K instance without scratch memory
+    if (result == NINETOOTHED_NO_KERNEL && is_split(choice)) {  // a split-K instance without scratch memory
         for (int fallback : {(int)kTail64x64x64, (int)kTail128x128x64, (int)kTail256x256x32, (int)kAnyStride})
             if (kInstances[fallback].accepts(q)) return (int)kInstances[fallback].launch(q, stream);
     }
@@ -700,7 +706,7 @@ NineToothedResult launch_nt_conv2d(NineToothedStream stream, NineToothedTensor i
             q.b_batch = input.strides[0];
             q.c_batch = output.strides[0];
             const int choice = heuristic_choice(q, 0, 0, 0);
-            if (choice > kAnyStride && choice != kSplit64x64x64 && choice != kSplit128x128x64) return (int)kInstances[choice].launch(q, (hipStream_t)stream);
+            if (choice > kAnyStride && !is_split(choice)) return (int)kInstances[choice].launch(q, (hipStream_t)stream);
         }
         const int fast = block_size_m == 1 ? NINETOOTHED_NO_KERNEL : conv2d_fast(request, (hipStream_t)stream);
         if (fast != NINETOOTHED_NO_KERNEL) return fast;

@@ -869,7 +869,7 @@ def test_gemm_transposed_rhs_any_number_of_columns(m, n, k, dtype):
 
 
 @pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
-@pytest.mark.parametrize("m, n, k", ((1, 2048, 4096), (16, 1024, 8192), (64, 520, 2056), (300, 200, 4104), (512, 512, 16384), (129, 136, 256)))
+@pytest.mark.parametrize("m, n, k", ((1, 2048, 4096), (16, 1024, 8192), (64, 520, 2056), (300, 200, 4104), (512, 512, 16384), (129, 136, 256), (768, 1032, 4096)))
 def test_gemm_split_k(m, n, k, dtype):
     """Few output tiles, long K: the k range is cut into parts that run as workgroups of their own
     and a second kernel sums them (fp32) and applies the epilogue.  Both rhs layouts, element-type /
