@@ -582,6 +582,21 @@ long long segment_offset_at(const NineToothedMapProgram &q, int segment, const l
 // row-major matrix) run with one wave per output element: the lanes stride the reduced positions, so
 // a wave reads consecutive elements, and combine their partial results with shuffles.  With one thread
 // per output the lanes of a wave would read a row each.  Returns the lanes per output element: 64 or 1.
+int cooperative_lanes(const NineToothedMapProgram &q);
+
+// Threads of a workgroup.  In tile mode (one workgroup per tile) a tile of up to 16384 elements gets enough
+// threads that each holds at most 16 elements, preferably 8, which the generated code then keeps in registers
+// (layer norm over 4096 rows of fp32, 256 threads -> this choice: 4096 wide 38 -> 27 us, 8192 wide 83 -> 54,
+// 16384 wide 168 -> 119; 1024 threads on 8192 columns: the same for the norms, softmax 64 us against 46).
+int workgroup_threads(const NineToothedMapProgram &q) {
+    if (q.num_phases == 0) return kMapThreads;
+    long long tile_elements = 1;
+    for (int v = q.num_grid; v < q.num_vars; ++v) tile_elements *= (long long)q.extents[v];
+    if (tile_elements > 2048 && tile_elements <= 8192) return 512;
+    if (tile_elements > 8192 && tile_elements <= 16384) return 1024;
+    return kMapThreads;
+}
+
 int cooperative_lanes(const NineToothedMapProgram &q) {
     const int num_out = q.num_vars - q.num_reduced;
     if (q.num_phases != 0 || q.reduce_op == NT_MAP_REDUCE_NONE || q.num_dynamic != 0 || q.num_reduced == 0 || q.store_op != NT_MAP_STORE_ASSIGN) return 1;
@@ -618,6 +633,7 @@ struct MapCodegen {
 
     bool narrow;  // index arithmetic in 32 bits: every index value provably fits
     int lanes;    // lanes per output element (cooperative_lanes)
+    int threads;  // of a workgroup (workgroup_threads)
     // Tile mode with small tiles: a thread's elements stay in registers between the phases.
     // `kept` lists the operands whose loaded values an earlier phase left in `ld<slot>[e]`,
     // `in_body` maps operands already loaded in the loop body being emitted to their temporaries.
@@ -630,7 +646,7 @@ struct MapCodegen {
     std::vector<bool> kept = std::vector<bool>(NT_MAP_MAX_OPERANDS, false);
     std::map<int, std::string> in_body;
 
-    explicit MapCodegen(const NineToothedMapProgram &program) : p(program), narrow(fits_int32(program)), lanes(cooperative_lanes(program)) {}
+    explicit MapCodegen(const NineToothedMapProgram &program) : p(program), narrow(fits_int32(program)), lanes(cooperative_lanes(program)), threads(workgroup_threads(program)) {}
 
     std::string fresh(const char *prefix) { return prefix + std::to_string(counter++); }
 
@@ -847,10 +863,10 @@ struct MapCodegen {
         if (keep_loads) {
             out << pad << "#pragma unroll\n"
                 << pad << "for (int e = 0; e < " << per_thread << "; ++e) {\n"
-                << pad << "    const nt_idx element = (nt_idx)threadIdx.x + e * " << kMapThreads << ";\n"
+                << pad << "    const nt_idx element = (nt_idx)threadIdx.x + e * " << threads << ";\n"
                 << pad << "    if (element >= " << lit(tile_elements) << ") break;\n";
         } else {
-            out << pad << "for (nt_idx element = threadIdx.x; element < " << lit(tile_elements) << "; element += " << kMapThreads << ") {\n";
+            out << pad << "for (nt_idx element = threadIdx.x; element < " << lit(tile_elements) << "; element += " << threads << ") {\n";
         }
         in_body.clear();
     }
@@ -867,10 +883,10 @@ struct MapCodegen {
         for (int v = 0; v < p.num_vars; ++v) (v < p.num_grid ? tiles : tile_elements) *= (long long)p.extents[v];
         // up to 16 elements per thread: every operand is read from memory once and kept in registers
         // (4096 rows of fp32: softmax(2x) 1024 wide 13 us against 16, 2048 wide 20 against 27, 4096 wide 33
-        // against 42; 32 per thread spills: 8192 wide rms norm 97 us against 62)
-        const int per_thread = (int)((tile_elements + kMapThreads - 1) / kMapThreads);
-        keep_loads = tile_elements <= (long long)kMapThreads * 16;
-        out << "    __shared__ double scratch[" << kMapThreads / 64 << "];\n"
+        // against 42; 32 per thread spills: 8192 wide rms norm 97 us against 62; longer rows get more threads)
+        const int per_thread = (int)((tile_elements + threads - 1) / threads);
+        keep_loads = tile_elements <= (long long)threads * 16;
+        out << "    __shared__ double scratch[" << threads / 64 << "];\n"
             << "    for (nt_idx tile = (nt_idx)blockIdx.x; tile < " << lit(tiles) << "; tile += (nt_idx)gridDim.x) {\n"
             << "        nt_uidx tile_rest = (nt_uidx)tile;\n";
         for (int v = p.num_grid - 1; v >= 0; --v)
@@ -895,7 +911,7 @@ struct MapCodegen {
                 << combine_expr(op, dtype, "acc", "other") << "; }\n"
                 << "            __syncthreads();\n            if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = acc;\n            __syncthreads();\n"
                 << "            acc = scratch[0];\n"
-                << "            for (int w = 1; w < " << kMapThreads / 64 << "; ++w) { const double other = scratch[w]; acc = " << combine_expr(op, dtype, "acc", "other")
+                << "            for (int w = 1; w < " << threads / 64 << "; ++w) { const double other = scratch[w]; acc = " << combine_expr(op, dtype, "acc", "other")
                 << "; }\n            r" << k << " = acc;\n        }\n";
             begin = p.phase_end[k];
         }
@@ -932,7 +948,7 @@ struct MapCodegen {
             << "    int x = (int)c0; if (x < 0) x = -x - 1;\n"
             << "    return (double)((float)x * 4.6566127342e-10f);\n"
             << "}\n"
-            << "extern \"C\" __global__ __launch_bounds__(" << kMapThreads << ") void nt_map_specialised(const MapJitArgs a) {\n"
+            << "extern \"C\" __global__ __launch_bounds__(" << threads << ") void nt_map_specialised(const MapJitArgs a) {\n"
             << "    const nt_idx stride = (nt_idx)gridDim.x * " << kMapThreads << ";\n"
             << "    const nt_idx total_out = (nt_idx)a.total_out;\n";
         if (p.num_phases > 0) return generate_tile();
@@ -1124,7 +1140,7 @@ extern "C" NineToothedResult launch_nt_map(NineToothedStream stream, const NineT
             args.total_out = total_out;
             size_t size = sizeof(args);
             void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
-            return (int)hipModuleLaunchKernel(function, (unsigned)blocks, 1, 1, kMapThreads, 1, 1, 0, (hipStream_t)stream, nullptr, config);
+            return (int)hipModuleLaunchKernel(function, (unsigned)blocks, 1, 1, (unsigned)workgroup_threads(p), 1, 1, 0, (hipStream_t)stream, nullptr, config);
         }
     }
     if (p.num_phases > 0)
