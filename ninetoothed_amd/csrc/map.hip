@@ -597,6 +597,14 @@ int workgroup_threads(const NineToothedMapProgram &q) {
     return kMapThreads;
 }
 
+// Threads that share a tile in tile mode: a wave for tiles of up to 512 elements (a workgroup then holds four
+// tiles and the reductions need no LDS exchange and no barrier), else the whole workgroup.
+int tile_group(const NineToothedMapProgram &q) {
+    long long tile_elements = 1;
+    for (int v = q.num_grid; v < q.num_vars; ++v) tile_elements *= (long long)q.extents[v];
+    return q.num_phases > 0 && tile_elements <= 512 ? 64 : workgroup_threads(q);
+}
+
 int cooperative_lanes(const NineToothedMapProgram &q) {
     const int num_out = q.num_vars - q.num_reduced;
     if (q.num_phases != 0 || q.reduce_op == NT_MAP_REDUCE_NONE || q.num_dynamic != 0 || q.num_reduced == 0 || q.store_op != NT_MAP_STORE_ASSIGN) return 1;
@@ -634,6 +642,7 @@ struct MapCodegen {
     bool narrow;  // index arithmetic in 32 bits: every index value provably fits
     int lanes;    // lanes per output element (cooperative_lanes)
     int threads;  // of a workgroup (workgroup_threads)
+    int group;    // threads that share a tile in tile mode (tile_group)
     // Tile mode with small tiles: a thread's elements stay in registers between the phases.
     // `kept` lists the operands whose loaded values an earlier phase left in `ld<slot>[e]`,
     // `in_body` maps operands already loaded in the loop body being emitted to their temporaries.
@@ -646,7 +655,7 @@ struct MapCodegen {
     std::vector<bool> kept = std::vector<bool>(NT_MAP_MAX_OPERANDS, false);
     std::map<int, std::string> in_body;
 
-    explicit MapCodegen(const NineToothedMapProgram &program) : p(program), narrow(fits_int32(program)), lanes(cooperative_lanes(program)), threads(workgroup_threads(program)) {}
+    explicit MapCodegen(const NineToothedMapProgram &program) : p(program), narrow(fits_int32(program)), lanes(cooperative_lanes(program)), threads(workgroup_threads(program)), group(tile_group(program)) {}
 
     std::string fresh(const char *prefix) { return prefix + std::to_string(counter++); }
 
@@ -863,10 +872,10 @@ struct MapCodegen {
         if (keep_loads) {
             out << pad << "#pragma unroll\n"
                 << pad << "for (int e = 0; e < " << per_thread << "; ++e) {\n"
-                << pad << "    const nt_idx element = (nt_idx)threadIdx.x + e * " << threads << ";\n"
+                << pad << "    const nt_idx element = member + e * " << group << ";\n"
                 << pad << "    if (element >= " << lit(tile_elements) << ") break;\n";
         } else {
-            out << pad << "for (nt_idx element = threadIdx.x; element < " << lit(tile_elements) << "; element += " << threads << ") {\n";
+            out << pad << "for (nt_idx element = member; element < " << lit(tile_elements) << "; element += " << group << ") {\n";
         }
         in_body.clear();
     }
@@ -884,10 +893,17 @@ struct MapCodegen {
         // up to 16 elements per thread: every operand is read from memory once and kept in registers
         // (4096 rows of fp32: softmax(2x) 1024 wide 13 us against 16, 2048 wide 20 against 27, 4096 wide 33
         // against 42; 32 per thread spills: 8192 wide rms norm 97 us against 62; longer rows get more threads)
-        const int per_thread = (int)((tile_elements + threads - 1) / threads);
-        keep_loads = tile_elements <= (long long)threads * 16;
-        out << "    __shared__ double scratch[" << threads / 64 << "];\n"
-            << "    for (nt_idx tile = (nt_idx)blockIdx.x; tile < " << lit(tiles) << "; tile += (nt_idx)gridDim.x) {\n"
+        const int per_thread = (int)((tile_elements + group - 1) / group);
+        keep_loads = tile_elements <= (long long)group * 16;
+        const bool wave_tiles = group == 64 && threads > 64;  // a wave per tile: no exchange through LDS
+        if (wave_tiles)
+            out << "    const nt_idx member = threadIdx.x & 63;\n"
+                << "    for (nt_idx tile = (nt_idx)blockIdx.x * " << threads / 64 << " + (threadIdx.x >> 6); tile < " << lit(tiles) << "; tile += (nt_idx)gridDim.x * " << threads / 64 << ") {\n";
+        else
+            out << "    __shared__ double scratch[" << threads / 64 << "];\n"
+                << "    const nt_idx member = threadIdx.x;\n"
+                << "    for (nt_idx tile = (nt_idx)blockIdx.x; tile < " << lit(tiles) << "; tile += (nt_idx)gridDim.x) {\n";
+        out
             << "        nt_uidx tile_rest = (nt_uidx)tile;\n";
         for (int v = p.num_grid - 1; v >= 0; --v)
             out << "        const nt_idx v" << v << " = (nt_idx)(tile_rest % " << ulit((long long)p.extents[v]) << "); tile_rest /= " << ulit((long long)p.extents[v]) << ";\n";
@@ -908,8 +924,13 @@ struct MapCodegen {
             out << indent << "acc = " << combine_expr(op, dtype, "acc", term) << ";\n";
             close_element_loop("            ");
             out << "            for (int offset = 32; offset > 0; offset >>= 1) { const double other = __shfl_xor(acc, offset, 64); acc = "
-                << combine_expr(op, dtype, "acc", "other") << "; }\n"
-                << "            __syncthreads();\n            if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = acc;\n            __syncthreads();\n"
+                << combine_expr(op, dtype, "acc", "other") << "; }\n";
+            if (wave_tiles) {
+                out << "            r" << k << " = acc;\n        }\n";
+                begin = p.phase_end[k];
+                continue;
+            }
+            out << "            __syncthreads();\n            if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = acc;\n            __syncthreads();\n"
                 << "            acc = scratch[0];\n"
                 << "            for (int w = 1; w < " << threads / 64 << "; ++w) { const double other = scratch[w]; acc = " << combine_expr(op, dtype, "acc", "other")
                 << "; }\n            r" << k << " = acc;\n        }\n";
@@ -1126,7 +1147,9 @@ extern "C" NineToothedResult launch_nt_map(NineToothedStream stream, const NineT
     int64_t tiles = 1, tile_elements = 1;
     if (p.num_phases > 0) {  // tile mode: one workgroup per tile
         for (int v = 0; v < p.num_vars; ++v) (v < p.num_grid ? tiles : tile_elements) *= p.extents[v];
-        blocks = tiles < 256 * 32 ? tiles : 256 * 32;
+        const int64_t tiles_per_block = tile_group(p) == 64 ? workgroup_threads(p) / 64 : 1;  // (only the generated kernel shares a workgroup)
+        blocks = (tiles + tiles_per_block - 1) / tiles_per_block;
+        if (blocks > 256 * 32) blocks = 256 * 32;
     }
     const char *interpret = getenv("NT_MAP_INTERPRET");
     if (!(interpret && interpret[0] == '1')) {

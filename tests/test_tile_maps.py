@@ -831,8 +831,9 @@ def test_tile_mode_program_layout():
 @pytest.mark.parametrize("dtype, tolerance", ((torch.float32, 1e-5), (torch.float16, 1e-2)))
 def test_whole_tile_reductions_on_the_gpu(dtype, tolerance, interpret, monkeypatch):
     monkeypatch.setenv("NT_MAP_INTERPRET", interpret)
-    # (rows of 2049 ... 8192 elements run 512 threads per row, up to 16384 1024 threads, longer ones 256 again)
-    for rows, cols in ((7, 300), (64, 4096), (3, 1), (5, 2049), (33, 8192), (9, 8200), (17, 16384), (3, 20000)):
+    # (rows of up to 512 elements take a wave each, four to a workgroup; rows of 2049 ... 8192 elements run
+    # 512 threads per row, up to 16384 1024 threads, longer ones 256 again)
+    for rows, cols in ((7, 300), (64, 4096), (3, 1), (1001, 32), (77, 512), (6, 513), (5, 2049), (33, 8192), (9, 8200), (17, 16384), (3, 20000)):
         for kernel, inputs, expected in _normalisation_cases("cuda", dtype, rows, cols):
             out = torch.full_like(inputs[0], float("nan"))
             kernel(*inputs, out)
