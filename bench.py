@@ -14,7 +14,9 @@ Prints ONE JSON line.  ``roofline.achieved`` = algorithmic FLOP (or bytes) per
 launch / average launch time from device events on the launch stream.
 ``cpu_baseline`` times the CPU oracle (oracle/programs.py, single thread) on a
 bounded sample of the same workload; ``torch_cpu`` times the stock torch CPU
-operator of every configuration (all host threads, bounded samples).  ``vendor_gpu`` times the stock PyTorch
+operator of every configuration (all host threads, bounded samples);
+``triton_interpreter_cpu`` times the 512^3 matmul as the reference runs on a CPU: a Triton kernel
+under ``TRITON_INTERPRET=1`` (one thread).  ``vendor_gpu`` times the stock PyTorch
 operator of each workload (hipBLASLt / MIOpen / the built-in SDPA) on the same
 GPU and inputs, for context only.
 
@@ -214,6 +216,29 @@ def cpu_baseline_addmm():
     }
 
 
+def triton_interpreter_cpu():
+    """The reference's CPU path for the 512^3 matmul: a Triton kernel with the structure of the one the
+    reference generates, run by Triton's interpreter (oracle/triton_cpu_matmul.py), in a process of its
+    own because the interpreter switch has to be set before Triton is imported.  The child uses CPU
+    tensors only."""
+    import subprocess
+
+    root = os.path.dirname(os.path.abspath(__file__))
+    env = dict(os.environ, TRITON_INTERPRET="1")
+    try:
+        done = subprocess.run([sys.executable, "-m", "oracle.triton_cpu_matmul", "512"], cwd=root, env=env, capture_output=True, text=True, timeout=600)
+        lines = [line for line in done.stdout.splitlines() if line.startswith("{")]
+        if done.returncode != 0 or not lines:
+            return {"error": (done.stderr or done.stdout).strip().splitlines()[-1][:200] if (done.stderr or done.stdout).strip() else f"exit code {done.returncode}"}
+        result = json.loads(lines[-1])
+    except Exception as error:
+        return {"error": str(error)[:200]}
+    if "error" not in result:
+        result["kind"] = "own Triton kernel of the reference's structure under TRITON_INTERPRET=1"
+        result["workload"] = "matmul fp16 M=N=K=512"
+    return result
+
+
 def torch_cpu_context():
     """The stock torch CPU operator of each configuration on the host, all threads,
     one warm-up and the median of three runs, on bounded samples (context only)."""
@@ -344,6 +369,7 @@ def main():
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline_addmm()
         result["torch_cpu"] = torch_cpu_context()
+        result["triton_interpreter_cpu"] = triton_interpreter_cpu()
     print(json.dumps(result))
 
 

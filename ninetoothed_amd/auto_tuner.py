@@ -60,12 +60,15 @@ def lookup(dtype, out_dtype, m, n, k, addmm):
 
 def tune(input, mat1, mat2, beta, alpha, output, dtype, out_dtype, iters=5):
     """Times the instances on these arguments (:class:`runtime.ArgumentTensor`), records the
-    winner in the library and on disk.  Returns ``(instance, milliseconds)``."""
+    winner in the library and on disk.  Returns ``(instance, milliseconds)``; the instance is -1
+    when the stream is being captured into a graph (nothing is timed or recorded then)."""
     lib = runtime.library()
     best, best_ms = ctypes.c_int(-1), ctypes.c_float(0.0)
     runtime.check(
         lib.nt_tune_gemm(runtime.current_stream(), input, mat1, mat2, beta, alpha, output, dtype, out_dtype, iters, ctypes.byref(best), ctypes.byref(best_ms))
     )
+    if best.value < 0:  # nothing was timed: the stream is being captured into a graph
+        return best.value, best_ms.value
     try:
         CACHE_DIR.mkdir(parents=True, exist_ok=True)
         lib.nt_tune_cache_save(str(cache_path()).encode())

@@ -782,8 +782,13 @@ extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineT
     p.k = k.data;
     p.v = v.data;
     p.o = o.data;
-    const double scale_value = scale.data ? Scalar0d::as_double(scale) : 1.0;
-    p.q_scale = (float)(scale_value * 1.4426950408889634);
+    // Q' = (Q * factor).to(element type).  Without a `scale` argument the factor is the literal of the
+    // reference program, `q * 1.44269504089` (tests/test_attention.py:46): a tile times a Python literal is
+    // computed in the tile's type with the literal rounded to that type first, and the fp32 product of two
+    // 16-bit floats is exact, so rounding it once is that multiplication.  A run-time `scale` is an fp32
+    // scalar: `q * (scale * 1.44269504089)` is an fp32 product rounded once.
+    if (scale.data) p.q_scale = (float)Scalar0d::as_double(scale) * 1.44269504089f;
+    else p.q_scale = dtype == NINETOOTHED_FLOAT16 ? 1.4423828125f : (dtype == NINETOOTHED_BFLOAT16 ? 1.4453125f : 1.44269504089f);
     p.causal = is_causal.data ? (Scalar0d::as_int64(is_causal) != 0) : 0;
     if (float32) return attention_float32(p, (int)head_dim, k, v, (hipStream_t)stream);
     // block sizes are hints: 256 query rows select the one-workgroup-per-CU

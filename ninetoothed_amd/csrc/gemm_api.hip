@@ -529,6 +529,11 @@ NineToothedResult nt_tune_gemm(NineToothedStream stream_, NineToothedTensor inpu
     GemmProblem q;
     if (int err = build_problem(q, &input, mat1, mat2, &beta, &alpha, output, dtype, output_dtype)) return err;
     if (iters <= 0) iters = 5;
+    if (best_config) *best_config = -1;
+    if (best_ms) *best_ms = 0.0f;
+    // timing needs event synchronisation and rewrites the output several times: not inside a graph
+    // capture.  The problem stays untuned (launches use the fixed preference order) and nothing is recorded.
+    if (stream_is_capturing(stream)) return 0;
     hipEvent_t start, stop;
     hipError_t err;
     if ((err = hipEventCreate(&start)) != hipSuccess) return (int)err;

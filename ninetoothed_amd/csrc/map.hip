@@ -1065,7 +1065,9 @@ struct Hiprtc {
 std::mutex g_jit_mutex;
 std::unordered_map<std::string, hipFunction_t> g_jit_cache;  // a null function = "do not try again"
 
-hipFunction_t specialised_kernel(const NineToothedMapProgram &p) {
+// `may_compile` false (the stream is being captured into a graph: compiling and loading code would break
+// the capture): only a kernel specialised earlier is returned, and a miss is not remembered
+hipFunction_t specialised_kernel(const NineToothedMapProgram &p, bool may_compile) {
     static Hiprtc rtc;
     if (!rtc.ok) return nullptr;
     int device = 0;
@@ -1089,6 +1091,7 @@ hipFunction_t specialised_kernel(const NineToothedMapProgram &p) {
     std::lock_guard<std::mutex> lock(g_jit_mutex);
     auto found = g_jit_cache.find(key);
     if (found != g_jit_cache.end()) return found->second;
+    if (!may_compile) return nullptr;
     MapCodegen generator(p);
     const std::string source = generator.generate();
     hipFunction_t function = nullptr;
@@ -1153,7 +1156,7 @@ extern "C" NineToothedResult launch_nt_map(NineToothedStream stream, const NineT
     }
     const char *interpret = getenv("NT_MAP_INTERPRET");
     if (!(interpret && interpret[0] == '1')) {
-        if (hipFunction_t function = specialised_kernel(p)) {
+        if (hipFunction_t function = specialised_kernel(p, !stream_is_capturing((hipStream_t)stream))) {
             MapJitArgs args;
             for (int i = 0; i < NT_MAP_MAX_OPERANDS; ++i) {
                 args.data[i] = i < p.num_operands ? p.operands[i].data : nullptr;

@@ -99,6 +99,17 @@ NT_DEVICE void wait_lgkmcnt() {
 
 NT_HOST_DEVICE constexpr int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
+// True while `stream` records into a graph (or when that cannot be told): the caller then
+// must not synchronise, time, allocate, or load code, all of which break a capture.
+inline bool stream_is_capturing(hipStream_t stream) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+        (void)hipGetLastError();
+        return true;
+    }
+    return status != hipStreamCaptureStatusNone;
+}
+
 struct Scalar0d {
     static double as_double(const NineToothedTensor &t) { return *(const double *)t.data; }
     static int64_t as_int64(const NineToothedTensor &t) { return *(const int64_t *)t.data; }

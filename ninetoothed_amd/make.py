@@ -326,7 +326,9 @@ class Kernel:
             # timing launches rewrite the output; skip when it overlaps an operand
             if any(t.untyped_storage().data_ptr() == out.untyped_storage().data_ptr() for t in sources):
                 return
-            auto_tuner.tune(input_arg, a_arg, b_arg, beta, alpha, c_arg, dtype, out_dtype)
+            instance, _ = auto_tuner.tune(input_arg, a_arg, b_arg, beta, alpha, c_arg, dtype, out_dtype)
+            # inside a graph capture nothing is timed: the next call outside one tunes
+            state["tune"] = instance < 0
 
         if i is not None:
             i_arg = runtime.ArgumentTensor.from_layout(0, (m, n), (i.row_stride, i.col_stride))  # (a stride of 0 is a broadcast here)

@@ -436,6 +436,9 @@ class Tracer:
                 if isinstance(frame.locals[name], TensorRef):
                     continue  # assignments to tensor parameters are stores
                 carried.append(name)
+        # slots are numbered by what the names hold on entry (ties: first assignment in the body), so that
+        # two bodies with the same dataflow get the same graph whatever the order of their statements
+        carried.sort(key=lambda name: _digest_of(self._value(frame.locals[name])))
         initial = [frame.locals[name] for name in carried]
         for slot, name in enumerate(carried):
             frame.locals[name] = Carried(loop, slot)

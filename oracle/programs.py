@@ -26,7 +26,9 @@ Pinned (tests/test_oracle_programs.py) against the library routines the
 reference's own tests compare with -- ``torch.matmul``, ``torch.addmm``,
 ``torch.softmax``, ``F.scaled_dot_product_attention``, ``F.conv2d`` -- and
 against closed forms (identity matrices, constant rows, one-key attention,
-1x1 convolution == matmul).
+1x1 convolution == matmul).  The typing rules above and ``triton_rand`` are
+pinned by vectors the installed Triton package itself produced under its CPU
+interpreter (tests/golden/make_triton_*_vectors.py).
 """
 
 import numpy as np
@@ -123,9 +125,17 @@ def softmax(x, block_size=None):
     return out.reshape(rows, cols)
 
 
-def attention(q, k, v, is_causal=False, scale=1.0, bm=64, bn=32, dtype="fp16"):
+def attention(q, k, v, is_causal=False, scale=None, bm=64, bn=32, dtype="fp16"):
     """Online-softmax attention forward, q block by q block, k/v block by k/v
-    block (no block is skipped; causal and tail positions are masked to -inf)."""
+    block (no block is skipped; causal and tail positions are masked to -inf).
+
+    ``scale=None`` is the reference program as it stands (tests/test_attention.py:46):
+    ``q * 1.44269504089`` multiplies a tile by a Python literal, which Triton first
+    turns into a constant of the tile's type (fp16: 1.4423828125, bf16: 1.4453125) and
+    then multiplies in that type -- one rounding of the exact product.  With a number,
+    the program is this build's variant with a run-time ``scale`` argument,
+    ``q * (scale * 1.44269504089)``: a run-time scalar is fp32, so the factor and the
+    product are fp32 and ``.to(q.dtype)`` rounds once."""
     batch, heads, seq_q, dim = q.shape
     seq_k = k.shape[2]
 
@@ -142,7 +152,10 @@ def attention(q, k, v, is_causal=False, scale=1.0, bm=64, bn=32, dtype="fp16"):
     v_view = arrange_k_or_v(v.shape, q_view.table.shape[2])
     q_flat, k_flat, v_flat = q.reshape(-1), k.reshape(-1), v.reshape(-1)
     out = np.zeros(q.size, dtype=np.float32)
-    factor = np.float32(scale * LOG2E) if scale != 1.0 else np.float32(LOG2E)
+    if scale is None:
+        factor = _round(np.float32(LOG2E), dtype).astype(np.float32)
+    else:
+        factor = np.float32(scale) * np.float32(LOG2E)
 
     for b in range(batch):
         for h in range(heads):
@@ -253,7 +266,9 @@ def triton_rand(seed, offsets):
     ``(offset_lo, offset_hi, 0, 0)`` keyed by the two halves of ``seed``; the
     first output word, read as int32 and mirrored when negative, times 2^-31
     (the published algorithm of Triton's ``language/random.py``, the package the
-    reference's ``ntl.rand`` resolves to, src/ninetoothed/generation.py:849-855)."""
+    reference's ``ntl.rand`` resolves to, src/ninetoothed/generation.py:849-855).
+    Pinned bit for bit by outputs of the installed Triton's own ``tl.rand`` for 32- and
+    64-bit offsets and seeds up to 2^62 (tests/golden/triton_rand_vectors.json)."""
     offsets = np.asarray(offsets, dtype=np.int64).astype(np.uint64)
     seed = np.uint64(seed)
     mask = np.uint64(0xFFFFFFFF)

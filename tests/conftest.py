@@ -30,3 +30,20 @@ def seed_per_test(request):
     np.random.seed(seed % 2**32)
     torch.manual_seed(seed)
     yield
+
+
+@pytest.fixture(autouse=True, scope="session")
+def caches_in_a_temporary_directory(tmp_path_factory):
+    """Tuned choices and kernel descriptions go to a directory of this test session, not to the
+    home directory: what one run found does not steer the next, and nothing is left behind."""
+    import importlib
+
+    from ninetoothed_amd import auto_tuner
+
+    make = importlib.import_module("ninetoothed_amd.make")  # (the package attribute `make` is the function)
+
+    root = tmp_path_factory.mktemp("ninetoothed_amd_cache")
+    saved = auto_tuner.CACHE_DIR, make.CACHE_DIR
+    auto_tuner.CACHE_DIR, make.CACHE_DIR = root / "auto_tuning", root
+    yield root
+    auto_tuner.CACHE_DIR, make.CACHE_DIR = saved

@@ -381,16 +381,18 @@ def test_attention_other_head_dims(emb_dim, dtype, is_causal):
 
 
 @pytest.mark.parametrize("batch, heads, seq_q, seq_k, emb_dim", ((32, 32, 1, 2048, 128), (8, 32, 128, 8192, 128), (2, 8, 4096, 512, 64), (1, 8, 16, 65536, 128), (3, 5, 77, 1000, 64)))
-def test_attention_with_its_own_key_length(batch, heads, seq_q, seq_k, emb_dim):
-    """Queries against a longer (decoding, cross attention) or shorter key / value sequence."""
+@pytest.mark.parametrize("is_causal", (False, True))
+def test_attention_with_its_own_key_length(batch, heads, seq_q, seq_k, emb_dim, is_causal):
+    """Queries against a longer (decoding, cross attention) or shorter key / value sequence; the
+    causal mask keeps key j for query i when i >= j, counted from the start of both sequences."""
     q = _randn(batch, heads, seq_q, emb_dim).cuda()
     k, v = _randn(batch, heads, seq_k, emb_dim).cuda(), _randn(batch, heads, seq_k, emb_dim).cuda()
     o = torch.full_like(q, float("nan"))
     scale = emb_dim**-0.5
     kernel = ninetoothed.make(programs.attention.arrangement_with_scale, programs.attention.application_with_scale, programs.attention.tensors(True))
-    kernel(q, k, v, False, scale, o)
+    kernel(q, k, v, is_causal, scale, o)
     _native_only(kernel, "launch_nt_attention")
-    assert torch.allclose(o.float(), _attention_reference(q, k, v, False, scale), **HALF_TOL)
+    assert torch.allclose(o.float(), _attention_reference(q, k, v, is_causal, scale), **HALF_TOL)
 
 
 @pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
@@ -399,9 +401,9 @@ def test_attention_with_its_own_key_length(batch, heads, seq_q, seq_k, emb_dim):
 def test_attention_split_key_range(batch, heads, seq_q, seq_k, emb_dim, is_causal, dtype):
     """Few (batch, head, query block) groups and many keys: parts of the key range run as
     workgroups of their own and a second kernel merges them.  With a causal mask, parts past
-    the diagonal have no keys at all.  Twice in a row on the same scratch memory."""
-    if is_causal and seq_q != seq_k:
-        pytest.skip("the causal mask of the program assumes equal lengths")
+    the diagonal have no keys at all (the mask `q.offsets(-2) >= k.offsets(-2)` of the program,
+    reference tests/test_attention.py:55, is aligned top-left whatever the two lengths are).
+    Twice in a row on the same scratch memory."""
     q = _randn(batch, heads, seq_q, emb_dim).cuda().to(dtype)
     k, v = _randn(batch, heads, seq_k, emb_dim).cuda().to(dtype), _randn(batch, heads, seq_k, emb_dim).cuda().to(dtype)
     scale = emb_dim**-0.5
@@ -600,6 +602,60 @@ def test_scratch_buffers_are_reused_grown_and_released():
         assert torch.allclose(o, F.scaled_dot_product_attention(q, k, v, scale=0.125), rtol=0.025, atol=0.025)
         torch.cuda.synchronize()
         runtime.library().nt_release_workspaces()
+
+
+def test_first_call_of_an_untuned_problem_inside_a_captured_graph():
+    """Nothing has run these problems before the capture starts: the first-launch tuner of the product
+    (event synchronisation, repeated launches) and the specialisation of the tile map (compiling and
+    loading code) would both break a capture.  Inside one the product takes the untuned choice and the
+    tile map its interpreter kernel; the first call outside a capture then tunes / specialises."""
+    from ninetoothed_amd import auto_tuner, runtime
+
+    m, n, k = 264, 520, 776  # sizes no other test uses
+    a, b, bias = _randn(m, k).cuda(), _randn(k, n, scale=0.1).cuda(), _randn(m, n).cuda()
+    c, d = torch.empty(m, n, dtype=torch.float16, device="cuda"), torch.empty(m, n, dtype=torch.float16, device="cuda")
+    x, y = torch.randn(1237, device="cuda"), torch.randn(1237, device="cuda")
+    z = torch.empty_like(x)
+    matmul = _matmul_kernel()
+    addmm = ninetoothed.make(programs.addmm.arrangement, programs.addmm.application, programs.addmm.tensors())
+
+    def arrangement(lhs, rhs, output, block=ninetoothed.block_size()):
+        return lhs.tile((block,)), rhs.tile((block,)), output.tile((block,))
+
+    def application(lhs, rhs, output):
+        output = lhs * 3.25 + rhs * rhs - 0.0078125  # noqa: F841
+
+    tile_map = ninetoothed.make(arrangement, application, (Tensor(1),) * 3)
+    fp16 = runtime.DATA_TYPE_INDEX["fp16"]
+    assert auto_tuner.enabled() and auto_tuner.lookup(fp16, fp16, m, n, k, False) < 0 and auto_tuner.lookup(fp16, fp16, m, n, k, True) < 0
+
+    def run():
+        matmul(a, b, c)
+        addmm(bias, a, b, 0.5, 2.0, d)
+        tile_map(x, y, z)
+
+    stream = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        run()
+    assert auto_tuner.lookup(fp16, fp16, m, n, k, False) < 0  # nothing was timed during the capture
+    product = a.float() @ b.float()
+    expected = (product, 0.5 * bias.float() + 2.0 * product.half().float(), x * 3.25 + y * y - 0.0078125)
+    for replay in range(3):
+        for t in (c, d, z):
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.allclose(c.float(), expected[0], **HALF_TOL), replay
+        assert torch.allclose(d.float(), expected[1], rtol=1e-2, atol=2e-2), replay
+        assert torch.allclose(z, expected[2], rtol=1e-6, atol=1e-6), replay
+        if replay == 0:
+            run()  # the first eager call tunes the products and specialises the tile map
+            torch.cuda.synchronize()
+            assert auto_tuner.lookup(fp16, fp16, m, n, k, False) >= 0 and auto_tuner.lookup(fp16, fp16, m, n, k, True) >= 0
+            assert torch.allclose(z, expected[2], rtol=1e-6, atol=1e-6)
 
 
 @pytest.mark.parametrize("warm_on_capture_stream", (False, True))

@@ -42,6 +42,23 @@ def test_addmm_8192_whole_output_and_repeatability(dtype):
             assert torch.equal(out, first)
 
 
+def test_addmm_8192_at_the_stated_input_distribution():
+    """All three operands N(0, 1), alpha = 1.0, beta = 0.5 (the inputs the throughput figure is quoted
+    on): whole output against the program's arithmetic done by torch in fp32 -- product rounded to
+    fp16, combined in fp32, rounded once -- at rtol = atol = 1e-2, and against ``torch.addmm``."""
+    n = 8192
+    input, mat1, mat2 = (_seeded(n, n, seed=seed) for seed in (10, 11, 12))
+    kernel = ninetoothed.make(programs.addmm.arrangement, programs.addmm.application, programs.addmm.tensors())
+    out = torch.full((n, n), float("nan"), dtype=torch.float16, device="cuda")
+    kernel(input, mat1, mat2, 0.5, 1.0, out)
+    assert kernel.last_plan.startswith("launch_nt_addmm")
+    product = (mat1.float() @ mat2.float()).half().float()
+    expected = (0.5 * input.float() + 1.0 * product).half()
+    del product
+    assert torch.allclose(out, expected, **HALF_TOL)
+    assert torch.allclose(out, torch.addmm(input, mat1, mat2, beta=0.5, alpha=1.0), rtol=1e-2, atol=0.075)  # reference tolerance, tests/test_addmm.py:59
+
+
 def test_every_gemm_instance_whole_output():
     lib = runtime.library()
     fp16 = runtime.DATA_TYPE_INDEX["fp16"]

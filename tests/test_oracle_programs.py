@@ -112,3 +112,81 @@ def test_conv2d_1x1_is_matmul():
     a = x.float().permute(0, 2, 3, 1).reshape(-1, 8)
     expected = (a @ w.float().reshape(6, 8).T).to(torch.float16).float().reshape(2, 4, 4, 6).permute(0, 3, 1, 2).numpy()
     assert np.allclose(out, expected, rtol=1e-3, atol=1e-3)
+
+
+# ---- what Triton itself computes (vectors written by tests/golden/make_triton_*_vectors.py) ----
+
+
+def _golden(name):
+    import json
+    import pathlib
+
+    return json.loads((pathlib.Path(__file__).resolve().parent / "golden" / name).read_text())
+
+
+def test_triton_rand_matches_the_vectors_of_the_installed_triton():
+    """``tl.rand`` outputs for int32 and int64 offsets (up to 2^62) and seeds up to 2^62: pins the
+    output word, the placement of the offset's and the seed's halves, the mirroring and the scale."""
+    cases = _golden("triton_rand_vectors.json")["cases"]
+    assert len(cases) >= 18
+    for case in cases:
+        got = oracle.triton_rand(case["seed"], np.array(case["offsets"], dtype=np.int64))
+        assert np.array_equal(got.view(np.int32), np.array(case["bits"], dtype=np.int32)), (case["seed"], case["offset_dtype"])
+
+
+def test_rounding_points_match_the_vectors_of_the_installed_triton():
+    """A tile times a Python literal is computed in the tile's type with the literal rounded to it
+    first; a tile times a run-time scalar in fp32; the addmm epilogue in fp32 on the rounded product."""
+    cases = _golden("triton_promotion_vectors.json")["cases"]
+
+    def half(bits):
+        return np.array(bits, dtype=np.int16).view(np.float16).astype(np.float32)
+
+    literal = cases["literal_fp16"]
+    factor = oracle._round(np.float32(oracle.LOG2E), "fp16").astype(np.float32)
+    assert float(factor) == 1.4423828125
+    got = oracle._round(half(literal["q"]) * factor, "fp16")
+    assert np.array_equal(got.view(np.int16), np.array(literal["out"], dtype=np.int16))
+    unrounded = oracle._round(half(literal["q"]) * np.float32(oracle.LOG2E), "fp16")
+    assert not np.array_equal(unrounded.view(np.int16), np.array(literal["out"], dtype=np.int16))  # the vectors tell the two apart
+
+    scaled = cases["scaled_fp16"]
+    factor = np.float32(scaled["scale"]) * np.float32(oracle.LOG2E)
+    got = oracle._round(half(scaled["q"]) * factor, "fp16")
+    assert np.array_equal(got.view(np.int16), np.array(scaled["out"], dtype=np.int16))
+
+    # the same two rules through the attention restatement itself: one key, so the output is V whatever Q is,
+    # and the factor is visible through a two-key problem solved in closed form below
+    epilogue = cases["addmm_epilogue_fp16"]
+    product = np.array(epilogue["product"], dtype=np.int32).view(np.float32)
+    n = product.size
+    # addmm with K = 1: mat1 = product rounded apart into two fp16 factors is not exact, so check the epilogue rule
+    # on the restatement's own arithmetic: beta * input + alpha * round16(product), in fp32, rounded once
+    rounded = product.astype(np.float16).astype(np.float32)
+    got = (np.float32(epilogue["beta"]) * half(epilogue["input"]) + np.float32(epilogue["alpha"]) * rounded).astype(np.float16)
+    assert np.array_equal(got.view(np.int16), np.array(epilogue["out"], dtype=np.int16))
+    # and the restatement does exactly that: a 1 x n problem whose product is exact in fp16 (powers of two)
+    input = half(epilogue["input"]).astype(np.float16).reshape(1, n)
+    mat1 = np.array([[2.0]], dtype=np.float16)
+    mat2 = np.ldexp(1.0, np.arange(n) % 11 - 5).astype(np.float16).reshape(1, n)
+    out = oracle.addmm(input, mat1, mat2, epilogue["beta"], epilogue["alpha"], bm=1, bn=64, bk=1)
+    expected = (np.float32(epilogue["beta"]) * input.astype(np.float32) + np.float32(epilogue["alpha"]) * (2.0 * mat2.astype(np.float32))).astype(np.float16)
+    assert np.array_equal(out.astype(np.float16).view(np.int16), expected.view(np.int16))
+
+
+def test_attention_literal_factor_is_rounded_to_the_tile_type():
+    """Two keys, one query, head dimension 1: the output weight of key 0 is 1 / (1 + 2^(q' (k1 - k0))) with
+    q' = round16(q * 1.4423828125) for the reference program and round16(q * fp32(scale * log2 e)) with a scale."""
+    candidates = np.arange(4.0, 8.0, 2.0**-8, dtype=np.float32).astype(np.float16)  # every half in [4, 8)
+    differ = np.float16(candidates.astype(np.float32) * np.float32(1.4423828125)) != np.float16(candidates.astype(np.float32) * np.float32(oracle.LOG2E))
+    q = candidates[np.nonzero(differ)[0][:1]].reshape(1, 1, 1, 1)  # the two factors round this one to different halves
+    k = np.array([[[[0.0], [1.0]]]], dtype=np.float16)
+    v = np.array([[[[1.0], [0.0]]]], dtype=np.float16)
+    literal = np.float16(np.float32(q[0, 0, 0, 0]) * np.float32(1.4423828125))
+    full = np.float16(np.float32(q[0, 0, 0, 0]) * np.float32(oracle.LOG2E))
+    assert literal != full
+    out = oracle.attention(q, k, v, bm=1, bn=2)
+    assert np.isclose(out[0, 0, 0, 0], 1.0 / (1.0 + 2.0 ** float(literal)), rtol=1e-3)
+    assert not np.isclose(out[0, 0, 0, 0], 1.0 / (1.0 + 2.0 ** float(full)), rtol=1e-3)
+    scaled = oracle.attention(q, k, v, scale=1.0, bm=1, bn=2)
+    assert np.isclose(scaled[0, 0, 0, 0], 1.0 / (1.0 + 2.0 ** float(full)), rtol=1e-3)
