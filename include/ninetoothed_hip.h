@@ -43,6 +43,11 @@ extern "C" {
 /* returned when no kernel matches the request (dtype / rank / block sizes) */
 #define NINETOOTHED_NO_KERNEL 1
 
+/* returned by launch_nt_matmul_static_scratch when the call would need more scratch memory than the
+ * library's fixed array holds (NINETOOTHED_STATIC_SCRATCH_BYTES); nothing has been launched then */
+#define NINETOOTHED_SCRATCH_LIMIT 2
+#define NINETOOTHED_STATIC_SCRATCH_BYTES (16u << 20)
+
 /* same member order as the reference's enum (src/ninetoothed/aot.py:524-537) */
 enum NineToothedDataType {
     NINETOOTHED_INT8,
@@ -182,6 +187,32 @@ NineToothedResult launch_nt_conv2d(NineToothedStream stream,
                                    int padding_h, int padding_w,
                                    int block_size_m, int block_size_n,
                                    int block_size_k);
+
+/*
+ * launch_nt_matmul for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ *
+ * Same arguments, kernels, tile choice and results as launch_nt_matmul.  The difference is where the
+ * partial products of a split-K launch go (problems with few output tiles and a long K: parts x M x N
+ * floats): not into a workspace that the library allocates, but into a fixed array of
+ * NINETOOTHED_STATIC_SCRATCH_BYTES (16 MiB) that is part of the library's code object -- every GPU the
+ * library runs on holds its copy until the process ends.  This function never calls hipMalloc / hipFree
+ * or any allocating routine.  A call whose partial products exceed the array returns
+ * NINETOOTHED_SCRATCH_LIMIT and launches nothing (it does not fall back to another kernel); problems
+ * that run in one pass need no scratch memory and are accepted at any size.
+ *
+ * All calls on one GPU share that GPU's array, on whatever stream: calls whose kernels may overlap on a
+ * GPU (different streams, or replays of graphs captured from them) race on it and must be ordered by the
+ * caller.  Every launch overwrites all of the array it later reads, so nothing has to be cleared between
+ * calls.
+ */
+NineToothedResult launch_nt_matmul_static_scratch(NineToothedStream stream,
+                                                  NineToothedTensor lhs,
+                                                  NineToothedTensor rhs,
+                                                  NineToothedTensor output,
+                                                  int dtype, int output_dtype,
+                                                  int block_size_m, int block_size_n,
+                                                  int block_size_k);
 
 /* ---- tile selection (stands in for the reference's Triton autotuner,
  * src/ninetoothed/generation.py:372-516 and src/ninetoothed/auto_tuner.py:11-152) ---- */

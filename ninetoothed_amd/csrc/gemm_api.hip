@@ -27,6 +27,9 @@ struct GemmProblem {
     float alpha, beta;
     int batch = 1;  // independent products that share the shapes; operands move by these element strides
     int64_t a_batch = 0, b_batch = 0, c_batch = 0, bias_batch = 0;
+    // set by the entry point that allocates nothing: split-K parts go here instead of the stream's workspace
+    float *fixed_scratch = nullptr;
+    size_t fixed_scratch_bytes = 0;
     bool addmm() const { return bias != nullptr; }
 };
 
@@ -190,9 +193,17 @@ hipError_t split_launch_typed(const GemmProblem &q, hipStream_t stream) {
     int kt_per_part = 0;
     const int parts = split_parts(q, BM, BN, BK, &kt_per_part);
     if (parts < 2) return (hipError_t)NINETOOTHED_NO_KERNEL;
+    const size_t scratch_bytes = (size_t)parts * q.m * q.n * sizeof(float);
+    // the lock of the workspace registry also serialises host threads that enqueue onto the fixed array
     WorkspaceLease lease(stream);
-    float *scratch = (float *)lease.get(kWorkspaceGemmParts, (size_t)parts * q.m * q.n * sizeof(float));
-    if (scratch == nullptr) return (hipError_t)NINETOOTHED_NO_KERNEL;  // no scratch (graph capture, out of memory): the caller takes a one-pass instance
+    float *scratch;
+    if (q.fixed_scratch != nullptr) {
+        if (scratch_bytes > q.fixed_scratch_bytes) return (hipError_t)NINETOOTHED_SCRATCH_LIMIT;
+        scratch = q.fixed_scratch;
+    } else {
+        scratch = (float *)lease.get(kWorkspaceGemmParts, scratch_bytes);
+        if (scratch == nullptr) return (hipError_t)NINETOOTHED_NO_KERNEL;  // no scratch (graph capture, out of memory): the caller takes a one-pass instance
+    }
     GemmParams p;
     fill_params(p, q, BM, BN);
     p.c = scratch;
@@ -498,6 +509,57 @@ NineToothedResult launch_nt_addmm(NineToothedStream stream, NineToothedTensor in
     GemmProblem q;
     const int output_dtype = dtype == NINETOOTHED_FLOAT8_E5M2 ? NINETOOTHED_FLOAT16 : dtype;  // fp8 operands: the rounded product is fp16
     if (int err = build_problem(q, &input, mat1, mat2, &beta, &alpha, output, dtype, output_dtype)) return err;
+    return run_gemm((hipStream_t)stream, q, block_size_m, block_size_n, block_size_k);
+}
+
+}  // extern "C"
+
+namespace nt {
+namespace {
+
+// Scratch memory of launch_nt_matmul_static_scratch: part of the library's code object, so every GPU the
+// library runs on holds its own copy from the first use until the process ends.  Host code never uses the
+// array's name as an address (on the host it is a stand-in, not device memory): the device address is
+// asked for once per device and only that pointer is handed to kernels.
+constexpr size_t kStaticScratchBytes = size_t(NINETOOTHED_STATIC_SCRATCH_BYTES);
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_static_scratch_mutex;
+void *g_static_scratch_address[kMaxDevices] = {};
+
+// the array's address on the current device
+int static_scratch_address(void **address) {
+    int device = 0;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess) return (int)err;
+    if (device < 0 || device >= kMaxDevices) return (int)hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+    if (g_static_scratch_address[device] == nullptr) {
+        void *found = nullptr;
+        err = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+        if (err != hipSuccess) return (int)err;
+        if (found == nullptr) return (int)hipErrorInvalidSymbol;
+        g_static_scratch_address[device] = found;
+    }
+    *address = g_static_scratch_address[device];
+    return 0;
+}
+
+}  // namespace
+}  // namespace nt
+
+extern "C" {
+
+NineToothedResult launch_nt_matmul_static_scratch(NineToothedStream stream, NineToothedTensor lhs, NineToothedTensor rhs,
+                                                  NineToothedTensor output, int dtype, int output_dtype, int block_size_m,
+                                                  int block_size_n, int block_size_k) {
+    GemmProblem q;
+    if (int err = build_problem(q, nullptr, lhs, rhs, nullptr, nullptr, output, dtype, output_dtype)) return err;
+    void *address = nullptr;
+    if (int err = static_scratch_address(&address)) return err;
+    q.fixed_scratch = (float *)address;
+    q.fixed_scratch_bytes = kStaticScratchBytes;
     return run_gemm((hipStream_t)stream, q, block_size_m, block_size_n, block_size_k);
 }
 

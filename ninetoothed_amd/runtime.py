@@ -17,6 +17,8 @@ import threading
 LIBRARY_PATH = pathlib.Path(__file__).resolve().parent / "lib" / "libnt_hip.so"
 
 NO_KERNEL = 1
+SCRATCH_LIMIT = 2  # launch_nt_matmul_static_scratch: the call needs more than the fixed scratch array
+STATIC_SCRATCH_BYTES = 16 << 20
 
 # order of the reference's NineToothedDataType enum (src/ninetoothed/aot.py:524-537)
 DATA_TYPES = ("i8", "i16", "i32", "i64", "u8", "u16", "u32", "u64", "fp16", "bf16", "fp32", "fp64", "fp8e5m2")  # the last one extends the enum
@@ -69,6 +71,7 @@ _S = ctypes.c_void_p
 
 _SIGNATURES = {
     "launch_nt_matmul": (_S, _T, _T, _T, _I, _I, _I, _I, _I),
+    "launch_nt_matmul_static_scratch": (_S, _T, _T, _T, _I, _I, _I, _I, _I),
     "launch_nt_addmm": (_S, _T, _T, _T, _T, _T, _T, _I, _I, _I, _I),
     "launch_nt_softmax": (_S, _T, _T, _I, _I),
     "launch_nt_softmax_config": (_S, _I, _T, _T, _I, _I),

@@ -1,0 +1,80 @@
+"""``launch_nt_matmul_static_scratch``: the matmul entry point that allocates nothing (split-K partial
+products go to a fixed array inside the library) against ``launch_nt_matmul``, through the C ABI, on two
+calls in a row -- the second with a smaller input, so it runs on what the first one left in the array --
+bit for bit: both entry points run the same kernels with the same split."""
+
+import pytest
+import torch
+
+from ninetoothed_amd import runtime
+
+pytestmark = pytest.mark.gpu
+
+
+def _operands(m, n, k, dtype, seed):
+    generator = torch.Generator().manual_seed(seed)
+    a = torch.randn(m, k, generator=generator).to(dtype).cuda()
+    b = (torch.randn(k, n, generator=generator) * 0.1).to(dtype).cuda()
+    return a, b
+
+
+def _call(entry, a, b, out, dtype_tag, out_tag="same"):
+    tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (a, b, out)]
+    dtype = runtime.DATA_TYPE_INDEX[dtype_tag]
+    out_dtype = dtype if out_tag == "same" else runtime.DATA_TYPE_INDEX[out_tag]
+    return entry(runtime.current_stream(), tensors[0], tensors[1], tensors[2], dtype, out_dtype, 0, 0, 0)
+
+
+@pytest.mark.parametrize("dtype, tag", ((torch.float16, "fp16"), (torch.bfloat16, "bf16")))
+def test_static_scratch_matmul_matches_the_allocating_entry_point(dtype, tag):
+    lib = runtime.library()
+    # split-K problems (few output tiles, long K); partial products: 4 x 16 x 8192 and 32 x 16 x 1024 floats = 2 MiB each
+    problems = ((16, 8192, 8192), (16, 1024, 4096), (100, 520, 4104))
+    print("static-scratch matmul", tag, problems, flush=True)
+    warm_a, warm_b = _operands(256, 256, 256, dtype, 1)
+    warm = torch.empty(256, 256, dtype=dtype, device="cuda")
+    assert _call(lib.launch_nt_matmul_static_scratch, warm_a, warm_b, warm, tag) == 0  # code objects and the array are resident from here on
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    outputs = []
+    for index, (m, n, k) in enumerate(problems):
+        a, b = _operands(m, n, k, dtype, 10 + index)
+        out = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+        outputs.append((a, b, out))
+    free_before = torch.cuda.mem_get_info()[0]
+    for a, b, out in outputs:
+        assert _call(lib.launch_nt_matmul_static_scratch, a, b, out, tag) == 0
+    torch.cuda.synchronize()
+    # a workspace for these calls would have taken 2 MiB or more from the device
+    assert free_before - torch.cuda.mem_get_info()[0] < (1 << 20)
+    for a, b, out in outputs:
+        expected = torch.full_like(out, float("nan"))
+        assert _call(lib.launch_nt_matmul, a, b, expected, tag) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(out, expected), tuple(out.shape)
+        assert torch.allclose(out.float(), a.float() @ b.float(), rtol=1e-2 if dtype == torch.float16 else 3e-2, atol=1e-2 if dtype == torch.float16 else 3e-2)
+
+
+def test_static_scratch_matmul_fp32_output_one_pass_problems_and_the_limit():
+    lib = runtime.library()
+    print("static-scratch matmul: fp32 output, one-pass problem, scratch limit", flush=True)
+    a, b = _operands(64, 2048, 8192, torch.float16, 20)
+    out, expected = (torch.full((64, 2048), float("nan"), dtype=torch.float32, device="cuda") for _ in range(2))
+    assert _call(lib.launch_nt_matmul_static_scratch, a, b, out, "fp16", "fp32") == 0
+    assert _call(lib.launch_nt_matmul, a, b, expected, "fp16", "fp32") == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out, expected)
+    # a problem with enough tiles runs in one pass and needs no scratch memory: any size goes
+    a, b = _operands(2048, 2048, 512, torch.float16, 21)
+    out, expected = (torch.full((2048, 2048), float("nan"), dtype=torch.float16, device="cuda") for _ in range(2))
+    assert _call(lib.launch_nt_matmul_static_scratch, a, b, out, "fp16") == 0
+    assert _call(lib.launch_nt_matmul, a, b, expected, "fp16") == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out, expected)
+    # 32 parts x 512 x 512 floats = 32 MiB of partial products: beyond the 16 MiB array -> refused, nothing written
+    a, b = _operands(512, 512, 65536, torch.float16, 22)
+    out = torch.full((512, 512), float("nan"), dtype=torch.float16, device="cuda")
+    assert _call(lib.launch_nt_matmul_static_scratch, a, b, out, "fp16") == runtime.SCRATCH_LIMIT
+    torch.cuda.synchronize()
+    assert bool(torch.isnan(out).all())
+    assert runtime.STATIC_SCRATCH_BYTES == 16 << 20
