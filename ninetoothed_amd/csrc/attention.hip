@@ -50,7 +50,7 @@ constexpr int kAttnWaves = 4;
 // are converted to T beforehand; Q is converted while it is scaled, O is stored unrounded)
 // kPadded: the head dimension in memory (p.head_dim, a multiple of 8) is smaller than D: the missing
 // columns of Q, K and V read as zeros (scores and the stored columns are unchanged by them)
-template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined, typename TIO = T, int kWaves = kAttnWaves, bool kPadded = false, bool kSplitKV = false>
+template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined, typename TIO = T, int kWaves = kAttnWaves, bool kPadded = false, bool kSplitKV = false, bool kFold = true>
 __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(AttentionParams p) {
     static_assert(!kSplitKV || !kPipelined, "the key range is split in the plain loop only");
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -260,19 +260,37 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
     float m_run[kQTiles], l_run[kQTiles];  // l_run: this lane's half of the row sum
 #pragma unroll
     for (int qt = 0; qt < kQTiles; ++qt) {
-        m_run[qt] = -INFINITY;
+        m_run[qt] = kFold ? 0.0f : -INFINITY;
         l_run[qt] = 0.0f;
+    }
+    // kFold: scores are computed relative to a per-row REFERENCE m_run that is at most kFoldSlack below the
+    // row's running maximum, and the subtraction happens inside the matrix pipe: the accumulators of
+    // S^T = K . Q'^T start from -m_run (a lane's accumulators all belong to one query row) instead of
+    // from zero.  The reference moves only when a block's row maximum exceeds it by more than the slack
+    // (or when the row sees its first key), which after the first blocks is rare, so the steady state has
+    // no subtraction, no rescale factor and no rescaling of the output.  Probabilities are then at most
+    // 2^kFoldSlack instead of at most 1; the final division by the row sum cancels the reference.
+    constexpr float kFoldSlack = 8.0f;
+    float16_t c_init[kQTiles];     // -m_run in all 16 registers
+    float fold_limit[kQTiles];     // -inf until the row has seen a key, kFoldSlack afterwards
+#pragma unroll
+    for (int qt = 0; qt < kQTiles; ++qt) {
+        fold_limit[qt] = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) c_init[qt][r] = 0.0f;
     }
 
     // S^T = K . Q'^T for the block held in a K stage
     auto scores = [&](auto stage_tag, float16_t (&s_acc)[KT][kQTiles]) __attribute__((always_inline)) {
         const NT_LDS unsigned char *sk = stage_k(stage_tag);
+        if constexpr (!kFold) {
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt)
+            for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-            for (int qt = 0; qt < kQTiles; ++qt)
+                for (int qt = 0; qt < kQTiles; ++qt)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) s_acc[kt][qt][r] = 0.0f;
+                    for (int r = 0; r < 16; ++r) s_acc[kt][qt][r] = 0.0f;
+        }
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             vec8 kf[KT];
@@ -281,7 +299,10 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-                for (int qt = 0; qt < kQTiles; ++qt) s_acc[kt][qt] = E::mfma32(kf[kt], qf[qt][ks], s_acc[kt][qt]);
+                for (int qt = 0; qt < kQTiles; ++qt) {
+                    if (kFold && ks == 0) s_acc[kt][qt] = E::mfma32(kf[kt], qf[qt][ks], c_init[qt]);
+                    else s_acc[kt][qt] = E::mfma32(kf[kt], qf[qt][ks], s_acc[kt][qt]);
+                }
         }
     };
 
@@ -313,7 +334,78 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
     // online softmax: turns (masked) S^T into P^T operand fragments, updates the
     // running maximum / sum, returns the factor the output has to be rescaled by
     // (per q tile; 1 when the maximum did not move)
+    // kFold, in three pieces so that the pipelined loop can place matrix instructions between them:
+    // the row maxima of a block (relative to the reference) ...
+    auto row_max = [&](const float16_t (&s_acc)[KT][kQTiles], float (&mx)[kQTiles]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int qt = 0; qt < kQTiles; ++qt) {
+            float top = -INFINITY;
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) top = fmaxf(top, s_acc[kt][qt][r]);
+            const unsigned bits = __builtin_bit_cast(unsigned, top);
+            auto halves = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);  // exchange with lane ^ 32 in registers
+            mx[qt] = fmaxf(__builtin_bit_cast(float, (unsigned)halves[0]), __builtin_bit_cast(float, (unsigned)halves[1]));
+        }
+    };
+    // ... the move of the reference when some row of the wave needs it (wave-uniform branch, rare after
+    // the first blocks): the block's scores, the row sums and the accumulator start values follow the
+    // new reference; alpha is the factor for the output accumulators ...
+    auto rebase = [&](float16_t (&s_acc)[KT][kQTiles], const float (&mx)[kQTiles], float (&alpha)[kQTiles]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int qt = 0; qt < kQTiles; ++qt) {
+            alpha[qt] = 1.0f;
+            const bool move = mx[qt] > fold_limit[qt];  // (both lanes of a row hold the same maximum and limit)
+            if (__builtin_amdgcn_ballot_w64(move) != 0) {
+                const float delta = move ? mx[qt] : 0.0f;
+                // a row without keys so far has nothing accumulated: its factor stays 1 (2^-delta may overflow)
+                alpha[qt] = fold_limit[qt] == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(-delta);
+                m_run[qt] += delta;
+                l_run[qt] *= alpha[qt];
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) s_acc[kt][qt][r] -= delta;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) c_init[qt][r] = -m_run[qt];
+            }
+            if (mx[qt] > -INFINITY) fold_limit[qt] = kFoldSlack;
+        }
+    };
+    // ... and the probabilities with their row sums
+    auto exponentials = [&](float16_t (&s_acc)[KT][kQTiles], vec8 (&pf)[PS][kQTiles]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int qt = 0; qt < kQTiles; ++qt) {
+            // four independent partial sums: a single chain would tie every addition to
+            // the exponential right before it
+            float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float pv = __builtin_amdgcn_exp2f(s_acc[kt][qt][r]);
+                    s_acc[kt][qt][r] = pv;
+                    sum[r & 3] += pv;
+                }
+            l_run[qt] += (sum[0] + sum[1]) + (sum[2] + sum[3]);
+        }
+#pragma unroll
+        for (int ps = 0; ps < PS; ++ps)
+#pragma unroll
+            for (int qt = 0; qt < kQTiles; ++qt)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pf[ps][qt][e] = E::from_float(s_acc[ps / 2][qt][8 * (ps & 1) + e]);
+    };
+
     auto softmax = [&](float16_t (&s_acc)[KT][kQTiles], vec8 (&pf)[PS][kQTiles], float (&alpha)[kQTiles]) __attribute__((always_inline)) {
+        if constexpr (kFold) {
+            float mx[kQTiles];
+            row_max(s_acc, mx);
+            rebase(s_acc, mx, alpha);
+            exponentials(s_acc, pf);
+            return;
+        }
 #pragma unroll
         for (int qt = 0; qt < kQTiles; ++qt) {
             float mx = -INFINITY;
@@ -366,10 +458,10 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
     };
 
     // O^T += V^T . P^T for the block held in a V stage
-    auto accumulate = [&](auto stage_tag, const vec8 (&pf)[PS][kQTiles]) __attribute__((always_inline)) {
+    auto accumulate = [&](auto stage_tag, const vec8 (&pf)[PS][kQTiles], auto first_tag, auto last_tag) __attribute__((always_inline)) {
         const NT_LDS unsigned char *sv = stage_v(stage_tag);
 #pragma unroll
-        for (int ps = 0; ps < PS; ++ps) {
+        for (int ps = decltype(first_tag)::value; ps < decltype(last_tag)::value; ++ps) {
             vec8 vf[DT];
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
@@ -387,6 +479,8 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
 
     typedef std::integral_constant<int, 0> Stage0;
     typedef std::integral_constant<int, 1> Stage1;
+    typedef std::integral_constant<int, 0> PsBegin;
+    typedef std::integral_constant<int, PS> PsEnd;
     if constexpr (!kPipelined) {
         // two LDS stages, loop unrolled by two; an odd block count runs one fully
         // masked extra block, whose loads re-fetch the last block
@@ -398,7 +492,7 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
             if (needs_masks(blk)) apply_masks(s_acc, blk);
             softmax(s_acc, pf, alpha);
             rescale(alpha);
-            accumulate(stage_tag, pf);
+            accumulate(stage_tag, pf, PsBegin(), PsEnd());
         };
         if (num_blocks > first_block) {
             issue_k(Stage0(), first_block);
@@ -454,8 +548,51 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
                 issue_k(Own(), min(j + 2, last_block));
                 issue_v(Own(), j);
                 if constexpr (decltype(masked_tag)::value) apply_masks(s_buf[kParity], j);
+                if constexpr (kFold) {
+                    // Two scheduling regions with the (rare) move of the reference between them: the row
+                    // maxima run under the first MFMAs of P(j-1) . V(j-1); the exponentials, row sums and
+                    // conversions under the rest of them and under K(j+1) . Q, whose accumulators start
+                    // from the reference as it stands after the move.
+#ifndef NT_FOLD_SPLIT
+#define NT_FOLD_SPLIT 2
+#endif
+                    typedef std::integral_constant<int, (NT_FOLD_SPLIT < PS ? NT_FOLD_SPLIT : PS)> PsSplit;
+                    float mx[kQTiles];
+                    row_max(s_buf[kParity], mx);
+                    accumulate(Other(), p_buf[1 - kParity], PsBegin(), PsSplit());
+                    {
+                        constexpr int kMfma = PsSplit::value * DT * kQTiles;
+                        constexpr int kReads = PsSplit::value * DT * 2;
+                        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x020, 2 * kInstr, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+                        static_for<0, kMfma>([&](auto i_tag) __attribute__((always_inline)) {
+                            constexpr int i = decltype(i_tag)::value;
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                            if constexpr (6 + 2 * i < kReads) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+                        });
+                    }
+                    rebase(s_buf[kParity], mx, alpha);
+                    exponentials(s_buf[kParity], p_buf[kParity]);
+                    accumulate(Other(), p_buf[1 - kParity], PsSplit(), PsEnd());
+                    scores(Other(), s_buf[1 - kParity]);
+                    {
+                        constexpr int kMfma = ((PS - PsSplit::value) * DT + KS * KT) * kQTiles;
+                        constexpr int kReads = (PS - PsSplit::value) * DT * 2 + KS * KT;
+                        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
+                        static_for<0, kMfma>([&](auto i_tag) __attribute__((always_inline)) {
+                            constexpr int i = decltype(i_tag)::value;
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                            if constexpr (6 + 2 * i < kReads) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x400, (i % 3 == 0) ? 2 : 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+                        });
+                    }
+                } else {
                 softmax(s_buf[kParity], p_buf[kParity], alpha);
-                accumulate(Other(), p_buf[1 - kParity]);
+                accumulate(Other(), p_buf[1 - kParity], PsBegin(), PsEnd());
                 scores(Other(), s_buf[1 - kParity]);
                 // desired issue order inside this region: one MFMA, then the LDS reads
                 // and softmax arithmetic that fit under it
@@ -490,6 +627,7 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
                     }
                 });
 #endif
+                }
                 // P(j) and the row sums are only consumed in later steps; pin them here so
                 // that their arithmetic stays in this step, next to the MFMAs it overlaps with
 #pragma unroll
@@ -521,9 +659,9 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
             wait_vmcnt<0>();
             lds_barrier();
             if ((num_blocks - 1) & 1)
-                accumulate(Stage1(), p_buf[1]);
+                accumulate(Stage1(), p_buf[1], PsBegin(), PsEnd());
             else
-                accumulate(Stage0(), p_buf[0]);
+                accumulate(Stage0(), p_buf[0], PsBegin(), PsEnd());
         }
     }
 
@@ -642,13 +780,13 @@ int launch_split_keys(AttentionParams &p, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
-template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined, typename TIO = T, int kWaves = kAttnWaves, bool kPadded = false>
+template <typename T, int D, int kQTiles, int BN, int kOcc, bool kPipelined, typename TIO = T, int kWaves = kAttnWaves, bool kPadded = false, bool kFold = true>
 hipError_t launch_attention(AttentionParams &p, hipStream_t stream) {
     constexpr int BM = kWaves * 32 * kQTiles;
     p.q_blocks = ceil_div(p.seq_q, BM);
     const int64_t grid = (int64_t)p.batch * p.heads * p.q_blocks;
     if (grid == 0) return hipSuccess;
-    attention_fwd_kernel<T, D, kQTiles, BN, kOcc, kPipelined, TIO, kWaves, kPadded><<<dim3((unsigned)grid), dim3(kWaves * 64), 0, stream>>>(p);
+    attention_fwd_kernel<T, D, kQTiles, BN, kOcc, kPipelined, TIO, kWaves, kPadded, false, kFold><<<dim3((unsigned)grid), dim3(kWaves * 64), 0, stream>>>(p);
     return hipGetLastError();
 }
 
@@ -714,6 +852,11 @@ int dispatch_attention(AttentionParams &p, int head_dim, int variant, hipStream_
         if (variant == 4) return (int)launch_attention<T, 128, 1, 64, 2, true, T, 8>(p, stream);
 #ifdef NT_MEASUREMENT_AIDS
         if (variant == 5) return (int)launch_attention<T, 128, 1, 64, 2, false, T, 8>(p, stream);
+        // 10 + v: variant v with the subtraction of the running maximum done per element (no folding)
+        if (variant == 14) return (int)launch_attention<T, 128, 1, 64, 2, true, T, 8, false, false>(p, stream);
+        if (variant == 13) return (int)launch_attention<T, 128, 1, 64, 2, true, T, kAttnWaves, false, false>(p, stream);
+        if (variant == 11) return (int)launch_attention<T, 128, 2, 64, 1, false, T, kAttnWaves, false, false>(p, stream);
+        if (variant == 10) return (int)launch_attention<T, 128, 1, 64, 2, false, T, kAttnWaves, false, false>(p, stream);
 #endif
         if (variant == 3) return (int)launch_attention<T, 128, 1, 64, 2, true>(p, stream);
         if (variant == 1) return (int)launch_attention<T, 128, 2, 64, 1, false>(p, stream);
@@ -791,15 +934,14 @@ extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineT
     else p.q_scale = dtype == NINETOOTHED_FLOAT16 ? 1.4423828125f : (dtype == NINETOOTHED_BFLOAT16 ? 1.4453125f : 1.44269504089f);
     p.causal = is_causal.data ? (Scalar0d::as_int64(is_causal) != 0) : 0;
     if (float32) return attention_float32(p, (int)head_dim, k, v, (hipStream_t)stream);
-    // block sizes are hints: 256 query rows select the one-workgroup-per-CU
-    // variant, 32-key blocks the three-workgroups-per-CU variant.  Without a hint
-    // the pipelined variant runs non-causal problems and the plain 64-key loop causal
-    // ones (measured at [4, 32, 4096, 128]: 0.94 against 0.92 and 0.90 PFLOP/s); non-causal
-    // problems with enough 256-row blocks to fill the chip twice run the pipelined loop with
-    // eight waves per workgroup, which loads every K / V block once for 256 query rows
-    // (1.02 against 0.99 PFLOP/s).
-    int variant = block_size_m >= 256 ? 1 : (block_size_n > 0 && block_size_n <= 32 ? 2 : (block_size_n >= 64 || p.causal ? 0 : 3));
-    if (variant == 3 && block_size_m == 0 && head_dim >= 64 && (int64_t)p.batch * p.heads * ceil_div(p.seq_q, 256) >= 512) variant = 4;
+    // block sizes are hints: 256 query rows select the one-workgroup-per-CU variant, 32-key blocks the
+    // three-workgroups-per-CU variant, 64-key blocks the plain loop.  Without a hint the pipelined loop
+    // runs (measured at [4, 32, 4096, 128]: 1.12 against 1.08 PFLOP/s for the plain loop, causal 1.01
+    // against 0.98); non-causal problems with enough 256-row blocks to fill the chip twice run it with
+    // eight waves per workgroup, which loads every K / V block once for 256 query rows (1.16 PFLOP/s;
+    // causal 0.99, below the four-wave form).
+    int variant = block_size_m >= 256 ? 1 : (block_size_n > 0 && block_size_n <= 32 ? 2 : (block_size_n >= 64 ? 0 : 3));
+    if (variant == 3 && !p.causal && block_size_m == 0 && head_dim >= 64 && (int64_t)p.batch * p.heads * ceil_div(p.seq_q, 256) >= 512) variant = 4;
 #ifdef NT_MEASUREMENT_AIDS
     if (block_size_n >= 1000) variant = block_size_n - 1000;  // explicit variant, for timing harnesses only
 #endif
