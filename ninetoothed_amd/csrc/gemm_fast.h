@@ -97,6 +97,15 @@ NT_DEVICE void static_for(F &&f) {
 // LDS reads and only then arrives at the barrier.
 NT_DEVICE void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// The same without the wait, for loops whose LDS reads still in flight at the barrier are known to target
+// a stage that is not refilled after it.  No instruction is scheduled across it, so every MFMA of the
+// code before it -- and with it the wait for its operand reads -- is issued before the wave arrives.
+NT_DEVICE void lds_barrier_reads_in_flight() {
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
 // kAblate is a measurement aid (bit 0: no global loads inside the K loop,
 // bit 1: operand fragments read from LDS only once); 0 in every shipped instance.
 template <typename T, int BM, int BN, int BK, int WM, int WN, int kStages, int kWavesPerSimd, bool kAddmm, int kAblate = 0, int kLoad = 0, int kAux = 0,
@@ -370,12 +379,16 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     };
 
     // K loop, unrolled over the stages so every LDS array is named statically.
-    // Step for tile t: wait until tile t has landed, barrier (which also tells
-    // that all waves finished tile t-1), refill the stage tile t-1 used with
-    // tile t+kStages-1, multiply tile t.  Past the end the last tile is fetched
-    // again into a stage nobody reads, which keeps the outstanding-load count
-    // the same in every step.
+    // Past the end the last tile is fetched again into a stage nobody needs, which keeps the
+    // outstanding-load count the same in every step.
     const int main_k = num_k - num_k % kStages;
+    constexpr int KS = BK / 16;
+    // kCross (rings of three or more stages): the barrier that opens the step for tile t tells that every
+    // wave's fills of tile t+1 have landed (one tile EARLIER than needed for t itself) and that every wave
+    // is done with tile t-1, whose stage is refilled right after it.  A wave can then fetch the operand
+    // fragments of the first k step of tile t+1 during the last k step of tile t: the first MFMAs after a
+    // barrier have their operands in registers, and no wave starts a step by waiting for LDS.
+    constexpr bool kCross = kStages >= 3 && kAblate == 0 && KS % 2 == 0;
 
     static_for<0, kStages - 1>([&](auto s) { issue_loads(s, min((int)decltype(s)::value, last_k)); });
     if constexpr (kAblate & 2) {
@@ -383,21 +396,73 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         lds_barrier();
         read_frags(std::integral_constant<int, 0>(), 0, af_once, bf_once);
     }
-    auto step = [&](auto s, int kt) {
-        constexpr int kS = decltype(s)::value;
-        wait_vmcnt<(kAblate & 1) ? 0 : (kStages - 2) * kLoadsPerTile>();
+    if constexpr (kCross) {
+        vec8 af[2][TM];
+        vec8 bf[2][TN];
+        wait_vmcnt<(kStages - 2) * kLoadsPerTile>();
         lds_barrier();
-        if constexpr (!(kAblate & 1))
+        read_frags(std::integral_constant<int, 0>(), 0, af[0], bf[0]);
+        auto step = [&](auto s, int kt) {
+            constexpr int kS = decltype(s)::value;
+            typedef std::integral_constant<int, (kS + 1) % kStages> NextStage;
+            // (the reads in flight here fetch the first k step of this step's own tile; the stage refilled
+            // below belongs to the tile before it, whose reads fed MFMAs that have been issued)
+            wait_vmcnt<(kStages - 3) * kLoadsPerTile>();
+            lds_barrier_reads_in_flight();
             issue_loads(std::integral_constant<int, (kS + kStages - 1) % kStages>(), min(kt + kS + kStages - 1, last_k));
-        multiply_stage(s);
-    };
-    for (int kt = 0; kt < main_k; kt += kStages) {
-        static_for<0, kStages>([&](auto s) { step(s, kt); });
+            static_for<0, KS>([&](auto ks_tag) {
+                constexpr int ks = decltype(ks_tag)::value;
+                constexpr int cur = ks & 1, nxt = cur ^ 1;
+                if constexpr (ks + 1 < KS) read_frags(s, ks + 1, af[nxt], bf[nxt]);
+                else read_frags(NextStage(), 0, af[nxt], bf[nxt]);
+#pragma unroll
+                for (int ti = 0; ti < TM; ++ti)
+#pragma unroll
+                    for (int tj = 0; tj < TN; ++tj) acc[ti][tj] = E::mfma32(bf[cur][tj], af[cur][ti], acc[ti][tj]);  // transposed tile
+#ifndef NT_GEMM_SCHEDULE
+#define NT_GEMM_SCHEDULE 1
+#endif
+#if NT_GEMM_SCHEDULE
+                // issue order: the fragment reads of the next k step (and, in a step's first k step, the
+                // refills of the ring) spread under this k step's MFMAs
+                constexpr int kReads = TM + (kBT ? TN : 2 * TN);
+                constexpr int kFills = ks == 0 ? kLoadsPerTile : 0;
+                static_for<0, TM * TN>([&](auto i_tag) {
+                    constexpr int i = decltype(i_tag)::value;
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    constexpr int kPer = (kReads + TM * TN - 1) / (TM * TN);
+                    if constexpr (i * kPer < kReads) __builtin_amdgcn_sched_group_barrier(0x100, kPer, 0);
+                    if constexpr (i < kFills) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                });
+#endif
+            });
+        };
+        for (int kt = 0; kt < main_k; kt += kStages) {
+            static_for<0, kStages>([&](auto s) { step(s, kt); });
+        }
+        static_for<0, kStages - 1>([&](auto s) {
+            if (main_k + (int)decltype(s)::value < num_k) step(s, main_k);
+        });
+    } else {
+        // Step for tile t: wait until tile t has landed, barrier (which also tells
+        // that all waves finished tile t-1), refill the stage tile t-1 used with
+        // tile t+kStages-1, multiply tile t.
+        auto step = [&](auto s, int kt) {
+            constexpr int kS = decltype(s)::value;
+            wait_vmcnt<(kAblate & 1) ? 0 : (kStages - 2) * kLoadsPerTile>();
+            lds_barrier();
+            if constexpr (!(kAblate & 1))
+                issue_loads(std::integral_constant<int, (kS + kStages - 1) % kStages>(), min(kt + kS + kStages - 1, last_k));
+            multiply_stage(s);
+        };
+        for (int kt = 0; kt < main_k; kt += kStages) {
+            static_for<0, kStages>([&](auto s) { step(s, kt); });
+        }
+        // remaining num_k % kStages tiles continue the stage rotation
+        static_for<0, kStages - 1>([&](auto s) {
+            if (main_k + (int)decltype(s)::value < num_k) step(s, main_k);
+        });
     }
-    // remaining num_k % kStages tiles continue the stage rotation
-    static_for<0, kStages - 1>([&](auto s) {
-        if (main_k + (int)decltype(s)::value < num_k) step(s, main_k);
-    });
 
     // ---- epilogue ----
     // The accumulators hold C transposed per 32x32 tile: lane (l32, g) has, in
