@@ -19,4 +19,10 @@ struct Conv2dRequest {
 // NINETOOTHED_NO_KERNEL when it does not (the caller then uses the gather kernel).
 int conv2d_fast(const Conv2dRequest &request, hipStream_t stream);
 
+// Runs the convolution in one launch on the tensors as they lie (no repacking, no scratch memory) when the
+// request qualifies -- pixels of an input row contiguous, output width a multiple of 8, padding_w <= 1,
+// C*R*S a multiple of 32, contiguous filter and output, output channels filling 256-wide tiles --; returns
+// NINETOOTHED_NO_KERNEL when it does not.
+int conv2d_direct(const Conv2dRequest &request, hipStream_t stream);
+
 }  // namespace nt

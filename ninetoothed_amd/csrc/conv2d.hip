@@ -1,5 +1,10 @@
-// conv2d (stride 1, dilation 1, zero padding) as implicit GEMM on the direct-to-LDS
-// MFMA main loop of gemm_fast.h.
+// conv2d (stride 1, dilation 1, zero padding) as implicit GEMM on the MFMA main loop of gemm_fast.h.  Two paths:
+//
+// (1) conv2d_direct: one launch on the tensors as they lie, no scratch memory (described with its kernel
+//     below); needs an output width that is a multiple of 8, padding_w <= 1, C*R*S a multiple of 32, a contiguous
+//     filter and output, and output channels that fill 256-wide tiles.
+//
+// (2) conv2d_fast: a repacking pre-pass plus the GEMM loop, for the shapes (1) does not take.
 //
 //   GEMM row  m = (image, out_y, out_x)      M = N*P*Q
 //   GEMM col  j = output channel             K_out
@@ -23,7 +28,7 @@
 // laid out [channel][row] and leave as 16-byte stores when P*Q is a multiple of 8
 // (8 consecutive rows then lie in one image, aligned), element by element otherwise.
 //
-// Requirements of this path (anything else uses the any-stride gather kernel):
+// Requirements of path (2) (anything else uses the any-stride gather kernel):
 // fp16/bf16, K_out % 8 == 0, contiguous output.  The repacked operands hold C rounded up to a
 // multiple of 32 channels, the extra ones zero (a 3-channel stem layer multiplies ten times the
 // useful work and is still twice as fast as the gather kernel).
@@ -347,6 +352,404 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
 #endif
 }
 
+// ---- one launch, no scratch: the convolution on the tensors as they lie ----
+//
+// For NCHW the natural orientation of the product is  Y[k_out, pixel] = W[k_out, (c, r, s)] . X_col[(c, r, s), pixel]
+// per image: the filter tensor IS the row-major left operand (its rows are contiguous in (c, r, s)), the output
+// tensor IS the row-major result per image (pixels contiguous per output channel), and the right operand has
+// pixels contiguous, which is how NCHW stores them.  The filter tiles take the direct-to-LDS route of the GEMM
+// (rows of 32 contraction values, read back with ds_read_b128); a row of the right operand's tile is one
+// (channel, filter tap): 256 pixels of one channel shifted by the tap, fetched in 16-byte pieces of 8 pixels
+// -- through registers, because a tap that moves by one pixel leaves the pieces 2-byte aligned, which loads
+// into registers accept and loads into LDS do not -- and written to a [32][256] LDS tile that the transposing
+// ds_read_b64_tr_b16 turns into MFMA operands.  Pieces whose image row lies in the padding are fetched from
+// behind the buffer (zeros); pixels of a piece that fall into the left / right padding are cleared in registers.
+// Needs Q % 8 == 0 (a piece stays inside one image row), C*R*S % 32 == 0, contiguous filter and output.
+//
+// Tiles are 256 output channels x 256 pixels.  (Measured and dropped: cutting the pixels that are left after the
+// last full round of workgroups -- 392 tiles on 256 CUs -- into one round of narrower tiles, with the two waves
+// of a SIMD sharing a tile's pixels so that the round takes the fraction of a full one that its MFMAs are.  A
+// step of a narrow tile lasts as long as a full one: what the ring of loads has in flight does not cover the
+// memory latency once the MFMAs between two barriers shrink.)
+struct ConvDirectParams {
+    const void *x, *w;
+    void *y;
+    int C, H, W, K, R, S, P, Q, pad_h, pad_w;
+    int64_t xs0, xs1, xs2;  // element strides of the input's image, channel and row (pixels of a row are contiguous)
+    int M;                  // pixels of all images
+    int CRS;                // contraction length
+    int tiles_ch;           // tiles along the output channels
+    unsigned x_bytes, w_bytes;
+    int step_c, step_r, step_s;  // 32 contraction positions further: (c, r, s) += these, with carries
+};
+
+template <typename T>
+__global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef Elem<T> E;
+    typedef typename E::vec8 vec8;
+    constexpr int BM = 256, BN = 256, BK = 32, kStages = 4;  // BM: output channels, BN: pixels
+    constexpr int WM = 4, WN = 2, kWaves = 8;
+    constexpr int kWaveM = BM / WM, kWaveN = BN / WN;          // 64 channels x 128 pixels per wave
+    constexpr int TM = kWaveM / 32, TN = kWaveN / 32;
+    // pixel tile [32 rows][256 pixels]: rows 64 bytes longer than their pixels, so that the 8 rows a transposing
+    // read touches start in different banks and every address is affine in (row, pixel): fragments and k steps
+    // are immediate offsets of one address register
+    constexpr int kPitchB = BN * 2 + 64;
+    constexpr int kStageA = BM * BK * 2, kStageB = BK * kPitchB;
+    constexpr int kAChunksPerRow = BK / 8, kARowsPerInstr = 64 / kAChunksPerRow;
+    constexpr int kAInstr = kStageA / (kWaves * 1024);
+    constexpr int KS = BK / 16;
+    static_assert(kAInstr == 2, "thread assignment below");
+
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_a0[kStageA];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_a1[kStageA];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_a2[kStageA];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_a3[kStageA];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_b0[kStageB];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_b1[kStageB];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_b2[kStageB];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_b3[kStageB];
+    auto stage_a = [&](auto tag) -> NT_LDS unsigned char * {
+        constexpr int i = decltype(tag)::value;
+        if constexpr (i == 0) return (NT_LDS unsigned char *)lds_a0;
+        else if constexpr (i == 1) return (NT_LDS unsigned char *)lds_a1;
+        else if constexpr (i == 2) return (NT_LDS unsigned char *)lds_a2;
+        else return (NT_LDS unsigned char *)lds_a3;
+    };
+    auto stage_b = [&](auto tag) -> NT_LDS unsigned char * {
+        constexpr int i = decltype(tag)::value;
+        if constexpr (i == 0) return (NT_LDS unsigned char *)lds_b0;
+        else if constexpr (i == 1) return (NT_LDS unsigned char *)lds_b1;
+        else if constexpr (i == 2) return (NT_LDS unsigned char *)lds_b2;
+        else return (NT_LDS unsigned char *)lds_b3;
+    };
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_m = wave % WM, wave_n = wave / WM;
+
+    // ---- which tile ----
+    const int tile_ch = blockIdx.x % p.tiles_ch;
+    const int n0 = (blockIdx.x / p.tiles_ch) * BN;
+    const int tile_pixels = min(BN, p.M - n0);  // > 0 by construction of the grid
+    const int m0 = tile_ch * BM;
+    const int PQ = p.P * p.Q;
+    const int RS = p.R * p.S;
+
+    // ---- filter tile: rows of 32 contraction values, direct to LDS ----
+    const int64_t w_rows = min((int64_t)BM, (int64_t)p.K - m0);
+    const unsigned char *w_base = (const unsigned char *)((const T *)p.w + (int64_t)m0 * p.CRS);
+    __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)w_base, 0, (unsigned)(w_rows * p.CRS * 2), 0x00020000);
+    unsigned a_src[kAInstr];
+#pragma unroll
+    for (int j = 0; j < kAInstr; ++j) {
+        const int row = (j * kWaves + wave) * kARowsPerInstr + lane / kAChunksPerRow;
+        const int chunk = a_phys_chunk<BK>(row, lane % kAChunksPerRow);
+        a_src[j] = (unsigned)(row * p.CRS + chunk * 8) * 2u;
+    }
+    auto issue_filter = [&](auto stage_tag, int kt) {
+        NT_LDS unsigned char *sa = stage_a(stage_tag);
+#pragma unroll
+        for (int j = 0; j < kAInstr; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, sa + (j * kWaves + wave) * 1024, 16, a_src[j], kt * BK * 2, 0, 0);
+    };
+
+    // ---- pixel tile: a thread fetches one 16-byte piece (8 pixels) of two rows, 16 contraction positions apart ----
+    // A row is one (channel, filter tap).  A tap that moves the pixels by one column leaves the load 2-byte
+    // aligned, which loads into registers accept; the pixel that the first / last piece of an image row then
+    // takes from the neighbouring image row is cleared before the piece is stored.  A tap that moves the pixels
+    // above or below the image gets an offset with the top bit set: such loads return zeros.
+    constexpr int kGather = 2;
+    __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.x_bytes, 0x00020000);
+    const int piece = tid % (BN / 8);
+    const int krow0 = tid / (BN / 8);  // 0..15; the second row is krow0 + 16
+    int lane_off;            // byte offset of the piece for channel 0 and the filter's first tap
+    unsigned rows_outside;   // bit r: filter row r moves the pixels out of the image (or the piece lies past the tile's end)
+    bool at_left, at_right;  // the piece is the first / last of an image row
+    {
+        const int n = n0 + piece * 8;
+        const bool live = piece * 8 < tile_pixels;
+        const int image = n / PQ, pq = n - image * PQ;
+        const int oy = pq / p.Q, ox = pq - oy * p.Q;
+        lane_off = (int)(image * p.xs0 + (int64_t)(oy - p.pad_h) * p.xs2 + ox - p.pad_w) * 2;
+        rows_outside = 0xffffffffu;
+        for (int r = 0; r < p.R; ++r)
+            if (live && (unsigned)(oy - p.pad_h + r) < (unsigned)p.H) rows_outside &= ~(1u << r);
+        at_left = ox == 0;
+        at_right = ox == p.Q - 8;
+    }
+    // Loads that would reach below the tensor's first or beyond its last byte would lose their whole piece to the
+    // range check: the first image row of the whole tensor with a tap that moves it left, the last with one that
+    // moves it right.  Tiles that contain such a row run the careful form of the loop, which tests every load for
+    // this and, where it happens, loads the piece one pixel further in and moves the pixels back in registers.
+    const int last_live = min(BN / 8 - 1, (tile_pixels - 1) / 8);  // the lane with this piece in wave 0 has the largest offset
+    const int off_first = __builtin_amdgcn_readfirstlane(lane_off);
+    const int off_last = __builtin_amdgcn_readlane(lane_off, last_live);
+    const int64_t reach = ((int64_t)(p.C - 1) * p.xs1 + (int64_t)(p.R - 1) * p.xs2 + p.S - 1) * 2;  // largest row offset
+    const bool careful_tile = off_first < 0 || (int64_t)off_last + reach + 16 > (int64_t)p.x_bytes;
+    // masks that clear the pixel left / right of the image in a piece at an image border
+    const unsigned keep_left = at_left ? 0xffff0000u : 0xffffffffu;    // first dword of the piece
+    const unsigned keep_right = at_right ? 0x0000ffffu : 0xffffffffu;  // last dword
+    // this thread's rows in the tile fetched next: filter row and column, and the byte offset c * xs1 + r * xs2 + s
+    // that goes with them (the channel itself is not needed: the loop ends with the last one)
+    int gr[kGather], gs[kGather], goff[kGather];
+#pragma unroll
+    for (int j = 0; j < kGather; ++j) {
+        const int k = krow0 + 16 * j;
+        const int c = k / RS, rs = k - c * RS;
+        gr[j] = rs / p.S;
+        gs[j] = rs - gr[j] * p.S;
+        goff[j] = (c * (int)p.xs1 + gr[j] * (int)p.xs2 + gs[j]) * 2;
+    }
+    const int step_off = (p.step_c * (int)p.xs1 + p.step_r * (int)p.xs2 + p.step_s) * 2;  // 32 contraction positions further ...
+    const int carry_s = ((int)p.xs2 - p.S) * 2;                                           // ... when the column wraps
+    const int carry_r = ((int)p.xs1 - p.R * (int)p.xs2) * 2;                              // ... when the row wraps
+    typedef unsigned uint4_t __attribute__((ext_vector_type(4)));
+    const unsigned b_dst = (unsigned)(krow0 * kPitchB + piece * 16);  // the first piece in a stage; the second: 16 rows on
+    // fetches this thread's pieces of the next tile and moves on to the tile after it; `cols` keeps the rows' filter columns
+    auto gather = [&](auto careful_tag, uint4_t (&regs)[kGather], int (&cols)[kGather]) {
+#pragma unroll
+        for (int j = 0; j < kGather; ++j) {
+            cols[j] = gs[j];
+            // one and the same offset behind the buffer for every load that has to return zeros
+            int offset = (rows_outside >> gr[j]) & 1 ? (int)0x80000000 : lane_off + goff[j];
+
+            bool edge = false;  // the load would start below the tensor or end beyond it
+            if constexpr (decltype(careful_tag)::value) {
+                const bool outside = (rows_outside >> gr[j]) & 1;
+                edge = !outside && (offset < 0 || (unsigned)(offset + 16) > p.x_bytes);
+            }
+            if (decltype(careful_tag)::value && __builtin_amdgcn_ballot_w64(edge) != 0) {  // uniform, and rare
+                // the lanes concerned load one pixel further in and move the pixels back by one place
+                const int nudge = !edge ? 0 : (offset < 0 ? 1 : -1);
+                const uint4_t v = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, offset + 2 * nudge, 0, 0));
+                // byte selectors of v_perm_b32 over {high operand: bytes 4..7, low operand: bytes 0..3}
+                const unsigned up = nudge > 0 ? 0x05040302u : 0x07060504u;    // pixels move one place up: (v[i], v[i-1])
+                const unsigned down = nudge < 0 ? 0x05040302u : 0x03020100u;  // ... one place down: (v[i+1], v[i])
+                uint4_t w;
+                w[0] = __builtin_amdgcn_perm(v[0], 0u, up);
+                w[1] = __builtin_amdgcn_perm(v[1], v[0], up);
+                w[2] = __builtin_amdgcn_perm(v[2], v[1], up);
+                w[3] = __builtin_amdgcn_perm(v[3], v[2], up);
+                regs[j][0] = __builtin_amdgcn_perm(w[1], w[0], down);
+                regs[j][1] = __builtin_amdgcn_perm(w[2], w[1], down);
+                regs[j][2] = __builtin_amdgcn_perm(w[3], w[2], down);
+                regs[j][3] = __builtin_amdgcn_perm(0u, w[3], down);
+            } else {
+                regs[j] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, offset, 0, 0));
+            }
+            gs[j] += p.step_s;
+            const bool wrap_s = gs[j] >= p.S;
+            gs[j] -= wrap_s ? p.S : 0;
+            gr[j] += p.step_r + (wrap_s ? 1 : 0);
+            const bool wrap_r = gr[j] >= p.R;
+            gr[j] -= wrap_r ? p.R : 0;
+            goff[j] += step_off + (wrap_s ? carry_s : 0) + (wrap_r ? carry_r : 0);
+        }
+    };
+    // stores the pieces, the pixel that a shifted piece at an image border took from the neighbouring image row cleared
+    auto scatter = [&](auto stage_tag, const uint4_t (&regs)[kGather], const int (&cols)[kGather]) {
+        NT_LDS unsigned char *sb = stage_b(stage_tag) + b_dst;
+#pragma unroll
+        for (int j = 0; j < kGather; ++j) {
+            uint4_t v = regs[j];
+            v[0] &= cols[j] < p.pad_w ? keep_left : 0xffffffffu;
+            v[3] &= cols[j] > p.S - 1 - p.pad_w ? keep_right : 0xffffffffu;
+            *(NT_LDS uint4_t *)(sb + j * (16 * kPitchB)) = v;
+        }
+    };
+
+    // ---- LDS -> registers ----
+    const int g = lane >> 5, l32 = lane & 31;
+    const int a_row = wave_m * kWaveM + l32;                 // + 32 * ti
+    const int a_sw = a_phys_chunk<BK>(a_row, 0);             // the swizzle repeats every 16 rows
+    const int a_off = a_row * (BK * 2);
+    const int i16 = lane & 15, nhalf = (lane >> 4) & 1;
+    // transposing read: lane i of a 16-lane group addresses row i / 4 (+ 8 g, + 4 for the upper half, + 16 ks),
+    // pixels 4 * (i % 4) .. + 3 of the group's 16 (+ 32 tj)
+    const int b_off = (8 * g + (i16 >> 2)) * kPitchB + (wave_n * kWaveN + nhalf * 16 + 4 * (i16 & 3)) * 2;
+    auto read_frags = [&](auto stage_tag, int ks, vec8 (&af)[TM], vec8 (&bf)[TN]) {
+        const NT_LDS unsigned char *sa = stage_a(stage_tag);
+        const NT_LDS unsigned char *sb = stage_b(stage_tag);
+#pragma unroll
+        for (int ti = 0; ti < TM; ++ti) {
+            const int chunk = (ks * 2 + g) ^ a_sw;
+            af[ti] = *(const NT_LDS vec8 *)(sa + a_off + ti * (32 * BK * 2) + chunk * 16);
+        }
+#pragma unroll
+        for (int tj = 0; tj < TN; ++tj) {
+            short4_t lo = lds_read_tr16_b64(sb + b_off + (ks * 16) * kPitchB + tj * 64);
+            short4_t hi = lds_read_tr16_b64(sb + b_off + (ks * 16 + 4) * kPitchB + tj * 64);
+            short8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            bf[tj] = __builtin_bit_cast(vec8, both);
+        }
+    };
+
+    float16_t acc[TM][TN];
+#pragma unroll
+    for (int ti = 0; ti < TM; ++ti)
+#pragma unroll
+        for (int tj = 0; tj < TN; ++tj)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[ti][tj][r] = 0.0f;
+
+    // ---- main loop ----
+    // Tile t occupies stage t % 4.  The barrier that opens step t tells that tile t + 1 is complete in LDS (so
+    // that the fragments of its first k step can be fetched during step t) and that every wave is done with
+    // tile t - 1.  In step t a wave stores its pieces of the pixel part of tile t + 2, fetched two steps
+    // earlier, into that tile's stage, fetches its pieces of tile t + 4 into the registers that have become
+    // free, and requests the filter part of tile t + 3 into the stage of tile t - 1.
+    const int num_k = p.CRS / BK;
+    const int last_k = num_k - 1;
+    uint4_t held[2][kGather];  // pieces in flight, by tile parity
+    int held_cols[2][kGather];  // their filter columns (uniform)
+    auto run = [&](auto careful_tag) {
+        constexpr int kFrags = TN;
+        // prologue: tiles 0 and 1 complete, the pieces of tiles 2 and 3 and the filter part of tile 2 in flight
+        issue_filter(std::integral_constant<int, 0>(), 0);
+        gather(careful_tag, held[0], held_cols[0]);
+        issue_filter(std::integral_constant<int, 1>(), min(1, last_k));
+        gather(careful_tag, held[1], held_cols[1]);
+        wait_vmcnt<0>();
+        scatter(std::integral_constant<int, 0>(), held[0], held_cols[0]);
+        scatter(std::integral_constant<int, 1>(), held[1], held_cols[1]);
+        gather(careful_tag, held[0], held_cols[0]);
+        issue_filter(std::integral_constant<int, 2>(), min(2, last_k));
+        gather(careful_tag, held[1], held_cols[1]);
+        vec8 af[2][TM];
+        vec8 bf[2][TN];
+        lds_barrier();
+        read_frags(std::integral_constant<int, 0>(), 0, af[0], bf[0]);
+        auto step = [&](auto s, auto parity_tag, int t) {
+            constexpr int kS = decltype(s)::value;
+            constexpr int kParity = decltype(parity_tag)::value;  // of t, t + 2 and t + 4
+            typedef std::integral_constant<int, (kS + 1) % kStages> NextStage;
+            // Loads are issued as: pieces of tile t + 4, then the filter part of tile t + 3, in every step.  All but
+            // the last step's have arrived here: the pieces of tile t + 2, stored below, and the filter part of
+            // tile t + 1, which with that tile's pieces, stored one step ago (the barrier waits for this wave's LDS
+            // traffic), completes tile t + 1.
+            wait_vmcnt<kAInstr + kGather>();
+            lds_barrier();
+            scatter(std::integral_constant<int, (kS + 2) % kStages>(), held[kParity], held_cols[kParity]);
+            gather(careful_tag, held[kParity], held_cols[kParity]);
+            issue_filter(std::integral_constant<int, (kS + 3) % kStages>(), min(t + 3, last_k));
+            static_for<0, KS>([&](auto ks_tag) {
+                constexpr int ks = decltype(ks_tag)::value;
+                constexpr int cur = ks & 1, nxt = cur ^ 1;
+                if constexpr (ks + 1 < KS) read_frags(s, ks + 1, af[nxt], bf[nxt]);
+                else read_frags(NextStage(), 0, af[nxt], bf[nxt]);
+#pragma unroll
+                for (int ti = 0; ti < TM; ++ti)
+#pragma unroll
+                    for (int tj = 0; tj < kFrags; ++tj) acc[ti][tj] = E::mfma32(bf[cur][tj], af[cur][ti], acc[ti][tj]);
+                // issue order: the fragment reads of the next k step spread under this k step's MFMAs
+                constexpr int kMfma = TM * kFrags;
+                constexpr int kReads = TM + 2 * kFrags;
+                constexpr int kPer = kMfma > 0 ? (kReads + kMfma - 1) / kMfma : 1;
+                static_for<0, kMfma>([&](auto i_tag) {
+                    constexpr int i = decltype(i_tag)::value;
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    if constexpr (i * kPer < kReads) __builtin_amdgcn_sched_group_barrier(0x100, kPer, 0);
+                });
+            });
+        };
+        // stages and parities repeat every 4 tiles
+        int t = 0;
+        for (; t + 4 <= num_k; t += 4) {
+            static_for<0, 4>([&](auto i_tag) {
+                constexpr int i = decltype(i_tag)::value;
+                step(std::integral_constant<int, i>(), std::integral_constant<int, i & 1>(), t + i);
+            });
+        }
+        static_for<0, 3>([&](auto i_tag) {
+            constexpr int i = decltype(i_tag)::value;
+            if (t + i < num_k) step(std::integral_constant<int, i>(), std::integral_constant<int, i & 1>(), t + i);
+        });
+    };
+    if (careful_tile) run(std::true_type());  // (the first and the last tile of a launch)
+    else run(std::false_type());
+
+    // ---- epilogue ----
+    // lane (l32, g) holds, per 32 x 32 tile, output channel l32 and in registers 4 * r4 .. + 3 the pixels
+    // 8 * r4 + 4 * g .. + 3.  Each wave passes 32 channels x 128 pixels at a time through its own LDS slab
+    // (in the filter stages, idle by now: two slabs each), so that a lane stores 16 bytes of one channel's pixels.
+    constexpr int kRowBytes = kWaveN * 2;
+    constexpr int kCChunks = kRowBytes / 16;
+    constexpr int kSlabBytes = 32 * kRowBytes;
+    static_assert(2 * kSlabBytes == kStageA && kWaves == 2 * kStages, "slabs in the filter stages");
+    wait_vmcnt<0>();
+    lds_barrier();
+    NT_LDS unsigned char *slab = (wave < 2   ? (NT_LDS unsigned char *)lds_a0
+                                  : wave < 4 ? (NT_LDS unsigned char *)lds_a1
+                                  : wave < 6 ? (NT_LDS unsigned char *)lds_a2
+                                             : (NT_LDS unsigned char *)lds_a3) +
+                                 (wave & 1) * kSlabBytes;
+    T *Y = (T *)p.y;
+    const int slab_sw = l32 & (kCChunks - 1);
+#pragma unroll
+    for (int ti = 0; ti < TM; ++ti) {
+#pragma unroll
+        for (int tj = 0; tj < TN; ++tj)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                typedef T vec4 __attribute__((ext_vector_type(4)));
+                vec4 v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = E::from_float(acc[ti][tj][4 * r4 + e]);
+                const int chunk = (tj * 4 + r4) ^ slab_sw;
+                *(NT_LDS vec4 *)(slab + l32 * kRowBytes + chunk * 16 + 8 * g) = v;
+            }
+#pragma unroll
+        for (int it = 0; it < (32 * kCChunks) / 64; ++it) {
+            const int idx = it * 64 + lane;
+            const int row = idx / kCChunks;
+            const int phys = idx % kCChunks;
+            const int chunk = phys ^ (row & (kCChunks - 1));
+            vec8 v = *(const NT_LDS vec8 *)(slab + row * kRowBytes + phys * 16);
+            const int channel = m0 + wave_m * kWaveM + ti * 32 + row;
+            const int in_tile = wave_n * kWaveN + chunk * 8;
+            if (channel >= p.K || in_tile >= tile_pixels) continue;  // (tiles are multiples of 8 pixels wide)
+            const int n = n0 + in_tile;
+            const int image = n / PQ, pq = n - image * PQ;
+            __builtin_nontemporal_store(v, (vec8 *)(Y + ((int64_t)image * p.K + channel) * PQ + pq));
+        }
+    }
+#endif
+}
+
+// the one-launch path on the tensors as they lie; NINETOOTHED_NO_KERNEL when the request does not fit it
+template <typename T>
+int run_direct(const Conv2dRequest &q, hipStream_t stream) {
+    const int CRS = q.C * q.R * q.S;
+    if (q.Q % 8 || q.W < 8 || q.pad_w > 1 || CRS % 32 || q.R > 16 || q.S > 16) return NINETOOTHED_NO_KERNEL;
+    if (q.xs[3] != 1 || q.xs[0] < 0 || q.xs[1] < 0 || q.xs[2] < 0) return NINETOOTHED_NO_KERNEL;
+    if (q.ws[3] != 1 || q.ws[2] != q.S || q.ws[1] != (int64_t)q.R * q.S || q.ws[0] != CRS || ((uintptr_t)q.w & 15)) return NINETOOTHED_NO_KERNEL;
+    // at least four fifths of the 256 output channels of a tile in use
+    if ((int64_t)q.K * 5 < (int64_t)ceil_div(q.K, 256) * 256 * 4) return NINETOOTHED_NO_KERNEL;
+    const int64_t x_extent = ((int64_t)(q.N - 1) * q.xs[0] + (int64_t)(q.C - 1) * q.xs[1] + (int64_t)(q.H - 1) * q.xs[2] + q.W) * 2;
+    const int64_t w_bytes = (int64_t)q.K * CRS * 2;
+    if (x_extent >= (int64_t(1) << 31) || w_bytes >= (int64_t(1) << 31)) return NINETOOTHED_NO_KERNEL;  // 32-bit buffer offsets
+    ConvDirectParams p;
+    p.x = q.x; p.w = q.w; p.y = q.y;
+    p.C = q.C; p.H = q.H; p.W = q.W; p.K = q.K; p.R = q.R; p.S = q.S; p.P = q.P; p.Q = q.Q;
+    p.pad_h = q.pad_h; p.pad_w = q.pad_w;
+    p.xs0 = q.xs[0]; p.xs1 = q.xs[1]; p.xs2 = q.xs[2];
+    p.M = q.N * q.P * q.Q;
+    p.CRS = CRS;
+    p.x_bytes = (unsigned)x_extent;
+    p.w_bytes = (unsigned)w_bytes;
+    p.step_c = 32 / (q.R * q.S);
+    p.step_r = (32 % (q.R * q.S)) / q.S;
+    p.step_s = 32 % q.S;
+    p.tiles_ch = ceil_div(q.K, 256);
+    const int64_t grid = (int64_t)ceil_div(p.M, 256) * p.tiles_ch;
+    if (grid <= 0 || grid > 0x7fffffffll) return NINETOOTHED_NO_KERNEL;
+    conv2d_direct_kernel<T><<<dim3((unsigned)grid), dim3(512), 0, stream>>>(p);
+    return (int)hipGetLastError();
+}
+
 template <typename T>
 int run_fast(const Conv2dRequest &q, hipStream_t stream) {
     const int Cp = ceil_div(q.C, 32) * 32;
@@ -412,6 +815,14 @@ int conv2d_fast(const Conv2dRequest &q, hipStream_t stream) {
     // enough work to amortise the repacking pass
     if ((int64_t)q.N * q.P * q.Q < 1024) return NINETOOTHED_NO_KERNEL;
     return q.dtype == NINETOOTHED_FLOAT16 ? run_fast<half_t>(q, stream) : run_fast<bf16_t>(q, stream);
+}
+
+int conv2d_direct(const Conv2dRequest &q, hipStream_t stream) {
+    if (q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) return NINETOOTHED_NO_KERNEL;
+    if (q.ys[3] != 1 || q.ys[2] != q.Q || q.ys[1] != (int64_t)q.P * q.Q || q.ys[0] != (int64_t)q.K * q.P * q.Q) return NINETOOTHED_NO_KERNEL;
+    if (((uintptr_t)q.y & 15) != 0 || q.K % 8) return NINETOOTHED_NO_KERNEL;
+    if ((int64_t)q.N * q.P * q.Q > 0x7fffffffll - 512) return NINETOOTHED_NO_KERNEL;
+    return q.dtype == NINETOOTHED_FLOAT16 ? run_direct<half_t>(q, stream) : run_direct<bf16_t>(q, stream);
 }
 
 }  // namespace nt

@@ -775,6 +775,11 @@ NineToothedResult launch_nt_conv2d(NineToothedStream stream, NineToothedTensor i
             const int choice = heuristic_choice(q, 0, 0, 0);
             if (choice > kAnyStride && !is_split(choice)) return (int)kInstances[choice].launch(q, (hipStream_t)stream);
         }
+        // block_size_m: 1 = the gather kernel, 2 = the repacking path; otherwise the library's choice
+        if (block_size_m != 1 && block_size_m != 2) {
+            const int direct = conv2d_direct(request, (hipStream_t)stream);
+            if (direct != NINETOOTHED_NO_KERNEL) return direct;
+        }
         const int fast = block_size_m == 1 ? NINETOOTHED_NO_KERNEL : conv2d_fast(request, (hipStream_t)stream);
         if (fast != NINETOOTHED_NO_KERNEL) return fast;
     }
