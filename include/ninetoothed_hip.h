@@ -147,9 +147,13 @@ NineToothedResult launch_nt_softmax_config(NineToothedStream stream, int config,
  * block_size_m / block_size_n are hints (0 = library's choice): block_size_m
  * >= 256 selects 256 query rows per workgroup, block_size_n <= 32 the 32-key
  * blocks with three workgroups per CU, block_size_n >= 64 the plain 64-key
- * loop; without hints non-causal calls run the software-pipelined 64-key loop
- * (with 256 query rows and eight waves per workgroup when that still fills the
- * chip twice) and causal calls the plain one.  K and V of one (batch, head) must span
+ * loop; without hints a call runs the variant recorded for its problem by
+ * nt_tune_attention, else the software-pipelined 64-key loop (non-causal: with
+ * 256 query rows and eight waves per workgroup when that still fills the chip
+ * twice).  Without a scale tensor the scores are scaled by log2(e) rounded to
+ * the element type, as the reference program's literal is.  FLOAT32 tensors
+ * are computed on fp16 copies: values beyond the fp16 range overflow, which
+ * the reference's fp32 kernel does not.  K and V of one (batch, head) must span
  * less than 4 GiB.
  * head_dim: 32, 64, 128 and 256 have kernels of their size; any other multiple of
  * 8 up to 256 runs on the next of these sizes with the missing columns read as
@@ -169,16 +173,23 @@ NineToothedResult launch_nt_attention(NineToothedStream stream,
  * dilation 1 and zero padding (padding_h, padding_w), computed as the implicit
  * GEMM [N*P*Q, C*R*S] x [C*R*S, K] the arrangement of
  * tests/test_conv2d.py:13-48 describes.
- * When K % 8 == 0, C >= 2, the output is contiguous and
- * N*P*Q >= 1024, the call first repacks the input to channels-last and the
- * filter to [R*S*C', K] (C' = C rounded up to a multiple of 32, zero filled)
- * in the library's scratch buffers of `stream`
- * (N*C'*H*W + K*C'*R*S elements), then runs the direct-to-LDS main loop;
+ * Ways to run it, tried in this order unless block_size_m names one (3, 2, 1)
+ * or nt_tune_conv2d has recorded one for the problem:
+ * 3 -- one launch on the tensors as they lie, no scratch memory: the filter is
+ *   the row-major left operand, rows of the right operand are (channel, filter
+ *   tap)-shifted pixel runs of the NCHW input; needs an output width that is a
+ *   multiple of 8, padding_w <= 1, C*R*S a multiple of 32, pixels of an input row
+ *   contiguous, contiguous filter and output, K filling 256-wide tiles to 4/5;
+ * 2 -- when K % 8 == 0, C >= 2, the output is contiguous and N*P*Q >= 1024: the
+ *   input is first repacked to channels-last and the filter to [R*S*C', K]
+ *   (C' = C rounded up to a multiple of 32, zero filled) in the library's scratch
+ *   buffers of `stream` (N*C'*H*W + K*C'*R*S elements), then the direct-to-LDS
+ *   GEMM loop runs;
+ * 1 -- the scratch-free gather kernel, which serves every shape, and calls whose
+ *   scratch cannot be allocated (out of memory; a stream under graph capture that
+ *   has no buffer yet).
  * 1 x 1 filters without padding (P*Q and C multiples of 8) run as one batched
- * launch of the GEMM kernels on the tensors as they lie, without scratch;
- * block_size_m == 1 keeps the call on the scratch-free gather kernel, which
- * also serves every other shape and calls whose scratch cannot be allocated
- * (out of memory; a stream under graph capture that has no buffer yet). */
+ * launch of the GEMM kernels on the tensors as they lie, without scratch. */
 NineToothedResult launch_nt_conv2d(NineToothedStream stream,
                                    NineToothedTensor input,
                                    NineToothedTensor filter,
@@ -241,7 +252,8 @@ NineToothedResult launch_nt_gemm_config(NineToothedStream stream, int config,
  * `iters` launches each after 2 warm-ups; this call synchronises) and stores
  * the winner in the per-device cache that launch_nt_matmul / launch_nt_addmm
  * consult when block sizes are 0.  Returns 0 and the winner in *best_config,
- * its average time in *best_ms. */
+ * its average time in *best_ms.  On a stream that is being captured into a
+ * graph nothing is timed or recorded: returns 0 with *best_config = -1. */
 NineToothedResult nt_tune_gemm(NineToothedStream stream,
                                NineToothedTensor input,
                                NineToothedTensor mat1,
@@ -252,17 +264,47 @@ NineToothedResult nt_tune_gemm(NineToothedStream stream,
                                int dtype, int output_dtype, int iters,
                                int *best_config, float *best_ms);
 
+/* As nt_tune_gemm for launch_nt_attention: times its loop variants (plain 64-key blocks; 256 query rows per
+ * workgroup; 32-key blocks; software-pipelined; software-pipelined with eight waves) on the given tensors and
+ * records the fastest for later launches of the same problem (element type, batch, heads, both sequence
+ * lengths, head dimension, causal flag) without block-size hints.  *best_variant = -1 when nothing was timed (a
+ * stream that is being captured into a graph), -2 when the problem has no alternatives (FLOAT32 tensors, head
+ * dimensions other than 64 and 128, shapes whose key range is split). */
+NineToothedResult nt_tune_attention(NineToothedStream stream,
+                                    NineToothedTensor q, NineToothedTensor k, NineToothedTensor v,
+                                    NineToothedTensor is_causal, NineToothedTensor scale,
+                                    NineToothedTensor o,
+                                    int dtype, int iters, int *best_variant, float *best_ms);
+
+/* As nt_tune_gemm for launch_nt_conv2d: times the ways to run the convolution -- 3 = one launch on the tensors as
+ * they lie, 2 = repacking pass plus GEMM loop, 1 = gather kernel; a way that does not take the problem is skipped
+ * -- and records the fastest (the block_size_m value that selects it) for later launches of the same problem with
+ * block_size_m = 0.  *best_path = -1 when nothing was timed (graph capture). */
+NineToothedResult nt_tune_conv2d(NineToothedStream stream,
+                                 NineToothedTensor input, NineToothedTensor filter, NineToothedTensor output,
+                                 int dtype, int padding_h, int padding_w, int iters,
+                                 int *best_path, float *best_ms);
+
 /* Persistence of the tuned choices in the line-pair CSV format of the
  * reference's AutoTuningCache (src/ninetoothed/templates/auto_tuning_cache.h:27-75,
- * writer src/ninetoothed/build.py:683-703): a line of integers for the problem
- * (dtype, output dtype, M, N, K, addmm), then a line for the choice (block M,
- * block N, block K, instance index); the first pair has an empty problem line
- * and holds the default.  Both act on the cache of the current device. */
+ * writer src/ninetoothed/build.py:683-703): a line of integers for the problem,
+ * then a line for the choice; the first pair has an empty problem line and holds
+ * a default.  A problem line starts with the program (0 = matmul / addmm: dtype,
+ * output dtype, M, N, K, addmm, rhs layout [0 row-major, 1 transposed, 2 other
+ * strides]; 1 = attention: dtype, batch, heads, seq_q, seq_k, head_dim, causal;
+ * 2 = conv2d: dtype, N, C, H, W, K, R, S, padding_h, padding_w, dense input);
+ * a choice line starts with the variant (GEMM instance index, attention variant,
+ * conv2d path) and may go on with descriptive integers (the GEMM instance's
+ * block M, N, K).  Both act on the table of the current device. */
 NineToothedResult nt_tune_cache_save(const char *path);
 NineToothedResult nt_tune_cache_load(const char *path, int *entries);
 
-/* The cached instance for a problem, or -1. */
+/* The cached GEMM instance for a problem with a row-major rhs, or -1. */
 int nt_tune_cache_lookup(int dtype, int output_dtype, int m, int n, int k, int addmm);
+
+/* The recorded choice for a problem of program `kind` (as in the cache file: 0, 1, 2) given by the `count`
+ * integers of its problem line (without the program), or -1. */
+int nt_tune_lookup(int kind, const int *values, int count);
 
 /*
  * Element-wise / reducing tile programs that are none of the programs above.

@@ -6,11 +6,12 @@ with a new problem times every candidate and later calls reuse the winner; its
 AOT path persists winners in a line-pair CSV file
 (src/ninetoothed/build.py:683-703, templates/auto_tuning_cache.h:27-75) and
 its ``AutoTuner`` keeps timings on disk between processes
-(src/ninetoothed/auto_tuner.py:11-95).  Here the candidates are the GEMM
-instances of ``libnt_hip.so``: ``nt_tune_gemm`` times them on the caller's
-tensors, the library caches the winner per device and problem, and this module
-keeps that cache on disk in the reference's CSV format so that a new process
-starts tuned.
+(src/ninetoothed/auto_tuner.py:11-95).  Here the candidates are the
+kernel variants of ``libnt_hip.so`` -- GEMM instances, attention loop forms,
+conv2d paths: ``nt_tune_gemm`` / ``nt_tune_attention`` / ``nt_tune_conv2d`` time
+them on the caller's tensors, the library caches the winner per device and
+problem, and this module keeps that cache on disk in the reference's CSV format
+so that a new process starts tuned.
 
 ``NINETOOTHED_AMD_AUTOTUNE=0`` switches tuning off (launches then use the
 library's fixed preference order).
@@ -54,8 +55,43 @@ def load_once():
             runtime.library().nt_tune_cache_load(str(path).encode(), ctypes.byref(entries))
 
 
-def lookup(dtype, out_dtype, m, n, k, addmm):
-    return runtime.library().nt_tune_cache_lookup(dtype, out_dtype, m, n, k, int(addmm))
+def lookup_problem(kind, values):
+    """The recorded choice for a problem of program ``kind`` (``runtime.TUNE_*``), or -1."""
+    array = (ctypes.c_int * len(values))(*[int(v) for v in values])
+    return runtime.library().nt_tune_lookup(kind, array, len(values))
+
+
+def lookup(dtype, out_dtype, m, n, k, addmm, rhs_layout=0):
+    """The tuned GEMM instance, or -1.  ``rhs_layout``: 0 row-major ``[K, N]``, 1 transposed (``[N, K]`` storage), 2 other strides."""
+    return lookup_problem(runtime.TUNE_GEMM, (dtype, out_dtype, m, n, k, int(addmm), rhs_layout))
+
+
+def _save():
+    try:
+        CACHE_DIR.mkdir(parents=True, exist_ok=True)
+        runtime.library().nt_tune_cache_save(str(cache_path()).encode())
+    except OSError:
+        pass  # a read-only home directory only costs the persistence
+
+
+def tune_attention(q, k, v, is_causal, scale, o, dtype, iters=5):
+    """Times the loop variants of the attention kernel on these arguments.  Returns the variant, -1 when nothing
+    was timed (graph capture), -2 when the problem has no alternatives."""
+    best, best_ms = ctypes.c_int(-2), ctypes.c_float(0.0)
+    runtime.check(runtime.library().nt_tune_attention(runtime.current_stream(), q, k, v, is_causal, scale, o, dtype, iters, ctypes.byref(best), ctypes.byref(best_ms)))
+    if best.value >= 0:
+        _save()
+    return best.value
+
+
+def tune_conv2d(x, w, y, dtype, padding_h, padding_w, iters=5):
+    """Times the ways to run this convolution (one launch on the tensors as they lie, repacking pass plus GEMM loop,
+    gather kernel).  Returns the path (``block_size_m`` value that selects it), or -1 when nothing was timed."""
+    best, best_ms = ctypes.c_int(-1), ctypes.c_float(0.0)
+    runtime.check(runtime.library().nt_tune_conv2d(runtime.current_stream(), x, w, y, dtype, padding_h, padding_w, iters, ctypes.byref(best), ctypes.byref(best_ms)))
+    if best.value >= 0:
+        _save()
+    return best.value
 
 
 def tune(input, mat1, mat2, beta, alpha, output, dtype, out_dtype, iters=5):
@@ -69,11 +105,7 @@ def tune(input, mat1, mat2, beta, alpha, output, dtype, out_dtype, iters=5):
     )
     if best.value < 0:  # nothing was timed: the stream is being captured into a graph
         return best.value, best_ms.value
-    try:
-        CACHE_DIR.mkdir(parents=True, exist_ok=True)
-        lib.nt_tune_cache_save(str(cache_path()).encode())
-    except OSError:
-        pass  # a read-only home directory only costs the persistence
+    _save()
     return best.value, best_ms.value
 
 

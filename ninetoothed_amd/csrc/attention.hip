@@ -20,6 +20,7 @@
 #include <algorithm>
 
 #include "gemm_fast.h"  // swizzle helpers, static_for, lds_barrier
+#include "tune.h"
 #include "workspace.h"
 
 namespace nt {
@@ -879,16 +880,17 @@ int dispatch_attention(AttentionParams &p, int head_dim, int variant, hipStream_
 
 using namespace nt;
 
-extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineToothedTensor q, NineToothedTensor k,
-                                                 NineToothedTensor v, NineToothedTensor is_causal,
-                                                 NineToothedTensor scale, NineToothedTensor o, int dtype,
-                                                 int block_size_m, int block_size_n) {
+namespace nt {
+namespace {
+
+// validates the call and fills the parameters; returns 0, an error, or -1 when there is nothing to compute
+int attention_setup(AttentionParams &p, const NineToothedTensor &q, const NineToothedTensor &k, const NineToothedTensor &v,
+                    const NineToothedTensor &is_causal, const NineToothedTensor &scale, const NineToothedTensor &o, int dtype) {
     if (dtype != NINETOOTHED_FLOAT16 && dtype != NINETOOTHED_BFLOAT16 && dtype != NINETOOTHED_FLOAT32) return NINETOOTHED_NO_KERNEL;
     const bool float32 = dtype == NINETOOTHED_FLOAT32;
     const NineToothedTensor *ts[4] = {&q, &k, &v, &o};
     for (const NineToothedTensor *t : ts)
         if (!t->shape || !t->strides) return hipErrorInvalidValue;
-    AttentionParams p;
     p.parts = 1;
     p.blocks_per_part = 0;
     p.part_o = p.part_lse = nullptr;
@@ -912,7 +914,7 @@ extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineT
         if (t->strides[2] < 0) return NINETOOTHED_NO_KERNEL;
         if (((int64_t)t->shape[2] + 64) * t->strides[2] * 2 + 2 * head_dim > 0xffffffffll) return NINETOOTHED_NO_KERNEL;
     }
-    if (p.batch == 0 || p.heads == 0 || p.seq_q == 0) return 0;
+    if (p.batch == 0 || p.heads == 0 || p.seq_q == 0) return -1;
     if (p.seq_k == 0) return NINETOOTHED_NO_KERNEL;  // softmax over nothing
     for (int d = 0; d < 3; ++d) {
         p.q_strides[d] = q.strides[d];
@@ -933,26 +935,95 @@ extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineT
     if (scale.data) p.q_scale = (float)Scalar0d::as_double(scale) * 1.44269504089f;
     else p.q_scale = dtype == NINETOOTHED_FLOAT16 ? 1.4423828125f : (dtype == NINETOOTHED_BFLOAT16 ? 1.4453125f : 1.44269504089f);
     p.causal = is_causal.data ? (Scalar0d::as_int64(is_causal) != 0) : 0;
-    if (float32) return attention_float32(p, (int)head_dim, k, v, (hipStream_t)stream);
+    return 0;
+}
+
+constexpr int kAttentionVariants = 5;
+
+void attention_tune_values(const AttentionParams &p, int dtype, int (&values)[7]) {
+    const int v[7] = {dtype, p.batch, p.heads, p.seq_q, p.seq_k, p.head_dim, p.causal};
+    for (int i = 0; i < 7; ++i) values[i] = v[i];
+}
+
+// whether the variants are alternatives for this problem (they exist for head dimensions 64 and 128)
+bool attention_tunable(const AttentionParams &p, int dtype) { return dtype != NINETOOTHED_FLOAT32 && (p.head_dim == 128 || p.head_dim == 64); }
+
+// the key range is split instead (decoding-like shapes); returns NINETOOTHED_NO_KERNEL when that does not apply
+int attention_split(AttentionParams &p, int dtype, hipStream_t stream) {
+    if (p.head_dim != 128 && p.head_dim != 64) return NINETOOTHED_NO_KERNEL;
+    if (dtype == NINETOOTHED_FLOAT16) return p.head_dim == 128 ? launch_split_keys<half_t, 128>(p, stream) : launch_split_keys<half_t, 64>(p, stream);
+    if (dtype == NINETOOTHED_BFLOAT16) return p.head_dim == 128 ? launch_split_keys<bf16_t, 128>(p, stream) : launch_split_keys<bf16_t, 64>(p, stream);
+    return NINETOOTHED_NO_KERNEL;
+}
+
+bool attention_would_split(const AttentionParams &p) {
+    const int64_t groups = (int64_t)p.batch * p.heads * ceil_div(p.seq_q, kAttnWaves * 32);
+    const int key_blocks = ceil_div(p.seq_k, 64);
+    return groups > 0 && groups < 128 && key_blocks >= 8 && std::min<int64_t>((512 + groups - 1) / groups, key_blocks / 4) >= 2;
+}
+
+}  // namespace
+}  // namespace nt
+
+extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineToothedTensor q, NineToothedTensor k,
+                                                 NineToothedTensor v, NineToothedTensor is_causal,
+                                                 NineToothedTensor scale, NineToothedTensor o, int dtype,
+                                                 int block_size_m, int block_size_n) {
+    AttentionParams p;
+    const int status = attention_setup(p, q, k, v, is_causal, scale, o, dtype);
+    if (status != 0) return status < 0 ? 0 : status;
+    const int head_dim = p.head_dim;
+    if (dtype == NINETOOTHED_FLOAT32) return attention_float32(p, head_dim, k, v, (hipStream_t)stream);
     // block sizes are hints: 256 query rows select the one-workgroup-per-CU variant, 32-key blocks the
-    // three-workgroups-per-CU variant, 64-key blocks the plain loop.  Without a hint the pipelined loop
-    // runs (measured at [4, 32, 4096, 128]: 1.12 against 1.08 PFLOP/s for the plain loop, causal 1.01
-    // against 0.98); non-causal problems with enough 256-row blocks to fill the chip twice run it with
-    // eight waves per workgroup, which loads every K / V block once for 256 query rows (1.16 PFLOP/s;
-    // causal 0.99, below the four-wave form).
+    // three-workgroups-per-CU variant, 64-key blocks the plain loop.  Without a hint the choice is the one
+    // tuned for this problem (nt_tune_attention), else the pipelined loop (measured at [4, 32, 4096, 128]:
+    // 1.12 against 1.08 PFLOP/s for the plain loop, causal 1.01 against 0.98); non-causal problems with enough
+    // 256-row blocks to fill the chip twice run it with eight waves per workgroup, which loads every K / V
+    // block once for 256 query rows (1.16 PFLOP/s; causal 0.99, below the four-wave form).
     int variant = block_size_m >= 256 ? 1 : (block_size_n > 0 && block_size_n <= 32 ? 2 : (block_size_n >= 64 ? 0 : 3));
     if (variant == 3 && !p.causal && block_size_m == 0 && head_dim >= 64 && (int64_t)p.batch * p.heads * ceil_div(p.seq_q, 256) >= 512) variant = 4;
 #ifdef NT_MEASUREMENT_AIDS
     if (block_size_n >= 1000) variant = block_size_n - 1000;  // explicit variant, for timing harnesses only
 #endif
-    if (block_size_m == 0 && block_size_n == 0 && (head_dim == 128 || head_dim == 64)) {  // no hints: decoding-like shapes split the keys
-        int result;
-        if (dtype == NINETOOTHED_FLOAT16)
-            result = head_dim == 128 ? launch_split_keys<half_t, 128>(p, (hipStream_t)stream) : launch_split_keys<half_t, 64>(p, (hipStream_t)stream);
-        else
-            result = head_dim == 128 ? launch_split_keys<bf16_t, 128>(p, (hipStream_t)stream) : launch_split_keys<bf16_t, 64>(p, (hipStream_t)stream);
+    if (block_size_m == 0 && block_size_n == 0) {  // no hints
+        const int result = attention_split(p, dtype, (hipStream_t)stream);  // decoding-like shapes split the keys
         if (result != NINETOOTHED_NO_KERNEL) return result;
+        if (attention_tunable(p, dtype)) {
+            int values[7];
+            attention_tune_values(p, dtype, values);
+            const int tuned = tune_lookup(kTuneAttention, values, 7);
+            if (tuned >= 0 && tuned < kAttentionVariants) variant = tuned;
+        }
     }
-    if (dtype == NINETOOTHED_FLOAT16) return dispatch_attention<half_t>(p, (int)head_dim, variant, (hipStream_t)stream);
-    return dispatch_attention<bf16_t>(p, (int)head_dim, variant, (hipStream_t)stream);
+    if (dtype == NINETOOTHED_FLOAT16) return dispatch_attention<half_t>(p, head_dim, variant, (hipStream_t)stream);
+    return dispatch_attention<bf16_t>(p, head_dim, variant, (hipStream_t)stream);
+}
+
+// Times the loop variants of launch_nt_attention on this problem and records the fastest for later launches
+// without block-size hints.  *best_variant = -1 when nothing was timed (a stream under graph capture), -2 when
+// the problem has no alternatives (fp32 tensors, head dimensions other than 64 and 128, shapes that split the keys).
+extern "C" NineToothedResult nt_tune_attention(NineToothedStream stream, NineToothedTensor q, NineToothedTensor k, NineToothedTensor v,
+                                               NineToothedTensor is_causal, NineToothedTensor scale, NineToothedTensor o, int dtype,
+                                               int iters, int *best_variant, float *best_ms) {
+    if (best_variant) *best_variant = -2;
+    if (best_ms) *best_ms = 0.0f;
+    AttentionParams p;
+    const int status = attention_setup(p, q, k, v, is_causal, scale, o, dtype);
+    if (status != 0) return status < 0 ? 0 : status;
+    if (!attention_tunable(p, dtype) || attention_would_split(p)) return 0;
+    int best = -1;
+    float best_time = 0.0f;
+    const int result = tune_time((hipStream_t)stream, kAttentionVariants, iters, [&](int variant) -> int {
+        AttentionParams copy = p;
+        if (dtype == NINETOOTHED_FLOAT16) return dispatch_attention<half_t>(copy, p.head_dim, variant, (hipStream_t)stream);
+        return dispatch_attention<bf16_t>(copy, p.head_dim, variant, (hipStream_t)stream);
+    }, &best, &best_time);
+    if (result != 0) return result;
+    if (best_variant) *best_variant = best;
+    if (best < 0) return 0;
+    int values[7];
+    attention_tune_values(p, dtype, values);
+    tune_record(kTuneAttention, values, 7, best);
+    if (best_ms) *best_ms = best_time;
+    return 0;
 }

@@ -13,6 +13,7 @@
 #include "conv2d.h"
 #include "gemm_fast.h"
 #include "gemm_generic.h"
+#include "tune.h"
 #include "workspace.h"
 
 namespace nt {
@@ -357,35 +358,18 @@ static_assert(kNumInstances > kSplit256x256x32, "InstanceIndex names the first i
 
 inline bool is_split(int instance) { return instance >= kSplit64x64x64 && instance <= kSplit256x256x32; }
 
-// ---- per-device cache of tuned choices (device, problem signature) -> instance ----
-struct TuneKey {
-    int device, dtype, out_dtype, m, n, k, addmm;
-    bool operator==(const TuneKey &o) const {
-        return device == o.device && dtype == o.dtype && out_dtype == o.out_dtype && m == o.m && n == o.n && k == o.k && addmm == o.addmm;
-    }
-};
-struct TuneKeyHash {
-    size_t operator()(const TuneKey &x) const {
-        size_t h = 1469598103934665603ull;
-        const int v[] = {x.device, x.dtype, x.out_dtype, x.m, x.n, x.k, x.addmm};
-        for (int e : v) h = (h ^ (size_t)(unsigned)e) * 1099511628211ull;
-        return h;
-    }
-};
-std::shared_mutex g_tune_mutex;
-std::unordered_map<TuneKey, int, TuneKeyHash> g_tuned;
-
-TuneKey make_key(const GemmProblem &q) {
-    int device = 0;
-    (void)hipGetDevice(&device);
-    return TuneKey{device, q.dtype, q.out_dtype, q.m, q.n, q.k, q.addmm() ? 1 : 0};
+// ---- tuned choices: (dtype, output dtype, M, N, K, addmm, rhs layout) -> instance ----
+void tune_values(const GemmProblem &q, int (&values)[7]) {
+    const int layout = b_is_transposed(q) ? 1 : (q.sbn == 1 ? 0 : 2);  // rhs row-major, transposed, other strides
+    const int v[7] = {q.dtype, q.out_dtype, q.m, q.n, q.k, q.addmm() ? 1 : 0, layout};
+    for (int i = 0; i < 7; ++i) values[i] = v[i];
 }
 
 int lookup_tuned(const GemmProblem &q) {
-    const TuneKey key = make_key(q);
-    std::shared_lock<std::shared_mutex> lock(g_tune_mutex);
-    auto it = g_tuned.find(key);
-    return it == g_tuned.end() ? -1 : it->second;
+    int values[7];
+    tune_values(q, values);
+    const int choice = tune_lookup(kTuneGemm, values, 7);
+    return choice >= 0 && choice < kNumInstances ? choice : -1;
 }
 
 // Untuned choice: the largest direct-to-LDS tile that still gives every CU a
@@ -590,139 +574,43 @@ NineToothedResult nt_tune_gemm(NineToothedStream stream_, NineToothedTensor inpu
     hipStream_t stream = (hipStream_t)stream_;
     GemmProblem q;
     if (int err = build_problem(q, &input, mat1, mat2, &beta, &alpha, output, dtype, output_dtype)) return err;
-    if (iters <= 0) iters = 5;
-    if (best_config) *best_config = -1;
-    if (best_ms) *best_ms = 0.0f;
-    // timing needs event synchronisation and rewrites the output several times: not inside a graph
-    // capture.  The problem stays untuned (launches use the fixed preference order) and nothing is recorded.
-    if (stream_is_capturing(stream)) return 0;
-    hipEvent_t start, stop;
-    hipError_t err;
-    if ((err = hipEventCreate(&start)) != hipSuccess) return (int)err;
-    if ((err = hipEventCreate(&stop)) != hipSuccess) {
-        (void)hipEventDestroy(start);
-        return (int)err;
-    }
     int best = -1;
     float best_time = 0.0f;
-    for (int i = 0; i < kNumInstances && err == hipSuccess; ++i) {
-        if (!kInstances[i].accepts(q)) continue;
-        for (int w = 0; w < 2 && err == hipSuccess; ++w) err = kInstances[i].launch(q, stream);
-        if (err != hipSuccess) break;
-        (void)hipEventRecord(start, stream);
-        for (int r = 0; r < iters && err == hipSuccess; ++r) err = kInstances[i].launch(q, stream);
-        (void)hipEventRecord(stop, stream);
-        if (err != hipSuccess) break;
-        if ((err = hipEventSynchronize(stop)) != hipSuccess) break;
-        float ms = 0.0f;
-        (void)hipEventElapsedTime(&ms, start, stop);
-        ms /= (float)iters;
-        if (best < 0 || ms < best_time) {
-            best = i;
-            best_time = ms;
-        }
-    }
-    (void)hipEventDestroy(start);
-    (void)hipEventDestroy(stop);
-    if (err != hipSuccess) return (int)err;
-    if (best < 0) return NINETOOTHED_NO_KERNEL;
-    {
-        std::unique_lock<std::shared_mutex> lock(g_tune_mutex);
-        g_tuned[make_key(q)] = best;
-    }
+    // (inside a graph capture nothing is timed: the problem stays on the fixed preference order and nothing is recorded)
+    const int result = tune_time(stream, kNumInstances, iters, [&](int i) -> int {
+        if (!kInstances[i].accepts(q)) return NINETOOTHED_NO_KERNEL;
+        return (int)kInstances[i].launch(q, stream);
+    }, &best, &best_time);
     if (best_config) *best_config = best;
     if (best_ms) *best_ms = best_time;
+    if (result != 0) return result;
+    if (best < 0) return stream_is_capturing(stream) ? 0 : NINETOOTHED_NO_KERNEL;
+    int values[7];
+    tune_values(q, values);
+    const int blocks[3] = {kInstances[best].bm, kInstances[best].bn, kInstances[best].bk};
+    tune_record(kTuneGemm, values, 7, best, blocks, 3);
     return 0;
 }
 
-// On-disk form of the tuned choices: the line-pair CSV the reference's AutoTuningCache reads
-// (src/ninetoothed/templates/auto_tuning_cache.h:27-75; written by src/ninetoothed/build.py:683-703):
-// a line of integers describing the problem, then a line of integers with the choice; the first
-// pair has an empty problem line and carries the default.  Problem = dtype, output dtype, M, N, K,
-// addmm flag; choice = block M, block N, block K, instance index.
-NineToothedResult nt_tune_cache_save(const char *path) {
-    if (path == nullptr) return hipErrorInvalidValue;
-    int device = 0;
-    (void)hipGetDevice(&device);
-    FILE *file = fopen(path, "w");
-    if (file == nullptr) return hipErrorInvalidValue;
-    const GemmInstance &fallback = kInstances[k256x256x32];
-    fprintf(file, "\n%d,%d,%d,%d\n", fallback.bm, fallback.bn, fallback.bk, (int)k256x256x32);
-    {
-        std::shared_lock<std::shared_mutex> lock(g_tune_mutex);
-        for (const auto &entry : g_tuned) {
-            const TuneKey &key = entry.first;
-            if (key.device != device || entry.second < 0 || entry.second >= kNumInstances) continue;
-            const GemmInstance &instance = kInstances[entry.second];
-            fprintf(file, "%d,%d,%d,%d,%d,%d\n%d,%d,%d,%d\n", key.dtype, key.out_dtype, key.m, key.n, key.k, key.addmm, instance.bm,
-                    instance.bn, instance.bk, entry.second);
-        }
-    }
-    return fclose(file) == 0 ? 0 : (int)hipErrorInvalidValue;
-}
-
-// Reads such a file into the cache of the current device.  *entries (may be NULL) receives the
-// number of choices taken over; lines that do not parse, or name an instance this build does not
-// have, are skipped.
-NineToothedResult nt_tune_cache_load(const char *path, int *entries) {
-    if (entries) *entries = 0;
-    if (path == nullptr) return hipErrorInvalidValue;
-    FILE *file = fopen(path, "r");
-    if (file == nullptr) return hipErrorInvalidValue;
-    int device = 0;
-    (void)hipGetDevice(&device);
-    auto parse = [](const char *line, std::vector<long> &values) {
-        values.clear();
-        const char *cursor = line;
-        while (*cursor) {
-            while (*cursor == ' ' || *cursor == '\t' || *cursor == '\r' || *cursor == '\n' || *cursor == ',') ++cursor;
-            if (!*cursor) break;
-            char *end = nullptr;
-            const long value = strtol(cursor, &end, 10);
-            if (end == cursor) return false;
-            values.push_back(value);
-            cursor = end;
-        }
-        return true;
-    };
-    char problem_line[512], choice_line[512];
-    std::vector<long> problem, choice;
-    bool first = true;
-    int taken = 0;
-    while (fgets(problem_line, sizeof(problem_line), file) && fgets(choice_line, sizeof(choice_line), file)) {
-        const bool parsed = parse(problem_line, problem) && parse(choice_line, choice);
-        if (first) {  // the default pair
-            first = false;
-            continue;
-        }
-        if (!parsed || problem.size() != 6 || choice.size() != 4) continue;
-        const int instance = (int)choice[3];
-        if (instance < 0 || instance >= kNumInstances) continue;
-        if (kInstances[instance].bm != choice[0] || kInstances[instance].bn != choice[1] || kInstances[instance].bk != choice[2]) continue;
-        TuneKey key{device, (int)problem[0], (int)problem[1], (int)problem[2], (int)problem[3], (int)problem[4], (int)problem[5]};
-        std::unique_lock<std::shared_mutex> lock(g_tune_mutex);
-        g_tuned[key] = instance;
-        ++taken;
-    }
-    fclose(file);
-    if (entries) *entries = taken;
-    return 0;
-}
-
-// The cached choice for a problem given by its sizes (no tensors needed): instance index, or -1.
+// The cached instance for a problem given by its sizes (row-major rhs), or -1.
 int nt_tune_cache_lookup(int dtype, int output_dtype, int m, int n, int k, int addmm) {
-    int device = 0;
-    (void)hipGetDevice(&device);
-    std::shared_lock<std::shared_mutex> lock(g_tune_mutex);
-    auto it = g_tuned.find(TuneKey{device, dtype, output_dtype, m, n, k, addmm ? 1 : 0});
-    return it == g_tuned.end() ? -1 : it->second;
+    const int values[7] = {dtype, output_dtype, m, n, k, addmm ? 1 : 0, 0};
+    const int choice = tune_lookup(kTuneGemm, values, 7);
+    return choice >= 0 && choice < kNumInstances ? choice : -1;
 }
 
-NineToothedResult launch_nt_conv2d(NineToothedStream stream, NineToothedTensor input, NineToothedTensor filter,
-                                   NineToothedTensor output, int dtype, int padding_h, int padding_w, int block_size_m,
-                                   int block_size_n, int block_size_k) {
-    (void)block_size_n;
-    (void)block_size_k;
+}  // extern "C"
+
+namespace nt {
+namespace {
+
+// the ways to run a convolution; kConvAuto tries them from the top (a 1 x 1 filter without padding first runs
+// as a batch of plain products when it can)
+enum ConvPath { kConvAuto = 0, kConvGather = 1, kConvRepack = 2, kConvDirect = 3 };
+
+// validates the call and fills the request; returns 0, an error, or -1 when there is nothing to compute
+int conv2d_request(Conv2dRequest &request, const NineToothedTensor &input, const NineToothedTensor &filter, const NineToothedTensor &output,
+                   int dtype, int padding_h, int padding_w) {
     if (dtype != NINETOOTHED_FLOAT16 && dtype != NINETOOTHED_BFLOAT16) return NINETOOTHED_NO_KERNEL;
     if (!input.shape || !filter.shape || !output.shape || !input.strides || !filter.strides || !output.strides)
         return hipErrorInvalidValue;
@@ -733,85 +621,135 @@ NineToothedResult launch_nt_conv2d(NineToothedStream stream, NineToothedTensor i
     const int64_t P = H + 2 * padding_h - R + 1, Q = W + 2 * padding_w - S + 1;
     if ((int64_t)output.shape[0] != N || (int64_t)output.shape[1] != K) return hipErrorInvalidValue;
     if ((int64_t)output.shape[2] != P || (int64_t)output.shape[3] != Q) return hipErrorInvalidValue;
-    if (P <= 0 || Q <= 0 || N == 0 || K == 0) return 0;  // nothing to write
-    const int64_t gm = N * P * Q, gk = C * R * S;
-    if (gm > 0x7fffffffll || gk > 0x7fffffffll || K > 0x7fffffffll) return NINETOOTHED_NO_KERNEL;
-    {
-        Conv2dRequest request;
-        request.dtype = dtype;
-        request.x = input.data;
-        request.w = filter.data;
-        request.y = output.data;
-        request.N = (int)N; request.C = (int)C; request.H = (int)H; request.W = (int)W;
-        request.K = (int)K; request.R = (int)R; request.S = (int)S; request.P = (int)P; request.Q = (int)Q;
-        request.pad_h = padding_h; request.pad_w = padding_w;
-        for (int d = 0; d < 4; ++d) {
-            request.xs[d] = input.strides[d];
-            request.ws[d] = filter.strides[d];
-            request.ys[d] = output.strides[d];
-        }
-        // 1 x 1 filters without padding: per image Y[K, P*Q] = W[K, C] . X[C, P*Q], a batch of row-major
-        // products on the tensors as they lie (no repacking, no scratch memory)
-        if (block_size_m != 1 && R == 1 && S == 1 && padding_h == 0 && padding_w == 0 && input.strides[3] == 1 && input.strides[2] == W &&
-            output.strides[3] == 1 && output.strides[2] == Q && filter.strides[1] == 1 && N <= 0x7fffffffll) {
-            GemmProblem q;
-            q.dtype = q.out_dtype = dtype;
-            q.m = (int)K;
-            q.n = (int)(P * Q);
-            q.k = (int)C;
-            q.a = filter.data;
-            q.b = input.data;
-            q.c = output.data;
-            q.bias = nullptr;
-            q.sam = filter.strides[0]; q.sak = 1;
-            q.sbk = input.strides[1]; q.sbn = 1;
-            q.scm = output.strides[1]; q.scn = 1;
-            q.sim = q.sin = 0;
-            q.alpha = 1.0f; q.beta = 0.0f;
-            q.batch = (int)N;
-            q.a_batch = 0;
-            q.b_batch = input.strides[0];
-            q.c_batch = output.strides[0];
-            const int choice = heuristic_choice(q, 0, 0, 0);
-            if (choice > kAnyStride && !is_split(choice)) return (int)kInstances[choice].launch(q, (hipStream_t)stream);
-        }
-        // block_size_m: 1 = the gather kernel, 2 = the repacking path; otherwise the library's choice
-        if (block_size_m != 1 && block_size_m != 2) {
-            const int direct = conv2d_direct(request, (hipStream_t)stream);
-            if (direct != NINETOOTHED_NO_KERNEL) return direct;
-        }
-        const int fast = block_size_m == 1 ? NINETOOTHED_NO_KERNEL : conv2d_fast(request, (hipStream_t)stream);
-        if (fast != NINETOOTHED_NO_KERNEL) return fast;
+    if (P <= 0 || Q <= 0 || N == 0 || K == 0) return -1;  // nothing to write
+    if (N * P * Q > 0x7fffffffll || C * R * S > 0x7fffffffll || K > 0x7fffffffll || N > 0x7fffffffll) return NINETOOTHED_NO_KERNEL;
+    request.dtype = dtype;
+    request.x = input.data;
+    request.w = filter.data;
+    request.y = output.data;
+    request.N = (int)N; request.C = (int)C; request.H = (int)H; request.W = (int)W;
+    request.K = (int)K; request.R = (int)R; request.S = (int)S; request.P = (int)P; request.Q = (int)Q;
+    request.pad_h = padding_h; request.pad_w = padding_w;
+    for (int d = 0; d < 4; ++d) {
+        request.xs[d] = input.strides[d];
+        request.ws[d] = filter.strides[d];
+        request.ys[d] = output.strides[d];
     }
-    auto launch = [&](auto tag) -> hipError_t {
-        typedef decltype(tag) T;
-        Conv2dProblem<T> prob;
-        prob.m = (int)gm;
-        prob.n = (int)K;
-        prob.k = (int)gk;
-        prob.x = (const T *)input.data;
-        prob.w = (const T *)filter.data;
-        prob.y = (T *)output.data;
-        prob.C = (int)C;
-        prob.H = (int)H;
-        prob.W = (int)W;
-        prob.R = (int)R;
-        prob.S = (int)S;
-        prob.P = (int)P;
-        prob.Q = (int)Q;
-        prob.pad_h = padding_h;
-        prob.pad_w = padding_w;
-        for (int d = 0; d < 4; ++d) {
-            prob.xs[d] = input.strides[d];
-            prob.ws[d] = filter.strides[d];
-            prob.ys[d] = output.strides[d];
-        }
-        const int64_t tiles = (int64_t)ceil_div(prob.m, kGenBM) * ceil_div(prob.n, kGenBN);
-        gemm_generic_kernel<Conv2dProblem<T>><<<dim3((unsigned)tiles), dim3(kGenThreads), 0, (hipStream_t)stream>>>(prob);
-        return hipGetLastError();
-    };
-    if (dtype == NINETOOTHED_FLOAT16) return (int)launch(half_t());
-    return (int)launch(bf16_t());
+    return 0;
+}
+
+template <typename T>
+hipError_t conv2d_gather(const Conv2dRequest &r, hipStream_t stream) {
+    Conv2dProblem<T> prob;
+    prob.m = r.N * r.P * r.Q;
+    prob.n = r.K;
+    prob.k = r.C * r.R * r.S;
+    prob.x = (const T *)r.x;
+    prob.w = (const T *)r.w;
+    prob.y = (T *)r.y;
+    prob.C = r.C; prob.H = r.H; prob.W = r.W; prob.R = r.R; prob.S = r.S; prob.P = r.P; prob.Q = r.Q;
+    prob.pad_h = r.pad_h;
+    prob.pad_w = r.pad_w;
+    for (int d = 0; d < 4; ++d) {
+        prob.xs[d] = r.xs[d];
+        prob.ws[d] = r.ws[d];
+        prob.ys[d] = r.ys[d];
+    }
+    const int64_t tiles = (int64_t)ceil_div(prob.m, kGenBM) * ceil_div(prob.n, kGenBN);
+    gemm_generic_kernel<Conv2dProblem<T>><<<dim3((unsigned)tiles), dim3(kGenThreads), 0, stream>>>(prob);
+    return hipGetLastError();
+}
+
+int conv2d_run(const Conv2dRequest &r, int path, hipStream_t stream) {
+    // 1 x 1 filters without padding: per image Y[K, P*Q] = W[K, C] . X[C, P*Q], a batch of row-major
+    // products on the tensors as they lie (no repacking, no scratch memory)
+    if (path == kConvAuto && r.R == 1 && r.S == 1 && r.pad_h == 0 && r.pad_w == 0 && r.xs[3] == 1 && r.xs[2] == r.W && r.ys[3] == 1 &&
+        r.ys[2] == r.Q && r.ws[1] == 1) {
+        GemmProblem q;
+        q.dtype = q.out_dtype = r.dtype;
+        q.m = r.K;
+        q.n = r.P * r.Q;
+        q.k = r.C;
+        q.a = r.w;
+        q.b = r.x;
+        q.c = r.y;
+        q.bias = nullptr;
+        q.sam = r.ws[0]; q.sak = 1;
+        q.sbk = r.xs[1]; q.sbn = 1;
+        q.scm = r.ys[1]; q.scn = 1;
+        q.sim = q.sin = 0;
+        q.alpha = 1.0f; q.beta = 0.0f;
+        q.batch = r.N;
+        q.a_batch = 0;
+        q.b_batch = r.xs[0];
+        q.c_batch = r.ys[0];
+        const int choice = heuristic_choice(q, 0, 0, 0);
+        if (choice > kAnyStride && !is_split(choice)) return (int)kInstances[choice].launch(q, stream);
+    }
+    if (path == kConvAuto || path == kConvDirect) {
+        const int direct = conv2d_direct(r, stream);
+        if (direct != NINETOOTHED_NO_KERNEL || path == kConvDirect) return direct;
+    }
+    if (path == kConvAuto || path == kConvRepack) {
+        const int fast = conv2d_fast(r, stream);
+        if (fast != NINETOOTHED_NO_KERNEL || path == kConvRepack) return fast;
+    }
+    return r.dtype == NINETOOTHED_FLOAT16 ? (int)conv2d_gather<half_t>(r, stream) : (int)conv2d_gather<bf16_t>(r, stream);
+}
+
+void conv2d_tune_values(const Conv2dRequest &r, int (&values)[11]) {
+    const int dense_x = r.xs[3] == 1 && r.xs[2] == r.W && r.xs[1] == (int64_t)r.H * r.W && r.xs[0] == (int64_t)r.C * r.H * r.W;
+    const int v[11] = {r.dtype, r.N, r.C, r.H, r.W, r.K, r.R, r.S, r.pad_h, r.pad_w, dense_x};
+    for (int i = 0; i < 11; ++i) values[i] = v[i];
+}
+
+}  // namespace
+}  // namespace nt
+
+extern "C" {
+
+NineToothedResult launch_nt_conv2d(NineToothedStream stream, NineToothedTensor input, NineToothedTensor filter,
+                                   NineToothedTensor output, int dtype, int padding_h, int padding_w, int block_size_m,
+                                   int block_size_n, int block_size_k) {
+    (void)block_size_n;
+    (void)block_size_k;
+    Conv2dRequest request;
+    const int status = conv2d_request(request, input, filter, output, dtype, padding_h, padding_w);
+    if (status != 0) return status < 0 ? 0 : status;
+    // block_size_m: 1 = the gather kernel, 2 = the repacking path, 3 = the one-launch path; otherwise the
+    // tuned choice for this problem, else the library's order
+    int path = block_size_m >= kConvGather && block_size_m <= kConvDirect ? block_size_m : kConvAuto;
+    if (block_size_m == 0) {
+        int values[11];
+        conv2d_tune_values(request, values);
+        const int tuned = tune_lookup(kTuneConv2d, values, 11);
+        if (tuned >= kConvGather && tuned <= kConvDirect) path = tuned;
+    }
+    int result = conv2d_run(request, path, (hipStream_t)stream);
+    // (a tuned path that needs scratch memory it cannot get, e.g. under graph capture: the library's order)
+    if (result == NINETOOTHED_NO_KERNEL && path != kConvAuto && block_size_m == 0) result = conv2d_run(request, kConvAuto, (hipStream_t)stream);
+    return result;
+}
+
+NineToothedResult nt_tune_conv2d(NineToothedStream stream, NineToothedTensor input, NineToothedTensor filter, NineToothedTensor output,
+                                 int dtype, int padding_h, int padding_w, int iters, int *best_path, float *best_ms) {
+    if (best_path) *best_path = -1;
+    if (best_ms) *best_ms = 0.0f;
+    Conv2dRequest request;
+    const int status = conv2d_request(request, input, filter, output, dtype, padding_h, padding_w);
+    if (status != 0) return status < 0 ? 0 : status;
+    int values[11];
+    conv2d_tune_values(request, values);
+    const int paths[3] = {kConvDirect, kConvRepack, kConvGather};
+    int best = -1;
+    float best_time = 0.0f;
+    const int result = tune_time((hipStream_t)stream, 3, iters, [&](int i) -> int { return conv2d_run(request, paths[i], (hipStream_t)stream); }, &best, &best_time);
+    if (result != 0) return result;
+    if (best < 0) return 0;  // (a stream under graph capture: nothing was timed)
+    tune_record(kTuneConv2d, values, 11, paths[best]);
+    if (best_path) *best_path = paths[best];
+    if (best_ms) *best_ms = best_time;
+    return 0;
 }
 
 #ifdef NT_GEMM_ABLATION

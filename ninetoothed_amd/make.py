@@ -317,7 +317,8 @@ class Kernel:
         state = {"tune": blocks == [0, 0, 0] and min(m, n, k) > 0 and auto_tuner.enabled()}
         if state["tune"]:
             auto_tuner.load_once()
-            state["tune"] = auto_tuner.lookup(dtype, out_dtype, m, n, k, i is not None) < 0
+            rhs_layout = 0 if b_arg.strides[1] == 1 else (1 if b_arg.strides[0] == 1 else 2)
+            state["tune"] = auto_tuner.lookup(dtype, out_dtype, m, n, k, i is not None, rhs_layout) < 0
 
         def maybe_tune(call_args, input_arg, beta, alpha):
             state["tune"] = False
@@ -363,8 +364,21 @@ class Kernel:
         pad_h, pad_w = info["pad_h"], info["pad_w"]
         blocks = [info["blocks"][axis] if info["blocks"][axis] > 1 else 0 for axis in ("m", "n", "k")]
 
+        from ninetoothed_amd import auto_tuner
+
+        # block sizes left to the tuner: the first launch of a new problem times the ways to run it
+        state = {"tune": blocks == [0, 0, 0] and auto_tuner.enabled()}
+        if state["tune"]:
+            auto_tuner.load_once()
+
         def launch(call_args):
             x, w, y = (runtime.ArgumentTensor.from_torch_tensor(tensor) for tensor in call_args)
+            if state["tune"]:
+                state["tune"] = False
+                out = call_args[2]
+                if all(t.untyped_storage().data_ptr() != out.untyped_storage().data_ptr() for t in call_args[:2]):
+                    # (timing launches rewrite the output; inside a graph capture nothing is timed: try again later)
+                    state["tune"] = auto_tuner.tune_conv2d(x, w, y, dtype, pad_h, pad_w) == -1
             runtime.check(lib.launch_nt_conv2d(runtime.current_stream(), x, w, y, dtype, pad_h, pad_w, *blocks))
 
         return _Plan(f"launch_nt_conv2d gemm {info['m']}x{info['n']}x{info['k']} {tag} padding ({pad_h}, {pad_w})", launch)
@@ -481,11 +495,24 @@ class Kernel:
         lib = runtime.library()
         dtype = runtime.DATA_TYPE_INDEX[tag]
         o_pos = 5 if scaled else 4
+        from ninetoothed_amd import auto_tuner
+
+        # the first launch of a new problem times the loop variants (as the reference's autotuned kernel times its
+        # block-size configurations, tests/test_attention.py:10-11 with src/ninetoothed/generation.py:372-516)
+        state = {"tune": auto_tuner.enabled()}
+        if state["tune"]:
+            auto_tuner.load_once()
 
         def launch(call_args):
             tensors = [runtime.ArgumentTensor.from_torch_tensor(call_args[p]) for p in (0, 1, 2, o_pos)]
             causal = runtime.ArgumentTensor.from_scalar(int(bool(call_args[3])))
             scale_arg = runtime.ArgumentTensor.from_scalar(float(call_args[4])) if scaled else runtime.ArgumentTensor.null()
+            if state["tune"]:
+                state["tune"] = False
+                out = call_args[o_pos]
+                if all(call_args[p].untyped_storage().data_ptr() != out.untyped_storage().data_ptr() for p in (0, 1, 2)):
+                    # (timing launches rewrite the output; inside a graph capture nothing is timed: try again later)
+                    state["tune"] = auto_tuner.tune_attention(tensors[0], tensors[1], tensors[2], causal, scale_arg, tensors[3], dtype) == -1
             runtime.check(lib.launch_nt_attention(runtime.current_stream(), tensors[0], tensors[1], tensors[2], causal, scale_arg, tensors[3], dtype, 0, 0))
 
         return _Plan(f"launch_nt_attention q{info['q']['shape']} k{info['k']['shape']} {tag}", launch)

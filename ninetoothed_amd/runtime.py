@@ -17,6 +17,8 @@ import threading
 LIBRARY_PATH = pathlib.Path(__file__).resolve().parent / "lib" / "libnt_hip.so"
 
 NO_KERNEL = 1
+# programs of the tuned-choice table (nt_tune_lookup, the cache file's problem lines)
+TUNE_GEMM, TUNE_ATTENTION, TUNE_CONV2D = 0, 1, 2
 SCRATCH_LIMIT = 2  # launch_nt_matmul_static_scratch: the call needs more than the fixed scratch array
 STATIC_SCRATCH_BYTES = 16 << 20
 
@@ -79,6 +81,9 @@ _SIGNATURES = {
     "launch_nt_conv2d": (_S, _T, _T, _T, _I, _I, _I, _I, _I, _I),
     "launch_nt_gemm_config": (_S, _I, _T, _T, _T, _T, _T, _T, _I, _I),
     "nt_tune_gemm": (_S, _T, _T, _T, _T, _T, _T, _I, _I, _I, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_float)),
+    "nt_tune_attention": (_S, _T, _T, _T, _T, _T, _T, _I, _I, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_float)),
+    "nt_tune_conv2d": (_S, _T, _T, _T, _I, _I, _I, _I, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_float)),
+    "nt_tune_lookup": (_I, ctypes.POINTER(ctypes.c_int), _I),
     "launch_nt_map": (_S, ctypes.c_void_p),
     "nt_map_source": (ctypes.c_void_p, ctypes.c_char_p, _I),
     "nt_tune_cache_save": (ctypes.c_char_p,),

@@ -76,11 +76,12 @@ def test_requests_without_a_kernel_are_refused_on_the_host():
 
 def test_tuning_cache_reads_and_writes_the_reference_csv_format(tmp_path):
     # the file layout of src/ninetoothed/build.py:683-703 (csv.writer rows: an empty row and the
-    # default first, then problem / choice pairs), read by templates/auto_tuning_cache.h:27-75
+    # default first, then problem / choice pairs), read by templates/auto_tuning_cache.h:27-75;
+    # a problem row starts with the program (0 matmul / addmm, 1 attention, 2 conv2d)
     import csv
     import ctypes
 
-    from ninetoothed_amd import runtime
+    from ninetoothed_amd import auto_tuner, runtime
 
     lib = runtime.library()
     names = runtime.gemm_config_names()
@@ -90,23 +91,38 @@ def test_tuning_cache_reads_and_writes_the_reference_csv_format(tmp_path):
     with open(path, "w") as handle:
         writer = csv.writer(handle)
         writer.writerow(())
-        writer.writerow((256, 256, 32, fast))
-        writer.writerow((fp16, fp16, 4096, 2048, 1024, 1))
-        writer.writerow((256, 256, 32, fast))
-        writer.writerow((fp16, fp16, 64, 64, 64, 0))
-        writer.writerow((7, 7, 7, 999))  # an instance this build does not have: skipped
+        writer.writerow((0,))
+        writer.writerow((runtime.TUNE_GEMM, fp16, fp16, 4096, 2048, 1024, 1, 0))
+        writer.writerow((fast, 256, 256, 32))
+        writer.writerow((runtime.TUNE_GEMM, fp16, fp16, 4096, 2048, 1024, 1, 1))  # the same sizes with a transposed rhs
+        writer.writerow((fast + 1, 256, 256, 64))
+        writer.writerow((runtime.TUNE_ATTENTION, fp16, 4, 32, 4096, 4096, 128, 1))
+        writer.writerow((3,))
+        writer.writerow((runtime.TUNE_CONV2D, fp16, 32, 256, 56, 56, 256, 3, 3, 1, 1, 1))
+        writer.writerow((2,))
+        writer.writerow((7, 1, 2, 3))  # a program this build does not have: skipped
+        writer.writerow((1,))
+        writer.writerow((runtime.TUNE_GEMM, fp16, fp16, 64, 64, 64, 0, 0))
+        writer.writerow((-5,))  # no choice: skipped
     entries = ctypes.c_int(-1)
     assert lib.nt_tune_cache_load(str(path).encode(), ctypes.byref(entries)) == 0
-    assert entries.value == 1
+    assert entries.value == 4
     assert lib.nt_tune_cache_lookup(fp16, fp16, 4096, 2048, 1024, 1) == fast
+    assert auto_tuner.lookup(fp16, fp16, 4096, 2048, 1024, True, rhs_layout=1) == fast + 1
     assert lib.nt_tune_cache_lookup(fp16, fp16, 64, 64, 64, 0) == -1
     assert lib.nt_tune_cache_lookup(fp16, fp16, 4096, 2048, 1024, 0) == -1
+    assert auto_tuner.lookup_problem(runtime.TUNE_ATTENTION, (fp16, 4, 32, 4096, 4096, 128, 1)) == 3
+    assert auto_tuner.lookup_problem(runtime.TUNE_ATTENTION, (fp16, 4, 32, 4096, 4096, 128, 0)) == -1
+    assert auto_tuner.lookup_problem(runtime.TUNE_CONV2D, (fp16, 32, 256, 56, 56, 256, 3, 3, 1, 1, 1)) == 2
 
     saved = tmp_path / "saved.csv"
     assert lib.nt_tune_cache_save(str(saved).encode()) == 0
     rows = list(csv.reader(open(saved)))
-    assert rows[0] == [] and len(rows[1]) == 4  # the default pair
-    assert [str(v) for v in (fp16, fp16, 4096, 2048, 1024, 1)] in rows
+    assert rows[0] == [] and len(rows[1]) == 1  # the default pair
+    pairs = {tuple(rows[i]): tuple(rows[i + 1]) for i in range(2, len(rows) - 1, 2)}
+    assert pairs[tuple(str(v) for v in (0, fp16, fp16, 4096, 2048, 1024, 1, 0))] == (str(fast), "256", "256", "32")
+    assert pairs[tuple(str(v) for v in (1, fp16, 4, 32, 4096, 4096, 128, 1))] == ("3",)
+    assert pairs[tuple(str(v) for v in (2, fp16, 32, 256, 56, 56, 256, 3, 3, 1, 1, 1))] == ("2",)
     assert lib.nt_tune_cache_load(str(tmp_path / "missing.csv").encode(), None) != 0
 
 

@@ -604,6 +604,50 @@ def test_scratch_buffers_are_reused_grown_and_released():
         runtime.library().nt_release_workspaces()
 
 
+def test_first_launch_times_the_attention_variants_and_the_conv2d_paths():
+    """Like a product with tunable block sizes, the first launch of a new attention / conv2d problem times the
+    alternatives (loop variants; one launch on NCHW, repacking pass, gather kernel), records the winner, and
+    later launches -- also of a kernel object made afterwards -- run it.  Every launch is checked."""
+    from ninetoothed_amd import auto_tuner, runtime
+
+    fp16 = runtime.DATA_TYPE_INDEX["fp16"]
+    batch, heads, seq, dim = 3, 16, 640, 128  # sizes no other test uses (enough query blocks not to split the keys)
+    q, k, v = (_randn(batch, heads, seq, dim).cuda() for _ in range(3))
+    for is_causal in (False, True):
+        problem = (fp16, batch, heads, seq, seq, dim, int(is_causal))
+        assert auto_tuner.lookup_problem(runtime.TUNE_ATTENTION, problem) < 0
+        expected = _attention_reference(q, k, v, is_causal, dim**-0.5)
+        for _ in range(2):  # the second kernel object starts from the recorded choice
+            kernel = ninetoothed.make(programs.attention.arrangement_with_scale, programs.attention.application_with_scale, programs.attention.tensors(True))
+            for _ in range(2):
+                o = torch.full_like(q, float("nan"))
+                kernel(q, k, v, is_causal, dim**-0.5, o)
+                assert torch.allclose(o.float(), expected, **HALF_TOL)
+            assert 0 <= auto_tuner.lookup_problem(runtime.TUNE_ATTENTION, problem) <= 4
+    # one query against a long key range splits the keys: nothing to choose from, nothing recorded
+    q1 = _randn(1, 8, 1, 128).cuda()
+    k1, v1 = _randn(1, 8, 8192, 128).cuda(), _randn(1, 8, 8192, 128).cuda()
+    o1 = torch.full_like(q1, float("nan"))
+    kernel(q1, k1, v1, False, dim**-0.5, o1)
+    assert torch.allclose(o1.float(), _attention_reference(q1, k1, v1, False, dim**-0.5), **HALF_TOL)
+    assert auto_tuner.lookup_problem(runtime.TUNE_ATTENTION, (fp16, 1, 8, 1, 8192, 128, 0)) < 0
+
+    n, c, h, w, kk = 3, 64, 24, 40, 256
+    x, weight = _randn(n, c, h, w, scale=0.2).cuda(), _randn(kk, c, 3, 3, scale=0.2).cuda()
+    problem = (fp16, n, c, h, w, kk, 3, 3, 1, 1, 1)
+    assert auto_tuner.lookup_problem(runtime.TUNE_CONV2D, problem) < 0
+    expected = F.conv2d(x.float(), weight.float(), padding=1)
+    for _ in range(2):
+        assert torch.allclose(_conv2d(x, weight, (1, 1)).float(), expected, **HALF_TOL)
+    assert auto_tuner.lookup_problem(runtime.TUNE_CONV2D, problem) in (1, 2, 3)
+    # each way by name (block_size_m of the C entry point), whole output
+    for path in (1, 2, 3):
+        y = torch.full((n, kk, h, w), float("nan"), dtype=torch.float16, device="cuda")
+        tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (x, weight, y)]
+        assert runtime.library().launch_nt_conv2d(runtime.current_stream(), *tensors, fp16, 1, 1, path, 0, 0) == 0
+        assert torch.allclose(y.float(), expected, **HALF_TOL), path
+
+
 def test_first_call_of_an_untuned_problem_inside_a_captured_graph():
     """Nothing has run these problems before the capture starts: the first-launch tuner of the product
     (event synchronisation, repeated launches) and the specialisation of the tile map (compiling and
@@ -629,10 +673,21 @@ def test_first_call_of_an_untuned_problem_inside_a_captured_graph():
     fp16 = runtime.DATA_TYPE_INDEX["fp16"]
     assert auto_tuner.enabled() and auto_tuner.lookup(fp16, fp16, m, n, k, False) < 0 and auto_tuner.lookup(fp16, fp16, m, n, k, True) < 0
 
+    qa, ka, va = (_randn(2, 3, 328, 64).cuda() for _ in range(3))
+    oa = torch.empty_like(qa)
+    xc, wc = _randn(2, 32, 16, 24, scale=0.2).cuda(), _randn(256, 32, 3, 3, scale=0.2).cuda()
+    yc = torch.empty(2, 256, 16, 24, dtype=torch.float16, device="cuda")
+    attention = ninetoothed.make(programs.attention.arrangement, programs.attention.application, programs.attention.tensors())
+    conv = ninetoothed.make(programs.conv2d.arrangement, programs.conv2d.application, programs.conv2d.tensors())
+    attention_problem = (fp16, 2, 3, 328, 328, 64, 1)
+    conv_problem = (fp16, 2, 32, 16, 24, 256, 3, 3, 1, 1, 1)
+
     def run():
         matmul(a, b, c)
         addmm(bias, a, b, 0.5, 2.0, d)
         tile_map(x, y, z)
+        attention(qa, ka, va, True, oa)
+        conv(xc, wc, yc, padding_h=1, padding_w=1)
 
     stream = torch.cuda.Stream()
     torch.cuda.synchronize()
@@ -640,10 +695,14 @@ def test_first_call_of_an_untuned_problem_inside_a_captured_graph():
     with torch.cuda.graph(graph, stream=stream):
         run()
     assert auto_tuner.lookup(fp16, fp16, m, n, k, False) < 0  # nothing was timed during the capture
+    assert auto_tuner.lookup_problem(runtime.TUNE_ATTENTION, attention_problem) < 0
+    assert auto_tuner.lookup_problem(runtime.TUNE_CONV2D, conv_problem) < 0
     product = a.float() @ b.float()
     expected = (product, 0.5 * bias.float() + 2.0 * product.half().float(), x * 3.25 + y * y - 0.0078125)
+    expected_attention = _attention_reference(qa, ka, va, True, 1.4423828125 / 1.4426950408889634)  # (the program's literal, rounded to fp16)
+    expected_conv = F.conv2d(xc.float(), wc.float(), padding=1)
     for replay in range(3):
-        for t in (c, d, z):
+        for t in (c, d, z, oa, yc):
             t.fill_(float("nan"))
         torch.cuda.synchronize()
         graph.replay()
@@ -651,10 +710,14 @@ def test_first_call_of_an_untuned_problem_inside_a_captured_graph():
         assert torch.allclose(c.float(), expected[0], **HALF_TOL), replay
         assert torch.allclose(d.float(), expected[1], rtol=1e-2, atol=2e-2), replay
         assert torch.allclose(z, expected[2], rtol=1e-6, atol=1e-6), replay
+        assert torch.allclose(oa.float(), expected_attention, **HALF_TOL), replay
+        assert torch.allclose(yc.float(), expected_conv, **HALF_TOL), replay
         if replay == 0:
-            run()  # the first eager call tunes the products and specialises the tile map
+            run()  # the first eager call tunes the products, attention and the convolution and specialises the tile map
             torch.cuda.synchronize()
             assert auto_tuner.lookup(fp16, fp16, m, n, k, False) >= 0 and auto_tuner.lookup(fp16, fp16, m, n, k, True) >= 0
+            assert auto_tuner.lookup_problem(runtime.TUNE_ATTENTION, attention_problem) >= 0
+            assert auto_tuner.lookup_problem(runtime.TUNE_CONV2D, conv_problem) >= 1
             assert torch.allclose(z, expected[2], rtol=1e-6, atol=1e-6)
 
 
