@@ -136,7 +136,40 @@ def build_workloads():
         return dict(step=lambda: dst.copy_(src), work=2.0 * (1 << 30), bound="hbm", kernel=_Copy(),
                     describe={"workload": "device copy of 1 GiB (2 GiB of traffic), counter calibration only"})
 
+    def mfma_ceiling(constant):
+        # not a program of the library: MFMAs on register operands taken from the addmm workload's own inputs
+        # (or from constants), which bounds what the GEMM and attention kernels can reach on this data
+        def make():
+            import ctypes
+
+            from ninetoothed_amd import runtime
+
+            n = 8192
+            if constant:
+                mat1, mat2 = (torch.full((n, n), 0.5, dtype=torch.float16, device="cuda") for _ in range(2))
+            else:
+                mat1, mat2 = (seeded(n, n, seed=s).cuda() for s in (1, 2))
+            sink = torch.zeros(1, device="cuda")
+            loops = 4096
+            count = ctypes.c_int64(0)
+            lib = runtime.library()
+
+            def step():
+                runtime.check(lib.nt_probe_mfma_rate(runtime.current_stream(), runtime.ArgumentTensor.from_torch_tensor(mat1), runtime.ArgumentTensor.from_torch_tensor(mat2),
+                                                     loops, sink.data_ptr(), ctypes.byref(count)))
+
+            step()
+
+            class _Probe:
+                last_plan = "nt_probe_mfma_rate (measurement aid, not a program)"
+
+            return dict(step=step, work=float(count.value) * 2 * 32 * 32 * 16, bound="mfma", kernel=_Probe(),
+                        describe={"workload": "MFMA 32x32x16 fp16 issue rate on register operands, " + ("constant 0.5" if constant else "the addmm workload's N(0,1) inputs")})
+        return make
+
     workloads["addmm_8192"] = addmm_8192
+    workloads["mfma_ceiling"] = mfma_ceiling(False)
+    workloads["mfma_ceiling_constant"] = mfma_ceiling(True)
     workloads["matmul_512"] = matmul_512
     workloads["softmax_4096"] = softmax_4096
     workloads["attention"] = attention(False)
@@ -333,7 +366,7 @@ def main():
     others = {}
     if not args.only:
         for name, factory in workloads.items():
-            if name == args.workload or name == "copy_1gib":
+            if name == args.workload or name in ("copy_1gib", "mfma_ceiling_constant"):
                 continue
             workload = factory()
             ms, _ = measure(workload, max(5, args.steps // 2), args.warmup)

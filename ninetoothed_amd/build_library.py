@@ -15,7 +15,7 @@ PACKAGE_DIR = pathlib.Path(__file__).resolve().parent
 CSRC_DIR = PACKAGE_DIR / "csrc"
 LIBRARY_PATH = PACKAGE_DIR / "lib" / "libnt_hip.so"
 
-SOURCES = ("gemm_api.hip", "conv2d.hip", "softmax.hip", "attention.hip", "map.hip", "workspace.hip", "tune.hip")
+SOURCES = ("gemm_api.hip", "conv2d.hip", "softmax.hip", "attention.hip", "map.hip", "workspace.hip", "tune.hip", "probe.hip")
 
 OFFLOAD_ARCH = "gfx950"
 

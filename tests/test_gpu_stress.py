@@ -246,3 +246,24 @@ def test_attention_on_random_shapes():
         expected = torch.softmax(scores, dim=-1) @ v.float()
         tolerance = 1e-2 if dtype == torch.float16 else 3e-2
         assert torch.allclose(o.float(), expected, rtol=tolerance, atol=tolerance), (case, batch, heads, seq_q, seq_k, emb_dim, is_causal, dtype, packed)
+
+
+def test_mfma_rate_probe_runs_and_counts():
+    """The measurement aid behind bench.py's ``mfma_ceiling`` workloads: launches, reports the MFMAs it issued
+    (8 waves per compute unit x loops x 8) and leaves its sink untouched."""
+    import ctypes
+
+    from ninetoothed_amd import runtime
+
+    a = torch.randn(64, 64, dtype=torch.float16, device="cuda")
+    sink = torch.zeros(1, device="cuda")
+    count = ctypes.c_int64(0)
+    lib = runtime.library()
+    tensor = runtime.ArgumentTensor.from_torch_tensor(a)
+    runtime.check(lib.nt_probe_mfma_rate(runtime.current_stream(), tensor, tensor, 3, sink.data_ptr(), ctypes.byref(count)))
+    torch.cuda.synchronize()
+    units = torch.cuda.get_device_properties(0).multi_processor_count
+    assert count.value == units * 8 * 3 * 8
+    assert sink.item() == 0.0
+    small = runtime.ArgumentTensor.from_torch_tensor(a[:8, :8].contiguous())
+    assert lib.nt_probe_mfma_rate(runtime.current_stream(), small, small, 3, sink.data_ptr(), ctypes.byref(count)) != 0
