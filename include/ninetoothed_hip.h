@@ -91,6 +91,8 @@ typedef int NineToothedResult;
  * generated launch function src/ninetoothed/generation.py:545-600.
  * `dtype` is the element type of lhs/rhs; `output_dtype` that of output
  * (FLOAT16, BFLOAT16 or FLOAT32).  Any strides are accepted.
+ * FLOAT32 operands (output FLOAT32) are multiplied as they are on the fp32
+ * MFMA (32x32x2), products and sums in fp32, by the any-stride kernel.
  * FLOAT8_E5M2 operands (output FLOAT16 or FLOAT32) are widened to fp16 on the
  * way into LDS -- exact, the format is the upper byte of fp16 -- and multiplied
  * on the fp16 MFMA path with fp32 accumulation. */
@@ -105,7 +107,8 @@ NineToothedResult launch_nt_matmul(NineToothedStream stream,
 /* output = beta * input + alpha * round_to_dtype(mat1 @ mat2), epilogue in fp32.
  * Replaces the kernel generated for tests/test_addmm.py:13-38 (argument order
  * input, mat1, mat2, beta, alpha, output as in its application).  beta and
- * alpha are 0-d tensors holding a host double. */
+ * alpha are 0-d tensors holding a host double.  dtype FLOAT32: all four tensors
+ * hold fp32 and the product is not rounded. */
 NineToothedResult launch_nt_addmm(NineToothedStream stream,
                                   NineToothedTensor input,
                                   NineToothedTensor mat1,
@@ -188,6 +191,7 @@ NineToothedResult launch_nt_attention(NineToothedStream stream,
  * 1 -- the scratch-free gather kernel, which serves every shape, and calls whose
  *   scratch cannot be allocated (out of memory; a stream under graph capture that
  *   has no buffer yet).
+ * FLOAT32 tensors run on way 1 with the fp32 MFMA.
  * 1 x 1 filters without padding (P*Q and C multiples of 8) run as one batched
  * launch of the GEMM kernels on the tensors as they lie, without scratch. */
 NineToothedResult launch_nt_conv2d(NineToothedStream stream,

@@ -238,7 +238,7 @@ bool generic_accepts(const GemmProblem &q) {
     if (q.batch != 1) return false;
     if (q.dtype == NINETOOTHED_FLOAT8_E5M2)  // widened to fp16; addmm rounds its product to fp16, so it writes fp16
         return (q.out_dtype == NINETOOTHED_FLOAT16 || (q.out_dtype == NINETOOTHED_FLOAT32 && !q.addmm())) && q.m >= 0 && q.n >= 0 && q.k >= 0;
-    if (q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) return false;
+    if (q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16 && q.dtype != NINETOOTHED_FLOAT32) return false;
     if (q.out_dtype != q.dtype && q.out_dtype != NINETOOTHED_FLOAT32) return false;
     return q.m >= 0 && q.n >= 0 && q.k >= 0;
 }
@@ -298,6 +298,7 @@ hipError_t fp8_launch_typed(const GemmProblem &q, hipStream_t stream) {
 hipError_t generic_launch(const GemmProblem &q, hipStream_t stream) {
     const bool f32out = q.out_dtype == NINETOOTHED_FLOAT32;
     if (q.dtype == NINETOOTHED_FLOAT8_E5M2) return f32out ? fp8_launch_typed<float>(q, stream) : fp8_launch_typed<half_t>(q, stream);
+    if (q.dtype == NINETOOTHED_FLOAT32) return generic_launch_typed<float, float>(q, stream);
     if (q.dtype == NINETOOTHED_FLOAT16)
         return f32out ? generic_launch_typed<half_t, float>(q, stream) : generic_launch_typed<half_t, half_t>(q, stream);
     return f32out ? generic_launch_typed<bf16_t, float>(q, stream) : generic_launch_typed<bf16_t, bf16_t>(q, stream);
@@ -611,7 +612,7 @@ enum ConvPath { kConvAuto = 0, kConvGather = 1, kConvRepack = 2, kConvDirect = 3
 // validates the call and fills the request; returns 0, an error, or -1 when there is nothing to compute
 int conv2d_request(Conv2dRequest &request, const NineToothedTensor &input, const NineToothedTensor &filter, const NineToothedTensor &output,
                    int dtype, int padding_h, int padding_w) {
-    if (dtype != NINETOOTHED_FLOAT16 && dtype != NINETOOTHED_BFLOAT16) return NINETOOTHED_NO_KERNEL;
+    if (dtype != NINETOOTHED_FLOAT16 && dtype != NINETOOTHED_BFLOAT16 && dtype != NINETOOTHED_FLOAT32) return NINETOOTHED_NO_KERNEL;
     if (!input.shape || !filter.shape || !output.shape || !input.strides || !filter.strides || !output.strides)
         return hipErrorInvalidValue;
     if (padding_h < 0 || padding_w < 0) return hipErrorInvalidValue;
@@ -663,6 +664,8 @@ hipError_t conv2d_gather(const Conv2dRequest &r, hipStream_t stream) {
 int conv2d_run(const Conv2dRequest &r, int path, hipStream_t stream) {
     // 1 x 1 filters without padding: per image Y[K, P*Q] = W[K, C] . X[C, P*Q], a batch of row-major
     // products on the tensors as they lie (no repacking, no scratch memory)
+    // fp32 tensors: the gathering kernel on fp32 MFMAs (the other paths move 16-bit elements)
+    if (r.dtype == NINETOOTHED_FLOAT32) return path == kConvAuto || path == kConvGather ? (int)conv2d_gather<float>(r, stream) : NINETOOTHED_NO_KERNEL;
     if (path == kConvAuto && r.R == 1 && r.S == 1 && r.pad_h == 0 && r.pad_w == 0 && r.xs[3] == 1 && r.xs[2] == r.W && r.ys[3] == 1 &&
         r.ys[2] == r.Q && r.ws[1] == 1) {
         GemmProblem q;

@@ -20,7 +20,7 @@ constexpr int kGenPitch = 40;  // elements per LDS row
 constexpr int kGenThreads = 256;
 
 // Policy concept:
-//   typedef ... elem;                       // half_t or bf16_t
+//   typedef ... elem;                       // half_t, bf16_t or float
 //   int m, n, k;                            // GEMM extents
 //   void load_a16(int row, int k0, elem out[16]) const;  // A[row][k0..k0+15], zero outside
 //   void load_b16(int col, int k0, elem out[16]) const;  // B[k0..k0+15][col], zero outside
@@ -31,8 +31,8 @@ __global__ __launch_bounds__(kGenThreads) void gemm_generic_kernel(Problem prob)
     typedef Elem<T> E;
     typedef typename E::vec8 vec8;
 
-    __shared__ __attribute__((aligned(16))) T lds_a[kGenBM * kGenPitch];
-    __shared__ __attribute__((aligned(16))) T lds_b[kGenBN * kGenPitch];
+    __shared__ __attribute__((aligned(32))) T lds_a[kGenBM * kGenPitch];
+    __shared__ __attribute__((aligned(32))) T lds_b[kGenBN * kGenPitch];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;

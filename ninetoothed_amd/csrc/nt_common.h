@@ -64,6 +64,21 @@ struct Elem<bf16_t> {
     static NT_DEVICE bf16_t from_float(float x) { return (bf16_t)x; }
 };
 
+// fp32 operands: the matrix pipe multiplies them as they are (32x32x2, one k value per lane and
+// instruction); a lane's 8 k values go through 8 chained instructions.  No 16x16 form.
+template <>
+struct Elem<float> {
+    typedef float vec8 __attribute__((ext_vector_type(8)));
+    static constexpr int kDataType = NINETOOTHED_FLOAT32;
+    static NT_DEVICE float16_t mfma32(vec8 a, vec8 b, float16_t c) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[i], c, 0, 0, 0);
+        return c;
+    }
+    static NT_DEVICE float to_float(float x) { return x; }
+    static NT_DEVICE float from_float(float x) { return x; }
+};
+
 template <typename T>
 NT_DEVICE T from_float(float x) {
     return (T)x;

@@ -258,7 +258,7 @@ class Kernel:
         kind, info = recognition.analyze_gemm(self.types[0], self.types[1], self.types[2], env)
         if kind == "empty":
             return _Plan("empty launch", lambda call_args: None)
-        tag = self._tensor_dtype(lhs, rhs, allowed=("fp16", "bf16", "fp8e5m2"))
+        tag = self._tensor_dtype(lhs, rhs, allowed=("fp16", "bf16", "fp32", "fp8e5m2"))
         out_tag = _dtype_tag(out.dtype)
         cast = self.details.get("cast")
         if tag == "fp8e5m2":  # the second case of the reference's tests/test_matmul.py:61-88
@@ -285,14 +285,14 @@ class Kernel:
             if self.details.get("cast") != "fp16" or _dtype_tag(out.dtype) != "fp16":
                 raise UnsupportedProgram("addmm on fp8 operands rounds the product to fp16 and writes an fp16 tensor.")
             return self._gemm_plan(info, tag, "fp16", positions=(0, 1, 2, 3, 4, 5))
-        tag = self._tensor_dtype(input, mat1, mat2, out, allowed=("fp16", "bf16"))
-        if self.details.get("cast") != tag:
+        tag = self._tensor_dtype(input, mat1, mat2, out, allowed=("fp16", "bf16", "fp32"))
+        if self.details.get("cast") not in ((tag, None) if tag == "fp32" else (tag,)):
             raise UnsupportedProgram(f"The application rounds the product to `{self.details.get('cast')}` but the tensors hold `{tag}`.")
         return self._gemm_plan(info, tag, tag, positions=(0, 1, 2, 3, 4, 5))
 
     def _gemm_plan(self, info, tag, out_tag, positions):
         lib = runtime.library()
-        itemsize = 1 if tag == "fp8e5m2" else 2
+        itemsize = {"fp8e5m2": 1, "fp32": 4}.get(tag, 2)
         out_itemsize = 4 if out_tag == "fp32" else 2
         a, b, c, i = info["a"], info["b"], info["c"], info["input"]
         m, n, k = info["m"], info["n"], info["k"]
@@ -447,7 +447,7 @@ class Kernel:
             return _Plan("empty launch", lambda call_args: None)
         if kind != "strided":
             raise UnsupportedProgram("A product with an element-wise epilogue needs plain strided matrices.")
-        tag = self._tensor_dtype(args[lhs_pos], args[rhs_pos], allowed=("fp16", "bf16"))
+        tag = self._tensor_dtype(args[lhs_pos], args[rhs_pos], allowed=("fp16", "bf16", "fp32"))
         out = args[out_pos]
         if out.numel() and not (out.is_contiguous() or out.t().is_contiguous()):
             raise UnsupportedProgram("The output of a product with an epilogue must be a dense matrix.")

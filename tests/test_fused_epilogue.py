@@ -51,7 +51,7 @@ def test_recognised_as_a_product_with_an_epilogue():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16, torch.float32))
 @pytest.mark.parametrize("m, n, k", ((512, 384, 256), (300, 200, 136), (1024, 1024, 2048)))
 def test_linear_with_bias_activation_and_residual(m, n, k, dtype):
     kernel = _kernel()

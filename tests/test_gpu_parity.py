@@ -76,6 +76,38 @@ def test_matmul_bfloat16_and_float32_output():
     assert torch.allclose(out32, a.cuda().float() @ b.cuda().float(), rtol=1e-4, atol=1e-3)
 
 
+@pytest.mark.parametrize("m, n, k", ((512, 512, 512), (300, 200, 100), (64, 48, 8), (1, 1, 1), (257, 129, 65)))
+def test_matmul_float32_operands(m, n, k):
+    """fp32 tensors run on the fp32 MFMA (products and sums in fp32, no narrowing): against the oracle in
+    fp32 and against torch at fp32 tolerances, contiguous and strided."""
+    a, b = _randn(m, k, dtype=torch.float32), _randn(k, n, dtype=torch.float32)
+    kernel = _matmul_kernel()
+    out = torch.empty(m, n, dtype=torch.float32, device="cuda")
+    kernel(a.cuda(), b.cuda(), out)
+    _native_only(kernel, "launch_nt_matmul")
+    expected = oracle.matmul(a.numpy(), b.numpy(), 64, 64, 64, out_dtype="fp32")
+    assert np.allclose(out.cpu().numpy(), expected, rtol=1e-4, atol=1e-4)
+    assert torch.allclose(out.cpu(), a.double().matmul(b.double()).float(), rtol=1e-4, atol=1e-4)
+    out_t = torch.zeros(n, 2 * m, dtype=torch.float32, device="cuda")
+    kernel(a.cuda(), b.t().contiguous().cuda().t(), out_t.t()[::2])
+    assert torch.equal(out_t.t()[::2], out) and torch.count_nonzero(out_t.t()[1::2]) == 0
+
+
+def test_addmm_float32_through_the_c_abi():
+    from ninetoothed_amd import runtime
+
+    lib = runtime.library()
+    m, n, k = 200, 136, 72
+    bias, a, b = (_randn(*shape, dtype=torch.float32).cuda() for shape in ((m, n), (m, k), (k, n)))
+    out = torch.empty(m, n, dtype=torch.float32, device="cuda")
+    tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (bias, a, b, out)]
+    beta, alpha = runtime.ArgumentTensor.from_scalar(0.5), runtime.ArgumentTensor.from_scalar(-1.25)
+    fp32 = runtime.DATA_TYPE_INDEX["fp32"]
+    runtime.check(lib.launch_nt_addmm(runtime.current_stream(), tensors[0], tensors[1], tensors[2], beta, alpha, tensors[3], fp32, 0, 0, 0))
+    expected = 0.5 * bias.double() - 1.25 * (a.double() @ b.double())
+    assert torch.allclose(out.double(), expected, rtol=1e-4, atol=1e-4)
+
+
 @pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
 @pytest.mark.parametrize("m, n, k", ((512, 512, 512), (1000, 768, 1024), (4096, 2048, 4096)))
 def test_matmul_float32_output_on_the_fast_instances(m, n, k, dtype):
@@ -493,12 +525,12 @@ def test_attention_many_short_sequences(emb_dim, dtype):
 # ---- conv2d ---------------------------------------------------------------
 
 
-def _conv2d(x, w, padding):
+def _conv2d(x, w, padding, application=programs.conv2d.application):
     n, _, h, width = x.shape
     k, _, r, s = w.shape
     p, q = h + 2 * padding[0] - r + 1, width + 2 * padding[1] - s + 1
     out = torch.empty(n, k, p, q, dtype=x.dtype, device=x.device)
-    kernel = ninetoothed.make(programs.conv2d.arrangement, programs.conv2d.application, programs.conv2d.tensors())
+    kernel = ninetoothed.make(programs.conv2d.arrangement, application, programs.conv2d.tensors())
     kernel(x, w, out, padding_h=padding[0], padding_w=padding[1])
     _native_only(kernel, "launch_nt_conv2d")
     return out
@@ -511,6 +543,22 @@ def test_conv2d_against_oracle(padding):
     out = _conv2d(x.cuda(), w.cuda(), padding)
     expected = oracle.conv2d(x.numpy(), w.numpy(), padding=padding, bm=16, bn=4, bk=8)
     assert np.allclose(out.cpu().float().numpy(), expected, **HALF_TOL)
+
+
+@pytest.mark.parametrize("padding", ((0, 0), (1, 1), (2, 0)))
+def test_conv2d_float32_tensors(padding):
+    # (the accumulator is stored as it is: the reference's conv2d application rounds it to fp16 first)
+    application = programs.matmul.application
+    x = torch.rand(2, 6, 9, 8)
+    w = torch.rand(5, 6, 3, 3)
+    with pytest.raises(ninetoothed.UnsupportedProgram):
+        _conv2d(x.cuda(), w.cuda(), padding)
+    out = _conv2d(x.cuda(), w.cuda(), padding, application)
+    assert out.dtype == torch.float32
+    expected = oracle.conv2d(x.numpy(), w.numpy(), padding=padding, bm=16, bn=4, bk=8, dtype="fp32")
+    assert np.allclose(out.cpu().numpy(), expected, rtol=1e-4, atol=1e-4)
+    big_x, big_w = torch.randn(3, 32, 20, 24, device="cuda"), torch.randn(48, 32, 3, 3, device="cuda")
+    assert torch.allclose(_conv2d(big_x, big_w, padding, application).cpu(), F.conv2d(big_x.cpu().double(), big_w.cpu().double(), padding=padding).float(), rtol=1e-4, atol=1e-3)
 
 
 @pytest.mark.parametrize("padding", ((0, 0), (1, 1), (0, 1), (2, 0)))
