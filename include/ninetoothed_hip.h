@@ -181,7 +181,7 @@ NineToothedResult launch_nt_attention(NineToothedStream stream,
  * 3 -- one launch on the tensors as they lie, no scratch memory: the filter is
  *   the row-major left operand, rows of the right operand are (channel, filter
  *   tap)-shifted pixel runs of the NCHW input; needs an output width that is a
- *   multiple of 8, padding_w <= 1, C*R*S a multiple of 32, pixels of an input row
+ *   multiple of 8, padding_w <= 1, C*R*S a multiple of 32, R*S / gcd(32, R*S) <= 25, pixels of an input row
  *   contiguous, contiguous filter and output, K filling 256-wide tiles to 4/5;
  * 2 -- when K % 8 == 0, C >= 2, the output is contiguous and N*P*Q >= 1024: the
  *   input is first repacked to channels-last and the filter to [R*S*C', K]
@@ -283,7 +283,8 @@ NineToothedResult nt_tune_attention(NineToothedStream stream,
 /* As nt_tune_gemm for launch_nt_conv2d: times the ways to run the convolution -- 3 = one launch on the tensors as
  * they lie, 2 = repacking pass plus GEMM loop, 1 = gather kernel; a way that does not take the problem is skipped
  * -- and records the fastest (the block_size_m value that selects it) for later launches of the same problem with
- * block_size_m = 0.  *best_path = -1 when nothing was timed (graph capture). */
+ * block_size_m = 0; a way that needs scratch memory or more launches replaces one before it in that order only
+ * when it is more than 3 % faster.  *best_path = -1 when nothing was timed (graph capture). */
 NineToothedResult nt_tune_conv2d(NineToothedStream stream,
                                  NineToothedTensor input, NineToothedTensor filter, NineToothedTensor output,
                                  int dtype, int padding_h, int padding_w, int iters,

@@ -364,7 +364,8 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
 // into registers accept and loads into LDS do not -- and written to a [32][256] LDS tile that the transposing
 // ds_read_b64_tr_b16 turns into MFMA operands.  Pieces whose image row lies in the padding are fetched from
 // behind the buffer (zeros); pixels of a piece that fall into the left / right padding are cleared in registers.
-// Needs Q % 8 == 0 (a piece stays inside one image row), C*R*S % 32 == 0, contiguous filter and output.
+// Needs Q % 8 == 0 (a piece stays inside one image row), C*R*S % 32 == 0, contiguous filter and output, and a
+// filter whose taps repeat within 25 tiles of the contraction (R*S / gcd(32, R*S) <= 25: 1x1 ... 5x5).
 //
 // Tiles are 256 output channels x 256 pixels.  (Measured and dropped: cutting the pixels that are left after the
 // last full round of workgroups -- 392 tiles on 256 CUs -- into one round of narrower tiles, with the two waves
@@ -380,8 +381,12 @@ struct ConvDirectParams {
     int CRS;                // contraction length
     int tiles_ch;           // tiles along the output channels
     unsigned x_bytes, w_bytes;
-    int step_c, step_r, step_s;  // 32 contraction positions further: (c, r, s) += these, with carries
+    int period;             // tiles after which the filter taps of a tile's 32 rows repeat: R*S / gcd(32, R*S)
+    int period_bytes;       // ... and by how many bytes the rows' channels have moved on by then
 };
+
+// rows of the table of filter taps kept in LDS: at most this many tiles per period (5 x 5 filters: 25)
+constexpr int kConvDirectMaxPeriod = 25;
 
 template <typename T>
 __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams p) {
@@ -410,6 +415,10 @@ __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams 
     __shared__ __attribute__((aligned(1024))) unsigned char lds_b1[kStageB];
     __shared__ __attribute__((aligned(1024))) unsigned char lds_b2[kStageB];
     __shared__ __attribute__((aligned(1024))) unsigned char lds_b3[kStageB];
+    // what the 32 rows of a pixel tile are, for every tile of a period: {byte offset of the row's (channel, tap)
+    // relative to the period's first channel, 31 - filter row, border mask, unused}
+    typedef unsigned uint4_t __attribute__((ext_vector_type(4)));
+    __shared__ __attribute__((aligned(16))) uint4_t lds_taps[kConvDirectMaxPeriod * BK];
     auto stage_a = [&](auto tag) -> NT_LDS unsigned char * {
         constexpr int i = decltype(tag)::value;
         if constexpr (i == 0) return (NT_LDS unsigned char *)lds_a0;
@@ -492,35 +501,41 @@ __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams 
     // masks that clear the pixel left / right of the image in a piece at an image border
     const unsigned keep_left = at_left ? 0xffff0000u : 0xffffffffu;    // first dword of the piece
     const unsigned keep_right = at_right ? 0x0000ffffu : 0xffffffffu;  // last dword
-    // this thread's rows in the tile fetched next: filter row and column, and the byte offset c * xs1 + r * xs2 + s
-    // that goes with them (the channel itself is not needed: the loop ends with the last one)
-    int gr[kGather], gs[kGather], goff[kGather];
-#pragma unroll
-    for (int j = 0; j < kGather; ++j) {
-        const int k = krow0 + 16 * j;
+    // The rows of a tile are 32 consecutive (channel, tap) pairs; which taps they are repeats every `period`
+    // tiles, `period_bytes` of channels further on.  A table in LDS holds, for every tile of a period and each of
+    // its rows, the row's byte offset (c * xs1 + r * xs2 + s) * 2 relative to the period's first channel, the
+    // shift that brings the bit of its filter row in rows_outside to the top, and a mask over a piece's first and
+    // last pixel that is zero where the tap moves the pixels across the left (low half) / right (high half)
+    // image border.  A lane then derives a load's offset with three instructions and keeps no per-row state.
+    for (int idx = tid; idx < p.period * BK; idx += 512) {
+        const int k = idx;  // tile idx / 32 of the period, row idx % 32
         const int c = k / RS, rs = k - c * RS;
-        gr[j] = rs / p.S;
-        gs[j] = rs - gr[j] * p.S;
-        goff[j] = (c * (int)p.xs1 + gr[j] * (int)p.xs2 + gs[j]) * 2;
+        const int r = rs / p.S, sx = rs - r * p.S;
+        uint4_t entry;
+        entry[0] = (unsigned)((c * (int)p.xs1 + r * (int)p.xs2 + sx) * 2);
+        entry[1] = (unsigned)(31 - r);
+        entry[2] = (sx < p.pad_w ? 0u : 0x0000ffffu) | (sx > p.S - 1 - p.pad_w ? 0u : 0xffff0000u);
+        entry[3] = 0u;
+        lds_taps[idx] = entry;
     }
-    const int step_off = (p.step_c * (int)p.xs1 + p.step_r * (int)p.xs2 + p.step_s) * 2;  // 32 contraction positions further ...
-    const int carry_s = ((int)p.xs2 - p.S) * 2;                                           // ... when the column wraps
-    const int carry_r = ((int)p.xs1 - p.R * (int)p.xs2) * 2;                              // ... when the row wraps
-    typedef unsigned uint4_t __attribute__((ext_vector_type(4)));
+    __syncthreads();
+    const NT_LDS uint4_t *my_taps = (const NT_LDS uint4_t *)lds_taps + krow0;  // + 16 for the second row, + 32 per tile of the period
+    int tap_tile = 0;        // position of the tile fetched next in its period (uniform)
+    int period_base = 0;     // byte offset of that period's first channel (uniform)
     const unsigned b_dst = (unsigned)(krow0 * kPitchB + piece * 16);  // the first piece in a stage; the second: 16 rows on
-    // fetches this thread's pieces of the next tile and moves on to the tile after it; `cols` keeps the rows' filter columns
-    auto gather = [&](auto careful_tag, uint4_t (&regs)[kGather], int (&cols)[kGather]) {
+    // fetches this thread's pieces of the next tile and moves on to the tile after it; `cols` keeps the rows' border masks
+    auto gather = [&](auto careful_tag, uint4_t (&regs)[kGather], unsigned (&cols)[kGather]) {
 #pragma unroll
         for (int j = 0; j < kGather; ++j) {
-            cols[j] = gs[j];
-            // one and the same offset behind the buffer for every load that has to return zeros
-            int offset = (rows_outside >> gr[j]) & 1 ? (int)0x80000000 : lane_off + goff[j];
+            const uint4_t entry = my_taps[tap_tile * BK + 16 * j];
+            cols[j] = entry[2];
+            // a row outside the image (or a piece past the tile's end) gets the top bit: one and the same kind of
+            // offset behind the buffer for every load that has to return zeros
+            const unsigned outside = (rows_outside << entry[1]) & 0x80000000u;
+            int offset = (int)((unsigned)(lane_off + period_base + (int)entry[0]) | outside);
 
             bool edge = false;  // the load would start below the tensor or end beyond it
-            if constexpr (decltype(careful_tag)::value) {
-                const bool outside = (rows_outside >> gr[j]) & 1;
-                edge = !outside && (offset < 0 || (unsigned)(offset + 16) > p.x_bytes);
-            }
+            if constexpr (decltype(careful_tag)::value) edge = !outside && (offset < 0 || (unsigned)(offset + 16) > p.x_bytes);
             if (decltype(careful_tag)::value && __builtin_amdgcn_ballot_w64(edge) != 0) {  // uniform, and rare
                 // the lanes concerned load one pixel further in and move the pixels back by one place
                 const int nudge = !edge ? 0 : (offset < 0 ? 1 : -1);
@@ -540,23 +555,23 @@ __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams 
             } else {
                 regs[j] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, offset, 0, 0));
             }
-            gs[j] += p.step_s;
-            const bool wrap_s = gs[j] >= p.S;
-            gs[j] -= wrap_s ? p.S : 0;
-            gr[j] += p.step_r + (wrap_s ? 1 : 0);
-            const bool wrap_r = gr[j] >= p.R;
-            gr[j] -= wrap_r ? p.R : 0;
-            goff[j] += step_off + (wrap_s ? carry_s : 0) + (wrap_r ? carry_r : 0);
+        }
+        if (++tap_tile == p.period) {
+            tap_tile = 0;
+            period_base += p.period_bytes;
         }
     };
     // stores the pieces, the pixel that a shifted piece at an image border took from the neighbouring image row cleared
-    auto scatter = [&](auto stage_tag, const uint4_t (&regs)[kGather], const int (&cols)[kGather]) {
+    // (keep_left always keeps the upper pixel of a dword, keep_right the lower one: the other half of a row's mask is inert)
+    auto scatter = [&](auto stage_tag, const uint4_t (&regs)[kGather], const unsigned (&cols)[kGather]) {
         NT_LDS unsigned char *sb = stage_b(stage_tag) + b_dst;
 #pragma unroll
         for (int j = 0; j < kGather; ++j) {
             uint4_t v = regs[j];
-            v[0] &= cols[j] < p.pad_w ? keep_left : 0xffffffffu;
-            v[3] &= cols[j] > p.S - 1 - p.pad_w ? keep_right : 0xffffffffu;
+            // (the masking belongs here, two steps after the load: placed right behind the load it would wait for it)
+            asm volatile("" : "+v"(v));
+            v[0] &= keep_left | cols[j];
+            v[3] &= keep_right | cols[j];
             *(NT_LDS uint4_t *)(sb + j * (16 * kPitchB)) = v;
         }
     };
@@ -604,7 +619,7 @@ __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams 
     const int num_k = p.CRS / BK;
     const int last_k = num_k - 1;
     uint4_t held[2][kGather];  // pieces in flight, by tile parity
-    int held_cols[2][kGather];  // their filter columns (uniform)
+    unsigned held_cols[2][kGather];  // their rows' border masks
     auto run = [&](auto careful_tag) {
         constexpr int kFrags = TN;
         // prologue: tiles 0 and 1 complete, the pieces of tiles 2 and 3 and the filter part of tile 2 in flight
@@ -740,9 +755,15 @@ int run_direct(const Conv2dRequest &q, hipStream_t stream) {
     p.CRS = CRS;
     p.x_bytes = (unsigned)x_extent;
     p.w_bytes = (unsigned)w_bytes;
-    p.step_c = 32 / (q.R * q.S);
-    p.step_r = (32 % (q.R * q.S)) / q.S;
-    p.step_s = 32 % q.S;
+    int divisor = q.R * q.S;  // gcd(32, R * S)
+    for (int rest = 32 % divisor; rest != 0;) {
+        const int next = divisor % rest;
+        divisor = rest;
+        rest = next;
+    }
+    p.period = q.R * q.S / divisor;
+    if (p.period > kConvDirectMaxPeriod) return NINETOOTHED_NO_KERNEL;
+    p.period_bytes = (int)((32 / divisor) * q.xs[1] * 2);  // (the extent check above covers this product)
     p.tiles_ch = ceil_div(q.K, 256);
     const int64_t grid = (int64_t)ceil_div(p.M, 256) * p.tiles_ch;
     if (grid <= 0 || grid > 0x7fffffffll) return NINETOOTHED_NO_KERNEL;

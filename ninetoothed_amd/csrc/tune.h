@@ -21,10 +21,11 @@ void tune_record(int kind, const int *values, int count, int choice, const int *
 
 // Times candidates 0 .. candidates - 1 on `stream` with device events: 2 warm-up launches and `iters` timed ones
 // each.  `launch(i)` returns 0, NINETOOTHED_NO_KERNEL (the candidate does not take the problem: skipped) or an
-// error (returned).  *best receives the fastest candidate (-1 when none ran).  Synchronises; returns without
-// timing anything (*best = -1, result 0) when the stream is being captured into a graph.
+// error (returned).  *best receives the fastest candidate (-1 when none ran); with a `margin`, a later candidate
+// replaces an earlier one only when it is faster by more than that fraction (candidates in order of preference).
+// Synchronises; returns without timing anything (*best = -1, result 0) when the stream is being captured into a graph.
 template <typename Launch>
-int tune_time(hipStream_t stream, int candidates, int iters, Launch launch, int *best, float *best_ms) {
+int tune_time(hipStream_t stream, int candidates, int iters, Launch launch, int *best, float *best_ms, float margin = 0.0f) {
     *best = -1;
     *best_ms = 0.0f;
     hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
@@ -64,7 +65,7 @@ int tune_time(hipStream_t stream, int candidates, int iters, Launch launch, int 
         float ms = 0.0f;
         (void)hipEventElapsedTime(&ms, start, stop);
         ms /= (float)iters;
-        if (*best < 0 || ms < *best_ms) {
+        if (*best < 0 || ms < *best_ms * (1.0f - margin)) {
             *best = i;
             *best_ms = ms;
         }

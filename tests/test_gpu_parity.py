@@ -625,6 +625,62 @@ def test_conv2d_layer_shapes_on_the_direct_to_lds_path(n, c, h, w, k, r, s, padd
     assert bool((guard[n * k * p_out * q_out :] == 7.0).all())
 
 
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
+@pytest.mark.parametrize(
+    "n, c, h, w, k, r, s, padding",
+    (
+        (2, 32, 8, 8, 256, 3, 3, (1, 1)),      # one tile that holds the tensor's first and last rows
+        (1, 32, 16, 24, 256, 3, 3, (1, 1)),
+        (3, 64, 24, 40, 256, 3, 3, (1, 1)),
+        (4, 64, 28, 32, 256, 3, 3, (1, 1)),    # 14 tiles
+        (2, 32, 10, 18, 256, 3, 3, (0, 0)),    # no padding
+        (2, 32, 8, 16, 256, 3, 3, (2, 1)),     # two rows of padding above and below
+        (2, 32, 12, 18, 512, 5, 5, (2, 1)),    # taps repeat after 25 tiles
+        (2, 64, 10, 16, 256, 1, 1, (0, 0)),
+        (2, 32, 9, 17, 256, 2, 2, (0, 0)),
+        (2, 16, 12, 9, 424, 3, 2, (1, 0)),     # a partial second tile of output channels, input rows of 9 pixels
+        (5, 96, 14, 8, 256, 3, 3, (1, 1)),     # image rows of one piece: every piece is at both borders
+    ),
+)
+def test_conv2d_one_launch_path(n, c, h, w, k, r, s, padding, dtype):
+    """launch_nt_conv2d with block_size_m = 3 (the tensors as they lie, no scratch memory), whole output against an
+    fp32 convolution of the same operands.  The input is a channel slice of a larger Inf-filled tensor, so a
+    load that strays outside an image's rows, or is not cleared at a border, shows up."""
+    from ninetoothed_amd import runtime
+
+    big = torch.full((n, c + 2, h, w), float("inf"), dtype=dtype, device="cuda")
+    x = big[:, 1 : c + 1]
+    x.copy_((torch.randn(n, c, h, w, device="cuda") * 0.5).to(dtype))
+    weight = (torch.randn(k, c, r, s, device="cuda") * 0.1).to(dtype)
+    p_out, q_out = h + 2 * padding[0] - r + 1, w + 2 * padding[1] - s + 1
+    guard = torch.full((n * k * p_out * q_out + 64,), 7.0, dtype=dtype, device="cuda")
+    out = guard[: n * k * p_out * q_out].view(n, k, p_out, q_out)
+    out.fill_(float("nan"))
+    tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (x, weight, out)]
+    tag = runtime.DATA_TYPE_INDEX["fp16" if dtype == torch.float16 else "bf16"]
+    assert runtime.library().launch_nt_conv2d(runtime.current_stream(), *tensors, tag, padding[0], padding[1], 3, 0, 0) == 0
+    expected = F.conv2d(x.float(), weight.float(), padding=padding)
+    tolerance = HALF_TOL if dtype == torch.float16 else dict(rtol=2e-2, atol=2e-2)
+    assert torch.allclose(out.float(), expected, **tolerance)
+    assert bool((guard[n * k * p_out * q_out :] == 7.0).all())
+
+
+def test_conv2d_one_launch_path_refuses_what_it_cannot_run():
+    from ninetoothed_amd import runtime
+
+    def call(n, c, h, w, k, r, s, padding):
+        x = torch.zeros(n, c, h, w, dtype=torch.float16, device="cuda")
+        weight = torch.zeros(k, c, r, s, dtype=torch.float16, device="cuda")
+        out = torch.zeros(n, k, h + 2 * padding[0] - r + 1, w + 2 * padding[1] - s + 1, dtype=torch.float16, device="cuda")
+        tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (x, weight, out)]
+        return runtime.library().launch_nt_conv2d(runtime.current_stream(), *tensors, runtime.DATA_TYPE_INDEX["fp16"], padding[0], padding[1], 3, 0, 0)
+
+    assert call(2, 32, 16, 16, 256, 7, 7, (3, 1)) == runtime.NO_KERNEL   # taps repeat only after 49 tiles
+    assert call(2, 32, 16, 15, 256, 3, 3, (1, 1)) == runtime.NO_KERNEL   # output rows of 15 pixels
+    assert call(2, 24, 16, 16, 256, 3, 3, (1, 1)) == runtime.NO_KERNEL   # C * R * S not a multiple of 32
+    assert call(2, 32, 16, 16, 64, 3, 3, (1, 1)) == runtime.NO_KERNEL    # a quarter of a tile of output channels
+
+
 def test_scratch_buffers_are_reused_grown_and_released():
     """conv2d's repacked operands and fp32 attention's narrowed K / V live in buffers the library
     keeps per stream: a smaller call after a larger one, a larger one after that, another stream and
