@@ -313,7 +313,7 @@ int nt_tune_lookup(int kind, const int *values, int count);
 
 /* Measurement aid (no counterpart in the reference): one workgroup of eight waves per compute unit issues
  * `loops` x 8 MFMAs (32x32x16 fp16) per wave on operand fragments read once from the FLOAT16 tensors `a` and
- * `b` -- no LDS, no memory traffic inside the loop.  The rate bounds what a GEMM or attention kernel can reach on
+ * `b` (dense row-major matrices of at least 4096 elements) -- no LDS, no memory traffic inside the loop.  The rate bounds what a GEMM or attention kernel can reach on
  * the same operand values (random values draw more power in the matrix pipe than constants, and the clock
  * follows).  `sink` is a device float the kernel may write; *mfma_count receives the MFMAs issued in total
  * (65536 FLOP each).  Asynchronous on `stream`. */

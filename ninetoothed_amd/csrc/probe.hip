@@ -55,7 +55,9 @@ __global__ __launch_bounds__(512, 2) void mfma_rate_kernel(const half_t *a, cons
 // receives the number of MFMAs issued in total (each 2 x 32 x 32 x 16 FLOP).  Asynchronous on `stream`.
 extern "C" NineToothedResult nt_probe_mfma_rate(NineToothedStream stream, NineToothedTensor a, NineToothedTensor b, int loops, float *sink,
                                                 int64_t *mfma_count) {
-    if (!a.shape || !b.shape || a.data == nullptr || b.data == nullptr || sink == nullptr || loops <= 0) return hipErrorInvalidValue;
+    if (!a.shape || !b.shape || !a.strides || !b.strides || a.data == nullptr || b.data == nullptr || sink == nullptr || loops <= 0) return hipErrorInvalidValue;
+    // the kernel reads the first shape[0] * shape[1] elements behind each pointer: dense row-major matrices only
+    if (a.strides[1] != 1 || b.strides[1] != 1 || a.strides[0] != (int64_t)a.shape[1] || b.strides[0] != (int64_t)b.shape[1]) return hipErrorInvalidValue;
     const int64_t elements = std::min<int64_t>((int64_t)a.shape[0] * (int64_t)a.shape[1], (int64_t)b.shape[0] * (int64_t)b.shape[1]);
     if (elements < 4096) return hipErrorInvalidValue;
     int device = 0, units = 0;
