@@ -255,7 +255,9 @@ NineToothedResult launch_nt_gemm_config(NineToothedStream stream, int config,
 /* Times every instance that accepts the problem (hipEvents on `stream`,
  * `iters` launches each after 2 warm-ups; this call synchronises) and stores
  * the winner in the per-device cache that launch_nt_matmul / launch_nt_addmm
- * consult when block sizes are 0.  Returns 0 and the winner in *best_config,
+ * consult when block sizes are 0.  The instance of the untuned rule is timed
+ * first and stays the choice unless another one is more than 2 % faster (the
+ * timings scatter by about that much).  Returns 0 and the winner in *best_config,
  * its average time in *best_ms.  On a stream that is being captured into a
  * graph nothing is timed or recorded: returns 0 with *best_config = -1. */
 NineToothedResult nt_tune_gemm(NineToothedStream stream,
