@@ -321,15 +321,16 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
         const int kv0 = blk * BN;
         const int limit = blk > last_block ? 0 : p.seq_k;
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt)
+        for (int qt = 0; qt < kQTiles; ++qt) {
+            // the last key this lane's row may see, relative to the first key of the lane's registers: one
+            // comparison with a constant per element
+            const int last_key = (p.causal ? min(limit - 1, q_row[qt]) : limit - 1) - kv0 - 4 * g;
 #pragma unroll
-            for (int qt = 0; qt < kQTiles; ++qt)
+            for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int kv = kv0 + kt * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
-                    const bool keep = kv < limit && (!p.causal || q_row[qt] >= kv);
-                    if (!keep) s_acc[kt][qt][r] = -INFINITY;
-                }
+                for (int r = 0; r < 16; ++r)
+                    if (kt * 32 + 8 * (r >> 2) + (r & 3) > last_key) s_acc[kt][qt][r] = -INFINITY;
+        }
     };
 
     // online softmax: turns (masked) S^T into P^T operand fragments, updates the
