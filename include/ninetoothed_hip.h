@@ -143,10 +143,13 @@ NineToothedResult launch_nt_softmax_config(NineToothedStream stream, int config,
  * library's extension for the 1/sqrt(head_dim) configuration.
  * is_causal is a 0-d tensor holding a host int64_t.
  * dtype FLOAT16 / BFLOAT16, or FLOAT32 (the fp32 case of
- * tests/test_attention.py:99-117, rtol = atol = 0.025 there): K and V are first
- * narrowed to fp16 copies in the library's scratch buffer of `stream`,
- * Q is narrowed while it is scaled, the products run on the fp16 MFMA path with
- * fp32 accumulation and O is written unrounded.
+ * tests/test_attention.py:99-117, rtol = atol = 0.025 there).  FLOAT32 tensors
+ * with head_dim 32, 64 or 128 and no block-size hints run in fp32 throughout on
+ * the fp32 MFMA (a sixteenth of the fp16 rate, nothing narrowed, no scratch
+ * memory).  Other head dimensions, and calls that give a hint -- the fast way
+ * -- run on fp16 copies: K and V are first narrowed into the library's scratch
+ * buffer of `stream`, Q is narrowed while it is scaled, the products run on
+ * the fp16 MFMA path with fp32 accumulation and O is written unrounded.
  * block_size_m / block_size_n are hints (0 = library's choice): block_size_m
  * >= 256 selects 256 query rows per workgroup, block_size_n <= 32 the 32-key
  * blocks with three workgroups per CU, block_size_n >= 64 the plain 64-key
@@ -154,10 +157,10 @@ NineToothedResult launch_nt_softmax_config(NineToothedStream stream, int config,
  * nt_tune_attention, else the software-pipelined 64-key loop (non-causal: with
  * 256 query rows and eight waves per workgroup when that still fills the chip
  * twice).  Without a scale tensor the scores are scaled by log2(e) rounded to
- * the element type, as the reference program's literal is.  FLOAT32 tensors
- * are computed on fp16 copies: values beyond the fp16 range overflow, which
- * the reference's fp32 kernel does not.  K and V of one (batch, head) must span
- * less than 4 GiB.
+ * the element type, as the reference program's literal is.  On the fp16
+ * copies of FLOAT32 tensors values beyond the fp16 range overflow, which the
+ * reference's fp32 kernel does not.  K and V of one (batch, head) must span
+ * less than 4 GiB (16-bit tensors).
  * head_dim: 32, 64, 128 and 256 have kernels of their size; any other multiple of
  * 8 up to 256 runs on the next of these sizes with the missing columns read as
  * zeros (K and V of one (batch, head) then span less than 2 GiB); anything else

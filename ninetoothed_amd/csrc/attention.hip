@@ -821,7 +821,141 @@ __global__ __launch_bounds__(256) void attention_narrow_kernel(const float *src,
     }
 }
 
-int attention_float32(AttentionParams p, int head_dim, const NineToothedTensor &k, const NineToothedTensor &v, hipStream_t stream) {
+// fp32 tensors as they are, for head dimensions 32, 64 and 128: every product and sum in fp32 on the 32x32x2 fp32
+// MFMA (a sixteenth of the fp16 rate), nothing narrowed.  One wave per 32 query rows, four waves per workgroup, no
+// LDS and no barriers: operands go from global memory straight into MFMA registers.  Same transposed formulation
+// as the fp16 kernel -- S^T[kv, q] = K[kv, :] . Q'[q, :], O^T[d, q] += V^T[d, kv] . P^T[kv, q] -- with 32-key blocks.
+// The two contraction slots of an MFMA belong to lane halves g = 0, 1: for S^T they are d = g * D/2 + step (a lane
+// reads half a row of K, contiguous), for O^T the keys that the lane's S^T accumulator `r` holds for g = 0 and 1.
+template <int D>
+__global__ __launch_bounds__(256) void attention_f32_kernel(AttentionParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    constexpr int BM = 128, BN = 32, DT = D / 32, kHalf = D / 2;
+    typedef float float4_t __attribute__((ext_vector_type(4)));
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int g = lane >> 5, l32 = lane & 31;
+    const int q_blocks = p.q_blocks;
+    // causal: long query blocks first
+    const int qb = p.causal ? q_blocks - 1 - (int)(blockIdx.x % q_blocks) : (int)(blockIdx.x % q_blocks);
+    const int bh = blockIdx.x / q_blocks;
+    const int head = bh % p.heads, batch = bh / p.heads;
+    const int q0 = qb * BM + wave * 32;
+    if (q0 >= p.seq_q) return;  // (no barriers in this kernel)
+    const int q_row = q0 + l32;
+    const float *Q = (const float *)p.q + batch * p.q_strides[0] + head * p.q_strides[1];
+    const float *K = (const float *)p.k + batch * p.k_strides[0] + head * p.k_strides[1];
+    const float *V = (const float *)p.v + batch * p.v_strides[0] + head * p.v_strides[1];
+    float *O = (float *)p.o + batch * p.o_strides[0] + head * p.o_strides[1];
+
+    float qf[kHalf];
+    {
+        const float *src = Q + (int64_t)min(q_row, p.seq_q - 1) * p.q_strides[2] + g * kHalf;
+#pragma unroll
+        for (int c = 0; c < kHalf / 4; ++c) {
+            const float4_t v = *(const float4_t *)(src + 4 * c);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) qf[4 * c + e] = v[e] * p.q_scale;
+        }
+    }
+    float16_t o_acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o_acc[dt][r] = 0.0f;
+    float m_run = -INFINITY, l_run = 0.0f;  // l_run: this lane's half of the row sum
+
+    const int kv_end = p.causal ? min(p.seq_k, q0 + 32) : p.seq_k;  // keys beyond the wave's last row are masked for all of its rows
+    for (int kv0 = 0; kv0 < kv_end; kv0 += BN) {
+        float16_t s_acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s_acc[r] = 0.0f;
+        {
+            const float *src = K + (int64_t)min(kv0 + l32, p.seq_k - 1) * p.k_strides[2] + g * kHalf;
+#pragma unroll
+            for (int c = 0; c < kHalf / 4; ++c) {
+                const float4_t v = *(const float4_t *)(src + 4 * c);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) s_acc = __builtin_amdgcn_mfma_f32_32x32x2f32(v[e], qf[4 * c + e], s_acc, 0, 0, 0);
+            }
+        }
+        const bool tail = kv0 + BN > p.seq_k;
+        if (tail || (p.causal && kv0 + BN - 1 > q0)) {  // (uniform over the wave)
+            const int last_key = (p.causal ? min(p.seq_k - 1, q_row) : p.seq_k - 1) - kv0 - 4 * g;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                if (8 * (r >> 2) + (r & 3) > last_key) s_acc[r] = -INFINITY;
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s_acc[r]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);
+        const float m_use = m_new == -INFINITY ? 0.0f : m_new;  // fully masked so far
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+        m_run = m_new;
+        float sum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            s_acc[r] = __builtin_amdgcn_exp2f(s_acc[r] - m_use);
+            sum += s_acc[r];
+        }
+        l_run = l_run * alpha + sum;
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o_acc[dt][r] *= alpha;
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int kv = kv0 + 8 * (r >> 2) + 4 * g + (r & 3);
+            const float *src = V + (int64_t)min(kv, p.seq_k - 1) * p.v_strides[2] + l32;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                float value = src[dt * 32];
+                if (tail && kv >= p.seq_k) value = 0.0f;  // (its probability is 0; the row read instead may hold anything)
+                o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(value, s_acc[r], o_acc[dt], 0, 0, 0);
+            }
+        }
+    }
+    const float l_total = l_run + __shfl_xor(l_run, 32, 64);
+    const float inv = 1.0f / l_total;
+    if (q_row < p.seq_q) {
+        float *dst = O + (int64_t)q_row * p.o_strides[2];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                float4_t out;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) out[e] = o_acc[dt][r4 * 4 + e] * inv;
+                *(float4_t *)(dst + dt * 32 + 8 * r4 + 4 * g) = out;
+            }
+    }
+#endif
+}
+
+template <int D>
+int launch_attention_f32(AttentionParams &p, hipStream_t stream) {
+    p.q_blocks = ceil_div(p.seq_q, 128);
+    const int64_t grid = (int64_t)p.batch * p.heads * p.q_blocks;
+    if (grid == 0) return 0;
+    if (grid > 0x7fffffffll) return NINETOOTHED_NO_KERNEL;
+    attention_f32_kernel<D><<<dim3((unsigned)grid), dim3(256), 0, stream>>>(p);
+    return (int)hipGetLastError();
+}
+
+// fp32 tensors.  Head dimensions 32, 64 and 128 without block-size hints: the fp32 kernel above.  Other head
+// dimensions, and calls with a hint (the fast way: sixteen times the MFMA rate): the 16-bit kernels on fp16 copies
+// of K and V (values beyond the fp16 range overflow there).
+int attention_float32(AttentionParams p, int head_dim, const NineToothedTensor &k, const NineToothedTensor &v, bool exact, hipStream_t stream) {
+    // (rows of K are read 16 bytes at a time)
+    if (exact && k.strides[3] == 1 && v.strides[3] == 1 && ((uintptr_t)k.data & 15) == 0 && k.strides[0] % 4 == 0 && k.strides[1] % 4 == 0 && k.strides[2] % 4 == 0) {
+        if (head_dim == 128) return launch_attention_f32<128>(p, stream);
+        if (head_dim == 64) return launch_attention_f32<64>(p, stream);
+        if (head_dim == 32) return launch_attention_f32<32>(p, stream);
+    }
     const int64_t total = (int64_t)p.batch * p.heads * p.seq_k * head_dim;
     WorkspaceLease lease(stream);
     half_t *narrow = (half_t *)lease.get(kWorkspaceAttentionNarrow, (size_t)total * 2 * sizeof(half_t));
@@ -974,7 +1108,7 @@ extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineT
     const int status = attention_setup(p, q, k, v, is_causal, scale, o, dtype);
     if (status != 0) return status < 0 ? 0 : status;
     const int head_dim = p.head_dim;
-    if (dtype == NINETOOTHED_FLOAT32) return attention_float32(p, head_dim, k, v, (hipStream_t)stream);
+    if (dtype == NINETOOTHED_FLOAT32) return attention_float32(p, head_dim, k, v, block_size_m == 0 && block_size_n == 0, (hipStream_t)stream);
     // block sizes are hints: 256 query rows select the one-workgroup-per-CU variant, 32-key blocks the
     // three-workgroups-per-CU variant, 64-key blocks the plain loop.  Without a hint the choice is the one
     // tuned for this problem (nt_tune_attention), else the pipelined loop (measured at [4, 32, 4096, 128]:

@@ -956,6 +956,43 @@ def test_attention_float32_tensors(seq_len, is_causal):
     assert torch.allclose(_attention(q.cuda(), k_view.cuda(), v.cuda(), is_causal), expected, rtol=0.025, atol=0.025)
 
 
+@pytest.mark.parametrize("is_causal", (False, True))
+@pytest.mark.parametrize("batch, heads, seq_q, seq_k, emb_dim", ((2, 3, 200, 200, 64), (1, 2, 77, 77, 128), (2, 2, 130, 130, 32), (1, 3, 50, 211, 64), (1, 2, 300, 45, 128)))
+def test_attention_float32_tensors_are_not_narrowed(batch, heads, seq_q, seq_k, emb_dim, is_causal):
+    """Head dimensions 32, 64 and 128 of fp32 tensors run in fp32 throughout: against a float64 reference at fp32
+    tolerances, on operands that the fp16 range does not hold (keys around 1e5 against queries around 1e-5, values
+    around 1e6), ragged and unequal lengths, K and V inside Inf-filled rows."""
+    generator = torch.Generator().manual_seed(seq_q + emb_dim)
+    q = torch.randn(batch, heads, seq_q, emb_dim, generator=generator) * 1e-5
+    wide_k = torch.full((batch, heads, seq_k, emb_dim + 4), float("inf"))
+    wide_v = torch.full((batch, heads, seq_k, emb_dim + 4), float("inf"))
+    wide_k[..., :emb_dim] = torch.randn(batch, heads, seq_k, emb_dim, generator=generator) * 1e5
+    wide_v[..., :emb_dim] = torch.randn(batch, heads, seq_k, emb_dim, generator=generator) * 1e6
+    k, v = wide_k.cuda()[..., :emb_dim], wide_v.cuda()[..., :emb_dim]
+    scale = emb_dim**-0.5
+    out = _attention(q.cuda(), k, v, is_causal, scale)
+    assert out.dtype == torch.float32
+    scores = (q.double().cuda() * scale) @ k.double().transpose(-1, -2)
+    assert float(scores.abs().max()) > 2.0  # (the softmax is not flat)
+    if is_causal:
+        visible = torch.ones(seq_q, seq_k, dtype=torch.bool, device="cuda").tril()
+        scores = scores.masked_fill(~visible, float("-inf"))
+    expected = torch.softmax(scores, dim=-1) @ v.double()
+    assert torch.allclose(out.double(), expected, rtol=2e-4, atol=2e-4 * 1e6)
+
+
+def test_attention_float32_with_block_size_hints_runs_on_narrowed_copies():
+    from ninetoothed_amd import runtime
+
+    q, k, v = (torch.randn(2, 2, 150, 64, device="cuda") for _ in range(3))
+    o = torch.full_like(q, float("nan"))
+    tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (q, k, v)]
+    causal, scale = runtime.ArgumentTensor.from_scalar(0), runtime.ArgumentTensor.from_scalar(0.125)
+    fp32 = runtime.DATA_TYPE_INDEX["fp32"]
+    runtime.check(runtime.library().launch_nt_attention(runtime.current_stream(), *tensors, causal, scale, runtime.ArgumentTensor.from_torch_tensor(o), fp32, 128, 64))
+    assert torch.allclose(o, F.scaled_dot_product_attention(q, k, v, scale=0.125), rtol=0.025, atol=0.025)
+
+
 @pytest.mark.parametrize("m", (1, 100, 1000, 4097))
 @pytest.mark.parametrize("addmm", (False, True))
 def test_gemm_any_number_of_rows_on_the_direct_to_lds_path(m, addmm):
