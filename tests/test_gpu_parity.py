@@ -691,17 +691,24 @@ def test_scratch_buffers_are_reused_grown_and_released():
         x, w = _randn(n, c, hw, hw, scale=0.1).cuda(), _randn(k, c, 3, 3, scale=0.1).cuda()
         return x, w, F.conv2d(x.float(), w.float(), padding=1).half()
 
-    cases = [conv_case(4, 64, 16, 256), conv_case(2, 32, 8, 256), conv_case(8, 64, 24, 512)]
+    def repacked(x, w):  # the way that uses scratch memory, by name
+        out = torch.full((x.shape[0], w.shape[0], x.shape[2], x.shape[3]), float("nan"), dtype=x.dtype, device="cuda")
+        tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (x, w, out)]
+        runtime.check(runtime.library().launch_nt_conv2d(runtime.current_stream(), *tensors, runtime.DATA_TYPE_INDEX["fp16"], 1, 1, 2, 0, 0))
+        return out
+
+    cases = [conv_case(4, 64, 16, 256), conv_case(2, 32, 24, 256), conv_case(8, 64, 24, 512)]
     side = torch.cuda.Stream()
     for round_ in range(2):
         for x, w, expected in cases:
-            assert torch.allclose(_conv2d(x, w, (1, 1)), expected, **HALF_TOL)
+            assert torch.allclose(repacked(x, w), expected, **HALF_TOL)
         torch.cuda.synchronize()
         with torch.cuda.stream(side):
             x, w, expected = cases[0]
-            assert torch.allclose(_conv2d(x, w, (1, 1)), expected, **HALF_TOL)
+            assert torch.allclose(repacked(x, w), expected, **HALF_TOL)
         side.synchronize()
-        q, k, v = (torch.randn(1, 2, 300 - 100 * round_, 64, device="cuda") for _ in range(3))
+        # (a head dimension without an fp32 kernel of its own: K and V are narrowed into the scratch buffer)
+        q, k, v = (torch.randn(1, 2, 300 - 100 * round_, 96, device="cuda") for _ in range(3))
         o = _attention(q, k, v, scale=0.125)
         assert torch.allclose(o, F.scaled_dot_product_attention(q, k, v, scale=0.125), rtol=0.025, atol=0.025)
         torch.cuda.synchronize()
