@@ -25,7 +25,9 @@ import threading
 
 from ninetoothed_amd import runtime
 
-CACHE_DIR = pathlib.Path.home() / ".ninetoothed_amd" / "auto_tuning"
+# where tuned choices are kept between processes; NINETOOTHED_AMD_CACHE_DIR moves it (and make's kernel
+# descriptions) away from the home directory
+CACHE_DIR = pathlib.Path(os.environ.get("NINETOOTHED_AMD_CACHE_DIR") or pathlib.Path.home() / ".ninetoothed_amd") / "auto_tuning"
 
 _lock = threading.Lock()
 _loaded = False

@@ -18,6 +18,7 @@ shapes / strides / dtypes, prepares a launch plan for ``libnt_hip.so``.
 
 import hashlib
 import inspect
+import os
 import pathlib
 
 from ninetoothed_amd import recognition, runtime
@@ -25,7 +26,7 @@ from ninetoothed_amd.recognition import UnsupportedProgram
 from ninetoothed_amd.symbol import Symbol
 from ninetoothed_amd.tensor import Tensor
 
-CACHE_DIR = pathlib.Path.home() / ".ninetoothed_amd"
+CACHE_DIR = pathlib.Path(os.environ.get("NINETOOTHED_AMD_CACHE_DIR") or pathlib.Path.home() / ".ninetoothed_amd")
 
 _TORCH_DTYPE_TAGS = None
 
