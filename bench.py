@@ -45,16 +45,21 @@ def parse_args():
     parser.add_argument("--only", action="store_true", help="measure only --workload")
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-vendor", action="store_true", help="skip the stock PyTorch operators")
+    parser.add_argument("--inputs", choices=("randn", "constant"), default="randn",
+                        help="`constant` fills every tensor with one value instead of the seeded normal values the metric is quoted on: "
+                             "the matrix pipe then draws far less power and the part keeps its clock (a diagnostic, never the reported figure)")
     return parser.parse_args()
 
 
-def build_workloads():
+def build_workloads(inputs="randn"):
     import torch
 
     import ninetoothed_amd as ninetoothed
     from ninetoothed_amd import programs
 
     def seeded(*shape, dtype=torch.float16, scale=1.0, seed=0):
+        if inputs == "constant":
+            return torch.full(shape, 0.5 * scale, dtype=dtype)
         generator = torch.Generator().manual_seed(seed)
         return (torch.randn(*shape, generator=generator) * scale).to(dtype)
 
@@ -336,7 +341,7 @@ def main():
         sys.exit(2)
     torch.cuda.set_device(0)
 
-    workloads = build_workloads()
+    workloads = build_workloads(args.inputs)
     if args.workload not in workloads:
         print(f"unknown workload `{args.workload}`; choose from {sorted(workloads)}", file=sys.stderr)
         sys.exit(2)
@@ -392,7 +397,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f16" if main_roofline["bound"] == "mfma" else "f32",
-        "data": "synthetic",
+        "data": "synthetic" if args.inputs == "randn" else "synthetic, every operand a constant (diagnostic run: not the inputs the metric is quoted on)",
         "config": dict(main_workload["describe"], launch=launch_plan),
         "roofline": main_roofline,
         "per_launch": single,
