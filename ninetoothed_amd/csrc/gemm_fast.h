@@ -106,6 +106,13 @@ NT_DEVICE void lds_barrier_reads_in_flight() {
     __builtin_amdgcn_sched_barrier(0);
 }
 
+#ifndef NT_GEMM_SCHEDULE
+#define NT_GEMM_SCHEDULE 1
+#endif
+#ifndef NT_GEMM_M16
+#define NT_GEMM_M16 1
+#endif
+
 // kAblate is a measurement aid (bit 0: no global loads inside the K loop,
 // bit 1: operand fragments read from LDS only once); 0 in every shipped instance.
 template <typename T, int BM, int BN, int BK, int WM, int WN, int kStages, int kWavesPerSimd, bool kAddmm, int kAblate = 0, int kLoad = 0, int kAux = 0,
@@ -390,13 +397,154 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     // barrier have their operands in registers, and no wave starts a step by waiting for LDS.
     constexpr bool kCross = kStages >= 3 && kAblate == 0 && KS % 2 == 0;
 
+    // kM16: the wave's tile is computed with 16x16x32 MFMAs instead of 32x32x16 ones.  Per FLOP they move
+    // half as many accumulator values through the register file, and on operands with random bits that
+    // is what the power limit of the part charges for (8192^3 addmm, N(0,1) fp16: +8 %).
+    constexpr bool kM16 = NT_GEMM_M16 && kAblate == 0 && BK % 32 == 0 && sizeof(T) == 2;
+    constexpr int TM16 = kWaveM / 16, TN16 = kWaveN / 16, KS16 = BK / 32;
+    // ... with the fragment reads of the next k step under the MFMAs of this one, across the barrier
+    constexpr bool kCross16 = kM16 && kStages >= 3 && (KS16 * TM16) % 4 == 0 && TM16 >= TN16;
+    float4_t acc16[kM16 ? TM16 : 1][kM16 ? TN16 : 1];
+#pragma unroll
+    for (int ti = 0; ti < (kM16 ? TM16 : 1); ++ti)
+#pragma unroll
+        for (int tj = 0; tj < (kM16 ? TN16 : 1); ++tj) acc16[ti][tj] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    // Operand fragments of the 16x16x32 MFMA: A block ti (16 rows) is one 16-byte read per lane (row i16,
+    // k chunk kg of the k step); B block tj (16 columns) is two transposing reads (16-lane group kg reads
+    // k rows 8 kg .. + 7 of the k step), or, for a k-contiguous B, one read like A's.
+    const int kg = lane >> 4;
+    int a16_off[KS16], bt16_off[KS16];
+    {
+        const int a_row = wave_m * kWaveM + i16;  // + 16 * ti, which leaves the swizzle term as it is
+        const int bt_row = wave_n * kWaveN + i16;
+#pragma unroll
+        for (int ks = 0; ks < KS16; ++ks) {
+            a16_off[ks] = a_row * (BK * 2) + (((ks * 4 + kg) ^ a_phys_chunk<BK>(a_row, 0)) * 16);
+            bt16_off[ks] = bt_row * (BK * 2) + (((ks * 4 + kg) ^ a_phys_chunk<BK>(bt_row, 0)) * 16);
+        }
+    }
+    int b16_lo[kM16 && !kBT ? TN16 : 1], b16_hi[kM16 && !kBT ? TN16 : 1];
+    if constexpr (kM16 && !kBT) {
+#pragma unroll
+        for (int tj = 0; tj < TN16; ++tj) {
+            const int k_lo = 8 * kg + (i16 >> 2), k_hi = k_lo + 4;  // + 32 * ks: the swizzle only looks at k % 8
+            const int ncol = wave_n * kWaveN + tj * 16 + 4 * (i16 & 3);
+            b16_lo[tj] = k_lo * (BN * 2) + b_phys_chunk<BN>(k_lo, ncol >> 3) * 16 + (ncol & 7) * 2;
+            b16_hi[tj] = k_hi * (BN * 2) + b_phys_chunk<BN>(k_hi, ncol >> 3) * 16 + (ncol & 7) * 2;
+        }
+    }
+    auto read_a16 = [&](auto stage_tag, int ks, int ti) -> vec8 {
+        return *(const NT_LDS vec8 *)(stage_a(stage_tag) + a16_off[ks] + ti * 16 * (BK * 2));
+    };
+    auto read_b16 = [&](auto stage_tag, int ks, int tj) -> vec8 {
+        const NT_LDS unsigned char *sb = stage_b(stage_tag);
+        if constexpr (kBT) {
+            return *(const NT_LDS vec8 *)(sb + bt16_off[ks] + tj * 16 * (BK * 2));
+        } else {
+            short4_t lo = lds_read_tr16_b64(sb + b16_lo[kBT ? 0 : tj] + ks * 32 * (BN * 2));
+            short4_t hi = lds_read_tr16_b64(sb + b16_hi[kBT ? 0 : tj] + ks * 32 * (BN * 2));
+            short8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            return __builtin_bit_cast(vec8, both);
+        }
+    };
+
     static_for<0, kStages - 1>([&](auto s) { issue_loads(s, min((int)decltype(s)::value, last_k)); });
+    if constexpr (kCross16) {
+        // All TN16 B fragments of a k step stay in registers (two sets, taking turns k step by k step); the
+        // A fragments stream through four slots, each read two blocks ahead of its MFMAs.
+        constexpr int Q = KS16 * TM16;  // A fragments of a k tile, in the order they are used
+        vec8 as[4];
+        vec8 bs[2][TN16];
+        wait_vmcnt<(kStages - 2) * kLoadsPerTile>();
+        lds_barrier();
+#pragma unroll
+        for (int tj = 0; tj < TN16; ++tj) bs[0][tj] = read_b16(std::integral_constant<int, 0>(), 0, tj);
+        as[0] = read_a16(std::integral_constant<int, 0>(), 0, 0);
+        as[1] = read_a16(std::integral_constant<int, 0>(), 1 / TM16, 1 % TM16);
+        auto step = [&](auto i_tag, int kt) {
+            constexpr int kI = decltype(i_tag)::value;  // position in the unrolled loop body: stage and B set follow from it
+            constexpr int kS = kI % kStages;
+            typedef std::integral_constant<int, kS> Stage;
+            typedef std::integral_constant<int, (kS + 1) % kStages> NextStage;
+            wait_vmcnt<(kStages - 3) * kLoadsPerTile>();
+            lds_barrier_reads_in_flight();
+            issue_loads(std::integral_constant<int, (kS + kStages - 1) % kStages>(), min(kt + kI + kStages - 1, last_k));
+            static_for<0, Q>([&](auto q_tag) {
+                constexpr int q = decltype(q_tag)::value;
+                constexpr int ks = q / TM16, ti = q % TM16;
+                constexpr int cur = (kI * KS16 + ks) & 1, nxt = cur ^ 1;
+                constexpr int kBReadsPerBlock = kBT ? 1 : 2;
+                constexpr bool kReadsB = ti >= TM16 - TN16;
+                if constexpr (q + 2 < Q) as[(q + 2) % 4] = read_a16(Stage(), (q + 2) / TM16, (q + 2) % TM16);
+                else as[(q + 2) % 4] = read_a16(NextStage(), (q + 2 - Q) / TM16, (q + 2 - Q) % TM16);
+                if constexpr (kReadsB) {
+                    constexpr int tj = ti - (TM16 - TN16);
+                    if constexpr (ks + 1 < KS16) bs[nxt][tj] = read_b16(Stage(), ks + 1, tj);
+                    else bs[nxt][tj] = read_b16(NextStage(), 0, tj);
+                }
+#pragma unroll
+                for (int tj = 0; tj < TN16; ++tj) acc16[ti][tj] = E::mfma16(bs[cur][tj], as[q % 4], acc16[ti][tj]);  // transposed block
+#if NT_GEMM_SCHEDULE
+                // issue order: reads and ring refills spread under the MFMAs
+                constexpr int kReads = 1 + (kReadsB ? kBReadsPerBlock : 0);
+                constexpr int kFillsPer = (kLoadsPerTile + Q - 1) / Q;
+                constexpr int kFills = q * kFillsPer < kLoadsPerTile ? (kLoadsPerTile - q * kFillsPer < kFillsPer ? kLoadsPerTile - q * kFillsPer : kFillsPer) : 0;
+                static_for<0, TN16>([&](auto j_tag) {
+                    constexpr int j = decltype(j_tag)::value;
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    if constexpr (TN16 >= kReads) {
+                        if constexpr (j < kReads) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    } else if constexpr (j == 0) {
+                        __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
+                    }
+                    if constexpr (j == (TN16 > 1 ? 1 : 0) && kFills > 0) __builtin_amdgcn_sched_group_barrier(0x020, kFills, 0);
+                });
+#endif
+            });
+        };
+        // (with an odd number of k steps per tile the B sets are back in place after an even number of tiles)
+        constexpr int kBody = (KS16 & 1) ? 2 * kStages : kStages;
+        const int body_k = num_k - num_k % kBody;
+        for (int kt = 0; kt < body_k; kt += kBody) {
+            static_for<0, kBody>([&](auto i) { step(i, kt); });
+        }
+        static_for<0, kBody - 1>([&](auto i) {
+            if (body_k + (int)decltype(i)::value < num_k) step(i, body_k);
+        });
+    } else if constexpr (kM16) {
+        auto step = [&](auto s, int kt) {
+            constexpr int kS = decltype(s)::value;
+            wait_vmcnt<(kStages - 2) * kLoadsPerTile>();
+            lds_barrier();
+            issue_loads(std::integral_constant<int, (kS + kStages - 1) % kStages>(), min(kt + kS + kStages - 1, last_k));
+#pragma unroll
+            for (int ks = 0; ks < KS16; ++ks) {
+                vec8 bfr[TN16];
+#pragma unroll
+                for (int tj = 0; tj < TN16; ++tj) bfr[tj] = read_b16(s, ks, tj);
+#pragma unroll
+                for (int ti = 0; ti < TM16; ++ti) {
+                    const vec8 afr = read_a16(s, ks, ti);
+#pragma unroll
+                    for (int tj = 0; tj < TN16; ++tj) acc16[ti][tj] = E::mfma16(bfr[tj], afr, acc16[ti][tj]);  // transposed block
+                }
+            }
+        };
+        for (int kt = 0; kt < main_k; kt += kStages) {
+            static_for<0, kStages>([&](auto s) { step(s, kt); });
+        }
+        static_for<0, kStages - 1>([&](auto s) {
+            if (main_k + (int)decltype(s)::value < num_k) step(s, main_k);
+        });
+    }
     if constexpr (kAblate & 2) {
         wait_vmcnt<0>();
         lds_barrier();
         read_frags(std::integral_constant<int, 0>(), 0, af_once, bf_once);
     }
-    if constexpr (kCross) {
+    if constexpr (kM16) {
+        // (done above)
+    } else if constexpr (kCross) {
         vec8 af[2][TM];
         vec8 bf[2][TN];
         wait_vmcnt<(kStages - 2) * kLoadsPerTile>();
@@ -419,9 +567,6 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
                 for (int ti = 0; ti < TM; ++ti)
 #pragma unroll
                     for (int tj = 0; tj < TN; ++tj) acc[ti][tj] = E::mfma32(bf[cur][tj], af[cur][ti], acc[ti][tj]);  // transposed tile
-#ifndef NT_GEMM_SCHEDULE
-#define NT_GEMM_SCHEDULE 1
-#endif
 #if NT_GEMM_SCHEDULE
                 // issue order: the fragment reads of the next k step (and, in a step's first k step, the
                 // refills of the ring) spread under this k step's MFMAs
@@ -506,6 +651,29 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     const int slab_sw = (l32 >> kCShift) & (kCChunks - 1);
 #pragma unroll
     for (int ti = 0; ti < TM; ++ti) {
+        if constexpr (kM16) {
+            // 16x16 blocks: lane (i16, kg) holds columns 4 kg .. + 3 of row i16; two blocks of rows fill a slab
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const int row = half * 16 + i16;
+                const int sw = (row >> kCShift) & (kCChunks - 1);
+#pragma unroll
+                for (int tj = 0; tj < TN16; ++tj) {
+                    typedef TOut vec4 __attribute__((ext_vector_type(4)));
+                    const float4_t a4 = acc16[kM16 ? 2 * ti + half : 0][kM16 ? tj : 0];
+                    vec4 v;
+                    if constexpr (kFloatOut) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = a4[e];
+                        *(NT_LDS vec4 *)(slab + row * kRowBytes + ((tj * 4 + kg) ^ sw) * 16) = v;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = E::from_float(a4[e]);
+                        *(NT_LDS vec4 *)(slab + row * kRowBytes + ((tj * 2 + (kg >> 1)) ^ sw) * 16 + 8 * (kg & 1)) = v;
+                    }
+                }
+            }
+        } else
 #pragma unroll
         for (int tj = 0; tj < TN; ++tj) {
 #pragma unroll
