@@ -141,7 +141,7 @@ def build_workloads(inputs="randn"):
         return dict(step=lambda: dst.copy_(src), work=2.0 * (1 << 30), bound="hbm", kernel=_Copy(),
                     describe={"workload": "device copy of 1 GiB (2 GiB of traffic), counter calibration only"})
 
-    def mfma_ceiling(constant):
+    def mfma_ceiling(constant, form="32x32x16"):
         # not a program of the library: MFMAs on register operands taken from the addmm workload's own inputs
         # (or from constants), which bounds what the GEMM and attention kernels can reach on this data
         def make():
@@ -158,23 +158,26 @@ def build_workloads(inputs="randn"):
             loops = 4096
             count = ctypes.c_int64(0)
             lib = runtime.library()
+            probe = lib.nt_probe_mfma_rate if form == "32x32x16" else lib.nt_probe_mfma_rate_16x16x32
+            flop_per_mfma = 2 * 32 * 32 * 16 if form == "32x32x16" else 2 * 16 * 16 * 32
 
             def step():
-                runtime.check(lib.nt_probe_mfma_rate(runtime.current_stream(), runtime.ArgumentTensor.from_torch_tensor(mat1), runtime.ArgumentTensor.from_torch_tensor(mat2),
-                                                     loops, sink.data_ptr(), ctypes.byref(count)))
+                runtime.check(probe(runtime.current_stream(), runtime.ArgumentTensor.from_torch_tensor(mat1), runtime.ArgumentTensor.from_torch_tensor(mat2),
+                                    loops, sink.data_ptr(), ctypes.byref(count)))
 
             step()
 
             class _Probe:
-                last_plan = "nt_probe_mfma_rate (measurement aid, not a program)"
+                last_plan = ("nt_probe_mfma_rate" if form == "32x32x16" else "nt_probe_mfma_rate_16x16x32") + " (measurement aid, not a program)"
 
-            return dict(step=step, work=float(count.value) * 2 * 32 * 32 * 16, bound="mfma", kernel=_Probe(),
-                        describe={"workload": "MFMA 32x32x16 fp16 issue rate on register operands, " + ("constant 0.5" if constant else "the addmm workload's N(0,1) inputs")})
+            return dict(step=step, work=float(count.value) * flop_per_mfma, bound="mfma", kernel=_Probe(),
+                        describe={"workload": "MFMA " + form + " fp16 issue rate on register operands, " + ("constant 0.5" if constant else "the addmm workload's N(0,1) inputs")})
         return make
 
     workloads["addmm_8192"] = addmm_8192
     workloads["mfma_ceiling"] = mfma_ceiling(False)
     workloads["mfma_ceiling_constant"] = mfma_ceiling(True)
+    workloads["mfma_ceiling_16x16x32"] = mfma_ceiling(False, "16x16x32")  # the form the GEMM kernel issues
     workloads["matmul_512"] = matmul_512
     workloads["softmax_4096"] = softmax_4096
     workloads["attention"] = attention(False)
@@ -371,7 +374,7 @@ def main():
     others = {}
     if not args.only:
         # (the MFMA-only probe goes last: it heats the part more than any program does)
-        for name, factory in sorted(workloads.items(), key=lambda item: item[0] == "mfma_ceiling"):
+        for name, factory in sorted(workloads.items(), key=lambda item: item[0].startswith("mfma_ceiling")):
             if name == args.workload or name in ("copy_1gib", "mfma_ceiling_constant"):
                 continue
             workload = factory()

@@ -321,9 +321,15 @@ int nt_tune_lookup(int kind, const int *values, int count);
  * `b` (dense row-major matrices of at least 4096 elements) -- no LDS, no memory traffic inside the loop.  The rate bounds what a GEMM or attention kernel can reach on
  * the same operand values (random values draw more power in the matrix pipe than constants, and the clock
  * follows).  `sink` is a device float the kernel may write; *mfma_count receives the MFMAs issued in total
- * (65536 FLOP each).  Asynchronous on `stream`. */
+ * (2 x 32 x 32 x 16 = 32768 FLOP each).  Asynchronous on `stream`. */
 NineToothedResult nt_probe_mfma_rate(NineToothedStream stream, NineToothedTensor a, NineToothedTensor b,
                                      int loops, float *sink, int64_t *mfma_count);
+
+/* The same with the 16x16x32 form of the instruction, which the fast GEMM kernel uses: `loops` x 32 MFMAs per
+ * wave, 2 x 16 x 16 x 32 = 16384 FLOP each.  Same FLOP per clock; on random operands the part sustains a
+ * higher clock with it (per FLOP half as many accumulator values move through the register file). */
+NineToothedResult nt_probe_mfma_rate_16x16x32(NineToothedStream stream, NineToothedTensor a, NineToothedTensor b,
+                                              int loops, float *sink, int64_t *mfma_count);
 
 /*
  * Element-wise / reducing tile programs that are none of the programs above.

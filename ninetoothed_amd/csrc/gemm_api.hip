@@ -345,9 +345,6 @@ const GemmInstance kInstances[] = {
     NT_LOAD_INSTANCE(256, 256, 32, 2, 4, 4, 2, 1, 0),
     NT_LOAD_INSTANCE(256, 256, 32, 2, 2, 4, 1, 1, 0),
     NT_LOAD_INSTANCE(256, 256, 64, 2, 2, 2, 1, 1, 0),
-    NT_LOAD_INSTANCE(128, 256, 32, 2, 2, 4, 2, 1, 0),
-    NT_LOAD_INSTANCE(128, 256, 32, 2, 2, 3, 2, 1, 0),
-    NT_LOAD_INSTANCE(256, 128, 32, 2, 2, 3, 2, 1, 0),
     NT_LOAD_INSTANCE(128, 256, 32, 1, 4, 3, 2, 1, 0),
     NT_ABLATED_INSTANCE(256, 256, 32, 2, 4, 4, 2, 1),
     NT_ABLATED_INSTANCE(256, 256, 32, 2, 4, 4, 2, 2),

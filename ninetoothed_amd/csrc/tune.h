@@ -23,6 +23,7 @@ void tune_record(int kind, const int *values, int count, int choice, const int *
 // each.  `launch(i)` returns 0, NINETOOTHED_NO_KERNEL (the candidate does not take the problem: skipped) or an
 // error (returned).  *best receives the fastest candidate (-1 when none ran); with a `margin`, a later candidate
 // replaces an earlier one only when it is faster by more than that fraction (candidates in order of preference).
+// The first candidate is preceded by an untimed warm-up of about 20 ms.
 // Synchronises; returns without timing anything (*best = -1, result 0) when the stream is being captured into a graph.
 template <typename Launch>
 int tune_time(hipStream_t stream, int candidates, int iters, Launch launch, int *best, float *best_ms, float margin = 0.0f) {
@@ -43,10 +44,28 @@ int tune_time(hipStream_t stream, int candidates, int iters, Launch launch, int 
         return (int)err;
     }
     int result = 0;
+    bool warm = false;
     for (int i = 0; i < candidates && result == 0; ++i) {
         int rc = launch(i);
         if (rc == 1) continue;  // NINETOOTHED_NO_KERNEL
         if (rc == 0) rc = launch(i);
+        if (rc != 0) {
+            result = rc;
+            break;
+        }
+        // The first candidate that runs would otherwise be timed on an idle part whose clocks are still ramping up,
+        // and lose to a slower one timed later: it first runs untimed for about 20 ms (at most 64 rounds).
+        float warmed_ms = 0.0f;
+        for (int round = 0; !warm && round < 64 && warmed_ms < 20.0f && rc == 0; ++round) {
+            (void)hipEventRecord(start, stream);
+            for (int r = 0; r < iters && rc == 0; ++r) rc = launch(i);
+            (void)hipEventRecord(stop, stream);
+            if (rc == 0 && (err = hipEventSynchronize(stop)) != hipSuccess) rc = (int)err;
+            float ms = 0.0f;
+            if (rc == 0) (void)hipEventElapsedTime(&ms, start, stop);
+            warmed_ms += ms;
+        }
+        warm = true;
         if (rc != 0) {
             result = rc;
             break;

@@ -85,6 +85,7 @@ _SIGNATURES = {
     "nt_tune_conv2d": (_S, _T, _T, _T, _I, _I, _I, _I, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_float)),
     "nt_tune_lookup": (_I, ctypes.POINTER(ctypes.c_int), _I),
     "nt_probe_mfma_rate": (_S, _T, _T, _I, ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64)),
+    "nt_probe_mfma_rate_16x16x32": (_S, _T, _T, _I, ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64)),
     "launch_nt_map": (_S, ctypes.c_void_p),
     "nt_map_source": (ctypes.c_void_p, ctypes.c_char_p, _I),
     "nt_tune_cache_save": (ctypes.c_char_p,),

@@ -250,7 +250,7 @@ def test_attention_on_random_shapes():
 
 def test_mfma_rate_probe_runs_and_counts():
     """The measurement aid behind bench.py's ``mfma_ceiling`` workloads: launches, reports the MFMAs it issued
-    (8 waves per compute unit x loops x 8) and leaves its sink untouched."""
+    (8 waves per compute unit x loops x 8; x 32 in the 16x16x32 form) and leaves its sink untouched."""
     import ctypes
 
     from ninetoothed_amd import runtime
@@ -267,3 +267,8 @@ def test_mfma_rate_probe_runs_and_counts():
     assert sink.item() == 0.0
     small = runtime.ArgumentTensor.from_torch_tensor(a[:8, :8].contiguous())
     assert lib.nt_probe_mfma_rate(runtime.current_stream(), small, small, 3, sink.data_ptr(), ctypes.byref(count)) != 0
+    runtime.check(lib.nt_probe_mfma_rate_16x16x32(runtime.current_stream(), tensor, tensor, 3, sink.data_ptr(), ctypes.byref(count)))
+    torch.cuda.synchronize()
+    assert count.value == units * 8 * 3 * 32
+    assert sink.item() == 0.0
+    assert lib.nt_probe_mfma_rate_16x16x32(runtime.current_stream(), small, small, 3, sink.data_ptr(), ctypes.byref(count)) != 0
