@@ -540,7 +540,8 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
             softmax(s_buf[0], p_buf[0], alpha);
             scores(Stage1(), s_buf[1]);
 
-            auto step_body = [&](auto parity_tag, auto masked_tag, int j) __attribute__((always_inline)) {
+            auto step_body = [&](auto parity_tag, auto masked_tag, auto scores_tag, int j) __attribute__((always_inline)) {
+                constexpr bool kScores = decltype(scores_tag)::value;  // false in a wave's last step: no block follows
                 constexpr int kParity = decltype(parity_tag)::value;
                 typedef std::integral_constant<int, kParity> Own;
                 typedef std::integral_constant<int, 1 - kParity> Other;
@@ -578,10 +579,10 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
                     rebase(s_buf[kParity], mx, alpha);
                     exponentials(s_buf[kParity], p_buf[kParity]);
                     accumulate(Other(), p_buf[1 - kParity], PsSplit(), PsEnd());
-                    scores(Other(), s_buf[1 - kParity]);
+                    if constexpr (kScores) scores(Other(), s_buf[1 - kParity]);
                     {
-                        constexpr int kMfma = ((PS - PsSplit::value) * DT + KS * KT) * kQTiles;
-                        constexpr int kReads = (PS - PsSplit::value) * DT * 2 + KS * KT;
+                        constexpr int kMfma = ((PS - PsSplit::value) * DT + (kScores ? KS * KT : 0)) * kQTiles;
+                        constexpr int kReads = (PS - PsSplit::value) * DT * 2 + (kScores ? KS * KT : 0);
                         __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
                         __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
                         static_for<0, kMfma>([&](auto i_tag) __attribute__((always_inline)) {
@@ -595,7 +596,7 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
                 } else {
                 softmax(s_buf[kParity], p_buf[kParity], alpha);
                 accumulate(Other(), p_buf[1 - kParity], PsBegin(), PsEnd());
-                scores(Other(), s_buf[1 - kParity]);
+                if constexpr (kScores) scores(Other(), s_buf[1 - kParity]);
                 // desired issue order inside this region: one MFMA, then the LDS reads
                 // and softmax arithmetic that fit under it
 #ifndef NT_ATTN_SCHEDULE
@@ -607,7 +608,7 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
                 // later one and by at most 28 cycles of softmax arithmetic (4 per VALU
                 // instruction, 8 per exponential).  The first MFMAs overlap the running-max
                 // chain, the exponentials start once the maximum is known.
-                constexpr int kMfmaPerStep = (PS * DT + KS * KT) * kQTiles;
+                constexpr int kMfmaPerStep = (PS * DT + (kScores ? KS * KT : 0)) * kQTiles;
 #ifndef NT_ATTN_HEAD_VALU
 #define NT_ATTN_HEAD_VALU 12
 #endif
@@ -640,6 +641,29 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
                 for (int qt = 0; qt < kQTiles; ++qt) asm volatile("" : "+v"(l_run[qt]));
                 rescale(alpha);
             };
+            // A wave needs the key blocks up to the one that holds the key of its last query row (causal; all of
+            // them otherwise): `mine` of the workgroup's num_blocks.  Its
+            // step `mine` only multiplies P(mine - 1) by V(mine - 1), and later steps only take part in the loads
+            // and barriers of the workgroup -- on the diagonal of a causal problem this spares the waves with the
+            // upper query rows the blocks that the masks would zero entirely.
+            int mine = num_blocks;
+            if (p.causal) mine = min(mine, (q0 + wave * kQTiles * 32 + kQTiles * 32 - 1) / BN + 1);
+            auto product_step = [&](auto parity_tag, int j) __attribute__((always_inline)) {
+                constexpr int kParity = decltype(parity_tag)::value;
+                wait_vmcnt<0>();
+                lds_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+                issue_k(std::integral_constant<int, kParity>(), min(j + 2, last_block));
+                issue_v(std::integral_constant<int, kParity>(), j);
+                accumulate(std::integral_constant<int, 1 - kParity>(), p_buf[1 - kParity], PsBegin(), PsEnd());
+            };
+            auto idle_step = [&](auto parity_tag, int j) __attribute__((always_inline)) {
+                constexpr int kParity = decltype(parity_tag)::value;
+                wait_vmcnt<0>();
+                lds_barrier();
+                issue_k(std::integral_constant<int, kParity>(), min(j + 2, last_block));
+                issue_v(std::integral_constant<int, kParity>(), j);
+            };
             // The blocks that need masks are the last ones.  A first loop runs the pairs
             // of steps that lie entirely before them without the masking arithmetic, a
             // second one the rest with it (masking a block that does not need it changes
@@ -649,21 +673,36 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
             if (p.causal) unmasked = min(unmasked, (q0 + wave * kQTiles * 32 + 1) / BN);
             int j = 1;
             for (; j + 1 < unmasked; j += 2) {
-                step_body(Stage1(), std::false_type(), j);
-                step_body(Stage0(), std::false_type(), j + 1);
+                step_body(Stage1(), std::false_type(), std::true_type(), j);
+                step_body(Stage0(), std::false_type(), std::true_type(), j + 1);
             }
-            for (; j + 1 < num_blocks; j += 2) {
-                step_body(Stage1(), std::true_type(), j);
-                step_body(Stage0(), std::true_type(), j + 1);
+            for (; j + 1 < mine; j += 2) {
+                step_body(Stage1(), std::true_type(), std::true_type(), j);
+                step_body(Stage0(), std::true_type(), std::true_type(), j + 1);
             }
-            if (j < num_blocks) step_body(Stage1(), std::true_type(), j);
+            if (j < mine) {
+                step_body(Stage1(), std::true_type(), std::true_type(), j);
+                ++j;
+            }
+            // (j == mine; the scores of block `mine`, computed in the step before, are never used)
+            for (; j < num_blocks; ++j) {
+                if (j == mine) {
+                    if (j & 1) product_step(Stage1(), j);
+                    else product_step(Stage0(), j);
+                } else {
+                    if (j & 1) idle_step(Stage1(), j);
+                    else idle_step(Stage0(), j);
+                }
+            }
             // drain: P(last) . V(last); V(last) was requested into the stage of its parity
             wait_vmcnt<0>();
             lds_barrier();
-            if ((num_blocks - 1) & 1)
-                accumulate(Stage1(), p_buf[1], PsBegin(), PsEnd());
-            else
-                accumulate(Stage0(), p_buf[0], PsBegin(), PsEnd());
+            if (mine == num_blocks) {
+                if ((num_blocks - 1) & 1)
+                    accumulate(Stage1(), p_buf[1], PsBegin(), PsEnd());
+                else
+                    accumulate(Stage0(), p_buf[0], PsBegin(), PsEnd());
+            }
         }
     }
 

@@ -504,6 +504,24 @@ def test_attention_block_size_hints(block_size_m, block_size_n, emb_dim, is_caus
     assert torch.allclose(out, expected, **HALF_TOL)
 
 
+@pytest.mark.parametrize("emb_dim", (64, 128))
+@pytest.mark.parametrize("batch, heads, seq_q, seq_k", ((8, 32, 300, 333), (8, 32, 600, 200), (2, 16, 1100, 1500), (1, 8, 2048 + 17, 2048 + 17)))
+def test_attention_causal_waves_stop_at_their_last_key_block(batch, heads, seq_q, seq_k, emb_dim):
+    # with a causal mask the waves of a workgroup need different numbers of key blocks (the ones with the upper
+    # query rows fewer); they leave the block loop at different steps but keep loading and synchronising:
+    # ragged ends, more and fewer keys than queries, few and many query blocks
+    q = _randn(batch, heads, seq_q, emb_dim).cuda()
+    k, v = (_randn(batch, heads, seq_k, emb_dim).cuda() for _ in range(2))
+    kernel = ninetoothed.make(
+        programs.attention.arrangement_with_scale, programs.attention.application_with_scale, programs.attention.tensors(True)
+    )
+    expected = _attention_reference(q, k, v, True, emb_dim**-0.5)
+    for _ in range(2):
+        out = torch.full_like(q, float("nan"))
+        kernel(q, k, v, True, emb_dim**-0.5, out)
+        assert torch.allclose(out.float(), expected, **HALF_TOL)
+
+
 @pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
 @pytest.mark.parametrize("emb_dim", (64, 128))
 def test_attention_many_short_sequences(emb_dim, dtype):
