@@ -57,6 +57,25 @@ NT_HOST_DEVICE constexpr int b_phys_chunk(int krow, int chunk) {
     return chunk ^ ((krow & kMask) << 2);
 }
 
+// The A tile for the 16x16x32 MFMA form, whose 16-byte reads address row lane % 16, chunk lane / 16: the LDS
+// serves such a read in four passes of 16 lanes -- {0-3, 12-15, 20-27}, {4-11, 16-19, 28-31} and the same
+// + 32 (measured with two active lanes at a time) -- and with rows of 64 bytes the plain XOR of the row
+// group puts two row groups of a pass on the same banks; XOR with the negated row group does not.  Rows of
+// 128 bytes and more are conflict-free as they are.
+template <int BK>
+NT_HOST_DEVICE constexpr int a_phys_chunk16(int row, int chunk) {
+    if (BK == 32) return chunk ^ ((4 - (row / 4) % 4) % 4);
+    return a_phys_chunk<BK>(row, chunk);
+}
+
+// The same for the 16x16x32 MFMA's transposing reads, where the four 16-lane groups of a wave read k rows
+// 8 apart (k % 8 equal): rows with bit 3 of k set move by another 32 bytes, so that two groups served
+// together do not meet in a bank.
+template <int BN>
+NT_HOST_DEVICE constexpr int b_phys_chunk16(int krow, int chunk) {
+    return b_phys_chunk<BN>(krow, chunk) ^ (((krow >> 3) & 1) << 1);
+}
+
 // Maps the hardware workgroup id to an output tile.  Workgroup ids are dealt
 // round-robin to the 8 XCDs, so ids congruent mod 8 share an L2: give each
 // XCD a contiguous range of tile ids, ordered in column strips of kGroupM
@@ -135,6 +154,8 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     constexpr int kBRowsPerInstr = 64 / kBChunksPerRow > 0 ? 64 / kBChunksPerRow : 1;
     constexpr int kBInstr = kStageB / (kWaves * 1024);
     constexpr int kLoadsPerTile = kAInstr + kBInstr;
+    // the tiles are laid out for the reads of the 16x16x32 MFMA form (see kM16 below)
+    constexpr bool kTile16 = NT_GEMM_M16 && kAblate == 0 && BK % 32 == 0 && sizeof(T) == 2;
     // kTail: N and K need not fit the tile (multiples of 8 elements, so that 16-byte chunks stay whole).
     // Columns of B past N feed only columns of C that are not stored; the k positions past K of the last
     // tile must read as zeros in both operands (a stray Inf times a zero would be a NaN): rows of a
@@ -212,7 +233,7 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     for (int j = 0; j < kAInstr; ++j) {
         const int row = (j * kWaves + wave) * kARowsPerInstr + lane / kAChunksPerRow;
         const int phys = lane % kAChunksPerRow;
-        const int chunk = a_phys_chunk<BK>(row, phys);  // XOR is an involution
+        const int chunk = kTile16 ? a_phys_chunk16<BK>(row, phys) : a_phys_chunk<BK>(row, phys);  // XOR is an involution
         a_src[j] = (unsigned)(row * (int)p.lda + chunk * 8) * 2u;
     }
     unsigned b_src[kBInstr];
@@ -220,12 +241,12 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     for (int j = 0; j < kBInstr; ++j) {
         if constexpr (kBT) {
             const int row = (j * kWaves + wave) * kARowsPerInstr + lane / kAChunksPerRow;
-            const int chunk = a_phys_chunk<BK>(row, lane % kAChunksPerRow);
+            const int chunk = kTile16 ? a_phys_chunk16<BK>(row, lane % kAChunksPerRow) : a_phys_chunk<BK>(row, lane % kAChunksPerRow);
             b_src[j] = (unsigned)(row * (int)p.ldb + chunk * 8) * 2u;
         } else {
             const int krow = (j * kWaves + wave) * kBRowsPerInstr + lane / kBChunksPerRow;
             const int phys = lane % kBChunksPerRow;
-            const int chunk = b_phys_chunk<BN>(krow, phys);
+            const int chunk = kTile16 ? b_phys_chunk16<BN>(krow, phys) : b_phys_chunk<BN>(krow, phys);
             b_src[j] = (unsigned)(krow * (int)p.ldb + chunk * 8) * 2u;
         }
     }
@@ -263,7 +284,7 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
 #pragma unroll
                 for (int j = 0; j < kAInstr; ++j) {
                     const int row = (j * kWaves + wave) * kARowsPerInstr + lane / kAChunksPerRow;
-                    const bool inside = a_phys_chunk<BK>(row, lane % kAChunksPerRow) < tail_chunks;
+                    const bool inside = (kTile16 ? a_phys_chunk16<BK>(row, lane % kAChunksPerRow) : a_phys_chunk<BK>(row, lane % kAChunksPerRow)) < tail_chunks;
                     __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, sa + (j * kWaves + wave) * 1024, 16, inside ? a_src[j] : kBehind, a_k, 0, kAux);
                 }
 #pragma unroll
@@ -271,7 +292,7 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
                     bool inside = true;
                     if constexpr (kBT) {
                         const int row = (j * kWaves + wave) * kARowsPerInstr + lane / kAChunksPerRow;
-                        inside = a_phys_chunk<BK>(row, lane % kAChunksPerRow) < tail_chunks;
+                        inside = (kTile16 ? a_phys_chunk16<BK>(row, lane % kAChunksPerRow) : a_phys_chunk<BK>(row, lane % kAChunksPerRow)) < tail_chunks;
                     }
                     __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, sb + (j * kWaves + wave) * 1024, 16, inside ? b_src[j] : kBehind, b_k, 0, kAux);
                 }
@@ -419,18 +440,18 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         const int bt_row = wave_n * kWaveN + i16;
 #pragma unroll
         for (int ks = 0; ks < KS16; ++ks) {
-            a16_off[ks] = a_row * (BK * 2) + (((ks * 4 + kg) ^ a_phys_chunk<BK>(a_row, 0)) * 16);
-            bt16_off[ks] = bt_row * (BK * 2) + (((ks * 4 + kg) ^ a_phys_chunk<BK>(bt_row, 0)) * 16);
+            a16_off[ks] = a_row * (BK * 2) + (a_phys_chunk16<BK>(a_row, ks * 4 + kg) * 16);
+            bt16_off[ks] = bt_row * (BK * 2) + (a_phys_chunk16<BK>(bt_row, ks * 4 + kg) * 16);
         }
     }
     int b16_lo[kM16 && !kBT ? TN16 : 1], b16_hi[kM16 && !kBT ? TN16 : 1];
     if constexpr (kM16 && !kBT) {
 #pragma unroll
         for (int tj = 0; tj < TN16; ++tj) {
-            const int k_lo = 8 * kg + (i16 >> 2), k_hi = k_lo + 4;  // + 32 * ks: the swizzle only looks at k % 8
+            const int k_lo = 8 * kg + (i16 >> 2), k_hi = k_lo + 4;  // + 32 * ks: the swizzle only looks at k % 16
             const int ncol = wave_n * kWaveN + tj * 16 + 4 * (i16 & 3);
-            b16_lo[tj] = k_lo * (BN * 2) + b_phys_chunk<BN>(k_lo, ncol >> 3) * 16 + (ncol & 7) * 2;
-            b16_hi[tj] = k_hi * (BN * 2) + b_phys_chunk<BN>(k_hi, ncol >> 3) * 16 + (ncol & 7) * 2;
+            b16_lo[tj] = k_lo * (BN * 2) + b_phys_chunk16<BN>(k_lo, ncol >> 3) * 16 + (ncol & 7) * 2;
+            b16_hi[tj] = k_hi * (BN * 2) + b_phys_chunk16<BN>(k_hi, ncol >> 3) * 16 + (ncol & 7) * 2;
         }
     }
     auto read_a16 = [&](auto stage_tag, int ks, int ti) -> vec8 {
