@@ -256,7 +256,10 @@ NineToothedResult launch_nt_gemm_config(NineToothedStream stream, int config,
                                         int dtype, int output_dtype);
 
 /* Times every instance that accepts the problem (hipEvents on `stream`,
- * `iters` launches each after 2 warm-ups; this call synchronises) and stores
+ * `iters` launches each after 2 warm-ups -- more for short kernels, whose timed
+ * region is brought to about 0.75 ms; the first candidate runs untimed for about
+ * 20 ms beforehand, so that it is not measured on a part that is still raising
+ * its clocks; this call synchronises) and stores
  * the winner in the per-device cache that launch_nt_matmul / launch_nt_addmm
  * consult when block sizes are 0.  The instance of the untuned rule is timed
  * first and stays the choice unless another one is more than 2 % faster (the

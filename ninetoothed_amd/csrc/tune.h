@@ -20,7 +20,7 @@ int tune_lookup(int kind, const int *values, int count);
 void tune_record(int kind, const int *values, int count, int choice, const int *extra = nullptr, int extras = 0);
 
 // Times candidates 0 .. candidates - 1 on `stream` with device events: 2 warm-up launches and `iters` timed ones
-// each.  `launch(i)` returns 0, NINETOOTHED_NO_KERNEL (the candidate does not take the problem: skipped) or an
+// each (a candidate whose `iters` launches take less than 0.5 ms is timed again over about 0.75 ms, at most 256 launches).  `launch(i)` returns 0, NINETOOTHED_NO_KERNEL (the candidate does not take the problem: skipped) or an
 // error (returned).  *best receives the fastest candidate (-1 when none ran); with a `margin`, a later candidate
 // replaces an earlier one only when it is faster by more than that fraction (candidates in order of preference).
 // The first candidate is preceded by an untimed warm-up of about 20 ms.
@@ -70,20 +70,25 @@ int tune_time(hipStream_t stream, int candidates, int iters, Launch launch, int 
             result = rc;
             break;
         }
-        (void)hipEventRecord(start, stream);
-        for (int r = 0; r < iters && rc == 0; ++r) rc = launch(i);
-        (void)hipEventRecord(stop, stream);
+        // short kernels are timed over more launches: a timed region of a few microseconds says little
+        float ms = 0.0f;
+        int timed = iters;
+        for (int attempt = 0; attempt < 2 && rc == 0; ++attempt) {
+            (void)hipEventRecord(start, stream);
+            for (int r = 0; r < timed && rc == 0; ++r) rc = launch(i);
+            (void)hipEventRecord(stop, stream);
+            if (rc == 0 && (err = hipEventSynchronize(stop)) != hipSuccess) rc = (int)err;
+            if (rc != 0) break;
+            (void)hipEventElapsedTime(&ms, start, stop);
+            if (ms >= 0.5f || timed >= 256) break;
+            const int wanted = ms > 0.0f ? (int)(0.75f * (float)timed / ms) + 1 : 256;  // about 0.75 ms
+            if (attempt == 0) timed = wanted < 256 ? (wanted > timed ? wanted : timed) : 256;
+        }
         if (rc != 0) {
             result = rc;
             break;
         }
-        if ((err = hipEventSynchronize(stop)) != hipSuccess) {
-            result = (int)err;
-            break;
-        }
-        float ms = 0.0f;
-        (void)hipEventElapsedTime(&ms, start, stop);
-        ms /= (float)iters;
+        ms /= (float)timed;
         if (*best < 0 || ms < *best_ms * (1.0f - margin)) {
             *best = i;
             *best_ms = ms;
