@@ -1,5 +1,5 @@
 // Tiled GEMM for gfx950: C[M,N] = A[M,K] @ B[K,N] (+ addmm epilogue), fp16/bf16
-// inputs, fp32 accumulation on 32x32x16 MFMA.
+// inputs, fp32 accumulation on 16x16x32 MFMAs (32x32x16 in the measurement instances).
 //
 // Fast path requirements (checked on the host before launch):
 //   A row-major with unit K stride, B row-major with unit N stride, C with unit
