@@ -131,6 +131,9 @@ NT_DEVICE void lds_barrier_reads_in_flight() {
 #ifndef NT_GEMM_M16
 #define NT_GEMM_M16 1
 #endif
+#ifndef NT_GEMM_PAIR_A
+#define NT_GEMM_PAIR_A 1
+#endif
 
 // kAblate is a measurement aid (bit 0: no global loads inside the K loop,
 // bit 1: operand fragments read from LDS only once); 0 in every shipped instance.
@@ -156,6 +159,14 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     constexpr int kLoadsPerTile = kAInstr + kBInstr;
     // the tiles are laid out for the reads of the 16x16x32 MFMA form (see kM16 below)
     constexpr bool kTile16 = NT_GEMM_M16 && kAblate == 0 && BK % 32 == 0 && sizeof(T) == 2;
+    // kPairA (the 5 x 32 KiB ring of the large tile): A is staged two k tiles at a time, in three stages of rows of
+    // 128 bytes, B one k tile at a time in four stages.  A fill instruction then asks for whole cache lines of A
+    // (16 half lines otherwise: a k tile of A is 64 bytes per row), which is worth 3 % at 8192^3.  The compute
+    // steps stay one k tile long; a tile of B stays in flight across a barrier, and the pair of A that is
+    // requested in an even step has three steps to arrive.
+    constexpr bool kPairA = NT_GEMM_PAIR_A && kTile16 && BK == 32 && kStages == 5 && kLoad == 1 && !kBT && !kTail && !kSplit &&
+                            (BM / WM / 16) % 4 == 0 && BM / WM >= BN / WN;
+    constexpr int kBytesA = kPairA ? 2 * kStageA : kStageA;
     // kTail: N and K need not fit the tile (multiples of 8 elements, so that 16-byte chunks stay whole).
     // Columns of B past N feed only columns of C that are not stored; the k positions past K of the last
     // tile must read as zeros in both operands (a stray Inf times a zero would be a NaN): rows of a
@@ -175,9 +186,10 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     // One array per stage and operand: distinct LDS objects let the compiler prove
     // that the asynchronous fill of one stage does not alias reads of another,
     // so it does not wait for the fill before the MFMA operand reads.
-    __shared__ __attribute__((aligned(1024))) unsigned char lds_a0[kStageA];
-    __shared__ __attribute__((aligned(1024))) unsigned char lds_a1[kStageA];
-    __shared__ __attribute__((aligned(1024))) unsigned char lds_a2[kStages > 2 ? kStageA : 16];
+    // (kPairA uses a0 .. a2 and b0 .. b3; arrays that nothing refers to take no LDS)
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_a0[kBytesA];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_a1[kBytesA];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_a2[kStages > 2 ? kBytesA : 16];
     __shared__ __attribute__((aligned(1024))) unsigned char lds_a3[kStages > 3 ? kStageA : 16];
     __shared__ __attribute__((aligned(1024))) unsigned char lds_a4[kStages > 4 ? kStageA : 16];
     __shared__ __attribute__((aligned(1024))) unsigned char lds_b0[kStageB];
@@ -248,6 +260,18 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
             const int phys = lane % kBChunksPerRow;
             const int chunk = kTile16 ? b_phys_chunk16<BN>(krow, phys) : b_phys_chunk<BN>(krow, phys);
             b_src[j] = (unsigned)(krow * (int)p.ldb + chunk * 8) * 2u;
+        }
+    }
+
+    // kPairA: instruction j of a wave fills rows [(j * kWaves + wave) * 8, + 8) of a pair stage, 128 bytes each
+    constexpr int kPairInstr = 2 * kAInstr;
+    unsigned a_pair_src[kPairA ? kPairInstr : 1];
+    if constexpr (kPairA) {
+#pragma unroll
+        for (int j = 0; j < kPairInstr; ++j) {
+            const int row = (j * kWaves + wave) * 8 + lane / 8;
+            const int chunk = a_phys_chunk16<64>(row, lane % 8);
+            a_pair_src[j] = (unsigned)(row * (int)p.lda + chunk * 8) * 2u;
         }
     }
 
@@ -469,8 +493,95 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         }
     };
 
-    static_for<0, kStages - 1>([&](auto s) { issue_loads(s, min((int)decltype(s)::value, last_k)); });
-    if constexpr (kCross16) {
+    if constexpr (kPairA) {
+        // Tile t uses B stage t % 4 and half t % 2 of A pair stage (t / 2) % 3.  The barrier that opens step t tells that
+        // tile t + 1 is complete in LDS and that every wave is done with tile t - 1; after it B of tile t + 3 is
+        // requested into the stage of tile t - 1 and, in even steps, A of tiles t + 4, t + 5 into the stage of tiles
+        // t - 2, t - 1.  Stage, half, B set and A slot are compile-time constants over a body of 12 steps.
+        const int last_pair = last_k >> 1;
+        int a16p_off[2];
+        {
+            const int a_row = wave_m * kWaveM + i16;  // + 16 * ti, which leaves the swizzle term as it is
+#pragma unroll
+            for (int h = 0; h < 2; ++h) a16p_off[h] = a_row * 128 + a_phys_chunk16<64>(a_row, 4 * h + kg) * 16;
+        }
+        auto read_a_pair = [&](auto stage_tag, int half, int ti) -> vec8 {
+            return *(const NT_LDS vec8 *)(stage_a(stage_tag) + a16p_off[half] + ti * 16 * 128);
+        };
+        auto issue_a_pair = [&](auto stage_tag, int pair) {
+            NT_LDS unsigned char *sa = stage_a(stage_tag);
+#pragma unroll
+            for (int j = 0; j < kPairInstr; ++j)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, sa + (j * kWaves + wave) * 1024, 16, a_pair_src[j], pair * 128, 0, kAux);
+        };
+        auto issue_b = [&](auto stage_tag, int kt) {
+            NT_LDS unsigned char *sb = stage_b(stage_tag);
+            const int b_k = kt * BK * (int)p.ldb * 2;
+#pragma unroll
+            for (int j = 0; j < kBInstr; ++j)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, sb + (j * kWaves + wave) * 1024, 16, b_src[j], b_k, 0, kAux);
+        };
+        typedef std::integral_constant<int, 0> S0;
+        typedef std::integral_constant<int, 1> S1;
+        typedef std::integral_constant<int, 2> S2;
+        issue_a_pair(S0(), 0);
+        issue_a_pair(S1(), min(1, last_pair));
+        issue_b(S0(), 0);
+        issue_b(S1(), min(1, last_k));
+        issue_b(S2(), min(2, last_k));
+        vec8 as[4];
+        vec8 bs[2][TN16];
+        wait_vmcnt<2 * kBInstr>();
+        lds_barrier();
+#pragma unroll
+        for (int tj = 0; tj < TN16; ++tj) bs[0][tj] = read_b16(S0(), 0, tj);
+        as[0] = read_a_pair(S0(), 0, 0);
+        as[1] = read_a_pair(S0(), 0, 1);
+        auto step = [&](auto i_tag, int kt) {
+            constexpr int kI = decltype(i_tag)::value;  // position in the body of 12 steps
+            typedef std::integral_constant<int, (kI / 2) % 3> PairStage;
+            typedef std::integral_constant<int, ((kI + 1) / 2) % 3> NextPairStage;
+            typedef std::integral_constant<int, (kI + 1) % 4> NextStageB;
+            constexpr int half = kI & 1, next_half = half ^ 1;
+            constexpr int cur = kI & 1, nxt = cur ^ 1;
+            constexpr int kFillsOfStep = (half == 0 ? kPairInstr : 0) + kBInstr;
+            // in flight across the barrier: what the step before requested
+            wait_vmcnt<(half == 1 ? kPairInstr : 0) + kBInstr>();
+            lds_barrier_reads_in_flight();
+            if constexpr (half == 0) issue_a_pair(std::integral_constant<int, (kI / 2 + 2) % 3>(), min((kt + kI) / 2 + 2, last_pair));
+            issue_b(std::integral_constant<int, (kI + 3) % 4>(), min(kt + kI + 3, last_k));
+            static_for<0, TM16>([&](auto q_tag) {
+                constexpr int q = decltype(q_tag)::value;
+                constexpr bool kReadsB = q >= TM16 - TN16;
+                if constexpr (q + 2 < TM16) as[(q + 2) % 4] = read_a_pair(PairStage(), half, q + 2);
+                else as[(q + 2) % 4] = read_a_pair(NextPairStage(), next_half, q + 2 - TM16);
+                if constexpr (kReadsB) bs[nxt][q - (TM16 - TN16)] = read_b16(NextStageB(), 0, q - (TM16 - TN16));
+#pragma unroll
+                for (int tj = 0; tj < TN16; ++tj) acc16[q][tj] = E::mfma16(bs[cur][tj], as[q % 4], acc16[q][tj]);  // transposed block
+#if NT_GEMM_SCHEDULE
+                constexpr int kReads = 1 + (kReadsB ? 2 : 0);
+                static_for<0, TN16>([&](auto j_tag) {
+                    constexpr int j = decltype(j_tag)::value;
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    if constexpr (j < kReads) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    if constexpr (j == 1 && q < kFillsOfStep) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                });
+#endif
+            });
+        };
+        constexpr int kBody = 12;
+        const int body_k = num_k - num_k % kBody;
+        for (int kt = 0; kt < body_k; kt += kBody) {
+            static_for<0, kBody>([&](auto i) { step(i, kt); });
+        }
+        static_for<0, kBody - 1>([&](auto i) {
+            if (body_k + (int)decltype(i)::value < num_k) step(i, body_k);
+        });
+    }
+    if constexpr (!kPairA) static_for<0, kStages - 1>([&](auto s) { issue_loads(s, min((int)decltype(s)::value, last_k)); });
+    if constexpr (kPairA) {
+        // (done above)
+    } else if constexpr (kCross16) {
         // All TN16 B fragments of a k step stay in registers (two sets, taking turns k step by k step); the
         // A fragments stream through four slots, each read two blocks ahead of its MFMAs.
         constexpr int Q = KS16 * TM16;  // A fragments of a k tile, in the order they are used

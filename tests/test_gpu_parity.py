@@ -1058,6 +1058,48 @@ def test_gemm_any_number_of_rows_on_the_direct_to_lds_path(m, addmm):
 
 
 @pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
+def test_gemm_large_tile_every_k_tile_count(dtype):
+    """The 256x256x32 instance stages its lhs two k tiles at a time in a ring of three, its rhs one at a time in a
+    ring of four, over a loop body of twelve steps: every number of k tiles from 1 to 27 (all residues of the body,
+    odd counts leave half a pair unused), a partial tile of rows, through the C ABI by instance.  The lhs is a view
+    into a wider matrix whose other columns hold Inf: reading past the k range of a row would show."""
+    import ctypes
+
+    from ninetoothed_amd import runtime
+
+    lib = runtime.library()
+    tag = runtime.DATA_TYPE_INDEX["fp16" if dtype == torch.float16 else "bf16"]
+    buffer = ctypes.create_string_buffer(128)
+    instance = None
+    for index in range(lib.nt_gemm_num_configs()):
+        runtime.check(lib.nt_gemm_config_name(index, buffer, len(buffer)))
+        if buffer.value.decode().startswith("256x256x32 waves 2x4 stages 5") and "tails" not in buffer.value.decode():
+            instance = index
+            break
+    assert instance is not None
+    null = runtime.ArgumentTensor.null()
+    m, n = 300, 512
+    for tiles in list(range(1, 28)) + [61]:
+        k = 32 * tiles
+        wide = torch.full((m, k + 64), float("inf"), dtype=dtype, device="cuda")
+        wide[:, :k] = _randn(m, k, dtype=dtype).cuda()
+        a = wide[:, :k]
+        b = _randn(k, n, dtype=dtype).cuda()
+        bias = _randn(m, n, dtype=dtype).cuda()
+        out = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+        code = lib.launch_nt_gemm_config(
+            runtime.current_stream(), instance, runtime.ArgumentTensor.from_torch_tensor(bias), runtime.ArgumentTensor.from_torch_tensor(a),
+            runtime.ArgumentTensor.from_torch_tensor(b), runtime.ArgumentTensor.from_scalar(0.5), runtime.ArgumentTensor.from_scalar(2.0),
+            runtime.ArgumentTensor.from_torch_tensor(out), tag, tag,
+        )
+        assert code == 0, (tiles, code)
+        product = (a.float() @ b.float()).to(dtype).float()
+        expected = 0.5 * bias.float() + 2.0 * product
+        tolerance = dict(rtol=2e-2, atol=2e-2) if dtype == torch.float16 else dict(rtol=5e-2, atol=2e-1)
+        assert torch.allclose(out.float(), expected, **tolerance), (tiles, float((out.float() - expected).abs().max()))
+
+
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
 @pytest.mark.parametrize("m, n, k", ((300, 200, 104), (1000, 1000, 1000), (257, 264, 72), (512, 520, 8), (2100, 3000, 2056)))
 def test_gemm_partial_tiles_along_n_and_k(m, n, k, dtype):
     """N and K that do not fit the tile (multiples of 8) stay on the direct-to-LDS kernels: the
