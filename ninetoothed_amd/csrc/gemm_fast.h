@@ -164,7 +164,7 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     // (16 half lines otherwise: a k tile of A is 64 bytes per row), which is worth 3 % at 8192^3.  The compute
     // steps stay one k tile long; a tile of B stays in flight across a barrier, and the pair of A that is
     // requested in an even step has three steps to arrive.
-    constexpr bool kPairA = NT_GEMM_PAIR_A && kTile16 && BK == 32 && kStages == 5 && kLoad == 1 && !kBT && !kTail && !kSplit &&
+    constexpr bool kPairA = NT_GEMM_PAIR_A && kTile16 && BK == 32 && kStages == 5 && kLoad == 1 && !kTail && !kSplit &&
                             (BM / WM / 16) % 4 == 0 && BM / WM >= BN / WN;
     constexpr int kBytesA = kPairA ? 2 * kStageA : kStageA;
     // kTail: N and K need not fit the tile (multiples of 8 elements, so that 16-byte chunks stay whole).
@@ -516,7 +516,7 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         };
         auto issue_b = [&](auto stage_tag, int kt) {
             NT_LDS unsigned char *sb = stage_b(stage_tag);
-            const int b_k = kt * BK * (int)p.ldb * 2;
+            const int b_k = kBT ? kt * BK * 2 : kt * BK * (int)p.ldb * 2;
 #pragma unroll
             for (int j = 0; j < kBInstr; ++j)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, sb + (j * kWaves + wave) * 1024, 16, b_src[j], b_k, 0, kAux);
@@ -559,7 +559,7 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
 #pragma unroll
                 for (int tj = 0; tj < TN16; ++tj) acc16[q][tj] = E::mfma16(bs[cur][tj], as[q % 4], acc16[q][tj]);  // transposed block
 #if NT_GEMM_SCHEDULE
-                constexpr int kReads = 1 + (kReadsB ? 2 : 0);
+                constexpr int kReads = 1 + (kReadsB ? (kBT ? 1 : 2) : 0);
                 static_for<0, TN16>([&](auto j_tag) {
                     constexpr int j = decltype(j_tag)::value;
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
