@@ -164,7 +164,7 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     // (16 half lines otherwise: a k tile of A is 64 bytes per row), which is worth 3 % at 8192^3.  The compute
     // steps stay one k tile long; a tile of B stays in flight across a barrier, and the pair of A that is
     // requested in an even step has three steps to arrive.
-    constexpr bool kPairA = NT_GEMM_PAIR_A && kTile16 && BK == 32 && kStages == 5 && kLoad == 1 && !kTail && !kSplit &&
+    constexpr bool kPairA = NT_GEMM_PAIR_A && kTile16 && BK == 32 && kStages == 5 && kLoad == 1 && !kSplit &&
                             (BM / WM / 16) % 4 == 0 && BM / WM >= BN / WN;
     constexpr int kBytesA = kPairA ? 2 * kStageA : kStageA;
     // kTail: N and K need not fit the tile (multiples of 8 elements, so that 16-byte chunks stay whole).
@@ -508,8 +508,20 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         auto read_a_pair = [&](auto stage_tag, int half, int ti) -> vec8 {
             return *(const NT_LDS vec8 *)(stage_a(stage_tag) + a16p_off[half] + ti * 16 * 128);
         };
+        // (kTail: 16-byte chunks of the last pair that lie inside K; the others must read as zeros, see kTail above)
+        const int pair_chunks = kTail ? min(8, (p.k - last_pair * 64) / 8) : 8;
         auto issue_a_pair = [&](auto stage_tag, int pair) {
             NT_LDS unsigned char *sa = stage_a(stage_tag);
+            if (kTail && pair == last_pair && pair_chunks < 8) {  // uniform
+                constexpr unsigned kBehind = 0x7fffffffu;  // behind every descriptor (their sizes stay below 2^31)
+#pragma unroll
+                for (int j = 0; j < kPairInstr; ++j) {
+                    const int row = (j * kWaves + wave) * 8 + lane / 8;
+                    const bool inside = a_phys_chunk16<64>(row, lane % 8) < pair_chunks;
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, sa + (j * kWaves + wave) * 1024, 16, inside ? a_pair_src[j] : kBehind, pair * 128, 0, kAux);
+                }
+                return;
+            }
 #pragma unroll
             for (int j = 0; j < kPairInstr; ++j)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, sa + (j * kWaves + wave) * 1024, 16, a_pair_src[j], pair * 128, 0, kAux);
@@ -517,6 +529,16 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         auto issue_b = [&](auto stage_tag, int kt) {
             NT_LDS unsigned char *sb = stage_b(stage_tag);
             const int b_k = kBT ? kt * BK * 2 : kt * BK * (int)p.ldb * 2;
+            if (kTail && kBT && kt == last_k && tail_chunks < kAChunksPerRow) {  // uniform: the partial last k tile of a k-contiguous rhs
+                constexpr unsigned kBehind = 0x7fffffffu;
+#pragma unroll
+                for (int j = 0; j < kBInstr; ++j) {
+                    const int row = (j * kWaves + wave) * kARowsPerInstr + lane / kAChunksPerRow;
+                    const bool inside = a_phys_chunk16<BK>(row, lane % kAChunksPerRow) < tail_chunks;
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, sb + (j * kWaves + wave) * 1024, 16, inside ? b_src[j] : kBehind, b_k, 0, kAux);
+                }
+                return;
+            }
 #pragma unroll
             for (int j = 0; j < kBInstr; ++j)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, sb + (j * kWaves + wave) * 1024, 16, b_src[j], b_k, 0, kAux);
