@@ -162,8 +162,8 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     // kPairA (the 5 x 32 KiB ring of the large tile): A is staged two k tiles at a time, in three stages of rows of
     // 128 bytes, B one k tile at a time in four stages.  A fill instruction then asks for whole cache lines of A
     // (16 half lines otherwise: a k tile of A is 64 bytes per row), which is worth 3 % at 8192^3.  The compute
-    // steps stay one k tile long; a tile of B stays in flight across a barrier, and the pair of A that is
-    // requested in an even step has three steps to arrive.
+    // steps stay one k tile long; a tile of B and half a pair of A stay in flight across a barrier (the pair whose
+    // stage becomes free in an even step is requested half in that step and half in the next).
     constexpr bool kPairA = NT_GEMM_PAIR_A && kTile16 && BK == 32 && kStages == 5 && kLoad == 1 && !kSplit &&
                             (BM / WM / 16) % 4 == 0 && BM / WM >= BN / WN;
     constexpr int kBytesA = kPairA ? 2 * kStageA : kStageA;
@@ -496,8 +496,8 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
     if constexpr (kPairA) {
         // Tile t uses B stage t % 4 and half t % 2 of A pair stage (t / 2) % 3.  The barrier that opens step t tells that
         // tile t + 1 is complete in LDS and that every wave is done with tile t - 1; after it B of tile t + 3 is
-        // requested into the stage of tile t - 1 and, in even steps, A of tiles t + 4, t + 5 into the stage of tiles
-        // t - 2, t - 1.  Stage, half, B set and A slot are compile-time constants over a body of 12 steps.
+        // requested into the stage of tile t - 1 and A of tiles t + 4, t + 5 (t even; half of it in step t, half in
+        // step t + 1) into the stage of tiles t - 2, t - 1.  Stage, half, B set and A slot are compile-time constants over a body of 12 steps.
         const int last_pair = last_k >> 1;
         int a16p_off[2];
         {
@@ -510,12 +510,13 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         };
         // (kTail: 16-byte chunks of the last pair that lie inside K; the others must read as zeros, see kTail above)
         const int pair_chunks = kTail ? min(8, (p.k - last_pair * 64) / 8) : 8;
-        auto issue_a_pair = [&](auto stage_tag, int pair) {
+        auto issue_a_pair = [&](auto stage_tag, int pair, auto first_tag, auto last_tag) {
+            constexpr int kFirst = decltype(first_tag)::value, kLast = decltype(last_tag)::value;  // instructions [kFirst, kLast) of the pair
             NT_LDS unsigned char *sa = stage_a(stage_tag);
             if (kTail && pair == last_pair && pair_chunks < 8) {  // uniform
                 constexpr unsigned kBehind = 0x7fffffffu;  // behind every descriptor (their sizes stay below 2^31)
 #pragma unroll
-                for (int j = 0; j < kPairInstr; ++j) {
+                for (int j = kFirst; j < kLast; ++j) {
                     const int row = (j * kWaves + wave) * 8 + lane / 8;
                     const bool inside = a_phys_chunk16<64>(row, lane % 8) < pair_chunks;
                     __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, sa + (j * kWaves + wave) * 1024, 16, inside ? a_pair_src[j] : kBehind, pair * 128, 0, kAux);
@@ -523,9 +524,12 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
                 return;
             }
 #pragma unroll
-            for (int j = 0; j < kPairInstr; ++j)
+            for (int j = kFirst; j < kLast; ++j)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, sa + (j * kWaves + wave) * 1024, 16, a_pair_src[j], pair * 128, 0, kAux);
         };
+        typedef std::integral_constant<int, 0> I0;
+        typedef std::integral_constant<int, kPairInstr / 2> IHalf;
+        typedef std::integral_constant<int, kPairInstr> IAll;
         auto issue_b = [&](auto stage_tag, int kt) {
             NT_LDS unsigned char *sb = stage_b(stage_tag);
             const int b_k = kBT ? kt * BK * 2 : kt * BK * (int)p.ldb * 2;
@@ -546,14 +550,16 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         typedef std::integral_constant<int, 0> S0;
         typedef std::integral_constant<int, 1> S1;
         typedef std::integral_constant<int, 2> S2;
-        issue_a_pair(S0(), 0);
-        issue_a_pair(S1(), min(1, last_pair));
+        // (in the order of the steps: the last requests before step 0 are half a pair and a tile of B, as after any step)
+        issue_a_pair(S0(), 0, I0(), IAll());
+        issue_a_pair(S1(), min(1, last_pair), I0(), IHalf());
         issue_b(S0(), 0);
         issue_b(S1(), min(1, last_k));
+        issue_a_pair(S1(), min(1, last_pair), IHalf(), IAll());
         issue_b(S2(), min(2, last_k));
         vec8 as[4];
         vec8 bs[2][TN16];
-        wait_vmcnt<2 * kBInstr>();
+        wait_vmcnt<2 * kBInstr + kPairInstr / 2>();
         lds_barrier();
 #pragma unroll
         for (int tj = 0; tj < TN16; ++tj) bs[0][tj] = read_b16(S0(), 0, tj);
@@ -566,11 +572,12 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
             typedef std::integral_constant<int, (kI + 1) % 4> NextStageB;
             constexpr int half = kI & 1, next_half = half ^ 1;
             constexpr int cur = kI & 1, nxt = cur ^ 1;
-            constexpr int kFillsOfStep = (half == 0 ? kPairInstr : 0) + kBInstr;
-            // in flight across the barrier: what the step before requested
-            wait_vmcnt<(half == 1 ? kPairInstr : 0) + kBInstr>();
+            // the pair that becomes free in an even step is requested half in that step, half in the next one
+            constexpr int kFillsOfStep = kPairInstr / 2 + kBInstr;
+            wait_vmcnt<kPairInstr / 2 + kBInstr>();  // in flight across the barrier: what the step before requested
             lds_barrier_reads_in_flight();
-            if constexpr (half == 0) issue_a_pair(std::integral_constant<int, (kI / 2 + 2) % 3>(), min((kt + kI) / 2 + 2, last_pair));
+            if constexpr (half == 0) issue_a_pair(std::integral_constant<int, (kI / 2 + 2) % 3>(), min((kt + kI) / 2 + 2, last_pair), I0(), IHalf());
+            else issue_a_pair(std::integral_constant<int, (kI / 2 + 2) % 3>(), min((kt + kI) / 2 + 2, last_pair), IHalf(), IAll());
             issue_b(std::integral_constant<int, (kI + 3) % 4>(), min(kt + kI + 3, last_k));
             static_for<0, TM16>([&](auto q_tag) {
                 constexpr int q = decltype(q_tag)::value;
