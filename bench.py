@@ -157,7 +157,7 @@ def build_workloads(inputs="randn"):
             sink = torch.zeros(1, device="cuda")
             loops = 4096
             count = ctypes.c_int64(0)
-            lib = runtime.library()
+            lib = load_probe_library()
             probe = lib.nt_probe_mfma_rate if form == "32x32x16" else lib.nt_probe_mfma_rate_16x16x32
             flop_per_mfma = 2 * 32 * 32 * 16 if form == "32x32x16" else 2 * 16 * 16 * 32
 
@@ -186,6 +186,34 @@ def build_workloads(inputs="randn"):
     workloads["map_add"] = map_add
     workloads["copy_1gib"] = copy_1gib
     return workloads
+
+
+def load_probe_library():
+    """``libnt_probe.so``: the MFMA issue-rate kernels (measurement aids, built beside the product library and
+    loaded by nothing else)."""
+    import ctypes
+
+    from ninetoothed_amd import runtime
+    from ninetoothed_amd.build_library import PROBE_LIBRARY_PATH
+
+    if not PROBE_LIBRARY_PATH.exists():
+        raise RuntimeError(f"{PROBE_LIBRARY_PATH} is missing: build it with `python -m ninetoothed_amd.build_library`")
+    lib = ctypes.CDLL(str(PROBE_LIBRARY_PATH))
+    for name in ("nt_probe_mfma_rate", "nt_probe_mfma_rate_16x16x32"):
+        function = getattr(lib, name)
+        function.argtypes = [ctypes.c_void_p, runtime.ArgumentTensor, runtime.ArgumentTensor, ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64)]
+        function.restype = ctypes.c_int
+    return lib
+
+
+def launch_description(workload):
+    """The prepared launch of the workload's latest call plus the kernel variant the library ran for it."""
+    from ninetoothed_amd import runtime
+
+    plan = workload["kernel"].last_plan
+    if not str(plan).startswith("launch_nt_"):
+        return plan
+    return f"{plan}; {runtime.last_launch()}"
 
 
 def measure(workload, steps, warmup, which="step"):
@@ -353,7 +381,7 @@ def main():
     main_workload = workloads[args.workload]()
     device_ms, wall_ms = measure(main_workload, args.steps, args.warmup)
     main_roofline = roofline(main_workload, device_ms, traffic.get(args.workload))
-    launch_plan = main_workload["kernel"].last_plan
+    launch_plan = launch_description(main_workload)
     single = per_launch(main_workload)
     vendor = {}
 
@@ -381,7 +409,7 @@ def main():
             ms, _ = measure(workload, max(5, args.steps // 2), args.warmup)
             entry = roofline(workload, ms, traffic.get(name))
             entry["ms_per_step"] = ms
-            entry["config"] = workload["describe"]
+            entry["config"] = dict(workload["describe"], launch=launch_description(workload))
             others[name] = entry
             vendor_line(name, workload, max(5, args.steps // 2))
             del workload

@@ -179,8 +179,10 @@ NineToothedResult launch_nt_attention(NineToothedStream stream,
  * dilation 1 and zero padding (padding_h, padding_w), computed as the implicit
  * GEMM [N*P*Q, C*R*S] x [C*R*S, K] the arrangement of
  * tests/test_conv2d.py:13-48 describes.
- * Ways to run it, tried in this order unless block_size_m names one (3, 2, 1)
+ * Ways to run it, tried in this order unless block_size_m names one (4, 3, 2, 1)
  * or nt_tune_conv2d has recorded one for the problem:
+ * 4 -- 1 x 1 filters without padding (P*Q and C multiples of 8): one batched
+ *   launch of the GEMM kernels on the tensors as they lie, without scratch;
  * 3 -- one launch on the tensors as they lie, no scratch memory: the filter is
  *   the row-major left operand, rows of the right operand are (channel, filter
  *   tap)-shifted pixel runs of the NCHW input; needs an output width that is a
@@ -194,9 +196,7 @@ NineToothedResult launch_nt_attention(NineToothedStream stream,
  * 1 -- the scratch-free gather kernel, which serves every shape, and calls whose
  *   scratch cannot be allocated (out of memory; a stream under graph capture that
  *   has no buffer yet).
- * FLOAT32 tensors run on way 1 with the fp32 MFMA.
- * 1 x 1 filters without padding (P*Q and C multiples of 8) run as one batched
- * launch of the GEMM kernels on the tensors as they lie, without scratch. */
+ * FLOAT32 tensors run on way 1 with the fp32 MFMA. */
 NineToothedResult launch_nt_conv2d(NineToothedStream stream,
                                    NineToothedTensor input,
                                    NineToothedTensor filter,
@@ -215,7 +215,9 @@ NineToothedResult launch_nt_conv2d(NineToothedStream stream,
  * floats): not into a workspace that the library allocates, but into a fixed array of
  * NINETOOTHED_STATIC_SCRATCH_BYTES (16 MiB) that is part of the library's code object -- every GPU the
  * library runs on holds its copy until the process ends.  This function never calls hipMalloc / hipFree
- * or any allocating routine.  A call whose partial products exceed the array returns
+ * or any allocating routine.  When the partial products of the split that launch_nt_matmul would use
+ * exceed the array, the K range is cut into as many parts as fit (same kernels, another summation order);
+ * a call for which not even two parts fit (M x N x 8 bytes > the array) returns
  * NINETOOTHED_SCRATCH_LIMIT and launches nothing (it does not fall back to another kernel); problems
  * that run in one pass need no scratch memory and are accepted at any size.
  *
@@ -255,17 +257,20 @@ NineToothedResult launch_nt_gemm_config(NineToothedStream stream, int config,
                                         NineToothedTensor output,
                                         int dtype, int output_dtype);
 
-/* Times every instance that accepts the problem (hipEvents on `stream`,
- * `iters` launches each after 2 warm-ups -- more for short kernels, whose timed
- * region is brought to about 0.75 ms; the first candidate runs untimed for about
- * 20 ms beforehand, so that it is not measured on a part that is still raising
- * its clocks; this call synchronises) and stores
+/* Times every instance that accepts the problem with hipEvents on `stream` and stores
  * the winner in the per-device cache that launch_nt_matmul / launch_nt_addmm
- * consult when block sizes are 0.  The instance of the untuned rule is timed
- * first and stays the choice unless another one is more than 2 % faster (the
- * timings scatter by about that much).  Returns 0 and the winner in *best_config,
- * its average time in *best_ms.  On a stream that is being captured into a
- * graph nothing is timed or recorded: returns 0 with *best_config = -1. */
+ * consult when block sizes are 0.  How: the instance of the untuned rule first
+ * runs untimed for about 20 ms (so that nothing is measured on a part that is
+ * still raising its clocks); each instance's launch time is estimated over
+ * `iters` launches; then the instances take turns over five rounds (three or one
+ * when a round takes longer than 0.1 / 0.4 s), each timed over a region of about
+ * 3 ms per round, and an instance's figure is the minimum of its rounds -- a
+ * clock dip has to hit the same instance in every round to change the choice.
+ * The instance of the untuned rule stays the choice unless another one is more
+ * than 2 % faster.  This call synchronises.  Returns 0 and the winner in
+ * *best_config, its time per launch in *best_ms.  On a stream that is being
+ * captured into a graph nothing is timed or recorded: returns 0 with
+ * *best_config = -1. */
 NineToothedResult nt_tune_gemm(NineToothedStream stream,
                                NineToothedTensor input,
                                NineToothedTensor mat1,
@@ -276,23 +281,25 @@ NineToothedResult nt_tune_gemm(NineToothedStream stream,
                                int dtype, int output_dtype, int iters,
                                int *best_config, float *best_ms);
 
-/* As nt_tune_gemm for launch_nt_attention: times its loop variants (plain 64-key blocks; 256 query rows per
- * workgroup; 32-key blocks; software-pipelined; software-pipelined with eight waves) on the given tensors and
- * records the fastest for later launches of the same problem (element type, batch, heads, both sequence
- * lengths, head dimension, causal flag) without block-size hints.  *best_variant = -1 when nothing was timed (a
- * stream that is being captured into a graph), -2 when the problem has no alternatives (FLOAT32 tensors, head
- * dimensions other than 64 and 128, shapes whose key range is split). */
+/* As nt_tune_gemm for launch_nt_attention: times its loop variants (0 plain 64-key blocks; 1 256 query rows per
+ * workgroup; 2 32-key blocks; 3 software-pipelined; 4 software-pipelined with eight waves) on the given tensors the
+ * same way and records the fastest for later launches of the same problem (element type, batch, heads, both
+ * sequence lengths, head dimension, causal flag) without block-size hints; the variant of the untuned rule stays
+ * unless another one is more than 2 % faster.  *best_variant = -1 when nothing was timed (a stream that is being
+ * captured into a graph), -2 when the problem has no alternatives (FLOAT32 tensors, head dimensions other than 64
+ * and 128, shapes whose key range is split). */
 NineToothedResult nt_tune_attention(NineToothedStream stream,
                                     NineToothedTensor q, NineToothedTensor k, NineToothedTensor v,
                                     NineToothedTensor is_causal, NineToothedTensor scale,
                                     NineToothedTensor o,
                                     int dtype, int iters, int *best_variant, float *best_ms);
 
-/* As nt_tune_gemm for launch_nt_conv2d: times the ways to run the convolution -- 3 = one launch on the tensors as
- * they lie, 2 = repacking pass plus GEMM loop, 1 = gather kernel; a way that does not take the problem is skipped
- * -- and records the fastest (the block_size_m value that selects it) for later launches of the same problem with
- * block_size_m = 0; a way that needs scratch memory or more launches replaces one before it in that order only
- * when it is more than 3 % faster.  *best_path = -1 when nothing was timed (graph capture). */
+/* As nt_tune_gemm for launch_nt_conv2d: times the ways to run the convolution -- 4 = a 1 x 1 filter as a batch of
+ * plain products, 3 = one launch on the tensors as they lie, 2 = repacking pass plus GEMM loop, 1 = gather kernel; a
+ * way that does not take the problem is skipped -- and records the fastest (the block_size_m value that selects
+ * it) for later launches of the same problem with block_size_m = 0; a way that needs scratch memory or more
+ * launches replaces one before it in that order only when it is more than 3 % faster.  *best_path = -1 when
+ * nothing was timed (graph capture). */
 NineToothedResult nt_tune_conv2d(NineToothedStream stream,
                                  NineToothedTensor input, NineToothedTensor filter, NineToothedTensor output,
                                  int dtype, int padding_h, int padding_w, int iters,
@@ -319,20 +326,12 @@ int nt_tune_cache_lookup(int dtype, int output_dtype, int m, int n, int k, int a
  * integers of its problem line (without the program), or -1. */
 int nt_tune_lookup(int kind, const int *values, int count);
 
-/* Measurement aid (no counterpart in the reference): one workgroup of eight waves per compute unit issues
- * `loops` x 8 MFMAs (32x32x16 fp16) per wave on operand fragments read once from the FLOAT16 tensors `a` and
- * `b` (dense row-major matrices of at least 4096 elements) -- no LDS, no memory traffic inside the loop.  The rate bounds what a GEMM or attention kernel can reach on
- * the same operand values (random values draw more power in the matrix pipe than constants, and the clock
- * follows).  `sink` is a device float the kernel may write; *mfma_count receives the MFMAs issued in total
- * (2 x 32 x 32 x 16 = 32768 FLOP each).  Asynchronous on `stream`. */
-NineToothedResult nt_probe_mfma_rate(NineToothedStream stream, NineToothedTensor a, NineToothedTensor b,
-                                     int loops, float *sink, int64_t *mfma_count);
-
-/* The same with the 16x16x32 form of the instruction, which the fast GEMM kernel uses: `loops` x 32 MFMAs per
- * wave, 2 x 16 x 16 x 32 = 16384 FLOP each.  Same FLOP per clock; on random operands the part sustains a
- * higher clock with it (per FLOP half as many accumulator values move through the register file). */
-NineToothedResult nt_probe_mfma_rate_16x16x32(NineToothedStream stream, NineToothedTensor a, NineToothedTensor b,
-                                              int loops, float *sink, int64_t *mfma_count);
+/* Writes which kernel served the calling host thread's latest launch_nt_* call into `buffer` (at most `size`
+ * bytes, NUL terminated): the program's kind, the index of the GEMM instance / attention variant / conv2d path /
+ * softmax kernel, and a description, e.g. "attention variant 3: software-pipelined loop, 64-key blocks, four waves
+ * (128 query rows), two workgroups per CU"; "none" before the first launch.  The counterpart of reading the
+ * winning configuration off a Triton autotuner (`best_config`), which the reference's generated kernels allow. */
+NineToothedResult nt_last_launch(char *buffer, int size);
 
 /*
  * Element-wise / reducing tile programs that are none of the programs above.

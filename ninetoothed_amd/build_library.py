@@ -1,4 +1,5 @@
-"""Builds ``libnt_hip.so`` (the gfx950 kernels behind the C ABI) in-tree with hipcc.
+"""Builds ``libnt_hip.so`` (the gfx950 kernels behind the C ABI) and ``libnt_probe.so`` (measurement kernels
+that only bench.py loads) in-tree with hipcc.
 
 Usage: ``python -m ninetoothed_amd.build_library`` or ``build_library()``.  The library
 is written to ``ninetoothed_amd/lib/libnt_hip.so``; object files go to
@@ -15,7 +16,12 @@ PACKAGE_DIR = pathlib.Path(__file__).resolve().parent
 CSRC_DIR = PACKAGE_DIR / "csrc"
 LIBRARY_PATH = PACKAGE_DIR / "lib" / "libnt_hip.so"
 
-SOURCES = ("gemm_api.hip", "conv2d.hip", "softmax.hip", "attention.hip", "map.hip", "workspace.hip", "tune.hip", "probe.hip")
+SOURCES = ("gemm_api.hip", "conv2d.hip", "softmax.hip", "attention.hip", "map.hip", "workspace.hip", "tune.hip")
+
+# Measurement aids (MFMA issue-rate kernels that bench.py times next to the programs) are no part of the C ABI:
+# they are built into a library of their own that only bench.py loads.
+PROBE_LIBRARY_PATH = PACKAGE_DIR / "lib" / "libnt_probe.so"
+PROBE_SOURCES = ("probe.hip",)
 
 OFFLOAD_ARCH = "gfx950"
 
@@ -65,15 +71,19 @@ def build_library(verbose=False, extra_flags=()):
         _run(command)
         return obj
 
-    with concurrent.futures.ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
-        objects = list(pool.map(compile_one, SOURCES))
+    def link(objects, path):
+        temporary = path.with_suffix(".so.tmp")
+        command = [hipcc, f"--offload-arch={OFFLOAD_ARCH}", "-shared", "-fPIC", *map(str, objects), "-o", str(temporary)]
+        if verbose:
+            print(" ".join(command), flush=True)
+        _run(command)
+        temporary.replace(path)
 
-    temporary = LIBRARY_PATH.with_suffix(".so.tmp")
-    command = [hipcc, f"--offload-arch={OFFLOAD_ARCH}", "-shared", "-fPIC", *map(str, objects), "-o", str(temporary)]
-    if verbose:
-        print(" ".join(command), flush=True)
-    _run(command)
-    temporary.replace(LIBRARY_PATH)
+    with concurrent.futures.ThreadPoolExecutor(max_workers=4) as pool:
+        objects = list(pool.map(compile_one, SOURCES + PROBE_SOURCES))
+
+    link(objects[: len(SOURCES)], LIBRARY_PATH)
+    link(objects[len(SOURCES) :], PROBE_LIBRARY_PATH)
     return LIBRARY_PATH
 
 

@@ -794,16 +794,25 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(AttentionParams p)
 }
 
 // Few (batch, head, query block) workgroups and a long key sequence (decoding): the key range is split
-// so that about 512 workgroups run; returns NINETOOTHED_NO_KERNEL when that does not apply.
+// so that about 512 workgroups run.  The number of parts for a problem, 0 when it runs in one pass.
+constexpr int kSplitKeysBM = kAttnWaves * 32, kSplitKeysBN = 64;
+inline int64_t split_key_parts(const AttentionParams &p) {
+    const int64_t groups = (int64_t)p.batch * p.heads * ceil_div(p.seq_q, kSplitKeysBM);
+    const int key_blocks = ceil_div(p.seq_k, kSplitKeysBN);
+    if (groups == 0 || groups >= 128 || key_blocks < 8) return 0;
+    const int64_t parts = std::min<int64_t>((512 + groups - 1) / groups, key_blocks / 4);  // at least four key blocks each
+    return parts < 2 ? 0 : parts;
+}
+
+// returns NINETOOTHED_NO_KERNEL when the problem is not split
 template <typename T, int D>
 int launch_split_keys(AttentionParams &p, hipStream_t stream) {
-    constexpr int BM = kAttnWaves * 32, BN = 64;
+    constexpr int BM = kSplitKeysBM, BN = kSplitKeysBN;
     p.q_blocks = ceil_div(p.seq_q, BM);
     const int64_t groups = (int64_t)p.batch * p.heads * p.q_blocks;
     const int key_blocks = ceil_div(p.seq_k, BN);
-    if (groups == 0 || groups >= 128 || key_blocks < 8) return NINETOOTHED_NO_KERNEL;
-    const int64_t parts = std::min<int64_t>((512 + groups - 1) / groups, key_blocks / 4);  // at least four key blocks each
-    if (parts < 2) return NINETOOTHED_NO_KERNEL;
+    const int64_t parts = split_key_parts(p);
+    if (parts == 0) return NINETOOTHED_NO_KERNEL;
     p.blocks_per_part = ceil_div(key_blocks, (int)parts);
     p.parts = ceil_div(key_blocks, p.blocks_per_part);
     const int64_t rows = (int64_t)p.batch * p.heads * p.seq_q;
@@ -814,6 +823,7 @@ int launch_split_keys(AttentionParams &p, hipStream_t stream) {
     if (scratch == nullptr) return NINETOOTHED_NO_KERNEL;  // (graph capture without a buffer, out of memory): one pass
     p.part_o = scratch;
     p.part_lse = scratch + (size_t)p.parts * rows * D;
+    note_launch(kLaunchAttention, (int)p.parts, "split key range (this many parts), plain loop, then attention_merge_kernel");
     attention_fwd_kernel<T, D, 1, BN, 2, false, T, kAttnWaves, false, true><<<dim3((unsigned)(groups * p.parts)), dim3(kAttnWaves * 64), 0, stream>>>(p);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return (int)err;
@@ -981,6 +991,7 @@ int launch_attention_f32(AttentionParams &p, hipStream_t stream) {
     const int64_t grid = (int64_t)p.batch * p.heads * p.q_blocks;
     if (grid == 0) return 0;
     if (grid > 0x7fffffffll) return NINETOOTHED_NO_KERNEL;
+    note_launch(kLaunchAttention, 0, "attention_f32_kernel, fp32 MFMA throughout");
     attention_f32_kernel<D><<<dim3((unsigned)grid), dim3(256), 0, stream>>>(p);
     return (int)hipGetLastError();
 }
@@ -1021,8 +1032,20 @@ int attention_float32(AttentionParams p, int head_dim, const NineToothedTensor &
 //          2 = 128 query rows per workgroup, 32-key blocks, three workgroups per CU
 //          3 = variant 0 with the software-pipelined main loop
 //          4 = variant 3 with eight waves (256 query rows) per workgroup, one workgroup per CU
+constexpr int kAttentionVariants = 5;
+const char *const kAttentionVariantNames[kAttentionVariants] = {
+    "plain loop, 64-key blocks, four waves (128 query rows), two workgroups per CU",
+    "plain loop, 64-key blocks, 256 query rows per four-wave workgroup, one workgroup per CU",
+    "plain loop, 32-key blocks, four waves, three workgroups per CU",
+    "software-pipelined loop, 64-key blocks, four waves (128 query rows), two workgroups per CU",
+    "software-pipelined loop, 64-key blocks, eight waves (256 query rows), one workgroup per CU",
+};
+
 template <typename T>
 int dispatch_attention(AttentionParams &p, int head_dim, int variant, hipStream_t stream) {
+    if (head_dim == 32) note_launch(kLaunchAttention, 0, "plain loop, 64-key blocks, head dimension 32");
+    else if (head_dim != 128 && head_dim != 64) note_launch(kLaunchAttention, 0, "head dimension padded to the next kernel size");
+    else note_launch(kLaunchAttention, variant, variant >= 0 && variant < kAttentionVariants ? kAttentionVariantNames[variant] : "measurement variant");
     if (head_dim == 128) {
         if (variant == 4) return (int)launch_attention<T, 128, 1, 64, 2, true, T, 8>(p, stream);
 #ifdef NT_MEASUREMENT_AIDS
@@ -1112,8 +1135,6 @@ int attention_setup(AttentionParams &p, const NineToothedTensor &q, const NineTo
     return 0;
 }
 
-constexpr int kAttentionVariants = 5;
-
 void attention_tune_values(const AttentionParams &p, int dtype, int (&values)[7]) {
     const int v[7] = {dtype, p.batch, p.heads, p.seq_q, p.seq_k, p.head_dim, p.causal};
     for (int i = 0; i < 7; ++i) values[i] = v[i];
@@ -1130,11 +1151,13 @@ int attention_split(AttentionParams &p, int dtype, hipStream_t stream) {
     return NINETOOTHED_NO_KERNEL;
 }
 
-bool attention_would_split(const AttentionParams &p) {
-    const int64_t groups = (int64_t)p.batch * p.heads * ceil_div(p.seq_q, kAttnWaves * 32);
-    const int key_blocks = ceil_div(p.seq_k, 64);
-    return groups > 0 && groups < 128 && key_blocks >= 8 && std::min<int64_t>((512 + groups - 1) / groups, key_blocks / 4) >= 2;
+// the variant a call without hints runs before anything is tuned: the pipelined loop, with eight waves for
+// non-causal problems that have enough 256-row query blocks to fill the chip twice
+int attention_untuned_variant(const AttentionParams &p) {
+    return !p.causal && p.head_dim >= 64 && (int64_t)p.batch * p.heads * ceil_div(p.seq_q, 256) >= 512 ? 4 : 3;
 }
+
+bool attention_would_split(const AttentionParams &p) { return (p.head_dim == 128 || p.head_dim == 64) && split_key_parts(p) > 0; }
 
 }  // namespace
 }  // namespace nt
@@ -1155,7 +1178,7 @@ extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineT
     // 256-row blocks to fill the chip twice run it with eight waves per workgroup, which loads every K / V
     // block once for 256 query rows (1.16 PFLOP/s; causal 0.99, below the four-wave form).
     int variant = block_size_m >= 256 ? 1 : (block_size_n > 0 && block_size_n <= 32 ? 2 : (block_size_n >= 64 ? 0 : 3));
-    if (variant == 3 && !p.causal && block_size_m == 0 && head_dim >= 64 && (int64_t)p.batch * p.heads * ceil_div(p.seq_q, 256) >= 512) variant = 4;
+    if (variant == 3 && block_size_m == 0) variant = attention_untuned_variant(p);
 #ifdef NT_MEASUREMENT_AIDS
     if (block_size_n >= 1000) variant = block_size_n - 1000;  // explicit variant, for timing harnesses only
 #endif
@@ -1187,12 +1210,18 @@ extern "C" NineToothedResult nt_tune_attention(NineToothedStream stream, NineToo
     if (!attention_tunable(p, dtype) || attention_would_split(p)) return 0;
     int best = -1;
     float best_time = 0.0f;
-    const int result = tune_time((hipStream_t)stream, kAttentionVariants, iters, [&](int variant) -> int {
+    // the untuned rule's variant comes first and stays unless another one is more than 2 % faster: the pipelined
+    // variants lie within a few per cent of each other, and the choice should not change from process to process
+    // for nothing
+    const int preferred = attention_untuned_variant(p);
+    auto variant_of = [&](int i) { return i == 0 ? preferred : (i - 1 < preferred ? i - 1 : i); };
+    const int result = tune_time((hipStream_t)stream, kAttentionVariants, iters, [&](int i) -> int {
         AttentionParams copy = p;
-        if (dtype == NINETOOTHED_FLOAT16) return dispatch_attention<half_t>(copy, p.head_dim, variant, (hipStream_t)stream);
-        return dispatch_attention<bf16_t>(copy, p.head_dim, variant, (hipStream_t)stream);
-    }, &best, &best_time);
+        if (dtype == NINETOOTHED_FLOAT16) return dispatch_attention<half_t>(copy, p.head_dim, variant_of(i), (hipStream_t)stream);
+        return dispatch_attention<bf16_t>(copy, p.head_dim, variant_of(i), (hipStream_t)stream);
+    }, &best, &best_time, 0.02f);
     if (result != 0) return result;
+    if (best >= 0) best = variant_of(best);
     if (best_variant) *best_variant = best;
     if (best < 0) return 0;
     int values[7];

@@ -740,6 +740,11 @@ int run_direct(const Conv2dRequest &q, hipStream_t stream) {
     const int CRS = q.C * q.R * q.S;
     if (q.Q % 8 || q.W < 8 || q.pad_w > 1 || CRS % 32 || q.R > 16 || q.S > 16) return NINETOOTHED_NO_KERNEL;
     if (q.xs[3] != 1 || q.xs[0] < 0 || q.xs[1] < 0 || q.xs[2] < 0) return NINETOOTHED_NO_KERNEL;
+    // Offsets must grow with (image, channel, row): the kernel decides from the first and the last piece of a tile
+    // whether any of its loads could start before the tensor or end behind it, which an input whose images, channels
+    // or rows overlap in memory (a stride of 0 from `expand`, say) would defeat.
+    const int64_t row_span = q.W, channel_span = (int64_t)(q.H - 1) * q.xs[2] + row_span, image_span = (int64_t)(q.C - 1) * q.xs[1] + channel_span;
+    if ((q.H > 1 && q.xs[2] < row_span) || (q.C > 1 && q.xs[1] < channel_span) || (q.N > 1 && q.xs[0] < image_span)) return NINETOOTHED_NO_KERNEL;
     if (q.ws[3] != 1 || q.ws[2] != q.S || q.ws[1] != (int64_t)q.R * q.S || q.ws[0] != CRS || ((uintptr_t)q.w & 15)) return NINETOOTHED_NO_KERNEL;
     // at least four fifths of the 256 output channels of a tile in use
     if ((int64_t)q.K * 5 < (int64_t)ceil_div(q.K, 256) * 256 * 4) return NINETOOTHED_NO_KERNEL;

@@ -134,7 +134,8 @@ hipError_t fast_launch(const GemmProblem &q, hipStream_t stream) {
 // memory of the stream, and a second kernel sums the parts and applies the epilogue.
 
 // number of parts for tiles of bm x bn x bk, 1 = do not split
-int split_parts(const GemmProblem &q, int bm, int bn, int bk, int *kt_per_part) {
+// (`scratch_limit`: bytes the partial products may take)
+int split_parts(const GemmProblem &q, int bm, int bn, int bk, int *kt_per_part, int64_t scratch_limit = int64_t(64) << 20) {
     const int64_t tiles = (int64_t)((q.m + bm - 1) / bm) * ((q.n + bn - 1) / bn);
     const int num_kt = (q.k + bk - 1) / bk;
     if (tiles >= 320) return 1;  // (the untuned choice only splits below 192 tiles; between, the tuner decides)
@@ -142,7 +143,7 @@ int split_parts(const GemmProblem &q, int bm, int bn, int bk, int *kt_per_part) 
     int64_t parts = bm * bn >= 256 * 256 ? 256 / tiles : (512 + tiles - 1) / tiles;
     parts = std::min<int64_t>(parts, num_kt / 2);                  // at least two k tiles each
     parts = std::min<int64_t>(parts, 256);
-    while (parts >= 2 && parts * q.m * q.n * 4 > (int64_t(64) << 20)) --parts;  // scratch of at most 64 MiB
+    while (parts >= 2 && parts * q.m * q.n * 4 > scratch_limit) --parts;  // scratch of at most 64 MiB, or what the caller's fixed array holds
     if (parts < 2) return 1;
     const int per_part = (int)((num_kt + parts - 1) / parts);
     if (kt_per_part) *kt_per_part = per_part;
@@ -192,8 +193,9 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float *par
 template <typename T, int BM, int BN, int BK, int WM, int WN, int kStages, int kOcc>
 hipError_t split_launch_typed(const GemmProblem &q, hipStream_t stream) {
     int kt_per_part = 0;
-    const int parts = split_parts(q, BM, BN, BK, &kt_per_part);
-    if (parts < 2) return (hipError_t)NINETOOTHED_NO_KERNEL;
+    // with a fixed array the part count shrinks until the partial products fit; the call is refused when not even two parts do
+    const int parts = q.fixed_scratch != nullptr ? split_parts(q, BM, BN, BK, &kt_per_part, (int64_t)q.fixed_scratch_bytes) : split_parts(q, BM, BN, BK, &kt_per_part);
+    if (parts < 2) return (hipError_t)(q.fixed_scratch != nullptr && split_parts(q, BM, BN, BK, nullptr) >= 2 ? NINETOOTHED_SCRATCH_LIMIT : NINETOOTHED_NO_KERNEL);
     const size_t scratch_bytes = (size_t)parts * q.m * q.n * sizeof(float);
     // the lock of the workspace registry also serialises host threads that enqueue onto the fixed array
     WorkspaceLease lease(stream);
@@ -460,10 +462,14 @@ int run_gemm(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk) {
     if (bm <= 0 || bn <= 0) choice = lookup_tuned(q);
     if (choice < 0 || !kInstances[choice].accepts(q)) choice = heuristic_choice(q, bm, bn, bk);
     if (choice < 0) return NINETOOTHED_NO_KERNEL;
+    note_launch(kLaunchGemm, choice, kInstances[choice].name);
     int result = (int)kInstances[choice].launch(q, stream);
     if (result == NINETOOTHED_NO_KERNEL && is_split(choice)) {  // a split-K instance without scratch memory
         for (int fallback : {(int)kTail64x64x64, (int)kTail128x128x64, (int)kTail256x256x32, (int)kAnyStride})
-            if (kInstances[fallback].accepts(q)) return (int)kInstances[fallback].launch(q, stream);
+            if (kInstances[fallback].accepts(q)) {
+                note_launch(kLaunchGemm, fallback, kInstances[fallback].name);
+                return (int)kInstances[fallback].launch(q, stream);
+            }
     }
     return result;
 }
@@ -610,7 +616,7 @@ namespace {
 
 // the ways to run a convolution; kConvAuto tries them from the top (a 1 x 1 filter without padding first runs
 // as a batch of plain products when it can)
-enum ConvPath { kConvAuto = 0, kConvGather = 1, kConvRepack = 2, kConvDirect = 3 };
+enum ConvPath { kConvAuto = 0, kConvGather = 1, kConvRepack = 2, kConvDirect = 3, kConvPointwise = 4 };
 
 // validates the call and fills the request; returns 0, an error, or -1 when there is nothing to compute
 int conv2d_request(Conv2dRequest &request, const NineToothedTensor &input, const NineToothedTensor &filter, const NineToothedTensor &output,
@@ -664,42 +670,58 @@ hipError_t conv2d_gather(const Conv2dRequest &r, hipStream_t stream) {
     return hipGetLastError();
 }
 
+// 1 x 1 filters without padding: per image Y[K, P*Q] = W[K, C] . X[C, P*Q], a batch of row-major products on
+// the tensors as they lie (no repacking, no scratch memory).  NINETOOTHED_NO_KERNEL when the call is not that
+// or no one-pass GEMM instance of the fast kind takes it.
+int conv2d_pointwise(const Conv2dRequest &r, hipStream_t stream) {
+    if (!(r.R == 1 && r.S == 1 && r.pad_h == 0 && r.pad_w == 0 && r.xs[3] == 1 && r.xs[2] == r.W && r.ys[3] == 1 && r.ys[2] == r.Q && r.ws[1] == 1))
+        return NINETOOTHED_NO_KERNEL;
+    GemmProblem q;
+    q.dtype = q.out_dtype = r.dtype;
+    q.m = r.K;
+    q.n = r.P * r.Q;
+    q.k = r.C;
+    q.a = r.w;
+    q.b = r.x;
+    q.c = r.y;
+    q.bias = nullptr;
+    q.sam = r.ws[0]; q.sak = 1;
+    q.sbk = r.xs[1]; q.sbn = 1;
+    q.scm = r.ys[1]; q.scn = 1;
+    q.sim = q.sin = 0;
+    q.alpha = 1.0f; q.beta = 0.0f;
+    q.batch = r.N;
+    q.a_batch = 0;
+    q.b_batch = r.xs[0];
+    q.c_batch = r.ys[0];
+    const int choice = heuristic_choice(q, 0, 0, 0);
+    if (choice <= kAnyStride || is_split(choice)) return NINETOOTHED_NO_KERNEL;
+    note_launch(kLaunchConv2d, kConvPointwise, kInstances[choice].name);
+    return (int)kInstances[choice].launch(q, stream);
+}
+
 int conv2d_run(const Conv2dRequest &r, int path, hipStream_t stream) {
-    // 1 x 1 filters without padding: per image Y[K, P*Q] = W[K, C] . X[C, P*Q], a batch of row-major
-    // products on the tensors as they lie (no repacking, no scratch memory)
     // fp32 tensors: the gathering kernel on fp32 MFMAs (the other paths move 16-bit elements)
-    if (r.dtype == NINETOOTHED_FLOAT32) return path == kConvAuto || path == kConvGather ? (int)conv2d_gather<float>(r, stream) : NINETOOTHED_NO_KERNEL;
-    if (path == kConvAuto && r.R == 1 && r.S == 1 && r.pad_h == 0 && r.pad_w == 0 && r.xs[3] == 1 && r.xs[2] == r.W && r.ys[3] == 1 &&
-        r.ys[2] == r.Q && r.ws[1] == 1) {
-        GemmProblem q;
-        q.dtype = q.out_dtype = r.dtype;
-        q.m = r.K;
-        q.n = r.P * r.Q;
-        q.k = r.C;
-        q.a = r.w;
-        q.b = r.x;
-        q.c = r.y;
-        q.bias = nullptr;
-        q.sam = r.ws[0]; q.sak = 1;
-        q.sbk = r.xs[1]; q.sbn = 1;
-        q.scm = r.ys[1]; q.scn = 1;
-        q.sim = q.sin = 0;
-        q.alpha = 1.0f; q.beta = 0.0f;
-        q.batch = r.N;
-        q.a_batch = 0;
-        q.b_batch = r.xs[0];
-        q.c_batch = r.ys[0];
-        const int choice = heuristic_choice(q, 0, 0, 0);
-        if (choice > kAnyStride && !is_split(choice)) return (int)kInstances[choice].launch(q, stream);
+    if (r.dtype == NINETOOTHED_FLOAT32) {
+        if (path != kConvAuto && path != kConvGather) return NINETOOTHED_NO_KERNEL;
+        note_launch(kLaunchConv2d, kConvGather, "gemm_generic_kernel with an im2col gather, fp32 MFMA");
+        return (int)conv2d_gather<float>(r, stream);
+    }
+    if (path == kConvAuto || path == kConvPointwise) {
+        const int pointwise = conv2d_pointwise(r, stream);
+        if (pointwise != NINETOOTHED_NO_KERNEL || path == kConvPointwise) return pointwise;
     }
     if (path == kConvAuto || path == kConvDirect) {
+        note_launch(kLaunchConv2d, kConvDirect, "conv2d_direct_kernel, one launch on the tensors as they lie");
         const int direct = conv2d_direct(r, stream);
         if (direct != NINETOOTHED_NO_KERNEL || path == kConvDirect) return direct;
     }
     if (path == kConvAuto || path == kConvRepack) {
+        note_launch(kLaunchConv2d, kConvRepack, "conv2d_repack_kernel, then conv2d_nhwc_kernel on channels-last copies");
         const int fast = conv2d_fast(r, stream);
         if (fast != NINETOOTHED_NO_KERNEL || path == kConvRepack) return fast;
     }
+    note_launch(kLaunchConv2d, kConvGather, "gemm_generic_kernel with an im2col gather");
     return r.dtype == NINETOOTHED_FLOAT16 ? (int)conv2d_gather<half_t>(r, stream) : (int)conv2d_gather<bf16_t>(r, stream);
 }
 
@@ -722,14 +744,14 @@ NineToothedResult launch_nt_conv2d(NineToothedStream stream, NineToothedTensor i
     Conv2dRequest request;
     const int status = conv2d_request(request, input, filter, output, dtype, padding_h, padding_w);
     if (status != 0) return status < 0 ? 0 : status;
-    // block_size_m: 1 = the gather kernel, 2 = the repacking path, 3 = the one-launch path; otherwise the
-    // tuned choice for this problem, else the library's order
-    int path = block_size_m >= kConvGather && block_size_m <= kConvDirect ? block_size_m : kConvAuto;
+    // block_size_m: 1 = the gather kernel, 2 = the repacking path, 3 = the one-launch path, 4 = a 1 x 1 filter as a
+    // batch of plain products; otherwise the tuned choice for this problem, else the library's order
+    int path = block_size_m >= kConvGather && block_size_m <= kConvPointwise ? block_size_m : kConvAuto;
     if (block_size_m == 0) {
         int values[11];
         conv2d_tune_values(request, values);
         const int tuned = tune_lookup(kTuneConv2d, values, 11);
-        if (tuned >= kConvGather && tuned <= kConvDirect) path = tuned;
+        if (tuned >= kConvGather && tuned <= kConvPointwise) path = tuned;
     }
     int result = conv2d_run(request, path, (hipStream_t)stream);
     // (a tuned path that needs scratch memory it cannot get, e.g. under graph capture: the library's order)
@@ -746,11 +768,11 @@ NineToothedResult nt_tune_conv2d(NineToothedStream stream, NineToothedTensor inp
     if (status != 0) return status < 0 ? 0 : status;
     int values[11];
     conv2d_tune_values(request, values);
-    const int paths[3] = {kConvDirect, kConvRepack, kConvGather};
+    const int paths[4] = {kConvPointwise, kConvDirect, kConvRepack, kConvGather};
     int best = -1;
     float best_time = 0.0f;
-    // the one-launch path needs no scratch memory: it stays unless another way is more than 3 % faster
-    const int result = tune_time((hipStream_t)stream, 3, iters, [&](int i) -> int { return conv2d_run(request, paths[i], (hipStream_t)stream); }, &best, &best_time, 0.03f);
+    // an earlier way stays unless a later one is more than 3 % faster: the first two need no scratch memory and one launch
+    const int result = tune_time((hipStream_t)stream, 4, iters, [&](int i) -> int { return conv2d_run(request, paths[i], (hipStream_t)stream); }, &best, &best_time, 0.03f);
     if (result != 0) return result;
     if (best < 0) return 0;  // (a stream under graph capture: nothing was timed)
     tune_record(kTuneConv2d, values, 11, paths[best]);

@@ -34,6 +34,7 @@
 #include <vector>
 
 #include "nt_common.h"
+#include "tune.h"
 
 namespace nt {
 namespace {
@@ -1166,9 +1167,11 @@ extern "C" NineToothedResult launch_nt_map(NineToothedStream stream, const NineT
             args.total_out = total_out;
             size_t size = sizeof(args);
             void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+            nt::note_launch(nt::kLaunchMap, 0, "kernel generated for the program and compiled with hipRTC");
             return (int)hipModuleLaunchKernel(function, (unsigned)blocks, 1, 1, (unsigned)workgroup_threads(p), 1, 1, 0, (hipStream_t)stream, nullptr, config);
         }
     }
+    nt::note_launch(nt::kLaunchMap, 1, "interpreter kernel");
     if (p.num_phases > 0)
         map_tile_kernel<<<dim3((unsigned)blocks), dim3(kMapThreads), 0, (hipStream_t)stream>>>(p, tiles, tile_elements);
     else

@@ -5,6 +5,7 @@
 // columns [s * block, min((s + 1) * block, N)) of one row.  With block >= N
 // (the usual call) a segment is a whole row.
 #include "nt_common.h"
+#include "tune.h"
 
 namespace nt {
 namespace {
@@ -231,6 +232,7 @@ hipError_t launch_vec(const SoftmaxParams &p, int vecs_needed, hipStream_t strea
     const int64_t total = p.rows * p.segments;
     constexpr int kGroups = kRowThreads > 256 ? 1 : 256 / kRowThreads;
     const dim3 grid((unsigned)((total + kGroups - 1) / kGroups)), block(kRowThreads > 256 ? kRowThreads : 256);
+    note_launch(kLaunchSoftmax, kRowThreads, "softmax_vec_kernel, 16-byte vectors, this many threads per row segment");
     if (vecs_needed <= 1)
         softmax_vec_kernel<T, kRowThreads, 1><<<grid, block, 0, stream>>>(p);
     else if (vecs_needed <= 2)
@@ -249,6 +251,7 @@ hipError_t launch_elem(const SoftmaxParams &p, hipStream_t stream) {
     const int64_t total = p.rows * p.segments;
     constexpr int kGroups = kRowThreads > 256 ? 1 : 256 / kRowThreads;
     const dim3 grid((unsigned)((total + kGroups - 1) / kGroups)), block(kRowThreads > 256 ? kRowThreads : 256);
+    note_launch(kLaunchSoftmax, kRowThreads, "softmax_elem_kernel, element by element, this many threads per row segment");
     softmax_elem_kernel<T, kRowThreads, kElems><<<grid, block, 0, stream>>>(p);
     return hipGetLastError();
 }
@@ -295,6 +298,7 @@ int run_softmax(const SoftmaxParams &p, int variant, hipStream_t stream) {
     // 2048 x 30001 fp32 2.1 in registers of 1024 threads, 3.9 with the loop kernel)
     if (len <= 256 * 32) return (int)launch_elem<T, 256, 64>(p, stream);
     if (len <= 1024 * 16) return (int)launch_elem<T, 1024, 16>(p, stream);
+    note_launch(kLaunchSoftmax, kLoopThreads, "softmax_loop_kernel, two sweeps over a long row segment");
     softmax_loop_kernel<T><<<dim3((unsigned)total), dim3(kLoopThreads), 0, stream>>>(p);
     return (int)hipGetLastError();
 }

@@ -19,12 +19,27 @@ int tune_lookup(int kind, const int *values, int count);
 // (`extra`: up to three descriptive integers kept with the choice and written after it to the cache file)
 void tune_record(int kind, const int *values, int count, int choice, const int *extra = nullptr, int extras = 0);
 
-// Times candidates 0 .. candidates - 1 on `stream` with device events: 2 warm-up launches and `iters` timed ones
-// each (a candidate whose `iters` launches take less than 0.5 ms is timed again over about 0.75 ms, at most 256 launches).  `launch(i)` returns 0, NINETOOTHED_NO_KERNEL (the candidate does not take the problem: skipped) or an
-// error (returned).  *best receives the fastest candidate (-1 when none ran); with a `margin`, a later candidate
-// replaces an earlier one only when it is faster by more than that fraction (candidates in order of preference).
-// The first candidate is preceded by an untimed warm-up of about 20 ms.
+// Which kernel served the latest launch_nt_* call of the calling host thread: the launch functions leave a note
+// (three thread-local stores), nt_last_launch formats it.  `name` must point to a string that lives as long as
+// the library (a literal or an instance table entry).
+enum LaunchProgram { kLaunchNone = 0, kLaunchGemm, kLaunchAttention, kLaunchConv2d, kLaunchSoftmax, kLaunchMap };
+void note_launch(int program, int choice, const char *name);
+
+// Times candidates 0 .. candidates - 1 on `stream` with device events and reports the fastest.  `launch(i)` returns 0,
+// NINETOOTHED_NO_KERNEL (the candidate does not take the problem: skipped) or an error (returned).
+//
+// A choice made from one short timed region per candidate is a matter of luck on a part whose clock moves with
+// load and temperature: a dip during one candidate's few milliseconds decides the variant for the rest of the
+// process.  So (as triton.testing.do_bench, which the reference's autotuner uses, runs every configuration for a
+// fixed time): the first candidate that runs is launched untimed for about 20 ms, every candidate's launch time is
+// estimated over `iters` launches, and then the candidates take turns over several rounds -- each round times
+// every candidate over a region of about 3 ms (at least one launch, at most 256) -- and a candidate's figure is the
+// minimum of its rounds, so that a slow spell has to hit the same candidate in every round to mislead.
+// Candidates are in order of preference: with a `margin`, a later candidate replaces an earlier one only when it
+// is faster by more than that fraction.  *best = -1 when none ran.
 // Synchronises; returns without timing anything (*best = -1, result 0) when the stream is being captured into a graph.
+constexpr int kTuneMaxCandidates = 64;
+
 template <typename Launch>
 int tune_time(hipStream_t stream, int candidates, int iters, Launch launch, int *best, float *best_ms, float margin = 0.0f) {
     *best = -1;
@@ -36,6 +51,7 @@ int tune_time(hipStream_t stream, int candidates, int iters, Launch launch, int 
     }
     if (status != hipStreamCaptureStatusNone) return 0;
     if (iters <= 0) iters = 5;
+    if (candidates > kTuneMaxCandidates) candidates = kTuneMaxCandidates;
     hipEvent_t start, stop;
     hipError_t err;
     if ((err = hipEventCreate(&start)) != hipSuccess) return (int)err;
@@ -43,55 +59,61 @@ int tune_time(hipStream_t stream, int candidates, int iters, Launch launch, int 
         (void)hipEventDestroy(start);
         return (int)err;
     }
-    int result = 0;
-    bool warm = false;
-    for (int i = 0; i < candidates && result == 0; ++i) {
+    // milliseconds that `count` launches of candidate i take (negative: an error code, negated)
+    auto region = [&](int i, int count, float *ms) -> int {
+        int rc = 0;
+        (void)hipEventRecord(start, stream);
+        for (int r = 0; r < count && rc == 0; ++r) rc = launch(i);
+        (void)hipEventRecord(stop, stream);
+        const hipError_t waited = hipEventSynchronize(stop);
+        if (rc == 0 && waited != hipSuccess) rc = (int)waited;
+        *ms = 0.0f;
+        if (rc == 0) (void)hipEventElapsedTime(ms, start, stop);
+        return rc;
+    };
+    int live[kTuneMaxCandidates], launches[kTuneMaxCandidates];
+    float fastest[kTuneMaxCandidates];
+    int alive = 0, result = 0;
+    for (int i = 0; i < candidates && result == 0; ++i) {  // which candidates take the problem
         int rc = launch(i);
         if (rc == 1) continue;  // NINETOOTHED_NO_KERNEL
         if (rc == 0) rc = launch(i);
-        if (rc != 0) {
-            result = rc;
-            break;
-        }
-        // The first candidate that runs would otherwise be timed on an idle part whose clocks are still ramping up,
-        // and lose to a slower one timed later: it first runs untimed for about 20 ms (at most 64 rounds).
-        float warmed_ms = 0.0f;
-        for (int round = 0; !warm && round < 64 && warmed_ms < 20.0f && rc == 0; ++round) {
-            (void)hipEventRecord(start, stream);
-            for (int r = 0; r < iters && rc == 0; ++r) rc = launch(i);
-            (void)hipEventRecord(stop, stream);
-            if (rc == 0 && (err = hipEventSynchronize(stop)) != hipSuccess) rc = (int)err;
-            float ms = 0.0f;
-            if (rc == 0) (void)hipEventElapsedTime(&ms, start, stop);
+        if (rc != 0) result = rc;
+        else live[alive++] = i;
+    }
+    if (result == 0 && alive > 0) {
+        float ms = 0.0f, warmed_ms = 0.0f;
+        for (int round = 0; round < 64 && warmed_ms < 20.0f && result == 0; ++round) {  // let the part raise its clocks
+            result = region(live[0], iters, &ms);
             warmed_ms += ms;
         }
-        warm = true;
-        if (rc != 0) {
-            result = rc;
-            break;
+        float round_ms = 0.0f;
+        for (int c = 0; c < alive && result == 0; ++c) {  // how many launches make a region of about 3 ms
+            result = region(live[c], iters, &ms);
+            const float one = ms > 0.0f ? ms / (float)iters : 0.01f;
+            const int wanted = (int)(3.0f / one) + 1;
+            launches[c] = wanted > 256 ? 256 : wanted;
+            fastest[c] = one;
+            round_ms += one * (float)launches[c];
         }
-        // short kernels are timed over more launches: a timed region of a few microseconds says little
-        float ms = 0.0f;
-        int timed = iters;
-        for (int attempt = 0; attempt < 2 && rc == 0; ++attempt) {
-            (void)hipEventRecord(start, stream);
-            for (int r = 0; r < timed && rc == 0; ++r) rc = launch(i);
-            (void)hipEventRecord(stop, stream);
-            if (rc == 0 && (err = hipEventSynchronize(stop)) != hipSuccess) rc = (int)err;
-            if (rc != 0) break;
-            (void)hipEventElapsedTime(&ms, start, stop);
-            if (ms >= 0.5f || timed >= 256) break;
-            const int wanted = ms > 0.0f ? (int)(0.75f * (float)timed / ms) + 1 : 256;  // about 0.75 ms
-            if (attempt == 0) timed = wanted < 256 ? (wanted > timed ? wanted : timed) : 256;
+        // long kernels get fewer rounds: a choice between candidates of 100 ms each is not worth seconds
+        const int rounds = round_ms <= 100.0f ? 5 : (round_ms <= 400.0f ? 3 : 1);
+        for (int round = 0; round < rounds && result == 0; ++round) {
+            for (int c = 0; c < alive && result == 0; ++c) {
+                result = region(live[c], launches[c], &ms);
+                const float one = ms / (float)launches[c];
+                if (result == 0 && (round == 0 || one < fastest[c])) fastest[c] = one;
+            }
         }
-        if (rc != 0) {
-            result = rc;
-            break;
+        for (int c = 0; c < alive && result == 0; ++c) {
+            if (*best < 0 || fastest[c] < *best_ms * (1.0f - margin)) {
+                *best = live[c];
+                *best_ms = fastest[c];
+            }
         }
-        ms /= (float)timed;
-        if (*best < 0 || ms < *best_ms * (1.0f - margin)) {
-            *best = i;
-            *best_ms = ms;
+        if (result != 0) {
+            *best = -1;
+            *best_ms = 0.0f;
         }
     }
     (void)hipEventDestroy(start);

@@ -67,11 +67,34 @@ void tune_record(int kind, const int *values, int count, int choice, const int *
     g_choices[key] = entry;
 }
 
+namespace {
+thread_local int t_launch_program = kLaunchNone;
+thread_local int t_launch_choice = -1;
+thread_local const char *t_launch_name = nullptr;
+}  // namespace
+
+void note_launch(int program, int choice, const char *name) {
+    t_launch_program = program;
+    t_launch_choice = choice;
+    t_launch_name = name;
+}
+
 }  // namespace nt
 
 using namespace nt;
 
 extern "C" {
+
+// Describes the kernel that served the calling thread's latest launch_nt_* call, e.g.
+// "attention variant 3: software-pipelined loop, 64-key blocks, four waves".
+NineToothedResult nt_last_launch(char *buffer, int size) {
+    if (buffer == nullptr || size <= 0) return hipErrorInvalidValue;
+    static const char *const programs[] = {"none", "gemm instance", "attention variant", "conv2d path", "softmax kernel", "tile map"};
+    const int program = t_launch_program >= kLaunchNone && t_launch_program <= kLaunchMap ? t_launch_program : kLaunchNone;
+    if (program == kLaunchNone) snprintf(buffer, (size_t)size, "none");
+    else snprintf(buffer, (size_t)size, "%s %d: %s", programs[program], t_launch_choice, t_launch_name ? t_launch_name : "");
+    return 0;
+}
 
 int nt_tune_lookup(int kind, const int *values, int count) { return tune_lookup(kind, values, count); }
 

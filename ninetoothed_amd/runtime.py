@@ -84,8 +84,7 @@ _SIGNATURES = {
     "nt_tune_attention": (_S, _T, _T, _T, _T, _T, _T, _I, _I, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_float)),
     "nt_tune_conv2d": (_S, _T, _T, _T, _I, _I, _I, _I, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_float)),
     "nt_tune_lookup": (_I, ctypes.POINTER(ctypes.c_int), _I),
-    "nt_probe_mfma_rate": (_S, _T, _T, _I, ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64)),
-    "nt_probe_mfma_rate_16x16x32": (_S, _T, _T, _I, ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64)),
+    "nt_last_launch": (ctypes.c_char_p, _I),
     "launch_nt_map": (_S, ctypes.c_void_p),
     "nt_map_source": (ctypes.c_void_p, ctypes.c_char_p, _I),
     "nt_tune_cache_save": (ctypes.c_char_p,),
@@ -142,6 +141,14 @@ def current_stream():
         return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(torch.cuda.current_device()))
     except AttributeError:  # a torch without the private accessor
         return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def last_launch():
+    """Which kernel served this thread's latest ``launch_nt_*`` call (instance, variant or path by index and
+    description), as the library reports it."""
+    buffer = ctypes.create_string_buffer(256)
+    check(library().nt_last_launch(buffer, len(buffer)))
+    return buffer.value.decode()
 
 
 def gemm_config_names():

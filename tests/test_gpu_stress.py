@@ -29,13 +29,22 @@ def test_addmm_8192_whole_output_and_repeatability(dtype):
     input, mat1, mat2 = _seeded(n, n, dtype=dtype, seed=0), _seeded(n, n, dtype=dtype, seed=1), _seeded(n, n, dtype=dtype, scale=0.05, seed=2)
     application = programs.addmm.application if dtype == torch.float16 else programs.addmm.application_bfloat16
     kernel = ninetoothed.make(programs.addmm.arrangement, application, programs.addmm.tensors())
-    expected = torch.addmm(input, mat1, mat2, beta=0.5, alpha=1.0)
+    # the program's arithmetic in fp32: product rounded to the element type, combined in fp32, rounded once
+    product = (mat1.float() @ mat2.float()).to(dtype).float()
+    expected = (0.5 * input.float() + product).to(dtype)
+    # fp16: rtol = atol = 1e-2.  bf16: two correct fp32 sums may round to neighbouring bf16 products, one ulp apart
+    # (2^-7 of a product of magnitude up to ~16 here = 0.06 at most, typically 0.03), and the input term may cancel
+    # the rest of the value: the absolute tolerance is one bf16 ulp of the typical product, not a hundredth.
+    tolerance = dict(rtol=1e-2, atol=1e-2) if dtype == torch.float16 else dict(rtol=1e-2, atol=2.0**-7 * float(product.abs().max()))
+    del product
+    vendor = torch.addmm(input, mat1, mat2, beta=0.5, alpha=1.0)
     first = None
     for _ in range(3):
         out = torch.full((n, n), float("nan"), dtype=dtype, device="cuda")
         kernel(input, mat1, mat2, 0.5, 1.0, out)
         assert kernel.last_plan.startswith("launch_nt_addmm")
-        assert torch.allclose(out, expected, rtol=2e-2, atol=2e-2)
+        assert torch.allclose(out, expected, **tolerance)
+        assert torch.allclose(out, vendor, rtol=2e-2, atol=2e-2 if dtype == torch.float16 else tolerance["atol"])
         if first is None:
             first = out
         else:
@@ -87,12 +96,14 @@ def test_conv2d_baseline_whole_output_and_repeatability():
     x = _seeded(32, 256, 56, 56, scale=0.1, seed=5)
     w = _seeded(256, 256, 3, 3, scale=0.1, seed=6)
     kernel = ninetoothed.make(programs.conv2d.arrangement, programs.conv2d.application, programs.conv2d.tensors())
-    expected = F.conv2d(x, w, padding=1)
+    expected = F.conv2d(x.float(), w.float(), padding=1)  # fp32 convolution of the same operands
+    vendor = F.conv2d(x, w, padding=1)
     first = None
     for _ in range(3):
         out = torch.full((32, 256, 56, 56), float("nan"), dtype=torch.float16, device="cuda")
         kernel(x, w, out, padding_h=1, padding_w=1)
-        assert torch.allclose(out, expected, **HALF_TOL)
+        assert torch.allclose(out.float(), expected, **HALF_TOL)
+        assert torch.allclose(out, vendor, **HALF_TOL)  # the stock fp16 operator of the same GPU
         if first is None:
             first = out
         else:
@@ -106,13 +117,26 @@ def test_attention_whole_output_and_repeatability(is_causal, head_dim, dtype):
     shape = (4, 16, 4096 if head_dim == 128 else 2048 + 64, head_dim)
     q, k, v = (_seeded(*shape, dtype=dtype, seed=s) for s in (7, 8, 9))
     kernel = ninetoothed.make(programs.attention.arrangement_with_scale, programs.attention.application_with_scale, programs.attention.tensors(True))
-    expected = torch.cat([F.scaled_dot_product_attention(q[b : b + 1], k[b : b + 1], v[b : b + 1], is_causal=is_causal, scale=head_dim**-0.5) for b in range(4)])
-    tolerance = HALF_TOL if dtype == torch.float16 else dict(rtol=2e-2, atol=2e-2)
+    # fp32 attention on the same (rounded) operands, four heads at a time, at rtol = atol = 1e-2 for both types;
+    # the stock operator of the same GPU as a second check (bf16: its output is two bf16 roundings away)
+    seq = shape[2]
+    mask = torch.ones(seq, seq, dtype=torch.bool, device="cuda").tril() if is_causal else None
+
+    def reference(qs, ks, vs):
+        scores = (qs.float() * head_dim**-0.5) @ ks.float().transpose(-1, -2)
+        if mask is not None:
+            scores = scores.masked_fill(~mask, float("-inf"))
+        return torch.softmax(scores, dim=-1) @ vs.float()
+
+    expected = torch.cat([torch.cat([reference(q[b : b + 1, h : h + 4], k[b : b + 1, h : h + 4], v[b : b + 1, h : h + 4]) for h in range(0, 16, 4)], dim=1) for b in range(4)])
+    vendor = torch.cat([F.scaled_dot_product_attention(q[b : b + 1], k[b : b + 1], v[b : b + 1], is_causal=is_causal, scale=head_dim**-0.5) for b in range(4)])
+    vendor_tolerance = HALF_TOL if dtype == torch.float16 else dict(rtol=2e-2, atol=2e-2)
     first = None
     for _ in range(3):
         out = torch.full_like(q, float("nan"))
         kernel(q, k, v, is_causal, head_dim**-0.5, out)
-        assert torch.allclose(out, expected, **tolerance)
+        assert torch.allclose(out.float(), expected, **HALF_TOL)
+        assert torch.allclose(out, vendor, **vendor_tolerance)
         if first is None:
             first = out
         else:
@@ -244,8 +268,7 @@ def test_attention_on_random_shapes():
         if is_causal:
             scores = scores.masked_fill(~torch.ones(seq_q, seq_k, dtype=torch.bool, device="cuda").tril(), float("-inf"))
         expected = torch.softmax(scores, dim=-1) @ v.float()
-        tolerance = 1e-2 if dtype == torch.float16 else 3e-2
-        assert torch.allclose(o.float(), expected, rtol=tolerance, atol=tolerance), (case, batch, heads, seq_q, seq_k, emb_dim, is_causal, dtype, packed)
+        assert torch.allclose(o.float(), expected, **HALF_TOL), (case, batch, heads, seq_q, seq_k, emb_dim, is_causal, dtype, packed)
 
 
 def test_mfma_rate_probe_runs_and_counts():
@@ -253,12 +276,14 @@ def test_mfma_rate_probe_runs_and_counts():
     (8 waves per compute unit x loops x 8; x 32 in the 16x16x32 form) and leaves its sink untouched."""
     import ctypes
 
+    import bench
     from ninetoothed_amd import runtime
 
     a = torch.randn(64, 64, dtype=torch.float16, device="cuda")
     sink = torch.zeros(1, device="cuda")
     count = ctypes.c_int64(0)
-    lib = runtime.library()
+    lib = bench.load_probe_library()  # (a library of its own: the product library does not export measurement aids)
+    assert not hasattr(runtime.library(), "nt_probe_mfma_rate")
     tensor = runtime.ArgumentTensor.from_torch_tensor(a)
     runtime.check(lib.nt_probe_mfma_rate(runtime.current_stream(), tensor, tensor, 3, sink.data_ptr(), ctypes.byref(count)))
     torch.cuda.synchronize()
