@@ -104,6 +104,20 @@ NineToothedResult launch_nt_matmul(NineToothedStream stream,
                                    int block_size_m, int block_size_n,
                                    int block_size_k);
 
+/* output[b] = lhs[b] @ rhs[b] for tensors [B, M, K], [B, K, N], [B, M, N]: the kernel the reference generates
+ * (src/ninetoothed/generation.py:46-133) for the matmul application of tests/test_matmul.py:41-45 under an
+ * arrangement that tiles a leading batch dimension by 1 (`tile((1, BLOCK_SIZE_M, BLOCK_SIZE_N))`, the level
+ * squeezed) -- the reference has no test of its own for it.  One launch: the grid holds tiles x B workgroups.
+ * An operand whose first extent is 1 is shared by all products; everything else as launch_nt_matmul (the
+ * fast instances need batch strides that are multiples of 8 elements; FLOAT8_E5M2 operands are not taken). */
+NineToothedResult launch_nt_batched_matmul(NineToothedStream stream,
+                                           NineToothedTensor lhs,
+                                           NineToothedTensor rhs,
+                                           NineToothedTensor output,
+                                           int dtype, int output_dtype,
+                                           int block_size_m, int block_size_n,
+                                           int block_size_k);
+
 /* output = beta * input + alpha * round_to_dtype(mat1 @ mat2), epilogue in fp32.
  * Replaces the kernel generated for tests/test_addmm.py:13-38 (argument order
  * input, mat1, mat2, beta, alpha, output as in its application).  beta and
@@ -176,7 +190,7 @@ NineToothedResult launch_nt_attention(NineToothedStream stream,
                                       int block_size_m, int block_size_n);
 
 /* output[N,K,P,Q] = conv2d(input[N,C,H,W], filter[K,C,R,S]) with stride 1,
- * dilation 1 and zero padding (padding_h, padding_w), computed as the implicit
+ * dilation 1 (launch_nt_conv2d_strided takes others) and zero padding (padding_h, padding_w), computed as the implicit
  * GEMM [N*P*Q, C*R*S] x [C*R*S, K] the arrangement of
  * tests/test_conv2d.py:13-48 describes.
  * Ways to run it, tried in this order unless block_size_m names one (4, 3, 2, 1)
@@ -205,6 +219,26 @@ NineToothedResult launch_nt_conv2d(NineToothedStream stream,
                                    int padding_h, int padding_w,
                                    int block_size_m, int block_size_n,
                                    int block_size_k);
+
+/* launch_nt_conv2d for windows that move by (stride_h, stride_w) over the padded input and whose taps lie
+ * (dilation_h, dilation_w) apart: output position (p, q) and tap (r, s) read input (p * stride_h + r * dilation_h -
+ * padding_h, q * stride_w + s * dilation_w - padding_w), zeros outside the input.  This is the arrangement of
+ * tests/test_conv2d.py:28-36 with `tile(..., strides=(-1, -1, stride_h, stride_w), dilation=(1, 1, dilation_h,
+ * dilation_w))` (src/ninetoothed/tensor.py:199-286).  The output holds, per dimension, either the windows that fit
+ * (`floor_mode=True`: (H + 2 padding - dilation (R - 1) - 1) / stride + 1, rounded down) or one more that hangs over
+ * the edge (`Tensor.tile`'s default rounds up; what hangs over reads as padding); other sizes are rejected.
+ * Steps of 1 with the fitting output are launch_nt_conv2d.  Otherwise way 2 (repacking pass plus GEMM loop, same
+ * conditions and scratch buffers) or way 1 (gather kernel) runs; block_size_m = 2 or 1 names one. */
+NineToothedResult launch_nt_conv2d_strided(NineToothedStream stream,
+                                           NineToothedTensor input,
+                                           NineToothedTensor filter,
+                                           NineToothedTensor output,
+                                           int dtype,
+                                           int padding_h, int padding_w,
+                                           int stride_h, int stride_w,
+                                           int dilation_h, int dilation_w,
+                                           int block_size_m, int block_size_n,
+                                           int block_size_k);
 
 /*
  * launch_nt_matmul for callers that cannot allocate device memory (code under HIP graph capture,

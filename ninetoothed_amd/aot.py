@@ -100,6 +100,8 @@ def _check_structure(kernel, constexprs):
         if result != "conv2d":
             raise UnsupportedProgram("The arrangement is not the implicit-GEMM view of a convolution the packaged dispatcher forwards.")
         return {"conv2d": True, "pad_h": info["pad_h"], "pad_w": info["pad_w"], **info["blocks"]}
+    if kind == "matmul" and kernel.types[0].source.ndim == 3:
+        raise UnsupportedProgram("Batched products are not packaged ahead of time (call them through `make`).")
     if kind in ("matmul", "addmm"):
         m, n, k = 96, 160, 224
         if kind == "matmul":

@@ -13,6 +13,9 @@ struct Conv2dRequest {
     void *y;
     int N, C, H, W, K, R, S, P, Q, pad_h, pad_w;
     int64_t xs[4], ws[4], ys[4];  // element strides of input, filter, output
+    // output position (p, q) and filter tap (r, s) read input (p * stride_h + r * dil_h - pad_h, q * stride_w + s * dil_w - pad_w)
+    int stride_h = 1, stride_w = 1, dil_h = 1, dil_w = 1;
+    bool unit_steps() const { return stride_h == 1 && stride_w == 1 && dil_h == 1 && dil_w == 1; }
 };
 
 // Runs the direct-to-LDS implicit GEMM when the request qualifies; returns

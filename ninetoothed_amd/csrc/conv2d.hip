@@ -48,6 +48,7 @@ struct ConvParams {
     int N, C, H, W, K, R, S, P, Q, pad_h, pad_w;
     int M, tiles_m, tiles_n;  // M = N*P*Q rows
     unsigned xt_bytes, wt_bytes;
+    int stride_h, stride_w, dil_h, dil_w;  // steps of the window over the input and between its taps
 };
 
 // ---- pre-pass: one launch, two jobs ----
@@ -186,8 +187,8 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
         const int m = m0 + row;
         const int image = m / PQ, pq = m - image * PQ;
         const int oy = pq / p.Q, ox = pq - oy * p.Q;
-        a_y[j] = m < p.M ? oy - p.pad_h : -(1 << 20);  // rows past the last image never pass the bounds test
-        a_x[j] = ox - p.pad_w;
+        a_y[j] = m < p.M ? oy * p.stride_h - p.pad_h : -(1 << 20);  // rows past the last image never pass the bounds test
+        a_x[j] = ox * p.stride_w - p.pad_w;
         a_base[j] = m < p.M ? (((image * p.H + a_y[j]) * p.W + a_x[j]) * p.C + chunk * 8) * 2 : 0;
     }
     unsigned b_src[kBInstr];
@@ -206,7 +207,7 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
         const int cb = kt / taps;
         const int tap = kt - cb * taps;
         const int c0 = cb * BK;
-        const int fy = tap / p.S, fx = tap - fy * p.S;
+        const int fy = (tap / p.S) * p.dil_h, fx = (tap % p.S) * p.dil_w;  // the tap's distance from the window's corner
         const int delta = ((fy * p.W + fx) * p.C + c0) * 2;
 #pragma unroll
         for (int j = 0; j < kAInstr; ++j) {
@@ -383,10 +384,23 @@ struct ConvDirectParams {
     unsigned x_bytes, w_bytes;
     int period;             // tiles after which the filter taps of a tile's 32 rows repeat: R*S / gcd(32, R*S)
     int period_bytes;       // ... and by how many bytes the rows' channels have moved on by then
+#ifdef NT_CONV_STAMPS
+    unsigned long long *stamps;  // measurement builds: per wave {loop, waiting for loads, waiting for own LDS traffic, waiting at the barrier}
+#endif
 };
+
+#ifdef NT_CONV_STAMPS
+unsigned long long *g_conv_stamps = nullptr;
+#endif
 
 // rows of the table of filter taps kept in LDS: at most this many tiles per period (5 x 5 filters: 25)
 constexpr int kConvDirectMaxPeriod = 25;
+
+// Measurement builds only (wrong results): bit 0 = no pixel loads inside the loop, bit 1 = no pixel stores into
+// LDS, bit 2 = no filter fills, bit 3 = no MFMAs, bit 4 = no fragment reads.  0 in the library.
+#ifndef NT_CONV_ABLATE
+#define NT_CONV_ABLATE 0
+#endif
 
 template <typename T>
 __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams p) {
@@ -618,6 +632,10 @@ __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams 
     // free, and requests the filter part of tile t + 3 into the stage of tile t - 1.
     const int num_k = p.CRS / BK;
     const int last_k = num_k - 1;
+#ifdef NT_CONV_STAMPS
+    unsigned long long stamp_loads = 0, stamp_lds = 0, stamp_sync = 0;
+    const unsigned long long stamp_begin = __builtin_amdgcn_s_memtime();
+#endif
     uint4_t held[2][kGather];  // pieces in flight, by tile parity
     unsigned held_cols[2][kGather];  // their rows' border masks
     auto run = [&](auto careful_tag) {
@@ -645,16 +663,29 @@ __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams 
             // the last step's have arrived here: the pieces of tile t + 2, stored below, and the filter part of
             // tile t + 1, which with that tile's pieces, stored one step ago (the barrier waits for this wave's LDS
             // traffic), completes tile t + 1.
+#if defined(NT_CONV_STAMPS) && NT_CONV_STAMPS == 1
+            {
+                unsigned long long t0, t1, t2, t3;
+                asm volatile("s_memtime %0\n\ts_waitcnt vmcnt(4)\n\ts_memtime %1\n\ts_waitcnt lgkmcnt(0)\n\ts_memtime %2\n\ts_barrier\n\ts_memtime %3\n\ts_waitcnt lgkmcnt(0)"
+                             : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3)::"memory");
+                stamp_loads += t1 - t0;
+                stamp_lds += t2 - t1;
+                stamp_sync += t3 - t2;
+            }
+#else
             wait_vmcnt<kAInstr + kGather>();
             lds_barrier();
-            scatter(std::integral_constant<int, (kS + 2) % kStages>(), held[kParity], held_cols[kParity]);
-            gather(careful_tag, held[kParity], held_cols[kParity]);
-            issue_filter(std::integral_constant<int, (kS + 3) % kStages>(), min(t + 3, last_k));
+#endif
+            if constexpr (!(NT_CONV_ABLATE & 2)) scatter(std::integral_constant<int, (kS + 2) % kStages>(), held[kParity], held_cols[kParity]);
+            if constexpr (!(NT_CONV_ABLATE & 1)) gather(careful_tag, held[kParity], held_cols[kParity]);
+            if constexpr (!(NT_CONV_ABLATE & 4)) issue_filter(std::integral_constant<int, (kS + 3) % kStages>(), min(t + 3, last_k));
             static_for<0, KS>([&](auto ks_tag) {
                 constexpr int ks = decltype(ks_tag)::value;
                 constexpr int cur = ks & 1, nxt = cur ^ 1;
-                if constexpr (ks + 1 < KS) read_frags(s, ks + 1, af[nxt], bf[nxt]);
+                if constexpr (NT_CONV_ABLATE & 16) {
+                } else if constexpr (ks + 1 < KS) read_frags(s, ks + 1, af[nxt], bf[nxt]);
                 else read_frags(NextStage(), 0, af[nxt], bf[nxt]);
+                if constexpr (!(NT_CONV_ABLATE & 8))
 #pragma unroll
                 for (int ti = 0; ti < TM; ++ti)
 #pragma unroll
@@ -685,6 +716,15 @@ __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams 
     };
     if (careful_tile) run(std::true_type());  // (the first and the last tile of a launch)
     else run(std::false_type());
+#ifdef NT_CONV_STAMPS
+    if (p.stamps && lane == 0) {
+        unsigned long long *dst = p.stamps + ((size_t)blockIdx.x * kWaves + wave) * 4;
+        dst[0] = __builtin_amdgcn_s_memtime() - stamp_begin;
+        dst[1] = stamp_loads;
+        dst[2] = stamp_lds;
+        dst[3] = stamp_sync;
+    }
+#endif
 
     // ---- epilogue ----
     // lane (l32, g) holds, per 32 x 32 tile, output channel l32 and in registers 4 * r4 .. + 3 the pixels
@@ -738,6 +778,8 @@ __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams 
 template <typename T>
 int run_direct(const Conv2dRequest &q, hipStream_t stream) {
     const int CRS = q.C * q.R * q.S;
+    if (!q.unit_steps()) return NINETOOTHED_NO_KERNEL;  // pixels of a row must be consecutive, taps one pixel apart
+    if (q.P != q.H + 2 * q.pad_h - q.R + 1 || q.Q != q.W + 2 * q.pad_w - q.S + 1) return NINETOOTHED_NO_KERNEL;
     if (q.Q % 8 || q.W < 8 || q.pad_w > 1 || CRS % 32 || q.R > 16 || q.S > 16) return NINETOOTHED_NO_KERNEL;
     if (q.xs[3] != 1 || q.xs[0] < 0 || q.xs[1] < 0 || q.xs[2] < 0) return NINETOOTHED_NO_KERNEL;
     // Offsets must grow with (image, channel, row): the kernel decides from the first and the last piece of a tile
@@ -772,6 +814,9 @@ int run_direct(const Conv2dRequest &q, hipStream_t stream) {
     p.tiles_ch = ceil_div(q.K, 256);
     const int64_t grid = (int64_t)ceil_div(p.M, 256) * p.tiles_ch;
     if (grid <= 0 || grid > 0x7fffffffll) return NINETOOTHED_NO_KERNEL;
+#ifdef NT_CONV_STAMPS
+    p.stamps = g_conv_stamps;
+#endif
     conv2d_direct_kernel<T><<<dim3((unsigned)grid), dim3(512), 0, stream>>>(p);
     return (int)hipGetLastError();
 }
@@ -803,6 +848,7 @@ int run_fast(const Conv2dRequest &q, hipStream_t stream) {
     p.wt = wt;
     p.y = q.y;
     p.N = q.N; p.C = Cp; p.H = q.H; p.W = q.W; p.K = q.K; p.R = q.R; p.S = q.S; p.P = q.P; p.Q = q.Q;
+    p.stride_h = q.stride_h; p.stride_w = q.stride_w; p.dil_h = q.dil_h; p.dil_w = q.dil_w;
     p.pad_h = q.pad_h; p.pad_w = q.pad_w;
     p.M = q.N * q.P * q.Q;
     p.xt_bytes = (unsigned)xt_bytes;
@@ -852,3 +898,7 @@ int conv2d_direct(const Conv2dRequest &q, hipStream_t stream) {
 }
 
 }  // namespace nt
+
+#ifdef NT_CONV_STAMPS
+extern "C" void nt_debug_conv_stamps(void *buffer) { nt::g_conv_stamps = (unsigned long long *)buffer; }
+#endif

@@ -237,7 +237,8 @@ hipError_t split_launch(const GemmProblem &q, hipStream_t stream) {
 }
 
 bool generic_accepts(const GemmProblem &q) {
-    if (q.batch != 1) return false;
+    if (q.batch < 1 || q.batch > 65535) return false;  // (the batch is the grid's y extent)
+    if (q.dtype == NINETOOTHED_FLOAT8_E5M2 && q.batch != 1) return false;
     if (q.dtype == NINETOOTHED_FLOAT8_E5M2)  // widened to fp16; addmm rounds its product to fp16, so it writes fp16
         return (q.out_dtype == NINETOOTHED_FLOAT16 || (q.out_dtype == NINETOOTHED_FLOAT32 && !q.addmm())) && q.m >= 0 && q.n >= 0 && q.k >= 0;
     if (q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16 && q.dtype != NINETOOTHED_FLOAT32) return false;
@@ -265,9 +266,13 @@ hipError_t generic_launch_typed(const GemmProblem &q, hipStream_t stream) {
     prob.sbn_ = q.sin;
     prob.alpha = q.alpha;
     prob.beta = q.beta;
+    prob.a_batch = q.a_batch;
+    prob.b_batch = q.b_batch;
+    prob.c_batch = q.c_batch;
+    prob.bias_batch = q.bias_batch;
     const int64_t tiles = (int64_t)ceil_div(q.m, kGenBM) * ceil_div(q.n, kGenBN);
     if (tiles == 0) return hipSuccess;  // empty launch is legal
-    gemm_generic_kernel<StridedProblem<T, TOut>><<<dim3((unsigned)tiles), dim3(kGenThreads), 0, stream>>>(prob);
+    gemm_generic_kernel<StridedProblem<T, TOut>><<<dim3((unsigned)tiles, (unsigned)q.batch), dim3(kGenThreads), 0, stream>>>(prob);
     return hipGetLastError();
 }
 
@@ -395,7 +400,7 @@ int heuristic_choice(const GemmProblem &q, int bm, int bn, int bk) {
     const auto few_tiles = [&](int instance) {
         const GemmInstance &inst = kInstances[instance];
         // (with a short K the second kernel costs more than the idle CUs: 512^3 8 us split, 5 in one pass)
-        return q.k >= 2048 && (int64_t)((q.m + inst.bm - 1) / inst.bm) * ((q.n + inst.bn - 1) / inst.bn) < 192 && inst.accepts(q);
+        return q.batch == 1 && q.k >= 2048 && (int64_t)((q.m + inst.bm - 1) / inst.bm) * ((q.n + inst.bn - 1) / inst.bn) < 192 && inst.accepts(q);
     };
     if (q.m <= 64 && few_tiles(kSplit64x64x64)) return kSplit64x64x64;
     if (few_tiles(kSplit128x128x64)) return kSplit128x128x64;
@@ -459,7 +464,7 @@ int build_problem(GemmProblem &q, const NineToothedTensor *input, const NineToot
 int run_gemm(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk) {
     if (q.m == 0 || q.n == 0) return 0;
     int choice = -1;
-    if (bm <= 0 || bn <= 0) choice = lookup_tuned(q);
+    if ((bm <= 0 || bn <= 0) && q.batch == 1) choice = lookup_tuned(q);  // (tuned choices are recorded for single products)
     if (choice < 0 || !kInstances[choice].accepts(q)) choice = heuristic_choice(q, bm, bn, bk);
     if (choice < 0) return NINETOOTHED_NO_KERNEL;
     note_launch(kLaunchGemm, choice, kInstances[choice].name);
@@ -486,6 +491,26 @@ NineToothedResult launch_nt_matmul(NineToothedStream stream, NineToothedTensor l
                                    int block_size_n, int block_size_k) {
     GemmProblem q;
     if (int err = build_problem(q, nullptr, lhs, rhs, nullptr, nullptr, output, dtype, output_dtype)) return err;
+    return run_gemm((hipStream_t)stream, q, block_size_m, block_size_n, block_size_k);
+}
+
+NineToothedResult launch_nt_batched_matmul(NineToothedStream stream, NineToothedTensor lhs, NineToothedTensor rhs,
+                                           NineToothedTensor output, int dtype, int output_dtype, int block_size_m,
+                                           int block_size_n, int block_size_k) {
+    if (!lhs.shape || !rhs.shape || !output.shape || !lhs.strides || !rhs.strides || !output.strides) return hipErrorInvalidValue;
+    const uint64_t batch = output.shape[0];
+    // an operand with a single matrix is shared by all products
+    if ((lhs.shape[0] != batch && lhs.shape[0] != 1) || (rhs.shape[0] != batch && rhs.shape[0] != 1)) return hipErrorInvalidValue;
+    if (batch > 0x7fffffffull) return NINETOOTHED_NO_KERNEL;
+    const NineToothedTensor a = {lhs.data, lhs.shape + 1, lhs.strides + 1}, b = {rhs.data, rhs.shape + 1, rhs.strides + 1},
+                            c = {output.data, output.shape + 1, output.strides + 1};
+    GemmProblem q;
+    if (int err = build_problem(q, nullptr, a, b, nullptr, nullptr, c, dtype, output_dtype)) return err;
+    if (batch == 0) return 0;
+    q.batch = (int)batch;
+    q.a_batch = lhs.shape[0] == 1 ? 0 : lhs.strides[0];
+    q.b_batch = rhs.shape[0] == 1 ? 0 : rhs.strides[0];
+    q.c_batch = output.strides[0];
     return run_gemm((hipStream_t)stream, q, block_size_m, block_size_n, block_size_k);
 }
 
@@ -620,17 +645,27 @@ enum ConvPath { kConvAuto = 0, kConvGather = 1, kConvRepack = 2, kConvDirect = 3
 
 // validates the call and fills the request; returns 0, an error, or -1 when there is nothing to compute
 int conv2d_request(Conv2dRequest &request, const NineToothedTensor &input, const NineToothedTensor &filter, const NineToothedTensor &output,
-                   int dtype, int padding_h, int padding_w) {
+                   int dtype, int padding_h, int padding_w, int stride_h = 1, int stride_w = 1, int dilation_h = 1, int dilation_w = 1) {
     if (dtype != NINETOOTHED_FLOAT16 && dtype != NINETOOTHED_BFLOAT16 && dtype != NINETOOTHED_FLOAT32) return NINETOOTHED_NO_KERNEL;
     if (!input.shape || !filter.shape || !output.shape || !input.strides || !filter.strides || !output.strides)
         return hipErrorInvalidValue;
-    if (padding_h < 0 || padding_w < 0) return hipErrorInvalidValue;
+    if (padding_h < 0 || padding_w < 0 || stride_h < 1 || stride_w < 1 || dilation_h < 1 || dilation_w < 1) return hipErrorInvalidValue;
     const int64_t N = (int64_t)input.shape[0], C = (int64_t)input.shape[1], H = (int64_t)input.shape[2], W = (int64_t)input.shape[3];
     const int64_t K = (int64_t)filter.shape[0], R = (int64_t)filter.shape[2], S = (int64_t)filter.shape[3];
     if ((int64_t)filter.shape[1] != C) return hipErrorInvalidValue;
-    const int64_t P = H + 2 * padding_h - R + 1, Q = W + 2 * padding_w - S + 1;
+    // Windows start every `stride` positions of the padded input, as many as the output has rows / columns: either the
+    // number that fit (floor, the usual convolution) or one more that hangs over the edge (the reference's
+    // `Tensor.tile` without `floor_mode`, src/ninetoothed/tensor.py:237-248; what hangs over reads as padding).
+    const int64_t span_h = H + 2 * padding_h - dilation_h * (R - 1) - 1, span_w = W + 2 * padding_w - dilation_w * (S - 1) - 1;
+    const int64_t P = (int64_t)output.shape[2], Q = (int64_t)output.shape[3];
     if ((int64_t)output.shape[0] != N || (int64_t)output.shape[1] != K) return hipErrorInvalidValue;
-    if ((int64_t)output.shape[2] != P || (int64_t)output.shape[3] != Q) return hipErrorInvalidValue;
+    if (span_h < 0 || span_w < 0) {
+        if (P > 0 && Q > 0) return hipErrorInvalidValue;  // the filter does not fit the padded input: no output positions
+    } else {
+        const int64_t fit_h = span_h / stride_h + 1, fit_w = span_w / stride_w + 1;
+        const int64_t over_h = (span_h + stride_h - 1) / stride_h + 1, over_w = (span_w + stride_w - 1) / stride_w + 1;
+        if ((P != fit_h && P != over_h) || (Q != fit_w && Q != over_w)) return hipErrorInvalidValue;
+    }
     if (P <= 0 || Q <= 0 || N == 0 || K == 0) return -1;  // nothing to write
     if (N * P * Q > 0x7fffffffll || C * R * S > 0x7fffffffll || K > 0x7fffffffll || N > 0x7fffffffll) return NINETOOTHED_NO_KERNEL;
     request.dtype = dtype;
@@ -640,6 +675,7 @@ int conv2d_request(Conv2dRequest &request, const NineToothedTensor &input, const
     request.N = (int)N; request.C = (int)C; request.H = (int)H; request.W = (int)W;
     request.K = (int)K; request.R = (int)R; request.S = (int)S; request.P = (int)P; request.Q = (int)Q;
     request.pad_h = padding_h; request.pad_w = padding_w;
+    request.stride_h = stride_h; request.stride_w = stride_w; request.dil_h = dilation_h; request.dil_w = dilation_w;
     for (int d = 0; d < 4; ++d) {
         request.xs[d] = input.strides[d];
         request.ws[d] = filter.strides[d];
@@ -660,6 +696,7 @@ hipError_t conv2d_gather(const Conv2dRequest &r, hipStream_t stream) {
     prob.C = r.C; prob.H = r.H; prob.W = r.W; prob.R = r.R; prob.S = r.S; prob.P = r.P; prob.Q = r.Q;
     prob.pad_h = r.pad_h;
     prob.pad_w = r.pad_w;
+    prob.stride_h = r.stride_h; prob.stride_w = r.stride_w; prob.dil_h = r.dil_h; prob.dil_w = r.dil_w;
     for (int d = 0; d < 4; ++d) {
         prob.xs[d] = r.xs[d];
         prob.ws[d] = r.ws[d];
@@ -674,7 +711,7 @@ hipError_t conv2d_gather(const Conv2dRequest &r, hipStream_t stream) {
 // the tensors as they lie (no repacking, no scratch memory).  NINETOOTHED_NO_KERNEL when the call is not that
 // or no one-pass GEMM instance of the fast kind takes it.
 int conv2d_pointwise(const Conv2dRequest &r, hipStream_t stream) {
-    if (!(r.R == 1 && r.S == 1 && r.pad_h == 0 && r.pad_w == 0 && r.xs[3] == 1 && r.xs[2] == r.W && r.ys[3] == 1 && r.ys[2] == r.Q && r.ws[1] == 1))
+    if (!(r.R == 1 && r.S == 1 && r.pad_h == 0 && r.pad_w == 0 && r.stride_h == 1 && r.stride_w == 1 && r.P == r.H && r.Q == r.W && r.xs[3] == 1 && r.xs[2] == r.W && r.ys[3] == 1 && r.ys[2] == r.Q && r.ws[1] == 1))
         return NINETOOTHED_NO_KERNEL;
     GemmProblem q;
     q.dtype = q.out_dtype = r.dtype;
@@ -756,6 +793,29 @@ NineToothedResult launch_nt_conv2d(NineToothedStream stream, NineToothedTensor i
     int result = conv2d_run(request, path, (hipStream_t)stream);
     // (a tuned path that needs scratch memory it cannot get, e.g. under graph capture: the library's order)
     if (result == NINETOOTHED_NO_KERNEL && path != kConvAuto && block_size_m == 0) result = conv2d_run(request, kConvAuto, (hipStream_t)stream);
+    return result;
+}
+
+NineToothedResult launch_nt_conv2d_strided(NineToothedStream stream, NineToothedTensor input, NineToothedTensor filter,
+                                           NineToothedTensor output, int dtype, int padding_h, int padding_w, int stride_h,
+                                           int stride_w, int dilation_h, int dilation_w, int block_size_m, int block_size_n,
+                                           int block_size_k) {
+    if (stride_h == 1 && stride_w == 1 && dilation_h == 1 && dilation_w == 1) {
+        Conv2dRequest plain;  // (an output with one more window than fits is not launch_nt_conv2d's problem)
+        const int status = conv2d_request(plain, input, filter, output, dtype, padding_h, padding_w);
+        if (status != 0) return status < 0 ? 0 : status;
+        if (plain.P == plain.H + 2 * padding_h - plain.R + 1 && plain.Q == plain.W + 2 * padding_w - plain.S + 1)
+            return launch_nt_conv2d(stream, input, filter, output, dtype, padding_h, padding_w, block_size_m, block_size_n, block_size_k);
+    }
+    (void)block_size_n;
+    (void)block_size_k;
+    Conv2dRequest request;
+    const int status = conv2d_request(request, input, filter, output, dtype, padding_h, padding_w, stride_h, stride_w, dilation_h, dilation_w);
+    if (status != 0) return status < 0 ? 0 : status;
+    // the ways that take windows with steps: 2 = repacking pass plus GEMM loop, 1 = gather kernel (nothing is tuned here)
+    const int path = block_size_m == kConvGather || block_size_m == kConvRepack ? block_size_m : kConvAuto;
+    int result = conv2d_run(request, path, (hipStream_t)stream);
+    if (result == NINETOOTHED_NO_KERNEL && path == kConvRepack) result = conv2d_run(request, kConvGather, (hipStream_t)stream);
     return result;
 }
 

@@ -25,6 +25,7 @@ constexpr int kGenThreads = 256;
 //   void load_a16(int row, int k0, elem out[16]) const;  // A[row][k0..k0+15], zero outside
 //   void load_b16(int col, int k0, elem out[16]) const;  // B[k0..k0+15][col], zero outside
 //   void store_c(int row, int col, float v) const;        // row < m, col < n guaranteed
+//   void select_batch(int index);                         // the grid's y coordinate: which of several independent products
 template <typename Problem>
 __global__ __launch_bounds__(kGenThreads) void gemm_generic_kernel(Problem prob) {
     typedef typename Problem::elem T;
@@ -34,6 +35,7 @@ __global__ __launch_bounds__(kGenThreads) void gemm_generic_kernel(Problem prob)
     __shared__ __attribute__((aligned(32))) T lds_a[kGenBM * kGenPitch];
     __shared__ __attribute__((aligned(32))) T lds_b[kGenBN * kGenPitch];
 
+    prob.select_batch((int)blockIdx.y);  // independent products of one launch: the operands move by the batch strides
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -131,6 +133,14 @@ struct StridedProblem {
     const T *bias;
     int64_t sam, sak, sbk, sbn, scm, scn, sbm_, sbn_;  // sbm_/sbn_: bias strides
     float alpha, beta;
+    int64_t a_batch, b_batch, c_batch, bias_batch;  // element strides between the products of a batched launch
+
+    NT_DEVICE void select_batch(int index) {
+        a += index * a_batch;
+        b += index * b_batch;
+        c += index * c_batch;
+        if (bias != nullptr) bias += index * bias_batch;
+    }
 
     NT_DEVICE void load_a16(int row, int k0, T out[16]) const {
         const T *src = a + (int64_t)row * sam + (int64_t)k0 * sak;
@@ -190,6 +200,8 @@ struct Fp8E5m2Problem {
     int64_t sam, sak, sbk, sbn, scm, scn, sbm_, sbn_;
     float alpha, beta;
 
+    NT_DEVICE void select_batch(int) {}
+
     static NT_DEVICE half_t widen(uint8_t byte) {
         const unsigned short bits = (unsigned short)((unsigned short)byte << 8);
         return __builtin_bit_cast(half_t, bits);
@@ -217,7 +229,7 @@ struct Fp8E5m2Problem {
     }
 };
 
-// ---- policy: conv2d as implicit GEMM (stride 1, dilation 1, zero padding) ----
+// ---- policy: conv2d as implicit GEMM (any window stride and dilation, zero padding) ----
 // GEMM row  = (image, out_y, out_x), GEMM k = (channel, filter_y, filter_x),
 // GEMM col  = output channel.
 template <typename T>
@@ -228,7 +240,10 @@ struct Conv2dProblem {
     const T *w;
     T *y;
     int C, H, W, R, S, P, Q, pad_h, pad_w;
+    int stride_h, stride_w, dil_h, dil_w;  // steps of the window over the input and between its taps
     int64_t xs[4], ws[4], ys[4];
+
+    NT_DEVICE void select_batch(int) {}
 
     NT_DEVICE void load_a16(int row, int k0, T out[16]) const {
         if (row >= m) {
@@ -247,8 +262,8 @@ struct Conv2dProblem {
         int fx = rs - fy * S;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const int iy = oy + fy - pad_h;
-            const int ix = ox + fx - pad_w;
+            const int iy = oy * stride_h + fy * dil_h - pad_h;
+            const int ix = ox * stride_w + fx * dil_w - pad_w;
             const bool ok = (k0 + i < k) && iy >= 0 && iy < H && ix >= 0 && ix < W;
             out[i] = ok ? base[(int64_t)c * xs[1] + (int64_t)iy * xs[2] + (int64_t)ix * xs[3]] : (T)0.0f;
             if (++fx == S) {

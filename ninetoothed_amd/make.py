@@ -263,7 +263,7 @@ class Kernel:
         out_tag = _dtype_tag(out.dtype)
         cast = self.details.get("cast")
         if tag == "fp8e5m2":  # the second case of the reference's tests/test_matmul.py:61-88
-            if kind == "conv2d" or out_tag not in ("fp16", "fp32") or cast not in (None, out_tag):
+            if kind in ("conv2d", "batched") or out_tag not in ("fp16", "fp32") or cast not in (None, out_tag):
                 raise UnsupportedProgram("fp8 operands are supported for plain matmul into fp16 / fp32 only.")
             return self._gemm_plan(info, tag, out_tag, positions=(None, 0, 1, None, None, 2))
         if kind == "conv2d":
@@ -274,7 +274,36 @@ class Kernel:
             raise UnsupportedProgram(f"The application rounds to `{cast}` but the output tensor holds `{out_tag}`.")
         if out_tag not in (tag, "fp32"):
             raise UnsupportedProgram(f"No matmul kernel writing `{out_tag}` from `{tag}` operands.")
+        if kind == "batched":
+            return self._batched_gemm_plan(info, tag, out_tag)
         return self._gemm_plan(info, tag, out_tag, positions=(None, 0, 1, None, None, 2))
+
+    def _batched_gemm_plan(self, info, tag, out_tag):
+        """One launch for all products of a batch (``launch_nt_batched_matmul``)."""
+        lib = runtime.library()
+        itemsize = 4 if tag == "fp32" else 2
+        out_itemsize = 4 if out_tag == "fp32" else 2
+        batch, m, n, k = info["batch"], info["m"], info["n"], info["k"]
+        blocks = [info["blocks"][axis] if info["blocks"][axis] > 1 else 0 for axis in ("m", "n", "k")]
+        dtype, out_dtype = runtime.DATA_TYPE_INDEX[tag], runtime.DATA_TYPE_INDEX[out_tag]
+
+        def layout(matrix, rows, cols, shared_allowed):
+            # (a dimension of one element has no coefficient in the index map: give it the stride of a dense matrix)
+            col_stride = matrix.col_stride if cols > 1 or matrix.col_stride else 1
+            row_stride = matrix.row_stride if rows > 1 or matrix.row_stride else (cols if col_stride == 1 else 1)
+            shared = shared_allowed and batch > 1 and matrix.batch_stride == 0  # one matrix for every product
+            return runtime.ArgumentTensor.from_layout(0, (1 if shared else batch, rows, cols), (matrix.batch_stride, row_stride, col_stride))
+
+        a, b, c = info["a"], info["b"], info["c"]
+        a_arg, b_arg, c_arg = layout(a, m, k, True), layout(b, k, n, True), layout(c, m, n, False)
+
+        def launch(call_args):
+            a_arg.data = call_args[0].data_ptr() + a.base * itemsize
+            b_arg.data = call_args[1].data_ptr() + b.base * itemsize
+            c_arg.data = call_args[2].data_ptr() + c.base * out_itemsize
+            runtime.check(lib.launch_nt_batched_matmul(runtime.current_stream(), a_arg, b_arg, c_arg, dtype, out_dtype, *blocks))
+
+        return _Plan(f"launch_nt_batched_matmul {batch}x{m}x{n}x{k} {tag}->{out_tag} blocks {blocks}", launch)
 
     def _prepare_addmm(self, args, env):
         input, mat1, mat2, beta, alpha, out = args
@@ -364,6 +393,17 @@ class Kernel:
         dtype = runtime.DATA_TYPE_INDEX[tag]
         pad_h, pad_w = info["pad_h"], info["pad_w"]
         blocks = [info["blocks"][axis] if info["blocks"][axis] > 1 else 0 for axis in ("m", "n", "k")]
+        steps = (info.get("stride_h", 1), info.get("stride_w", 1), info.get("dilation_h", 1), info.get("dilation_w", 1))
+        if steps != (1, 1, 1, 1) or not info.get("fits", True):
+            # windows that move by more than one position, taps that lie apart, or one window hanging over the edge
+
+            def launch_strided(call_args):
+                x, w, y = (runtime.ArgumentTensor.from_torch_tensor(tensor) for tensor in call_args)
+                runtime.check(lib.launch_nt_conv2d_strided(runtime.current_stream(), x, w, y, dtype, pad_h, pad_w, *steps, *blocks))
+
+            return _Plan(
+                f"launch_nt_conv2d_strided gemm {info['m']}x{info['n']}x{info['k']} {tag} padding ({pad_h}, {pad_w}) stride {steps[:2]} dilation {steps[2:]}", launch_strided
+            )
 
         from ninetoothed_amd import auto_tuner
 

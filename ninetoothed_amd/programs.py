@@ -57,6 +57,26 @@ class matmul:
 
     tensors = staticmethod(lambda: (Tensor(2), Tensor(2), Tensor(2)))
 
+    # The same application over a batch of products: tensors [B, M, K], [B, K, N], [B, M, N], the batch
+    # dimension tiled by 1 and squeezed out of the tiles, so that `lhs[k]` / `rhs[k]` / `output` are the
+    # matrices' blocks as before and the grid is (batch, blocks of M, blocks of N).
+    @staticmethod
+    def batched_arrangement(lhs, rhs, output, BLOCK_SIZE_M=BLOCK_SIZE_M, BLOCK_SIZE_N=BLOCK_SIZE_N, BLOCK_SIZE_K=BLOCK_SIZE_K):
+        output_arranged = output.tile((1, BLOCK_SIZE_M, BLOCK_SIZE_N))
+        output_arranged.dtype = output_arranged.dtype.squeeze(0)
+
+        lhs_arranged = lhs.tile((1, BLOCK_SIZE_M, BLOCK_SIZE_K)).tile((1, 1, -1)).expand((-1, -1, output_arranged.shape[2]))
+        lhs_arranged.dtype = lhs_arranged.dtype.squeeze((0, 1))
+        lhs_arranged.dtype.dtype = lhs_arranged.dtype.dtype.squeeze(0)
+
+        rhs_arranged = rhs.tile((1, BLOCK_SIZE_K, BLOCK_SIZE_N)).tile((1, -1, 1)).expand((-1, output_arranged.shape[1], -1))
+        rhs_arranged.dtype = rhs_arranged.dtype.squeeze((0, 2))
+        rhs_arranged.dtype.dtype = rhs_arranged.dtype.dtype.squeeze(0)
+
+        return lhs_arranged, rhs_arranged, output_arranged
+
+    batched_tensors = staticmethod(lambda: (Tensor(3), Tensor(3), Tensor(3)))
+
 
 class addmm:
     @staticmethod
@@ -195,13 +215,17 @@ class attention:
 
 class conv2d:
     @staticmethod
-    def arrangement(input, filter, output, enable_padding=True, BLOCK_SIZE_M=BLOCK_SIZE_M, BLOCK_SIZE_N=BLOCK_SIZE_N, BLOCK_SIZE_K=BLOCK_SIZE_K):
+    def arrangement(input, filter, output, enable_padding=True, BLOCK_SIZE_M=BLOCK_SIZE_M, BLOCK_SIZE_N=BLOCK_SIZE_N, BLOCK_SIZE_K=BLOCK_SIZE_K,
+                    stride=(1, 1), dilation=(1, 1), floor_mode=False):
+        """`stride`, `dilation`: steps of the window over the (padded) input and between its taps -- one more
+        argument to `tile` (src/ninetoothed/tensor.py:199-286).  With a stride, `floor_mode=True` gives the output
+        size of the usual convolution; `tile` otherwise adds a window that hangs over the edge."""
         if enable_padding:
             padding_h = Symbol("padding_h", constexpr=True)
             padding_w = Symbol("padding_w", constexpr=True)
             input = input.pad(((0, 0), (0, 0), (padding_h, padding_h), (padding_w, padding_w)))
 
-        input_tiled = input.tile((1, *filter.shape[1:]), strides=(-1, -1, 1, 1))
+        input_tiled = input.tile((1, *filter.shape[1:]), strides=(-1, -1, *stride), dilation=(1, 1, *dilation), floor_mode=floor_mode)
         input_squeezed = input_tiled.squeeze(1)
         input_squeezed.dtype = input_squeezed.dtype.squeeze(0)
         input_flattened = input_squeezed.ravel().flatten(end_dim=3).flatten(start_dim=1)

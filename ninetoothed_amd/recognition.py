@@ -250,6 +250,14 @@ class Operand:
         lo, hi = self.ranges.bounds[name]
         return hi - lo + 1
 
+    def rename(self, old, new):
+        """Gives a variable the name the operands of a program share (``b`` for a batch index)."""
+        self.ranges.bounds[new] = self.ranges.bounds.get(old, (0, 0))
+        self.extents[new] = self.extents.get(old, 1)
+        substitution = {old: Affine.var(new)}
+        self.indices = [self.ranges.rewrite(index, substitution) for index in self.indices]
+        self.constraints = [(self.ranges.rewrite(index, substitution), size) for index, size in self.constraints]
+
     def offset(self):
         total = Affine(0)
         for index, stride in zip(self.indices, self.source_strides):
@@ -289,9 +297,66 @@ def _strided(operand, row, col):
     return Strided2d(operand.extent(row), operand.extent(col), offset.const, offset.coef(row), offset.coef(col))
 
 
+class Strided3d(Strided2d):
+    """offset(batch, row, col) = base + batch * batch_stride + row * row_stride + col * col_stride."""
+
+    def __init__(self, batches, rows, cols, base, batch_stride, row_stride, col_stride):
+        super().__init__(rows, cols, base, row_stride, col_stride)
+        self.batches, self.batch_stride = batches, batch_stride
+
+
+def _strided_batched(operand, row, col):
+    if operand.constraints:
+        return None
+    offset = operand.offset()
+    if not offset.is_linear() or (offset.variables() - {"b", row, col}):
+        return None
+    return Strided3d(operand.extent("b"), operand.extent(row), operand.extent(col), offset.const, offset.coef("b"), offset.coef(row), offset.coef(col))
+
+
+def _analyze_batched_gemm(lhs, rhs, out):
+    """The matmul application under an arrangement with a leading batch dimension tiled by 1: grid
+    (batch, blocks of M, blocks of N), the operands' K blocks on a middle level (the batched product of
+    the reference's users; src/ninetoothed/generation.py:46-133 generates a kernel for any such
+    arrangement).  Returns ``("batched", {...})``."""
+    _level_shape(lhs, [3, 1, 2])
+    _level_shape(rhs, [3, 1, 2])
+    _level_shape(out, [3, 2])
+    operands = [lhs, rhs, out]
+    if any(operand.empty for operand in operands):
+        return "empty", {}
+    blocks = {}
+    blocks["m"] = lhs.fuse(lhs.names[0][1], lhs.names[2][0], "m")
+    blocks["k"] = lhs.fuse(lhs.names[1][0], lhs.names[2][1], "k")
+    rhs_block_k = rhs.fuse(rhs.names[1][0], rhs.names[2][0], "k")
+    blocks["n"] = rhs.fuse(rhs.names[0][2], rhs.names[2][1], "n")
+    if out.fuse(out.names[0][1], out.names[1][0], "m") != blocks["m"] or out.fuse(out.names[0][2], out.names[1][1], "n") != blocks["n"]:
+        raise UnsupportedProgram("Operands are tiled with different block sizes.")
+    if rhs_block_k != blocks["k"]:
+        raise UnsupportedProgram("`lhs` and `rhs` are tiled with different block sizes along K.")
+    for operand in operands:
+        operand.rename(operand.names[0][0], "b")
+        operand.settle()
+    lhs.require_absent(lhs.names[0][2])
+    rhs.require_absent(rhs.names[0][1])
+    if lhs.extents[lhs.names[1][0]] != rhs.extents[rhs.names[1][0]]:
+        raise UnsupportedProgram("`lhs` and `rhs` disagree on the number of K blocks.")
+    a, b, c = _strided_batched(lhs, "m", "k"), _strided_batched(rhs, "k", "n"), _strided_batched(out, "m", "n")
+    if not (a and b and c):
+        raise UnsupportedProgram("The operands of the batched product are not plain strided matrices per batch entry.")
+    if a.cols != b.rows:
+        raise UnsupportedProgram(f"Inner dimensions differ: {a.cols} and {b.rows}.")
+    batch, m, n, k = c.batches, c.rows, c.cols, a.cols
+    if a.rows < m or b.cols < n or a.batches != batch or b.batches != batch:
+        raise UnsupportedProgram("The output is larger than the product of the operands.")
+    return "batched", {"batch": batch, "m": m, "n": n, "k": k, "a": a, "b": b, "c": c, "blocks": blocks}
+
+
 def analyze_gemm(lhs_type, rhs_type, out_type, env, input_type=None):
-    """Returns ``("strided", {...})`` or ``("conv2d", {...})``."""
+    """Returns ``("strided", {...})``, ``("batched", {...})`` or ``("conv2d", {...})``."""
     lhs, rhs, out = Operand(lhs_type, env), Operand(rhs_type, env), Operand(out_type, env)
+    if input_type is None and len(out.names[0]) == 3:
+        return _analyze_batched_gemm(lhs, rhs, out)
     operands = [lhs, rhs, out]
     _level_shape(lhs, [2, 1, 2])
     _level_shape(rhs, [2, 1, 2])
@@ -345,8 +410,10 @@ def analyze_gemm(lhs_type, rhs_type, out_type, env, input_type=None):
 
 
 def _match_conv2d(lhs, rhs, out):
-    """Checks that lhs / rhs / out are the implicit-GEMM views of
-    x[N,C,H,W], w[K,C,R,S], y[N,K,P,Q] (stride 1, dilation 1, zero padding)."""
+    """Checks that lhs / rhs / out are the implicit-GEMM views of x[N,C,H,W], w[K,C,R,S], y[N,K,P,Q]: GEMM row
+    (image, out_y, out_x) and k (channel, f_y, f_x) read x[image, channel, out_y * stride_h + f_y * dilation_h -
+    pad_h, out_x * stride_w + f_x * dilation_w - pad_w], zero outside (`tile` with strides and dilation over the
+    padded input, src/ninetoothed/tensor.py:199-286)."""
 
     if len(lhs.indices) != 4 or len(rhs.indices) != 4 or len(out.indices) != 4:
         return None
@@ -356,7 +423,7 @@ def _match_conv2d(lhs, rhs, out):
     if C != C2 or N != N2 or K != K2 or min(P, Q, R, S) <= 0:
         return None
     pad_h, pad_w = -lhs.indices[2].const, -lhs.indices[3].const
-    if pad_h < 0 or pad_w < 0 or P != H + 2 * pad_h - R + 1 or Q != W + 2 * pad_w - S + 1:
+    if pad_h < 0 or pad_w < 0:
         return None
     if lhs.extent("m") != N * P * Q or lhs.extent("k") != C * R * S:
         return None
@@ -376,19 +443,48 @@ def _match_conv2d(lhs, rhs, out):
     def column(ranges):
         return Affine.var("n") if ranges.bounds["n"][1] > 0 else Affine(0)
 
+    def step(index, part):
+        """The factor `part` (an output coordinate or a tap coordinate) carries in a source index: the window's
+        stride or the dilation.  1 when the part is constant (a single position), None when it is not plain."""
+        if part.is_const():
+            return 1
+        if part.const != 0 or len(part.terms) != 1:
+            return None
+        (atom, unit), = part.terms.items()
+        factor = index.terms.get(atom, 0)
+        return factor // unit if unit and factor % unit == 0 and factor // unit >= 1 else None
+
     image, out_y, out_x = row_parts(lhs.ranges)
     channel, f_y, f_x = k_parts(lhs.ranges)
-    expected_x = [image, channel, out_y + f_y - pad_h, out_x + f_x - pad_w]
+    stride_h, dil_h = step(lhs.indices[2], out_y), step(lhs.indices[2], f_y)
+    stride_w, dil_w = step(lhs.indices[3], out_x), step(lhs.indices[3], f_x)
+    if None in (stride_h, dil_h, stride_w, dil_w):
+        return None
+    expected_x = [image, channel, out_y * stride_h + f_y * dil_h - pad_h, out_x * stride_w + f_x * dil_w - pad_w]
     channel, f_y, f_x = k_parts(rhs.ranges)
     expected_w = [column(rhs.ranges), channel, f_y, f_x]
     image, out_y, out_x = row_parts(out.ranges)
     expected_y = [image, column(out.ranges), out_y, out_x]
     if lhs.indices != expected_x or rhs.indices != expected_w or out.indices != expected_y:
         return None
-    allowed = [(expected_x[2], H), (expected_x[3], W)]
+    # windows: as many as fit, or one more that hangs over the edge (`tile` rounds up unless `floor_mode`)
+    fits = True
+    for size, pad, taps, dil, stride, count in ((H, pad_h, R, dil_h, stride_h, P), (W, pad_w, S, dil_w, stride_w, Q)):
+        span = size + 2 * pad - dil * (taps - 1) - 1
+        if span < 0 or count not in (span // stride + 1, -(-span // stride) + 1):
+            return None
+        fits = fits and count == span // stride + 1
+    # the masks of the source (and, implied by them, of the padded view a hanging window runs out of)
+    allowed = [(expected_x[2], H), (expected_x[3], W), (expected_x[2] + pad_h, H + 2 * pad_h), (expected_x[3] + pad_w, W + 2 * pad_w)]
     if any(constraint not in allowed for constraint in lhs.constraints) or rhs.constraints or out.constraints:
         return None
-    return {"pad_h": pad_h, "pad_w": pad_w, "m": N * P * Q, "n": K, "k": C * R * S}
+    required = [(expected_x[2], H), (expected_x[3], W)]
+    for constraint in required:
+        lo, hi = lhs.ranges.interval(constraint[0])
+        if (lo < 0 or hi >= constraint[1]) and constraint not in lhs.constraints:
+            return None  # positions outside the input must be masked (they read as zero)
+    return {"fits": fits, "pad_h": pad_h, "pad_w": pad_w, "stride_h": stride_h, "stride_w": stride_w, "dilation_h": dil_h, "dilation_w": dil_w,
+            "m": N * P * Q, "n": K, "k": C * R * S}
 
 
 def analyze_softmax(input_type, output_type, env):

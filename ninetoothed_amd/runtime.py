@@ -74,11 +74,13 @@ _S = ctypes.c_void_p
 _SIGNATURES = {
     "launch_nt_matmul": (_S, _T, _T, _T, _I, _I, _I, _I, _I),
     "launch_nt_matmul_static_scratch": (_S, _T, _T, _T, _I, _I, _I, _I, _I),
+    "launch_nt_batched_matmul": (_S, _T, _T, _T, _I, _I, _I, _I, _I),
     "launch_nt_addmm": (_S, _T, _T, _T, _T, _T, _T, _I, _I, _I, _I),
     "launch_nt_softmax": (_S, _T, _T, _I, _I),
     "launch_nt_softmax_config": (_S, _I, _T, _T, _I, _I),
     "launch_nt_attention": (_S, _T, _T, _T, _T, _T, _T, _I, _I, _I),
     "launch_nt_conv2d": (_S, _T, _T, _T, _I, _I, _I, _I, _I, _I),
+    "launch_nt_conv2d_strided": (_S, _T, _T, _T, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I),
     "launch_nt_gemm_config": (_S, _I, _T, _T, _T, _T, _T, _T, _I, _I),
     "nt_tune_gemm": (_S, _T, _T, _T, _T, _T, _T, _I, _I, _I, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_float)),
     "nt_tune_attention": (_S, _T, _T, _T, _T, _T, _T, _I, _I, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_float)),

@@ -187,15 +187,23 @@ def attention(q, k, v, is_causal=False, scale=None, bm=64, bn=32, dtype="fp16"):
     return out.reshape(q.shape)
 
 
-def conv2d(x, w, padding=(0, 0), bm=64, bn=64, bk=64, dtype="fp16"):
-    """conv2d (stride 1, dilation 1) through the implicit-GEMM arrangement."""
+def conv2d(x, w, padding=(0, 0), bm=64, bn=64, bk=64, dtype="fp16", stride=(1, 1), dilation=(1, 1), floor_mode=True):
+    """conv2d through the implicit-GEMM arrangement (reference tests/test_conv2d.py:13-48); `stride`, `dilation`
+    and `floor_mode` go to the `tile` that cuts the padded input into windows (src/ninetoothed/tensor.py:199-286:
+    without `floor_mode` the count of windows is rounded up, and what the last one reads beyond the padded input
+    is masked, i.e. zero)."""
     n, c, h, width = x.shape
     k, _, r, s = w.shape
     pad_h, pad_w = padding
-    p, q = h + 2 * pad_h - r + 1, width + 2 * pad_w - s + 1
+
+    def windows(size, pad, taps, spacing, step):
+        span = size + 2 * pad - spacing * (taps - 1) - 1
+        return max(span // step + 1 if floor_mode else -(-span // step) + 1, 0)
+
+    p, q = windows(h, pad_h, r, dilation[0], stride[0]), windows(width, pad_w, s, dilation[1], stride[1])
 
     x_view = View.of_shape(x.shape).pad(((0, 0), (0, 0), (pad_h, pad_h), (pad_w, pad_w)))
-    x_view = x_view.tile((1, c, r, s), strides=(-1, -1, 1, 1)).squeeze(1).squeeze(0, level=1)
+    x_view = x_view.tile((1, c, r, s), strides=(-1, -1, *stride), dilation=(1, 1, *dilation), floor_mode=floor_mode).squeeze(1).squeeze(0, level=1)
     x_view = x_view.ravel().flatten(end_dim=3).flatten(start_dim=1)
     w_view = View.of_shape(w.shape).flatten(start_dim=1).permute((1, 0))
     y_view = View.of_shape((n, k, p, q)).permute((0, 2, 3, 1)).flatten(end_dim=3)

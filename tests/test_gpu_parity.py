@@ -187,6 +187,67 @@ def test_transposed_rhs_on_the_fast_instances(m, n, k, dtype):
     assert torch.allclose(out.float(), product, **HALF_TOL)
 
 
+def _batched_matmul_kernel(application=programs.matmul.application, **blocks):
+    arrangement = functools.partial(programs.matmul.batched_arrangement, **blocks) if blocks else programs.matmul.batched_arrangement
+    return ninetoothed.make(arrangement, application, programs.matmul.batched_tensors())
+
+
+@pytest.mark.parametrize("batch, m, n, k", ((3, 300, 200, 100), (2, 64, 48, 8), (5, 1, 1, 1), (4, 256, 256, 64)))
+def test_batched_matmul_against_oracle(batch, m, n, k):
+    """The matmul application under an arrangement with a leading batch dimension: every batch entry is the
+    matmul program of the oracle; one launch of ``launch_nt_batched_matmul`` serves all of them."""
+    a, b = _randn(batch, m, k), _randn(batch, k, n)
+    out = torch.full((batch, m, n), float("nan"), dtype=torch.float16, device="cuda")
+    kernel = _batched_matmul_kernel()
+    kernel(a.cuda(), b.cuda(), out)
+    _native_only(kernel, "launch_nt_batched_matmul")
+    expected = np.stack([oracle.matmul(a[i].numpy(), b[i].numpy(), 64, 64, 64) for i in range(batch)])
+    assert np.allclose(out.cpu().float().numpy(), expected, **HALF_TOL)
+
+
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
+def test_batched_matmul_layouts_and_output_types(dtype):
+    from ninetoothed_amd import runtime
+
+    batch, m, n, k = 12, 1024, 768, 512
+    a, b = torch.randn(batch, m, k, dtype=dtype, device="cuda"), torch.randn(batch, k, n, dtype=dtype, device="cuda")
+    product = torch.bmm(a.float(), b.float())
+    kernel = _batched_matmul_kernel()
+    out = torch.full((batch, m, n), float("nan"), dtype=dtype, device="cuda")
+    kernel(a, b, out)
+    assert torch.allclose(out.float(), product, **HALF_TOL)
+    assert "any-stride" not in runtime.last_launch(), runtime.last_launch()  # dense operands: a direct-to-LDS instance
+    # fp32 output, fixed blocks
+    out32 = torch.full((batch, m, n), float("nan"), dtype=torch.float32, device="cuda")
+    _batched_matmul_kernel(BLOCK_SIZE_M=128, BLOCK_SIZE_N=128, BLOCK_SIZE_K=64)(a, b, out32)
+    assert torch.allclose(out32, product, rtol=1e-3, atol=1e-2)
+    # rhs stored [batch, n, k] (`x @ w.transpose(1, 2)`), an lhs shared by every product, an output inside a wider buffer
+    w = torch.randn(batch, n, k, dtype=dtype, device="cuda")
+    shared = a[:1].expand(batch, m, k)
+    wide = torch.full((batch, m, n + 8), 7.0, dtype=dtype, device="cuda")
+    kernel(shared, w.transpose(1, 2), wide[:, :, :n])
+    assert torch.allclose(wide[:, :, :n].float(), torch.bmm(shared.float(), w.transpose(1, 2).float()), **HALF_TOL)
+    assert bool((wide[:, :, n:] == 7.0).all())
+    # sizes that are no multiples of 8 and a batch order reversed by strides: the any-stride kernel, batch in the grid
+    a2, b2 = torch.randn(5, 77, 45, dtype=dtype, device="cuda"), torch.randn(5, 45, 51, dtype=dtype, device="cuda")
+    out2 = torch.full((5, 77, 51), float("nan"), dtype=dtype, device="cuda")
+    kernel(a2.flip(0), b2, out2)
+    assert torch.allclose(out2.float(), torch.bmm(a2.flip(0).float(), b2.float()), **HALF_TOL)
+    assert "any-stride" in runtime.last_launch(), runtime.last_launch()
+
+
+def test_batched_matmul_float32_operands_and_empty_batches():
+    a, b = torch.randn(3, 130, 70, device="cuda"), torch.randn(3, 70, 90, device="cuda")
+    out = torch.full((3, 130, 90), float("nan"), device="cuda")
+    kernel = _batched_matmul_kernel()
+    kernel(a, b, out)
+    assert torch.allclose(out, torch.bmm(a, b), rtol=1e-4, atol=1e-3)
+    empty = torch.empty(0, 130, 90, device="cuda")
+    kernel(a[:0], b[:0], empty)  # nothing to launch
+    with pytest.raises(ninetoothed.UnsupportedProgram):
+        kernel(a[:2], b, out)  # operands that disagree on the batch
+
+
 def test_matmul_empty_and_errors():
     kernel = _matmul_kernel()
     out = torch.empty(0, 16, dtype=torch.float16, device="cuda")
@@ -692,6 +753,79 @@ def test_conv2d_one_launch_path(n, c, h, w, k, r, s, padding, dtype):
     expected = F.conv2d(x.float(), weight.float(), padding=padding)
     assert torch.allclose(out.float(), expected, **HALF_TOL)
     assert bool((guard[n * k * p_out * q_out :] == 7.0).all())
+
+
+def _conv2d_with_steps(x, w, padding, stride, dilation, floor_mode=True, **blocks):
+    n, _, h, width = x.shape
+    k, _, r, s = w.shape
+
+    def windows(size, pad, taps, spacing, step):
+        span = size + 2 * pad - spacing * (taps - 1) - 1
+        return span // step + 1 if floor_mode else -(-span // step) + 1
+
+    p, q = windows(h, padding[0], r, dilation[0], stride[0]), windows(width, padding[1], s, dilation[1], stride[1])
+    out = torch.full((n, k, p, q), float("nan"), dtype=x.dtype, device=x.device)
+    arrangement = functools.partial(programs.conv2d.arrangement, stride=stride, dilation=dilation, floor_mode=floor_mode, **blocks)
+    kernel = ninetoothed.make(arrangement, programs.conv2d.application, programs.conv2d.tensors())
+    kernel(x, w, out, padding_h=padding[0], padding_w=padding[1])
+    _native_only(kernel, "launch_nt_conv2d")
+    return out, kernel
+
+
+@pytest.mark.parametrize("floor_mode", (True, False))
+@pytest.mark.parametrize("stride, dilation, padding", (((2, 2), (1, 1), (1, 1)), ((1, 2), (2, 1), (0, 1)), ((3, 1), (1, 2), (2, 2))))
+def test_conv2d_with_stride_and_dilation_against_oracle(stride, dilation, padding, floor_mode):
+    """`tile(..., strides, dilation)` in the conv2d arrangement (reference src/ninetoothed/tensor.py:199-286): the
+    HIP path against the oracle's arrangement-driven execution, both roundings of the number of windows."""
+    x = (torch.rand(2, 8, 11, 10) - 0.5).to(torch.float16)
+    w = (torch.rand(16, 8, 3, 2) - 0.5).to(torch.float16)
+    out, kernel = _conv2d_with_steps(x.cuda(), w.cuda(), padding, stride, dilation, floor_mode)
+    expected = oracle.conv2d(x.numpy(), w.numpy(), padding=padding, bm=32, bn=16, bk=16, stride=stride, dilation=dilation, floor_mode=floor_mode)
+    assert out.shape == expected.shape
+    assert np.allclose(out.cpu().float().numpy(), expected, **HALF_TOL)
+    if stride != (1, 1) or dilation != (1, 1):
+        assert kernel.last_plan.startswith("launch_nt_conv2d_strided")
+
+
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16, torch.float32))
+@pytest.mark.parametrize(
+    "n, c, h, w, k, r, s, padding, stride, dilation",
+    (
+        (8, 64, 56, 56, 128, 3, 3, (1, 1), (2, 2), (1, 1)),   # a down-sampling layer
+        (4, 256, 28, 28, 256, 3, 3, (2, 2), (1, 1), (2, 2)),  # a dilated layer
+        (4, 128, 30, 30, 256, 1, 1, (0, 0), (2, 2), (1, 1)),  # 1 x 1 with stride: not the batched product
+        (2, 3, 64, 64, 32, 7, 7, (3, 3), (2, 2), (1, 1)),     # a stem layer on three channels
+        (3, 20, 19, 23, 24, 3, 5, (1, 2), (2, 3), (2, 1)),
+    ),
+)
+def test_conv2d_with_stride_and_dilation_layer_shapes(n, c, h, w, k, r, s, padding, stride, dilation, dtype):
+    from ninetoothed_amd import runtime
+
+    x = _randn(n, c, h, w, dtype=dtype, scale=0.2).cuda()
+    weight = _randn(k, c, r, s, dtype=dtype, scale=0.2).cuda()
+    application = {torch.float16: programs.conv2d.application, torch.bfloat16: programs.matmul.application_with_bfloat16_cast, torch.float32: programs.matmul.application}[dtype]
+    expected = F.conv2d(x.float(), weight.float(), padding=padding, stride=stride, dilation=dilation)
+    out = torch.full(expected.shape, float("nan"), dtype=dtype, device="cuda")
+    arrangement = functools.partial(programs.conv2d.arrangement, stride=stride, dilation=dilation, floor_mode=True)
+    kernel = ninetoothed.make(arrangement, application, programs.conv2d.tensors())
+    for _ in range(2):
+        kernel(x, weight, out, padding_h=padding[0], padding_w=padding[1])
+    assert kernel.last_plan.startswith("launch_nt_conv2d_strided"), kernel.last_plan
+    tolerance = dict(rtol=1e-3, atol=1e-3) if dtype == torch.float32 else HALF_TOL
+    assert torch.allclose(out.float(), expected, **tolerance), float((out.float() - expected).abs().max())
+    if dtype != torch.float32 and k % 8 == 0 and c >= 2 and n * expected.shape[2] * expected.shape[3] >= 1024:
+        assert runtime.last_launch().startswith("conv2d path 2"), runtime.last_launch()  # the repacking way takes these
+    # each way by name through the C ABI
+    tag = runtime.DATA_TYPE_INDEX[{torch.float16: "fp16", torch.bfloat16: "bf16", torch.float32: "fp32"}[dtype]]
+    for path in (1, 2):
+        y = torch.full_like(out, float("nan"))
+        tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (x, weight, y)]
+        assert runtime.library().launch_nt_conv2d_strided(runtime.current_stream(), *tensors, tag, *padding, *stride, *dilation, path, 0, 0) == 0
+        assert torch.allclose(y.float(), expected, **tolerance), path
+    # an output of another size is refused
+    y = torch.empty(n, k, expected.shape[2] + 2, expected.shape[3], dtype=dtype, device="cuda")
+    tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (x, weight, y)]
+    assert runtime.library().launch_nt_conv2d_strided(runtime.current_stream(), *tensors, tag, *padding, *stride, *dilation, 0, 0, 0) == 1  # hipErrorInvalidValue
 
 
 def test_conv2d_one_launch_path_refuses_what_it_cannot_run():

@@ -105,6 +105,24 @@ def test_conv2d_against_torch(padding):
     assert np.allclose(out, expected, rtol=1e-3, atol=1e-3)
 
 
+@pytest.mark.parametrize("stride, dilation, padding", (((2, 2), (1, 1), (1, 1)), ((1, 2), (2, 1), (0, 1)), ((3, 1), (1, 2), (2, 2)), ((2, 3), (2, 2), (2, 0))))
+def test_conv2d_with_stride_and_dilation_against_torch(stride, dilation, padding):
+    """`tile(..., strides, dilation)` of the arrangement (reference src/ninetoothed/tensor.py:199-286): with
+    `floor_mode` the windows are those of `F.conv2d`; without it `tile` rounds the count up, and the extra
+    window equals what `F.conv2d` computes on an input that is zero-padded further at the bottom / right."""
+    x = torch.rand(2, 5, 11, 10).to(torch.float16)
+    w = torch.rand(4, 5, 3, 2).to(torch.float16)
+    out = oracle.conv2d(x.numpy(), w.numpy(), padding=padding, bm=16, bn=4, bk=8, stride=stride, dilation=dilation, floor_mode=True)
+    expected = F.conv2d(x.float(), w.float(), padding=padding, stride=stride, dilation=dilation).to(torch.float16).float().numpy()
+    assert out.shape == expected.shape
+    assert np.allclose(out, expected, rtol=1e-3, atol=1e-3)
+    hanging = oracle.conv2d(x.numpy(), w.numpy(), padding=padding, bm=16, bn=4, bk=8, stride=stride, dilation=dilation, floor_mode=False)
+    padded = F.pad(x.float(), (padding[1], padding[1] + stride[1], padding[0], padding[0] + stride[0]))
+    wider = F.conv2d(padded, w.float(), stride=stride, dilation=dilation).to(torch.float16).float().numpy()
+    assert hanging.shape[2] in (out.shape[2], out.shape[2] + 1) and hanging.shape[3] in (out.shape[3], out.shape[3] + 1)
+    assert np.allclose(hanging, wider[:, :, : hanging.shape[2], : hanging.shape[3]], rtol=1e-3, atol=1e-3)
+
+
 def test_conv2d_1x1_is_matmul():
     x = _half(2, 8, 4, 4)
     w = _half(6, 8, 1, 1)

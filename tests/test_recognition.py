@@ -99,6 +99,30 @@ def test_matmul_analysis_strided_and_ragged():
     assert info["blocks"] == {"m": 64, "n": 32, "k": 16}
 
 
+def test_batched_matmul_analysis():
+    """The matmul application under an arrangement with a leading batch dimension tiled by 1 is the
+    batched product: grid (batch, blocks of M, blocks of N), per operand a batch stride."""
+    kernel = ninetoothed.make(programs.matmul.batched_arrangement, programs.matmul.application, programs.matmul.batched_tensors())
+    assert kernel.kind == "matmul"
+    env = _env(kernel.types, [(5, 300, 100), (5, 100, 200), (5, 300, 200)], _metas(kernel))
+    kind, info = recognition.analyze_gemm(*kernel.types, env)
+    assert kind == "batched" and (info["batch"], info["m"], info["n"], info["k"]) == (5, 300, 200, 100)
+    assert (info["a"].batch_stride, info["a"].row_stride, info["a"].col_stride) == (30000, 100, 1)
+    assert (info["b"].batch_stride, info["b"].row_stride, info["b"].col_stride) == (20000, 200, 1)
+    assert (info["c"].batch_stride, info["c"].row_stride, info["c"].col_stride) == (60000, 200, 1)
+    # fixed blocks, a transposed rhs and an lhs that every product shares (batch stride 0, as `expand` gives)
+    arrangement = functools.partial(programs.matmul.batched_arrangement, BLOCK_SIZE_M=64, BLOCK_SIZE_N=32, BLOCK_SIZE_K=16)
+    kernel = ninetoothed.make(arrangement, programs.matmul.application, programs.matmul.batched_tensors())
+    env = _env(kernel.types, [(5, 300, 100), (5, 100, 200), (5, 300, 200)], strides=[[0, 100, 1], [20000, 1, 100], None])
+    kind, info = recognition.analyze_gemm(*kernel.types, env)
+    assert kind == "batched" and info["blocks"] == {"m": 64, "n": 32, "k": 16}
+    assert info["a"].batch_stride == 0 and (info["b"].row_stride, info["b"].col_stride) == (1, 100)
+    # operands that disagree on the batch
+    env = _env(kernel.types, [(4, 300, 100), (5, 100, 200), (5, 300, 200)])
+    with pytest.raises(recognition.UnsupportedProgram):
+        recognition.analyze_gemm(*kernel.types, env)
+
+
 def test_matmul_analysis_rejects_inconsistent_operands():
     kernel = ninetoothed.make(programs.matmul.arrangement, programs.matmul.application, programs.matmul.tensors())
     env = _env(kernel.types, [(64, 32), (48, 64), (64, 64)], _metas(kernel))
@@ -131,6 +155,33 @@ def test_conv2d_analysis(padding, blocks):
     assert kind == "conv2d"
     assert (info["pad_h"], info["pad_w"]) == padding
     assert (info["m"], info["n"], info["k"]) == (n * p * q, k, c * r * s)
+
+
+@pytest.mark.parametrize("floor_mode", (True, False))
+@pytest.mark.parametrize("stride, dilation, padding", (((2, 2), (1, 1), (1, 1)), ((1, 2), (2, 1), (0, 1)), ((3, 1), (1, 2), (2, 2))))
+def test_conv2d_analysis_with_stride_and_dilation(stride, dilation, padding, floor_mode):
+    """`tile(..., strides=(-1, -1, sh, sw), dilation=(1, 1, dh, dw))` in the conv2d arrangement is recognised, with
+    the output size of either rounding (`floor_mode` or the default, which adds a window hanging over the edge)."""
+    arrangement = functools.partial(programs.conv2d.arrangement, stride=stride, dilation=dilation, floor_mode=floor_mode)
+    kernel = ninetoothed.make(arrangement, programs.conv2d.application, programs.conv2d.tensors())
+    n, c, h, w, k, r, s = 2, 8, 17, 14, 16, 3, 3
+
+    def windows(size, pad, taps, spacing, step):
+        span = size + 2 * pad - spacing * (taps - 1) - 1
+        return span // step + 1 if floor_mode else -(-span // step) + 1
+
+    p, q = windows(h, padding[0], r, dilation[0], stride[0]), windows(w, padding[1], s, dilation[1], stride[1])
+    env = _env(kernel.types, [(n, c, h, w), (k, c, r, s), (n, k, p, q)], {**_metas(kernel), "padding_h": padding[0], "padding_w": padding[1]})
+    kind, info = recognition.analyze_gemm(*kernel.types, env)
+    assert kind == "conv2d"
+    assert (info["stride_h"], info["stride_w"], info["dilation_h"], info["dilation_w"]) == (*stride, *dilation)
+    assert (info["pad_h"], info["pad_w"]) == padding and (info["m"], info["n"], info["k"]) == (n * p * q, k, c * r * s)
+    fits = p == (h + 2 * padding[0] - dilation[0] * (r - 1) - 1) // stride[0] + 1 and q == (w + 2 * padding[1] - dilation[1] * (s - 1) - 1) // stride[1] + 1
+    assert info["fits"] == fits
+    # an output of another size is not that convolution
+    env = _env(kernel.types, [(n, c, h, w), (k, c, r, s), (n, k, p + 1, q)], {**_metas(kernel), "padding_h": padding[0], "padding_w": padding[1]})
+    with pytest.raises(ninetoothed.UnsupportedProgram):
+        recognition.analyze_gemm(*kernel.types, env)
 
 
 def test_conv2d_analysis_rejects_wrong_output_shape():
