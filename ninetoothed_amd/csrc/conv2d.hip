@@ -402,7 +402,11 @@ constexpr int kConvDirectMaxPeriod = 25;
 #define NT_CONV_ABLATE 0
 #endif
 
-template <typename T>
+// kM16: the tile is computed with 16x16x32 MFMAs (per FLOP half as many accumulator values pass through the
+// register file as with 32x32x16 ones, which is what the part's power limit charges for): per wave 4 blocks of
+// 16 channels, whose fragments stay in registers for a k tile (two sets taking turns), times 8 blocks of 16
+// pixels, whose fragments stream through four slots, each read two blocks ahead of its MFMAs.
+template <typename T, bool kM16>
 __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     typedef Elem<T> E;
@@ -448,14 +452,22 @@ __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams 
         else return (NT_LDS unsigned char *)lds_b3;
     };
 
+#ifdef NT_CONV_STAMPS
+    const unsigned long long real_entry = __builtin_amdgcn_s_memrealtime();
+#endif
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wave_m = wave % WM, wave_n = wave / WM;
 
     // ---- which tile ----
+    // The first and the last tile of pixels run the careful form of the loop, which is slower: both are dealt out first
+    // (workgroup ids 0 and 1 per tile of channels), so that a launch does not end with one of them.
     const int tile_ch = blockIdx.x % p.tiles_ch;
-    const int n0 = (blockIdx.x / p.tiles_ch) * BN;
+    const int pixel_tiles = (p.M + BN - 1) / BN;
+    int pixel_tile = blockIdx.x / p.tiles_ch;
+    if (pixel_tiles >= 3 && pixel_tile >= 1) pixel_tile = pixel_tile == 1 ? pixel_tiles - 1 : pixel_tile - 1;
+    const int n0 = pixel_tile * BN;
     const int tile_pixels = min(BN, p.M - n0);  // > 0 by construction of the grid
     const int m0 = tile_ch * BM;
     const int PQ = p.P * p.Q;
@@ -469,7 +481,7 @@ __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams 
 #pragma unroll
     for (int j = 0; j < kAInstr; ++j) {
         const int row = (j * kWaves + wave) * kARowsPerInstr + lane / kAChunksPerRow;
-        const int chunk = a_phys_chunk<BK>(row, lane % kAChunksPerRow);
+        const int chunk = kM16 ? a_phys_chunk16<BK>(row, lane % kAChunksPerRow) : a_phys_chunk<BK>(row, lane % kAChunksPerRow);
         a_src[j] = (unsigned)(row * p.CRS + chunk * 8) * 2u;
     }
     auto issue_filter = [&](auto stage_tag, int kt) {
@@ -527,6 +539,7 @@ __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams 
         const int r = rs / p.S, sx = rs - r * p.S;
         uint4_t entry;
         entry[0] = (unsigned)((c * (int)p.xs1 + r * (int)p.xs2 + sx) * 2);
+        if ((NT_CONV_ABLATE & 32) && sx != p.pad_w) entry[0] |= 0x80000000u;  // measurement: only the aligned taps fetch
         entry[1] = (unsigned)(31 - r);
         entry[2] = (sx < p.pad_w ? 0u : 0x0000ffffu) | (sx > p.S - 1 - p.pad_w ? 0u : 0xffff0000u);
         entry[3] = 0u;
@@ -536,9 +549,11 @@ __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams 
     const NT_LDS uint4_t *my_taps = (const NT_LDS uint4_t *)lds_taps + krow0;  // + 16 for the second row, + 32 per tile of the period
     int tap_tile = 0;        // position of the tile fetched next in its period (uniform)
     int period_base = 0;     // byte offset of that period's first channel (uniform)
-    const unsigned b_dst = (unsigned)(krow0 * kPitchB + piece * 16);  // the first piece in a stage; the second: 16 rows on
+    // (kM16: the four 16-lane groups of a transposing read fetch k rows 8 apart, so rows with bit 3 of k set lie another
+    // 32 bytes to the right -- inside the 64 spare bytes of a row -- and two groups served together do not meet in a bank)
+    const unsigned b_dst = (unsigned)(krow0 * kPitchB + (kM16 ? ((krow0 >> 3) & 1) * 32 : 0) + piece * 16);  // the first piece in a stage; the second: 16 rows on
     // fetches this thread's pieces of the next tile and moves on to the tile after it; `cols` keeps the rows' border masks
-    auto gather = [&](auto careful_tag, uint4_t (&regs)[kGather], unsigned (&cols)[kGather]) {
+    auto gather = [&](auto careful_tag, uint4_t (&regs)[kGather], unsigned (&cols)[kGather], int (&nudges)[kGather]) {
 #pragma unroll
         for (int j = 0; j < kGather; ++j) {
             const uint4_t entry = my_taps[tap_tile * BK + 16 * j];
@@ -548,27 +563,16 @@ __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams 
             const unsigned outside = (rows_outside << entry[1]) & 0x80000000u;
             int offset = (int)((unsigned)(lane_off + period_base + (int)entry[0]) | outside);
 
-            bool edge = false;  // the load would start below the tensor or end beyond it
-            if constexpr (decltype(careful_tag)::value) edge = !outside && (offset < 0 || (unsigned)(offset + 16) > p.x_bytes);
-            if (decltype(careful_tag)::value && __builtin_amdgcn_ballot_w64(edge) != 0) {  // uniform, and rare
-                // the lanes concerned load one pixel further in and move the pixels back by one place
+            if constexpr (decltype(careful_tag)::value) {
+                // A load that would start below the tensor or end beyond it (and is no load of zeros anyway) is moved one
+                // pixel further in; its pixels are moved back by one place when the piece is stored.  Every load of a
+                // careful tile goes this way, without a branch: the lanes that need no move shift by zero places.
+                const bool edge = !outside && (offset < 0 || (unsigned)(offset + 16) > p.x_bytes);
                 const int nudge = !edge ? 0 : (offset < 0 ? 1 : -1);
-                const uint4_t v = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, offset + 2 * nudge, 0, 0));
-                // byte selectors of v_perm_b32 over {high operand: bytes 4..7, low operand: bytes 0..3}
-                const unsigned up = nudge > 0 ? 0x05040302u : 0x07060504u;    // pixels move one place up: (v[i], v[i-1])
-                const unsigned down = nudge < 0 ? 0x05040302u : 0x03020100u;  // ... one place down: (v[i+1], v[i])
-                uint4_t w;
-                w[0] = __builtin_amdgcn_perm(v[0], 0u, up);
-                w[1] = __builtin_amdgcn_perm(v[1], v[0], up);
-                w[2] = __builtin_amdgcn_perm(v[2], v[1], up);
-                w[3] = __builtin_amdgcn_perm(v[3], v[2], up);
-                regs[j][0] = __builtin_amdgcn_perm(w[1], w[0], down);
-                regs[j][1] = __builtin_amdgcn_perm(w[2], w[1], down);
-                regs[j][2] = __builtin_amdgcn_perm(w[3], w[2], down);
-                regs[j][3] = __builtin_amdgcn_perm(0u, w[3], down);
-            } else {
-                regs[j] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, offset, 0, 0));
+                offset += 2 * nudge;
+                nudges[j] = nudge;
             }
+            regs[j] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, offset, 0, 0));
         }
         if (++tap_tile == p.period) {
             tap_tile = 0;
@@ -577,13 +581,28 @@ __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams 
     };
     // stores the pieces, the pixel that a shifted piece at an image border took from the neighbouring image row cleared
     // (keep_left always keeps the upper pixel of a dword, keep_right the lower one: the other half of a row's mask is inert)
-    auto scatter = [&](auto stage_tag, const uint4_t (&regs)[kGather], const unsigned (&cols)[kGather]) {
+    auto scatter = [&](auto careful_tag, auto stage_tag, const uint4_t (&regs)[kGather], const unsigned (&cols)[kGather], const int (&nudges)[kGather]) {
         NT_LDS unsigned char *sb = stage_b(stage_tag) + b_dst;
 #pragma unroll
         for (int j = 0; j < kGather; ++j) {
             uint4_t v = regs[j];
             // (the masking belongs here, two steps after the load: placed right behind the load it would wait for it)
             asm volatile("" : "+v"(v));
+            if constexpr (decltype(careful_tag)::value) {
+                // pixels of a piece that was loaded one pixel further in move back (byte selectors of v_perm_b32 over
+                // {high operand: bytes 4..7, low operand: bytes 0..3}); what falls off is a border pixel, cleared below
+                const unsigned up = nudges[j] > 0 ? 0x05040302u : 0x07060504u;    // one place up: (v[i], v[i-1])
+                const unsigned down = nudges[j] < 0 ? 0x05040302u : 0x03020100u;  // one place down: (v[i+1], v[i])
+                uint4_t w;
+                w[0] = __builtin_amdgcn_perm(v[0], 0u, up);
+                w[1] = __builtin_amdgcn_perm(v[1], v[0], up);
+                w[2] = __builtin_amdgcn_perm(v[2], v[1], up);
+                w[3] = __builtin_amdgcn_perm(v[3], v[2], up);
+                v[0] = __builtin_amdgcn_perm(w[1], w[0], down);
+                v[1] = __builtin_amdgcn_perm(w[2], w[1], down);
+                v[2] = __builtin_amdgcn_perm(w[3], w[2], down);
+                v[3] = __builtin_amdgcn_perm(0u, w[3], down);
+            }
             v[0] &= keep_left | cols[j];
             v[3] &= keep_right | cols[j];
             *(NT_LDS uint4_t *)(sb + j * (16 * kPitchB)) = v;
@@ -624,6 +643,22 @@ __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams 
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[ti][tj][r] = 0.0f;
 
+    // 16x16x32 form: channel block ti (16 channels) is one 16-byte read per lane (row i16, 16-byte chunk kg of the k
+    // tile); pixel block tj (16 pixels) is two transposing reads (16-lane group kg fetches k rows 8 kg .. + 7)
+    const int kg = lane >> 4;
+    constexpr int TM16 = kWaveM / 16, TN16 = kWaveN / 16;
+    const int a16_off = (wave_m * kWaveM + i16) * (BK * 2) + a_phys_chunk16<BK>(wave_m * kWaveM + i16, kg) * 16;  // + ti * 16 rows (the swizzle repeats)
+    const int b16_lo = (8 * kg + (i16 >> 2)) * kPitchB + (kg & 1) * 32 + (wave_n * kWaveN + 4 * (i16 & 3)) * 2;    // + tj * 32 bytes; + 4 rows for the upper half
+    auto read_a16 = [&](auto stage_tag, int ti) -> vec8 { return *(const NT_LDS vec8 *)(stage_a(stage_tag) + a16_off + ti * (16 * BK * 2)); };
+    auto read_b16 = [&](auto stage_tag, int tj) -> vec8 {
+        const NT_LDS unsigned char *sb = stage_b(stage_tag);
+        short4_t lo = lds_read_tr16_b64(sb + b16_lo + tj * 32);
+        short4_t hi = lds_read_tr16_b64(sb + b16_lo + 4 * kPitchB + tj * 32);
+        short8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        return __builtin_bit_cast(vec8, both);
+    };
+    float4_t acc16[kM16 ? TM16 : 1][kM16 ? TN16 : 1];  // (cleared after the prologue, whose loads borrow the registers)
+
     // ---- main loop ----
     // Tile t occupies stage t % 4.  The barrier that opens step t tells that tile t + 1 is complete in LDS (so
     // that the fragments of its first k step can be fetched during step t) and that every wave is done with
@@ -635,26 +670,76 @@ __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams 
 #ifdef NT_CONV_STAMPS
     unsigned long long stamp_loads = 0, stamp_lds = 0, stamp_sync = 0;
     const unsigned long long stamp_begin = __builtin_amdgcn_s_memtime();
+    const unsigned long long real_begin = __builtin_amdgcn_s_memrealtime();
 #endif
     uint4_t held[2][kGather];  // pieces in flight, by tile parity
     unsigned held_cols[2][kGather];  // their rows' border masks
+    int held_nudges[2][kGather];     // (careful tiles) by how many pixels a piece was loaded further in
     auto run = [&](auto careful_tag) {
         constexpr int kFrags = TN;
         // prologue: tiles 0 and 1 complete, the pieces of tiles 2 and 3 and the filter part of tile 2 in flight
-        issue_filter(std::integral_constant<int, 0>(), 0);
-        gather(careful_tag, held[0], held_cols[0]);
-        issue_filter(std::integral_constant<int, 1>(), min(1, last_k));
-        gather(careful_tag, held[1], held_cols[1]);
-        wait_vmcnt<0>();
-        scatter(std::integral_constant<int, 0>(), held[0], held_cols[0]);
-        scatter(std::integral_constant<int, 1>(), held[1], held_cols[1]);
-        gather(careful_tag, held[0], held_cols[0]);
-        issue_filter(std::integral_constant<int, 2>(), min(2, last_k));
-        gather(careful_tag, held[1], held_cols[1]);
+        // every load of the prologue is requested before the first one is waited for: the pieces of tiles 0 and 1 pass
+        // through registers that the accumulators take over afterwards
+        {
+            uint4_t first[2][kGather];
+            unsigned first_cols[2][kGather];
+            int first_nudges[2][kGather];
+            issue_filter(std::integral_constant<int, 0>(), 0);
+            gather(careful_tag, first[0], first_cols[0], first_nudges[0]);
+            issue_filter(std::integral_constant<int, 1>(), min(1, last_k));
+            gather(careful_tag, first[1], first_cols[1], first_nudges[1]);
+            gather(careful_tag, held[0], held_cols[0], held_nudges[0]);
+            issue_filter(std::integral_constant<int, 2>(), min(2, last_k));
+            gather(careful_tag, held[1], held_cols[1], held_nudges[1]);
+            wait_vmcnt<kAInstr + 2 * kGather>();  // (in flight: the pieces of tiles 2 and 3 and the filter part of tile 2)
+            scatter(careful_tag, std::integral_constant<int, 0>(), first[0], first_cols[0], first_nudges[0]);
+            scatter(careful_tag, std::integral_constant<int, 1>(), first[1], first_cols[1], first_nudges[1]);
+        }
+#pragma unroll
+        for (int ti = 0; ti < (kM16 ? TM16 : 1); ++ti)
+#pragma unroll
+            for (int tj = 0; tj < (kM16 ? TN16 : 1); ++tj) acc16[ti][tj] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
         vec8 af[2][TM];
         vec8 bf[2][TN];
+        vec8 ch[2][kM16 ? TM16 : 1];  // kM16: the channel fragments of a k tile, two sets taking turns
+        vec8 px[4];                   // ... and the slots the pixel fragments stream through
         lds_barrier();
-        read_frags(std::integral_constant<int, 0>(), 0, af[0], bf[0]);
+        if constexpr (kM16) {
+#pragma unroll
+            for (int ti = 0; ti < TM16; ++ti) ch[0][ti] = read_a16(std::integral_constant<int, 0>(), ti);
+            px[0] = read_b16(std::integral_constant<int, 0>(), 0);
+            px[1] = read_b16(std::integral_constant<int, 0>(), 1);
+        } else {
+            read_frags(std::integral_constant<int, 0>(), 0, af[0], bf[0]);
+        }
+        auto step16 = [&](auto s, auto parity_tag, int t) {
+            constexpr int kS = decltype(s)::value;
+            constexpr int kParity = decltype(parity_tag)::value;  // of t, t + 2 and t + 4; also the set of channel fragments in use
+            typedef std::integral_constant<int, (kS + 1) % kStages> NextStage;
+            constexpr int cur = kParity, nxt = cur ^ 1;
+            wait_vmcnt<kAInstr + kGather>();
+            lds_barrier();
+            if constexpr (!(NT_CONV_ABLATE & 2)) scatter(careful_tag, std::integral_constant<int, (kS + 2) % kStages>(), held[kParity], held_cols[kParity], held_nudges[kParity]);
+            if constexpr (!(NT_CONV_ABLATE & 1)) gather(careful_tag, held[kParity], held_cols[kParity], held_nudges[kParity]);
+            if constexpr (!(NT_CONV_ABLATE & 4)) issue_filter(std::integral_constant<int, (kS + 3) % kStages>(), min(t + 3, last_k));
+            static_for<0, TN16>([&](auto q_tag) {
+                constexpr int q = decltype(q_tag)::value;
+                // the pixel fragment two blocks ahead (of the next tile for the last two blocks) ...
+                if constexpr (q + 2 < TN16) px[(q + 2) % 4] = read_b16(s, q + 2);
+                else px[(q + 2) % 4] = read_b16(NextStage(), q + 2 - TN16);
+                // ... and, under the last blocks, the channel fragments of the next tile
+                constexpr bool kReadsChannels = q >= TN16 - TM16;
+                if constexpr (kReadsChannels) ch[nxt][q - (TN16 - TM16)] = read_a16(NextStage(), q - (TN16 - TM16));
+#pragma unroll
+                for (int ti = 0; ti < TM16; ++ti) acc16[ti][q] = E::mfma16(px[q % 4], ch[cur][ti], acc16[ti][q]);
+                constexpr int kReads = 2 + (kReadsChannels ? 1 : 0);
+                static_for<0, TM16>([&](auto j_tag) {
+                    constexpr int j = decltype(j_tag)::value;
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    if constexpr (j < kReads) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                });
+            });
+        };
         auto step = [&](auto s, auto parity_tag, int t) {
             constexpr int kS = decltype(s)::value;
             constexpr int kParity = decltype(parity_tag)::value;  // of t, t + 2 and t + 4
@@ -676,8 +761,8 @@ __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams 
             wait_vmcnt<kAInstr + kGather>();
             lds_barrier();
 #endif
-            if constexpr (!(NT_CONV_ABLATE & 2)) scatter(std::integral_constant<int, (kS + 2) % kStages>(), held[kParity], held_cols[kParity]);
-            if constexpr (!(NT_CONV_ABLATE & 1)) gather(careful_tag, held[kParity], held_cols[kParity]);
+            if constexpr (!(NT_CONV_ABLATE & 2)) scatter(careful_tag, std::integral_constant<int, (kS + 2) % kStages>(), held[kParity], held_cols[kParity], held_nudges[kParity]);
+            if constexpr (!(NT_CONV_ABLATE & 1)) gather(careful_tag, held[kParity], held_cols[kParity], held_nudges[kParity]);
             if constexpr (!(NT_CONV_ABLATE & 4)) issue_filter(std::integral_constant<int, (kS + 3) % kStages>(), min(t + 3, last_k));
             static_for<0, KS>([&](auto ks_tag) {
                 constexpr int ks = decltype(ks_tag)::value;
@@ -706,24 +791,23 @@ __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams 
         for (; t + 4 <= num_k; t += 4) {
             static_for<0, 4>([&](auto i_tag) {
                 constexpr int i = decltype(i_tag)::value;
-                step(std::integral_constant<int, i>(), std::integral_constant<int, i & 1>(), t + i);
+                if constexpr (kM16) step16(std::integral_constant<int, i>(), std::integral_constant<int, i & 1>(), t + i);
+                else step(std::integral_constant<int, i>(), std::integral_constant<int, i & 1>(), t + i);
             });
         }
         static_for<0, 3>([&](auto i_tag) {
             constexpr int i = decltype(i_tag)::value;
-            if (t + i < num_k) step(std::integral_constant<int, i>(), std::integral_constant<int, i & 1>(), t + i);
+            if (t + i < num_k) {
+                if constexpr (kM16) step16(std::integral_constant<int, i>(), std::integral_constant<int, i & 1>(), t + i);
+                else step(std::integral_constant<int, i>(), std::integral_constant<int, i & 1>(), t + i);
+            }
         });
     };
     if (careful_tile) run(std::true_type());  // (the first and the last tile of a launch)
     else run(std::false_type());
 #ifdef NT_CONV_STAMPS
-    if (p.stamps && lane == 0) {
-        unsigned long long *dst = p.stamps + ((size_t)blockIdx.x * kWaves + wave) * 4;
-        dst[0] = __builtin_amdgcn_s_memtime() - stamp_begin;
-        dst[1] = stamp_loads;
-        dst[2] = stamp_lds;
-        dst[3] = stamp_sync;
-    }
+    const unsigned long long stamp_loop_ticks = __builtin_amdgcn_s_memtime() - stamp_begin;
+    const unsigned long long real_loop_end = __builtin_amdgcn_s_memrealtime();
 #endif
 
     // ---- epilogue ----
@@ -745,6 +829,23 @@ __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams 
     const int slab_sw = l32 & (kCChunks - 1);
 #pragma unroll
     for (int ti = 0; ti < TM; ++ti) {
+        if constexpr (kM16) {
+            // 16 x 16 blocks: lane (i16, kg) holds, of channel i16, the pixels 4 kg .. + 3; two blocks of channels fill a slab
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const int row = half * 16 + i16;
+#pragma unroll
+                for (int tj = 0; tj < TN16; ++tj) {
+                    typedef T vec4 __attribute__((ext_vector_type(4)));
+                    const float4_t a4 = acc16[kM16 ? 2 * ti + half : 0][kM16 ? tj : 0];
+                    vec4 v;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = E::from_float(a4[e]);
+                    const int chunk = (tj * 2 + (kg >> 1)) ^ (row & (kCChunks - 1));
+                    *(NT_LDS vec4 *)(slab + row * kRowBytes + chunk * 16 + 8 * (kg & 1)) = v;
+                }
+            }
+        } else
 #pragma unroll
         for (int tj = 0; tj < TN; ++tj)
 #pragma unroll
@@ -771,6 +872,15 @@ __global__ __launch_bounds__(512, 2) void conv2d_direct_kernel(ConvDirectParams 
             __builtin_nontemporal_store(v, (vec8 *)(Y + ((int64_t)image * p.K + channel) * PQ + pq));
         }
     }
+#ifdef NT_CONV_STAMPS
+    if (p.stamps && lane == 0) {  // (100 MHz counter: loop, entry to loop, loop end to the last store issued)
+        unsigned long long *dst = p.stamps + ((size_t)blockIdx.x * kWaves + wave) * 4;
+        dst[0] = stamp_loop_ticks;
+        dst[1] = NT_CONV_STAMPS == 2 ? real_loop_end - real_begin : stamp_loads;
+        dst[2] = NT_CONV_STAMPS == 2 ? real_begin - real_entry : stamp_lds;
+        dst[3] = NT_CONV_STAMPS == 2 ? __builtin_amdgcn_s_memrealtime() - real_loop_end : stamp_sync;
+    }
+#endif
 #endif
 }
 
@@ -817,7 +927,16 @@ int run_direct(const Conv2dRequest &q, hipStream_t stream) {
 #ifdef NT_CONV_STAMPS
     p.stamps = g_conv_stamps;
 #endif
-    conv2d_direct_kernel<T><<<dim3((unsigned)grid), dim3(512), 0, stream>>>(p);
+    // 16x16x32 MFMAs draw less power per FLOP and finish a tile sooner (at [32, 256, 56, 56] * [256, 256, 3, 3]: 55 against
+    // 59 us per tile), but the careful form of that loop -- the first and the last tile of pixels -- runs out of registers
+    // and is slower than the 32x32x16 one (92 against 80 us): with more tiles than compute units those two are dealt out
+    // first and the others hide them; a launch of a single round would wait for them.
+    int units = compute_units();
+#ifdef NT_CONV_M32
+    units = 0;
+#endif
+    if (units > 0 && grid > units) conv2d_direct_kernel<T, true><<<dim3((unsigned)grid), dim3(512), 0, stream>>>(p);
+    else conv2d_direct_kernel<T, false><<<dim3((unsigned)grid), dim3(512), 0, stream>>>(p);
     return (int)hipGetLastError();
 }
 

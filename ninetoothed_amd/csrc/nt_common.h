@@ -125,6 +125,19 @@ inline bool stream_is_capturing(hipStream_t stream) {
     return status != hipStreamCaptureStatusNone;
 }
 
+// Compute units of the current device (looked up once per device; 0 when it cannot be told).
+inline int compute_units() {
+    static int cached[64] = {};  // (written with the same value by whoever comes first: no lock needed)
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 0;
+    int units = __atomic_load_n(&cached[device], __ATOMIC_RELAXED);
+    if (units == 0) {
+        if (hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || units <= 0) units = -1;
+        __atomic_store_n(&cached[device], units, __ATOMIC_RELAXED);
+    }
+    return units > 0 ? units : 0;
+}
+
 struct Scalar0d {
     static double as_double(const NineToothedTensor &t) { return *(const double *)t.data; }
     static int64_t as_int64(const NineToothedTensor &t) { return *(const int64_t *)t.data; }
