@@ -41,7 +41,14 @@ struct AttentionParams {
     int parts, blocks_per_part;
     float *part_o;    // [parts][batch * heads][seq_q][D]
     float *part_lse;  // [parts][batch * heads][seq_q]
+#ifdef NT_ATTN_STAMPS
+    unsigned long long *stamps;  // measurement builds: per wave {entry to loop, loop, epilogue} in 10 ns units and the loop in clocks
+#endif
 };
+
+#ifdef NT_ATTN_STAMPS
+unsigned long long *g_attn_stamps = nullptr;
+#endif
 
 constexpr int kAttnWaves = 4;
 
@@ -82,6 +89,9 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
         else return (NT_LDS unsigned char *)lds_v1;
     };
 
+#ifdef NT_ATTN_STAMPS
+    const unsigned long long real_entry = __builtin_amdgcn_s_memrealtime();
+#endif
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -153,13 +163,25 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
                     raw[4 + e] = E::from_float(hi[e] * p.q_scale);
                 }
             } else {
-                raw = *(const vec8 *)(src + ks * 16 + 8 * g);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) raw[e] = E::from_float(E::to_float(raw[e]) * p.q_scale);
+                raw = *(const vec8 *)(src + ks * 16 + 8 * g);  // (scaled below, once the first K blocks have been requested)
             }
             qf[qt][ks] = raw;
         }
     }
+    // Q' = round(Q * scale * log2 e).  Called after the first K / V blocks have been requested, so that the queries and
+    // those blocks are on their way at the same time (the multiplication is the first thing that waits for the queries).
+    auto scale_queries = [&]() __attribute__((always_inline)) {
+        if constexpr (!std::is_same<TIO, float>::value) {
+#pragma unroll
+            for (int qt = 0; qt < kQTiles; ++qt)
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    if (kPadded && ks * 16 + 8 * g >= p.head_dim) continue;  // (zeros stay zeros)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) qf[qt][ks][e] = E::from_float(E::to_float(qf[qt][ks][e]) * p.q_scale);
+                }
+        }
+    };
 
     // ---- number of kv blocks this query block needs ----
     int kv_end = p.seq_k;
@@ -281,6 +303,11 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
         for (int r = 0; r < 16; ++r) c_init[qt][r] = 0.0f;
     }
 
+#ifdef NT_ATTN_STAMPS
+    asm volatile("" ::"v"(qf[0][0]));  // (the queries have arrived)
+    const unsigned long long real_loop = __builtin_amdgcn_s_memrealtime();
+    const unsigned long long tick_loop = __builtin_amdgcn_s_memtime();
+#endif
     // S^T = K . Q'^T for the block held in a K stage
     auto scores = [&](auto stage_tag, float16_t (&s_acc)[KT][kQTiles]) __attribute__((always_inline)) {
         const NT_LDS unsigned char *sk = stage_k(stage_tag);
@@ -499,6 +526,7 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
         if (num_blocks > first_block) {
             issue_k(Stage0(), first_block);
             issue_v(Stage0(), first_block);
+            scale_queries();
             for (int blk = first_block; blk < num_blocks; blk += 2) {
                 wait_vmcnt<0>();
                 lds_barrier();
@@ -528,6 +556,7 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
             float alpha[kQTiles];
             issue_k(Stage0(), 0);
             issue_k(Stage1(), min(1, last_block));
+            scale_queries();
             wait_vmcnt<kInstr>();
             lds_barrier();
             scores(Stage0(), s_buf[0]);
@@ -706,6 +735,10 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
         }
     }
 
+#ifdef NT_ATTN_STAMPS
+    const unsigned long long real_epilogue = __builtin_amdgcn_s_memrealtime();
+    const unsigned long long tick_epilogue = __builtin_amdgcn_s_memtime();
+#endif
     // ---- epilogue: O[q, d] = O^T[d, q] / l ----
     if constexpr (kSplitKV) {
 #pragma unroll
@@ -730,6 +763,60 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
         }
         return;
     }
+    // A lane holds four consecutive columns of one query row at a time, so stores straight from the registers put
+    // 8 bytes into each of 32 rows per instruction.  Where the workgroup's K / V stages have room for one 32-row
+    // tile of O per wave (BN >= 32 always holds one or more whole tiles per stage), the tile goes through them instead (16-byte chunks of a row exchanged by the row number,
+    // so that neither side meets bank conflicts) and leaves in whole rows: 16 bytes per lane, 64 lanes on
+    // consecutive addresses.
+    constexpr int kChunks = D / 8;
+    constexpr bool kStagedStore = !kPadded && std::is_same<TIO, T>::value && (kChunks & (kChunks - 1)) == 0 && kChunks <= 64 &&
+                                  kWaves * 32 * D * 2 <= 4 * kTileBytes;
+    if constexpr (kStagedStore) {
+        typedef TIO vec4 __attribute__((ext_vector_type(4)));
+        typedef unsigned uint4_t __attribute__((ext_vector_type(4)));
+        constexpr int kSwizzle = (kChunks < 16 ? kChunks : 16) - 1;
+        constexpr int kRowsPerStore = 64 / kChunks;
+        lds_barrier();  // every wave has read its last V block
+        // the addresses of this exchange are derived from copies of the lane and wave numbers that the compiler
+        // cannot trace back, or it computes them before the loop and the loop pays for the registers they hold
+        int late_lane = lane, late_wave = wave;
+        asm volatile("" : "+v"(late_lane), "+s"(late_wave));
+        const int late_l32 = late_lane & 31, late_g = late_lane >> 5;
+        // (the four stages stay separate arrays: the compiler orders a read of one stage behind the fills of
+        // another only if it cannot tell them apart)
+        constexpr int kTilesPerStage = kTileBytes / (32 * D * 2);
+        const int stage = late_wave / kTilesPerStage;
+        NT_LDS unsigned char *tile = (NT_LDS unsigned char *)(stage == 0 ? lds_k0 : stage == 1 ? lds_v0 : stage == 2 ? lds_k1 : lds_v1) +
+                                     (late_wave % kTilesPerStage) * (32 * D * 2);
+        NT_LDS unsigned char *put = tile + late_l32 * (D * 2) + late_g * 8;
+        const int get_row = late_lane / kChunks, get_chunk = late_lane % kChunks;
+#pragma unroll
+        for (int qt = 0; qt < kQTiles; ++qt) {
+            const float l_total = l_run[qt] + __shfl_xor(l_run[qt], 32, 64);
+            const float inv = 1.0f / l_total;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    vec4 out;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) out[e] = E::from_float(o_acc[dt][qt][r4 * 4 + e] * inv);
+                    *(NT_LDS vec4 *)(put + (((dt * 4 + r4) ^ (late_l32 & kSwizzle)) * 16)) = out;
+                }
+            // (the LDS serves a wave's requests in order; the fence only keeps the compiler from moving them)
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            const int tile_row0 = q0 + (late_wave * kQTiles + qt) * 32;
+#pragma unroll
+            for (int i = 0; i < 32 / kRowsPerStore; ++i) {
+                const int row = i * kRowsPerStore + get_row;
+                const uint4_t chunk = *(NT_LDS const uint4_t *)(tile + row * (D * 2) + ((get_chunk ^ (row & kSwizzle)) * 16));
+                if (tile_row0 + row < p.seq_q) *(uint4_t *)(O + (int64_t)(tile_row0 + row) * p.o_strides[2] + get_chunk * 8) = chunk;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        }
+    } else
 #pragma unroll
     for (int qt = 0; qt < kQTiles; ++qt) {
         const float l_total = l_run[qt] + __shfl_xor(l_run[qt], 32, 64);
@@ -753,6 +840,15 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
                 }
         }
     }
+#ifdef NT_ATTN_STAMPS
+    if (p.stamps && lane == 0) {
+        unsigned long long *dst = p.stamps + ((size_t)blockIdx.x * kWaves + wave) * 4;
+        dst[0] = real_loop - real_entry;
+        dst[1] = real_epilogue - real_loop;
+        dst[2] = __builtin_amdgcn_s_memrealtime() - real_epilogue;
+        dst[3] = tick_epilogue - tick_loop;
+    }
+#endif
 #endif
 }
 
@@ -1132,6 +1228,9 @@ int attention_setup(AttentionParams &p, const NineToothedTensor &q, const NineTo
     if (scale.data) p.q_scale = (float)Scalar0d::as_double(scale) * 1.44269504089f;
     else p.q_scale = dtype == NINETOOTHED_FLOAT16 ? 1.4423828125f : (dtype == NINETOOTHED_BFLOAT16 ? 1.4453125f : 1.44269504089f);
     p.causal = is_causal.data ? (Scalar0d::as_int64(is_causal) != 0) : 0;
+#ifdef NT_ATTN_STAMPS
+    p.stamps = g_attn_stamps;
+#endif
     return 0;
 }
 
@@ -1230,3 +1329,7 @@ extern "C" NineToothedResult nt_tune_attention(NineToothedStream stream, NineToo
     if (best_ms) *best_ms = best_time;
     return 0;
 }
+
+#ifdef NT_ATTN_STAMPS
+extern "C" void nt_debug_attention_stamps(void *buffer) { nt::g_attn_stamps = (unsigned long long *)buffer; }
+#endif
