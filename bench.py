@@ -406,9 +406,13 @@ def main():
             if name == args.workload or name in ("copy_1gib", "mfma_ceiling_constant"):
                 continue
             workload = factory()
-            ms, _ = measure(workload, max(5, args.steps // 2), args.warmup)
+            ms, wall = measure(workload, max(5, args.steps // 2), args.warmup)
             entry = roofline(workload, ms, traffic.get(name))
             entry["ms_per_step"] = ms
+            # a step that the device finishes sooner than the host can ask for the next one (the 512^3 product)
+            # is timed at the host's pace: the wall time says so, the single launches give the kernel's own time
+            entry["wall_ms_per_step"] = wall
+            entry["per_launch"] = per_launch(workload)
             entry["config"] = dict(workload["describe"], launch=launch_description(workload))
             others[name] = entry
             vendor_line(name, workload, max(5, args.steps // 2))

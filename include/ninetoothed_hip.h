@@ -349,9 +349,16 @@ NineToothedResult nt_tune_conv2d(NineToothedStream stream,
  * 2 = conv2d: dtype, N, C, H, W, K, R, S, padding_h, padding_w, dense input);
  * a choice line starts with the variant (GEMM instance index, attention variant,
  * conv2d path) and may go on with descriptive integers (the GEMM instance's
- * block M, N, K).  Both act on the table of the current device. */
+ * block M, N, K).  Both act on the table of the current device.
+ * The default pair's choice line holds nt_tune_file_format(), a number that changes with the numbering of the
+ * variants: loading ignores a file that holds another one (0 entries, no error), and it drops every choice that
+ * the program does not recognise -- a GEMM instance index without this build's block M, N, K of that instance
+ * next to it, an attention variant or conv2d path outside the range.  (The reference's reader takes any line
+ * pair, src/ninetoothed/templates/auto_tuning_cache.h:52-75; its files are bound to one build by a fingerprint
+ * in build.py:619-662 instead.) */
 NineToothedResult nt_tune_cache_save(const char *path);
 NineToothedResult nt_tune_cache_load(const char *path, int *entries);
+int nt_tune_file_format(void);
 
 /* The cached GEMM instance for a problem with a row-major rhs, or -1. */
 int nt_tune_cache_lookup(int dtype, int output_dtype, int m, int n, int k, int addmm);

@@ -1137,6 +1137,9 @@ const char *const kAttentionVariantNames[kAttentionVariants] = {
     "software-pipelined loop, 64-key blocks, eight waves (256 query rows), one workgroup per CU",
 };
 
+bool attention_choice_known(int index, const int *, int) { return index >= 0 && index < kAttentionVariants; }
+const bool g_attention_check_registered = tune_register_check(kTuneAttention, attention_choice_known);
+
 template <typename T>
 int dispatch_attention(AttentionParams &p, int head_dim, int variant, hipStream_t stream) {
     if (head_dim == 32) note_launch(kLaunchAttention, 0, "plain loop, 64-key blocks, head dimension 32");

@@ -351,6 +351,7 @@ const GemmInstance kInstances[] = {
     {#BM "x" #BN "x" #BK " waves " #WM "x" #WN " stages " #ST " ABLATED " #AB " (wrong results)", BM, BN, BK, fast_accepts<BM, BN, BK, ST>, fast_launch<BM, BN, BK, WM, WN, ST, OCC, AB>}
     NT_LOAD_INSTANCE(256, 256, 32, 2, 4, 4, 2, 1, 0),
     NT_LOAD_INSTANCE(256, 256, 32, 2, 2, 4, 1, 1, 0),
+    NT_LOAD_INSTANCE(256, 256, 32, 2, 2, 5, 1, 1, 0),
     NT_LOAD_INSTANCE(256, 256, 64, 2, 2, 2, 1, 1, 0),
     NT_LOAD_INSTANCE(128, 256, 32, 1, 4, 3, 2, 1, 0),
     NT_ABLATED_INSTANCE(256, 256, 32, 2, 4, 4, 2, 1),
@@ -362,6 +363,13 @@ constexpr int kNumInstances = sizeof(kInstances) / sizeof(kInstances[0]);
 static_assert(kNumInstances > kSplit256x256x32, "InstanceIndex names the first instances of the table");
 
 inline bool is_split(int instance) { return instance >= kSplit64x64x64 && instance <= kSplit256x256x32; }
+
+// choices read from a tuning file: an instance index counts only together with the block sizes saved next to it
+bool gemm_choice_known(int index, const int *extra, int extras) {
+    return index >= 0 && index < kNumInstances && extras == 3 && extra[0] == kInstances[index].bm && extra[1] == kInstances[index].bn &&
+           extra[2] == kInstances[index].bk;
+}
+const bool g_gemm_check_registered = tune_register_check(kTuneGemm, gemm_choice_known);
 
 // ---- tuned choices: (dtype, output dtype, M, N, K, addmm, rhs layout) -> instance ----
 void tune_values(const GemmProblem &q, int (&values)[7]) {
@@ -642,6 +650,8 @@ namespace {
 // the ways to run a convolution; kConvAuto tries them from the top (a 1 x 1 filter without padding first runs
 // as a batch of plain products when it can)
 enum ConvPath { kConvAuto = 0, kConvGather = 1, kConvRepack = 2, kConvDirect = 3, kConvPointwise = 4 };
+bool conv2d_choice_known(int index, const int *, int) { return index >= kConvGather && index <= kConvPointwise; }
+const bool g_conv2d_check_registered = tune_register_check(kTuneConv2d, conv2d_choice_known);
 
 // validates the call and fills the request; returns 0, an error, or -1 when there is nothing to compute
 int conv2d_request(Conv2dRequest &request, const NineToothedTensor &input, const NineToothedTensor &filter, const NineToothedTensor &output,

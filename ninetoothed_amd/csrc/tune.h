@@ -19,6 +19,16 @@ int tune_lookup(int kind, const int *values, int count);
 // (`extra`: up to three descriptive integers kept with the choice and written after it to the cache file)
 void tune_record(int kind, const int *values, int count, int choice, const int *extra = nullptr, int extras = 0);
 
+// A choice read from a file is taken over only if the program's own source still knows it: each program registers,
+// from a static initialiser, a function that says whether (index, descriptive integers) names one of its variants
+// as this build numbers them.  Programs without such a function accept any index >= 0.
+typedef bool (*TuneChoiceCheck)(int index, const int *extra, int extras);
+bool tune_register_check(int kind, TuneChoiceCheck check);
+
+// Written into the default pair of a saved file and compared on load: raised whenever the numbering of the GEMM
+// instances, attention variants or conv2d paths changes, so that a file from another numbering is ignored whole.
+constexpr int kTuneFileFormat = 3;
+
 // Which kernel served the latest launch_nt_* call of the calling host thread: the launch functions leave a note
 // (three thread-local stores), nt_last_launch formats it.  `name` must point to a string that lives as long as
 // the library (a literal or an instance table entry).

@@ -68,6 +68,16 @@ void tune_record(int kind, const int *values, int count, int choice, const int *
 }
 
 namespace {
+TuneChoiceCheck g_checks[kTuneKinds] = {};
+}  // namespace
+
+bool tune_register_check(int kind, TuneChoiceCheck check) {
+    if (kind < 0 || kind >= kTuneKinds) return false;
+    g_checks[kind] = check;
+    return true;
+}
+
+namespace {
 thread_local int t_launch_program = kLaunchNone;
 thread_local int t_launch_choice = -1;
 thread_local const char *t_launch_name = nullptr;
@@ -98,19 +108,21 @@ NineToothedResult nt_last_launch(char *buffer, int size) {
 
 int nt_tune_lookup(int kind, const int *values, int count) { return tune_lookup(kind, values, count); }
 
+int nt_tune_file_format(void) { return kTuneFileFormat; }
+
 // On-disk form: the line-pair CSV the reference's AutoTuningCache reads
 // (src/ninetoothed/templates/auto_tuning_cache.h:27-75; written by src/ninetoothed/build.py:683-703): a line of
 // integers describing the problem, then a line of integers with the choice; the first pair has an empty problem
 // line and carries a default.  A problem line is the program (0 = matmul / addmm, 1 = attention, 2 = conv2d)
 // followed by the problem's values; a choice line is the variant's index followed by optional descriptive
-// integers (the GEMM instances add their block sizes).
+// integers (the GEMM instances add their block sizes).  The default pair's choice line holds kTuneFileFormat.
 NineToothedResult nt_tune_cache_save(const char *path) {
     if (path == nullptr) return hipErrorInvalidValue;
     int device = 0;
     (void)hipGetDevice(&device);
     FILE *file = fopen(path, "w");
     if (file == nullptr) return hipErrorInvalidValue;
-    fprintf(file, "\n0\n");
+    fprintf(file, "\n%d\n", kTuneFileFormat);
     {
         std::shared_lock<std::shared_mutex> lock(g_mutex);
         for (const auto &entry : g_choices) {
@@ -127,8 +139,10 @@ NineToothedResult nt_tune_cache_save(const char *path) {
 }
 
 // Reads such a file into the table of the current device.  *entries (may be NULL) receives the number of choices
-// taken over; lines that do not parse are skipped.  A choice that names a variant this build does not have is
-// harmless: the launch functions check a looked-up choice before they use it.
+// taken over; lines that do not parse are skipped.  A file whose default pair does not hold this build's
+// kTuneFileFormat is ignored whole (0 entries, no error), and so is every choice that the program it belongs to
+// does not recognise (a GEMM instance index whose block sizes differ from the ones written next to it): the
+// numbering of the variants may differ between builds, and a stale choice would be a valid but slow kernel.
 NineToothedResult nt_tune_cache_load(const char *path, int *entries) {
     if (entries) *entries = 0;
     if (path == nullptr) return hipErrorInvalidValue;
@@ -156,6 +170,7 @@ NineToothedResult nt_tune_cache_load(const char *path, int *entries) {
         const bool parsed = parse(problem_line, problem) && parse(choice_line, choice);
         if (first) {  // the default pair
             first = false;
+            if (!parsed || choice.empty() || choice[0] != kTuneFileFormat) break;
             continue;
         }
         if (!parsed || problem.empty() || choice.empty() || problem.size() > (size_t)kTuneMaxValues + 1) continue;
@@ -166,6 +181,8 @@ NineToothedResult nt_tune_cache_load(const char *path, int *entries) {
         int extra[3] = {0, 0, 0};
         const int extras = (int)std::min<size_t>(choice.size() - 1, 3);
         for (int i = 0; i < extras; ++i) extra[i] = (int)choice[i + 1];
+        const TuneChoiceCheck check = g_checks[problem[0]];
+        if (check != nullptr && !check((int)choice[0], extra, extras)) continue;
         tune_record((int)problem[0], values, count, (int)choice[0], extra, extras);
         ++taken;
     }

@@ -92,6 +92,7 @@ _SIGNATURES = {
     "nt_tune_cache_save": (ctypes.c_char_p,),
     "nt_tune_cache_load": (ctypes.c_char_p, ctypes.POINTER(ctypes.c_int)),
     "nt_tune_cache_lookup": (_I, _I, _I, _I, _I, _I),
+    "nt_tune_file_format": (),
     "nt_gemm_num_configs": (),
     "nt_gemm_config_name": (_I, ctypes.c_char_p, _I),
 }

@@ -87,15 +87,24 @@ def test_tuning_cache_reads_and_writes_the_reference_csv_format(tmp_path):
     names = runtime.gemm_config_names()
     fast = next(index for index, name in enumerate(names) if name.startswith("256x256x32"))
     fp16 = runtime.DATA_TYPE_INDEX["fp16"]
+    file_format = lib.nt_tune_file_format()
     path = tmp_path / "cache.csv"
     with open(path, "w") as handle:
         writer = csv.writer(handle)
         writer.writerow(())
-        writer.writerow((0,))
+        writer.writerow((file_format,))
         writer.writerow((runtime.TUNE_GEMM, fp16, fp16, 4096, 2048, 1024, 1, 0))
         writer.writerow((fast, 256, 256, 32))
         writer.writerow((runtime.TUNE_GEMM, fp16, fp16, 4096, 2048, 1024, 1, 1))  # the same sizes with a transposed rhs
         writer.writerow((fast + 1, 256, 256, 64))
+        writer.writerow((runtime.TUNE_GEMM, fp16, fp16, 1024, 1024, 1024, 0, 0))
+        writer.writerow((fast, 128, 128, 64))  # block sizes of another instance: a file from another numbering, dropped
+        writer.writerow((runtime.TUNE_GEMM, fp16, fp16, 2048, 1024, 1024, 0, 0))
+        writer.writerow((fast,))  # no block sizes: dropped
+        writer.writerow((runtime.TUNE_ATTENTION, fp16, 4, 32, 2048, 2048, 128, 1))
+        writer.writerow((99,))  # no such variant: dropped
+        writer.writerow((runtime.TUNE_CONV2D, fp16, 32, 256, 28, 28, 256, 3, 3, 1, 1, 1))
+        writer.writerow((0,))  # no such path: dropped
         writer.writerow((runtime.TUNE_ATTENTION, fp16, 4, 32, 4096, 4096, 128, 1))
         writer.writerow((3,))
         writer.writerow((runtime.TUNE_CONV2D, fp16, 32, 256, 56, 56, 256, 3, 3, 1, 1, 1))
@@ -110,6 +119,10 @@ def test_tuning_cache_reads_and_writes_the_reference_csv_format(tmp_path):
     assert lib.nt_tune_cache_lookup(fp16, fp16, 4096, 2048, 1024, 1) == fast
     assert auto_tuner.lookup(fp16, fp16, 4096, 2048, 1024, True, rhs_layout=1) == fast + 1
     assert lib.nt_tune_cache_lookup(fp16, fp16, 64, 64, 64, 0) == -1
+    assert lib.nt_tune_cache_lookup(fp16, fp16, 1024, 1024, 1024, 0) == -1
+    assert lib.nt_tune_cache_lookup(fp16, fp16, 2048, 1024, 1024, 0) == -1
+    assert auto_tuner.lookup_problem(runtime.TUNE_ATTENTION, (fp16, 4, 32, 2048, 2048, 128, 1)) == -1
+    assert auto_tuner.lookup_problem(runtime.TUNE_CONV2D, (fp16, 32, 256, 28, 28, 256, 3, 3, 1, 1, 1)) == -1
     assert lib.nt_tune_cache_lookup(fp16, fp16, 4096, 2048, 1024, 0) == -1
     assert auto_tuner.lookup_problem(runtime.TUNE_ATTENTION, (fp16, 4, 32, 4096, 4096, 128, 1)) == 3
     assert auto_tuner.lookup_problem(runtime.TUNE_ATTENTION, (fp16, 4, 32, 4096, 4096, 128, 0)) == -1
@@ -118,12 +131,24 @@ def test_tuning_cache_reads_and_writes_the_reference_csv_format(tmp_path):
     saved = tmp_path / "saved.csv"
     assert lib.nt_tune_cache_save(str(saved).encode()) == 0
     rows = list(csv.reader(open(saved)))
-    assert rows[0] == [] and len(rows[1]) == 1  # the default pair
+    assert rows[0] == [] and rows[1] == [str(file_format)]  # the default pair carries the numbering's format
     pairs = {tuple(rows[i]): tuple(rows[i + 1]) for i in range(2, len(rows) - 1, 2)}
     assert pairs[tuple(str(v) for v in (0, fp16, fp16, 4096, 2048, 1024, 1, 0))] == (str(fast), "256", "256", "32")
     assert pairs[tuple(str(v) for v in (1, fp16, 4, 32, 4096, 4096, 128, 1))] == ("3",)
     assert pairs[tuple(str(v) for v in (2, fp16, 32, 256, 56, 56, 256, 3, 3, 1, 1, 1))] == ("2",)
     assert lib.nt_tune_cache_load(str(tmp_path / "missing.csv").encode(), None) != 0
+
+    # a file written under another numbering of the variants is ignored whole
+    other = tmp_path / "other_format.csv"
+    with open(other, "w") as handle:
+        writer = csv.writer(handle)
+        writer.writerow(())
+        writer.writerow((file_format - 1,))
+        writer.writerow((runtime.TUNE_GEMM, fp16, fp16, 512, 1024, 2048, 0, 0))
+        writer.writerow((fast, 256, 256, 32))
+    assert lib.nt_tune_cache_load(str(other).encode(), ctypes.byref(entries)) == 0
+    assert entries.value == 0
+    assert lib.nt_tune_cache_lookup(fp16, fp16, 512, 1024, 2048, 0) == -1
 
 
 def test_auto_tuner_json_caches(tmp_path):
