@@ -421,8 +421,11 @@ int heuristic_choice(const GemmProblem &q, int bm, int bn, int bk) {
     for (const Rule &rule : rules) {
         const GemmInstance &inst = kInstances[rule.instance];
         if (!inst.accepts(q)) continue;
-        const int64_t tiles = (int64_t)((q.m + inst.bm - 1) / inst.bm) * ((q.n + inst.bn - 1) / inst.bn) * q.batch;
-        if (tiles >= rule.min_tiles) return rule.instance;
+        const int64_t per_matrix = (int64_t)((q.m + inst.bm - 1) / inst.bm) * ((q.n + inst.bn - 1) / inst.bn);
+        // (a batch of small matrices reaches any number of tiles: a tile that such a matrix fills to less than
+        // 60 % is left to the rules of the second pass, which start from the small tiles)
+        if (q.batch > 1 && rule.min_tiles > 1 && (int64_t)q.m * q.n * 5 < per_matrix * inst.bm * inst.bn * 3) continue;
+        if (per_matrix * q.batch >= rule.min_tiles) return rule.instance;
     }
     return kInstances[kAnyStride].accepts(q) ? kAnyStride : -1;
 }
