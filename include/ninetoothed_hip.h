@@ -20,7 +20,8 @@
  * parts x batch x heads x seq_q x (head_dim + 1) floats; not when the caller
  * passes block sizes), and launch_nt_matmul / launch_nt_addmm on problems with few
  * output tiles and a long K (split-K: parts x M x N floats, at most 64 MiB; not
- * when the caller passes block sizes) use scratch device memory: one buffer per (device, stream,
+ * when the caller passes block sizes) or on FLOAT8_E5M2 operands (fp16 copies of the operands, and of addmm's
+ * input: 2 bytes per element) use scratch device memory: one buffer per (device, stream,
  * purpose) that the library allocates (hipMalloc) the first time a call needs
  * it, grows (hipFree + hipMalloc, which wait for the device) when a later call
  * needs more, and otherwise reuses, so that steady-state calls allocate
@@ -65,7 +66,12 @@ enum NineToothedDataType {
     /* extension beyond the reference's enum: 8-bit floating point with 5 exponent
      * and 2 mantissa bits, the operand type of the second case of
      * tests/test_matmul.py:61-88 and tests/test_addmm.py:57-90; accepted by
-     * launch_nt_matmul and launch_nt_addmm (input, mat1, mat2 fp8, output fp16) */
+     * launch_nt_matmul and launch_nt_addmm (input, mat1, mat2 fp8, output fp16).
+     * An e5m2 value is the upper byte of the fp16 value it equals: the operands are
+     * widened exactly into fp16 copies in the stream's scratch buffers and the product runs
+     * on the fp16 kernels (products exact, sums in fp32); without scratch memory (graph
+     * capture before an eager call of the same size) a kernel that widens while it loads
+     * serves the call, much slower. */
     NINETOOTHED_FLOAT8_E5M2
 };
 

@@ -15,11 +15,15 @@
 
 namespace nt {
 
-enum WorkspacePurpose { kWorkspaceConvInput, kWorkspaceConvFilter, kWorkspaceAttentionNarrow, kWorkspaceGemmParts, kWorkspaceAttentionParts, kWorkspacePurposes };
+enum WorkspacePurpose {
+    kWorkspaceConvInput, kWorkspaceConvFilter, kWorkspaceAttentionNarrow, kWorkspaceGemmParts, kWorkspaceAttentionParts,
+    kWorkspaceGemmWidenedLhs, kWorkspaceGemmWidenedRhs, kWorkspaceGemmWidenedBias, kWorkspacePurposes
+};
 
 // Holds the registry lock from construction to destruction: create it, take the buffers,
 // enqueue every kernel that uses them, then let it go.  Two host threads that launch on the
-// same stream then cannot interleave their kernels on a shared buffer.
+// same stream then cannot interleave their kernels on a shared buffer.  A thread may hold
+// several leases at once (a caller that keeps its own buffers alive across a call that takes more).
 class WorkspaceLease {
 public:
     explicit WorkspaceLease(hipStream_t stream);

@@ -14,7 +14,7 @@ struct Buffer {
     size_t bytes = 0;
 };
 
-std::mutex g_mutex;
+std::recursive_mutex g_mutex;
 std::map<std::tuple<int, hipStream_t, int>, Buffer> g_buffers;
 
 }  // namespace
@@ -53,7 +53,7 @@ void *WorkspaceLease::get(WorkspacePurpose purpose, size_t bytes) {
 }  // namespace nt
 
 extern "C" void nt_release_workspaces(void) {
-    std::lock_guard<std::mutex> lock(nt::g_mutex);
+    std::lock_guard<std::recursive_mutex> lock(nt::g_mutex);
     for (auto &entry : nt::g_buffers) {
         if (entry.second.data != nullptr) (void)hipFree(entry.second.data);
     }

@@ -1175,6 +1175,58 @@ def test_matmul_float8_e5m2_operands(m, n, k):
 
 
 @pytest.mark.skipif(not hasattr(torch, "float8_e5m2"), reason="this torch has no float8_e5m2")
+def test_matmul_float8_e5m2_large_products_run_on_widened_copies():
+    """fp8 operands are widened into fp16 copies (exact) and the product runs on the fp16 instances, direct-to-LDS
+    where the copies allow: every layout the copies have to follow, against the fp32 product of the widened operands
+    and against the widening any-stride kernel named through the C ABI."""
+    from ninetoothed_amd import runtime
+
+    lib = runtime.library()
+    fp8, fp16, fp32 = (runtime.DATA_TYPE_INDEX[name] for name in ("fp8e5m2", "fp16", "fp32"))
+    null = runtime.ArgumentTensor.null()
+    kernel = ninetoothed.make(programs.matmul.arrangement, programs.matmul.application, programs.matmul.tensors())
+
+    def check(lhs, rhs, out_dtype=torch.float16, fast=True):
+        m, n = lhs.shape[0], rhs.shape[1]
+        out = torch.full((m, n), float("nan"), dtype=out_dtype, device="cuda")
+        kernel(lhs, rhs, out)
+        _native_only(kernel, "launch_nt_matmul")
+        assert ("any-stride" not in runtime.last_launch()) == fast, runtime.last_launch()
+        product = lhs.to(torch.float16).float() @ rhs.to(torch.float16).float()
+        k = lhs.shape[1]
+        assert torch.allclose(out.float(), product, rtol=1e-2, atol=1e-2 * (k / 512) ** 0.5)
+        plain = torch.full_like(out, float("nan"))
+        tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (lhs, rhs, plain)]
+        assert lib.launch_nt_gemm_config(runtime.current_stream(), 0, null, tensors[0], tensors[1], null, null, tensors[2], fp8, fp32 if out_dtype == torch.float32 else fp16) == 0
+        assert torch.allclose(out.float(), plain.float(), rtol=1e-2, atol=1e-2 * (k / 512) ** 0.5)
+
+    m, n, k = 2048, 1024, 1024
+    lhs = torch.randn(m, k, device="cuda").to(torch.float8_e5m2)
+    rhs = torch.randn(k, n, device="cuda").to(torch.float8_e5m2)
+    check(lhs, rhs)                                      # both row-major
+    check(lhs, rhs, out_dtype=torch.float32)
+    check(lhs, torch.randn(n, k, device="cuda").to(torch.float8_e5m2).T)   # the reference's case: the rhs column-major
+    check(torch.randn(k, m, device="cuda").to(torch.float8_e5m2).T, rhs, fast=False)  # a column-major lhs: copies follow it, the any-stride fp16 kernel runs
+    # operands inside wider buffers, rows that start off 16-byte boundaries (byte-wise widening)
+    wide = torch.randn(m + 3, k + 5, device="cuda").to(torch.float8_e5m2)
+    lhs2 = wide[3:, 5:]
+    lhs2.view(torch.uint8)[0, 0] = 0x5C  # 256.0
+    check(lhs2, rhs)
+    # sizes that are no multiples of 8: the copies get padded rows, the any-stride fp16 kernel runs on them
+    check(torch.randn(2050, 1030, device="cuda").to(torch.float8_e5m2), torch.randn(1030, 1001, device="cuda").to(torch.float8_e5m2), fast=False)
+    # addmm: the bias is widened as well (tests/test_addmm.py:57-90 of the reference at a larger size)
+    bias = torch.randn(m, n, device="cuda").to(torch.float8_e5m2)
+    rhs_t = torch.randn(n, k, device="cuda").to(torch.float8_e5m2).T
+    out = torch.full((m, n), float("nan"), dtype=torch.float16, device="cuda")
+    addmm = ninetoothed.make(programs.addmm.arrangement, programs.addmm.application, programs.addmm.tensors())
+    addmm(bias, lhs, rhs_t, 0.37, 0.81, out)
+    _native_only(addmm, "launch_nt_addmm")
+    assert "any-stride" not in runtime.last_launch(), runtime.last_launch()
+    product = (lhs.to(torch.float16).float() @ rhs_t.to(torch.float16).float()).half().float()
+    assert torch.allclose(out.float(), 0.37 * bias.to(torch.float16).float() + 0.81 * product, rtol=1e-2, atol=2e-2 * (k / 512) ** 0.5)
+
+
+@pytest.mark.skipif(not hasattr(torch, "float8_e5m2"), reason="this torch has no float8_e5m2")
 def test_addmm_float8_e5m2_operands():
     # tests/test_addmm.py:57-90 of the reference: fp8 input, mat1, mat2 (the last column-major), fp16 output
     m, n, k = 512, 512, 512
