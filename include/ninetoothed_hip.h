@@ -20,8 +20,9 @@
  * parts x batch x heads x seq_q x (head_dim + 1) floats; not when the caller
  * passes block sizes), and launch_nt_matmul / launch_nt_addmm on problems with few
  * output tiles and a long K (split-K: parts x M x N floats, at most 64 MiB; not
- * when the caller passes block sizes) or on FLOAT8_E5M2 operands (fp16 copies of the operands, and of addmm's
- * input: 2 bytes per element) use scratch device memory: one buffer per (device, stream,
+ * when the caller passes block sizes), on FLOAT8_E5M2 operands (fp16 copies of the operands, and of addmm's
+ * input: 2 bytes per element) or, from 2^31 multiply-adds on, on fp16 / bf16 operands that the direct-to-LDS kernels
+ * cannot read in place (dense copies, (M + N) x K elements) use scratch device memory: one buffer per (device, stream,
  * purpose) that the library allocates (hipMalloc) the first time a call needs
  * it, grows (hipFree + hipMalloc, which wait for the device) when a later call
  * needs more, and otherwise reuses, so that steady-state calls allocate
@@ -310,7 +311,10 @@ NineToothedResult launch_nt_gemm_config(NineToothedStream stream, int config,
  * than 2 % faster.  This call synchronises.  Returns 0 and the winner in
  * *best_config, its time per launch in *best_ms.  On a stream that is being
  * captured into a graph nothing is timed or recorded: returns 0 with
- * *best_config = -1. */
+ * *best_config = -1.  A problem that a single instance takes (fp32 or fp8 operands; fp16 / bf16 operands that the
+ * direct-to-LDS instances cannot read in place -- a K that is no multiple of 8, rows off 16-byte boundaries, an lhs
+ * stored by columns: launch_nt_matmul / launch_nt_addmm run those on dense copies from 2^31 multiply-adds on) has
+ * nothing to time: returns 0 with *best_config = -2 and records nothing. */
 NineToothedResult nt_tune_gemm(NineToothedStream stream,
                                NineToothedTensor input,
                                NineToothedTensor mat1,
@@ -350,8 +354,8 @@ NineToothedResult nt_tune_conv2d(NineToothedStream stream,
  * writer src/ninetoothed/build.py:683-703): a line of integers for the problem,
  * then a line for the choice; the first pair has an empty problem line and holds
  * a default.  A problem line starts with the program (0 = matmul / addmm: dtype,
- * output dtype, M, N, K, addmm, rhs layout [0 row-major, 1 transposed, 2 other
- * strides]; 1 = attention: dtype, batch, heads, seq_q, seq_k, head_dim, causal;
+ * output dtype, M, N, K, addmm, rhs layout [0 row-major, 1 transposed, 2 other strides; + 4 for operands that
+ * the direct-to-LDS instances cannot read in place]; 1 = attention: dtype, batch, heads, seq_q, seq_k, head_dim, causal;
  * 2 = conv2d: dtype, N, C, H, W, K, R, S, padding_h, padding_w, dense input);
  * a choice line starts with the variant (GEMM instance index, attention variant,
  * conv2d path) and may go on with descriptive integers (the GEMM instance's

@@ -99,7 +99,8 @@ def tune_conv2d(x, w, y, dtype, padding_h, padding_w, iters=5):
 def tune(input, mat1, mat2, beta, alpha, output, dtype, out_dtype, iters=5):
     """Times the instances on these arguments (:class:`runtime.ArgumentTensor`), records the
     winner in the library and on disk.  Returns ``(instance, milliseconds)``; the instance is -1
-    when the stream is being captured into a graph (nothing is timed or recorded then)."""
+    when the stream is being captured into a graph (nothing is timed or recorded then) and -2
+    when a single instance takes the problem (nothing to time)."""
     lib = runtime.library()
     best, best_ms = ctypes.c_int(-1), ctypes.c_float(0.0)
     runtime.check(

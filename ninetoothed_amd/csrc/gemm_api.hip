@@ -373,7 +373,12 @@ const bool g_gemm_check_registered = tune_register_check(kTuneGemm, gemm_choice_
 
 // ---- tuned choices: (dtype, output dtype, M, N, K, addmm, rhs layout) -> instance ----
 void tune_values(const GemmProblem &q, int (&values)[7]) {
-    const int layout = b_is_transposed(q) ? 1 : (q.sbn == 1 ? 0 : 2);  // rhs row-major, transposed, other strides
+    int layout = b_is_transposed(q) ? 1 : (q.sbn == 1 ? 0 : 2);  // rhs row-major, transposed, other strides
+    // + 4: operands that the direct-to-LDS instances cannot read in place (they run on dense copies, whose own
+    // problem -- same sizes when K is a multiple of 8 -- must not share this one's entry)
+    const bool in_place = q.sak == 1 && q.sam % 8 == 0 && q.k % 8 == 0 && (((uintptr_t)q.a | (uintptr_t)q.b) & 15) == 0 &&
+                          (b_is_transposed(q) ? q.sbn % 8 == 0 : (q.sbn == 1 && q.sbk % 8 == 0 && q.n % 8 == 0));
+    if (!in_place && (q.dtype == NINETOOTHED_FLOAT16 || q.dtype == NINETOOTHED_BFLOAT16)) layout += 4;
     const int v[7] = {q.dtype, q.out_dtype, q.m, q.n, q.k, q.addmm() ? 1 : 0, layout};
     for (int i = 0; i < 7; ++i) values[i] = v[i];
 }
@@ -520,7 +525,81 @@ hipError_t widen_e5m2(hipStream_t stream, const void *src, int64_t d0, int64_t d
     return hipGetLastError();
 }
 
-int run_gemm(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk);
+int run_gemm(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk, bool may_copy = true);
+
+// ---- fp16 / bf16 operands that the direct-to-LDS instances cannot read in place ----
+// A K that is no multiple of 8, rows that do not start on 16-byte boundaries, an lhs stored by columns, operands with
+// other strides: the any-stride kernel gathers such operands two bytes at a time and reaches a fifth of the fast
+// instances' rate.  For products that are large enough, one pass per operand writes a dense copy with k contiguous --
+// the lhs as [M][K8], the rhs as [N][K8], K8 = K rounded up to 8 with zeros in between, which add nothing to the sums --
+// and the product runs on the instances with tails, which take a k-contiguous rhs with any N.
+// dst[i][j] = j < d1 ? src[i * s0 + j * s1] : 0 for j < pitch; 64 x 64 tiles through LDS, so that the reads run along
+// whichever dimension has the smaller stride and the writes along j
+__global__ __launch_bounds__(256) void repack_operand_kernel(const uint16_t *src, int64_t d0, int64_t d1, int64_t s0, int64_t s1, uint16_t *dst, int64_t pitch) {
+    __shared__ uint16_t tile[64][66];
+    const int64_t tiles_j = (pitch + 63) / 64;
+    const int64_t i0 = (int64_t)(blockIdx.x / tiles_j) * 64, j0 = (int64_t)(blockIdx.x % tiles_j) * 64;
+    const int t = threadIdx.x;
+    const bool along_i = s0 < s1;  // consecutive threads read consecutive i
+#pragma unroll 4
+    for (int e = t; e < 64 * 64; e += 256) {
+        const int fast = e & 63, slow = e >> 6;
+        const int i = along_i ? fast : slow, j = along_i ? slow : fast;
+        uint16_t value = 0;
+        if (i0 + i < d0 && j0 + j < d1) value = src[(i0 + i) * s0 + (j0 + j) * s1];
+        tile[i][j] = value;
+    }
+    __syncthreads();
+    // four consecutive j per thread: 8-byte stores (pitch is a multiple of 8, so is j0 + 4 * quad)
+    typedef uint16_t ushort4_t __attribute__((ext_vector_type(4)));
+#pragma unroll 4
+    for (int e = t; e < 64 * 16; e += 256) {
+        const int quad = e & 15, i = e >> 4;
+        if (i0 + i >= d0 || j0 + 4 * quad >= pitch) continue;
+        ushort4_t out;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) out[c] = tile[i][4 * quad + c];
+        *(ushort4_t *)(dst + (i0 + i) * pitch + j0 + 4 * quad) = out;
+    }
+}
+
+hipError_t repack_operand(hipStream_t stream, const void *src, int64_t d0, int64_t d1, int64_t s0, int64_t s1, uint16_t *dst, int64_t pitch) {
+    const int64_t tiles = ((d0 + 63) / 64) * ((pitch + 63) / 64);
+    if (tiles == 0) return hipSuccess;
+    if (tiles > 0x7fffffffll) return hipErrorInvalidValue;
+    repack_operand_kernel<<<dim3((unsigned)tiles), dim3(256), 0, stream>>>((const uint16_t *)src, d0, d1, s0, s1, dst, pitch);
+    return hipGetLastError();
+}
+
+int heuristic_choice(const GemmProblem &q, int bm, int bn, int bk);
+
+// 0 / an error when the product ran on copies, NINETOOTHED_NO_KERNEL when this way does not apply
+int run_gemm_on_repacked_copies(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk) {
+    if ((q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) || q.batch != 1) return NINETOOTHED_NO_KERNEL;
+    // below about 1300^3 the two extra passes cost what they save
+    if ((int64_t)q.m * q.n * q.k < ((int64_t)1 << 31) || q.fixed_scratch != nullptr) return NINETOOTHED_NO_KERNEL;
+    const int64_t k8 = ((int64_t)q.k + 7) / 8 * 8;
+    GemmProblem dense = q;
+    dense.k = (int)k8;
+    dense.sam = k8;
+    dense.sak = 1;
+    dense.sbk = 1;
+    dense.sbn = k8;
+    // (alignment of the copies is a fact, not a property of these placeholder addresses)
+    dense.a = dense.b = (const void *)(uintptr_t)256;
+    const int choice = heuristic_choice(dense, bm, bn, bk);
+    if (choice < 0 || choice == kAnyStride) return NINETOOTHED_NO_KERNEL;  // (the output's layout rules the fast instances out)
+    WorkspaceLease lease(stream);  // held until the product is enqueued: it reads the copies
+    // (buffers of their own: the sources may be the widened copies of fp8 operands)
+    uint16_t *a = (uint16_t *)lease.get(kWorkspaceGemmLhsDense, (size_t)q.m * k8 * 2);
+    uint16_t *b = a != nullptr ? (uint16_t *)lease.get(kWorkspaceGemmRhsDense, (size_t)q.n * k8 * 2) : nullptr;
+    if (a == nullptr || b == nullptr) return NINETOOTHED_NO_KERNEL;
+    dense.a = a;
+    dense.b = b;
+    if (hipError_t err = repack_operand(stream, q.a, q.m, q.k, q.sam, q.sak, a, k8)) return (int)err;
+    if (hipError_t err = repack_operand(stream, q.b, q.n, q.k, q.sbn, q.sbk, b, k8)) return (int)err;
+    return run_gemm(stream, dense, bm, bn, bk, false);
+}
 
 // 0 / an error when the product ran on widened copies, NINETOOTHED_NO_KERNEL when this way does not apply (tiny
 // products; negative strides; no scratch memory, as under graph capture before a call of the same size outside one):
@@ -533,9 +612,9 @@ int run_gemm_on_widened_copies(hipStream_t stream, const GemmProblem &q, int bm,
     if (q.sam < 0 || q.sak < 0 || q.sbk < 0 || q.sbn < 0 || (q.addmm() && (q.sim < 0 || q.sin < 0))) return NINETOOTHED_NO_KERNEL;
     WorkspaceLease lease(stream);  // held until the product is enqueued: it reads the copies
     const auto bytes = [](int64_t d0, int64_t d1) { return (size_t)(std::max(d0, d1) + 8) * (size_t)(std::min(d0, d1) + 8) * 2; };  // (either orientation, padded rows)
-    uint16_t *a = (uint16_t *)lease.get(kWorkspaceGemmWidenedLhs, bytes(q.m, q.k));
-    uint16_t *b = a != nullptr ? (uint16_t *)lease.get(kWorkspaceGemmWidenedRhs, bytes(q.k, q.n)) : nullptr;
-    uint16_t *bias = b != nullptr && q.addmm() ? (uint16_t *)lease.get(kWorkspaceGemmWidenedBias, bytes(q.m, q.n)) : nullptr;
+    uint16_t *a = (uint16_t *)lease.get(kWorkspaceGemmLhsWidened, bytes(q.m, q.k));
+    uint16_t *b = a != nullptr ? (uint16_t *)lease.get(kWorkspaceGemmRhsWidened, bytes(q.k, q.n)) : nullptr;
+    uint16_t *bias = b != nullptr && q.addmm() ? (uint16_t *)lease.get(kWorkspaceGemmBiasWidened, bytes(q.m, q.n)) : nullptr;
     if (a == nullptr || b == nullptr || (q.addmm() && bias == nullptr)) return NINETOOTHED_NO_KERNEL;
     GemmProblem wide = q;
     wide.dtype = NINETOOTHED_FLOAT16;
@@ -550,7 +629,7 @@ int run_gemm_on_widened_copies(hipStream_t stream, const GemmProblem &q, int bm,
     return run_gemm(stream, wide, bm, bn, bk);
 }
 
-int run_gemm(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk) {
+int run_gemm(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk, bool may_copy) {
     if (q.m == 0 || q.n == 0) return 0;
     if (q.dtype == NINETOOTHED_FLOAT8_E5M2) {
         const int widened = run_gemm_on_widened_copies(stream, q, bm, bn, bk);
@@ -560,6 +639,10 @@ int run_gemm(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk) {
     if ((bm <= 0 || bn <= 0) && q.batch == 1) choice = lookup_tuned(q);  // (tuned choices are recorded for single products)
     if (choice < 0 || !kInstances[choice].accepts(q)) choice = heuristic_choice(q, bm, bn, bk);
     if (choice < 0) return NINETOOTHED_NO_KERNEL;
+    if (choice == kAnyStride && may_copy) {
+        const int copied = run_gemm_on_repacked_copies(stream, q, bm, bn, bk);
+        if (copied != NINETOOTHED_NO_KERNEL) return copied;
+    }
     note_launch(kLaunchGemm, choice, kInstances[choice].name);
     int result = (int)kInstances[choice].launch(q, stream);
     if (result == NINETOOTHED_NO_KERNEL && is_split(choice)) {  // a split-K instance without scratch memory
@@ -698,6 +781,15 @@ NineToothedResult nt_tune_gemm(NineToothedStream stream_, NineToothedTensor inpu
     if (int err = build_problem(q, &input, mat1, mat2, &beta, &alpha, output, dtype, output_dtype)) return err;
     int best = -1;
     float best_time = 0.0f;
+    // a problem that a single instance accepts (operands that only the any-stride kernel reads in place: the launch
+    // functions run large ones on dense copies) has nothing to time, and nothing is recorded for it
+    int accepting = 0;
+    for (int i = 0; i < kNumInstances; ++i) accepting += kInstances[i].accepts(q) ? 1 : 0;
+    if (accepting <= 1) {
+        if (best_config) *best_config = accepting == 1 ? -2 : -1;
+        if (best_ms) *best_ms = 0.0f;
+        return accepting == 1 ? 0 : NINETOOTHED_NO_KERNEL;
+    }
     // (inside a graph capture nothing is timed: the problem stays on the fixed preference order and nothing is recorded)
     // the untuned rule's instance is timed first and stays unless another one is more than 2 % faster: timings of a
     // few launches scatter by about that much, and the choice should not differ from process to process for nothing

@@ -872,6 +872,11 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
                 vec8 in;
                 if (p.bias_vector) {
                     in = *(const vec8 *)src;
+                } else if (p.bias_stride_n == 1 && (!kTail || gcol + 8 <= p.n)) {
+                    // a whole chunk of a row that does not start on a 16-byte boundary: one load all the same
+                    // (global accesses need no more than the element's alignment)
+                    typedef vec8 unaligned_vec8 __attribute__((aligned(2)));
+                    in = *(const unaligned_vec8 *)src;
                 } else {
 #pragma unroll
                     for (int e = 0; e < 8; ++e) in[e] = (!kTail || gcol + e < p.n) ? src[(int64_t)e * p.bias_stride_n] : E::from_float(0.0f);
@@ -879,9 +884,14 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
 #pragma unroll
                 for (int e = 0; e < 8; ++e) v[e] = E::from_float(p.beta * E::to_float(in[e]) + p.alpha * E::to_float(v[e]));
             }
-            if (kTail && !p.c_vector) {  // N or the row pitch of C no multiple of 8: element by element
+            if (kTail && !p.c_vector) {  // N or the row pitch of C no multiple of 8
+                if (gcol + kChunkElems <= p.n) {  // a whole chunk, only not on a 16-byte boundary
+                    typedef vec_out unaligned_vec_out __attribute__((aligned(sizeof(TOut))));
+                    *(unaligned_vec_out *)(C + (int64_t)grow * p.ldc + gcol) = v;
+                    continue;
+                }
 #pragma unroll
-                for (int e = 0; e < kChunkElems; ++e)
+                for (int e = 0; e < kChunkElems; ++e)  // the row's last, partial chunk: element by element
                     if (gcol + e < p.n) C[(int64_t)grow * p.ldc + gcol + e] = v[e];
                 continue;
             }

@@ -27,7 +27,7 @@ bool tune_register_check(int kind, TuneChoiceCheck check);
 
 // Written into the default pair of a saved file and compared on load: raised whenever the numbering of the GEMM
 // instances, attention variants or conv2d paths changes, so that a file from another numbering is ignored whole.
-constexpr int kTuneFileFormat = 3;
+constexpr int kTuneFileFormat = 4;
 
 // Which kernel served the latest launch_nt_* call of the calling host thread: the launch functions leave a note
 // (three thread-local stores), nt_last_launch formats it.  `name` must point to a string that lives as long as

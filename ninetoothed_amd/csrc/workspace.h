@@ -1,7 +1,8 @@
 // Device scratch buffers that outlive a call.
 //
-// conv2d's repacked operands, the narrowed K / V of fp32 attention and the partial products of
-// split-K GEMMs are temporaries of up to tens of megabytes.  Taking them from the stream-ordered allocator at every call leaves the
+// conv2d's repacked operands, the narrowed K / V of fp32 attention, the partial products of
+// split-K GEMMs and the dense copies of GEMM operands that the direct-to-LDS kernels cannot read in place
+// are temporaries of up to tens of megabytes.  Taking them from the stream-ordered allocator at every call leaves the
 // GPU idle for ~10 us between calls (the allocation that follows a pending free is not handed
 // out before the free has executed).  Instead the library keeps one buffer per (device, stream,
 // purpose), grows it when a call needs more, and reuses it otherwise: work on one stream
@@ -17,7 +18,8 @@ namespace nt {
 
 enum WorkspacePurpose {
     kWorkspaceConvInput, kWorkspaceConvFilter, kWorkspaceAttentionNarrow, kWorkspaceGemmParts, kWorkspaceAttentionParts,
-    kWorkspaceGemmWidenedLhs, kWorkspaceGemmWidenedRhs, kWorkspaceGemmWidenedBias, kWorkspacePurposes
+    kWorkspaceGemmLhsWidened, kWorkspaceGemmRhsWidened, kWorkspaceGemmBiasWidened, kWorkspaceGemmLhsDense, kWorkspaceGemmRhsDense,
+    kWorkspacePurposes
 };
 
 // Holds the registry lock from construction to destruction: create it, take the buffers,

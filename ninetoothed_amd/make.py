@@ -358,8 +358,8 @@ class Kernel:
             if any(t.untyped_storage().data_ptr() == out.untyped_storage().data_ptr() for t in sources):
                 return
             instance, _ = auto_tuner.tune(input_arg, a_arg, b_arg, beta, alpha, c_arg, dtype, out_dtype)
-            # inside a graph capture nothing is timed: the next call outside one tunes
-            state["tune"] = instance < 0
+            # inside a graph capture nothing is timed (-1): the next call outside one tunes; -2: nothing to choose from
+            state["tune"] = instance == -1
 
         if i is not None:
             i_arg = runtime.ArgumentTensor.from_layout(0, (m, n), (i.row_stride, i.col_stride))  # (a stride of 0 is a broadcast here)

@@ -1174,6 +1174,58 @@ def test_matmul_float8_e5m2_operands(m, n, k):
     assert np.allclose(out.cpu().float().numpy(), reference, **HALF_TOL)
 
 
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
+def test_large_products_on_operands_the_fast_instances_cannot_read_run_on_dense_copies(dtype):
+    """A K that is no multiple of 8, rows off 16-byte boundaries, an lhs stored by columns, other strides: from 2^31
+    multiply-adds on such operands are copied (k contiguous, K padded to 8 with zeros) and the product runs on the
+    direct-to-LDS instances.  What lies next to the operands in memory is Inf and must not reach the sums; what
+    lies next to the output must stay as it was."""
+    from ninetoothed_amd import runtime
+
+    kernel = _matmul_kernel()
+
+    def inside(rows, cols, pad_rows=1, pad_cols=3, transposed=False):
+        # a [rows, cols] matrix inside an Inf-filled buffer; `transposed`: stored by columns
+        shape = (cols + pad_rows, rows + pad_cols) if transposed else (rows + pad_rows, cols + pad_cols)
+        buffer = torch.full(shape, float("inf"), dtype=dtype, device="cuda")
+        view = buffer[: shape[0] - pad_rows, : shape[1] - pad_cols]
+        view.copy_(torch.randn(view.shape, device="cuda").to(dtype))
+        return view.T if transposed else view
+
+    def check(lhs, rhs, out_cols_pad=0, fast=True):
+        m, k, n = lhs.shape[0], lhs.shape[1], rhs.shape[1]
+        buffer = torch.full((m + 1, n + out_cols_pad + 8), 7.0, dtype=dtype, device="cuda")
+        out = buffer[:m, :n]
+        kernel(lhs, rhs, out)
+        _native_only(kernel, "launch_nt_matmul")
+        assert ("any-stride" not in runtime.last_launch()) == fast, runtime.last_launch()
+        expected = lhs.float() @ rhs.float()
+        assert torch.allclose(out.float(), expected, rtol=1e-2, atol=1e-2 * (k / 512) ** 0.5), float((out.float() - expected).abs().max())
+        assert bool((buffer[m:] == 7.0).all()) and bool((buffer[:, n:] == 7.0).all())
+
+    check(inside(2050, 1029), inside(1029, 1100))                      # K = 1029, rows off 16-byte boundaries, N no multiple of 8
+    check(inside(2048, 1024, transposed=True), inside(1024, 1024))     # the lhs stored by columns
+    check(inside(2048, 1024, transposed=True), inside(1024, 1031, transposed=True), out_cols_pad=1)  # both, C rows off 16-byte boundaries
+    wide_l, wide_r = inside(2048, 2048), inside(1024, 2048)
+    check(wide_l[:, ::2], wide_r[:, ::2])                              # every other column
+    # below the threshold the any-stride kernel serves the call as before
+    check(inside(300, 205), inside(205, 301), fast=False)
+    # addmm on such operands, the bias with rows off 16-byte boundaries as well
+    m, k, n = 2050, 1029, 1100
+    bias, lhs, rhs = inside(m, n), inside(m, k), inside(k, n)
+    buffer = torch.full((m + 1, n + 9), 7.0, dtype=dtype, device="cuda")
+    out = buffer[:m, :n]
+    application = programs.addmm.application if dtype == torch.float16 else programs.addmm.application_bfloat16
+    addmm = ninetoothed.make(programs.addmm.arrangement, application, programs.addmm.tensors())
+    addmm(bias, lhs, rhs, 0.5, 2.0, out)
+    _native_only(addmm, "launch_nt_addmm")
+    assert "any-stride" not in runtime.last_launch(), runtime.last_launch()
+    expected = 0.5 * bias.float() + 2.0 * (lhs.float() @ rhs.float()).to(dtype).float()
+    tolerance = dict(rtol=2e-2, atol=2e-2 * (k / 512) ** 0.5) if dtype == torch.bfloat16 else dict(rtol=1e-2, atol=1e-2 * (k / 512) ** 0.5)
+    assert torch.allclose(out.float(), expected, **tolerance), float((out.float() - expected).abs().max())
+    assert bool((buffer[m:] == 7.0).all()) and bool((buffer[:, n:] == 7.0).all())
+
+
 @pytest.mark.skipif(not hasattr(torch, "float8_e5m2"), reason="this torch has no float8_e5m2")
 def test_matmul_float8_e5m2_large_products_run_on_widened_copies():
     """fp8 operands are widened into fp16 copies (exact) and the product runs on the fp16 instances, direct-to-LDS
@@ -1206,13 +1258,14 @@ def test_matmul_float8_e5m2_large_products_run_on_widened_copies():
     check(lhs, rhs)                                      # both row-major
     check(lhs, rhs, out_dtype=torch.float32)
     check(lhs, torch.randn(n, k, device="cuda").to(torch.float8_e5m2).T)   # the reference's case: the rhs column-major
-    check(torch.randn(k, m, device="cuda").to(torch.float8_e5m2).T, rhs, fast=False)  # a column-major lhs: copies follow it, the any-stride fp16 kernel runs
+    check(torch.randn(k, m, device="cuda").to(torch.float8_e5m2).T, rhs)  # a column-major lhs: the widened copy follows it and is copied once more, k contiguous
     # operands inside wider buffers, rows that start off 16-byte boundaries (byte-wise widening)
     wide = torch.randn(m + 3, k + 5, device="cuda").to(torch.float8_e5m2)
     lhs2 = wide[3:, 5:]
     lhs2.view(torch.uint8)[0, 0] = 0x5C  # 256.0
     check(lhs2, rhs)
-    # sizes that are no multiples of 8: the copies get padded rows, the any-stride fp16 kernel runs on them
+    # sizes that are no multiples of 8, below the size from which such fp16 operands are copied: the widened copies
+    # get padded rows and the any-stride fp16 kernel runs on them
     check(torch.randn(2050, 1030, device="cuda").to(torch.float8_e5m2), torch.randn(1030, 1001, device="cuda").to(torch.float8_e5m2), fast=False)
     # addmm: the bias is widened as well (tests/test_addmm.py:57-90 of the reference at a larger size)
     bias = torch.randn(m, n, device="cuda").to(torch.float8_e5m2)
