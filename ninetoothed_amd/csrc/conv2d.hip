@@ -179,7 +179,11 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
     // the filter descriptor ends with the matrix: a partial last tile of output channels reads the next
     // row's values (they only feed channels that are not stored) and, in the last row, zeros
     __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)((const T *)p.wt + n0), 0, p.wt_bytes - (unsigned)n0 * 2u, 0x00020000);
-    int a_base[kAInstr], a_y[kAInstr], a_x[kAInstr];
+    // Few input channels (p.C = 8 or 16 after padding): a k step of 32 contraction positions then holds 4 or 2
+    // filter taps, and which tap a lane fetches follows from its chunk of the step.
+    const bool narrow = p.C < BK;
+    const int chunks_per_tap = narrow ? p.C / 8 : kAChunksPerRow;
+    int a_base[kAInstr], a_y[kAInstr], a_x[kAInstr], a_tap[kAInstr];
 #pragma unroll
     for (int j = 0; j < kAInstr; ++j) {
         const int row = (j * kWaves + wave) * kARowsPerInstr + lane / kAChunksPerRow;
@@ -189,7 +193,8 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
         const int oy = pq / p.Q, ox = pq - oy * p.Q;
         a_y[j] = m < p.M ? oy * p.stride_h - p.pad_h : -(1 << 20);  // rows past the last image never pass the bounds test
         a_x[j] = ox * p.stride_w - p.pad_w;
-        a_base[j] = m < p.M ? (((image * p.H + a_y[j]) * p.W + a_x[j]) * p.C + chunk * 8) * 2 : 0;
+        a_tap[j] = chunk / chunks_per_tap;  // (narrow) the lane's tap within a k step
+        a_base[j] = m < p.M ? (((image * p.H + a_y[j]) * p.W + a_x[j]) * p.C + (chunk % chunks_per_tap) * 8) * 2 : 0;
     }
     unsigned b_src[kBInstr];
 #pragma unroll
@@ -204,6 +209,22 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
         // k order: channel block outer, filter taps inner -- the R*S taps of a block of 32 channels read the
         // same pixels shifted by a row or a column, so they hit in L2 while the lines are still there
         const int taps = p.R * p.S;
+        if (narrow) {  // (uniform) rows of the repacked filter are (tap, channel) pairs in this order: k step kt is rows 32 kt ...
+            const int taps_per_step = BK / p.C;
+#pragma unroll
+            for (int j = 0; j < kAInstr; ++j) {
+                const int tap = kt * taps_per_step + a_tap[j];
+                const int fy = (tap / p.S) * p.dil_h, fx = (tap % p.S) * p.dil_w;
+                const bool inside = tap < taps && (unsigned)(a_y[j] + fy) < (unsigned)p.H && (unsigned)(a_x[j] + fx) < (unsigned)p.W;
+                const unsigned offset = inside ? (unsigned)(a_base[j] + (fy * p.W + fx) * p.C * 2) : 0x80000000u;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, sa + (j * kWaves + wave) * 1024, 16, offset, 0, 0, 0);
+            }
+            const int b_k = kt * BK * p.K * 2;  // (rows past the last tap lie behind the descriptor: zeros)
+#pragma unroll
+            for (int j = 0; j < kBInstr; ++j)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, sb + (j * kWaves + wave) * 1024, 16, b_src[j], b_k, 0, 0);
+            return;
+        }
         const int cb = kt / taps;
         const int tap = kt - cb * taps;
         const int c0 = cb * BK;
@@ -276,7 +297,7 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
         }
     };
 
-    const int num_k = p.R * p.S * (p.C / BK);
+    const int num_k = (p.R * p.S * p.C + BK - 1) / BK;
     const int last_k = num_k - 1;
     const int main_k = num_k - num_k % kStages;
     static_for<0, kStages - 1>([&](auto s) { issue_loads(s, min((int)decltype(s)::value, last_k)); });
@@ -940,9 +961,13 @@ int run_direct(const Conv2dRequest &q, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
+// channels of the repacked operands: the k step of 32 holds whole blocks of channels -- or, for up to 16 channels
+// (the first layer of an image network), 4 or 2 filter taps of 8 or 16 channels each; the extra channels are zeros
+inline int conv2d_padded_channels(int channels) { return channels <= 16 ? ceil_div(channels, 8) * 8 : ceil_div(channels, 32) * 32; }
+
 template <typename T>
 int run_fast(const Conv2dRequest &q, hipStream_t stream) {
-    const int Cp = ceil_div(q.C, 32) * 32;
+    const int Cp = conv2d_padded_channels(q.C);
     const int64_t xt_bytes = (int64_t)q.N * q.H * q.W * Cp * 2;
     const int64_t wt_bytes = (int64_t)q.K * Cp * q.R * q.S * 2;
     WorkspaceLease lease(stream);
@@ -998,8 +1023,8 @@ int conv2d_fast(const Conv2dRequest &q, hipStream_t stream) {
     if (q.K % 8 || q.C < 2) return NINETOOTHED_NO_KERNEL;  // (rows of the repacked filter are read in 16-byte pieces)
     if (q.ys[3] != 1 || q.ys[2] != q.Q || q.ys[1] != (int64_t)q.P * q.Q || q.ys[0] != (int64_t)q.K * q.P * q.Q) return NINETOOTHED_NO_KERNEL;
     if (((uintptr_t)q.y & 15) != 0) return NINETOOTHED_NO_KERNEL;
-    const int64_t xt_bytes = (int64_t)q.N * q.H * q.W * ceil_div(q.C, 32) * 32 * 2;
-    const int64_t wt_bytes = (int64_t)q.K * ceil_div(q.C, 32) * 32 * q.R * q.S * 2;
+    const int64_t xt_bytes = (int64_t)q.N * q.H * q.W * conv2d_padded_channels(q.C) * 2;
+    const int64_t wt_bytes = (int64_t)q.K * conv2d_padded_channels(q.C) * q.R * q.S * 2;
     if (xt_bytes >= (int64_t(1) << 31) || wt_bytes >= (int64_t(1) << 31)) return NINETOOTHED_NO_KERNEL;  // 32-bit buffer offsets
     if ((int64_t)q.N * q.P * q.Q > 0x7fffffffll || (int64_t)ceil_div(q.N * q.P * q.Q, 128) * ceil_div(q.K, 64) > 0x7fffffffll) return NINETOOTHED_NO_KERNEL;
     if (q.N >= 65535 - 512 || ceil_div(q.C, 64) > 65535) return NINETOOTHED_NO_KERNEL;  // grid of the repacking pass: (positions, channels, filter layers + images)

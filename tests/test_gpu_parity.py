@@ -828,6 +828,28 @@ def test_conv2d_with_stride_and_dilation_layer_shapes(n, c, h, w, k, r, s, paddi
     assert runtime.library().launch_nt_conv2d_strided(runtime.current_stream(), *tensors, tag, *padding, *stride, *dilation, 0, 0, 0) == 1  # hipErrorInvalidValue
 
 
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
+@pytest.mark.parametrize("channels", (2, 3, 4, 8, 9, 13, 16, 17))
+def test_conv2d_few_input_channels_on_the_repacked_path(channels, dtype):
+    """Up to 16 input channels are padded to 8 or 16, not 32, on the repacked path: a k step then holds 4 or 2 filter
+    taps, the last step of a filter whose taps do not fill it reads zeros (7 x 7 = 49 taps, 3 x 5 = 15)."""
+    from ninetoothed_amd import runtime
+
+    tag = runtime.DATA_TYPE_INDEX["fp16" if dtype == torch.float16 else "bf16"]
+    for (n, h, w, k, r, s_, padding, stride, dilation) in ((3, 40, 36, 64, 7, 7, (3, 3), (2, 2), (1, 1)), (2, 33, 31, 24, 3, 5, (1, 2), (1, 1), (2, 1)), (2, 32, 32, 40, 1, 1, (0, 0), (1, 1), (1, 1))):
+        x = _randn(n, channels, h, w, dtype=dtype, scale=0.3).cuda()
+        weight = _randn(k, channels, r, s_, dtype=dtype, scale=0.3).cuda()
+        expected = F.conv2d(x.float(), weight.float(), padding=padding, stride=stride, dilation=dilation)
+        y = torch.full(expected.shape, float("nan"), dtype=dtype, device="cuda")
+        tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (x, weight, y)]
+        if stride == (1, 1) and dilation == (1, 1):
+            assert runtime.library().launch_nt_conv2d(runtime.current_stream(), *tensors, tag, *padding, 2, 0, 0) == 0
+        else:
+            assert runtime.library().launch_nt_conv2d_strided(runtime.current_stream(), *tensors, tag, *padding, *stride, *dilation, 2, 0, 0) == 0
+        assert runtime.last_launch().startswith("conv2d path 2"), runtime.last_launch()
+        assert torch.allclose(y.float(), expected, **HALF_TOL), (channels, r, s_, float((y.float() - expected).abs().max()))
+
+
 def test_conv2d_one_launch_path_refuses_what_it_cannot_run():
     from ninetoothed_amd import runtime
 
