@@ -209,10 +209,11 @@ NineToothedResult launch_nt_attention(NineToothedStream stream,
  *   tap)-shifted pixel runs of the NCHW input; needs an output width that is a
  *   multiple of 8, padding_w <= 1, C*R*S a multiple of 32, R*S / gcd(32, R*S) <= 25, pixels of an input row
  *   contiguous, contiguous filter and output, K filling 256-wide tiles to 4/5;
- * 2 -- when K % 8 == 0, C >= 2, the output is contiguous and N*P*Q >= 1024: the
- *   input is first repacked to channels-last and the filter to [R*S*C', K]
- *   (C' = C rounded up to a multiple of 32, zero filled) in the library's scratch
- *   buffers of `stream` (N*C'*H*W + K*C'*R*S elements), then the direct-to-LDS
+ * 2 -- when the output is contiguous (fp16 / bf16 tensors): the
+ *   input is first repacked to channels-last and the filter to [R*S*C', K']
+ *   (C' = C rounded up to a multiple of 32 -- to 8 or 16 for up to 16 channels --, K' = K
+ *   rounded up to 8, zero filled) in the library's scratch
+ *   buffers of `stream` (N*C'*H*W + K'*C'*R*S elements), then the direct-to-LDS
  *   GEMM loop runs;
  * 1 -- the scratch-free gather kernel, which serves every shape, and calls whose
  *   scratch cannot be allocated (out of memory; a stream under graph capture that

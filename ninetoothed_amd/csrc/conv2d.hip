@@ -46,6 +46,7 @@ struct ConvParams {
     const void *wt;
     void *y;
     int N, C, H, W, K, R, S, P, Q, pad_h, pad_w;
+    int Kp;                   // row pitch of the repacked filter: K rounded up to 8 (its rows are read in 16-byte pieces)
     int M, tiles_m, tiles_n;  // M = N*P*Q rows
     unsigned xt_bytes, wt_bytes;
     int stride_h, stride_w, dil_h, dil_w;  // steps of the window over the input and between its taps
@@ -63,6 +64,7 @@ struct FilterRepack {
     int64_t s_k, s_c, s_r, s_s;
     int layers;
     int Cp;  // channels of the repacked operands: C rounded up to the k step, the extra ones zero
+    int Kp;  // row pitch of the repacked filter: K rounded up to 8, the extra columns zero
 };
 
 template <typename T>
@@ -75,14 +77,14 @@ __global__ __launch_bounds__(256) void conv2d_repack_kernel(const T *x, T *xt, i
     if ((int)blockIdx.z < f.layers) {
         const T *w = (const T *)f.w;
         T *wt = (T *)f.wt;
-        const int64_t total = (int64_t)f.K * f.Cp * f.R * f.S;
+        const int64_t total = (int64_t)f.Kp * f.Cp * f.R * f.S;
         const int64_t layer_threads = (int64_t)gridDim.x * gridDim.y * 256 * f.layers;
         for (int64_t index = (((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 256 + t; index < total; index += layer_threads) {
-            const int k = (int)(index % f.K);
-            const int64_t row = index / f.K;
+            const int k = (int)(index % f.Kp);
+            const int64_t row = index / f.Kp;
             const int c = (int)(row % f.Cp);
             const int rs = (int)(row / f.Cp);
-            wt[index] = c < f.C ? w[(int64_t)k * f.s_k + (int64_t)c * f.s_c + (int64_t)(rs / f.S) * f.s_r + (int64_t)(rs % f.S) * f.s_s] : (T)0.0f;
+            wt[index] = c < f.C && k < f.K ? w[(int64_t)k * f.s_k + (int64_t)c * f.s_c + (int64_t)(rs / f.S) * f.s_r + (int64_t)(rs % f.S) * f.s_s] : (T)0.0f;
         }
         return;
     }
@@ -201,7 +203,7 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
     for (int j = 0; j < kBInstr; ++j) {
         const int krow = (j * kWaves + wave) * kBRowsPerInstr + lane / kBChunksPerRow;
         const int chunk = b_phys_chunk<BN>(krow, lane % kBChunksPerRow);
-        b_src[j] = (unsigned)(krow * p.K + chunk * 8) * 2u;
+        b_src[j] = (unsigned)(krow * p.Kp + chunk * 8) * 2u;
     }
     auto issue_loads = [&](auto stage_tag, int kt) {
         NT_LDS unsigned char *sa = stage_a(stage_tag);
@@ -219,7 +221,7 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
                 const unsigned offset = inside ? (unsigned)(a_base[j] + (fy * p.W + fx) * p.C * 2) : 0x80000000u;
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, sa + (j * kWaves + wave) * 1024, 16, offset, 0, 0, 0);
             }
-            const int b_k = kt * BK * p.K * 2;  // (rows past the last tap lie behind the descriptor: zeros)
+            const int b_k = kt * BK * p.Kp * 2;  // (rows past the last tap lie behind the descriptor: zeros)
 #pragma unroll
             for (int j = 0; j < kBInstr; ++j)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, sb + (j * kWaves + wave) * 1024, 16, b_src[j], b_k, 0, 0);
@@ -236,7 +238,7 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
             const unsigned offset = inside ? (unsigned)(a_base[j] + delta) : 0x80000000u;  // beyond num_records: reads zeros
             __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, sa + (j * kWaves + wave) * 1024, 16, offset, 0, 0, 0);
         }
-        const int b_k = (tap * p.C + c0) * p.K * 2;
+        const int b_k = (tap * p.C + c0) * p.Kp * 2;
 #pragma unroll
         for (int j = 0; j < kBInstr; ++j)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, sb + (j * kWaves + wave) * 1024, 16, b_src[j], b_k, 0, 0);
@@ -969,7 +971,8 @@ template <typename T>
 int run_fast(const Conv2dRequest &q, hipStream_t stream) {
     const int Cp = conv2d_padded_channels(q.C);
     const int64_t xt_bytes = (int64_t)q.N * q.H * q.W * Cp * 2;
-    const int64_t wt_bytes = (int64_t)q.K * Cp * q.R * q.S * 2;
+    const int Kp = ceil_div(q.K, 8) * 8;
+    const int64_t wt_bytes = (int64_t)Kp * Cp * q.R * q.S * 2;
     WorkspaceLease lease(stream);
     void *xt = lease.get(kWorkspaceConvInput, (size_t)xt_bytes);
     void *wt = lease.get(kWorkspaceConvFilter, (size_t)wt_bytes);
@@ -979,11 +982,11 @@ int run_fast(const Conv2dRequest &q, hipStream_t stream) {
     FilterRepack f;
     f.w = q.w;
     f.wt = wt;
-    f.K = q.K; f.C = q.C; f.R = q.R; f.S = q.S; f.Cp = Cp;
+    f.K = q.K; f.C = q.C; f.R = q.R; f.S = q.S; f.Cp = Cp; f.Kp = Kp;
     f.s_k = q.ws[0]; f.s_c = q.ws[1]; f.s_r = q.ws[2]; f.s_s = q.ws[3];
     // about 512 workgroups for the filter, or one thread per element if that is less
     const int64_t per_layer = (int64_t)ceil_div(HW, 64) * ceil_div(Cp, 64);
-    const int64_t wanted = std::min<int64_t>(512, ((int64_t)q.K * Cp * q.R * q.S + 255) / 256);
+    const int64_t wanted = std::min<int64_t>(512, ((int64_t)Kp * Cp * q.R * q.S + 255) / 256);
     f.layers = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(wanted, per_layer), 512));
     conv2d_repack_kernel<T><<<dim3(ceil_div(HW, 64), ceil_div(Cp, 64), q.N + f.layers), dim3(256), 0, stream>>>(
         (const T *)q.x, (T *)xt, q.C, HW, q.W, q.xs[0], q.xs[1], q.xs[2], q.xs[3], vector_ok, f);
@@ -992,6 +995,7 @@ int run_fast(const Conv2dRequest &q, hipStream_t stream) {
     p.wt = wt;
     p.y = q.y;
     p.N = q.N; p.C = Cp; p.H = q.H; p.W = q.W; p.K = q.K; p.R = q.R; p.S = q.S; p.P = q.P; p.Q = q.Q;
+    p.Kp = Kp;
     p.stride_h = q.stride_h; p.stride_w = q.stride_w; p.dil_h = q.dil_h; p.dil_w = q.dil_w;
     p.pad_h = q.pad_h; p.pad_w = q.pad_w;
     p.M = q.N * q.P * q.Q;
@@ -1020,16 +1024,17 @@ int run_fast(const Conv2dRequest &q, hipStream_t stream) {
 int conv2d_fast(const Conv2dRequest &q, hipStream_t stream) {
     if (q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) return NINETOOTHED_NO_KERNEL;
     // channels are padded to the k step of 32 with zeros; below a sixteenth of useful work the gather kernel is as good
-    if (q.K % 8 || q.C < 2) return NINETOOTHED_NO_KERNEL;  // (rows of the repacked filter are read in 16-byte pieces)
+    if (q.C < 1) return NINETOOTHED_NO_KERNEL;
     if (q.ys[3] != 1 || q.ys[2] != q.Q || q.ys[1] != (int64_t)q.P * q.Q || q.ys[0] != (int64_t)q.K * q.P * q.Q) return NINETOOTHED_NO_KERNEL;
     if (((uintptr_t)q.y & 15) != 0) return NINETOOTHED_NO_KERNEL;
     const int64_t xt_bytes = (int64_t)q.N * q.H * q.W * conv2d_padded_channels(q.C) * 2;
-    const int64_t wt_bytes = (int64_t)q.K * conv2d_padded_channels(q.C) * q.R * q.S * 2;
+    const int64_t wt_bytes = (int64_t)ceil_div(q.K, 8) * 8 * conv2d_padded_channels(q.C) * q.R * q.S * 2;
     if (xt_bytes >= (int64_t(1) << 31) || wt_bytes >= (int64_t(1) << 31)) return NINETOOTHED_NO_KERNEL;  // 32-bit buffer offsets
     if ((int64_t)q.N * q.P * q.Q > 0x7fffffffll || (int64_t)ceil_div(q.N * q.P * q.Q, 128) * ceil_div(q.K, 64) > 0x7fffffffll) return NINETOOTHED_NO_KERNEL;
     if (q.N >= 65535 - 512 || ceil_div(q.C, 64) > 65535) return NINETOOTHED_NO_KERNEL;  // grid of the repacking pass: (positions, channels, filter layers + images)
-    // enough work to amortise the repacking pass
-    if ((int64_t)q.N * q.P * q.Q < 1024) return NINETOOTHED_NO_KERNEL;
+    // (even a few output positions are served sooner by two short launches than by the gather kernel, whose lanes
+    // fetch their 16 values of a k step one after another: [2, 32, 9, 9] * [16, 32, 3, 3] 48 against 13 us)
+    if ((int64_t)q.N * q.P * q.Q < 1) return NINETOOTHED_NO_KERNEL;
     return q.dtype == NINETOOTHED_FLOAT16 ? run_fast<half_t>(q, stream) : run_fast<bf16_t>(q, stream);
 }
 
