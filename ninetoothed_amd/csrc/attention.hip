@@ -107,7 +107,7 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
     // ids walk groups of kCausalGroup (batch, head) pairs, and inside a group the query
     // blocks from last (longest) to first, pair by pair: a CU gets a mix of long and
     // short blocks while only the K/V of one group (plus the next one's beginning)
-    // is live in the XCD's L2.  Other pair counts fall back to walking all pairs.
+    // is live in the XCD's L2.  Pair counts that are no multiple of 8 walk pair by pair.
     constexpr int kCausalGroup = 4;
     const int total = kSplitKV ? gridDim.x / p.parts : gridDim.x;
     const int part = kSplitKV ? blockIdx.x / total : 0;
@@ -117,15 +117,20 @@ __global__ __launch_bounds__(kWaves * 64, kOcc) void attention_fwd_kernel(Attent
     int qb, bh;
     if (p.causal) {
         const int pairs = p.batch * p.heads;
-        if (renumber && pairs % (8 * kCausalGroup) == 0) {
-            const int per_group = kCausalGroup * p.q_blocks;
+        if (renumber && pairs % 8 == 0) {
+            // (fewer pairs per XCD than a group: groups of two, or single pairs -- eight heads of a long sequence then
+            // run one per XCD, whose CUs stream that head's K / V together instead of eight heads' at once)
+            const int per_xcd = pairs >> 3;
+            const int in_a_group = per_xcd % kCausalGroup == 0 ? kCausalGroup : (per_xcd % 2 == 0 ? 2 : 1);
+            const int per_group = in_a_group * p.q_blocks;
             const int group = wg / per_group;
             const int in_group = wg % per_group;
-            qb = p.q_blocks - 1 - in_group / kCausalGroup;
-            bh = group * kCausalGroup + in_group % kCausalGroup;
+            qb = p.q_blocks - 1 - in_group / in_a_group;
+            bh = group * in_a_group + in_group % in_a_group;
         } else {
-            qb = p.q_blocks - 1 - wg / pairs;
-            bh = wg % pairs;
+            // pair by pair, each from its longest block down: ids that run at one time belong to one or two pairs
+            qb = p.q_blocks - 1 - wg % p.q_blocks;
+            bh = wg / p.q_blocks;
         }
     } else {
         qb = wg % p.q_blocks;
