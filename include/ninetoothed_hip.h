@@ -16,7 +16,7 @@
  *
  * Launches are asynchronous on the given stream and never synchronise; the
  * caller owns every tensor.  Only launch_nt_conv2d, launch_nt_attention on
- * FLOAT32 tensors or on few query blocks against many keys (split key range:
+ * FLOAT32 tensors, on tensors it cannot read in place (see there) or on few query blocks against many keys (split key range:
  * parts x batch x heads x seq_q x (head_dim + 1) floats; not when the caller
  * passes block sizes), and launch_nt_matmul / launch_nt_addmm on problems with few
  * output tiles and a long K (split-K: parts x M x N floats, at most 64 MiB; not
@@ -184,8 +184,10 @@ NineToothedResult launch_nt_softmax_config(NineToothedStream stream, int config,
  * less than 4 GiB (16-bit tensors).
  * head_dim: 32, 64, 128 and 256 have kernels of their size; any other multiple of
  * 8 up to 256 runs on the next of these sizes with the missing columns read as
- * zeros (K and V of one (batch, head) then span less than 2 GiB); anything else
- * returns NINETOOTHED_NO_KERNEL. */
+ * zeros (K and V of one (batch, head) then span less than 2 GiB).  Head dimensions up to 256 that are no multiples
+ * of 8, a last dimension with another stride than 1, and tensors whose rows do not start on 16-byte boundaries run on
+ * padded dense copies of Q, K and V in the stream's scratch buffers (4 x batch x heads x seq x head_dim rounded up
+ * to 8 elements), with O copied back; a head dimension above 256 returns NINETOOTHED_NO_KERNEL. */
 NineToothedResult launch_nt_attention(NineToothedStream stream,
                                       NineToothedTensor q,
                                       NineToothedTensor k,

@@ -1202,6 +1202,7 @@ int attention_setup(AttentionParams &p, const NineToothedTensor &q, const NineTo
     const int64_t head_dim = (int64_t)q.shape[3];
     for (const NineToothedTensor *t : ts) {
         if (t->shape[0] != q.shape[0] || t->shape[1] != q.shape[1] || (int64_t)t->shape[3] != head_dim) return hipErrorInvalidValue;
+        if (head_dim % 8 != 0) return NINETOOTHED_NO_KERNEL;  // (launch_nt_attention runs such tensors on padded copies)
         if (float32 && (t == &k || t == &v)) continue;  // converted copies: any strides
         if (t->strides[3] != 1 && head_dim > 1) return NINETOOTHED_NO_KERNEL;
         const int lanes = float32 ? 4 : 8;  // elements per 16 bytes
@@ -1269,12 +1270,97 @@ bool attention_would_split(const AttentionParams &p) { return (p.head_dim == 128
 }  // namespace
 }  // namespace nt
 
-extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineToothedTensor q, NineToothedTensor k,
-                                                 NineToothedTensor v, NineToothedTensor is_causal,
-                                                 NineToothedTensor scale, NineToothedTensor o, int dtype,
-                                                 int block_size_m, int block_size_n) {
+namespace nt {
+namespace {
+
+// ---- tensors the kernels cannot read in place: a head dimension that is no multiple of 8 (the reference pads it
+// to a power of two inside its kernel and masks), rows that do not start on 16-byte boundaries, a strided last
+// dimension.  Q, K and V are copied into dense [B, H, S, D8] buffers of the stream's scratch memory, D8 = D rounded
+// up to 8 with zeros (zero columns add nothing to Q K^T, and the columns of O they produce are dropped), the
+// attention runs on the copies, and O is copied back.
+template <typename E>
+__global__ __launch_bounds__(256) void attention_pad_kernel(const E *src, E *dst, int64_t rows, int heads, int seq, int d, int d8, int64_t s0, int64_t s1,
+                                                            int64_t s2, int64_t s3, int back) {
+    // back == 0: dst[row][0 .. d8) = src row, zero padded; back != 0: the first d columns of the dense `src` rows go to `dst`
+    const int64_t total = rows * (back ? d : d8);
+    for (int64_t index = (int64_t)blockIdx.x * 256 + threadIdx.x; index < total; index += (int64_t)gridDim.x * 256) {
+        const int width = back ? d : d8;
+        const int64_t row = index / width;
+        const int col = (int)(index - row * width);
+        const int64_t bh = row / seq;
+        const int64_t strided = (bh / heads) * s0 + (bh % heads) * s1 + (row % seq) * s2 + (int64_t)col * s3;
+        if (back) dst[strided] = src[row * d8 + col];
+        else dst[index] = col < d ? src[strided] : (E)0;
+    }
+}
+
+template <typename E>
+hipError_t attention_pad(hipStream_t stream, const NineToothedTensor &t, void *dense, int d8, bool back) {
+    const int64_t rows = (int64_t)t.shape[0] * t.shape[1] * t.shape[2];
+    const int64_t work = rows * (back ? (int64_t)t.shape[3] : d8);
+    if (work == 0) return hipSuccess;
+    const unsigned blocks = (unsigned)std::min<int64_t>((work + 255) / 256, 256 * 64);
+    if (back)
+        attention_pad_kernel<E><<<dim3(blocks), dim3(256), 0, stream>>>((const E *)dense, (E *)t.data, rows, (int)t.shape[1], (int)t.shape[2], (int)t.shape[3], d8,
+                                                                           t.strides[0], t.strides[1], t.strides[2], t.strides[3], 1);
+    else
+        attention_pad_kernel<E><<<dim3(blocks), dim3(256), 0, stream>>>((const E *)t.data, (E *)dense, rows, (int)t.shape[1], (int)t.shape[2], (int)t.shape[3], d8,
+                                                                           t.strides[0], t.strides[1], t.strides[2], t.strides[3], 0);
+    return hipGetLastError();
+}
+
+int launch_attention(hipStream_t stream, const NineToothedTensor &q, const NineToothedTensor &k, const NineToothedTensor &v, const NineToothedTensor &is_causal,
+                     const NineToothedTensor &scale, const NineToothedTensor &o, int dtype, int block_size_m, int block_size_n, bool may_copy);
+
+// 0 / an error when the attention ran on copies, NINETOOTHED_NO_KERNEL when this way does not apply either
+int attention_on_padded_copies(hipStream_t stream, const NineToothedTensor &q, const NineToothedTensor &k, const NineToothedTensor &v,
+                               const NineToothedTensor &is_causal, const NineToothedTensor &scale, const NineToothedTensor &o, int dtype,
+                               int block_size_m, int block_size_n) {
+    if (dtype != NINETOOTHED_FLOAT16 && dtype != NINETOOTHED_BFLOAT16 && dtype != NINETOOTHED_FLOAT32) return NINETOOTHED_NO_KERNEL;
+    const NineToothedTensor *ts[4] = {&q, &k, &v, &o};
+    for (const NineToothedTensor *t : ts)
+        if (!t->shape || !t->strides) return NINETOOTHED_NO_KERNEL;
+    const uint64_t d = q.shape[3];
+    if (d == 0 || d > 256) return NINETOOTHED_NO_KERNEL;
+    for (const NineToothedTensor *t : ts)
+        if (t->shape[0] != q.shape[0] || t->shape[1] != q.shape[1] || t->shape[3] != d) return NINETOOTHED_NO_KERNEL;
+    if (v.shape[2] != k.shape[2] || o.shape[2] != q.shape[2] || k.shape[2] == 0) return NINETOOTHED_NO_KERNEL;
+    const int d8 = (int)((d + 7) / 8 * 8);
+    const size_t size = dtype == NINETOOTHED_FLOAT32 ? 4 : 2;
+    WorkspaceLease lease(stream);  // held until the copy back is enqueued
+    const WorkspacePurpose purposes[4] = {kWorkspaceAttentionPaddedQ, kWorkspaceAttentionPaddedK, kWorkspaceAttentionPaddedV, kWorkspaceAttentionPaddedO};
+    void *dense[4];
+    uint64_t shapes[4][4];
+    int64_t strides[4][4];
+    NineToothedTensor copies[4];
+    for (int i = 0; i < 4; ++i) {
+        const NineToothedTensor &t = *ts[i];
+        const uint64_t rows = t.shape[0] * t.shape[1] * t.shape[2];
+        if (rows * (uint64_t)d8 > 0x7fffffffull * 8) return NINETOOTHED_NO_KERNEL;
+        dense[i] = lease.get(purposes[i], (size_t)rows * d8 * size + 256);
+        if (dense[i] == nullptr) return NINETOOTHED_NO_KERNEL;
+        for (int a = 0; a < 3; ++a) shapes[i][a] = t.shape[a];
+        shapes[i][3] = (uint64_t)d8;
+        strides[i][3] = 1;
+        strides[i][2] = d8;
+        strides[i][1] = (int64_t)t.shape[2] * d8;
+        strides[i][0] = (int64_t)t.shape[1] * strides[i][1];
+        copies[i] = NineToothedTensor{dense[i], shapes[i], strides[i]};
+    }
+    for (int i = 0; i < 3; ++i) {
+        const hipError_t err = size == 4 ? attention_pad<float>(stream, *ts[i], dense[i], d8, false) : attention_pad<uint16_t>(stream, *ts[i], dense[i], d8, false);
+        if (err != hipSuccess) return (int)err;
+    }
+    const int result = launch_attention(stream, copies[0], copies[1], copies[2], is_causal, scale, copies[3], dtype, block_size_m, block_size_n, false);
+    if (result != 0) return result;
+    return (int)(size == 4 ? attention_pad<float>(stream, o, dense[3], d8, true) : attention_pad<uint16_t>(stream, o, dense[3], d8, true));
+}
+
+int launch_attention(hipStream_t stream, const NineToothedTensor &q, const NineToothedTensor &k, const NineToothedTensor &v, const NineToothedTensor &is_causal,
+                     const NineToothedTensor &scale, const NineToothedTensor &o, int dtype, int block_size_m, int block_size_n, bool may_copy) {
     AttentionParams p;
     const int status = attention_setup(p, q, k, v, is_causal, scale, o, dtype);
+    if (status == NINETOOTHED_NO_KERNEL && may_copy) return attention_on_padded_copies(stream, q, k, v, is_causal, scale, o, dtype, block_size_m, block_size_n);
     if (status != 0) return status < 0 ? 0 : status;
     const int head_dim = p.head_dim;
     if (dtype == NINETOOTHED_FLOAT32) return attention_float32(p, head_dim, k, v, block_size_m == 0 && block_size_n == 0, (hipStream_t)stream);
@@ -1299,8 +1385,20 @@ extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineT
             if (tuned >= 0 && tuned < kAttentionVariants) variant = tuned;
         }
     }
-    if (dtype == NINETOOTHED_FLOAT16) return dispatch_attention<half_t>(p, head_dim, variant, (hipStream_t)stream);
-    return dispatch_attention<bf16_t>(p, head_dim, variant, (hipStream_t)stream);
+    int result;
+    if (dtype == NINETOOTHED_FLOAT16) result = dispatch_attention<half_t>(p, head_dim, variant, (hipStream_t)stream);
+    else result = dispatch_attention<bf16_t>(p, head_dim, variant, (hipStream_t)stream);
+    return result;
+}
+
+}  // namespace
+}  // namespace nt
+
+extern "C" NineToothedResult launch_nt_attention(NineToothedStream stream, NineToothedTensor q, NineToothedTensor k,
+                                                 NineToothedTensor v, NineToothedTensor is_causal,
+                                                 NineToothedTensor scale, NineToothedTensor o, int dtype,
+                                                 int block_size_m, int block_size_n) {
+    return launch_attention((hipStream_t)stream, q, k, v, is_causal, scale, o, dtype, block_size_m, block_size_n, true);
 }
 
 // Times the loop variants of launch_nt_attention on this problem and records the fastest for later launches
@@ -1313,6 +1411,7 @@ extern "C" NineToothedResult nt_tune_attention(NineToothedStream stream, NineToo
     if (best_ms) *best_ms = 0.0f;
     AttentionParams p;
     const int status = attention_setup(p, q, k, v, is_causal, scale, o, dtype);
+    if (status == NINETOOTHED_NO_KERNEL) return 0;  // (tensors that launch_nt_attention runs on padded copies: no alternatives)
     if (status != 0) return status < 0 ? 0 : status;
     if (!attention_tunable(p, dtype) || attention_would_split(p)) return 0;
     int best = -1;

@@ -19,7 +19,7 @@ namespace nt {
 enum WorkspacePurpose {
     kWorkspaceConvInput, kWorkspaceConvFilter, kWorkspaceAttentionNarrow, kWorkspaceGemmParts, kWorkspaceAttentionParts,
     kWorkspaceGemmLhsWidened, kWorkspaceGemmRhsWidened, kWorkspaceGemmBiasWidened, kWorkspaceGemmLhsDense, kWorkspaceGemmRhsDense,
-    kWorkspacePurposes
+    kWorkspaceAttentionPaddedQ, kWorkspaceAttentionPaddedK, kWorkspaceAttentionPaddedV, kWorkspaceAttentionPaddedO, kWorkspacePurposes
 };
 
 // Holds the registry lock from construction to destruction: create it, take the buffers,

@@ -1320,6 +1320,35 @@ def test_addmm_float8_e5m2_operands():
     assert np.allclose(out.cpu().float().numpy(), reference, **HALF_TOL)
 
 
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16, torch.float32))
+@pytest.mark.parametrize("is_causal", (False, True))
+def test_attention_tensors_the_kernels_cannot_read_in_place_run_on_padded_copies(is_causal, dtype):
+    """Head dimensions that are no multiples of 8 (the reference pads them to a power of two and masks:
+    src/ninetoothed/generation.py:563-574), rows off 16-byte boundaries, a strided last dimension: Q, K and V are
+    copied into padded dense buffers, O is copied back.  The tensors lie inside Inf-filled buffers (nothing next to
+    them may reach the sums) and O inside sentinels."""
+    tolerance = dict(rtol=1e-3, atol=1e-3) if dtype == torch.float32 else HALF_TOL
+    kernel = ninetoothed.make(programs.attention.arrangement_with_scale, programs.attention.application_with_scale, programs.attention.tensors(with_scale=True))
+
+    def inside(b, h, s, d, pad=3, step=1):
+        buffer = torch.full((b, h, s + 1, d * step + pad), float("inf"), dtype=dtype, device="cuda")
+        view = buffer[:, :, :s, 1 : 1 + d * step : step]
+        view.copy_(torch.randn(b, h, s, d, device="cuda").to(dtype))
+        return view
+
+    for (b, h, sq, sk, d, step) in ((2, 3, 200, 200, 100, 1), (1, 4, 130, 77, 20, 1), (2, 2, 64, 300, 12, 1), (1, 2, 257, 257, 64, 1), (1, 2, 100, 100, 36, 2), (1, 1, 50, 50, 250, 1)):
+        if is_causal and sq != sk:
+            continue
+        q, k, v = inside(b, h, sq, d, step=step), inside(b, h, sk, d, step=step), inside(b, h, sk, d, step=step)
+        buffer = torch.full((b, h, sq + 1, d + 5), 7.0, dtype=dtype, device="cuda")
+        o = buffer[:, :, :sq, 2 : 2 + d]
+        kernel(q, k, v, is_causal, d**-0.5, o)
+        _native_only(kernel, "launch_nt_attention")
+        expected = _attention_reference(q, k, v, is_causal, d**-0.5)
+        assert torch.allclose(o.float(), expected, **tolerance), (b, h, sq, sk, d, float((o.float() - expected).abs().max()))
+        assert bool((buffer[:, :, sq:] == 7.0).all()) and bool((buffer[:, :, :, :2] == 7.0).all()) and bool((buffer[:, :, :, 2 + d :] == 7.0).all())
+
+
 @pytest.mark.parametrize("is_causal", (False, True))
 @pytest.mark.parametrize("seq_len", (1024, 1))
 def test_attention_float32_tensors(seq_len, is_causal):
