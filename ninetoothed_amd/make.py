@@ -269,7 +269,7 @@ class Kernel:
         if kind == "conv2d":
             if out_tag != tag or cast not in (None, tag):
                 raise UnsupportedProgram("conv2d needs input, filter and output of one element type.")
-            return self._conv2d_plan(info, tag)
+            return self._conv2d_plan(info, tag, args)
         if cast is not None and cast != out_tag:
             raise UnsupportedProgram(f"The application rounds to `{cast}` but the output tensor holds `{out_tag}`.")
         if out_tag not in (tag, "fp32"):
@@ -388,7 +388,7 @@ class Kernel:
 
         return _Plan(f"launch_nt_matmul {m}x{n}x{k} {tag}->{out_tag} blocks {blocks}", launch)
 
-    def _conv2d_plan(self, info, tag):
+    def _conv2d_plan(self, info, tag, args):
         lib = runtime.library()
         dtype = runtime.DATA_TYPE_INDEX[tag]
         pad_h, pad_w = info["pad_h"], info["pad_w"]
@@ -397,8 +397,10 @@ class Kernel:
         if steps != (1, 1, 1, 1) or not info.get("fits", True):
             # windows that move by more than one position, taps that lie apart, or one window hanging over the edge
 
+            x, w, y = (runtime.ArgumentTensor.like(tensor) for tensor in args)  # (a plan serves one layout: only the addresses change)
+
             def launch_strided(call_args):
-                x, w, y = (runtime.ArgumentTensor.from_torch_tensor(tensor) for tensor in call_args)
+                x.data, w.data, y.data = call_args[0].data_ptr(), call_args[1].data_ptr(), call_args[2].data_ptr()
                 runtime.check(lib.launch_nt_conv2d_strided(runtime.current_stream(), x, w, y, dtype, pad_h, pad_w, *steps, *blocks))
 
             return _Plan(
@@ -412,8 +414,10 @@ class Kernel:
         if state["tune"]:
             auto_tuner.load_once()
 
+        x, w, y = (runtime.ArgumentTensor.like(tensor) for tensor in args)  # (a plan serves one layout: only the addresses change)
+
         def launch(call_args):
-            x, w, y = (runtime.ArgumentTensor.from_torch_tensor(tensor) for tensor in call_args)
+            x.data, w.data, y.data = call_args[0].data_ptr(), call_args[1].data_ptr(), call_args[2].data_ptr()
             if state["tune"]:
                 state["tune"] = False
                 out = call_args[2]
@@ -433,8 +437,10 @@ class Kernel:
         dtype = runtime.DATA_TYPE_INDEX[tag]
         block = info["input"]["block"]
 
+        input, output = (runtime.ArgumentTensor.like(tensor) for tensor in args[:2])  # (a plan serves one layout: only the addresses change)
+
         def launch(call_args):
-            input, output = (runtime.ArgumentTensor.from_torch_tensor(tensor) for tensor in call_args)
+            input.data, output.data = call_args[0].data_ptr(), call_args[1].data_ptr()
             runtime.check(lib.launch_nt_softmax(runtime.current_stream(), input, output, dtype, block))
 
         return _Plan(f"launch_nt_softmax {info['input']['rows']}x{info['input']['cols']} {tag} block {block}", launch)
@@ -544,10 +550,17 @@ class Kernel:
         if state["tune"]:
             auto_tuner.load_once()
 
+        positions = (0, 1, 2, o_pos)
+        tensors = [runtime.ArgumentTensor.like(args[p]) for p in positions]  # (a plan serves one layout: only the addresses change)
+        causal, causal_value = runtime.ArgumentTensor.scalar_slot(int)
+        scale_arg, scale_value = runtime.ArgumentTensor.scalar_slot(float) if scaled else (runtime.ArgumentTensor.null(), None)
+
         def launch(call_args):
-            tensors = [runtime.ArgumentTensor.from_torch_tensor(call_args[p]) for p in (0, 1, 2, o_pos)]
-            causal = runtime.ArgumentTensor.from_scalar(int(bool(call_args[3])))
-            scale_arg = runtime.ArgumentTensor.from_scalar(float(call_args[4])) if scaled else runtime.ArgumentTensor.null()
+            for tensor, p in zip(tensors, positions):
+                tensor.data = call_args[p].data_ptr()
+            causal_value.value = int(bool(call_args[3]))
+            if scaled:
+                scale_value.value = float(call_args[4])
             if state["tune"]:
                 state["tune"] = False
                 out = call_args[o_pos]

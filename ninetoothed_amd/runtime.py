@@ -55,6 +55,21 @@ class ArgumentTensor(ctypes.Structure):
         return argument
 
     @staticmethod
+    def like(tensor):
+        """The layout of ``tensor`` without its address: a launch that serves one (shape, strides) signature keeps
+        such an argument and only sets ``data`` per call."""
+        return ArgumentTensor.from_layout(0, tuple(tensor.shape), tuple(tensor.stride()))
+
+    @staticmethod
+    def scalar_slot(kind):
+        """A zero-dimensional tensor over a host buffer that stays (``float`` -> double, ``int`` -> int64); returns
+        the argument and the buffer, whose ``value`` a launch sets per call."""
+        buffer = ctypes.c_double(0.0) if kind is float else ctypes.c_int64(0)
+        argument = ArgumentTensor(ctypes.addressof(buffer), None, None)
+        argument._keepalive = buffer
+        return argument, buffer
+
+    @staticmethod
     def from_scalar(value):
         """A zero-dimensional tensor: host double for floats, host int64 otherwise."""
         buffer = ctypes.c_double(value) if isinstance(value, float) else ctypes.c_int64(int(value))
