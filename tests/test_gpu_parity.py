@@ -1025,6 +1025,72 @@ def test_conv2d_one_launch_path_leaves_overlapping_images_to_the_other_ways():
     assert runtime.library().launch_nt_conv2d(runtime.current_stream(), *tensors, fp16, 1, 1, 3, 0, 0) == runtime.NO_KERNEL
 
 
+@pytest.mark.skipif(not hasattr(torch, "float8_e5m2"), reason="this torch has no float8_e5m2")
+def test_calls_that_run_on_copies_inside_a_captured_graph():
+    """fp8 operands, operands the direct-to-LDS kernels cannot read in place and attention tensors with an odd head
+    dimension run on copies in scratch buffers.  A capture that meets such a call before any eager call of its size
+    cannot allocate: the products then take the kernels that need no scratch memory (an attention call of this kind
+    has none and would be refused there), and after one eager call on the stream a capture of the same calls uses its
+    buffers.
+    Every replay is checked against the eager result, with eager work between the replays."""
+    from ninetoothed_amd import runtime
+
+    matmul = _matmul_kernel()
+    attention = ninetoothed.make(programs.attention.arrangement_with_scale, programs.attention.application_with_scale, programs.attention.tensors(with_scale=True))
+    m, n, k = 1544, 1160, 1208  # sizes no other test uses; 2^31 multiply-adds and more
+    a8 = torch.randn(m, k, device="cuda").to(torch.float8_e5m2)
+    b8 = torch.randn(k, n, device="cuda").to(torch.float8_e5m2)
+    a_off = torch.randn(m, k + 1, dtype=torch.float16, device="cuda")[:, :k]  # rows off 16-byte boundaries
+    b16 = torch.randn(k, n, dtype=torch.float16, device="cuda")
+    q, kk, v = (torch.randn(2, 3, 150, 44, dtype=torch.float16, device="cuda") for _ in range(3))
+    c8, c16 = torch.empty(m, n, dtype=torch.float16, device="cuda"), torch.empty(m, n, dtype=torch.float16, device="cuda")
+    o = torch.empty_like(q)
+    expected8 = a8.to(torch.float16).float() @ b8.to(torch.float16).float()
+    expected16 = a_off.float() @ b16.float()
+    expected_o = _attention_reference(q, kk, v, False, 44**-0.5)
+    tolerance = dict(rtol=1e-2, atol=1e-2 * (k / 512) ** 0.5)
+
+    def products():
+        matmul(a8, b8, c8)
+        matmul(a_off, b16, c16)
+
+    def replay_and_check(graph, with_attention):
+        for replay in range(3):
+            for t in (c8, c16, o):
+                t.fill_(float("nan"))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.allclose(c8.float(), expected8, **tolerance), replay
+            assert torch.allclose(c16.float(), expected16, **tolerance), replay
+            if with_attention:
+                assert torch.allclose(o.float(), expected_o, **HALF_TOL), replay
+            (a_off.float() @ b16.float()).sum().item()  # eager work between the replays
+
+    runtime.library().nt_release_workspaces()  # no buffer of any size exists
+    stream = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    first = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(first, stream=stream):
+        products()
+        assert "any-stride" in runtime.last_launch(), runtime.last_launch()  # no scratch memory: the kernel that gathers in place
+    replay_and_check(first, with_attention=False)
+    # eager calls on that stream allocate its buffers (they are kept per stream) ...
+    with torch.cuda.stream(stream):
+        products()
+        assert "any-stride" not in runtime.last_launch(), runtime.last_launch()
+        attention(q, kk, v, False, 44**-0.5, o)
+    torch.cuda.synchronize()
+    assert torch.allclose(o.float(), expected_o, **HALF_TOL)
+    # ... and a capture of the same calls then runs on the copies
+    second = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(second, stream=stream):
+        products()
+        assert "any-stride" not in runtime.last_launch(), runtime.last_launch()
+        attention(q, kk, v, False, 44**-0.5, o)
+    replay_and_check(second, with_attention=True)
+
+
 def test_first_call_of_an_untuned_problem_inside_a_captured_graph():
     """Nothing has run these problems before the capture starts: the first-launch tuner of the product
     (event synchronisation, repeated launches) and the specialisation of the tile map (compiling and
