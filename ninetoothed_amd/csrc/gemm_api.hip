@@ -534,32 +534,59 @@ int run_gemm(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk, b
 // the lhs as [M][K8], the rhs as [N][K8], K8 = K rounded up to 8 with zeros in between, which add nothing to the sums --
 // and the product runs on the instances with tails, which take a k-contiguous rhs with any N.
 // dst[i][j] = j < d1 ? src[i * s0 + j * s1] : 0 for j < pitch; 64 x 64 tiles through LDS, so that the reads run along
-// whichever dimension has the smaller stride and the writes along j
+// whichever dimension has the smaller stride and the writes along j, 16 bytes per lane on both sides where the
+// source is contiguous along that dimension
 __global__ __launch_bounds__(256) void repack_operand_kernel(const uint16_t *src, int64_t d0, int64_t d1, int64_t s0, int64_t s1, uint16_t *dst, int64_t pitch) {
-    __shared__ uint16_t tile[64][66];
+    typedef uint16_t ushort8_t __attribute__((ext_vector_type(8)));
+    typedef ushort8_t unaligned_ushort8_t __attribute__((aligned(2)));  // (global accesses need the element's alignment only)
+    constexpr int kPitch = 72;  // rows of the tile start on 16-byte boundaries
+    __shared__ __attribute__((aligned(16))) uint16_t tile[64 * kPitch];
     const int64_t tiles_j = (pitch + 63) / 64;
     const int64_t i0 = (int64_t)(blockIdx.x / tiles_j) * 64, j0 = (int64_t)(blockIdx.x % tiles_j) * 64;
     const int t = threadIdx.x;
     const bool along_i = s0 < s1;  // consecutive threads read consecutive i
+    const int64_t fast_stride = along_i ? s0 : s1;
+    if (fast_stride != 1) {  // (uniform) no dimension is contiguous: consecutive threads fetch consecutive elements
 #pragma unroll 4
-    for (int e = t; e < 64 * 64; e += 256) {
-        const int fast = e & 63, slow = e >> 6;
+        for (int e = t; e < 64 * 64; e += 256) {
+            const int fast = e & 63, slow = e >> 6;
+            const int i = along_i ? fast : slow, j = along_i ? slow : fast;
+            uint16_t value = 0;
+            if (i0 + i < d0 && j0 + j < d1) value = src[(i0 + i) * s0 + (j0 + j) * s1];
+            tile[i * kPitch + j] = value;
+        }
+    } else
+    // eight consecutive elements of the source's contiguous dimension per thread, in one load
+#pragma unroll
+    for (int e = t; e < 64 * 8; e += 256) {
+        const int fast = (e & 7) * 8, slow = e >> 3;
         const int i = along_i ? fast : slow, j = along_i ? slow : fast;
-        uint16_t value = 0;
-        if (i0 + i < d0 && j0 + j < d1) value = src[(i0 + i) * s0 + (j0 + j) * s1];
-        tile[i][j] = value;
+        const int64_t limit = along_i ? d0 - (i0 + i) : d1 - (j0 + j);  // elements left along the faster dimension
+        const bool slow_inside = along_i ? j0 + j < d1 : i0 + i < d0;
+        ushort8_t values = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (slow_inside && limit > 0) {
+            const uint16_t *from = src + (i0 + i) * s0 + (j0 + j) * s1;
+            if (fast_stride == 1 && limit >= 8) {
+                values = *(const unaligned_ushort8_t *)from;
+            } else {
+#pragma unroll
+                for (int c = 0; c < 8; ++c)
+                    if (c < limit) values[c] = from[c * fast_stride];
+            }
+        }
+        if (along_i) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) tile[(i + c) * kPitch + j] = values[c];
+        } else {
+            *(ushort8_t *)&tile[i * kPitch + j] = values;
+        }
     }
     __syncthreads();
-    // four consecutive j per thread: 8-byte stores (pitch is a multiple of 8, so is j0 + 4 * quad)
-    typedef uint16_t ushort4_t __attribute__((ext_vector_type(4)));
-#pragma unroll 4
-    for (int e = t; e < 64 * 16; e += 256) {
-        const int quad = e & 15, i = e >> 4;
-        if (i0 + i >= d0 || j0 + 4 * quad >= pitch) continue;
-        ushort4_t out;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) out[c] = tile[i][4 * quad + c];
-        *(ushort4_t *)(dst + (i0 + i) * pitch + j0 + 4 * quad) = out;
+    for (int e = t; e < 64 * 8; e += 256) {
+        const int j = (e & 7) * 8, i = e >> 3;
+        if (i0 + i >= d0 || j0 + j >= pitch) continue;  // (pitch is a multiple of 8: whole vectors)
+        *(ushort8_t *)(dst + (i0 + i) * pitch + j0 + j) = *(const ushort8_t *)&tile[i * kPitch + j];
     }
 }
 
