@@ -1281,23 +1281,45 @@ namespace {
 template <typename E>
 __global__ __launch_bounds__(256) void attention_pad_kernel(const E *src, E *dst, int64_t rows, int heads, int seq, int d, int d8, int64_t s0, int64_t s1,
                                                             int64_t s2, int64_t s3, int back) {
-    // back == 0: dst[row][0 .. d8) = src row, zero padded; back != 0: the first d columns of the dense `src` rows go to `dst`
-    const int64_t total = rows * (back ? d : d8);
+    // back == 0: dst[row][0 .. d8) = src row, zero padded; back != 0: the first d columns of the dense `src` rows go to `dst`.
+    // One thread per 8 columns of a row: one load and one store of 8 elements where the strided side is contiguous
+    // (global accesses need the element's alignment only), element by element otherwise.
+    typedef E vec8 __attribute__((ext_vector_type(8)));
+    typedef vec8 unaligned_vec8 __attribute__((aligned(sizeof(E))));
+    const int chunks = d8 / 8;
+    const int64_t total = rows * chunks;
     for (int64_t index = (int64_t)blockIdx.x * 256 + threadIdx.x; index < total; index += (int64_t)gridDim.x * 256) {
-        const int width = back ? d : d8;
-        const int64_t row = index / width;
-        const int col = (int)(index - row * width);
+        const int64_t row = index / chunks;
+        const int col = (int)(index - row * chunks) * 8;
         const int64_t bh = row / seq;
         const int64_t strided = (bh / heads) * s0 + (bh % heads) * s1 + (row % seq) * s2 + (int64_t)col * s3;
-        if (back) dst[strided] = src[row * d8 + col];
-        else dst[index] = col < d ? src[strided] : (E)0;
+        const bool whole = s3 == 1 && col + 8 <= d;
+        if (back) {
+            const vec8 values = *(const vec8 *)(src + row * d8 + col);
+            if (whole) {
+                *(unaligned_vec8 *)(dst + strided) = values;
+            } else {
+#pragma unroll
+                for (int c = 0; c < 8; ++c)
+                    if (col + c < d) dst[strided + c * s3] = values[c];
+            }
+        } else {
+            vec8 values;
+            if (whole) {
+                values = *(const unaligned_vec8 *)(src + strided);
+            } else {
+#pragma unroll
+                for (int c = 0; c < 8; ++c) values[c] = col + c < d ? src[strided + c * s3] : (E)0;
+            }
+            *(vec8 *)(dst + row * d8 + col) = values;
+        }
     }
 }
 
 template <typename E>
 hipError_t attention_pad(hipStream_t stream, const NineToothedTensor &t, void *dense, int d8, bool back) {
     const int64_t rows = (int64_t)t.shape[0] * t.shape[1] * t.shape[2];
-    const int64_t work = rows * (back ? (int64_t)t.shape[3] : d8);
+    const int64_t work = rows * (d8 / 8);
     if (work == 0) return hipSuccess;
     const unsigned blocks = (unsigned)std::min<int64_t>((work + 255) / 256, 256 * 64);
     if (back)
