@@ -55,6 +55,15 @@ class _AliasFinder(importlib.abc.MetaPathFinder):
 if not any(isinstance(finder, _AliasFinder) for finder in sys.meta_path):
     sys.meta_path.insert(0, _AliasFinder())
 
+# `jit` and `eval` name a submodule AND a public function (src/ninetoothed/__init__.py:16-18 imports the functions
+# over the submodules).  The first import of a submodule binds it in its parent package, so both are imported here
+# once and the functions bound over them afterwards: a later `from ninetoothed.jit import jit` then finds the module
+# in `sys.modules` and leaves `ninetoothed.jit` the decorator.
+for _name in ("jit", "eval"):
+    importlib.import_module(_PREFIX + _name)
+jit = ninetoothed_amd.jit
+eval = ninetoothed_amd.eval  # noqa: A001
+
 
 def __getattr__(name):
     """``ninetoothed.<submodule>`` without an explicit import of the submodule."""

@@ -20,21 +20,14 @@ from ninetoothed_amd.dtype import (
     uint32,
     uint64,
 )
-from ninetoothed_amd.make import Kernel, jit, make
+from ninetoothed_amd.eval import _eval as eval  # noqa: A001  (the reference's public name, src/ninetoothed/__init__.py:16-17)
+from ninetoothed_amd.eval import _subs as subs
+from ninetoothed_amd.jit import jit  # (binds the decorator over the submodule of the same name, as the reference does)
+from ninetoothed_amd.make import Kernel, make
 from ninetoothed_amd.recognition import UnsupportedProgram
 from ninetoothed_amd.runtime import KernelLaunchError
 from ninetoothed_amd.symbol import Symbol, block_size
 from ninetoothed_amd.tensor import Tensor
-
-
-def eval(tensor, subs=None):
-    """Evaluates a symbolic tensor (see :meth:`Tensor.eval`)."""
-    return tensor.eval(subs)
-
-
-def subs(tensor, substitutions):
-    """Substitutes symbols in a tensor (see :meth:`Tensor.subs`)."""
-    return tensor.subs(substitutions)
 
 
 __all__ = [

@@ -167,3 +167,53 @@ def test_simulate_arrangement_matches_the_reference_vectors():
     for position in range(6):
         assert np.array_equal(sources[position].numpy(), vectors[position]), position
         assert np.array_equal(targets[position].numpy(), vectors[6 + position]), position
+
+
+def test_naming_prefixes_as_the_reference_spells_them():
+    """``ninetoothed.naming`` (reference tests/test_naming.py:4-49): the strings of the three kinds of prefix, that
+    they stack, that a meta name counts as a constant, and that removing them gives back the bare name -- also one
+    that itself starts with ``ninetoothed_``."""
+    import ninetoothed.naming as by_reference_name
+
+    from ninetoothed_amd import naming
+
+    assert by_reference_name is naming
+    name = "ninetoothed_name"
+    assert naming.make_constexpr(name) == "ninetoothed_constexpr_prefix_ninetoothed_name"
+    assert naming.make_meta(name) == "ninetoothed_meta_prefix_ninetoothed_name"
+    assert naming.make_next_power_of_2(name) == "ninetoothed_next_power_of_2_prefix_ninetoothed_name"
+    stacked = naming.make_next_power_of_2(naming.make_constexpr(name))
+    assert stacked == "ninetoothed_next_power_of_2_prefix_ninetoothed_constexpr_prefix_ninetoothed_name"
+    assert naming.is_constexpr(naming.make_constexpr(name)) and naming.is_constexpr(naming.make_meta(name)) and naming.is_constexpr(stacked)
+    assert naming.is_meta(naming.make_meta(name)) and not naming.is_meta(naming.make_constexpr(name))
+    assert naming.is_next_power_of_2(naming.make_next_power_of_2(name)) and naming.is_next_power_of_2(stacked)
+    assert not naming.is_constexpr(name) and not naming.is_meta(name) and not naming.is_next_power_of_2(name)
+    for mangled in (naming.make_constexpr(name), naming.make_meta(name), naming.make_next_power_of_2(name), stacked):
+        assert naming.remove_prefixes(mangled) == name
+    assert naming.remove_prefixes("x") == "x"
+    assert naming.auto_generate("libdevice") == "ninetoothed_libdevice"
+
+
+def test_submodules_that_share_a_name_with_a_public_function():
+    """``jit`` and ``eval`` are submodules and public functions at once in the reference
+    (src/ninetoothed/__init__.py:16-18); importing the submodule must not replace the function, under either
+    package name.  ``generation.CACHE_DIR`` and ``utils.calculate_default_configs`` are what the reference's
+    own tests and ``jit`` reach for in those modules (tests/test_aot.py:37, src/ninetoothed/jit.py:55-57)."""
+    import importlib
+    import pathlib
+
+    import ninetoothed
+    import ninetoothed.generation
+    import ninetoothed.utils
+    import ninetoothed_amd
+    from ninetoothed.eval import _eval, _subs
+    from ninetoothed.jit import jit
+
+    jit_module = importlib.import_module("ninetoothed.jit")
+    assert jit_module is importlib.import_module("ninetoothed_amd.jit")
+    assert jit is ninetoothed.jit is ninetoothed_amd.jit is jit_module.jit and callable(jit)
+    assert _eval is ninetoothed.eval is ninetoothed_amd.eval and _subs is ninetoothed.subs
+    assert isinstance(ninetoothed.generation.CACHE_DIR, pathlib.Path)
+    assert ninetoothed.utils.calculate_default_configs() == (8, 5)
+    x = ninetoothed.Tensor(shape=(4, 6))
+    assert ninetoothed.eval(x.tile((2, 3))).shape == (2, 2, 2, 3)
