@@ -582,7 +582,7 @@ long long segment_offset_at(const NineToothedMapProgram &q, int segment, const l
 // Reductions whose reduced positions lie closer together in memory than the outputs do (row sums of a
 // row-major matrix) run with one wave per output element: the lanes stride the reduced positions, so
 // a wave reads consecutive elements, and combine their partial results with shuffles.  With one thread
-// per output the lanes of a wave would read a row each.  Returns the lanes per output element: 64 or 1.
+// per output the lanes of a wave would read a row each.  Returns the lanes per output element: 1, 64, or -- few outputs over long ranges -- the whole workgroup.
 int cooperative_lanes(const NineToothedMapProgram &q);
 
 // Threads of a workgroup.  In tile mode (one workgroup per tile) a tile of up to 16384 elements gets enough
@@ -631,7 +631,12 @@ int cooperative_lanes(const NineToothedMapProgram &q) {
         step_out = std::llabs(segment_offset_at(q, segment, vars) - base);
         vars[v] = 0;
     }
-    return step_reduced != 0 && (step_out == 0 || step_reduced < step_out) ? 64 : 1;
+    if (!(step_reduced != 0 && (step_out == 0 || step_reduced < step_out))) return 1;
+    // few outputs over long ranges (64 rows of a million elements): a wave per output would leave most of the chip
+    // idle, so the whole workgroup shares an output and its waves exchange their partial results through LDS
+    long long outputs = 1;
+    for (int v = 0; v < num_out; ++v) outputs *= q.extents[v];
+    return outputs <= 2048 && reduced >= 16384 ? kMapThreads : 64;
 }
 
 struct MapCodegen {
@@ -974,6 +979,7 @@ struct MapCodegen {
             << "    const nt_idx stride = (nt_idx)gridDim.x * " << kMapThreads << ";\n"
             << "    const nt_idx total_out = (nt_idx)a.total_out;\n";
         if (p.num_phases > 0) return generate_tile();
+        if (lanes > 64) out << "    __shared__ double nt_partial[" << lanes / 64 << "];\n";
         if (lanes > 1)
             out << "    const nt_idx lane = threadIdx.x & " << lanes - 1 << ";\n"
                 << "    for (nt_idx element = ((nt_idx)blockIdx.x * " << kMapThreads << " + threadIdx.x) / " << lanes << "; element < total_out; element += stride / " << lanes << ") {\n"
@@ -993,6 +999,8 @@ struct MapCodegen {
             long long reduced_total = 1;
             for (int v = num_out; v < p.num_vars; ++v) reduced_total *= p.extents[v];
             if (lanes > 1) {  // the lanes of a wave stride the reduced positions
+                // (few waves per output: the loads of several iterations have to be in flight at once)
+                if (lanes > 64) out << indent << "#pragma unroll 8\n";
                 out << indent << "for (nt_idx position = lane; position < " << lit(reduced_total) << "; position += " << lanes << ") {\n";
                 indent += "    ";
                 out << indent << "nt_uidx inner = (nt_uidx)position;\n";
@@ -1013,8 +1021,16 @@ struct MapCodegen {
             if (lanes > 1) {
                 indent.resize(indent.size() - 4);
                 out << indent << "}\n";
-                for (int offset = lanes / 2; offset > 0; offset >>= 1)
+                for (int offset = 32; offset > 0; offset >>= 1)
                     out << indent << "{ const double other = __shfl_xor(acc, " << offset << ", 64); acc = " << combine_expr(p.reduce_op, p.reduce_dtype, "acc", "other") << "; }\n";
+                if (lanes > 64) {  // the waves of the workgroup (all of them work on this element: the loop is uniform)
+                    out << indent << "if ((threadIdx.x & 63) == 0) nt_partial[threadIdx.x >> 6] = acc;\n"
+                        << indent << "__syncthreads();\n"
+                        << indent << "acc = nt_partial[0];\n";
+                    for (int w = 1; w < lanes / 64; ++w)
+                        out << indent << "{ const double other = nt_partial[" << w << "]; acc = " << combine_expr(p.reduce_op, p.reduce_dtype, "acc", "other") << "; }\n";
+                    out << indent << "__syncthreads();\n";
+                }
             } else
             for (int v = num_out; v < p.num_vars; ++v) {
                 indent.resize(indent.size() - 4);

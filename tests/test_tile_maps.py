@@ -401,6 +401,31 @@ def test_row_sum():
     assert torch.allclose(out, x.sum(dim=1) * 2, rtol=1e-4, atol=1e-4)
 
 
+def _row_max_application(input, output):
+    output = ntl.max(input) - 1.0  # noqa: F841
+
+
+@gpu
+@pytest.mark.parametrize("rows, cols", ((3, 100003), (64, 16384), (2048, 16385), (1, 1 << 20)))
+def test_few_long_rows_are_reduced_by_whole_workgroups(rows, cols):
+    """Few outputs over long ranges: the workgroup shares an output, its waves exchange partial results through
+    LDS (one wave per output otherwise).  Sums against float64, maxima exactly, a NaN in a row reaches its maximum."""
+    x = torch.randn(rows, cols, device="cuda")
+    out = torch.empty(rows, device="cuda")
+    kernel = ninetoothed.make(row_sum_arrangement, row_sum_application, (Tensor(2), Tensor(1)))
+    kernel(x, out)
+    _served_by_map(kernel)
+    assert torch.allclose(out.double(), x.double().sum(dim=1) * 2, rtol=1e-5, atol=1e-2)
+    kernel = ninetoothed.make(row_sum_arrangement, _row_max_application, (Tensor(2, other=float("-inf")), Tensor(1)))
+    x[rows - 1, cols // 3] = 1000.0
+    if rows > 1:
+        x[0, cols - 1] = float("nan")
+    kernel(x, out)
+    _served_by_map(kernel)
+    expected = x.max(dim=1).values - 1.0
+    assert torch.equal(out.isnan(), expected.isnan()) and torch.equal(out.nan_to_num(0.0), expected.nan_to_num(0.0))
+
+
 @gpu
 def test_empty_tensor_and_no_store():
     def arrangement(x):
