@@ -127,6 +127,63 @@ __global__ __launch_bounds__(kRowThreads > 256 ? kRowThreads : 256) void softmax
     }
 }
 
+// Rows of up to 64 bytes (a softmax over 4 or 8 classes, for millions of rows): one THREAD per row.  A group of
+// 8 lanes per row, the smallest the vector path has, leaves most lanes without a vector on such rows.  A thread
+// fetches its row in pieces of kBytes (the largest power of two that divides the row's bytes and its pitch),
+// consecutive threads consecutive rows.
+template <typename T, int kBytes>
+__global__ __launch_bounds__(256) void softmax_thread_per_row_kernel(SoftmaxParams p, int pieces) {
+    constexpr int kWidth = kBytes / (int)sizeof(T);  // elements per piece
+    constexpr int kMaxPieces = 64 / kBytes;
+    typedef T piece_t __attribute__((ext_vector_type(kWidth)));
+    const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (row >= p.rows) return;
+    const piece_t *src = (const piece_t *)((const T *)p.in + row * p.in_row_stride);
+    piece_t *dst = (piece_t *)((T *)p.out + row * p.out_row_stride);
+    float x[kMaxPieces][kWidth];
+    float m = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < kMaxPieces; ++j) {
+        if (j < pieces) {
+            const piece_t raw = src[j];
+#pragma unroll
+            for (int e = 0; e < kWidth; ++e) {
+                x[j][e] = (float)raw[e];
+                m = fmaxf(m, x[j][e]);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < kWidth; ++e) x[j][e] = -INFINITY;
+        }
+    }
+    const float shift = m * kLog2e;
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kMaxPieces; ++j)
+#pragma unroll
+        for (int e = 0; e < kWidth; ++e) {
+            x[j][e] = __builtin_amdgcn_exp2f(fmaf(x[j][e], kLog2e, -shift));  // (as in softmax_vec_kernel)
+            s += x[j][e];
+        }
+    const float inv = 1.0f / s;
+#pragma unroll
+    for (int j = 0; j < kMaxPieces; ++j) {
+        if (j < pieces) {
+            piece_t o;
+#pragma unroll
+            for (int e = 0; e < kWidth; ++e) o[e] = (T)(x[j][e] * inv);
+            dst[j] = o;
+        }
+    }
+}
+
+template <typename T, int kBytes>
+hipError_t launch_thread_per_row(const SoftmaxParams &p, hipStream_t stream) {
+    note_launch(kLaunchSoftmax, 1, "softmax_thread_per_row_kernel, rows of up to 64 bytes");
+    softmax_thread_per_row_kernel<T, kBytes><<<dim3((unsigned)((p.rows + 255) / 256)), dim3(256), 0, stream>>>(p, (int)(p.cols * (int64_t)sizeof(T) / kBytes));
+    return hipGetLastError();
+}
+
 // Element path: any strides / alignment / length up to kRowThreads * kElems.
 template <typename T, int kRowThreads, int kElems>
 __global__ __launch_bounds__(kRowThreads > 256 ? kRowThreads : 256) void softmax_elem_kernel(SoftmaxParams p) {
@@ -267,6 +324,18 @@ int run_softmax(const SoftmaxParams &p, int variant, hipStream_t stream) {
     const bool vector_ok = p.in_col_stride == 1 && p.out_col_stride == 1 && p.cols % W == 0 &&
                            (p.segments == 1 || p.block % W == 0) && p.in_row_stride % W == 0 &&
                            p.out_row_stride % W == 0 && ((uintptr_t)p.in & 15) == 0 && ((uintptr_t)p.out & 15) == 0;
+    // rows of up to 64 bytes, many of them: a thread per row
+    if (variant == 0 && p.segments == 1 && p.in_col_stride == 1 && p.out_col_stride == 1 && p.cols * (int64_t)sizeof(T) <= 64 && p.rows >= 4096 &&
+        (p.rows + 255) / 256 <= 0x7fffffffll) {
+        const uint64_t bits = (uint64_t)(p.cols * sizeof(T)) | (uint64_t)(p.in_row_stride * (int64_t)sizeof(T)) | (uint64_t)(p.out_row_stride * (int64_t)sizeof(T)) |
+                              (uint64_t)(uintptr_t)p.in | (uint64_t)(uintptr_t)p.out;  // what every piece's address and size is a multiple of
+        if (bits % 16 == 0) return (int)launch_thread_per_row<T, 16>(p, stream);
+        if (bits % 8 == 0) return (int)launch_thread_per_row<T, 8>(p, stream);
+        if (bits % 4 == 0) return (int)launch_thread_per_row<T, 4>(p, stream);
+        if constexpr (sizeof(T) == 2) {
+            if (p.cols <= 8) return (int)launch_thread_per_row<T, 2>(p, stream);  // (up to 32 pieces of one element would not stay in registers)
+        }
+    }
     if (vector_ok && len <= (int64_t)1024 * 16 * W) {
         const bool wave_fits = len <= (int64_t)64 * 16 * W;
         bool use_wave = wave_fits && len <= (int64_t)64 * 8 * W;  // default: keep <= 8 vectors per lane

@@ -353,6 +353,36 @@ def test_softmax_short_rows_few_rows_and_long_rows(m, n, dtype):
     assert bool((buffer[:, n:] == 7.0).all())
 
 
+@pytest.mark.parametrize("dtype", (torch.float32, torch.float16, torch.bfloat16))
+@pytest.mark.parametrize("n", (1, 2, 3, 4, 5, 8, 10, 16, 17, 32))
+def test_softmax_many_rows_of_a_few_elements(n, dtype):
+    """Rows of up to 64 bytes, at least 4096 of them: one thread per row, fetched in the largest pieces that the
+    row's bytes, the pitches and the addresses allow.  Input and output lie in sentinel-filled buffers with pitches
+    of their own, once aligned and once one element off."""
+    from ninetoothed_amd import runtime
+
+    m = 5000
+    tolerance = {torch.float32: dict(rtol=1e-5, atol=1e-6), torch.float16: dict(rtol=2e-3, atol=1e-4), torch.bfloat16: dict(rtol=1.6e-2, atol=1e-3)}[dtype]
+    kernel = ninetoothed.make(programs.softmax.arrangement, programs.softmax.application, programs.softmax.tensors())
+    for pitch, first in ((n, 0), (n + 8, 0), (n + 3, 1)):
+        source = torch.full((m, pitch), float("inf"), dtype=dtype, device="cuda")
+        x = source[:, first : first + n]
+        x.copy_(torch.randn(m, n, device="cuda").to(dtype))
+        x[0, 0] = 30.0
+        if n > 1:
+            x[1, n // 2 :] = float("-inf")
+        buffer = torch.full((m, pitch), 7.0, dtype=dtype, device="cuda")
+        out = buffer[:, first : first + n]
+        kernel(x, out, BLOCK_SIZE=1 << (n - 1).bit_length() if n > 1 else 1)
+        _native_only(kernel, "launch_nt_softmax")
+        size = x.element_size()
+        common = n * size | pitch * size | first * size  # every piece's offset and size is a multiple of its lowest set bit
+        if n * size <= 64 and (common % 4 == 0 or (size == 2 and n <= 8)):
+            assert "thread_per_row" in runtime.last_launch(), runtime.last_launch()
+        assert torch.allclose(out.float(), torch.softmax(x.float(), dim=-1), **tolerance), (pitch, first)
+        assert bool((buffer[:, :first] == 7.0).all()) and bool((buffer[:, first + n :] == 7.0).all())
+
+
 def test_softmax_jit_decorator_form():
     # the decorator form with annotated parameters, as in the reference's tests/test_softmax.py:10-27
     import ninetoothed_amd.language as ntl
