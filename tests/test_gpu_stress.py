@@ -297,3 +297,69 @@ def test_mfma_rate_probe_runs_and_counts():
     assert count.value == units * 8 * 3 * 32
     assert sink.item() == 0.0
     assert lib.nt_probe_mfma_rate_16x16x32(runtime.current_stream(), small, small, 3, sink.data_ptr(), ctypes.byref(count)) != 0
+
+
+@pytest.mark.skipif(not hasattr(torch, "float8_e5m2"), reason="this torch has no float8_e5m2")
+def test_calls_that_share_scratch_buffers_from_several_host_threads():
+    """Split-K partial products, the fp16 copies of fp8 operands, dense copies of misaligned operands, padded copies
+    of attention tensors and conv2d's repacked operands all live in one buffer per (device, stream, purpose).  Four
+    host threads enqueue such calls onto the SAME stream with sizes of their own: the registry lock must keep a
+    call's copies and the kernel that reads them together (a buffer overwritten in between shows as wrong values),
+    also when a buffer has to grow in the middle."""
+    import threading
+
+    stream = torch.cuda.current_stream()
+    matmul = ninetoothed.make(programs.matmul.arrangement, programs.matmul.application, programs.matmul.tensors())
+    attention = ninetoothed.make(programs.attention.arrangement_with_scale, programs.attention.application_with_scale, programs.attention.tensors(with_scale=True))
+    conv = ninetoothed.make(programs.conv2d.arrangement, programs.conv2d.application, programs.conv2d.tensors())
+    failures = []
+
+    def worker(seed):
+        try:
+            with torch.cuda.stream(stream):
+                generator = torch.Generator(device="cuda").manual_seed(seed)
+
+                def randn(*shape, dtype=torch.float16, scale=1.0):
+                    return (torch.randn(*shape, device="cuda", generator=generator) * scale).to(dtype)
+
+                m = 1024 + 256 * seed
+                skinny_a, skinny_b = randn(16, 4096 + 512 * seed), randn(4096 + 512 * seed, 2048)  # few tiles, long K: split K
+                a8, b8 = randn(m, 512).to(torch.float8_e5m2), randn(512, 768).to(torch.float8_e5m2)
+                a_off, b16 = randn(2048 + 8 * seed, 1025)[:, :1024], randn(1024, 1024)  # rows off 16-byte boundaries, 2^31 multiply-adds
+                q, k, v = (randn(1, 2 + seed, 96, 20 + 4 * seed) for _ in range(3))
+                x, w = randn(2, 3 + seed, 20, 24, scale=0.3), randn(16, 3 + seed, 3, 3, scale=0.3)
+                expected = (
+                    skinny_a.float() @ skinny_b.float(),
+                    a8.to(torch.float16).float() @ b8.to(torch.float16).float(),
+                    a_off.float() @ b16.float(),
+                    torch.softmax((q.float() * q.shape[-1] ** -0.5) @ k.float().transpose(-1, -2), dim=-1) @ v.float(),
+                    F.conv2d(x.float(), w.float(), padding=1),
+                )
+                for _ in range(6):
+                    outs = (
+                        torch.full((16, 2048), float("nan"), dtype=torch.float16, device="cuda"),
+                        torch.full((m, 768), float("nan"), dtype=torch.float16, device="cuda"),
+                        torch.full((a_off.shape[0], 1024), float("nan"), dtype=torch.float16, device="cuda"),
+                        torch.full_like(q, float("nan")),
+                        torch.full((2, 16, 20, 24), float("nan"), dtype=torch.float16, device="cuda"),
+                    )
+                    matmul(skinny_a, skinny_b, outs[0])
+                    matmul(a8, b8, outs[1])
+                    matmul(a_off, b16, outs[2])
+                    attention(q, k, v, False, q.shape[-1] ** -0.5, outs[3])
+                    conv(x, w, outs[4], padding_h=1, padding_w=1)
+                    tolerances = (dict(rtol=1e-2, atol=1e-2 * (skinny_a.shape[1] / 512) ** 0.5), dict(rtol=1e-2, atol=1e-2), dict(rtol=1e-2, atol=1e-2 * 2**0.5), HALF_TOL, HALF_TOL)
+                    for index, (out, reference, tolerance) in enumerate(zip(outs, expected, tolerances)):
+                        if not torch.allclose(out.float(), reference, **tolerance):
+                            failures.append((seed, index, float((out.float() - reference).abs().max())))
+                            return
+        except Exception as error:  # noqa: BLE001  (a worker's exception must fail the test, not vanish with its thread)
+            failures.append((seed, repr(error)))
+
+    threads = [threading.Thread(target=worker, args=(seed,)) for seed in range(4)]
+    for thread in threads:
+        thread.start()
+    for thread in threads:
+        thread.join()
+    torch.cuda.synchronize()
+    assert not failures, failures
