@@ -361,6 +361,11 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
             int image = m / PQ, pq = m - image * PQ;
             if (whole_chunks) {  // the 8 rows lie in one image and start at a multiple of 8
                 __builtin_nontemporal_store(v, (vec8 *)(Y + ((int64_t)image * p.K + out_channel) * PQ + pq));  // +2 % over a plain store
+            } else if (pq + 8 <= PQ && m + 8 <= p.M) {
+                // the 8 rows lie in one image, only not on a 16-byte boundary (a 7 x 7 map): one store all the same
+                // (global accesses need the element's alignment only)
+                typedef vec8 unaligned_vec8 __attribute__((aligned(2)));
+                *(unaligned_vec8 *)(Y + ((int64_t)image * p.K + out_channel) * PQ + pq) = v;
             } else {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
