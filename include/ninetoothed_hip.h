@@ -263,7 +263,9 @@ NineToothedResult launch_nt_conv2d_strided(NineToothedStream stream,
  * exceed the array, the K range is cut into as many parts as fit (same kernels, another summation order);
  * a call for which not even two parts fit (M x N x 8 bytes > the array) returns
  * NINETOOTHED_SCRATCH_LIMIT and launches nothing (it does not fall back to another kernel); problems
- * that run in one pass need no scratch memory and are accepted at any size.
+ * that run in one pass need no scratch memory and are accepted at any size.  Operands that
+ * launch_nt_matmul would copy into allocated buffers (FLOAT8_E5M2; fp16 / bf16 operands that the
+ * direct-to-LDS kernels cannot read in place) run here on the kernels that read them in place, slower.
  *
  * All calls on one GPU share that GPU's array, on whatever stream: calls whose kernels may overlap on a
  * GPU (different streams, or replays of graphs captured from them) race on it and must be ordered by the

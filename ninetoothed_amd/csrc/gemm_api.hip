@@ -634,6 +634,7 @@ int run_gemm_on_repacked_copies(hipStream_t stream, const GemmProblem &q, int bm
 // 12 us this way, 8192^3: 16.8 ms against 0.83 ms)
 int run_gemm_on_widened_copies(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk) {
     if (q.dtype != NINETOOTHED_FLOAT8_E5M2 || q.batch != 1) return NINETOOTHED_NO_KERNEL;
+    if (q.fixed_scratch != nullptr) return NINETOOTHED_NO_KERNEL;  // (the entry point that allocates nothing: no buffers for copies)
     if (q.out_dtype != NINETOOTHED_FLOAT16 && (q.out_dtype != NINETOOTHED_FLOAT32 || q.addmm())) return NINETOOTHED_NO_KERNEL;
     if ((int64_t)q.m * q.n * q.k < ((int64_t)1 << 18)) return NINETOOTHED_NO_KERNEL;
     if (q.sam < 0 || q.sak < 0 || q.sbk < 0 || q.sbn < 0 || (q.addmm() && (q.sim < 0 || q.sin < 0))) return NINETOOTHED_NO_KERNEL;

@@ -86,3 +86,29 @@ def test_static_scratch_matmul_fp32_output_one_pass_problems_and_the_limit():
     torch.cuda.synchronize()
     assert bool(torch.isnan(out).all())
     assert runtime.STATIC_SCRATCH_BYTES == 16 << 20
+
+
+@pytest.mark.skipif(not hasattr(torch, "float8_e5m2"), reason="this torch has no float8_e5m2")
+def test_static_scratch_matmul_never_takes_buffers_for_copies():
+    """fp8 operands and operands the direct-to-LDS kernels cannot read in place run on copies in allocated buffers
+    under ``launch_nt_matmul``; the entry point that allocates nothing must take the kernels that read them in place."""
+    lib = runtime.library()
+    print("static-scratch matmul: fp8 and misaligned operands, no buffers", flush=True)
+    lib.nt_release_workspaces()
+    m, n, k = 2056, 1032, 1040  # 2^31 multiply-adds and more
+    a8 = torch.randn(m, k, device="cuda").to(torch.float8_e5m2)
+    b8 = torch.randn(k, n, device="cuda").to(torch.float8_e5m2)
+    a_off = torch.randn(m, k + 1, dtype=torch.float16, device="cuda")[:, :k]
+    b16 = torch.randn(k, n, dtype=torch.float16, device="cuda")
+    out8, out16 = (torch.full((m, n), float("nan"), dtype=torch.float16, device="cuda") for _ in range(2))
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    assert _call(lib.launch_nt_matmul_static_scratch, a8, b8, out8, "fp8e5m2", "fp16") == 0
+    assert "any-stride" in runtime.last_launch(), runtime.last_launch()
+    assert _call(lib.launch_nt_matmul_static_scratch, a_off, b16, out16, "fp16") == 0
+    assert "any-stride" in runtime.last_launch(), runtime.last_launch()
+    torch.cuda.synchronize()
+    assert free_before - torch.cuda.mem_get_info()[0] < (1 << 20)  # (the copies would have taken 8 MiB and more)
+    tolerance = dict(rtol=1e-2, atol=1e-2 * (k / 512) ** 0.5)
+    assert torch.allclose(out8.float(), a8.to(torch.float16).float() @ b8.to(torch.float16).float(), **tolerance)
+    assert torch.allclose(out16.float(), a_off.float() @ b16.float(), **tolerance)
