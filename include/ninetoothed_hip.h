@@ -21,7 +21,7 @@
  * passes block sizes), and launch_nt_matmul / launch_nt_addmm on problems with few
  * output tiles and a long K (split-K: parts x M x N floats, at most 64 MiB; not
  * when the caller passes block sizes), on FLOAT8_E5M2 operands (fp16 copies of the operands, and of addmm's
- * input: 2 bytes per element) or, from 2^31 multiply-adds on, on fp16 / bf16 operands that the direct-to-LDS kernels
+ * input: 2 bytes per element) or, from 2^21 multiply-adds on, on fp16 / bf16 operands that the direct-to-LDS kernels
  * cannot read in place (dense copies, (M + N) x K elements) use scratch device memory: one buffer per (device, stream,
  * purpose) that the library allocates (hipMalloc) the first time a call needs
  * it, grows (hipFree + hipMalloc, which wait for the device) when a later call
@@ -318,7 +318,8 @@ NineToothedResult launch_nt_gemm_config(NineToothedStream stream, int config,
  * captured into a graph nothing is timed or recorded: returns 0 with
  * *best_config = -1.  A problem that a single instance takes (fp32 or fp8 operands; fp16 / bf16 operands that the
  * direct-to-LDS instances cannot read in place -- a K that is no multiple of 8, rows off 16-byte boundaries, an lhs
- * stored by columns: launch_nt_matmul / launch_nt_addmm run those on dense copies from 2^31 multiply-adds on) has
+ * stored by columns: launch_nt_matmul / launch_nt_addmm run those on dense copies from 2^21 multiply-adds on: the
+ * instances are then timed on the copies and the winner recorded for the copies' problem) and no copies has
  * nothing to time: returns 0 with *best_config = -2 and records nothing. */
 NineToothedResult nt_tune_gemm(NineToothedStream stream,
                                NineToothedTensor input,

@@ -1,6 +1,7 @@
 // C ABI for the GEMM family: launch_nt_matmul, launch_nt_addmm,
 // launch_nt_conv2d and the tile-selection entry points.
 #include <algorithm>
+#include <memory>
 #include <mutex>
 #include <type_traits>
 #include <shared_mutex>
@@ -600,13 +601,19 @@ hipError_t repack_operand(hipStream_t stream, const void *src, int64_t d0, int64
 
 int heuristic_choice(const GemmProblem &q, int bm, int bn, int bk);
 
-// 0 / an error when the product ran on copies, NINETOOTHED_NO_KERNEL when this way does not apply
-int run_gemm_on_repacked_copies(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk) {
+// Writes the dense copies of q's operands into the stream's buffers (`lease` must stay alive until everything that
+// reads them is enqueued) and describes the product on them in `dense`.  0, an error, or NINETOOTHED_NO_KERNEL when
+// this way does not apply.
+int make_dense_copies(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk, WorkspaceLease &lease, GemmProblem &dense) {
     if ((q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) || q.batch != 1) return NINETOOTHED_NO_KERNEL;
-    // below about 1300^3 the two extra passes cost what they save
-    if ((int64_t)q.m * q.n * q.k < ((int64_t)1 << 31) || q.fixed_scratch != nullptr) return NINETOOTHED_NO_KERNEL;
+#ifndef NT_GEMM_COPY_LOG2
+#define NT_GEMM_COPY_LOG2 21
+#endif
+    // (the any-stride kernel is slower from small sizes on: 512^3 36-45 us in place against 11-13 us on copies,
+    // 256^3 22-25 against 12; below 128^3 everything is one launch's time)
+    if ((int64_t)q.m * q.n * q.k < ((int64_t)1 << NT_GEMM_COPY_LOG2) || q.fixed_scratch != nullptr) return NINETOOTHED_NO_KERNEL;
     const int64_t k8 = ((int64_t)q.k + 7) / 8 * 8;
-    GemmProblem dense = q;
+    dense = q;
     dense.k = (int)k8;
     dense.sam = k8;
     dense.sak = 1;
@@ -616,7 +623,6 @@ int run_gemm_on_repacked_copies(hipStream_t stream, const GemmProblem &q, int bm
     dense.a = dense.b = (const void *)(uintptr_t)256;
     const int choice = heuristic_choice(dense, bm, bn, bk);
     if (choice < 0 || choice == kAnyStride) return NINETOOTHED_NO_KERNEL;  // (the output's layout rules the fast instances out)
-    WorkspaceLease lease(stream);  // held until the product is enqueued: it reads the copies
     // (buffers of their own: the sources may be the widened copies of fp8 operands)
     uint16_t *a = (uint16_t *)lease.get(kWorkspaceGemmLhsDense, (size_t)q.m * k8 * 2);
     uint16_t *b = a != nullptr ? (uint16_t *)lease.get(kWorkspaceGemmRhsDense, (size_t)q.n * k8 * 2) : nullptr;
@@ -625,6 +631,14 @@ int run_gemm_on_repacked_copies(hipStream_t stream, const GemmProblem &q, int bm
     dense.b = b;
     if (hipError_t err = repack_operand(stream, q.a, q.m, q.k, q.sam, q.sak, a, k8)) return (int)err;
     if (hipError_t err = repack_operand(stream, q.b, q.n, q.k, q.sbn, q.sbk, b, k8)) return (int)err;
+    return 0;
+}
+
+// 0 / an error when the product ran on copies, NINETOOTHED_NO_KERNEL when this way does not apply
+int run_gemm_on_repacked_copies(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk) {
+    WorkspaceLease lease(stream);  // held until the product is enqueued: it reads the copies
+    GemmProblem dense;
+    if (const int status = make_dense_copies(stream, q, bm, bn, bk, lease, dense)) return status;
     return run_gemm(stream, dense, bm, bn, bk, false);
 }
 
@@ -657,8 +671,32 @@ int run_gemm_on_widened_copies(hipStream_t stream, const GemmProblem &q, int bm,
     return run_gemm(stream, wide, bm, bn, bk);
 }
 
+// an output stored by columns (`out.T`): C^T = B^T A^T is the same product with a row-major output, which the
+// direct-to-LDS instances write (the any-stride kernel would store it two bytes at a time)
+bool output_by_columns(const GemmProblem &q) { return q.scn != 1 && q.scm == 1 && q.n > 1; }
+
+GemmProblem transposed_problem(const GemmProblem &q) {
+    GemmProblem t = q;
+    t.m = q.n;
+    t.n = q.m;
+    t.a = q.b;
+    t.b = q.a;
+    t.sam = q.sbn;
+    t.sak = q.sbk;
+    t.sbk = q.sak;
+    t.sbn = q.sam;
+    t.scm = q.scn;
+    t.scn = q.scm;
+    t.sim = q.sin;
+    t.sin = q.sim;
+    t.a_batch = q.b_batch;
+    t.b_batch = q.a_batch;
+    return t;
+}
+
 int run_gemm(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk, bool may_copy) {
     if (q.m == 0 || q.n == 0) return 0;
+    if (output_by_columns(q)) return run_gemm(stream, transposed_problem(q), bn, bm, bk, may_copy);
     if (q.dtype == NINETOOTHED_FLOAT8_E5M2) {
         const int widened = run_gemm_on_widened_copies(stream, q, bm, bn, bk);
         if (widened != NINETOOTHED_NO_KERNEL) return widened;
@@ -805,18 +843,35 @@ NineToothedResult nt_tune_gemm(NineToothedStream stream_, NineToothedTensor inpu
                                NineToothedTensor output, int dtype, int output_dtype, int iters, int *best_config,
                                float *best_ms) {
     hipStream_t stream = (hipStream_t)stream_;
-    GemmProblem q;
-    if (int err = build_problem(q, &input, mat1, mat2, &beta, &alpha, output, dtype, output_dtype)) return err;
+    GemmProblem given;
+    if (int err = build_problem(given, &input, mat1, mat2, &beta, &alpha, output, dtype, output_dtype)) return err;
+    // (what the launch functions do first: an output stored by columns is the transposed product)
+    GemmProblem q = output_by_columns(given) ? transposed_problem(given) : given;
     int best = -1;
     float best_time = 0.0f;
-    // a problem that a single instance accepts (operands that only the any-stride kernel reads in place: the launch
-    // functions run large ones on dense copies) has nothing to time, and nothing is recorded for it
+    // A problem that a single instance accepts has nothing to time.  Operands that only the any-stride kernel reads
+    // in place run on dense copies (launch_nt_matmul / launch_nt_addmm): then the product on the copies is what
+    // gets timed and recorded, under its own key, where the launch functions look it up.
     int accepting = 0;
     for (int i = 0; i < kNumInstances; ++i) accepting += kInstances[i].accepts(q) ? 1 : 0;
+    std::unique_ptr<WorkspaceLease> lease;  // (keeps the copies in place while they are timed)
     if (accepting <= 1) {
-        if (best_config) *best_config = accepting == 1 ? -2 : -1;
-        if (best_ms) *best_ms = 0.0f;
-        return accepting == 1 ? 0 : NINETOOTHED_NO_KERNEL;
+        GemmProblem dense;
+        lease.reset(new WorkspaceLease(stream));
+        const int copied = stream_is_capturing(stream) ? NINETOOTHED_NO_KERNEL : make_dense_copies(stream, q, 0, 0, 0, *lease, dense);
+        if (copied != 0) {
+            if (best_config) *best_config = accepting == 1 ? -2 : -1;
+            if (best_ms) *best_ms = 0.0f;
+            if (copied != NINETOOTHED_NO_KERNEL) return copied;
+            return accepting == 1 ? 0 : NINETOOTHED_NO_KERNEL;
+        }
+        q = dense;
+        const int known = lookup_tuned(q);
+        if (known >= 0 && kInstances[known].accepts(q)) {  // (an earlier process has timed it: the file was loaded)
+            if (best_config) *best_config = known;
+            if (best_ms) *best_ms = 0.0f;
+            return 0;
+        }
     }
     // (inside a graph capture nothing is timed: the problem stays on the fixed preference order and nothing is recorded)
     // the untuned rule's instance is timed first and stays unless another one is more than 2 % faster: timings of a

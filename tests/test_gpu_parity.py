@@ -1294,9 +1294,9 @@ def test_matmul_float8_e5m2_operands(m, n, k):
 
 @pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
 def test_large_products_on_operands_the_fast_instances_cannot_read_run_on_dense_copies(dtype):
-    """A K that is no multiple of 8, rows off 16-byte boundaries, an lhs stored by columns, other strides: from 2^31
+    """A K that is no multiple of 8, rows off 16-byte boundaries, an lhs stored by columns, other strides: from 2^21
     multiply-adds on such operands are copied (k contiguous, K padded to 8 with zeros) and the product runs on the
-    direct-to-LDS instances.  What lies next to the operands in memory is Inf and must not reach the sums; what
+    direct-to-LDS instances; an output stored by columns runs as the transposed product.  What lies next to the operands in memory is Inf and must not reach the sums; what
     lies next to the output must stay as it was."""
     from ninetoothed_amd import runtime
 
@@ -1326,8 +1326,18 @@ def test_large_products_on_operands_the_fast_instances_cannot_read_run_on_dense_
     check(inside(2048, 1024, transposed=True), inside(1024, 1031, transposed=True), out_cols_pad=1)  # both, C rows off 16-byte boundaries
     wide_l, wide_r = inside(2048, 2048), inside(1024, 2048)
     check(wide_l[:, ::2], wide_r[:, ::2])                              # every other column
-    # below the threshold the any-stride kernel serves the call as before
-    check(inside(300, 205), inside(205, 301), fast=False)
+    # an output stored by columns: the transposed product, here on dense operands and on ones that need copies
+    for lhs, rhs in ((torch.randn(1024, 512, device="cuda").to(dtype), torch.randn(512, 768, device="cuda").to(dtype)), (inside(1030, 517), inside(517, 771))):
+        buffer = torch.full((rhs.shape[1] + 1, lhs.shape[0] + 8), 7.0, dtype=dtype, device="cuda")
+        out = buffer[: rhs.shape[1], : lhs.shape[0]].T
+        kernel(lhs, rhs, out)
+        assert "any-stride" not in runtime.last_launch(), runtime.last_launch()
+        assert torch.allclose(out.float(), lhs.float() @ rhs.float(), **HALF_TOL)
+        assert bool((buffer[rhs.shape[1] :] == 7.0).all()) and bool((buffer[:, lhs.shape[0] :] == 7.0).all())
+    # small products as well (the any-stride kernel is slower from 128^3 on) ...
+    check(inside(300, 205), inside(205, 301))
+    # ... and below that it serves the call as before
+    check(inside(100, 77), inside(77, 90), fast=False)
     # addmm on such operands, the bias with rows off 16-byte boundaries as well
     m, k, n = 2050, 1029, 1100
     bias, lhs, rhs = inside(m, n), inside(m, k), inside(k, n)
@@ -1382,9 +1392,8 @@ def test_matmul_float8_e5m2_large_products_run_on_widened_copies():
     lhs2 = wide[3:, 5:]
     lhs2.view(torch.uint8)[0, 0] = 0x5C  # 256.0
     check(lhs2, rhs)
-    # sizes that are no multiples of 8, below the size from which such fp16 operands are copied: the widened copies
-    # get padded rows and the any-stride fp16 kernel runs on them
-    check(torch.randn(2050, 1030, device="cuda").to(torch.float8_e5m2), torch.randn(1030, 1001, device="cuda").to(torch.float8_e5m2), fast=False)
+    # sizes that are no multiples of 8: the widened copies get padded rows and are copied once more, K padded to 8
+    check(torch.randn(2050, 1030, device="cuda").to(torch.float8_e5m2), torch.randn(1030, 1001, device="cuda").to(torch.float8_e5m2))
     # addmm: the bias is widened as well (tests/test_addmm.py:57-90 of the reference at a larger size)
     bias = torch.randn(m, n, device="cuda").to(torch.float8_e5m2)
     rhs_t = torch.randn(n, k, device="cuda").to(torch.float8_e5m2).T
