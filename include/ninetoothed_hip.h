@@ -211,8 +211,11 @@ NineToothedResult launch_nt_attention(NineToothedStream stream,
  *   tap)-shifted pixel runs of the NCHW input; needs an output width that is a
  *   multiple of 8, padding_w <= 1, C*R*S a multiple of 32, R*S / gcd(32, R*S) <= 25, pixels of an input row
  *   contiguous, contiguous filter and output, K filling 256-wide tiles to 4/5;
- * 2 -- when the output is contiguous (fp16 / bf16 tensors): the
- *   input is first repacked to channels-last and the filter to [R*S*C', K']
+ * 2 -- fp16 / bf16 tensors of any strides (a contiguous NCHW output is stored in
+ *   16-byte pieces of 8 positions, a channels-last one in pieces of 8 channels,
+ *   any other element by element): the
+ *   input is first repacked to channels-last (a contiguous channels-last input
+ *   with C' == C is read where it is) and the filter to [R*S*C', K']
  *   (C' = C rounded up to a multiple of 32 -- to 8 or 16 for up to 16 channels --, K' = K
  *   rounded up to 8, zero filled) in the library's scratch
  *   buffers of `stream` (N*C'*H*W + K'*C'*R*S elements), then the direct-to-LDS

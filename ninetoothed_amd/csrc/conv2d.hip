@@ -47,6 +47,9 @@ struct ConvParams {
     void *y;
     int N, C, H, W, K, R, S, P, Q, pad_h, pad_w;
     int Kp;                   // row pitch of the repacked filter: K rounded up to 8 (its rows are read in 16-byte pieces)
+    int dense_out;            // 1: the output is a contiguous NCHW tensor on a 16-byte boundary; 2: its channels are its
+                              // innermost dimension (channels last); 0: any strides, stored element by element
+    int64_t ys[4];            // element strides of the output
     int M, tiles_m, tiles_n;  // M = N*P*Q rows
     unsigned xt_bytes, wt_bytes;
     int stride_h, stride_w, dil_h, dil_w;  // steps of the window over the input and between its taps
@@ -56,7 +59,9 @@ struct ConvParams {
 // grid layers z <  f.layers: w[K,C,R,S] (any strides) -> wt[(r*S+s)*C + c][K], grid-stride over these layers' threads
 //                     (first, so that its scattered reads overlap the streaming layers behind it; as many
 //                     layers as give the filter a few hundred workgroups, whatever the image size)
-// grid layers z >= f.layers: x[z - f.layers] NCHW (any strides) -> xt NHWC contiguous (64 x 64 tiles through LDS)
+// grid layers z >= f.layers: x[z - f.layers] NCHW (any strides) -> xt NHWC contiguous (64 x 64 tiles through LDS;
+//                     vector_ok 1: 16-byte loads along the positions; 2 and 3: the channels are innermost in x
+//                     already and rows of them are copied, 3 with 16-byte loads)
 struct FilterRepack {
     const void *w;
     void *wt;
@@ -90,6 +95,27 @@ __global__ __launch_bounds__(256) void conv2d_repack_kernel(const T *x, T *xt, i
     }
     const int hw0 = blockIdx.x * 64, c0 = blockIdx.y * 64, n = blockIdx.z - f.layers;
     const T *src = x + (int64_t)n * s_n;
+    if (vector_ok >= 2) {
+        // the channels are the innermost dimension already (a channels-last tensor): rows of 8 channels are
+        // copied as they lie, padded to Cp with zeros
+#pragma unroll
+        for (int pass = 0; pass < 2; ++pass) {
+            const int hw = hw0 + pass * 32 + (t >> 3);
+            const int c = c0 + (t & 7) * 8;
+            if (hw < HW && c < f.Cp) {
+                const T *from = src + (int64_t)(hw / W) * s_h + (int64_t)(hw % W) * s_w + c;
+                vec8 v;
+                if (vector_ok == 3 && c + 8 <= C) {
+                    v = *(const vec8 *)from;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) v[e] = c + e < C ? from[e] : (T)0.0f;
+                }
+                *(vec8 *)(xt + ((int64_t)n * HW + hw) * f.Cp + c) = v;
+            }
+        }
+        return;
+    }
     // load: rows = channels, 8 consecutive positions per thread
 #pragma unroll
     for (int pass = 0; pass < 2; ++pass) {
@@ -333,7 +359,7 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
         slab += (wave % WM) * kSlabBytes;
     }
     T *Y = (T *)p.y;
-    const bool whole_chunks = PQ % 8 == 0;
+    const bool whole_chunks = PQ % 8 == 0 && p.dense_out == 1;
 #pragma unroll
     for (int tj = 0; tj < TN; ++tj) {
 #pragma unroll
@@ -347,6 +373,36 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
                 const int chunk = (ti * 4 + r4) ^ (l32 & (kChunks - 1));
                 *(NT_LDS vec4 *)(slab + l32 * kRowBytes + chunk * 16 + 8 * g) = v;
             }
+        if (p.dense_out == 2) {
+            // channels-last output: a lane gathers 8 channels of one row from the slab and stores them with one
+            // instruction (the 32 channels of the slab are 64 consecutive bytes of the tensor)
+#pragma unroll
+            for (int it = 0; it < (32 * kChunks) / 64; ++it) {
+                const int idx = it * 64 + lane;
+                const int row = idx >> 2, first = (idx & 3) * 8;
+                vec8 v;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int channel = first + e;
+                    v[e] = *(const NT_LDS T *)(slab + channel * kRowBytes + (((row >> 3) ^ (channel & (kChunks - 1))) * 16) + (row & 7) * 2);
+                }
+                const int m = m0 + wave_m * kWaveM + row;
+                const int out_channel = n0 + wave_n * kWaveN + tj * 32 + first;
+                if (m >= p.M || out_channel >= p.K) continue;
+                const int image = m / PQ, pq = m - image * PQ;
+                const int oy = pq / p.Q, ox = pq - oy * p.Q;
+                T *to = Y + (int64_t)image * p.ys[0] + (int64_t)oy * p.ys[2] + (int64_t)ox * p.ys[3] + out_channel;
+                if (out_channel + 8 <= p.K) {
+                    typedef vec8 unaligned_vec8 __attribute__((aligned(2)));
+                    *(unaligned_vec8 *)to = v;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (out_channel + e < p.K) to[e] = v[e];
+                }
+            }
+            continue;
+        }
 #pragma unroll
         for (int it = 0; it < (32 * kChunks) / 64; ++it) {
             const int idx = it * 64 + lane;
@@ -361,18 +417,23 @@ __global__ __launch_bounds__(WM *WN * 64, kOcc) void conv2d_nhwc_kernel(ConvPara
             int image = m / PQ, pq = m - image * PQ;
             if (whole_chunks) {  // the 8 rows lie in one image and start at a multiple of 8
                 __builtin_nontemporal_store(v, (vec8 *)(Y + ((int64_t)image * p.K + out_channel) * PQ + pq));  // +2 % over a plain store
-            } else if (pq + 8 <= PQ && m + 8 <= p.M) {
+            } else if (p.dense_out == 1 && pq + 8 <= PQ && m + 8 <= p.M) {
                 // the 8 rows lie in one image, only not on a 16-byte boundary (a 7 x 7 map): one store all the same
                 // (global accesses need the element's alignment only)
                 typedef vec8 unaligned_vec8 __attribute__((aligned(2)));
                 *(unaligned_vec8 *)(Y + ((int64_t)image * p.K + out_channel) * PQ + pq) = v;
             } else {
+                // (any output strides: a channels-last tensor, a slice of a wider one)
+                int oy = pq / p.Q, ox = pq - oy * p.Q;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    if (m + e < p.M) Y[((int64_t)image * p.K + out_channel) * PQ + pq] = v[e];
-                    if (++pq == PQ) {
-                        pq = 0;
-                        ++image;
+                    if (m + e < p.M) Y[(int64_t)image * p.ys[0] + (int64_t)out_channel * p.ys[1] + (int64_t)oy * p.ys[2] + (int64_t)ox * p.ys[3]] = v[e];
+                    if (++ox == p.Q) {
+                        ox = 0;
+                        if (++oy == p.P) {
+                            oy = 0;
+                            ++image;
+                        }
                     }
                 }
             }
@@ -979,11 +1040,15 @@ int run_fast(const Conv2dRequest &q, hipStream_t stream) {
     const int Kp = ceil_div(q.K, 8) * 8;
     const int64_t wt_bytes = (int64_t)Kp * Cp * q.R * q.S * 2;
     WorkspaceLease lease(stream);
-    void *xt = lease.get(kWorkspaceConvInput, (size_t)xt_bytes);
+    const int HW = q.H * q.W;
+    // an input that lies as the kernel reads it -- channels last, contiguous, whole k steps of channels -- is read where it is
+    const bool in_place = q.xs[1] == 1 && q.C == Cp && q.xs[3] == Cp && q.xs[2] == (int64_t)q.W * Cp && q.xs[0] == (int64_t)HW * Cp && ((uintptr_t)q.x & 15) == 0;
+    void *xt = in_place ? const_cast<void *>(q.x) : lease.get(kWorkspaceConvInput, (size_t)xt_bytes);
     void *wt = lease.get(kWorkspaceConvFilter, (size_t)wt_bytes);
     if (xt == nullptr || wt == nullptr) return NINETOOTHED_NO_KERNEL;  // no scratch: the caller falls back to the gather kernel
-    const int HW = q.H * q.W;
-    const int vector_ok = q.xs[3] == 1 && q.xs[2] == q.W && HW % 8 == 0 && q.xs[1] % 8 == 0 && q.xs[0] % 8 == 0 && ((uintptr_t)q.x & 15) == 0;
+    const bool aligned = ((uintptr_t)q.x & 15) == 0;
+    int vector_ok = q.xs[3] == 1 && q.xs[2] == q.W && HW % 8 == 0 && q.xs[1] % 8 == 0 && q.xs[0] % 8 == 0 && aligned;
+    if (q.xs[1] == 1 && q.C > 1) vector_ok = q.C % 8 == 0 && q.xs[3] % 8 == 0 && q.xs[2] % 8 == 0 && q.xs[0] % 8 == 0 && aligned ? 3 : 2;
     FilterRepack f;
     f.w = q.w;
     f.wt = wt;
@@ -993,7 +1058,7 @@ int run_fast(const Conv2dRequest &q, hipStream_t stream) {
     const int64_t per_layer = (int64_t)ceil_div(HW, 64) * ceil_div(Cp, 64);
     const int64_t wanted = std::min<int64_t>(512, ((int64_t)Kp * Cp * q.R * q.S + 255) / 256);
     f.layers = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(wanted, per_layer), 512));
-    conv2d_repack_kernel<T><<<dim3(ceil_div(HW, 64), ceil_div(Cp, 64), q.N + f.layers), dim3(256), 0, stream>>>(
+    conv2d_repack_kernel<T><<<dim3(ceil_div(HW, 64), ceil_div(Cp, 64), (in_place ? 0 : q.N) + f.layers), dim3(256), 0, stream>>>(
         (const T *)q.x, (T *)xt, q.C, HW, q.W, q.xs[0], q.xs[1], q.xs[2], q.xs[3], vector_ok, f);
     ConvParams p;
     p.xt = xt;
@@ -1001,6 +1066,9 @@ int run_fast(const Conv2dRequest &q, hipStream_t stream) {
     p.y = q.y;
     p.N = q.N; p.C = Cp; p.H = q.H; p.W = q.W; p.K = q.K; p.R = q.R; p.S = q.S; p.P = q.P; p.Q = q.Q;
     p.Kp = Kp;
+    p.dense_out = q.ys[3] == 1 && q.ys[2] == q.Q && q.ys[1] == (int64_t)q.P * q.Q && q.ys[0] == (int64_t)q.K * q.P * q.Q && ((uintptr_t)q.y & 15) == 0;
+    if (!p.dense_out && q.ys[1] == 1 && q.K > 1) p.dense_out = 2;
+    for (int d = 0; d < 4; ++d) p.ys[d] = q.ys[d];
     p.stride_h = q.stride_h; p.stride_w = q.stride_w; p.dil_h = q.dil_h; p.dil_w = q.dil_w;
     p.pad_h = q.pad_h; p.pad_w = q.pad_w;
     p.M = q.N * q.P * q.Q;
@@ -1030,8 +1098,7 @@ int conv2d_fast(const Conv2dRequest &q, hipStream_t stream) {
     if (q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) return NINETOOTHED_NO_KERNEL;
     // channels are padded to the k step of 32 with zeros; below a sixteenth of useful work the gather kernel is as good
     if (q.C < 1) return NINETOOTHED_NO_KERNEL;
-    if (q.ys[3] != 1 || q.ys[2] != q.Q || q.ys[1] != (int64_t)q.P * q.Q || q.ys[0] != (int64_t)q.K * q.P * q.Q) return NINETOOTHED_NO_KERNEL;
-    if (((uintptr_t)q.y & 15) != 0) return NINETOOTHED_NO_KERNEL;
+    // (an output that is no contiguous NCHW tensor -- channels last, a slice -- is stored element by element)
     const int64_t xt_bytes = (int64_t)q.N * q.H * q.W * conv2d_padded_channels(q.C) * 2;
     const int64_t wt_bytes = (int64_t)ceil_div(q.K, 8) * 8 * conv2d_padded_channels(q.C) * q.R * q.S * 2;
     if (xt_bytes >= (int64_t(1) << 31) || wt_bytes >= (int64_t(1) << 31)) return NINETOOTHED_NO_KERNEL;  // 32-bit buffer offsets

@@ -880,6 +880,44 @@ def test_conv2d_few_input_channels_on_the_repacked_path(channels, dtype):
         assert torch.allclose(y.float(), expected, **HALF_TOL), (channels, r, s_, float((y.float() - expected).abs().max()))
 
 
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
+@pytest.mark.parametrize("channels", (3, 20, 32, 64, 72))
+def test_conv2d_channels_last_and_sliced_tensors_on_the_repacked_path(channels, dtype):
+    """Channels-last inputs are read in place when their channels fill whole k steps (32, 64) and copied by rows of
+    channels otherwise; outputs that are no contiguous NCHW tensor (channels last, a window of a wider buffer whose
+    other elements must stay as they were) are stored element by element."""
+    from ninetoothed_amd import runtime
+
+    tag = runtime.DATA_TYPE_INDEX["fp16" if dtype == torch.float16 else "bf16"]
+    for (n, h, w, k, r, s_, padding) in ((3, 20, 18, 40, 3, 3, (1, 1)), (2, 15, 17, 64, 1, 1, (0, 0)), (2, 16, 16, 24, 5, 3, (2, 0))):
+        x = _randn(n, channels, h, w, dtype=dtype, scale=0.3).cuda()
+        weight = _randn(k, channels, r, s_, dtype=dtype, scale=0.3).cuda()
+        expected = F.conv2d(x.float(), weight.float(), padding=padding)
+        p, q = expected.shape[2:]
+        x_last = x.to(memory_format=torch.channels_last)
+        assert x_last.stride(1) == 1
+        wide = torch.full((n, k + 3, p + 2, q + 5), 7.0, dtype=dtype, device="cuda")
+        window = wide[:, 2 : 2 + k, 1 : 1 + p, 3 : 3 + q]
+        outputs = (
+            (x_last, weight.to(memory_format=torch.channels_last), torch.full(expected.shape, float("nan"), dtype=dtype, device="cuda").to(memory_format=torch.channels_last)),
+            (x_last, weight, torch.full(expected.shape, float("nan"), dtype=dtype, device="cuda")),
+            (x, weight, window),
+            (x_last[:, :, :, 1:], weight, None),  # a channels-last input that is not contiguous
+        )
+        for (x_in, w_in, y) in outputs:
+            want = expected
+            if y is None:
+                want = F.conv2d(x[:, :, :, 1:].float(), weight.float(), padding=padding)
+                y = torch.full(want.shape, float("nan"), dtype=dtype, device="cuda")
+            tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (x_in, w_in, y)]
+            assert runtime.library().launch_nt_conv2d(runtime.current_stream(), *tensors, tag, *padding, 2, 0, 0) == 0
+            assert runtime.last_launch().startswith("conv2d path 2"), runtime.last_launch()
+            assert torch.allclose(y.float(), want, **HALF_TOL), (channels, r, s_, tuple(y.stride()), float((y.float() - want).abs().max()))
+        untouched = torch.ones_like(wide, dtype=torch.bool)
+        untouched[:, 2 : 2 + k, 1 : 1 + p, 3 : 3 + q] = False
+        assert bool((wide[untouched] == 7).all())
+
+
 def test_conv2d_one_launch_path_refuses_what_it_cannot_run():
     from ninetoothed_amd import runtime
 
