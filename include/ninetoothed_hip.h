@@ -143,7 +143,12 @@ NineToothedResult launch_nt_addmm(NineToothedStream stream,
 
 /* output[r, :] = softmax(input[r, :]) over the last of two dims, in fp32
  * arithmetic.  Replaces the kernel generated for tests/test_softmax.py:10-27
- * (one program per row, BLOCK_SIZE >= row length). */
+ * (one program per row, BLOCK_SIZE >= row length).  Up to 128 row segments of
+ * 64 KiB or more each (256 KiB where a segment fits the registers of one
+ * workgroup, and then up to 16) are cut into parts that run on as many
+ * workgroups, in two launches; the parts' maxima and sums (8 bytes each, at
+ * most 256 per segment) go through a scratch buffer of `stream`, without which
+ * one workgroup per segment runs. */
 NineToothedResult launch_nt_softmax(NineToothedStream stream,
                                     NineToothedTensor input,
                                     NineToothedTensor output,

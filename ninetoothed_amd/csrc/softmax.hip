@@ -6,6 +6,10 @@
 // (the usual call) a segment is a whole row.
 #include "nt_common.h"
 #include "tune.h"
+#include "workspace.h"
+
+#include <algorithm>
+#include <cstdlib>
 
 namespace nt {
 namespace {
@@ -227,14 +231,61 @@ __global__ __launch_bounds__(kRowThreads > 256 ? kRowThreads : 256) void softmax
     }
 }
 
+// One access of the kernels for long segments: 16 bytes of a segment whose columns are one element apart (global
+// accesses need the element's alignment only), else one element.
+template <typename T, bool kVec>
+struct WideAccess {
+    static constexpr int kWidth = kVec ? Vec16<T>::kWidth : 1;
+    typedef typename Vec16<T>::type aligned_type;
+    typedef aligned_type type __attribute__((aligned(sizeof(T))));
+};
+
+template <typename T, bool kVec>
+NT_DEVICE void wide_load(const T *src, int64_t col_stride, int64_t index, int64_t count, float (&x)[WideAccess<T, kVec>::kWidth]) {
+    constexpr int W = WideAccess<T, kVec>::kWidth;
+    if constexpr (kVec) {
+        if ((index + 1) * W <= count) {
+            const typename WideAccess<T, kVec>::type v = *(const typename WideAccess<T, kVec>::type *)(src + index * W);
+#pragma unroll
+            for (int e = 0; e < W; ++e) x[e] = (float)v[e];
+        } else {
+#pragma unroll
+            for (int e = 0; e < W; ++e) x[e] = index * W + e < count ? (float)src[index * W + e] : -INFINITY;
+        }
+    } else {
+        x[0] = index < count ? (float)src[index * col_stride] : -INFINITY;
+    }
+}
+
+// exp(x - maximum) / sum of one access, stored
+template <typename T, bool kVec>
+NT_DEVICE void wide_store(T *dst, int64_t col_stride, int64_t index, int64_t count, const float (&x)[WideAccess<T, kVec>::kWidth], float shift, float inv) {
+    constexpr int W = WideAccess<T, kVec>::kWidth;
+    if constexpr (kVec) {
+        if ((index + 1) * W <= count) {
+            typename WideAccess<T, kVec>::type v;
+#pragma unroll
+            for (int e = 0; e < W; ++e) v[e] = (T)(__builtin_amdgcn_exp2f(fmaf(x[e], kLog2e, -shift)) * inv);
+            *(typename WideAccess<T, kVec>::type *)(dst + index * W) = v;
+        } else {
+#pragma unroll
+            for (int e = 0; e < W; ++e)
+                if (index * W + e < count) dst[index * W + e] = (T)(__builtin_amdgcn_exp2f(fmaf(x[e], kLog2e, -shift)) * inv);
+        }
+    } else {
+        if (index < count) dst[index * col_stride] = (T)(__builtin_amdgcn_exp2f(fmaf(x[0], kLog2e, -shift)) * inv);
+    }
+}
+
 // Long segments: one workgroup of 1024 threads per segment, two sweeps over memory: running
-// maximum and sum together (a thread rescales its sum once per round of eight independent loads),
+// maximum and sum together (a thread rescales its sum once per round of independent loads),
 // then the write; the second sweep hits L2 for segments that fit there.
 constexpr int kLoopThreads = 1024;
-constexpr int kLoopUnroll = 8;
 
-template <typename T>
+template <typename T, bool kVec>
 __global__ __launch_bounds__(kLoopThreads) void softmax_loop_kernel(SoftmaxParams p) {
+    constexpr int W = WideAccess<T, kVec>::kWidth;
+    constexpr int kLoopUnroll = kVec ? 2 : 8;
     __shared__ float scratch[kLoopThreads / 64];
     const int64_t seg = blockIdx.x;
     const int64_t row = seg / p.segments;
@@ -242,16 +293,17 @@ __global__ __launch_bounds__(kLoopThreads) void softmax_loop_kernel(SoftmaxParam
     const int64_t len = min(p.block, p.cols - start);
     const T *src = (const T *)p.in + row * p.in_row_stride + start * p.in_col_stride;
     T *dst = (T *)p.out + row * p.out_row_stride + start * p.out_col_stride;
+    const int64_t pieces = (len + W - 1) / W;
 
     float m = -INFINITY, s = 0.0f;
-    for (int64_t base = threadIdx.x; base < len; base += kLoopThreads * kLoopUnroll) {
-        float x[kLoopUnroll];
+    for (int64_t base = threadIdx.x; base < pieces; base += kLoopThreads * kLoopUnroll) {
+        float x[kLoopUnroll][W];
         float round_max = -INFINITY;
 #pragma unroll
         for (int u = 0; u < kLoopUnroll; ++u) {
-            const int64_t c = base + (int64_t)u * kLoopThreads;
-            x[u] = c < len ? (float)src[c * p.in_col_stride] : -INFINITY;
-            round_max = fmaxf(round_max, x[u]);
+            wide_load<T, kVec>(src, p.in_col_stride, base + u * kLoopThreads, len, x[u]);
+#pragma unroll
+            for (int e = 0; e < W; ++e) round_max = fmaxf(round_max, x[u][e]);
         }
         if (round_max > m) {  // (a first round of -inf only leaves m at -inf and s at 0)
             s *= __builtin_amdgcn_exp2f((m - round_max) * kLog2e);
@@ -260,7 +312,9 @@ __global__ __launch_bounds__(kLoopThreads) void softmax_loop_kernel(SoftmaxParam
         if (m > -INFINITY) {
             const float shift = m * kLog2e;
 #pragma unroll
-            for (int u = 0; u < kLoopUnroll; ++u) s += __builtin_amdgcn_exp2f(fmaf(x[u], kLog2e, -shift));
+            for (int u = 0; u < kLoopUnroll; ++u)
+#pragma unroll
+                for (int e = 0; e < W; ++e) s += __builtin_amdgcn_exp2f(fmaf(x[u][e], kLog2e, -shift));
         }
     }
     const float total_max = group_reduce<kLoopThreads, true>(m, scratch);
@@ -269,19 +323,127 @@ __global__ __launch_bounds__(kLoopThreads) void softmax_loop_kernel(SoftmaxParam
     s = group_reduce<kLoopThreads, false>(s, scratch);
     const float inv = 1.0f / s;
     const float shift = total_max * kLog2e;
-    for (int64_t base = threadIdx.x; base < len; base += kLoopThreads * kLoopUnroll) {
-        float x[kLoopUnroll];
+    for (int64_t base = threadIdx.x; base < pieces; base += kLoopThreads * kLoopUnroll) {
+        float x[kLoopUnroll][W];
 #pragma unroll
-        for (int u = 0; u < kLoopUnroll; ++u) {
-            const int64_t c = base + (int64_t)u * kLoopThreads;
-            x[u] = c < len ? (float)src[c * p.in_col_stride] : -INFINITY;
+        for (int u = 0; u < kLoopUnroll; ++u) wide_load<T, kVec>(src, p.in_col_stride, base + u * kLoopThreads, len, x[u]);
+#pragma unroll
+        for (int u = 0; u < kLoopUnroll; ++u) wide_store<T, kVec>(dst, p.out_col_stride, base + u * kLoopThreads, len, x[u], shift, inv);
+    }
+}
+
+// Few long segments: each is cut into parts, a workgroup of 256 threads per part, two launches.  The first leaves
+// every part's maximum and its sum of exponentials relative to that maximum in `partials`; the second combines
+// the parts of its segment and writes its own part (its input is the first launch's and comes from the caches).
+// kVec: unit column strides, 16 bytes per access (global accesses need the element's alignment only).
+constexpr int kSplitThreads = 256;
+constexpr int kSplitUnroll = 4;
+
+struct SplitPartial {
+    float max, sum;
+};
+
+template <typename T, bool kVec>
+__global__ __launch_bounds__(kSplitThreads) void softmax_split_partial_kernel(SoftmaxParams p, int64_t part_len, SplitPartial *partials) {
+    constexpr int W = WideAccess<T, kVec>::kWidth;
+    __shared__ float scratch[kSplitThreads / 64];
+    const int64_t seg = blockIdx.y;
+    const int64_t row = seg / p.segments;
+    const int64_t start = (seg % p.segments) * p.block + (int64_t)blockIdx.x * part_len;
+    const int64_t seg_end = min((seg % p.segments + 1) * p.block, p.cols);
+    const int64_t count = max((int64_t)0, min(part_len, seg_end - start));
+    const T *src = (const T *)p.in + row * p.in_row_stride + start * p.in_col_stride;
+    const int64_t pieces = (count + W - 1) / W;
+    float m = -INFINITY, s = 0.0f;
+    for (int64_t base = threadIdx.x; base < pieces; base += kSplitThreads * kSplitUnroll) {
+        float x[kSplitUnroll][W];
+        float round_max = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < kSplitUnroll; ++u) {
+            wide_load<T, kVec>(src, p.in_col_stride, base + u * kSplitThreads, count, x[u]);
+#pragma unroll
+            for (int e = 0; e < W; ++e) round_max = fmaxf(round_max, x[u][e]);
         }
+        if (round_max > m) {
+            s *= __builtin_amdgcn_exp2f((m - round_max) * kLog2e);
+            m = round_max;
+        }
+        if (m > -INFINITY) {
+            const float shift = m * kLog2e;
 #pragma unroll
-        for (int u = 0; u < kLoopUnroll; ++u) {
-            const int64_t c = base + (int64_t)u * kLoopThreads;
-            if (c < len) dst[c * p.out_col_stride] = (T)(__builtin_amdgcn_exp2f(fmaf(x[u], kLog2e, -shift)) * inv);
+            for (int u = 0; u < kSplitUnroll; ++u)
+#pragma unroll
+                for (int e = 0; e < W; ++e) s += __builtin_amdgcn_exp2f(fmaf(x[u][e], kLog2e, -shift));
         }
     }
+    const float part_max = group_reduce<kSplitThreads, true>(m, scratch);
+    s = m > -INFINITY ? s * __builtin_amdgcn_exp2f((m - part_max) * kLog2e) : 0.0f;
+    s = group_reduce<kSplitThreads, false>(s, scratch);
+    if (threadIdx.x == 0) {
+        SplitPartial r;
+        r.max = part_max;
+        r.sum = s;
+        partials[seg * gridDim.x + blockIdx.x] = r;
+    }
+}
+
+template <typename T, bool kVec>
+__global__ __launch_bounds__(kSplitThreads) void softmax_split_finish_kernel(SoftmaxParams p, int64_t part_len, const SplitPartial *partials) {
+    constexpr int W = WideAccess<T, kVec>::kWidth;
+    __shared__ float scratch[kSplitThreads / 64];
+    const int64_t seg = blockIdx.y;
+    const int64_t row = seg / p.segments;
+    const int64_t start = (seg % p.segments) * p.block + (int64_t)blockIdx.x * part_len;
+    const int64_t seg_end = min((seg % p.segments + 1) * p.block, p.cols);
+    const int64_t count = max((int64_t)0, min(part_len, seg_end - start));
+    // the parts of this segment (at most one per thread)
+    SplitPartial mine;
+    mine.max = -INFINITY;
+    mine.sum = 0.0f;
+    if (threadIdx.x < gridDim.x) mine = partials[seg * gridDim.x + threadIdx.x];
+    const float total_max = group_reduce<kSplitThreads, true>(mine.max, scratch);
+    const float scaled = mine.max > -INFINITY ? mine.sum * __builtin_amdgcn_exp2f((mine.max - total_max) * kLog2e) : 0.0f;
+    const float inv = 1.0f / group_reduce<kSplitThreads, false>(scaled, scratch);
+    const float shift = total_max * kLog2e;
+    const T *src = (const T *)p.in + row * p.in_row_stride + start * p.in_col_stride;
+    T *dst = (T *)p.out + row * p.out_row_stride + start * p.out_col_stride;
+    const int64_t pieces = (count + W - 1) / W;
+    for (int64_t base = threadIdx.x; base < pieces; base += kSplitThreads * kSplitUnroll) {
+        float x[kSplitUnroll][W];
+#pragma unroll
+        for (int u = 0; u < kSplitUnroll; ++u) wide_load<T, kVec>(src, p.in_col_stride, base + u * kSplitThreads, count, x[u]);
+#pragma unroll
+        for (int u = 0; u < kSplitUnroll; ++u) wide_store<T, kVec>(dst, p.out_col_stride, base + u * kSplitThreads, count, x[u], shift, inv);
+    }
+}
+
+// true when the segments were served by the two launches over parts.  `in_registers`: the segments are short
+// enough for the kernels that read them once (those win unless too few workgroups are left to fetch: measured
+// fp32 [128, 65536] 13 us against 18 us in parts, [16, 65536] 9.1 against 8.1, [16, 262144] fp16 77 against 12).
+template <typename T>
+bool run_split(const SoftmaxParams &p, int64_t len, bool in_registers, hipStream_t stream, hipError_t *status) {
+    const int64_t total = p.rows * p.segments;
+    const int64_t bytes = len * (int64_t)sizeof(T);
+    if (total > 128) return false;
+    if (in_registers ? (bytes < (1 << 18) || total > 16) : bytes < (1 << 16)) return false;
+    const int64_t wanted = std::min<int64_t>(kSplitThreads, std::max<int64_t>(2, 1024 / total));  // (the finishing launch reads one part per thread)
+    int64_t part_len = std::max<int64_t>(4096, (((len + wanted - 1) / wanted + 2047) / 2048) * 2048);
+    const int64_t parts = (len + part_len - 1) / part_len;
+    if (parts < 2 || parts > kSplitThreads) return false;
+    WorkspaceLease lease(stream);
+    SplitPartial *partials = (SplitPartial *)lease.get(kWorkspaceSoftmaxParts, (size_t)(total * parts) * sizeof(SplitPartial));
+    if (partials == nullptr) return false;  // no scratch: one workgroup per segment
+    const dim3 grid((unsigned)parts, (unsigned)total), block(kSplitThreads);
+    note_launch(kLaunchSoftmax, kSplitThreads, "softmax_split_partial_kernel + softmax_split_finish_kernel, long segments cut into parts");
+    if (p.in_col_stride == 1 && p.out_col_stride == 1) {
+        softmax_split_partial_kernel<T, true><<<grid, block, 0, stream>>>(p, part_len, partials);
+        softmax_split_finish_kernel<T, true><<<grid, block, 0, stream>>>(p, part_len, partials);
+    } else {
+        softmax_split_partial_kernel<T, false><<<grid, block, 0, stream>>>(p, part_len, partials);
+        softmax_split_finish_kernel<T, false><<<grid, block, 0, stream>>>(p, part_len, partials);
+    }
+    *status = hipGetLastError();
+    return true;
 }
 
 template <typename T, int kRowThreads>
@@ -336,7 +498,13 @@ int run_softmax(const SoftmaxParams &p, int variant, hipStream_t stream) {
             if (p.cols <= 8) return (int)launch_thread_per_row<T, 2>(p, stream);  // (up to 32 pieces of one element would not stay in registers)
         }
     }
-    if (vector_ok && len <= (int64_t)1024 * 16 * W) {
+    // (a row of 16 vectors of 2-byte elements per thread -- 128 floats -- does not stay in the registers of 1024 threads)
+    const bool in_registers = vector_ok && len <= (int64_t)1024 * 64;
+    if (variant == 0) {
+        hipError_t status = hipSuccess;
+        if (run_split<T>(p, len, in_registers, stream, &status)) return (int)status;
+    }
+    if (in_registers || (vector_ok && variant != 0 && len <= (int64_t)1024 * 16 * W)) {
         const bool wave_fits = len <= (int64_t)64 * 16 * W;
         bool use_wave = wave_fits && len <= (int64_t)64 * 8 * W;  // default: keep <= 8 vectors per lane
         // few segments: a workgroup each, so that more of the chip has something to fetch
@@ -368,7 +536,10 @@ int run_softmax(const SoftmaxParams &p, int variant, hipStream_t stream) {
     if (len <= 256 * 32) return (int)launch_elem<T, 256, 64>(p, stream);
     if (len <= 1024 * 16) return (int)launch_elem<T, 1024, 16>(p, stream);
     note_launch(kLaunchSoftmax, kLoopThreads, "softmax_loop_kernel, two sweeps over a long row segment");
-    softmax_loop_kernel<T><<<dim3((unsigned)total), dim3(kLoopThreads), 0, stream>>>(p);
+    if (p.in_col_stride == 1 && p.out_col_stride == 1)
+        softmax_loop_kernel<T, true><<<dim3((unsigned)total), dim3(kLoopThreads), 0, stream>>>(p);
+    else
+        softmax_loop_kernel<T, false><<<dim3((unsigned)total), dim3(kLoopThreads), 0, stream>>>(p);
     return (int)hipGetLastError();
 }
 

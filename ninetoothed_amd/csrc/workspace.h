@@ -19,7 +19,7 @@ namespace nt {
 enum WorkspacePurpose {
     kWorkspaceConvInput, kWorkspaceConvFilter, kWorkspaceAttentionNarrow, kWorkspaceGemmParts, kWorkspaceAttentionParts,
     kWorkspaceGemmLhsWidened, kWorkspaceGemmRhsWidened, kWorkspaceGemmBiasWidened, kWorkspaceGemmLhsDense, kWorkspaceGemmRhsDense,
-    kWorkspaceAttentionPaddedQ, kWorkspaceAttentionPaddedK, kWorkspaceAttentionPaddedV, kWorkspaceAttentionPaddedO, kWorkspacePurposes
+    kWorkspaceAttentionPaddedQ, kWorkspaceAttentionPaddedK, kWorkspaceAttentionPaddedV, kWorkspaceAttentionPaddedO, kWorkspaceSoftmaxParts, kWorkspacePurposes
 };
 
 // Holds the registry lock from construction to destruction: create it, take the buffers,

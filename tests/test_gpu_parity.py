@@ -420,6 +420,67 @@ def test_softmax_half_blocks_and_strides():
     assert torch.allclose(out, torch.softmax(view, dim=-1), rtol=1e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("dtype", (torch.float32, torch.float16, torch.bfloat16))
+def test_softmax_few_long_rows_are_cut_into_parts(dtype):
+    """Up to 128 segments too long for the one-sweep kernels (or a handful that would leave most of the chip idle) are
+    cut into parts: one launch for every part's maximum and sum, one that combines them and writes.  Checked: rows
+    at an odd element offset in sentinel-filled buffers, a part that is all -inf, columns two elements apart,
+    segments shorter than the row (against the oracle), a row of 2^24 elements (256 parts), and -- inside a captured
+    graph on a stream that has no scratch buffer yet -- the fallback to one workgroup per segment."""
+    from ninetoothed_amd import runtime
+
+    tolerance = {torch.float32: dict(rtol=1e-5, atol=1e-7), torch.float16: dict(rtol=2e-3, atol=1e-6), torch.bfloat16: dict(rtol=1.6e-2, atol=1e-6)}[dtype]
+    kernel = ninetoothed.make(programs.softmax.arrangement, programs.softmax.application, programs.softmax.tensors())
+    for (m, n, first, step) in ((3, 200001, 1, 1), (16, 262144, 0, 1), (1, 1 << 24, 0, 1), (128, 50257, 3, 1), (5, 70000, 0, 2), (2, 40000, 1, 1)):
+        pitch = first + n * step + 5
+        source = torch.full((m, pitch), float("inf"), dtype=dtype, device="cuda")
+        x = source[:, first : first + n * step : step]
+        x.copy_(torch.randn(m, n, device="cuda").to(dtype))
+        x[0, n - 1] = 12.0
+        x[m - 1, 8192:20000] = float("-inf")  # a whole part (and more) without a finite element
+        buffer = torch.full((m, pitch), 7.0, dtype=dtype, device="cuda")
+        out = buffer[:, first : first + n * step : step]
+        kernel(x, out, BLOCK_SIZE=1 << (n - 1).bit_length())
+        _native_only(kernel, "launch_nt_softmax")
+        assert "softmax_split" in runtime.last_launch(), (m, n, runtime.last_launch())
+        expected = torch.softmax(x.float(), dim=-1)
+        assert torch.allclose(out.float(), expected, **tolerance), (m, n, first, step)
+        if n <= 300000:  # (a longer row's fp16 outputs are denormals or zeros)
+            assert abs(float(out.float().sum(dim=-1).min()) - 1.0) < (1e-4 if dtype == torch.float32 else 2e-2)
+        untouched = torch.ones_like(buffer, dtype=torch.bool)
+        untouched[:, first : first + n * step : step] = False
+        assert bool((buffer[untouched] == 7.0).all())
+    if dtype == torch.float32:
+        # segments of 2^17 elements of rows of 300000: each segment is a softmax of its own
+        y = torch.randn(3, 300000)
+        out = _softmax(y.cuda(), block_size=1 << 17)
+        assert "softmax_split" in runtime.last_launch(), runtime.last_launch()
+        assert np.allclose(out.cpu().numpy(), oracle.softmax(y.numpy(), block_size=1 << 17), rtol=1e-5, atol=1e-7)
+    # under capture on a stream without a buffer for the parts: one workgroup per segment; afterwards, the parts
+    x = torch.randn(4, 300000, device="cuda").to(dtype)
+    out = torch.empty_like(x)
+    expected = torch.softmax(x.float(), dim=-1)
+    stream = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    runtime.library().nt_release_workspaces()  # (torch hands out its streams again and again: this one may have a buffer from an earlier test)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        kernel(x, out, BLOCK_SIZE=1 << 19)
+        inside = runtime.last_launch()
+    assert "softmax_loop_kernel" in inside, inside
+    for replay in range(3):
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.allclose(out.float(), expected, **tolerance), replay
+        with torch.cuda.stream(stream):
+            kernel(x, out, BLOCK_SIZE=1 << 19)  # eager work between the replays: takes the buffer, runs in parts
+        assert "softmax_split" in runtime.last_launch()
+        torch.cuda.synchronize()
+        assert torch.allclose(out.float(), expected, **tolerance), replay
+
+
 def test_softmax_baseline_shape_properties():
     x = torch.randn(4096, 4096, device="cuda")
     out = _softmax(x)
