@@ -1024,7 +1024,8 @@ __global__ __launch_bounds__(256) void attention_f32_kernel(AttentionParams p) {
             const float *src = K + (int64_t)min(kv0 + l32, p.seq_k - 1) * p.k_strides[2] + g * kHalf;
 #pragma unroll
             for (int c = 0; c < kHalf / 4; ++c) {
-                const float4_t v = *(const float4_t *)(src + 4 * c);
+                typedef float4_t unaligned_float4_t __attribute__((aligned(4)));  // (rows of K may start anywhere: global accesses need the element's alignment only)
+                const float4_t v = *(const unaligned_float4_t *)(src + 4 * c);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) s_acc = __builtin_amdgcn_mfma_f32_32x32x2f32(v[e], qf[4 * c + e], s_acc, 0, 0, 0);
             }
@@ -1101,8 +1102,7 @@ int launch_attention_f32(AttentionParams &p, hipStream_t stream) {
 // dimensions, and calls with a hint (the fast way: sixteen times the MFMA rate): the 16-bit kernels on fp16 copies
 // of K and V (values beyond the fp16 range overflow there).
 int attention_float32(AttentionParams p, int head_dim, const NineToothedTensor &k, const NineToothedTensor &v, bool exact, hipStream_t stream) {
-    // (rows of K are read 16 bytes at a time)
-    if (exact && k.strides[3] == 1 && v.strides[3] == 1 && ((uintptr_t)k.data & 15) == 0 && k.strides[0] % 4 == 0 && k.strides[1] % 4 == 0 && k.strides[2] % 4 == 0) {
+    if (exact && k.strides[3] == 1 && v.strides[3] == 1) {
         if (head_dim == 128) return launch_attention_f32<128>(p, stream);
         if (head_dim == 64) return launch_attention_f32<64>(p, stream);
         if (head_dim == 32) return launch_attention_f32<32>(p, stream);
@@ -1116,6 +1116,7 @@ int attention_float32(AttentionParams p, int head_dim, const NineToothedTensor &
                                                                   k.strides[1], k.strides[2], k.strides[3]);
     attention_narrow_kernel<<<dim3(blocks), dim3(256), 0, stream>>>((const float *)v.data, narrow + total, total, p.heads, p.seq_k, head_dim,
                                                                   v.strides[0], v.strides[1], v.strides[2], v.strides[3]);
+    note_launch(kLaunchAttention, 0, "fp32 tensors on fp16 copies of K and V: attention_narrow_kernel twice, then the 16-bit kernel");
     p.k = narrow;
     p.v = narrow + total;
     const int64_t contiguous[3] = {(int64_t)p.heads * p.seq_k * head_dim, (int64_t)p.seq_k * head_dim, head_dim};

@@ -1569,17 +1569,19 @@ def test_attention_float32_tensors(seq_len, is_causal):
 
 @pytest.mark.parametrize("is_causal", (False, True))
 @pytest.mark.parametrize("batch, heads, seq_q, seq_k, emb_dim", ((2, 3, 200, 200, 64), (1, 2, 77, 77, 128), (2, 2, 130, 130, 32), (1, 3, 50, 211, 64), (1, 2, 300, 45, 128)))
-def test_attention_float32_tensors_are_not_narrowed(batch, heads, seq_q, seq_k, emb_dim, is_causal):
+@pytest.mark.parametrize("pad", (4, 3))
+def test_attention_float32_tensors_are_not_narrowed(batch, heads, seq_q, seq_k, emb_dim, is_causal, pad):
     """Head dimensions 32, 64 and 128 of fp32 tensors run in fp32 throughout: against a float64 reference at fp32
     tolerances, on operands that the fp16 range does not hold (keys around 1e5 against queries around 1e-5, values
-    around 1e6), ragged and unequal lengths, K and V inside Inf-filled rows."""
+    around 1e6), ragged and unequal lengths, K and V inside Inf-filled rows -- whose pitch is a multiple of 16 bytes
+    or not: the precision of the result must not depend on where the rows of K start."""
     generator = torch.Generator().manual_seed(seq_q + emb_dim)
     q = torch.randn(batch, heads, seq_q, emb_dim, generator=generator) * 1e-5
-    wide_k = torch.full((batch, heads, seq_k, emb_dim + 4), float("inf"))
-    wide_v = torch.full((batch, heads, seq_k, emb_dim + 4), float("inf"))
-    wide_k[..., :emb_dim] = torch.randn(batch, heads, seq_k, emb_dim, generator=generator) * 1e5
+    wide_k = torch.full((batch, heads, seq_k, emb_dim + pad), float("inf"))
+    wide_v = torch.full((batch, heads, seq_k, emb_dim + pad), float("inf"))
+    wide_k[..., pad - 3 : pad - 3 + emb_dim] = torch.randn(batch, heads, seq_k, emb_dim, generator=generator) * 1e5
     wide_v[..., :emb_dim] = torch.randn(batch, heads, seq_k, emb_dim, generator=generator) * 1e6
-    k, v = wide_k.cuda()[..., :emb_dim], wide_v.cuda()[..., :emb_dim]
+    k, v = wide_k.cuda()[..., pad - 3 : pad - 3 + emb_dim], wide_v.cuda()[..., :emb_dim]
     scale = emb_dim**-0.5
     out = _attention(q.cuda(), k, v, is_causal, scale)
     assert out.dtype == torch.float32
