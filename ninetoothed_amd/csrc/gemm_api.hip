@@ -32,6 +32,7 @@ struct GemmProblem {
     // set by the entry point that allocates nothing: split-K parts go here instead of the stream's workspace
     float *fixed_scratch = nullptr;
     size_t fixed_scratch_bytes = 0;
+    bool hinted = false;  // the caller gave block sizes: the call stays on kernels without scratch memory
     bool addmm() const { return bias != nullptr; }
 };
 
@@ -247,9 +248,72 @@ bool generic_accepts(const GemmProblem &q) {
     return q.m >= 0 && q.n >= 0 && q.k >= 0;
 }
 
+// out = epilogue(sum over the parts of the k range), any output strides; fp32 throughout (an fp32 addmm does not round its product)
+__global__ __launch_bounds__(256) void gemm_generic_reduce_kernel(const float *parts, int num_parts, int m, int n, float *c, int64_t scm, int64_t scn, const float *bias,
+                                                                 int64_t bias_stride_m, int64_t bias_stride_n, float alpha, float beta) {
+    const int64_t total = (int64_t)m * n;
+    for (int64_t index = (int64_t)blockIdx.x * 256 + threadIdx.x; index < total; index += (int64_t)gridDim.x * 256) {
+        float sum = parts[index];
+        for (int part = 1; part < num_parts; ++part) sum += parts[index + (int64_t)part * total];
+        const int row = (int)(index / n), col = (int)(index - (int64_t)row * n);
+        if (bias != nullptr) sum = beta * bias[(int64_t)row * bias_stride_m + (int64_t)col * bias_stride_n] + alpha * sum;
+        c[(int64_t)row * scm + (int64_t)col * scn] = sum;
+    }
+}
+
+// fp32 products with too few 128 x 128 tiles for the chip: parts of the k range as the grid's y extent, each writing an
+// fp32 tile to scratch memory of the stream, then the sum (512^3 50 -> 23 us, 1024^3 96 -> 41, [128, 4096] x [4096, 128]
+// 347 -> 28, [64, 8192] x [8192, 64] 776 -> 38).  NINETOOTHED_NO_KERNEL: not worth it, or no scratch -- the caller runs the product in one pass.
+hipError_t generic_launch_in_parts(const GemmProblem &q, hipStream_t stream) {
+    const int64_t tiles = (int64_t)ceil_div(q.m, kGenBM) * ceil_div(q.n, kGenBN);
+    const int num_kt = ceil_div(q.k, kGenBK);
+    if (q.batch != 1 || q.hinted || q.fixed_scratch != nullptr || tiles == 0 || tiles >= 192) return (hipError_t)NINETOOTHED_NO_KERNEL;
+    int64_t parts = std::min<int64_t>({(512 + tiles - 1) / tiles, num_kt / 4, 256});
+    while (parts >= 2 && parts * q.m * q.n * 4 > (int64_t(64) << 20)) --parts;
+    if (parts < 2) return (hipError_t)NINETOOTHED_NO_KERNEL;
+    const int kt_per_part = (int)((num_kt + parts - 1) / parts);
+    parts = (num_kt + kt_per_part - 1) / kt_per_part;  // every part has at least one k tile
+    WorkspaceLease lease(stream);
+    float *scratch = (float *)lease.get(kWorkspaceGemmParts, (size_t)parts * q.m * q.n * sizeof(float));
+    if (scratch == nullptr) return (hipError_t)NINETOOTHED_NO_KERNEL;
+    StridedProblem<float, float> prob;
+    prob.m = q.m;
+    prob.n = q.n;
+    prob.k = q.k;
+    prob.a = (const float *)q.a;
+    prob.b = (const float *)q.b;
+    prob.c = scratch;
+    prob.bias = nullptr;
+    prob.sam = q.sam;
+    prob.sak = q.sak;
+    prob.sbk = q.sbk;
+    prob.sbn = q.sbn;
+    prob.scm = q.n;
+    prob.scn = 1;
+    prob.sbm_ = prob.sbn_ = 0;
+    prob.alpha = 1.0f;
+    prob.beta = 0.0f;
+    prob.a_batch = prob.b_batch = prob.bias_batch = 0;
+    prob.c_batch = (int64_t)q.m * q.n;
+    prob.k_chunk = kt_per_part * kGenBK;
+    note_launch(kLaunchGemm, 0, "128x128x32 waves 2x2 any-stride, k range in parts, then gemm_generic_reduce_kernel");
+    gemm_generic_kernel<StridedProblem<float, float>><<<dim3((unsigned)tiles, (unsigned)parts), dim3(kGenThreads), 0, stream>>>(prob);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return err;
+    const int64_t total = (int64_t)q.m * q.n;
+    gemm_generic_reduce_kernel<<<dim3((unsigned)std::min<int64_t>((total + 255) / 256, 256 * 8)), dim3(256), 0, stream>>>(
+        scratch, (int)parts, q.m, q.n, (float *)q.c, q.scm, q.scn, (const float *)q.bias, q.sim, q.sin, q.alpha, q.beta);
+    return hipGetLastError();
+}
+
 template <typename T, typename TOut>
 hipError_t generic_launch_typed(const GemmProblem &q, hipStream_t stream) {
+    if constexpr (std::is_same<T, float>::value) {
+        const hipError_t in_parts = generic_launch_in_parts(q, stream);
+        if ((int)in_parts != NINETOOTHED_NO_KERNEL) return in_parts;
+    }
     StridedProblem<T, TOut> prob;
+    prob.k_chunk = 0;
     prob.m = q.m;
     prob.n = q.n;
     prob.k = q.k;
@@ -710,7 +774,14 @@ int run_gemm(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk, b
         if (copied != NINETOOTHED_NO_KERNEL) return copied;
     }
     note_launch(kLaunchGemm, choice, kInstances[choice].name);
-    int result = (int)kInstances[choice].launch(q, stream);
+    int result;
+    if (bm > 0 || bn > 0 || bk > 0) {
+        GemmProblem hinted = q;
+        hinted.hinted = true;
+        result = (int)kInstances[choice].launch(hinted, stream);
+    } else {
+        result = (int)kInstances[choice].launch(q, stream);
+    }
     if (result == NINETOOTHED_NO_KERNEL && is_split(choice)) {  // a split-K instance without scratch memory
         for (int fallback : {(int)kTail64x64x64, (int)kTail128x128x64, (int)kTail256x256x32, (int)kAnyStride})
             if (kInstances[fallback].accepts(q)) {

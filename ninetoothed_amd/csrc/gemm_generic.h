@@ -134,8 +134,16 @@ struct StridedProblem {
     int64_t sam, sak, sbk, sbn, scm, scn, sbm_, sbn_;  // sbm_/sbn_: bias strides
     float alpha, beta;
     int64_t a_batch, b_batch, c_batch, bias_batch;  // element strides between the products of a batched launch
+    int k_chunk;  // > 0: the grid's y coordinate is a part of the k range of one product, this many positions long
 
     NT_DEVICE void select_batch(int index) {
+        if (k_chunk > 0) {
+            a += (int64_t)index * k_chunk * sak;
+            b += (int64_t)index * k_chunk * sbk;
+            c += index * c_batch;
+            k = min(k_chunk, k - index * k_chunk);
+            return;
+        }
         a += index * a_batch;
         b += index * b_batch;
         c += index * c_batch;

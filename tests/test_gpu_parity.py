@@ -110,6 +110,64 @@ def test_addmm_float32_through_the_c_abi():
     assert torch.allclose(out.double(), expected, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("m, n, k", ((128, 128, 4096), (100, 36, 5001), (1000, 1000, 1000), (512, 512, 512), (1, 7, 300)))
+def test_float32_products_with_few_tiles_run_the_k_range_in_parts(m, n, k):
+    """fp32 products of fewer than 192 tiles of 128 x 128 with at least 8 k tiles of 32: parts of the k range on
+    workgroups of their own, partial tiles in scratch memory, then the sum and the addmm epilogue -- against float64,
+    with operands and an output of any strides (the output inside a sentinel-filled buffer), as matmul and as addmm;
+    block sizes keep the call on the one-pass kernel, and so does a captured graph on a stream without scratch."""
+    from ninetoothed_amd import runtime
+
+    lib = runtime.library()
+    fp32 = runtime.DATA_TYPE_INDEX["fp32"]
+    a = _randn(m, k, dtype=torch.float32).cuda()
+    b_storage = _randn(n, k + 3, dtype=torch.float32).cuda()
+    b = b_storage[:, 1 : k + 1].t()  # [k, n] stored by columns, rows off 16-byte boundaries
+    bias = _randn(m, n, dtype=torch.float32).cuda()
+    buffer = torch.full((m, 2 * n + 1), 7.0, dtype=torch.float32, device="cuda")
+    out = buffer[:, 1::2]
+    exact = a.double() @ b.double()
+    tolerance = dict(rtol=1e-4, atol=1e-4 * max(1.0, (k / 512) ** 0.5))
+    tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (a, b, out, bias)]
+    beta, alpha = runtime.ArgumentTensor.from_scalar(0.5), runtime.ArgumentTensor.from_scalar(-1.25)
+    in_parts = k >= 8 * 32
+
+    runtime.check(lib.launch_nt_matmul(runtime.current_stream(), tensors[0], tensors[1], tensors[2], fp32, fp32, 0, 0, 0))
+    assert ("k range in parts" in runtime.last_launch()) == in_parts, runtime.last_launch()
+    assert torch.allclose(out.double(), exact, **tolerance)
+    assert bool((buffer[:, 0::2] == 7.0).all())
+    first = out.clone()
+    runtime.check(lib.launch_nt_matmul(runtime.current_stream(), tensors[0], tensors[1], tensors[2], fp32, fp32, 128, 128, 32))
+    assert "k range in parts" not in runtime.last_launch(), runtime.last_launch()
+    assert torch.allclose(out.double(), exact, **tolerance)
+    # (summing the k range in parts is the more accurate order)
+    assert float((first.double() - exact).abs().max()) <= 2.0 * float((out.double() - exact).abs().max()) + 1e-6
+
+    out.fill_(float("nan"))
+    runtime.check(lib.launch_nt_addmm(runtime.current_stream(), tensors[3], tensors[0], tensors[1], beta, alpha, tensors[2], fp32, 0, 0, 0))
+    assert ("k range in parts" in runtime.last_launch()) == in_parts, runtime.last_launch()
+    assert torch.allclose(out.double(), 0.5 * bias.double() - 1.25 * exact, **tolerance)
+    assert bool((buffer[:, 0::2] == 7.0).all())
+
+    # captured on a stream that has no scratch buffer: one pass; replays checked
+    torch.cuda.synchronize()
+    lib.nt_release_workspaces()
+    kernel = _matmul_kernel()
+    plain = torch.empty(m, n, dtype=torch.float32, device="cuda")
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        kernel(a, b, plain)
+        inside = runtime.last_launch()
+    assert "k range in parts" not in inside, inside
+    for replay in range(2):
+        plain.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.allclose(plain.double(), exact, **tolerance), replay
+
+
 @pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
 @pytest.mark.parametrize("m, n, k", ((512, 512, 512), (1000, 768, 1024), (4096, 2048, 4096)))
 def test_matmul_float32_output_on_the_fast_instances(m, n, k, dtype):
