@@ -758,9 +758,46 @@ GemmProblem transposed_problem(const GemmProblem &q) {
     return t;
 }
 
+// A product whose 256 x 256 tiles are a few more than whole rounds of the chip's 256 CUs (17 x 17 = 289 of them for
+// 4352^2) pays a whole round for the few: the tile rows that fill whole rounds run in one pass, the rows left over
+// -- at most 51 tiles -- as a product of their own with the k range in parts, so that they occupy the chip once for
+// a fraction of a round.  NINETOOTHED_NO_KERNEL when the shape is not of that kind or scratch memory is not to be had.
+int run_gemm_last_rows_in_parts(hipStream_t stream, const GemmProblem &q) {
+    if ((q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) || q.batch != 1 || q.fixed_scratch != nullptr) return NINETOOTHED_NO_KERNEL;
+    static const bool enabled = getenv("NT_GEMM_NO_ROW_SPLIT") == nullptr;
+    if (!enabled) return NINETOOTHED_NO_KERNEL;
+    const int64_t tiles_m = ceil_div(q.m, 256), tiles_n = ceil_div(q.n, 256), tiles = tiles_m * tiles_n;
+    // (measured, one pass -> this way: 4352 x 4096 x 4352 162 -> 147 us, 4096 x 4096 x 4352 158 -> 133, 5120 x 4096 x 3584
+    // 159 -> 142, 4104^3 226 -> 191; not for more than three rounds -- 8192 x 4096 x 8448 436 -> 447 --, for more than 51
+    // tiles left over -- 4608^2 x 4096, 72 of them: 162 -> 173 -- or a short k range -- 4352 x 1024 x 4352 49 -> 63)
+    if (tiles <= 256 || tiles > 768 || tiles % 256 == 0 || q.k < 2048) return NINETOOTHED_NO_KERNEL;
+    const int64_t top_rows = tiles / 256 * 256 / tiles_n;
+    const int64_t bottom_tiles = (tiles_m - top_rows) * tiles_n;
+    if (top_rows < 1 || top_rows >= tiles_m || bottom_tiles * 5 > 256) return NINETOOTHED_NO_KERNEL;
+    if (ceil_div(top_rows * tiles_n, (int64_t)256) >= ceil_div(tiles, (int64_t)256)) return NINETOOTHED_NO_KERNEL;  // (no round saved)
+    const int64_t size = q.dtype == NINETOOTHED_FLOAT16 || q.dtype == NINETOOTHED_BFLOAT16 ? 2 : 4;
+    const int64_t out_size = q.out_dtype == NINETOOTHED_FLOAT32 ? 4 : size;
+    GemmProblem top = q, bottom = q;
+    top.m = (int)(top_rows * 256);
+    bottom.m = q.m - top.m;
+    bottom.a = (const char *)q.a + (int64_t)top.m * q.sam * size;
+    bottom.c = (char *)q.c + (int64_t)top.m * q.scm * out_size;
+    if (q.bias != nullptr) bottom.bias = (const char *)q.bias + (int64_t)top.m * q.sim * size;
+    const int whole = kInstances[k256x256x32].accepts(top) ? (int)k256x256x32 : (int)kTail256x256x32;
+    if (!kInstances[whole].accepts(top) || !kInstances[kSplit256x256x32].accepts(bottom)) return NINETOOTHED_NO_KERNEL;
+    int result = (int)kInstances[kSplit256x256x32].launch(bottom, stream);  // (first: it is the one that may find no scratch memory)
+    if (result != 0) return result;
+    note_launch(kLaunchGemm, whole, "256x256x32 tiles: the tile rows that fill whole rounds in one pass, the last rows with the k range in parts");
+    return (int)kInstances[whole].launch(top, stream);
+}
+
 int run_gemm(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk, bool may_copy) {
     if (q.m == 0 || q.n == 0) return 0;
     if (output_by_columns(q)) return run_gemm(stream, transposed_problem(q), bn, bm, bk, may_copy);
+    if (bm <= 0 && bn <= 0 && bk <= 0) {
+        const int rows_split = run_gemm_last_rows_in_parts(stream, q);
+        if (rows_split != NINETOOTHED_NO_KERNEL) return rows_split;
+    }
     if (q.dtype == NINETOOTHED_FLOAT8_E5M2) {
         const int widened = run_gemm_on_widened_copies(stream, q, bm, bn, bk);
         if (widened != NINETOOTHED_NO_KERNEL) return widened;

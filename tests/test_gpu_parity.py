@@ -110,6 +110,40 @@ def test_addmm_float32_through_the_c_abi():
     assert torch.allclose(out.double(), expected, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
+@pytest.mark.parametrize("m, n, k", ((4352, 4352, 2048), (4096, 4352, 2304), (4104, 4104, 2056)))
+def test_products_a_few_tiles_over_whole_rounds_split_their_last_tile_rows(m, n, k, dtype):
+    """17 x 17 (16 x 17) tiles of 256 x 256 on 256 CUs: the tile rows that fill a whole round run in one pass, the rows
+    left over as a product of their own with the k range in parts.  Whole output of matmul and addmm against the
+    program's arithmetic in fp32; block sizes keep the call in one pass, and both ways agree."""
+    from ninetoothed_amd import runtime
+
+    lib = runtime.library()
+    tag = runtime.DATA_TYPE_INDEX["fp16" if dtype == torch.float16 else "bf16"]
+    a, b, bias = _randn(m, k, dtype=dtype).cuda(), _randn(k, n, dtype=dtype, scale=0.1).cuda(), _randn(m, n, dtype=dtype).cuda()
+    out = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+    tensors = [runtime.ArgumentTensor.from_torch_tensor(t) for t in (a, b, out, bias)]
+    product = a.float() @ b.float()
+    tolerance = dict(rtol=1e-2, atol=1e-2) if dtype == torch.float16 else dict(rtol=1e-2, atol=2.0**-7 * float(product.abs().max()))
+    runtime.check(lib.launch_nt_matmul(runtime.current_stream(), tensors[0], tensors[1], tensors[2], tag, tag, 0, 0, 0))
+    assert "last rows with the k range in parts" in runtime.last_launch(), runtime.last_launch()
+    assert torch.allclose(out.float(), product, **tolerance)
+    in_parts = out.clone()
+    out.fill_(float("nan"))
+    runtime.check(lib.launch_nt_matmul(runtime.current_stream(), tensors[0], tensors[1], tensors[2], tag, tag, 256, 256, 32))
+    assert "last rows" not in runtime.last_launch(), runtime.last_launch()
+    assert torch.allclose(out.float(), in_parts.float(), **tolerance)
+    top = (256 // ((n + 255) // 256)) * 256  # the rows of the one-pass part: the same kernel, the same bits
+    assert torch.equal(out[:top], in_parts[:top])
+    out.fill_(float("nan"))
+    beta, alpha = runtime.ArgumentTensor.from_scalar(0.5), runtime.ArgumentTensor.from_scalar(2.0)
+    runtime.check(lib.launch_nt_addmm(runtime.current_stream(), tensors[3], tensors[0], tensors[1], beta, alpha, tensors[2], tag, 0, 0, 0))
+    assert "last rows with the k range in parts" in runtime.last_launch(), runtime.last_launch()
+    expected = 0.5 * bias.float() + 2.0 * product.to(dtype).float()
+    wide = dict(rtol=1e-2, atol=tolerance["atol"] * 2.0 + 1e-2)  # (the product is rounded before it is doubled: two of its ulps)
+    assert torch.allclose(out.float(), expected, **wide)
+
+
 @pytest.mark.parametrize("m, n, k", ((128, 128, 4096), (100, 36, 5001), (1000, 1000, 1000), (512, 512, 512), (1, 7, 300)))
 def test_float32_products_with_few_tiles_run_the_k_range_in_parts(m, n, k):
     """fp32 products of fewer than 192 tiles of 128 x 128 with at least 8 k tiles of 32: parts of the k range on
