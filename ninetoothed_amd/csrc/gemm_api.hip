@@ -767,8 +767,8 @@ int run_gemm_last_rows_in_parts(hipStream_t stream, const GemmProblem &q) {
     static const bool enabled = getenv("NT_GEMM_NO_ROW_SPLIT") == nullptr;
     if (!enabled) return NINETOOTHED_NO_KERNEL;
     const int64_t tiles_m = ceil_div(q.m, 256), tiles_n = ceil_div(q.n, 256), tiles = tiles_m * tiles_n;
-    // (measured, one pass -> this way: 4352 x 4096 x 4352 162 -> 147 us, 4096 x 4096 x 4352 158 -> 133, 5120 x 4096 x 3584
-    // 159 -> 142, 4104^3 226 -> 191; not for more than three rounds -- 8192 x 4096 x 8448 436 -> 447 --, for more than 51
+    // (measured, one pass -> this way: 4352 x 4096 x 4352 160 -> 143 us, 4096 x 4096 x 4352 158 -> 135, 5120 x 4096 x 3584
+    // 159 -> 139, 4104^3 172 -> 143; not for more than three rounds -- 8192 x 4096 x 8448 436 -> 447 --, for more than 51
     // tiles left over -- 4608^2 x 4096, 72 of them: 162 -> 173 -- or a short k range -- 4352 x 1024 x 4352 49 -> 63)
     if (tiles <= 256 || tiles > 768 || tiles % 256 == 0 || q.k < 2048) return NINETOOTHED_NO_KERNEL;
     const int64_t top_rows = tiles / 256 * 256 / tiles_n;

@@ -303,23 +303,21 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         if constexpr (kLoad == 1) {
             const int a_k = kt * BK * 2;
             const int b_k = kBT ? a_k : kt * BK * (int)p.ldb * 2;
-            if (kTail && kt == all_k - 1 && tail_chunks < kAChunksPerRow) {  // uniform: the partial last k tile
+            if constexpr (kTail) {
+                // the partial last k tile, without a branch: a lane whose 16-byte chunk lies beyond K reads from behind
+                // the descriptor, zeros (the chunk a lane fills is the same for every instruction: their rows are a
+                // multiple of the swizzle's period of 16 apart)
                 constexpr unsigned kBehind = 0x7fffffffu;  // behind every descriptor (their sizes stay below 2^31)
+                static_assert(kWaves * kARowsPerInstr % 16 == 0, "the swizzle of a row repeats every 16 rows");
+                const int chunks = kt == all_k - 1 ? tail_chunks : kAChunksPerRow;
+                const int row = wave * kARowsPerInstr + lane / kAChunksPerRow;
+                const bool inside = (kTile16 ? a_phys_chunk16<BK>(row, lane % kAChunksPerRow) : a_phys_chunk<BK>(row, lane % kAChunksPerRow)) < chunks;
 #pragma unroll
-                for (int j = 0; j < kAInstr; ++j) {
-                    const int row = (j * kWaves + wave) * kARowsPerInstr + lane / kAChunksPerRow;
-                    const bool inside = (kTile16 ? a_phys_chunk16<BK>(row, lane % kAChunksPerRow) : a_phys_chunk<BK>(row, lane % kAChunksPerRow)) < tail_chunks;
+                for (int j = 0; j < kAInstr; ++j)
                     __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, sa + (j * kWaves + wave) * 1024, 16, inside ? a_src[j] : kBehind, a_k, 0, kAux);
-                }
 #pragma unroll
-                for (int j = 0; j < kBInstr; ++j) {
-                    bool inside = true;
-                    if constexpr (kBT) {
-                        const int row = (j * kWaves + wave) * kARowsPerInstr + lane / kAChunksPerRow;
-                        inside = (kTile16 ? a_phys_chunk16<BK>(row, lane % kAChunksPerRow) : a_phys_chunk<BK>(row, lane % kAChunksPerRow)) < tail_chunks;
-                    }
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, sb + (j * kWaves + wave) * 1024, 16, inside ? b_src[j] : kBehind, b_k, 0, kAux);
-                }
+                for (int j = 0; j < kBInstr; ++j)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, sb + (j * kWaves + wave) * 1024, 16, kBT && !inside ? kBehind : b_src[j], b_k, 0, kAux);
                 return;
             }
 #pragma unroll
@@ -513,14 +511,16 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         auto issue_a_pair = [&](auto stage_tag, int pair, auto first_tag, auto last_tag) {
             constexpr int kFirst = decltype(first_tag)::value, kLast = decltype(last_tag)::value;  // instructions [kFirst, kLast) of the pair
             NT_LDS unsigned char *sa = stage_a(stage_tag);
-            if (kTail && pair == last_pair && pair_chunks < 8) {  // uniform
+            if constexpr (kTail) {
+                // no branch: a lane whose chunk lies beyond K in the last pair reads from behind the descriptor
+                // (the chunk a lane fills is the same for every instruction: their rows are 8 * kWaves apart)
                 constexpr unsigned kBehind = 0x7fffffffu;  // behind every descriptor (their sizes stay below 2^31)
+                const int chunks = pair == last_pair ? pair_chunks : 8;
+                const bool inside = a_phys_chunk16<64>(wave * 8 + lane / 8, lane % 8) < chunks;
+                static_assert(kWaves * 8 % 16 == 0, "the swizzle of a row repeats every 16 rows");
 #pragma unroll
-                for (int j = kFirst; j < kLast; ++j) {
-                    const int row = (j * kWaves + wave) * 8 + lane / 8;
-                    const bool inside = a_phys_chunk16<64>(row, lane % 8) < pair_chunks;
+                for (int j = kFirst; j < kLast; ++j)
                     __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, sa + (j * kWaves + wave) * 1024, 16, inside ? a_pair_src[j] : kBehind, pair * 128, 0, kAux);
-                }
                 return;
             }
 #pragma unroll
@@ -533,14 +533,14 @@ __global__ __launch_bounds__(WM *WN * 64, kWavesPerSimd) void gemm_nn_fast_kerne
         auto issue_b = [&](auto stage_tag, int kt) {
             NT_LDS unsigned char *sb = stage_b(stage_tag);
             const int b_k = kBT ? kt * BK * 2 : kt * BK * (int)p.ldb * 2;
-            if (kTail && kBT && kt == last_k && tail_chunks < kAChunksPerRow) {  // uniform: the partial last k tile of a k-contiguous rhs
+            if constexpr (kTail && kBT) {  // the partial last k tile of a k-contiguous rhs, without a branch (see issue_a_pair)
                 constexpr unsigned kBehind = 0x7fffffffu;
+                static_assert(kWaves * kARowsPerInstr % 16 == 0, "the swizzle of a row repeats every 16 rows");
+                const int chunks = kt == last_k ? tail_chunks : kAChunksPerRow;
+                const bool inside = a_phys_chunk16<BK>(wave * kARowsPerInstr + lane / kAChunksPerRow, lane % kAChunksPerRow) < chunks;
 #pragma unroll
-                for (int j = 0; j < kBInstr; ++j) {
-                    const int row = (j * kWaves + wave) * kARowsPerInstr + lane / kAChunksPerRow;
-                    const bool inside = a_phys_chunk16<BK>(row, lane % kAChunksPerRow) < tail_chunks;
+                for (int j = 0; j < kBInstr; ++j)
                     __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, sb + (j * kWaves + wave) * 1024, 16, inside ? b_src[j] : kBehind, b_k, 0, kAux);
-                }
                 return;
             }
 #pragma unroll
