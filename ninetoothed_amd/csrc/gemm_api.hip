@@ -145,7 +145,7 @@ int split_parts(const GemmProblem &q, int bm, int bn, int bk, int *kt_per_part, 
     int64_t parts = bm * bn >= 256 * 256 ? 256 / tiles : (512 + tiles - 1) / tiles;
     parts = std::min<int64_t>(parts, num_kt / 2);                  // at least two k tiles each
     parts = std::min<int64_t>(parts, 256);
-    while (parts >= 2 && parts * q.m * q.n * 4 > scratch_limit) --parts;  // scratch of at most 64 MiB, or what the caller's fixed array holds
+    while (parts >= 2 && parts * q.m * ((q.n + 7) / 8 * 8) * 4 > scratch_limit) --parts;  // scratch of at most 64 MiB, or what the caller's fixed array holds
     if (parts < 2) return 1;
     const int per_part = (int)((num_kt + parts - 1) / parts);
     if (kt_per_part) *kt_per_part = per_part;
@@ -154,33 +154,37 @@ int split_parts(const GemmProblem &q, int bm, int bn, int bk, int *kt_per_part, 
 
 template <int BM, int BN, int BK, int kStages>
 bool split_accepts(const GemmProblem &q) {
-    // the operands, outputs and epilogues of the one-pass instances with tails (the second kernel writes
-    // four consecutive elements of C at a time, which their alignment rules cover)
-    if (q.n % 8 || q.scm % 8 || ((uintptr_t)q.c & 15) || q.batch != 1) return false;
+    // the operands, outputs and epilogues of the one-pass instances with tails (the second kernel writes four
+    // consecutive elements of C at a time where N, the row pitch and the address of C allow it, else one)
+    if (q.batch != 1) return false;
     return fast_accepts<BM, BN, BK, kStages, true>(q) && split_parts(q, BM, BN, BK, nullptr) >= 2;
 }
 
-// out[m][n] = epilogue(sum over parts): four consecutive columns per thread (N is a multiple of 8)
-template <typename T, typename TOut, bool kAddmm>
+// out[m][n] = epilogue(sum over parts): four consecutive columns per thread.  The parts are [m][pitch] tiles, pitch = N
+// rounded up to 8; kVector: N is a multiple of 4 and the rows of C start on 16-byte (fp32) / 8-byte boundaries -- else
+// the four values are stored one by one, those inside N
+template <typename T, typename TOut, bool kAddmm, bool kVector = true>
 __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float *parts, int num_parts, int m, int n, TOut *c, int64_t ldc, const T *bias,
                                                                int64_t bias_stride_m, int64_t bias_stride_n, float alpha, float beta) {
     typedef float float4_t __attribute__((ext_vector_type(4)));
     typedef TOut out4_t __attribute__((ext_vector_type(4)));
-    const int groups = n / 4;
+    const int pitch = (n + 7) / 8 * 8;
+    const int groups = pitch / 4;
     const int64_t total = (int64_t)m * groups;
     for (int64_t index = (int64_t)blockIdx.x * 256 + threadIdx.x; index < total; index += (int64_t)gridDim.x * 256) {
         const int row = (int)(index / groups);
         const int col = (int)(index - (int64_t)row * groups) * 4;
-        const float *src = parts + (int64_t)row * n + col;
+        if (col >= n) continue;
+        const float *src = parts + (int64_t)row * pitch + col;
         float4_t sum = *(const float4_t *)src;
-        for (int part = 1; part < num_parts; ++part) sum += *(const float4_t *)(src + (int64_t)part * m * n);
+        for (int part = 1; part < num_parts; ++part) sum += *(const float4_t *)(src + (int64_t)part * m * pitch);
         out4_t out;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             if constexpr (kAddmm) {
                 // as in the one-pass kernels: the product is rounded to the element type, then combined in fp32
                 const float product = Elem<T>::to_float(Elem<T>::from_float(sum[e]));
-                const float input = Elem<T>::to_float(bias[(int64_t)row * bias_stride_m + (int64_t)(col + e) * bias_stride_n]);
+                const float input = kVector || col + e < n ? Elem<T>::to_float(bias[(int64_t)row * bias_stride_m + (int64_t)(col + e) * bias_stride_n]) : 0.0f;
                 out[e] = Elem<T>::from_float(beta * input + alpha * product);
             } else if constexpr (std::is_same<TOut, float>::value) {
                 out[e] = sum[e];
@@ -188,7 +192,13 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float *par
                 out[e] = Elem<T>::from_float(sum[e]);
             }
         }
-        __builtin_nontemporal_store(out, (out4_t *)(c + (int64_t)row * ldc + col));
+        if constexpr (kVector) {
+            __builtin_nontemporal_store(out, (out4_t *)(c + (int64_t)row * ldc + col));
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (col + e < n) c[(int64_t)row * ldc + col + e] = out[e];
+        }
     }
 }
 
@@ -198,7 +208,8 @@ hipError_t split_launch_typed(const GemmProblem &q, hipStream_t stream) {
     // with a fixed array the part count shrinks until the partial products fit; the call is refused when not even two parts do
     const int parts = q.fixed_scratch != nullptr ? split_parts(q, BM, BN, BK, &kt_per_part, (int64_t)q.fixed_scratch_bytes) : split_parts(q, BM, BN, BK, &kt_per_part);
     if (parts < 2) return (hipError_t)(q.fixed_scratch != nullptr && split_parts(q, BM, BN, BK, nullptr) >= 2 ? NINETOOTHED_SCRATCH_LIMIT : NINETOOTHED_NO_KERNEL);
-    const size_t scratch_bytes = (size_t)parts * q.m * q.n * sizeof(float);
+    const int pitch = (q.n + 7) / 8 * 8;  // of the partial tiles: whole 16-byte chunks, whatever N is
+    const size_t scratch_bytes = (size_t)parts * q.m * pitch * sizeof(float);
     // the lock of the workspace registry also serialises host threads that enqueue onto the fixed array
     WorkspaceLease lease(stream);
     float *scratch;
@@ -212,8 +223,8 @@ hipError_t split_launch_typed(const GemmProblem &q, hipStream_t stream) {
     GemmParams p;
     fill_params(p, q, BM, BN);
     p.c = scratch;
-    p.ldc = q.n;
-    p.c_vector = 1;  // (N is a multiple of 8 here and the scratch tensor is aligned)
+    p.ldc = pitch;
+    p.c_vector = 1;  // (the scratch tensor is aligned and its rows hold whole chunks: a chunk that begins inside N is stored whole)
     p.bias = nullptr;
     p.kt_per_split = kt_per_part;
     const dim3 grid(p.tiles_m * p.tiles_n * parts), block(WM * WN * 64);
@@ -221,14 +232,21 @@ hipError_t split_launch_typed(const GemmProblem &q, hipStream_t stream) {
     else gemm_nn_fast_kernel<T, BM, BN, BK, WM, WN, kStages, kOcc, false, 0, 1, 0, true, false, true, true><<<grid, block, 0, stream>>>(p);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return err;
-    const int64_t groups = (int64_t)q.m * (q.n / 4);
+    const int64_t groups = (int64_t)q.m * (pitch / 4);
     const dim3 reduce_grid((unsigned)std::min<int64_t>((groups + 255) / 256, 256 * 8));
-    if (q.addmm())
-        gemm_split_reduce_kernel<T, T, true><<<reduce_grid, dim3(256), 0, stream>>>(scratch, parts, q.m, q.n, (T *)q.c, q.scm, (const T *)q.bias, q.sim, q.sin, q.alpha, q.beta);
-    else if (q.out_dtype == NINETOOTHED_FLOAT32)
-        gemm_split_reduce_kernel<T, float, false><<<reduce_grid, dim3(256), 0, stream>>>(scratch, parts, q.m, q.n, (float *)q.c, q.scm, nullptr, 0, 0, 1.0f, 0.0f);
-    else
-        gemm_split_reduce_kernel<T, T, false><<<reduce_grid, dim3(256), 0, stream>>>(scratch, parts, q.m, q.n, (T *)q.c, q.scm, nullptr, 0, 0, 1.0f, 0.0f);
+    const int64_t out_size = q.out_dtype == NINETOOTHED_FLOAT32 ? 4 : 2;
+    const bool vector = q.n % 4 == 0 && (q.scm * out_size) % (4 * out_size) == 0 && ((uintptr_t)q.c & (4 * out_size - 1)) == 0;
+    const auto reduce = [&](auto vector_tag) {
+        constexpr bool kVector = decltype(vector_tag)::value;
+        if (q.addmm())
+            gemm_split_reduce_kernel<T, T, true, kVector><<<reduce_grid, dim3(256), 0, stream>>>(scratch, parts, q.m, q.n, (T *)q.c, q.scm, (const T *)q.bias, q.sim, q.sin, q.alpha, q.beta);
+        else if (q.out_dtype == NINETOOTHED_FLOAT32)
+            gemm_split_reduce_kernel<T, float, false, kVector><<<reduce_grid, dim3(256), 0, stream>>>(scratch, parts, q.m, q.n, (float *)q.c, q.scm, nullptr, 0, 0, 1.0f, 0.0f);
+        else
+            gemm_split_reduce_kernel<T, T, false, kVector><<<reduce_grid, dim3(256), 0, stream>>>(scratch, parts, q.m, q.n, (T *)q.c, q.scm, nullptr, 0, 0, 1.0f, 0.0f);
+    };
+    if (vector) reduce(std::true_type());
+    else reduce(std::false_type());
     return hipGetLastError();
 }
 

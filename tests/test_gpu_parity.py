@@ -1880,12 +1880,15 @@ def test_gemm_transposed_rhs_any_number_of_columns(m, n, k, dtype):
 
 
 @pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
-@pytest.mark.parametrize("m, n, k", ((1, 2048, 4096), (16, 1024, 8192), (64, 520, 2056), (300, 200, 4104), (512, 512, 16384), (129, 136, 256), (768, 1032, 4096)))
+@pytest.mark.parametrize("m, n, k", ((1, 2048, 4096), (16, 1024, 8192), (64, 520, 2056), (300, 200, 4104), (512, 512, 16384), (129, 136, 256), (768, 1032, 4096),
+                                     (33, 515, 8192), (16, 1001, 4096), (100, 301, 5000), (7, 50, 2048)))
 def test_gemm_split_k(m, n, k, dtype):
     """Few output tiles, long K: the k range is cut into parts that run as workgroups of their own
     and a second kernel sums them (fp32) and applies the epilogue.  Both rhs layouts, element-type /
     fp32 / addmm outputs, NaN-poisoned output with sentinel columns beside it; twice in a row
-    (the scratch tensor of the stream is reused)."""
+    (the scratch tensor of the stream is reused).  An N that is no multiple of 8 goes with a k-contiguous
+    rhs (as in the one-pass instances): the partial tiles then have rows of N rounded up to 8 and the
+    second kernel stores element by element."""
     from ninetoothed_amd import runtime
 
     lib = runtime.library()
@@ -1923,7 +1926,7 @@ def test_gemm_split_k(m, n, k, dtype):
                     assert bool((buffer[:, n:] == 7.0).all()), name
                 else:
                     served += 1
-            assert served >= 1
+            assert served >= 1 or (n % 8 != 0 and b.stride(1) == 1)
         out = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
         _matmul_kernel()(a, b, out)
         assert torch.allclose(out.float(), product, **HALF_TOL)
