@@ -123,7 +123,9 @@ __global__ __launch_bounds__(256) void conv2d_repack_kernel(const T *x, T *xt, i
         const int hw = hw0 + (t & 7) * 8;
         vec8 v;
         if (vector_ok && c0 + c < C && hw + 8 <= HW) {
-            v = *(const vec8 *)(src + (int64_t)(c0 + c) * s_c + hw);
+            // (the positions of a channel are contiguous; where they start does not matter: global accesses need the element's alignment only)
+            typedef vec8 unaligned_vec8 __attribute__((aligned(2)));
+            v = *(const unaligned_vec8 *)(src + (int64_t)(c0 + c) * s_c + hw);
         } else {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
@@ -1047,7 +1049,7 @@ int run_fast(const Conv2dRequest &q, hipStream_t stream) {
     void *wt = lease.get(kWorkspaceConvFilter, (size_t)wt_bytes);
     if (xt == nullptr || wt == nullptr) return NINETOOTHED_NO_KERNEL;  // no scratch: the caller falls back to the gather kernel
     const bool aligned = ((uintptr_t)q.x & 15) == 0;
-    int vector_ok = q.xs[3] == 1 && q.xs[2] == q.W && HW % 8 == 0 && q.xs[1] % 8 == 0 && q.xs[0] % 8 == 0 && aligned;
+    int vector_ok = q.xs[3] == 1 && q.xs[2] == q.W;  // 16-byte loads along the positions of a channel
     if (q.xs[1] == 1 && q.C > 1) vector_ok = q.C % 8 == 0 && q.xs[3] % 8 == 0 && q.xs[2] % 8 == 0 && q.xs[0] % 8 == 0 && aligned ? 3 : 2;
     FilterRepack f;
     f.w = q.w;

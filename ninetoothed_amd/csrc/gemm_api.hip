@@ -782,7 +782,7 @@ GemmProblem transposed_problem(const GemmProblem &q) {
 // a fraction of a round.  NINETOOTHED_NO_KERNEL when the shape is not of that kind or scratch memory is not to be had.
 int run_gemm_last_rows_in_parts(hipStream_t stream, const GemmProblem &q) {
     if ((q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) || q.batch != 1 || q.fixed_scratch != nullptr) return NINETOOTHED_NO_KERNEL;
-    static const bool enabled = getenv("NT_GEMM_NO_ROW_SPLIT") == nullptr;
+    static const bool enabled = getenv("NT_GEMM_NO_ROW_SPLIT") == nullptr;  // (set for A/B measurements: every product in one pass)
     if (!enabled) return NINETOOTHED_NO_KERNEL;
     const int64_t tiles_m = ceil_div(q.m, 256), tiles_n = ceil_div(q.n, 256), tiles = tiles_m * tiles_n;
     // (measured, one pass -> this way: 4352 x 4096 x 4352 160 -> 143 us, 4096 x 4096 x 4352 158 -> 135, 5120 x 4096 x 3584

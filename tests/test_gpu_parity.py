@@ -1051,7 +1051,11 @@ def test_conv2d_channels_last_and_sliced_tensors_on_the_repacked_path(channels, 
         assert x_last.stride(1) == 1
         wide = torch.full((n, k + 3, p + 2, q + 5), 7.0, dtype=dtype, device="cuda")
         window = wide[:, 2 : 2 + k, 1 : 1 + p, 3 : 3 + q]
+        planes = torch.full((n, channels, h * w + 3), float("inf"), dtype=dtype, device="cuda")
+        x_odd = planes[:, :, 1 : 1 + h * w].view(n, channels, h, w)  # NCHW whose channel planes start at odd elements
+        x_odd.copy_(x)
         outputs = (
+            (x_odd, weight, torch.full(expected.shape, float("nan"), dtype=dtype, device="cuda")),
             (x_last, weight.to(memory_format=torch.channels_last), torch.full(expected.shape, float("nan"), dtype=dtype, device="cuda").to(memory_format=torch.channels_last)),
             (x_last, weight, torch.full(expected.shape, float("nan"), dtype=dtype, device="cuda")),
             (x, weight, window),
