@@ -769,6 +769,7 @@ struct MapCodegen {
             out << indent << "const double " << name << " = " << expr << ";\n";
             return name;
         };
+        std::map<std::string, std::string> integer_of;  // temporaries that are an index converted to fp64
         for (int pc = begin; pc < end; ++pc) {
             const int op = p.value_code[pc] & 0xff, arg = p.value_code[pc] >> 8;
             if (op == NT_MAP_V_LOAD && keep_loads && kept[arg]) {
@@ -791,7 +792,9 @@ struct MapCodegen {
             } else if (op == NT_MAP_V_OFFSET) {
                 const std::string valid = fresh("ok");
                 out << indent << "bool " << valid << " = true;\n";
-                stack.push_back(define("(double)" + index_segment(arg, valid)));
+                const std::string index = index_segment(arg, valid);
+                stack.push_back(define("(double)" + index));
+                integer_of[stack.back()] = index;
             } else if (op >= NT_MAP_V_ADD && op <= NT_MAP_V_OR) {
                 const std::string b = stack.back();
                 stack.pop_back();
@@ -850,7 +853,9 @@ struct MapCodegen {
             } else if (op == NT_MAP_V_RAND) {
                 const std::string offset = stack.back();
                 stack.pop_back();
-                stack.back() = define("nt_philox_uniform((unsigned long long)(long long)" + stack.back() + ", (unsigned long long)(long long)" + offset + ")");
+                // (an offset that is an index as it stands skips the detour through fp64)
+                const std::string counter = integer_of.count(offset) ? integer_of[offset] : offset;
+                stack.back() = define("nt_philox_uniform((unsigned long long)(long long)" + stack.back() + ", (unsigned long long)(long long)" + counter + ")");
             } else if (op == NT_MAP_V_SETVAR) {
                 out << indent << "v" << arg << " = (nt_idx)(" << stack.back() << ");\n";
                 stack.pop_back();
@@ -968,8 +973,8 @@ struct MapCodegen {
             << "    unsigned int c0 = (unsigned int)offset, c1 = (unsigned int)(offset >> 32), c2 = 0, c3 = 0;\n"
             << "    unsigned int k0 = (unsigned int)seed, k1 = (unsigned int)(seed >> 32);\n"
             << "    for (int round = 0; round < 10; ++round) {\n"
-            << "        const unsigned int ra = 0xD2511F53u, rb = 0xCD9E8D57u, p0 = c0, p2 = c2;\n"
-            << "        c0 = __umulhi(rb, p2) ^ c1 ^ k0; c2 = __umulhi(ra, p0) ^ c3 ^ k1; c1 = rb * p2; c3 = ra * p0;\n"
+            << "        const unsigned long long a0 = 0xD2511F53ull * c0, b2 = 0xCD9E8D57ull * c2;  // (one 32 x 32 -> 64 bit multiplication each)\n"
+            << "        c0 = (unsigned int)(b2 >> 32) ^ c1 ^ k0; c2 = (unsigned int)(a0 >> 32) ^ c3 ^ k1; c1 = (unsigned int)b2; c3 = (unsigned int)a0;\n"
             << "        k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;\n"
             << "    }\n"
             << "    int x = (int)c0; if (x < 0) x = -x - 1;\n"
