@@ -301,8 +301,9 @@ def test_mfma_rate_probe_runs_and_counts():
 
 @pytest.mark.skipif(not hasattr(torch, "float8_e5m2"), reason="this torch has no float8_e5m2")
 def test_calls_that_share_scratch_buffers_from_several_host_threads():
-    """Split-K partial products, the fp16 copies of fp8 operands, dense copies of misaligned operands, padded copies
-    of attention tensors and conv2d's repacked operands all live in one buffer per (device, stream, purpose).  Four
+    """Split-K partial products (of the fp16 and the fp32 kernels), the fp16 copies of fp8 operands, dense copies of
+    misaligned operands, padded copies of attention tensors, conv2d's repacked operands and the per-part maxima and sums
+    of a softmax over a few long rows all live in one buffer per (device, stream, purpose).  Four
     host threads enqueue such calls onto the SAME stream with sizes of their own: the registry lock must keep a
     call's copies and the kernel that reads them together (a buffer overwritten in between shows as wrong values),
     also when a buffer has to grow in the middle."""
@@ -312,6 +313,7 @@ def test_calls_that_share_scratch_buffers_from_several_host_threads():
     matmul = ninetoothed.make(programs.matmul.arrangement, programs.matmul.application, programs.matmul.tensors())
     attention = ninetoothed.make(programs.attention.arrangement_with_scale, programs.attention.application_with_scale, programs.attention.tensors(with_scale=True))
     conv = ninetoothed.make(programs.conv2d.arrangement, programs.conv2d.application, programs.conv2d.tensors())
+    softmax = ninetoothed.make(programs.softmax.arrangement, programs.softmax.application, programs.softmax.tensors())
     failures = []
 
     def worker(seed):
@@ -328,12 +330,16 @@ def test_calls_that_share_scratch_buffers_from_several_host_threads():
                 a_off, b16 = randn(2048 + 8 * seed, 1025)[:, :1024], randn(1024, 1024)  # rows off 16-byte boundaries, 2^31 multiply-adds
                 q, k, v = (randn(1, 2 + seed, 96, 20 + 4 * seed) for _ in range(3))
                 x, w = randn(2, 3 + seed, 20, 24, scale=0.3), randn(16, 3 + seed, 3, 3, scale=0.3)
+                a32, b32 = randn(100 + seed, 2048 + 64 * seed, dtype=torch.float32), randn(2048 + 64 * seed, 130, dtype=torch.float32)  # one tile row of the fp32 kernel: k range in parts
+                rows = randn(2 + seed, 100000 + 4096 * seed, dtype=torch.float32)  # a few long rows: parts of a row on workgroups of their own
                 expected = (
                     skinny_a.float() @ skinny_b.float(),
                     a8.to(torch.float16).float() @ b8.to(torch.float16).float(),
                     a_off.float() @ b16.float(),
                     torch.softmax((q.float() * q.shape[-1] ** -0.5) @ k.float().transpose(-1, -2), dim=-1) @ v.float(),
                     F.conv2d(x.float(), w.float(), padding=1),
+                    (a32.double() @ b32.double()).float(),
+                    torch.softmax(rows, dim=-1),
                 )
                 for _ in range(6):
                     outs = (
@@ -342,13 +348,18 @@ def test_calls_that_share_scratch_buffers_from_several_host_threads():
                         torch.full((a_off.shape[0], 1024), float("nan"), dtype=torch.float16, device="cuda"),
                         torch.full_like(q, float("nan")),
                         torch.full((2, 16, 20, 24), float("nan"), dtype=torch.float16, device="cuda"),
+                        torch.full((a32.shape[0], 130), float("nan"), dtype=torch.float32, device="cuda"),
+                        torch.full_like(rows, float("nan")),
                     )
                     matmul(skinny_a, skinny_b, outs[0])
                     matmul(a8, b8, outs[1])
                     matmul(a_off, b16, outs[2])
                     attention(q, k, v, False, q.shape[-1] ** -0.5, outs[3])
                     conv(x, w, outs[4], padding_h=1, padding_w=1)
-                    tolerances = (dict(rtol=1e-2, atol=1e-2 * (skinny_a.shape[1] / 512) ** 0.5), dict(rtol=1e-2, atol=1e-2), dict(rtol=1e-2, atol=1e-2 * 2**0.5), HALF_TOL, HALF_TOL)
+                    matmul(a32, b32, outs[5])
+                    softmax(rows, outs[6], BLOCK_SIZE=1 << 17)
+                    tolerances = (dict(rtol=1e-2, atol=1e-2 * (skinny_a.shape[1] / 512) ** 0.5), dict(rtol=1e-2, atol=1e-2), dict(rtol=1e-2, atol=1e-2 * 2**0.5), HALF_TOL, HALF_TOL,
+                                  dict(rtol=1e-4, atol=2e-4), dict(rtol=1e-5, atol=1e-8))
                     for index, (out, reference, tolerance) in enumerate(zip(outs, expected, tolerances)):
                         if not torch.allclose(out.float(), reference, **tolerance):
                             failures.append((seed, index, float((out.float() - reference).abs().max())))
