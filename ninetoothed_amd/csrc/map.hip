@@ -961,6 +961,156 @@ struct MapCodegen {
         return out.str();
     }
 
+    // ---- element-wise maps, several consecutive elements per thread ----
+    //
+    // How an index segment depends on the last output variable when that variable moves through an aligned group of
+    // `width` values: 0 = not at all (the group shares one element), 1 = it advances by one element per value and the
+    // segment's checks hold for the whole group or for none of it, -1 = anything else.  Abstract interpretation of
+    // the index program: a value is invariant, or `rest + k * last` with `rest` known to be a multiple of `width` or
+    // not; a division or remainder of such a sum by a multiple of `width` keeps the group together.
+    int group_step(int segment, int last, long long width) const {
+        struct Shape {
+            bool moves;
+            long long k;
+            bool multiple;  // the value at last = 0 is a multiple of `width`
+        };
+        std::vector<Shape> stack;
+        for (int pc = p.segment_begin[segment];; ++pc) {
+            const int op = p.index_code[pc] & 0xff, arg = p.index_code[pc] >> 8;
+            if (op == NT_MAP_I_END) break;
+            const long long c = op == NT_MAP_I_VAR || op == NT_MAP_I_ADD ? 0 : (long long)p.index_constants[arg];
+            switch (op) {
+                case NT_MAP_I_CONST: stack.push_back({false, 0, c % width == 0}); break;
+                case NT_MAP_I_VAR: stack.push_back(arg == last ? Shape{true, 1, true} : Shape{false, 0, false}); break;
+                case NT_MAP_I_MULC:
+                    stack.back().k *= c;
+                    stack.back().multiple = stack.back().multiple || c % width == 0;
+                    if (stack.back().moves && stack.back().k == 0) stack.back().moves = false;
+                    break;
+                case NT_MAP_I_ADD: {
+                    const Shape b = stack.back();
+                    stack.pop_back();
+                    Shape &a = stack.back();
+                    a = {a.moves || b.moves, a.k + b.k, a.multiple && b.multiple};
+                    if (a.moves && a.k == 0) return -1;  // (cancelling terms: not worth following)
+                    break;
+                }
+                case NT_MAP_I_DIVC:
+                case NT_MAP_I_MODC: {
+                    Shape &a = stack.back();
+                    if (c <= 0) return -1;
+                    if (!a.moves) {
+                        a = {false, 0, false};
+                    } else {
+                        if (a.k != 1 || !a.multiple || c % width != 0) return -1;
+                        a = op == NT_MAP_I_DIVC ? Shape{false, 0, false} : Shape{true, 1, true};
+                    }
+                    break;
+                }
+                case NT_MAP_I_CHECK: {
+                    const Shape a = stack.back();
+                    stack.pop_back();
+                    if (a.moves && (a.k != 1 || !a.multiple || c % width != 0)) return -1;
+                    break;
+                }
+                default: return -1;
+            }
+        }
+        if (stack.empty() || !stack.back().moves) return 0;
+        return stack.back().k == 1 ? 1 : -1;
+    }
+
+    // Elements per thread for a plain element-wise map (no reduction, no data-dependent index) over 16- and 32-bit
+    // floating-point tensors whose output and operands are contiguous along the last variable (or do not depend on
+    // it): 8 when a 16-bit tensor takes part (16 bytes of it per access).  0: one element per thread.
+    int vector_width() const {
+        if (p.num_phases > 0 || p.reduce_op != NT_MAP_REDUCE_NONE || p.num_reduced != 0 || p.num_dynamic != 0 || lanes != 1) return 0;
+        if (p.store_op == NT_MAP_STORE_ATOMIC_ADD || p.num_vars < 1) return 0;
+        std::vector<int> used(1, p.output);
+        bool random = false;
+        for (int pc = 0; pc < p.value_code_length; ++pc) {
+            const int op = p.value_code[pc] & 0xff;
+            if (op == NT_MAP_V_LOAD) used.push_back(p.value_code[pc] >> 8);
+            if (op == NT_MAP_V_RAND) random = true;
+            if (op == NT_MAP_V_SETVAR || op == NT_MAP_V_REDUCED) return 0;
+        }
+        // (measured on 2^26 elements, one per thread -> groups: fp16 copy 50 -> 39 us, fp16 add 59.5 -> 58; fp32 add
+        // 137 -> 151 with groups of 4 and 160 with groups of 2, so maps over fp32 tensors alone keep one element per
+        // thread -- unless they draw random numbers, whose rounds then run four chains deep: dropout 196 -> 160)
+        int width = random ? 4 : 0;
+        for (int slot : used) {
+            if (!kept_as_float(slot)) return 0;
+            if (p.operands[slot].dtype != NINETOOTHED_FLOAT32) width = 8;
+        }
+        if (width == 0) return 0;
+        const int last = p.num_vars - 1;
+        if (p.extents[last] <= 0 || p.extents[last] % width != 0) return 0;
+        if (group_step(p.operands[p.output].segment, last, width) != 1) return 0;
+        for (int slot : used)
+            if (group_step(p.operands[slot].segment, last, width) < 0) return 0;
+        return width;
+    }
+
+    std::string generate_vector(int width) {
+        const int last = p.num_vars - 1;
+        const auto vector_type = [&](int dtype) {  // (global accesses need the element's alignment only)
+            return std::string("nt_vec_") + (dtype == NINETOOTHED_FLOAT32 ? "f32" : dtype == NINETOOTHED_FLOAT16 ? "f16" : "bf16");
+        };
+        out << "    typedef float nt_vec_f32 __attribute__((ext_vector_type(" << width << "), aligned(4)));\n"
+            << "    typedef _Float16 nt_vec_f16 __attribute__((ext_vector_type(" << width << "), aligned(2)));\n"
+            << "    typedef __bf16 nt_vec_bf16 __attribute__((ext_vector_type(" << width << "), aligned(2)));\n"
+            << "    const nt_idx groups = total_out / " << width << ";\n"
+            << "    for (nt_idx group = (nt_idx)blockIdx.x * " << kMapThreads << " + threadIdx.x; group < groups; group += stride) {\n"
+            << "        nt_uidx rest = (nt_uidx)group * " << width << "u;\n";
+        for (int v = last; v >= 0; --v)
+            out << "        const nt_idx v" << v << " = (nt_idx)(rest % " << ulit((long long)p.extents[v]) << "); rest /= " << ulit((long long)p.extents[v]) << ";\n";
+        // the operands' values of the group, as floats
+        std::fill(kept.begin(), kept.end(), false);
+        for (int pc = 0; pc < p.value_code_length; ++pc) {
+            if ((p.value_code[pc] & 0xff) != NT_MAP_V_LOAD) continue;
+            const int slot = p.value_code[pc] >> 8;
+            if (kept[slot]) continue;
+            kept[slot] = true;
+            const NineToothedMapOperand &operand = p.operands[slot];
+            const std::string valid = fresh("ok");
+            out << indent << "float ld" << slot << "[" << width << "];\n" << indent << "bool " << valid << " = true;\n";
+            const std::string offset = index_segment(operand.segment, valid);
+            const std::string pointer = std::string("((const ") + c_type(operand.dtype) + " *)a.data[" + std::to_string(slot) + "] + " + offset + ")";
+            if (group_step(operand.segment, last, width) == 1) {
+                out << indent << "if (" << valid << ") {\n"
+                    << indent << "    const " << vector_type(operand.dtype) << " loaded = *(const " << vector_type(operand.dtype) << " *)" << pointer << ";\n"
+                    << indent << "    for (int e = 0; e < " << width << "; ++e) ld" << slot << "[e] = (float)loaded[e];\n"
+                    << indent << "} else {\n"
+                    << indent << "    for (int e = 0; e < " << width << "; ++e) ld" << slot << "[e] = (float)a.other[" << slot << "];\n"
+                    << indent << "}\n";
+            } else {
+                out << indent << "{\n"
+                    << indent << "    const float shared = " << valid << " ? (float)*" << pointer << " : (float)a.other[" << slot << "];\n"
+                    << indent << "    for (int e = 0; e < " << width << "; ++e) ld" << slot << "[e] = shared;\n"
+                    << indent << "}\n";
+            }
+        }
+        const NineToothedMapOperand &target = p.operands[p.output];
+        out << indent << "bool store_ok = true;\n";
+        const std::string target_offset = index_segment(target.segment, "store_ok");
+        out << indent << "const nt_idx nt_first = v" << last << ";\n"
+            << indent << vector_type(target.dtype) << " result;\n"
+            << indent << "#pragma unroll\n"
+            << indent << "for (int e = 0; e < " << width << "; ++e) {\n";
+        indent += "    ";
+        out << indent << "const nt_idx v" << last << " = nt_first + e;\n";
+        keep_loads = true;
+        const std::string value = value_range(0, p.value_code_length, "");
+        keep_loads = false;
+        out << indent << "result[e] = (" << c_type(target.dtype) << ")(float)(" << value << ");\n";
+        indent.resize(indent.size() - 4);
+        out << indent << "}\n"
+            << indent << "if (store_ok) __builtin_nontemporal_store(result, (" << vector_type(target.dtype) << " *)((" << c_type(target.dtype) << " *)a.data[" << p.output << "] + "
+            << target_offset << "));\n"
+            << "    }\n}\n";
+        return out.str();
+    }
+
     std::string generate() {
         const int num_out = p.num_vars - p.num_reduced;
         out << "struct MapJitArgs { void *data[" << NT_MAP_MAX_OPERANDS << "]; double other[" << NT_MAP_MAX_OPERANDS << "]; double constants["
@@ -984,6 +1134,7 @@ struct MapCodegen {
             << "    const nt_idx stride = (nt_idx)gridDim.x * " << kMapThreads << ";\n"
             << "    const nt_idx total_out = (nt_idx)a.total_out;\n";
         if (p.num_phases > 0) return generate_tile();
+        if (const int width = vector_width()) return generate_vector(width);
         if (lanes > 64) out << "    __shared__ double nt_partial[" << lanes / 64 << "];\n";
         if (lanes > 1)
             out << "    const nt_idx lane = threadIdx.x & " << lanes - 1 << ";\n"

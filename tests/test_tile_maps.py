@@ -1033,3 +1033,73 @@ def test_reductions_over_the_contiguous_dimension_share_a_wave(shape, dtype):
     kernel = ninetoothed.make(plane_arrangement, row_sum_application, (Tensor(3), Tensor(1)))
     kernel(planes, plane_out)
     assert torch.allclose(plane_out.float(), planes.float().sum(dim=(1, 2)) * 2, rtol=1e-2 if dtype == torch.float16 else 1e-4, atol=1.0 if dtype == torch.float16 else 1e-2)
+
+
+# ---- element-wise maps over 16-bit tensors: groups of eight consecutive elements per thread ---------
+
+
+def _generated_source(kernel, args, kwargs=None):
+    """HIP source that launch_nt_map would compile for the kernel's (single) store with these arguments."""
+    import ctypes
+
+    from ninetoothed_amd import mapping, runtime
+    from ninetoothed_amd.make import _dtype_tag
+
+    env = kernel._environment(args, kwargs or {}, check_device=False)
+    (store,) = kernel.program.stores
+    program, _, _, _ = mapping.build(store, kernel.types, args, env, lambda p: _dtype_tag(_storage(args, p).dtype), lambda p: 0)
+    buffer = ctypes.create_string_buffer(1 << 16)
+    assert runtime.library().nt_map_source(ctypes.addressof(program), buffer, len(buffer)) == 0
+    return buffer.value.decode()
+
+
+def test_generated_source_groups_elements_of_16_bit_tensors():
+    """Plain element-wise maps whose tensors are contiguous along the last variable read and write 16 bytes of a
+    16-bit tensor per access; fp32 tensors alone stay at one element per thread (measured: faster), and so does
+    anything whose last extent, padding or strides do not keep a group of eight together."""
+    half = lambda *shape: torch.empty(*shape, dtype=torch.float16)  # noqa: E731
+    grouped = _generated_source(add_kernel, (half(4096), half(4096), half(4096)), {"BLOCK_SIZE": 1024})
+    assert "nt_vec_f16" in grouped and "groups" in grouped
+    mixed = _generated_source(add_kernel, (half(4096), torch.empty(4096), torch.empty(4096)), {"BLOCK_SIZE": 1024})
+    assert "const nt_vec_f16 loaded" in mixed and "const nt_vec_f32 loaded" in mixed
+    assert "nt_vec" not in _generated_source(add_kernel, (torch.empty(4096), torch.empty(4096), torch.empty(4096)), {"BLOCK_SIZE": 1024})
+    # (a tile of 12 elements: the last variable's extent is no multiple of 8)
+    assert "nt_vec" not in _generated_source(add_kernel, (half(4096), half(4096), half(4096)), {"BLOCK_SIZE": 12})
+    # every other element of a wider tensor: the operand does not advance by one element
+    assert "nt_vec" not in _generated_source(add_kernel, (half(8192)[::2], half(4096), half(4096)), {"BLOCK_SIZE": 1024})
+    # a broadcast operand (one value per row) shares its element within a group
+    kernel = ninetoothed.make(_bias_arrangement, _bias_application, (Tensor(2), Tensor(1), Tensor(1), Tensor(2)))
+    source = _generated_source(kernel, (half(64, 128), half(128), half(64), half(64, 128)), {name: 32 for name in kernel.meta_symbols})
+    assert "nt_vec_f16" in source and "const float shared" in source
+    # dropout draws random numbers: groups of four even for fp32 tensors
+    dropout = ninetoothed.make(dropout_arrangement, dropout_application, (Tensor(1), Tensor(0), Tensor(0), Tensor(1)))
+    assert "nt_vec_f32" in _generated_source(dropout, (torch.empty(4096), 0.3, 7, torch.empty(4096)))
+
+
+@gpu
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
+def test_grouped_elements_of_16_bit_tensors(dtype):
+    """Results of the grouped kernels against torch: tensors at odd element offsets of sentinel-filled buffers (the
+    16-byte accesses are unaligned), a row pitch of its own, a broadcast row and column, an fp32 output, padding."""
+    n = 1 << 16
+    storage = torch.full((3, n + 9), float("inf"), dtype=dtype, device="cuda")
+    lhs, rhs = storage[0, 3 : 3 + n], storage[1, 5 : 5 + n]
+    lhs.copy_(torch.randn(n, device="cuda").to(dtype))
+    rhs.copy_(torch.randn(n, device="cuda").to(dtype))
+    buffer = torch.full((n + 9,), 7.0, dtype=dtype, device="cuda")
+    out = buffer[1 : 1 + n]
+    add_kernel(lhs, rhs, out, BLOCK_SIZE=1024)
+    _served_by_map(add_kernel)
+    assert torch.equal(out, lhs + rhs)
+    assert float(buffer[0]) == 7.0 and bool((buffer[1 + n :] == 7.0).all())
+    wide = torch.empty(n, dtype=torch.float32, device="cuda")
+    add_kernel(lhs, rhs, wide, BLOCK_SIZE=1024)
+    assert torch.equal(wide, (lhs + rhs).float())  # (the sum is the tiles' type, widened when it is stored)
+    kernel = ninetoothed.make(_bias_arrangement, _bias_application, (Tensor(2), Tensor(1), Tensor(1), Tensor(2)))
+    x = torch.randn(641, 280 + 8, device="cuda").to(dtype)[:, :280]
+    r, c = torch.randn(280, device="cuda").to(dtype), torch.randn(641, device="cuda").to(dtype)
+    result = torch.full((641, 280), float("nan"), dtype=dtype, device="cuda")
+    kernel(x, r, c, result)
+    _served_by_map(kernel)
+    # (every operation rounds to the tensors' type, as torch's do)
+    assert torch.equal(result, x + r[None, :] + c[:, None] * 2)
