@@ -653,6 +653,7 @@ struct MapCodegen {
     // `kept` lists the operands whose loaded values an earlier phase left in `ld<slot>[e]`,
     // `in_body` maps operands already loaded in the loop body being emitted to their temporaries.
     bool keep_loads = false;
+    int tile_width = 0;  // tile mode over 16-bit tensors: elements per group of consecutive ones that a thread handles (0: one by one)
     // a masked element takes the operand's `other`, which the host rounds to the element type: a float holds both
     bool kept_as_float(int slot) const {
         const int dtype = p.operands[slot].dtype;
@@ -882,9 +883,12 @@ struct MapCodegen {
     void open_element_loop(long long tile_elements, int per_thread, const char *pad) {
         if (keep_loads) {
             out << pad << "#pragma unroll\n"
-                << pad << "for (int e = 0; e < " << per_thread << "; ++e) {\n"
-                << pad << "    const nt_idx element = member + e * " << group << ";\n"
-                << pad << "    if (element >= " << lit(tile_elements) << ") break;\n";
+                << pad << "for (int e = 0; e < " << per_thread << "; ++e) {\n";
+            if (tile_width > 0)  // a thread's elements come in groups of `tile_width` consecutive ones
+                out << pad << "    const nt_idx element = (member + (e / " << tile_width << ") * " << group << ") * " << tile_width << " + e % " << tile_width << ";\n";
+            else
+                out << pad << "    const nt_idx element = member + e * " << group << ";\n";
+            out << pad << "    if (element >= " << lit(tile_elements) << ") break;\n";
         } else {
             out << pad << "for (nt_idx element = member; element < " << lit(tile_elements) << "; element += " << group << ") {\n";
         }
@@ -897,6 +901,110 @@ struct MapCodegen {
         in_body.clear();
     }
 
+    // Tile mode over 16-bit tensors whose elements a thread keeps in registers: groups of 8 consecutive elements per
+    // thread (one 16-byte access per tensor and group) when every tensor advances by one element or not at all along
+    // the tile's last variable.  0: element by element (fp32 tensors alone are as fast that way).
+    int tile_vector_width(long long tile_elements) const {
+        if (p.num_dynamic != 0 || p.store_op == NT_MAP_STORE_ATOMIC_ADD || p.num_vars <= p.num_grid) return 0;
+        std::vector<int> used(1, p.output);
+        for (int pc = 0; pc < p.value_code_length; ++pc) {
+            const int op = p.value_code[pc] & 0xff;
+            if (op == NT_MAP_V_LOAD) used.push_back(p.value_code[pc] >> 8);
+            if (op == NT_MAP_V_SETVAR) return 0;
+        }
+        bool narrow_type = false;
+        for (int slot : used) {
+            if (!kept_as_float(slot)) return 0;
+            if (p.operands[slot].dtype != NINETOOTHED_FLOAT32) narrow_type = true;
+        }
+        const int width = 8, last = p.num_vars - 1;
+        if (!narrow_type || p.extents[last] <= 0 || p.extents[last] % width != 0 || tile_elements % width != 0) return 0;
+        if (group_step(p.operands[p.output].segment, last, width) != 1) return 0;
+        for (int slot : used)
+            if (group_step(p.operands[slot].segment, last, width) < 0) return 0;
+        return width;
+    }
+
+    static std::string vector_type(int dtype) {  // (declared by vector_typedefs; global accesses need the element's alignment only)
+        return std::string("nt_vec_") + (dtype == NINETOOTHED_FLOAT32 ? "f32" : dtype == NINETOOTHED_FLOAT16 ? "f16" : "bf16");
+    }
+
+    void vector_typedefs(int width, const char *pad) {
+        out << pad << "typedef float nt_vec_f32 __attribute__((ext_vector_type(" << width << "), aligned(4)));\n"
+            << pad << "typedef _Float16 nt_vec_f16 __attribute__((ext_vector_type(" << width << "), aligned(2)));\n"
+            << pad << "typedef __bf16 nt_vec_bf16 __attribute__((ext_vector_type(" << width << "), aligned(2)));\n";
+    }
+
+    // `width` values of operand `slot` from the element the variables stand at into ld<slot>[first .. first + width)
+    void load_group(int slot, int width, const std::string &first) {
+        const int last = p.num_vars - 1;
+        const NineToothedMapOperand &operand = p.operands[slot];
+        const std::string valid = fresh("ok");
+        out << indent << "bool " << valid << " = true;\n";
+        const std::string offset = index_segment(operand.segment, valid);
+        const std::string pointer = std::string("((const ") + c_type(operand.dtype) + " *)a.data[" + std::to_string(slot) + "] + " + offset + ")";
+        if (group_step(operand.segment, last, width) == 1) {
+            out << indent << "if (" << valid << ") {\n"
+                << indent << "    const " << vector_type(operand.dtype) << " loaded = *(const " << vector_type(operand.dtype) << " *)" << pointer << ";\n"
+                << indent << "    _Pragma(\"unroll\") for (int j = 0; j < " << width << "; ++j) ld" << slot << "[" << first << " + j] = (float)loaded[j];\n"
+                << indent << "} else {\n"
+                << indent << "    _Pragma(\"unroll\") for (int j = 0; j < " << width << "; ++j) ld" << slot << "[" << first << " + j] = (float)a.other[" << slot << "];\n"
+                << indent << "}\n";
+        } else {
+            out << indent << "{\n"
+                << indent << "    const float shared = " << valid << " ? (float)*" << pointer << " : (float)a.other[" << slot << "];\n"
+                << indent << "    _Pragma(\"unroll\") for (int j = 0; j < " << width << "; ++j) ld" << slot << "[" << first << " + j] = shared;\n"
+                << indent << "}\n";
+        }
+    }
+
+    // tile mode in groups: every operand's values of the thread's groups, loaded once before the phases
+    void preload_groups(long long tile_elements, int per_thread) {
+        vector_typedefs(tile_width, "        ");
+        out << "        #pragma unroll\n"
+            << "        for (int g = 0; g < " << per_thread / tile_width << "; ++g) {\n"
+            << "            const nt_idx element = (member + g * " << group << ") * " << tile_width << ";\n"
+            << "            if (element >= " << lit(tile_elements) << ") break;\n";
+        indent = "            ";
+        decode_tile_variables();
+        for (int pc = 0; pc < p.value_code_length; ++pc) {
+            if ((p.value_code[pc] & 0xff) != NT_MAP_V_LOAD) continue;
+            const int slot = p.value_code[pc] >> 8;
+            if (kept[slot]) continue;
+            kept[slot] = true;
+            load_group(slot, tile_width, "g * " + std::to_string(tile_width));
+        }
+        out << "        }\n";
+    }
+
+    // tile mode in groups: the stored expression, a group's values in one store
+    void store_groups(long long tile_elements, int per_thread, int begin) {
+        const int last = p.num_vars - 1;
+        const NineToothedMapOperand &target = p.operands[p.output];
+        out << "        #pragma unroll\n"
+            << "        for (int g = 0; g < " << per_thread / tile_width << "; ++g) {\n"
+            << "            const nt_idx element = (member + g * " << group << ") * " << tile_width << ";\n"
+            << "            if (element >= " << lit(tile_elements) << ") break;\n";
+        indent = "            ";
+        decode_tile_variables();
+        out << indent << "bool store_ok = true;\n";
+        const std::string offset = index_segment(target.segment, "store_ok");
+        out << indent << "const nt_idx nt_first = v" << last << ";\n"
+            << indent << vector_type(target.dtype) << " result;\n"
+            << indent << "#pragma unroll\n"
+            << indent << "for (int j = 0; j < " << tile_width << "; ++j) {\n";
+        indent += "    ";
+        out << indent << "const nt_idx v" << last << " = nt_first + j;\n"
+            << indent << "const int e = g * " << tile_width << " + j;\n";
+        const std::string value = value_range(begin, p.value_code_length, "");
+        out << indent << "result[j] = (" << c_type(target.dtype) << ")(float)(" << value << ");\n";
+        indent.resize(indent.size() - 4);
+        out << indent << "}\n"
+            << indent << "if (store_ok) __builtin_nontemporal_store(result, (" << vector_type(target.dtype) << " *)((" << c_type(target.dtype) << " *)a.data[" << p.output << "] + " << offset
+            << "));\n"
+            << "        }\n";
+    }
+
     // one workgroup per tile: reduction phases, then the stored expression (see the tile mode of the header)
     std::string generate_tile() {
         long long tiles = 1, tile_elements = 1;
@@ -904,8 +1012,13 @@ struct MapCodegen {
         // up to 16 elements per thread: every operand is read from memory once and kept in registers
         // (4096 rows of fp32: softmax(2x) 1024 wide 13 us against 16, 2048 wide 20 against 27, 4096 wide 33
         // against 42; 32 per thread spills: 8192 wide rms norm 97 us against 62; longer rows get more threads)
-        const int per_thread = (int)((tile_elements + group - 1) / group);
+        int per_thread = (int)((tile_elements + group - 1) / group);
         keep_loads = tile_elements <= (long long)group * 16;
+        // (measured on 4096 rows of fp16, element by element -> groups: one reduction -- rms norm -- 4096 wide 18.9 -> 14.5 us,
+        // 8192 wide 40.7 -> 31.9, 16384 wide 73.3 -> 39.8; two reductions -- softmax, layer norm -- 16384 wide 109 -> 87 and
+        // 97 -> 48 us, but 8192 wide 44.5 -> 69.7 and 48.9 -> 47.8, 4096 wide 28.7 -> 33.9: those stay element by element)
+        tile_width = keep_loads && (p.num_phases == 1 || tile_elements >= 16384) ? tile_vector_width(tile_elements) : 0;
+        if (tile_width > 0) per_thread = (int)((tile_elements / tile_width + group - 1) / group) * tile_width;
         const bool wave_tiles = group == 64 && threads > 64;  // a wave per tile: no exchange through LDS
         if (wave_tiles)
             out << "    const nt_idx member = threadIdx.x & 63;\n"
@@ -923,6 +1036,7 @@ struct MapCodegen {
             // (values of 16- and 32-bit floating-point tensors are kept as floats: half the registers)
             for (int slot = 0; slot < p.num_operands; ++slot) out << "        " << (kept_as_float(slot) ? "float" : "double") << " ld" << slot << "[" << per_thread << "];\n";
         }
+        if (tile_width > 0) preload_groups(tile_elements, per_thread);
         int begin = 0;
         for (int k = 0; k < p.num_phases; ++k) {
             const int op = p.phase_op[k], dtype = p.phase_dtype[k];
@@ -948,6 +1062,13 @@ struct MapCodegen {
             begin = p.phase_end[k];
         }
         const NineToothedMapOperand &target = p.operands[p.output];
+        if (tile_width > 0) {
+            store_groups(tile_elements, per_thread, begin);
+            out << "    }\n}\n";
+            keep_loads = false;
+            tile_width = 0;
+            return out.str();
+        }
         open_element_loop(tile_elements, per_thread, "        ");
         indent = "            ";
         decode_tile_variables();
@@ -1053,13 +1174,8 @@ struct MapCodegen {
 
     std::string generate_vector(int width) {
         const int last = p.num_vars - 1;
-        const auto vector_type = [&](int dtype) {  // (global accesses need the element's alignment only)
-            return std::string("nt_vec_") + (dtype == NINETOOTHED_FLOAT32 ? "f32" : dtype == NINETOOTHED_FLOAT16 ? "f16" : "bf16");
-        };
-        out << "    typedef float nt_vec_f32 __attribute__((ext_vector_type(" << width << "), aligned(4)));\n"
-            << "    typedef _Float16 nt_vec_f16 __attribute__((ext_vector_type(" << width << "), aligned(2)));\n"
-            << "    typedef __bf16 nt_vec_bf16 __attribute__((ext_vector_type(" << width << "), aligned(2)));\n"
-            << "    const nt_idx groups = total_out / " << width << ";\n"
+        vector_typedefs(width, "    ");
+        out << "    const nt_idx groups = total_out / " << width << ";\n"
             << "    for (nt_idx group = (nt_idx)blockIdx.x * " << kMapThreads << " + threadIdx.x; group < groups; group += stride) {\n"
             << "        nt_uidx rest = (nt_uidx)group * " << width << "u;\n";
         for (int v = last; v >= 0; --v)
@@ -1071,24 +1187,8 @@ struct MapCodegen {
             const int slot = p.value_code[pc] >> 8;
             if (kept[slot]) continue;
             kept[slot] = true;
-            const NineToothedMapOperand &operand = p.operands[slot];
-            const std::string valid = fresh("ok");
-            out << indent << "float ld" << slot << "[" << width << "];\n" << indent << "bool " << valid << " = true;\n";
-            const std::string offset = index_segment(operand.segment, valid);
-            const std::string pointer = std::string("((const ") + c_type(operand.dtype) + " *)a.data[" + std::to_string(slot) + "] + " + offset + ")";
-            if (group_step(operand.segment, last, width) == 1) {
-                out << indent << "if (" << valid << ") {\n"
-                    << indent << "    const " << vector_type(operand.dtype) << " loaded = *(const " << vector_type(operand.dtype) << " *)" << pointer << ";\n"
-                    << indent << "    for (int e = 0; e < " << width << "; ++e) ld" << slot << "[e] = (float)loaded[e];\n"
-                    << indent << "} else {\n"
-                    << indent << "    for (int e = 0; e < " << width << "; ++e) ld" << slot << "[e] = (float)a.other[" << slot << "];\n"
-                    << indent << "}\n";
-            } else {
-                out << indent << "{\n"
-                    << indent << "    const float shared = " << valid << " ? (float)*" << pointer << " : (float)a.other[" << slot << "];\n"
-                    << indent << "    for (int e = 0; e < " << width << "; ++e) ld" << slot << "[e] = shared;\n"
-                    << indent << "}\n";
-            }
+            out << indent << "float ld" << slot << "[" << width << "];\n";
+            load_group(slot, width, "0");
         }
         const NineToothedMapOperand &target = p.operands[p.output];
         out << indent << "bool store_ok = true;\n";

@@ -1074,6 +1074,14 @@ def test_generated_source_groups_elements_of_16_bit_tensors():
     # dropout draws random numbers: groups of four even for fp32 tensors
     dropout = ninetoothed.make(dropout_arrangement, dropout_application, (Tensor(1), Tensor(0), Tensor(0), Tensor(1)))
     assert "nt_vec_f32" in _generated_source(dropout, (torch.empty(4096), 0.3, 7, torch.empty(4096)))
+    # tile mode: programs with one reduction, and rows of 16384 elements and more (measured: the others are faster element by element)
+    softmax, rms_norm, layer_norm = (kernel for kernel, _, _ in _normalisation_cases("cpu"))
+    assert "nt_vec_f16" in _generated_source(rms_norm, (half(64, 4096), half(4096), half(64, 4096)))
+    assert "nt_vec" not in _generated_source(rms_norm, (half(64, 4100), half(4100), half(64, 4100)))
+    assert "nt_vec" not in _generated_source(rms_norm, (torch.empty(64, 4096), torch.empty(4096), torch.empty(64, 4096)))
+    assert "nt_vec" not in _generated_source(softmax, (half(64, 4096), half(64, 4096)))
+    assert "nt_vec_f16" in _generated_source(softmax, (half(64, 16384), half(64, 16384)))
+    assert "nt_vec_f16" in _generated_source(layer_norm, (half(64, 16384), half(16384), half(64, 16384)))
 
 
 @gpu
@@ -1103,3 +1111,28 @@ def test_grouped_elements_of_16_bit_tensors(dtype):
     _served_by_map(kernel)
     # (every operation rounds to the tensors' type, as torch's do)
     assert torch.equal(result, x + r[None, :] + c[:, None] * 2)
+
+
+@gpu
+@pytest.mark.parametrize("dtype", (torch.float16, torch.bfloat16))
+def test_grouped_elements_in_tile_mode_match_the_interpreter(dtype, monkeypatch):
+    """Normalisations over rows of 16-bit tensors whose length is a multiple of 8 keep a thread's elements in groups
+    of eight (one 16-byte access per tensor and group): what the interpreter kernel computes element by element, up
+    to the order of the row sums (an ulp of the tensors' type), for rows that one wave, 256, 512 and 1024 threads
+    share, inputs at odd element offsets."""
+    ulp = 2.0**-10 if dtype == torch.float16 else 2.0**-7
+    for rows, cols in ((1001, 32), (77, 512), (64, 4096), (33, 8192), (17, 16384), (5, 2056)):
+        storage = torch.full((rows, cols + 9), float("inf"), dtype=dtype, device="cuda")
+        for kernel, inputs, expected in _normalisation_cases("cuda", dtype, rows, cols):
+            shifted = storage[:, 3 : 3 + cols]
+            shifted.copy_(inputs[0])
+            inputs = (shifted,) + tuple(inputs[1:])
+            results = []
+            for interpret in ("1", "0"):
+                monkeypatch.setenv("NT_MAP_INTERPRET", interpret)
+                out = torch.full((rows, cols), float("nan"), dtype=dtype, device="cuda")
+                kernel(*inputs, out)
+                _served_by_map(kernel)
+                results.append(out)
+            assert torch.allclose(results[0].float(), results[1].float(), rtol=2 * ulp, atol=2 * ulp), (rows, cols, kernel.kernel_name)
+            assert torch.allclose(results[1].float(), expected, rtol=2e-2, atol=2e-2), (rows, cols, kernel.kernel_name)
