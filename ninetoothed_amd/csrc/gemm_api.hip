@@ -619,7 +619,10 @@ int run_gemm(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk, b
 // dst[i][j] = j < d1 ? src[i * s0 + j * s1] : 0 for j < pitch; 64 x 64 tiles through LDS, so that the reads run along
 // whichever dimension has the smaller stride and the writes along j, 16 bytes per lane on both sides where the
 // source is contiguous along that dimension
-__global__ __launch_bounds__(256) void repack_operand_kernel(const uint16_t *src, int64_t d0, int64_t d1, int64_t s0, int64_t s1, uint16_t *dst, int64_t pitch) {
+__global__ __launch_bounds__(256) void repack_operand_kernel(const uint16_t *src, int64_t d0, int64_t d1, int64_t s0, int64_t s1, uint16_t *dst, int64_t pitch,
+                                                            int64_t src_batch) {
+    src += (int64_t)blockIdx.y * src_batch;  // a batch of matrices: the copies lie one after another
+    dst += (int64_t)blockIdx.y * d0 * pitch;
     typedef uint16_t ushort8_t __attribute__((ext_vector_type(8)));
     typedef ushort8_t unaligned_ushort8_t __attribute__((aligned(2)));  // (global accesses need the element's alignment only)
     constexpr int kPitch = 72;  // rows of the tile start on 16-byte boundaries
@@ -673,11 +676,12 @@ __global__ __launch_bounds__(256) void repack_operand_kernel(const uint16_t *src
     }
 }
 
-hipError_t repack_operand(hipStream_t stream, const void *src, int64_t d0, int64_t d1, int64_t s0, int64_t s1, uint16_t *dst, int64_t pitch) {
+hipError_t repack_operand(hipStream_t stream, const void *src, int64_t d0, int64_t d1, int64_t s0, int64_t s1, uint16_t *dst, int64_t pitch, int batch = 1,
+                          int64_t src_batch = 0) {
     const int64_t tiles = ((d0 + 63) / 64) * ((pitch + 63) / 64);
-    if (tiles == 0) return hipSuccess;
-    if (tiles > 0x7fffffffll) return hipErrorInvalidValue;
-    repack_operand_kernel<<<dim3((unsigned)tiles), dim3(256), 0, stream>>>((const uint16_t *)src, d0, d1, s0, s1, dst, pitch);
+    if (tiles == 0 || batch == 0) return hipSuccess;
+    if (tiles > 0x7fffffffll || batch > 65535) return hipErrorInvalidValue;
+    repack_operand_kernel<<<dim3((unsigned)tiles, (unsigned)batch), dim3(256), 0, stream>>>((const uint16_t *)src, d0, d1, s0, s1, dst, pitch, src_batch);
     return hipGetLastError();
 }
 
@@ -687,13 +691,13 @@ int heuristic_choice(const GemmProblem &q, int bm, int bn, int bk);
 // reads them is enqueued) and describes the product on them in `dense`.  0, an error, or NINETOOTHED_NO_KERNEL when
 // this way does not apply.
 int make_dense_copies(hipStream_t stream, const GemmProblem &q, int bm, int bn, int bk, WorkspaceLease &lease, GemmProblem &dense) {
-    if ((q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) || q.batch != 1) return NINETOOTHED_NO_KERNEL;
+    if ((q.dtype != NINETOOTHED_FLOAT16 && q.dtype != NINETOOTHED_BFLOAT16) || q.batch < 1 || q.batch > 65535) return NINETOOTHED_NO_KERNEL;
 #ifndef NT_GEMM_COPY_LOG2
 #define NT_GEMM_COPY_LOG2 21
 #endif
     // (the any-stride kernel is slower from small sizes on: 512^3 36-45 us in place against 11-13 us on copies,
     // 256^3 22-25 against 12; below 128^3 everything is one launch's time)
-    if ((int64_t)q.m * q.n * q.k < ((int64_t)1 << NT_GEMM_COPY_LOG2) || q.fixed_scratch != nullptr) return NINETOOTHED_NO_KERNEL;
+    if ((int64_t)q.m * q.n * q.k * q.batch < ((int64_t)1 << NT_GEMM_COPY_LOG2) || q.fixed_scratch != nullptr) return NINETOOTHED_NO_KERNEL;
     const int64_t k8 = ((int64_t)q.k + 7) / 8 * 8;
     dense = q;
     dense.k = (int)k8;
@@ -701,18 +705,21 @@ int make_dense_copies(hipStream_t stream, const GemmProblem &q, int bm, int bn, 
     dense.sak = 1;
     dense.sbk = 1;
     dense.sbn = k8;
+    dense.a_batch = (int64_t)q.m * k8;  // (a batch: one copy per product, also of an operand that the products share)
+    dense.b_batch = (int64_t)q.n * k8;
     // (alignment of the copies is a fact, not a property of these placeholder addresses)
     dense.a = dense.b = (const void *)(uintptr_t)256;
     const int choice = heuristic_choice(dense, bm, bn, bk);
     if (choice < 0 || choice == kAnyStride) return NINETOOTHED_NO_KERNEL;  // (the output's layout rules the fast instances out)
     // (buffers of their own: the sources may be the widened copies of fp8 operands)
-    uint16_t *a = (uint16_t *)lease.get(kWorkspaceGemmLhsDense, (size_t)q.m * k8 * 2);
-    uint16_t *b = a != nullptr ? (uint16_t *)lease.get(kWorkspaceGemmRhsDense, (size_t)q.n * k8 * 2) : nullptr;
+    if (((int64_t)q.m + q.n) * k8 * 2 * q.batch > (int64_t(1) << 32)) return NINETOOTHED_NO_KERNEL;  // (a batch whose copies would take more than 4 GiB)
+    uint16_t *a = (uint16_t *)lease.get(kWorkspaceGemmLhsDense, (size_t)q.m * k8 * 2 * q.batch);
+    uint16_t *b = a != nullptr ? (uint16_t *)lease.get(kWorkspaceGemmRhsDense, (size_t)q.n * k8 * 2 * q.batch) : nullptr;
     if (a == nullptr || b == nullptr) return NINETOOTHED_NO_KERNEL;
     dense.a = a;
     dense.b = b;
-    if (hipError_t err = repack_operand(stream, q.a, q.m, q.k, q.sam, q.sak, a, k8)) return (int)err;
-    if (hipError_t err = repack_operand(stream, q.b, q.n, q.k, q.sbn, q.sbk, b, k8)) return (int)err;
+    if (hipError_t err = repack_operand(stream, q.a, q.m, q.k, q.sam, q.sak, a, k8, q.batch, q.a_batch)) return (int)err;
+    if (hipError_t err = repack_operand(stream, q.b, q.n, q.k, q.sbn, q.sbk, b, k8, q.batch, q.b_batch)) return (int)err;
     return 0;
 }
 

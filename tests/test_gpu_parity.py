@@ -326,6 +326,15 @@ def test_batched_matmul_layouts_and_output_types(dtype):
     kernel(a2.flip(0), b2, out2)
     assert torch.allclose(out2.float(), torch.bmm(a2.flip(0).float(), b2.float()), **HALF_TOL)
     assert "any-stride" in runtime.last_launch(), runtime.last_launch()
+    # larger products with such sizes run on dense copies, one per product -- also of an lhs that the products share
+    a3, b3 = torch.randn(4, 300, 1001, dtype=dtype, device="cuda")[:, :, :1000], torch.randn(4, 1000, 500, dtype=dtype, device="cuda") * 0.1
+    out3 = torch.full((4, 300, 504), 7.0, dtype=dtype, device="cuda")
+    for lhs in (a3, a3[:1].expand(4, 300, 1000)):
+        out3[:, :, :500] = float("nan")
+        kernel(lhs, b3, out3[:, :, :500])
+        assert "any-stride" not in runtime.last_launch(), runtime.last_launch()
+        assert torch.allclose(out3[:, :, :500].float(), torch.bmm(lhs.float(), b3.float()), rtol=1e-2, atol=1e-2 * 2**0.5)
+        assert bool((out3[:, :, 500:] == 7.0).all())
 
 
 def test_batched_matmul_float32_operands_and_empty_batches():
