@@ -66,7 +66,8 @@ bool fast_accepts(const GemmProblem &q) {
     if (q.sam % 8 || q.sam < q.k || q.scm < q.n) return false;
     if (((uintptr_t)q.a & 15) || ((uintptr_t)q.b & 15)) return false;
     if (!kTail && (((uintptr_t)q.c & 15) || q.scm % 8)) return false;
-    if (q.batch > 1 && ((q.a_batch | q.b_batch | q.c_batch) % 8 || (int64_t)((q.m + BM - 1) / BM) * ((q.n + BN - 1) / BN) * q.batch > 0x7fffffffll)) return false;
+    // (a batch: the operands of every product on 16-byte boundaries; the outputs too, unless the instance stores element by element)
+    if (q.batch > 1 && ((q.a_batch | q.b_batch) % 8 || (!kTail && q.c_batch % 8) || (int64_t)((q.m + BM - 1) / BM) * ((q.n + BN - 1) / BN) * q.batch > 0x7fffffffll)) return false;
     // per-lane 32-bit byte offsets inside one tile panel
     if ((int64_t)BM * q.sam * 2 >= (int64_t(1) << 31)) return false;
     if (b_is_transposed(q)) {  // B as [N, K] with K contiguous (`x @ w.T`)
@@ -97,8 +98,8 @@ void fill_params(GemmParams &p, const GemmProblem &q, int bm, int bn) {
     p.tiles_m = (q.m + bm - 1) / bm;
     p.tiles_n = (q.n + bn - 1) / bn;
     p.order = g_tile_order;
-    p.bias_vector = q.bias != nullptr && q.sin == 1 && q.sim % 8 == 0 && ((uintptr_t)q.bias & 15) == 0 && q.n % 8 == 0;
-    p.c_vector = ((uintptr_t)q.c & 15) == 0 && q.scm % 8 == 0 && q.n % 8 == 0;
+    p.bias_vector = q.bias != nullptr && q.sin == 1 && q.sim % 8 == 0 && ((uintptr_t)q.bias & 15) == 0 && q.n % 8 == 0 && (q.batch == 1 || q.bias_batch % 8 == 0);
+    p.c_vector = ((uintptr_t)q.c & 15) == 0 && q.scm % 8 == 0 && q.n % 8 == 0 && (q.batch == 1 || q.c_batch % 8 == 0);
     p.kt_per_split = 0;
     p.batch = q.batch;
     p.a_batch = q.a_batch;
@@ -511,8 +512,10 @@ int heuristic_choice(const GemmProblem &q, int bm, int bn, int bk) {
         if (!inst.accepts(q)) continue;
         const int64_t per_matrix = (int64_t)((q.m + inst.bm - 1) / inst.bm) * ((q.n + inst.bn - 1) / inst.bn);
         // (a batch of small matrices reaches any number of tiles: a tile that such a matrix fills to less than
-        // 60 % is left to the rules of the second pass, which start from the small tiles)
-        if (q.batch > 1 && rule.min_tiles > 1 && (int64_t)q.m * q.n * 5 < per_matrix * inst.bm * inst.bn * 3) continue;
+        // 60 % is left to the rules of the second pass, which start from the small tiles -- unless 64 x 64 tiles
+        // would be as empty: 197 x 197 fills 59 % of one 256 x 256 tile and 59 % of sixteen 64 x 64 ones)
+        const int64_t small_tiles = (int64_t)((q.m + 63) / 64) * ((q.n + 63) / 64) * 64 * 64;
+        if (q.batch > 1 && rule.min_tiles > 1 && (int64_t)q.m * q.n * 5 < per_matrix * inst.bm * inst.bn * 3 && per_matrix * inst.bm * inst.bn * 9 > small_tiles * 10) continue;
         if (per_matrix * q.batch >= rule.min_tiles) return rule.instance;
     }
     return kInstances[kAnyStride].accepts(q) ? kAnyStride : -1;

@@ -326,6 +326,13 @@ def test_batched_matmul_layouts_and_output_types(dtype):
     kernel(a2.flip(0), b2, out2)
     assert torch.allclose(out2.float(), torch.bmm(a2.flip(0).float(), b2.float()), **HALF_TOL)
     assert "any-stride" in runtime.last_launch(), runtime.last_launch()
+    # outputs of 197 x 197 elements each (no multiple of 8 between them) against k-contiguous operands: the instances
+    # with tails, which then store element by element
+    q4, k4 = torch.randn(24, 197, 64, dtype=dtype, device="cuda"), torch.randn(24, 197, 64, dtype=dtype, device="cuda")
+    scores = torch.full((24, 197, 197), float("nan"), dtype=dtype, device="cuda")
+    kernel(q4, k4.transpose(1, 2), scores)
+    assert "any-stride" not in runtime.last_launch(), runtime.last_launch()
+    assert torch.allclose(scores.float(), torch.bmm(q4.float(), k4.float().transpose(1, 2)), **HALF_TOL)
     # larger products with such sizes run on dense copies, one per product -- also of an lhs that the products share
     a3, b3 = torch.randn(4, 300, 1001, dtype=dtype, device="cuda")[:, :, :1000], torch.randn(4, 1000, 500, dtype=dtype, device="cuda") * 0.1
     out3 = torch.full((4, 300, 504), 7.0, dtype=dtype, device="cuda")
