@@ -1016,7 +1016,8 @@ struct MapCodegen {
         keep_loads = tile_elements <= (long long)group * 16;
         // (measured on 4096 rows of fp16, element by element -> groups: one reduction -- rms norm -- 4096 wide 18.9 -> 14.5 us,
         // 8192 wide 40.7 -> 31.9, 16384 wide 73.3 -> 39.8; two reductions -- softmax, layer norm -- 16384 wide 109 -> 87 and
-        // 97 -> 48 us, but 8192 wide 44.5 -> 69.7 and 48.9 -> 47.8, 4096 wide 28.7 -> 33.9: those stay element by element)
+        // 97 -> 48 us, but 8192 wide 39.7 -> 62.4 and 36.7 -> 43.1, 4096 wide 24.2 -> 29.8 and 19.6 -> 17.4: those stay
+        // element by element)
         tile_width = keep_loads && (p.num_phases == 1 || tile_elements >= 16384) ? tile_vector_width(tile_elements) : 0;
         if (tile_width > 0) per_thread = (int)((tile_elements / tile_width + group - 1) / group) * tile_width;
         const bool wave_tiles = group == 64 && threads > 64;  // a wave per tile: no exchange through LDS
@@ -1041,14 +1042,21 @@ struct MapCodegen {
         for (int k = 0; k < p.num_phases; ++k) {
             const int op = p.phase_op[k], dtype = p.phase_dtype[k];
             const char *init = op == NT_MAP_REDUCE_SUM ? "0.0" : (op == NT_MAP_REDUCE_MAX ? "-__builtin_inf()" : "__builtin_inf()");
-            out << "        double r" << k << ";\n        {\n            double acc = " << init << ";\n";
+            // a reduction of fp32 values (terms rounded to a 16- or 32-bit floating-point type, sums rounded to one after
+            // every addition) is carried in a float: the same values, half the shuffles and no fp64 instructions
+            const int last_op = p.phase_end[k] > begin ? p.value_code[p.phase_end[k] - 1] : 0;
+            const auto single_type = [](int t) { return t == NINETOOTHED_FLOAT32 || t == NINETOOTHED_FLOAT16 || t == NINETOOTHED_BFLOAT16; };
+            const bool single = single_type(dtype) && (((last_op & 0xff) == NT_MAP_V_ROUND && single_type(last_op >> 8)) ||
+                                                       ((last_op & 0xff) == NT_MAP_V_LOAD && kept_as_float(last_op >> 8)));
+            const char *carried = single ? "float" : "double";
+            out << "        " << carried << " r" << k << ";\n        {\n            " << carried << " acc = " << init << ";\n";
             open_element_loop(tile_elements, per_thread, "            ");
             indent = "                ";
             decode_tile_variables();
             const std::string term = value_range(begin, p.phase_end[k], "");
             out << indent << "acc = " << combine_expr(op, dtype, "acc", term) << ";\n";
             close_element_loop("            ");
-            out << "            for (int offset = 32; offset > 0; offset >>= 1) { const double other = __shfl_xor(acc, offset, 64); acc = "
+            out << "            for (int offset = 32; offset > 0; offset >>= 1) { const " << carried << " other = __shfl_xor(acc, offset, 64); acc = "
                 << combine_expr(op, dtype, "acc", "other") << "; }\n";
             if (wave_tiles) {
                 out << "            r" << k << " = acc;\n        }\n";
@@ -1057,7 +1065,7 @@ struct MapCodegen {
             }
             out << "            __syncthreads();\n            if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = acc;\n            __syncthreads();\n"
                 << "            acc = scratch[0];\n"
-                << "            for (int w = 1; w < " << threads / 64 << "; ++w) { const double other = scratch[w]; acc = " << combine_expr(op, dtype, "acc", "other")
+                << "            for (int w = 1; w < " << threads / 64 << "; ++w) { const " << carried << " other = scratch[w]; acc = " << combine_expr(op, dtype, "acc", "other")
                 << "; }\n            r" << k << " = acc;\n        }\n";
             begin = p.phase_end[k];
         }
@@ -1251,7 +1259,13 @@ struct MapCodegen {
             result = value_range(0, p.value_code_length, "");
         } else {
             const char *init = p.reduce_op == NT_MAP_REDUCE_SUM ? "0.0" : (p.reduce_op == NT_MAP_REDUCE_MAX ? "-__builtin_inf()" : "__builtin_inf()");
-            out << "        double acc = " << init << ";\n";
+            // (a reduction of fp32 values is carried in a float, as in tile mode)
+            const int last_op = p.reduce_split > 0 ? p.value_code[p.reduce_split - 1] : 0;
+            const auto single_type = [](int t) { return t == NINETOOTHED_FLOAT32 || t == NINETOOTHED_FLOAT16 || t == NINETOOTHED_BFLOAT16; };
+            const bool single = single_type(p.reduce_dtype) && (((last_op & 0xff) == NT_MAP_V_ROUND && single_type(last_op >> 8)) ||
+                                                                ((last_op & 0xff) == NT_MAP_V_LOAD && kept_as_float(last_op >> 8)));
+            const char *carried = single ? "float" : "double";
+            out << "        " << carried << " acc = " << init << ";\n";
             long long reduced_total = 1;
             for (int v = num_out; v < p.num_vars; ++v) reduced_total *= p.extents[v];
             if (lanes > 1) {  // the lanes of a wave stride the reduced positions
@@ -1278,13 +1292,13 @@ struct MapCodegen {
                 indent.resize(indent.size() - 4);
                 out << indent << "}\n";
                 for (int offset = 32; offset > 0; offset >>= 1)
-                    out << indent << "{ const double other = __shfl_xor(acc, " << offset << ", 64); acc = " << combine_expr(p.reduce_op, p.reduce_dtype, "acc", "other") << "; }\n";
+                    out << indent << "{ const " << carried << " other = __shfl_xor(acc, " << offset << ", 64); acc = " << combine_expr(p.reduce_op, p.reduce_dtype, "acc", "other") << "; }\n";
                 if (lanes > 64) {  // the waves of the workgroup (all of them work on this element: the loop is uniform)
                     out << indent << "if ((threadIdx.x & 63) == 0) nt_partial[threadIdx.x >> 6] = acc;\n"
                         << indent << "__syncthreads();\n"
                         << indent << "acc = nt_partial[0];\n";
                     for (int w = 1; w < lanes / 64; ++w)
-                        out << indent << "{ const double other = nt_partial[" << w << "]; acc = " << combine_expr(p.reduce_op, p.reduce_dtype, "acc", "other") << "; }\n";
+                        out << indent << "{ const " << carried << " other = nt_partial[" << w << "]; acc = " << combine_expr(p.reduce_op, p.reduce_dtype, "acc", "other") << "; }\n";
                     out << indent << "__syncthreads();\n";
                 }
             } else
