@@ -112,3 +112,21 @@ def test_static_scratch_matmul_never_takes_buffers_for_copies():
     tolerance = dict(rtol=1e-2, atol=1e-2 * (k / 512) ** 0.5)
     assert torch.allclose(out8.float(), a8.to(torch.float16).float() @ b8.to(torch.float16).float(), **tolerance)
     assert torch.allclose(out16.float(), a_off.float() @ b16.float(), **tolerance)
+    # fp32 products of few tiles and products a few tiles over whole rounds of the chip put partial products into
+    # allocated buffers under launch_nt_matmul; here they run in one pass
+    print("static-scratch matmul: fp32 products of few tiles, 17 x 17 tiles, no buffers", flush=True)
+    lib.nt_release_workspaces()
+    a32, b32 = torch.randn(128, 4096, device="cuda"), torch.randn(4096, 128, device="cuda")
+    out32 = torch.full((128, 128), float("nan"), device="cuda")
+    big_a, big_b = torch.randn(4352, 2048, dtype=torch.float16, device="cuda"), torch.randn(2048, 4352, dtype=torch.float16, device="cuda") * 0.1
+    big_out = torch.full((4352, 4352), float("nan"), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    assert _call(lib.launch_nt_matmul_static_scratch, a32, b32, out32, "fp32") == 0
+    assert "parts" not in runtime.last_launch(), runtime.last_launch()
+    assert _call(lib.launch_nt_matmul_static_scratch, big_a, big_b, big_out, "fp16") == 0
+    assert "last rows" not in runtime.last_launch(), runtime.last_launch()
+    torch.cuda.synchronize()
+    assert free_before - torch.cuda.mem_get_info()[0] < (1 << 20)
+    assert torch.allclose(out32.double(), a32.double() @ b32.double(), rtol=1e-4, atol=1e-3)
+    assert torch.allclose(big_out.float(), big_a.float() @ big_b.float(), rtol=1e-2, atol=2e-2)
