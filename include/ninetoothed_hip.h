@@ -271,7 +271,10 @@ NineToothedResult launch_nt_conv2d_strided(NineToothedStream stream,
  * exceed the array, the K range is cut into as many parts as fit (same kernels, another summation order);
  * a call for which not even two parts fit (M x N x 8 bytes > the array) returns
  * NINETOOTHED_SCRATCH_LIMIT and launches nothing (it does not fall back to another kernel); problems
- * that run in one pass need no scratch memory and are accepted at any size.  Operands that
+ * that run in one pass need no scratch memory and are accepted at any size (the untuned choice splits
+ * only products of fewer than 256 tiles of 64 x 64, which always fit; a tuned choice may name a split-K
+ * instance for a larger one).  fp32 products and products a few tiles over whole rounds of the chip, whose
+ * partial products launch_nt_matmul puts into allocated buffers, run in one pass here.  Operands that
  * launch_nt_matmul would copy into allocated buffers (FLOAT8_E5M2; fp16 / bf16 operands that the
  * direct-to-LDS kernels cannot read in place) run here on the kernels that read them in place, slower.
  *

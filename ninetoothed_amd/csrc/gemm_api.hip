@@ -494,10 +494,16 @@ int heuristic_choice(const GemmProblem &q, int bm, int bn, int bk) {
     // 128x256 from 128 tiles up, 128x128 from 256 tiles up, else the smallest tile that divides
     struct Rule { int instance; int64_t min_tiles; };
     // too few tiles for the chip: split K (64-row tiles for up to 64 rows, else 128 x 128)
+    // (64 x 64 tiles of the product: where they fill the chip, a skinny product runs on them in one pass -- 256 x 4096 x 4096
+    // 19 us against 27 with K in parts of 128 x 128 tiles, 128 x 4096 x 14336 33 against 42 -- and tiles that the product
+    // fills to less than half along M or N are passed over: 64 x 4096 x 128256 259 us on 256 x 256 tiles, 220 on 64 x 64)
+    const int64_t tiles_64 = (int64_t)((q.m + 63) / 64) * ((q.n + 63) / 64);
+    const bool small_tiles_fill_the_chip = q.batch == 1 && tiles_64 >= 256 && kInstances[kTail64x64x64].accepts(q);
     const auto few_tiles = [&](int instance) {
         const GemmInstance &inst = kInstances[instance];
         // (with a short K the second kernel costs more than the idle CUs: 512^3 8 us split, 5 in one pass)
-        return q.batch == 1 && q.k >= 2048 && (int64_t)((q.m + inst.bm - 1) / inst.bm) * ((q.n + inst.bn - 1) / inst.bn) < 192 && inst.accepts(q);
+        return q.batch == 1 && !small_tiles_fill_the_chip && q.k >= 2048 && (int64_t)((q.m + inst.bm - 1) / inst.bm) * ((q.n + inst.bn - 1) / inst.bn) < 192 &&
+               inst.accepts(q);
     };
     if (q.m <= 64 && few_tiles(kSplit64x64x64)) return kSplit64x64x64;
     if (few_tiles(kSplit128x128x64)) return kSplit128x128x64;
@@ -514,7 +520,10 @@ int heuristic_choice(const GemmProblem &q, int bm, int bn, int bk) {
         // (a batch of small matrices reaches any number of tiles: a tile that such a matrix fills to less than
         // 60 % is left to the rules of the second pass, which start from the small tiles -- unless 64 x 64 tiles
         // would be as empty: 197 x 197 fills 59 % of one 256 x 256 tile and 59 % of sixteen 64 x 64 ones)
-        const int64_t small_tiles = (int64_t)((q.m + 63) / 64) * ((q.n + 63) / 64) * 64 * 64;
+        if (small_tiles_fill_the_chip && (inst.bm > 64 || inst.bn > 64) &&
+            ((int64_t)q.m * 2 < (int64_t)((q.m + inst.bm - 1) / inst.bm) * inst.bm || (int64_t)q.n * 2 < (int64_t)((q.n + inst.bn - 1) / inst.bn) * inst.bn))
+            continue;
+        const int64_t small_tiles = tiles_64 * 64 * 64;
         if (q.batch > 1 && rule.min_tiles > 1 && (int64_t)q.m * q.n * 5 < per_matrix * inst.bm * inst.bn * 3 && per_matrix * inst.bm * inst.bn * 9 > small_tiles * 10) continue;
         if (per_matrix * q.batch >= rule.min_tiles) return rule.instance;
     }

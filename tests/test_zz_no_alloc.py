@@ -55,7 +55,10 @@ def test_static_scratch_matmul_matches_the_allocating_entry_point(dtype, tag):
         assert torch.allclose(out.float(), a.float() @ b.float(), rtol=1e-2, atol=1e-2)
 
 
-def test_static_scratch_matmul_fp32_output_one_pass_problems_and_the_limit():
+def test_static_scratch_matmul_fp32_output_one_pass_problems_and_the_limit(tmp_path):
+    import csv
+    import ctypes
+
     lib = runtime.library()
     print("static-scratch matmul: fp32 output, one-pass problem, scratch limit", flush=True)
     a, b = _operands(64, 2048, 8192, torch.float16, 20)
@@ -79,12 +82,36 @@ def test_static_scratch_matmul_fp32_output_one_pass_problems_and_the_limit():
     assert _call(lib.launch_nt_matmul, a, b, expected, "fp16") == 0
     torch.cuda.synchronize()
     assert torch.allclose(out.float(), expected.float(), rtol=1e-2, atol=1e-2)
-    # 1024 x 2560 outputs: even two parts of partial products (20 MiB) exceed the array -> refused, nothing written
+    # 1024 x 2560 outputs: 64 x 64 tiles fill the chip, so the untuned choice is one pass and any size goes
     a, b = _operands(1024, 2560, 8192, torch.float16, 23)
-    out = torch.full((1024, 2560), float("nan"), dtype=torch.float16, device="cuda")
+    out, expected = (torch.full((1024, 2560), float("nan"), dtype=torch.float16, device="cuda") for _ in range(2))
+    assert _call(lib.launch_nt_matmul_static_scratch, a, b, out, "fp16") == 0
+    assert "split-k" not in runtime.last_launch(), runtime.last_launch()
+    assert _call(lib.launch_nt_matmul, a, b, expected, "fp16") == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out, expected)
+    # ... until a tuned choice names a split-K instance for the problem (here: read from a cache file): even two parts
+    # of partial products (20 MiB) exceed the array -> refused, nothing written
+    names = runtime.gemm_config_names()
+    split = next(i for i, name in enumerate(names) if name.startswith("256x256x32") and "split-k" in name)
+    fp16 = runtime.DATA_TYPE_INDEX["fp16"]
+    path = tmp_path / "tuned.csv"
+    with open(path, "w", newline="") as handle:
+        writer = csv.writer(handle)
+        writer.writerow(())
+        writer.writerow((lib.nt_tune_file_format(),))
+        writer.writerow((runtime.TUNE_GEMM, fp16, fp16, 1024, 2560, 8192, 0, 0))
+        writer.writerow((split, 256, 256, 32))
+    entries = ctypes.c_int(0)
+    assert lib.nt_tune_cache_load(str(path).encode(), ctypes.byref(entries)) == 0 and entries.value == 1
+    out.fill_(float("nan"))
     assert _call(lib.launch_nt_matmul_static_scratch, a, b, out, "fp16") == runtime.SCRATCH_LIMIT
     torch.cuda.synchronize()
     assert bool(torch.isnan(out).all())
+    assert _call(lib.launch_nt_matmul, a, b, out, "fp16") == 0  # (with the stream's buffer the tuned instance runs)
+    assert "split-k" in runtime.last_launch(), runtime.last_launch()
+    torch.cuda.synchronize()
+    assert torch.allclose(out.float(), expected.float(), rtol=1e-2, atol=1e-2 * 4)
     assert runtime.STATIC_SCRATCH_BYTES == 16 << 20
 
 
